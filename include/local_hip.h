@@ -1,0 +1,301 @@
+/*
+ * local_hip.h -- C ABI of the gfx950 (MI355X) decode hot-path library.
+ *
+ * The library replaces, for Q4_0 / TQ2_0 quantized weights and the TurboQuant
+ * KV cache, the kernel-dispatch layer that local-engine calls on local-metal
+ * (local-metal/src/kernels.rs `Kernels`, plus batch.rs / buffer.rs / context.rs /
+ * error.rs).  Every entry point below names the reference interface it stands
+ * in for.  Conventions:
+ *
+ *  - Opaque handles; plain integers by value; no C++ / torch types.
+ *  - Every call returns an lh_status (0 = OK).  On failure the message is kept
+ *    per thread and read with lh_last_error(); its text follows the Display
+ *    form of local_metal::Error (local-metal/src/error.rs:1-32), e.g.
+ *    "Invalid argument: matvec_q4_0: cols 100 not /32".
+ *  - `*_into` calls enqueue work on the context's single in-order HIP stream
+ *    (the stand-in for one serial MTLComputeCommandEncoder: later dispatches
+ *    see earlier dispatches' results) and return immediately; the blocking
+ *    forms without `_into` enqueue and wait, as the reference's do.
+ *  - Arguments are validated on the host (alignment of `cols`, buffer sizes
+ *    against the shapes) before anything is launched.
+ *  - Matrices are [rows(N), cols(K)] row-major in verbatim GGUF block layout
+ *    (local-engine/src/layer.rs:16-17, shaders/matvec_quant.metal:11-17).
+ *  - One owner thread per context (local-engine/src/cli/serve.rs:3-11).
+ */
+#ifndef LOCAL_HIP_H
+#define LOCAL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LH_API __attribute__((visibility("default")))
+
+/* local-metal/src/error.rs:1-32 */
+typedef enum lh_status {
+    LH_OK = 0,
+    LH_ERR_NO_DEVICE = 1,           /* NoMetalDevice / NoDevice */
+    LH_ERR_NO_COMMAND_QUEUE = 2,    /* NoCommandQueue (stream creation failed) */
+    LH_ERR_BUFFER_ALLOCATION = 3,   /* BufferAllocation{size,reason} */
+    LH_ERR_LIBRARY_CREATION = 4,    /* LibraryCreation */
+    LH_ERR_PIPELINE_CREATION = 5,   /* PipelineCreation (kernel unavailable) */
+    LH_ERR_SHADER_NOT_FOUND = 6,    /* ShaderNotFound */
+    LH_ERR_COMMAND_BUFFER = 7,      /* CommandBuffer("GPU error: ...") */
+    LH_ERR_INVALID_ARGUMENT = 8,    /* InvalidArgument */
+    LH_ERR_IO = 9                   /* Io */
+} lh_status;
+
+typedef struct lh_context lh_context;  /* local-metal/src/context.rs:31 MetalContext (device + queue) */
+typedef struct lh_buffer lh_buffer;    /* local-metal/src/buffer.rs:17 MetalBuffer */
+typedef struct lh_batch lh_batch;      /* local-metal/src/batch.rs:21 CommandBatch */
+
+/* Element types of activation / output buffers for the typed entry points. */
+typedef enum lh_dtype { LH_F16 = 0, LH_F32 = 1, LH_BF16 = 2 } lh_dtype;
+/* Weight block formats (local-engine/src/gguf.rs:247-268 block_size). */
+typedef enum lh_quant { LH_Q4_0 = 0, LH_TQ2_0 = 1 } lh_quant;
+
+LH_API const char* lh_last_error(void);
+LH_API const char* lh_version(void);
+
+/* ---- context: MetalContext::new / device_name / caps (context.rs:38-86) ---- */
+LH_API int lh_context_create(int device_index, lh_context** out);
+LH_API void lh_context_destroy(lh_context* ctx);
+LH_API int lh_context_device_name(const lh_context* ctx, char* dst, size_t dst_len);
+LH_API int lh_context_compute_units(const lh_context* ctx);
+LH_API void* lh_context_stream(const lh_context* ctx);          /* hipStream_t, for interop */
+LH_API int lh_context_synchronize(lh_context* ctx);
+
+/* ---- timing: HIP events recorded on the context's stream (stands in for the
+ *      reference's LOCAL_AI_TIMING wall-clock timers, local-engine/src/pipeline.rs:124-127,
+ *      with device-side time stamps). ---- */
+typedef struct lh_event lh_event;
+LH_API int lh_event_create(lh_context* ctx, lh_event** out);
+LH_API void lh_event_destroy(lh_event* ev);
+LH_API int lh_event_record(lh_event* ev);                       /* enqueue on the context stream */
+LH_API int lh_event_elapsed_ms(lh_event* start, lh_event* stop, float* ms); /* waits for `stop` */
+
+/* ---- buffers: MetalBuffer::{from_slice, empty, length, as_slice,
+ *      copy_from_bytes} (buffer.rs:28-131).  Device memory is not host-mapped
+ *      on a discrete GPU, so host access is an explicit copy, ordered after all
+ *      work already enqueued on the context. ---- */
+LH_API int lh_buffer_from_bytes(lh_context* ctx, const void* src, size_t len, lh_buffer** out);
+LH_API int lh_buffer_empty(lh_context* ctx, size_t len, lh_buffer** out);      /* zero-filled */
+LH_API int lh_buffer_view(lh_buffer* parent, size_t offset, size_t len, lh_buffer** out); /* non-owning */
+LH_API int lh_buffer_wrap(lh_context* ctx, void* device_ptr, size_t len, lh_buffer** out); /* non-owning */
+LH_API void lh_buffer_free(lh_buffer* buf);
+LH_API size_t lh_buffer_length(const lh_buffer* buf);
+LH_API void* lh_buffer_device_ptr(const lh_buffer* buf);
+LH_API int lh_buffer_write(lh_buffer* buf, size_t offset, const void* src, size_t len);
+LH_API int lh_buffer_read(const lh_buffer* buf, size_t offset, void* dst, size_t len);
+LH_API int lh_buffer_fill_zero(lh_buffer* buf);                 /* quant_cache.rs:367-380 reset() */
+
+/* ---- command batch: CommandBatch::{new, dispatch_count, blit_buffer_copies,
+ *      commit_and_wait, submit_and_renew, commit_and_renew} (batch.rs:154-291) ---- */
+LH_API int lh_batch_new(lh_context* ctx, lh_batch** out);
+LH_API void lh_batch_free(lh_batch* batch);
+LH_API uint32_t lh_batch_dispatch_count(const lh_batch* batch);
+LH_API int lh_batch_blit_copy(lh_batch* batch, const lh_buffer* src, size_t src_offset, lh_buffer* dst,
+                              size_t dst_offset, size_t len);
+LH_API int lh_batch_commit_and_wait(lh_batch* batch);
+LH_API int lh_batch_submit_and_renew(lh_batch* batch);
+LH_API int lh_batch_commit_and_renew(lh_batch* batch);
+
+/* ---- M = 1 fused dequant matvec: y[rows] = W[rows, cols] . x[cols] ----------
+ * kernels.rs:5711-5838 matvec_q4_0{,_into,_f32out,_f32out_into};
+ * kernels.rs:5848-6038 matvec_tq2_0{,_into,_f32out,_f32out_into};
+ * shaders/matvec_quant.metal:65-155, 173-312.  x is f16; y f16 or f32.
+ * cols % 32 (Q4_0) / % 256 (TQ2_0) != 0 -> LH_ERR_INVALID_ARGUMENT. */
+LH_API int lh_matvec_q4_0(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
+                          uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_q4_0_into(lh_batch* batch, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
+                               uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_q4_0_f32out(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector,
+                                 lh_buffer* output, uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_q4_0_f32out_into(lh_batch* batch, const lh_buffer* matrix, const lh_buffer* vector,
+                                      lh_buffer* output, uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_tq2_0(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
+                           uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_tq2_0_into(lh_batch* batch, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
+                                uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_tq2_0_f32out(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector,
+                                  lh_buffer* output, uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_tq2_0_f32out_into(lh_batch* batch, const lh_buffer* matrix, const lh_buffer* vector,
+                                       lh_buffer* output, uint32_t rows, uint32_t cols);
+/* kernels.rs:5919-5971 matvec_tq2_0_soa_into: qs[rows*cols/256*64] u8 and
+ * scales[rows*cols/256] f16 split out of the 66-byte blocks
+ * (shaders/matvec_quant.metal:314-387). */
+LH_API int lh_matvec_tq2_0_soa_into(lh_batch* batch, const lh_buffer* qs, const lh_buffer* scales,
+                                    const lh_buffer* vector, lh_buffer* output, uint32_t rows, uint32_t cols);
+/* Same matvec with the activation / output element type chosen by the caller
+ * (fp32 x and fp32 y are what the measured configurations use; the reference's
+ * GPU path is f16-only, its CPU path is f32).  No reference counterpart beyond
+ * the four variants above. */
+LH_API int lh_matvec_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* matrix,
+                                      const lh_buffer* vector, lh_dtype vector_dtype, lh_buffer* output,
+                                      lh_dtype output_dtype, uint32_t rows, uint32_t cols);
+/* `count` independent matvecs of one shape in a single launch (what the
+ * reference's decode loop issues back to back inside one command buffer,
+ * kernels.rs:8883-9020: e.g. gate+up, or Q/K/V, which share x).  Arrays are
+ * host arrays of buffer handles. */
+LH_API int lh_matvec_quant_grouped_into(lh_batch* batch, lh_quant fmt, uint32_t count,
+                                        const lh_buffer* const* matrices, const lh_buffer* const* vectors,
+                                        lh_dtype vector_dtype, lh_buffer* const* outputs, lh_dtype output_dtype,
+                                        uint32_t rows, uint32_t cols);
+
+/* ---- small-M / prefill quantized matmul: C[m,n] = A[m,k] . W[n,k]^T ----------
+ * kernels.rs:6459-6563 matmul_nt_{q4_0,tq2_0}_into (routes by m:
+ * batchm / smallm / mma / scalar), kernels.rs:6378-6457 multivec_nt_*_into
+ * (1 <= m <= 16), layer.rs:218-246.  A and C are f16 row-major. */
+LH_API int lh_matmul_nt_q4_0_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                  lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
+LH_API int lh_matmul_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                   lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
+LH_API int lh_multivec_nt_q4_0_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                    lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
+LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                     lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
+/* Typed form: A f16 / f32 / bf16, C f16 / f32 (the measured small-batch and
+ * prefill configurations use f32 and bf16 activations). */
+LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, lh_dtype input_dtype,
+                                         const lh_buffer* weight, lh_buffer* output, lh_dtype output_dtype,
+                                         uint32_t m, uint32_t k, uint32_t n);
+/* kernels.rs:5517-5568 matmul_nt_into: FP16 weights, shaders/matmul_f16.metal:74-114. */
+LH_API int lh_matmul_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, lh_buffer* output,
+                             uint32_t m, uint32_t k, uint32_t n);
+/* kernels.rs:6155, 6160, 6362 constants and 6277-6304 env-flag getters
+ * (LOCAL_AI_BATCHM / LOCAL_AI_MMA / LOCAL_AI_SMALLM, read once per process). */
+LH_API uint32_t lh_smallm_max_m(void);
+LH_API uint32_t lh_batchm_max_m(void);
+LH_API uint32_t lh_multivec_max_m(void);
+LH_API int lh_batchm_enabled(void);
+LH_API int lh_mma_enabled(void);
+LH_API int lh_smallm_enabled(void);
+
+/* ---- block dequant to f16 (bit-exact twin of the CPU path) ----------------
+ * local-engine/src/qat_recover.rs:23-97 dequant_{tq2_0,q4_0}_into; used by
+ * QuantWeight::dequant_row_into (layer.rs:269-281) for the embedding gather.
+ * `byte_offset` selects where in `data` the blocks start (a row of a matrix). */
+LH_API int lh_dequant_q4_0_into(lh_batch* batch, const lh_buffer* data, size_t byte_offset, lh_buffer* output,
+                                size_t num_elements);
+LH_API int lh_dequant_tq2_0_into(lh_batch* batch, const lh_buffer* data, size_t byte_offset, lh_buffer* output,
+                                 size_t num_elements);
+/* kernels.rs:6753-6802 tq2_dequant (legacy 2-bit unpack, shaders/tq2_dequant.metal:4-16). */
+LH_API int lh_tq2_dequant(lh_context* ctx, const lh_buffer* packed, const lh_buffer* scales, lh_buffer* output,
+                          uint32_t num_elements);
+
+/* ---- TurboQuant codec parameters (host side, no GPU work) --------------------
+ * local-engine/src/turboquant.rs:66-79 Rotation::new (splitmix64 signs),
+ * 114-166 lloyd_max_gaussian, 187-192 TurboQuant::new (levels / sqrt(dim)),
+ * 202-204 code_bytes; local-engine/src/kv_cache/quant_cache.rs:30,37 (seed,
+ * default bits), 48-54 swa_ring_capacity, 60-66 kv_bits_from_env.  `levels`
+ * receives 1 << bits floats, `signs` receives dim floats. */
+#define LH_TQ_SEED 0x7459C0DEull
+#define LH_DEFAULT_KV_BITS 2
+LH_API int lh_turboquant_levels(uint32_t dim, uint32_t bits, float* levels);
+LH_API int lh_turboquant_signs(uint32_t dim, uint64_t seed, float* signs);
+LH_API uint32_t lh_turboquant_code_bytes(uint32_t dim, uint32_t bits);
+LH_API size_t lh_swa_ring_capacity(size_t window, size_t max_positions);
+LH_API uint32_t lh_kv_bits_from_env(void);
+
+/* ---- TurboQuant KV cache ----------------------------------------------------
+ * kernels.rs:4819-4890 encode_kv_turboquant_into, 4988-5020 encode_kv_turboquant,
+ * shaders/dequantize_kv.metal:216-318.  input [num_tokens, n_kv_heads, head_dim]
+ * f16; slot g = ((position + token) % ring_capacity or absolute) * n_kv_heads +
+ * head; codes LSB-first, ceil(head_dim*bits/8) bytes per slot; norms f16.
+ * Codes and norms equal the CPU encoder's (turboquant.rs:241-276) bit for bit. */
+LH_API int lh_encode_kv_turboquant(lh_context* ctx, const lh_buffer* input, const lh_buffer* levels,
+                                   const lh_buffer* signs, lh_buffer* packed, lh_buffer* norms, uint32_t head_dim,
+                                   uint32_t n_kv_heads, uint32_t num_tokens, uint32_t bits, uint32_t position,
+                                   uint32_t ring_capacity);
+LH_API int lh_encode_kv_turboquant_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* levels,
+                                        const lh_buffer* signs, lh_buffer* packed, lh_buffer* norms,
+                                        uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens, uint32_t bits,
+                                        uint32_t position, uint32_t ring_capacity);
+/* kernels.rs:4901-4979 encode_kv_turboquant_batched_into,
+ * shaders/dequantize_kv.metal:327-407: slot (lane*lane_capacity +
+ * positions[lane] % ring) * n_kv_heads + head; positions u32[n_lanes]. */
+LH_API int lh_encode_kv_turboquant_batched_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* levels,
+                                                const lh_buffer* signs, lh_buffer* packed, lh_buffer* norms,
+                                                const lh_buffer* positions, uint32_t head_dim, uint32_t n_kv_heads,
+                                                uint32_t lane_capacity, uint32_t bits, uint32_t n_lanes,
+                                                uint32_t ring_capacity);
+/* kernels.rs:4641-4804 dequantize_kv_turboquant{,_into},
+ * shaders/dequantize_kv.metal:132-189: codes -> f16 [num_tokens, n_kv, head_dim]
+ * for tokens [token_start, num_tokens). */
+LH_API int lh_dequantize_kv_turboquant(lh_context* ctx, const lh_buffer* packed, const lh_buffer* norms,
+                                       const lh_buffer* levels, const lh_buffer* signs, lh_buffer* output,
+                                       uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens, uint32_t bits,
+                                       uint32_t token_start, uint32_t ring_capacity);
+LH_API int lh_dequantize_kv_turboquant_into(lh_batch* batch, const lh_buffer* packed, const lh_buffer* norms,
+                                            const lh_buffer* levels, const lh_buffer* signs, lh_buffer* output,
+                                            uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens,
+                                            uint32_t bits, uint32_t token_start, uint32_t ring_capacity);
+/* kernels.rs:5032-5163 hadamard_rotate{,_hf,_fh}_into,
+ * shaders/attention_flash_tq.metal:58-139: per head optional sign flip, FWHT,
+ * 1/sqrt(d), optional sign flip.  f32->f32, f16->f32, f32->f16. */
+LH_API int lh_hadamard_rotate_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs,
+                                   lh_buffer* output, uint32_t head_dim, uint32_t num_heads, int pre_sign,
+                                   int post_sign);
+LH_API int lh_hadamard_rotate_hf_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs,
+                                      lh_buffer* output, uint32_t head_dim, uint32_t num_heads, int pre_sign,
+                                      int post_sign);
+LH_API int lh_hadamard_rotate_fh_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs,
+                                      lh_buffer* output, uint32_t head_dim, uint32_t num_heads, int pre_sign,
+                                      int post_sign);
+/* kernels.rs:5176-5243 flash_attention_tq_into,
+ * shaders/attention_flash_tq.metal:154-274: single-query decode attention
+ * straight from packed codes (no 1/sqrt(d) scale), rq / out [num_q_heads,
+ * head_dim] f32 in rotated space. */
+LH_API int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                      const lh_buffer* k_norms, const lh_buffer* v_codes, const lh_buffer* v_norms,
+                                      const lh_buffer* levels, lh_buffer* out, uint32_t head_dim, uint32_t kv_len,
+                                      uint32_t current_pos, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                      uint32_t window, uint32_t bits, uint32_t ring_capacity);
+/* kernels.rs:5259-5420 flash_attention_tq_prefill{,_tiled}_into,
+ * shaders/attention_flash_tq.metal:290-556: n_rows causal query rows at
+ * positions start_pos..start_pos+n_rows-1; rq / out [n_rows, num_q_heads, head_dim]. */
+LH_API int lh_flash_attention_tq_prefill_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                              const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                              const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                              uint32_t head_dim, uint32_t kv_len, uint32_t start_pos,
+                                              uint32_t n_rows, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                              uint32_t window, uint32_t bits, uint32_t ring_capacity);
+LH_API int lh_flash_attention_tq_prefill_tiled_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                                    const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                                    const lh_buffer* v_norms, const lh_buffer* levels,
+                                                    lh_buffer* out, uint32_t head_dim, uint32_t kv_len,
+                                                    uint32_t start_pos, uint32_t n_rows, uint32_t num_q_heads,
+                                                    uint32_t num_kv_heads, uint32_t window, uint32_t bits,
+                                                    uint32_t ring_capacity);
+/* kernels.rs:5434-5506 flash_attention_tq_batched_into,
+ * shaders/attention_flash_tq.metal:569-690: one query per lane over the by-lane
+ * pool; rq / out [n_lanes, num_q_heads, head_dim]; positions u32[n_lanes]. */
+LH_API int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                              const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                              const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                              const lh_buffer* positions, uint32_t head_dim,
+                                              uint32_t lane_capacity, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                              uint32_t window, uint32_t bits, uint32_t n_lanes,
+                                              uint32_t ring_capacity);
+
+/* ---- FP16-KV split-K decode attention ---------------------------------------
+ * kernels.rs:1397-1557 flash_decoding_into, 1292-1392
+ * flash_attention_windowed_split_into, 1265-1278 flash_split_count;
+ * shaders/flash_decoding.metal:10-189.  q [H, hd], k/v [T, n_kv, hd], out [H, hd], all f16. */
+LH_API int lh_flash_decoding_into(lh_batch* batch, const lh_buffer* q, const lh_buffer* k, const lh_buffer* v,
+                                  lh_buffer* output, uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                  uint32_t num_q_heads, uint32_t num_kv_heads);
+LH_API int lh_flash_attention_windowed_split_into(lh_batch* batch, const lh_buffer* q, const lh_buffer* k,
+                                                  const lh_buffer* v, lh_buffer* output, lh_buffer* partial_max,
+                                                  lh_buffer* partial_sum, lh_buffer* partial_acc, uint32_t head_dim,
+                                                  uint32_t kv_len, uint32_t current_pos, uint32_t num_q_heads,
+                                                  uint32_t num_kv_heads, uint32_t window, uint32_t num_splits);
+LH_API uint32_t lh_flash_split_count(uint32_t eff_seq_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LOCAL_HIP_H */

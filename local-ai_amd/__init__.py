@@ -1,0 +1,468 @@
+"""local-hip: gfx950 (MI355X) decode hot path behind local-metal's kernel-dispatch API.
+
+This package is a thin ctypes mirror of the reference's host-side interface
+(``local_metal::{context::MetalContext, buffer::MetalBuffer,
+batch::CommandBatch, kernels::Kernels, error::Error}``) on top of the C ABI in
+``include/local_hip.h``.  All compute happens in ``liblocal_hip.so`` (hand-written
+HIP kernels); there is no CPU or PyTorch fallback -- if the library is missing or
+no gfx950 device is present the calls raise.
+
+The directory name carries a hyphen, so load it with ``__graft_entry__.load_package()``
+(registers it as ``local_ai_amd``) or ``importlib`` rather than a plain import.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblocal_hip.so")
+
+F16, F32, BF16 = 0, 1, 2
+Q4_0, TQ2_0 = 0, 1
+_DTYPE_SIZE = {F16: 2, F32: 4, BF16: 2}
+
+SMALLM_MAX_M = 8      # local-metal/src/kernels.rs:6155
+BATCHM_MAX_M = 4      # local-metal/src/kernels.rs:6160
+MULTIVEC_MAX_M = 16   # local-metal/src/kernels.rs:6362
+
+
+class Error(Exception):
+    """Mirror of ``local_metal::Error`` (local-metal/src/error.rs:1-32)."""
+    code = -1
+
+
+class NoDevice(Error):
+    code = 1
+
+
+class NoCommandQueue(Error):
+    code = 2
+
+
+class BufferAllocation(Error):
+    code = 3
+
+
+class LibraryCreation(Error):
+    code = 4
+
+
+class PipelineCreation(Error):
+    code = 5
+
+
+class ShaderNotFound(Error):
+    code = 6
+
+
+class CommandBuffer(Error):
+    code = 7
+
+
+class InvalidArgument(Error):
+    code = 8
+
+
+class Io(Error):
+    code = 9
+
+
+_ERRORS = {c.code: c for c in (NoDevice, NoCommandQueue, BufferAllocation, LibraryCreation, PipelineCreation,
+                               ShaderNotFound, CommandBuffer, InvalidArgument, Io)}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Load ``liblocal_hip.so``; raises ``LibraryCreation`` when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise LibraryCreation(f"{LIB_PATH} is missing: run __graft_entry__.build() (make -C local-ai_amd/csrc)")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.lh_last_error.restype = C.c_char_p
+        _lib.lh_version.restype = C.c_char_p
+        _lib.lh_buffer_length.restype = C.c_size_t
+        _lib.lh_buffer_device_ptr.restype = C.c_void_p
+        _lib.lh_context_stream.restype = C.c_void_p
+        for name in ("lh_smallm_max_m", "lh_batchm_max_m", "lh_multivec_max_m", "lh_batch_dispatch_count",
+                     "lh_flash_split_count"):
+            getattr(_lib, name).restype = C.c_uint32
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().lh_last_error().decode("utf-8", "replace")
+        raise _ERRORS.get(rc, Error)(msg)
+
+
+def _u32(v) -> C.c_uint32:
+    return C.c_uint32(int(v))
+
+
+class Context:
+    """``MetalContext`` (local-metal/src/context.rs:31-98): device + one in-order stream."""
+
+    def __init__(self, device_index: int = 0):
+        self._h = C.c_void_p()
+        _check(lib().lh_context_create(C.c_int(device_index), C.byref(self._h)))
+
+    def device_name(self) -> str:
+        buf = C.create_string_buffer(256)
+        _check(lib().lh_context_device_name(self._h, buf, C.c_size_t(256)))
+        return buf.value.decode()
+
+    def compute_units(self) -> int:
+        return int(lib().lh_context_compute_units(self._h))
+
+    def stream(self) -> int:
+        return int(lib().lh_context_stream(self._h) or 0)
+
+    def synchronize(self) -> None:
+        _check(lib().lh_context_synchronize(self._h))
+
+    def close(self) -> None:
+        if self._h:
+            lib().lh_context_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Event:
+    """HIP event on the context stream (device-side timing)."""
+
+    def __init__(self, ctx: Context):
+        self._h = C.c_void_p()
+        _check(lib().lh_event_create(ctx._h, C.byref(self._h)))
+
+    def record(self) -> None:
+        _check(lib().lh_event_record(self._h))
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        _check(lib().lh_event_elapsed_ms(self._h, stop._h, C.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib().lh_event_destroy(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+
+class Buffer:
+    """``MetalBuffer`` (local-metal/src/buffer.rs:17-141) in device memory.
+
+    Host access is an explicit copy (``as_array`` / ``copy_from_bytes``), ordered
+    after the work already enqueued on the context.
+    """
+
+    def __init__(self, handle, ctx, parent=None):
+        self._h = handle
+        self.ctx = ctx
+        self._parent = parent  # keeps the owner of a view alive
+
+    @classmethod
+    def from_slice(cls, ctx: Context, data) -> "Buffer":
+        a = np.ascontiguousarray(data)
+        h = C.c_void_p()
+        _check(lib().lh_buffer_from_bytes(ctx._h, C.c_void_p(a.ctypes.data), C.c_size_t(a.nbytes), C.byref(h)))
+        return cls(h, ctx)
+
+    @classmethod
+    def empty(cls, ctx: Context, byte_len: int) -> "Buffer":
+        h = C.c_void_p()
+        _check(lib().lh_buffer_empty(ctx._h, C.c_size_t(byte_len), C.byref(h)))
+        return cls(h, ctx)
+
+    @classmethod
+    def wrap(cls, ctx: Context, device_ptr: int, byte_len: int, owner=None) -> "Buffer":
+        """Non-owning handle over device memory allocated elsewhere (e.g. a torch tensor)."""
+        h = C.c_void_p()
+        _check(lib().lh_buffer_wrap(ctx._h, C.c_void_p(device_ptr), C.c_size_t(byte_len), C.byref(h)))
+        return cls(h, ctx, parent=owner)
+
+    def view(self, offset: int, byte_len: int) -> "Buffer":
+        h = C.c_void_p()
+        _check(lib().lh_buffer_view(self._h, C.c_size_t(offset), C.c_size_t(byte_len), C.byref(h)))
+        return Buffer(h, self.ctx, parent=self)
+
+    def length(self) -> int:
+        return int(lib().lh_buffer_length(self._h))
+
+    def device_ptr(self) -> int:
+        return int(lib().lh_buffer_device_ptr(self._h) or 0)
+
+    def copy_from_bytes(self, src, offset: int = 0) -> None:
+        a = np.ascontiguousarray(src)
+        _check(lib().lh_buffer_write(self._h, C.c_size_t(offset), C.c_void_p(a.ctypes.data), C.c_size_t(a.nbytes)))
+
+    def as_array(self, dtype, count: int | None = None, offset: int = 0) -> np.ndarray:
+        dt = np.dtype(dtype)
+        if count is None:
+            count = (self.length() - offset) // dt.itemsize
+        out = np.empty(count, dt)
+        _check(lib().lh_buffer_read(self._h, C.c_size_t(offset), C.c_void_p(out.ctypes.data), C.c_size_t(out.nbytes)))
+        return out
+
+    def fill_zero(self) -> None:
+        _check(lib().lh_buffer_fill_zero(self._h))
+
+    def free(self) -> None:
+        if self._h:
+            lib().lh_buffer_free(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class CommandBatch:
+    """``CommandBatch`` (local-metal/src/batch.rs:21-291): dispatches run in encode order."""
+
+    def __init__(self, ctx: Context):
+        self.ctx = ctx
+        self._h = C.c_void_p()
+        _check(lib().lh_batch_new(ctx._h, C.byref(self._h)))
+
+    def dispatch_count(self) -> int:
+        return int(lib().lh_batch_dispatch_count(self._h))
+
+    def blit_copy(self, src: Buffer, src_offset: int, dst: Buffer, dst_offset: int, length: int) -> None:
+        _check(lib().lh_batch_blit_copy(self._h, src._h, C.c_size_t(src_offset), dst._h, C.c_size_t(dst_offset),
+                                        C.c_size_t(length)))
+
+    def commit_and_wait(self) -> None:
+        _check(lib().lh_batch_commit_and_wait(self._h))
+
+    def submit_and_renew(self) -> None:
+        _check(lib().lh_batch_submit_and_renew(self._h))
+
+    def commit_and_renew(self) -> None:
+        _check(lib().lh_batch_commit_and_renew(self._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib().lh_batch_free(self._h)
+                self._h = C.c_void_p()
+        except Exception:
+            pass
+
+
+def _handles(bufs):
+    arr = (C.c_void_p * len(bufs))(*[b._h for b in bufs])
+    return arr
+
+
+class Kernels:
+    """``Kernels`` (local-metal/src/kernels.rs): one method per hot-path dispatch, same
+    names and argument order.  ``*_into`` methods encode into a batch; the others block."""
+
+    SMALLM_MAX_M = SMALLM_MAX_M
+    BATCHM_MAX_M = BATCHM_MAX_M
+    MULTIVEC_MAX_M = MULTIVEC_MAX_M
+
+    def __init__(self, ctx: Context):
+        self.ctx = ctx
+        self._l = lib()
+
+    # -- flags (kernels.rs:6277-6304) --
+    @staticmethod
+    def batchm_enabled() -> bool:
+        return bool(lib().lh_batchm_enabled())
+
+    @staticmethod
+    def mma_enabled() -> bool:
+        return bool(lib().lh_mma_enabled())
+
+    @staticmethod
+    def smallm_enabled() -> bool:
+        return bool(lib().lh_smallm_enabled())
+
+    # -- M = 1 matvec (kernels.rs:5711-6038) --
+    def matvec_q4_0(self, ctx, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_q4_0(ctx._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_q4_0_into(self, batch, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_q4_0_into(batch._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_q4_0_f32out(self, ctx, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_q4_0_f32out(ctx._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_q4_0_f32out_into(self, batch, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_q4_0_f32out_into(batch._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_tq2_0(self, ctx, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_tq2_0(ctx._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_tq2_0_into(self, batch, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_tq2_0_into(batch._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_tq2_0_f32out(self, ctx, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_tq2_0_f32out(ctx._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_tq2_0_f32out_into(self, batch, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec_tq2_0_f32out_into(batch._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_tq2_0_soa_into(self, batch, qs, scales, vector, output, rows, cols):
+        _check(self._l.lh_matvec_tq2_0_soa_into(batch._h, qs._h, scales._h, vector._h, output._h, _u32(rows),
+                                                _u32(cols)))
+
+    def matvec_quant_typed_into(self, batch, fmt, matrix, vector, vector_dtype, output, output_dtype, rows, cols):
+        _check(self._l.lh_matvec_quant_typed_into(batch._h, C.c_int(fmt), matrix._h, vector._h, C.c_int(vector_dtype),
+                                                  output._h, C.c_int(output_dtype), _u32(rows), _u32(cols)))
+
+    def matvec_quant_grouped_into(self, batch, fmt, matrices, vectors, vector_dtype, outputs, output_dtype, rows,
+                                  cols):
+        n = len(matrices)
+        assert len(vectors) == n and len(outputs) == n
+        _check(self._l.lh_matvec_quant_grouped_into(batch._h, C.c_int(fmt), _u32(n), _handles(matrices),
+                                                    _handles(vectors), C.c_int(vector_dtype), _handles(outputs),
+                                                    C.c_int(output_dtype), _u32(rows), _u32(cols)))
+
+    # -- small-M / prefill matmul (kernels.rs:6378-6563, 5517-5568) --
+    def matmul_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
+        _check(self._l.lh_matmul_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
+
+    def matmul_nt_tq2_0_into(self, batch, input, weight, output, m, k, n):
+        _check(self._l.lh_matmul_nt_tq2_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
+
+    def multivec_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
+        _check(self._l.lh_multivec_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
+
+    def multivec_nt_tq2_0_into(self, batch, input, weight, output, m, k, n):
+        _check(self._l.lh_multivec_nt_tq2_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
+
+    def matmul_nt_quant_typed_into(self, batch, fmt, input, input_dtype, weight, output, output_dtype, m, k, n):
+        _check(self._l.lh_matmul_nt_quant_typed_into(batch._h, C.c_int(fmt), input._h, C.c_int(input_dtype),
+                                                     weight._h, output._h, C.c_int(output_dtype), _u32(m), _u32(k),
+                                                     _u32(n)))
+
+    def matmul_nt_into(self, batch, input, weight, output, m, k, n):
+        _check(self._l.lh_matmul_nt_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
+
+    # -- block dequant (qat_recover.rs:23-97) and legacy unpack (kernels.rs:6753-6802) --
+    def dequant_q4_0_into(self, batch, data, byte_offset, output, num_elements):
+        _check(self._l.lh_dequant_q4_0_into(batch._h, data._h, C.c_size_t(byte_offset), output._h,
+                                            C.c_size_t(num_elements)))
+
+    def dequant_tq2_0_into(self, batch, data, byte_offset, output, num_elements):
+        _check(self._l.lh_dequant_tq2_0_into(batch._h, data._h, C.c_size_t(byte_offset), output._h,
+                                             C.c_size_t(num_elements)))
+
+    def tq2_dequant(self, ctx, packed, scales, output, num_elements):
+        _check(self._l.lh_tq2_dequant(ctx._h, packed._h, scales._h, output._h, _u32(num_elements)))
+
+    # -- TurboQuant KV (kernels.rs:4641-5506) --
+    def encode_kv_turboquant(self, ctx, input, levels, signs, packed, norms, head_dim, n_kv_heads, num_tokens, bits,
+                             position, ring_capacity):
+        _check(self._l.lh_encode_kv_turboquant(ctx._h, input._h, levels._h, signs._h, packed._h, norms._h,
+                                               _u32(head_dim), _u32(n_kv_heads), _u32(num_tokens), _u32(bits),
+                                               _u32(position), _u32(ring_capacity)))
+
+    def encode_kv_turboquant_into(self, batch, input, levels, signs, packed, norms, head_dim, n_kv_heads, num_tokens,
+                                  bits, position, ring_capacity):
+        _check(self._l.lh_encode_kv_turboquant_into(batch._h, input._h, levels._h, signs._h, packed._h, norms._h,
+                                                    _u32(head_dim), _u32(n_kv_heads), _u32(num_tokens), _u32(bits),
+                                                    _u32(position), _u32(ring_capacity)))
+
+    def encode_kv_turboquant_batched_into(self, batch, input, levels, signs, packed, norms, positions, head_dim,
+                                          n_kv_heads, lane_capacity, bits, n_lanes, ring_capacity):
+        _check(self._l.lh_encode_kv_turboquant_batched_into(batch._h, input._h, levels._h, signs._h, packed._h,
+                                                            norms._h, positions._h, _u32(head_dim), _u32(n_kv_heads),
+                                                            _u32(lane_capacity), _u32(bits), _u32(n_lanes),
+                                                            _u32(ring_capacity)))
+
+    def dequantize_kv_turboquant(self, ctx, packed, norms, levels, signs, output, head_dim, n_kv_heads, num_tokens,
+                                 bits, token_start, ring_capacity):
+        _check(self._l.lh_dequantize_kv_turboquant(ctx._h, packed._h, norms._h, levels._h, signs._h, output._h,
+                                                   _u32(head_dim), _u32(n_kv_heads), _u32(num_tokens), _u32(bits),
+                                                   _u32(token_start), _u32(ring_capacity)))
+
+    def dequantize_kv_turboquant_into(self, batch, packed, norms, levels, signs, output, head_dim, n_kv_heads,
+                                      num_tokens, bits, token_start, ring_capacity):
+        _check(self._l.lh_dequantize_kv_turboquant_into(batch._h, packed._h, norms._h, levels._h, signs._h, output._h,
+                                                        _u32(head_dim), _u32(n_kv_heads), _u32(num_tokens), _u32(bits),
+                                                        _u32(token_start), _u32(ring_capacity)))
+
+    def hadamard_rotate_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
+        _check(self._l.lh_hadamard_rotate_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
+                                               _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))
+
+    def hadamard_rotate_hf_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
+        _check(self._l.lh_hadamard_rotate_hf_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
+                                                  _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))
+
+    def hadamard_rotate_fh_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
+        _check(self._l.lh_hadamard_rotate_fh_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
+                                                  _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))
+
+    def flash_attention_tq_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim, kv_len,
+                                current_pos, num_q_heads, num_kv_heads, window, bits, ring_capacity):
+        _check(self._l.lh_flash_attention_tq_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h, v_norms._h,
+                                                  levels._h, out._h, _u32(head_dim), _u32(kv_len), _u32(current_pos),
+                                                  _u32(num_q_heads), _u32(num_kv_heads), _u32(window), _u32(bits),
+                                                  _u32(ring_capacity)))
+
+    def flash_attention_tq_prefill_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim,
+                                        kv_len, start_pos, n_rows, num_q_heads, num_kv_heads, window, bits,
+                                        ring_capacity):
+        _check(self._l.lh_flash_attention_tq_prefill_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                          v_norms._h, levels._h, out._h, _u32(head_dim), _u32(kv_len),
+                                                          _u32(start_pos), _u32(n_rows), _u32(num_q_heads),
+                                                          _u32(num_kv_heads), _u32(window), _u32(bits),
+                                                          _u32(ring_capacity)))
+
+    def flash_attention_tq_prefill_tiled_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out,
+                                              head_dim, kv_len, start_pos, n_rows, num_q_heads, num_kv_heads, window,
+                                              bits, ring_capacity):
+        _check(self._l.lh_flash_attention_tq_prefill_tiled_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                                v_norms._h, levels._h, out._h, _u32(head_dim),
+                                                                _u32(kv_len), _u32(start_pos), _u32(n_rows),
+                                                                _u32(num_q_heads), _u32(num_kv_heads), _u32(window),
+                                                                _u32(bits), _u32(ring_capacity)))
+
+    def flash_attention_tq_batched_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions,
+                                        head_dim, lane_capacity, num_q_heads, num_kv_heads, window, bits, n_lanes,
+                                        ring_capacity):
+        _check(self._l.lh_flash_attention_tq_batched_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                          v_norms._h, levels._h, out._h, positions._h, _u32(head_dim),
+                                                          _u32(lane_capacity), _u32(num_q_heads), _u32(num_kv_heads),
+                                                          _u32(window), _u32(bits), _u32(n_lanes),
+                                                          _u32(ring_capacity)))
+
+    # -- FP16-KV split-K decode (kernels.rs:1265-1557) --
+    def flash_split_count(self, eff_seq_len: int) -> int:
+        return int(self._l.lh_flash_split_count(_u32(eff_seq_len)))
+
+    def flash_decoding_into(self, batch, q, k, v, output, head_dim, kv_len, current_pos, num_q_heads, num_kv_heads):
+        _check(self._l.lh_flash_decoding_into(batch._h, q._h, k._h, v._h, output._h, _u32(head_dim), _u32(kv_len),
+                                              _u32(current_pos), _u32(num_q_heads), _u32(num_kv_heads)))
+
+    def flash_attention_windowed_split_into(self, batch, q, k, v, output, partial_max, partial_sum, partial_acc,
+                                            head_dim, kv_len, current_pos, num_q_heads, num_kv_heads, window,
+                                            num_splits):
+        _check(self._l.lh_flash_attention_windowed_split_into(batch._h, q._h, k._h, v._h, output._h, partial_max._h,
+                                                              partial_sum._h, partial_acc._h, _u32(head_dim),
+                                                              _u32(kv_len), _u32(current_pos), _u32(num_q_heads),
+                                                              _u32(num_kv_heads), _u32(window), _u32(num_splits)))
+
+
+from . import synth  # noqa: E402  (synthetic inputs of the measured configurations)
+from .quant_weight import QuantWeight  # noqa: E402
+from .kv_cache import QuantizedKvCache, swa_ring_capacity, kv_bits_from_env, TQ_SEED, DEFAULT_KV_BITS  # noqa: E402

@@ -1,0 +1,123 @@
+// Internal declarations shared by the HIP translation units of liblocal_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/local_hip.h"
+
+struct lh_context {
+    int device;
+    hipStream_t stream;
+    int cu_count;
+    char name[256];
+    // Split-K partial results of the attention kernels: (max, sum, acc[head_dim])
+    // per (query head, split). Allocated once with the context.
+    void* workspace;
+    size_t workspace_bytes;
+};
+
+struct lh_buffer {
+    lh_context* ctx;
+    void* ptr;
+    size_t len;
+    bool owns;
+};
+
+struct lh_batch {
+    lh_context* ctx;
+    uint32_t dispatch_count;
+};
+
+// Records the error text for lh_last_error() and returns `code`.
+int lh_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// Post-launch check: converts a pending HIP launch error into LH_ERR_COMMAND_BUFFER.
+int lh_check_launch(const char* what);
+
+#define LH_HIP_TRY(expr, code, what)                                                        \
+    do {                                                                                    \
+        hipError_t e__ = (expr);                                                            \
+        if (e__ != hipSuccess) return lh_fail((code), "%s: %s", (what), hipGetErrorString(e__)); \
+    } while (0)
+
+#define LH_REQUIRE(cond, ...)                                            \
+    do {                                                                 \
+        if (!(cond)) return lh_fail(LH_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+static inline int lh_need(const lh_buffer* b, size_t bytes, const char* op, const char* name) {
+    if (b == nullptr) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %s buffer is null", op, name);
+    if (b->len < bytes)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %s buffer holds %zu bytes, needs %zu", op, name, b->len, bytes);
+    return LH_OK;
+}
+#define LH_NEED(buf, bytes, op, name)                        \
+    do {                                                     \
+        int r__ = lh_need((buf), (bytes), (op), (name));     \
+        if (r__ != LH_OK) return r__;                        \
+    } while (0)
+
+static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }
+
+// ---- device helpers -------------------------------------------------------
+#define LH_DPP_QUAD_XOR1 0xB1   // quad_perm:[1,0,3,2]
+#define LH_DPP_QUAD_XOR2 0x4E   // quad_perm:[2,3,0,1]
+#define LH_DPP_HALF_MIRROR 0x141
+#define LH_DPP_ROW_MIRROR 0x140
+
+template <int CTRL>
+__device__ __forceinline__ float lh_dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int lh_dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+// Exchange with the lane 16 away (inside each group of 32) and 32 away.
+__device__ __forceinline__ float lh_swap16_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x1F | (16 << 10)));
+}
+__device__ __forceinline__ float lh_swap32_f(float v) {
+    return __shfl_xor(v, 32, 64);
+}
+
+// Sum over aligned groups of `width` lanes (power of two, 1..64); every lane of
+// a group ends with the group's total. Fixed pairing order: deterministic.
+__device__ __forceinline__ float lh_group_sum(float v, int width) {
+    if (width > 1) v += lh_dpp_f<LH_DPP_QUAD_XOR1>(v);
+    if (width > 2) v += lh_dpp_f<LH_DPP_QUAD_XOR2>(v);
+    if (width > 4) v += lh_dpp_f<LH_DPP_HALF_MIRROR>(v);
+    if (width > 8) v += lh_dpp_f<LH_DPP_ROW_MIRROR>(v);
+    if (width > 16) v += lh_swap16_f(v);
+    if (width > 32) v += lh_swap32_f(v);
+    return v;
+}
+__device__ __forceinline__ float lh_group_max(float v, int width) {
+    if (width > 1) v = fmaxf(v, lh_dpp_f<LH_DPP_QUAD_XOR1>(v));
+    if (width > 2) v = fmaxf(v, lh_dpp_f<LH_DPP_QUAD_XOR2>(v));
+    if (width > 4) v = fmaxf(v, lh_dpp_f<LH_DPP_HALF_MIRROR>(v));
+    if (width > 8) v = fmaxf(v, lh_dpp_f<LH_DPP_ROW_MIRROR>(v));
+    if (width > 16) v = fmaxf(v, lh_swap16_f(v));
+    if (width > 32) v = fmaxf(v, lh_swap32_f(v));
+    return v;
+}
+__device__ __forceinline__ int lh_group_sum_i(int v, int width) {
+    if (width > 1) v += lh_dpp_i<LH_DPP_QUAD_XOR1>(v);
+    if (width > 2) v += lh_dpp_i<LH_DPP_QUAD_XOR2>(v);
+    if (width > 4) v += lh_dpp_i<LH_DPP_HALF_MIRROR>(v);
+    if (width > 8) v += lh_dpp_i<LH_DPP_ROW_MIRROR>(v);
+    if (width > 16) v += __builtin_amdgcn_ds_swizzle(v, 0x1F | (16 << 10));
+    if (width > 32) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+__device__ __forceinline__ float lh_h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t lh_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+__device__ __forceinline__ float lh_bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+template <typename T> __device__ __forceinline__ float lh_load_as_f32(const T* p, size_t i);
+template <> __device__ __forceinline__ float lh_load_as_f32<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float lh_load_as_f32<uint16_t>(const uint16_t* p, size_t i) { return lh_h2f(p[i]); }
+
+template <typename T> __device__ __forceinline__ void lh_store_from_f32(T* p, size_t i, float v);
+template <> __device__ __forceinline__ void lh_store_from_f32<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void lh_store_from_f32<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = lh_f2h(v); }

@@ -1,0 +1,675 @@
+// Fused dequant matvec for GGUF Q4_0 / TQ2_0 weights at M = 1 (decode).
+//
+// Stands in for shaders/matvec_quant.metal:65-155 (matvec_q4_0*), 173-312
+// (matvec_tq2_0*), 314-387 (matvec_tq2_0_soa) and their dispatch in
+// local-metal/src/kernels.rs:5588-6038.
+//
+// Design (gfx950, wave64):
+//  * The weight stream is the only HBM traffic that matters.  A "unit" is 64
+//    weights: for TQ2_0 one 16-byte quarter of a 66-byte block, for Q4_0 a pair
+//    of 18-byte blocks (36 bytes, dword aligned).  Each lane owns one unit
+//    column of a row and loads it with 128-bit loads; consecutive lanes cover a
+//    contiguous span, so a wave reads 1-2.3 KB of consecutive bytes per load.
+//  * The activation vector is converted once per workgroup to block fixed point
+//    (per weight block: a float scale and 16- or 24-bit integers split into
+//    signed 8-bit limbs) and kept in registers for the lane's unit column, so
+//    the inner product is exact integer arithmetic on v_dot4_i32_i8:
+//        y = sum_blocks d_b * s_b * (sum_i q_i n_i  -  zp * sum_i n_i)
+//    2-bit / 4-bit codes are isolated with one AND per four weights; no
+//    per-weight shift, convert or float multiply.
+//  * Row sums use DPP / swizzle butterflies inside the wave (fixed pairing
+//    order, so results are bit-reproducible run to run).
+#include "common.hpp"
+#include <cstdlib>
+
+namespace {
+
+constexpr int kWG = 256;          // threads per workgroup (4 waves)
+constexpr int kWaves = kWG / 64;
+constexpr uint32_t kMaxFastCols = 16384;  // 4 unit columns per lane at most
+
+struct MatvecProblem {
+    const uint8_t* matrix;
+    const void* vector;
+    void* output;
+};
+
+template <int L> struct Limb;
+template <> struct Limb<2> { static constexpr float qmax = 32639.0f; };     // 127*256 + 127
+template <> struct Limb<3> { static constexpr float qmax = 8355711.0f; };   // 127*65536 + 127*256 + 127
+
+// ---- activation quantisation into LDS ----------------------------------------
+// xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
+// xs[K/G]: float scale of each group of G elements (G = weight block size).
+template <int L, int G, typename XT>
+__device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs) {
+    const int tid = threadIdx.x;
+    const uint32_t kq = K >> 2;
+    for (uint32_t base = 0; base < K; base += kWG * 8) {
+        const uint32_t e0 = base + tid * 8;
+        const bool valid = e0 < K;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        if (valid) {
+            if constexpr (sizeof(XT) == 4) {
+                const float4 a = *reinterpret_cast<const float4*>(x + e0);
+                const float4 b = *reinterpret_cast<const float4*>(x + e0 + 4);
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else {
+                const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
+                const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    v[2 * i] = lh_h2f((uint16_t)(w[i] & 0xFFFF));
+                    v[2 * i + 1] = lh_h2f((uint16_t)(w[i] >> 16));
+                }
+            }
+        }
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+        m = lh_group_max(m, G / 8);
+        const float inv = m > 0.0f ? Limb<L>::qmax / m : 0.0f;
+        uint32_t packed[L][2];
+#pragma unroll
+        for (int l = 0; l < L; l++) packed[l][0] = packed[l][1] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float r = rintf(v[i] * inv);
+            r = fminf(fmaxf(r, -Limb<L>::qmax), Limb<L>::qmax);
+            int n = (int)r;
+#pragma unroll
+            for (int l = 0; l < L; l++) {
+                int limb;
+                if (l == L - 1) limb = n;                       // top limb: what is left, fits a signed byte
+                else { limb = (int)(int8_t)(n & 0xFF); n = (n - limb) >> 8; }
+                packed[l][i >> 2] |= (uint32_t)(limb & 0xFF) << (8 * (i & 3));
+            }
+        }
+        if (valid) {
+#pragma unroll
+            for (int l = 0; l < L; l++)
+                *reinterpret_cast<uint2*>(&xq[l * kq + (e0 >> 2)]) = make_uint2(packed[l][0], packed[l][1]);
+            if ((e0 & (G - 1)) == 0) xs[e0 / G] = m * (1.0f / Limb<L>::qmax);
+        }
+    }
+}
+
+// ---- per-lane activation registers for one unit column -------------------------
+template <int FMT, int L>
+struct UnitX {
+    uint32_t xl[L][4][4];   // [limb][run of 16 elements][dword of 4 elements]
+    float scale[2];         // Q4_0: the unit's two blocks; TQ2_0: [0] only (pre-divided by 16)
+    int nsum[2];            // zero-point term: Q4_0 8*sum(n) per block; TQ2_0 16*sum(n) of the unit
+};
+
+template <int FMT, int L>
+__device__ __forceinline__ void load_unit_x(UnitX<FMT, L>& ux, uint32_t ucol, uint32_t K, const uint32_t* xq, const float* xs) {
+    const uint32_t kq = K >> 2;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        uint32_t eb;
+        if constexpr (FMT == LH_TQ2_0) {
+            const uint32_t b = ucol >> 2, a = ucol & 3;
+            eb = b * 256 + (a >> 1) * 128 + r * 32 + (a & 1) * 16;   // shaders/matvec_quant.metal:15-17
+        } else {
+            eb = ucol * 64 + r * 16;                                   // low nibbles then high nibbles of each block
+        }
+#pragma unroll
+        for (int l = 0; l < L; l++) {
+            const uint4 q = *reinterpret_cast<const uint4*>(&xq[l * kq + (eb >> 2)]);
+            ux.xl[l][r][0] = q.x; ux.xl[l][r][1] = q.y; ux.xl[l][r][2] = q.z; ux.xl[l][r][3] = q.w;
+        }
+    }
+    int s[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        int tot = 0;
+#pragma unroll
+        for (int l = L - 1; l >= 0; l--) {
+            int t = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) t = __builtin_amdgcn_sdot4((int)ux.xl[l][r][k], 0x01010101, t, false);
+            tot = (tot << 8) + t;
+        }
+        s[r] = tot;
+    }
+    if constexpr (FMT == LH_TQ2_0) {
+        ux.scale[0] = xs[ucol >> 2] * 0.0625f;
+        ux.scale[1] = 0.0f;
+        ux.nsum[0] = (s[0] + s[1] + s[2] + s[3]) << 4;
+        ux.nsum[1] = 0;
+    } else {
+        ux.scale[0] = xs[2 * ucol];
+        ux.scale[1] = xs[2 * ucol + 1];
+        ux.nsum[0] = (s[0] + s[1]) << 3;
+        ux.nsum[1] = (s[2] + s[3]) << 3;
+    }
+}
+
+// ---- weight unit in registers -----------------------------------------------------
+template <int FMT> struct UnitW;
+template <> struct UnitW<LH_TQ2_0> { uint4 q; uint32_t d; };
+template <> struct UnitW<LH_Q4_0> { uint4 a, b; uint32_t c; };
+
+// Weight bytes are read through pointers in the global address space (the
+// problem descriptors are loaded from memory, so the compiler cannot infer it).
+typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+__device__ __forceinline__ uint4 ld16_align2(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
+    const u32x4_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint4 ld16_align4(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(4))) u32x4_a4;
+    const u32x4_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a4*>(p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// The caller passes an in-range (row, ucol) for every lane, so the loads are
+// unconditional; lanes without work carry zero activations instead.
+template <int FMT>
+__device__ __forceinline__ void load_unit_w(UnitW<FMT>& w, gptr_t row, uint32_t ucol) {
+    if constexpr (FMT == LH_TQ2_0) {
+        gptr_t blk = row + (size_t)(ucol >> 2) * 66;
+        w.q = ld16_align2(blk + (ucol & 3) * 16);
+        // only quarter 0 needs d; the other three lanes re-read their own quarter's first half-word
+        w.d = *reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>(blk + ((ucol & 3) == 0 ? 64 : (ucol & 3) * 16));
+    } else {
+        gptr_t p = row + (size_t)ucol * 36;
+        w.a = ld16_align4(p); w.b = ld16_align4(p + 16);
+        w.c = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t*>(p + 32);
+    }
+}
+
+template <int L>
+__device__ __forceinline__ int combine_limbs(const int (&acc)[L]) {
+    int t = acc[L - 1];
+#pragma unroll
+    for (int l = L - 2; l >= 0; l--) t = (t << 8) + acc[l];
+    return t;
+}
+
+// Contribution of one unit to its row: d * s * (sum q n - zp sum n).
+template <int FMT, int L>
+__device__ __forceinline__ float unit_dot(const UnitW<FMT>& w, const UnitX<FMT, L>& ux) {
+    if constexpr (FMT == LH_TQ2_0) {
+        const uint32_t wv[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
+        int A[L], B[L], Cq[L];
+#pragma unroll
+        for (int l = 0; l < L; l++) A[l] = B[l] = Cq[l] = 0;
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const uint32_t v = wv[m], t = v >> 2;
+            const int f0 = (int)(v & 0x03030303u), f1 = (int)(t & 0x03030303u);
+            const int f2 = (int)(t & 0x0C0C0C0Cu), f3 = (int)(t & 0x30303030u);   // 4x and 16x the code
+#pragma unroll
+            for (int l = 0; l < L; l++) {
+                A[l] = __builtin_amdgcn_sdot4(f0, (int)ux.xl[l][0][m], A[l], false);
+                A[l] = __builtin_amdgcn_sdot4(f1, (int)ux.xl[l][1][m], A[l], false);
+                B[l] = __builtin_amdgcn_sdot4(f2, (int)ux.xl[l][2][m], B[l], false);
+                Cq[l] = __builtin_amdgcn_sdot4(f3, (int)ux.xl[l][3][m], Cq[l], false);
+            }
+        }
+        int T[L];
+#pragma unroll
+        for (int l = 0; l < L; l++) T[l] = (A[l] << 4) + (B[l] << 2) + Cq[l];   // 16 * sum(code * n)
+        const int i16 = combine_limbs<L>(T) - ux.nsum[0];                          // 16 * sum((code-1) * n)
+        const int dbits = __builtin_amdgcn_update_dpp(0, (int)w.d, 0x00, 0xF, 0xF, true);  // quad lane 0 holds d
+        return (float)i16 * (lh_h2f((uint16_t)dbits) * ux.scale[0]);
+    } else {
+        const uint32_t r[9] = {w.a.x, w.a.y, w.a.z, w.a.w, w.b.x, w.b.y, w.b.z, w.b.w, w.c};
+        // dwords: [d0|q0 q1] [q2..5] [q6..9] [q10..13] [q14 q15|d1] [16 quant bytes of block 1]
+        uint32_t q[2][4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) q[0][k] = __builtin_amdgcn_alignbyte(r[k + 1], r[k], 2);
+#pragma unroll
+        for (int k = 0; k < 4; k++) q[1][k] = r[5 + k];
+        const float d[2] = {lh_h2f((uint16_t)(r[0] & 0xFFFF)), lh_h2f((uint16_t)(r[4] >> 16))};
+        float p = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int acc[L];
+#pragma unroll
+            for (int l = 0; l < L; l++) acc[l] = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int lo = (int)(q[h][k] & 0x0F0F0F0Fu), hi = (int)((q[h][k] >> 4) & 0x0F0F0F0Fu);
+#pragma unroll
+                for (int l = 0; l < L; l++) {
+                    acc[l] = __builtin_amdgcn_sdot4(lo, (int)ux.xl[l][2 * h][k], acc[l], false);
+                    acc[l] = __builtin_amdgcn_sdot4(hi, (int)ux.xl[l][2 * h + 1][k], acc[l], false);
+                }
+            }
+            const int iq = combine_limbs<L>(acc) - ux.nsum[h];                     // sum((q-8) * n)
+            p += (float)iq * (d[h] * ux.scale[h]);
+        }
+        return p;
+    }
+}
+
+template <int FMT> __host__ __device__ constexpr int steps_in_flight(int npos) {
+    return FMT == LH_TQ2_0 ? (npos == 1 ? 8 : (npos == 2 ? 4 : 2)) : (npos == 1 ? 4 : (npos == 2 ? 2 : 1));
+}
+
+// One launch serves `count` problems of the same shape (count == 1 for the plain matvec).
+template <int FMT, int L, int NPOS, typename XT, typename YT>
+__global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, uint32_t count,
+                                                             uint32_t rows, uint32_t K, uint32_t lpr_log2,
+                                                             uint32_t steps_per_wg) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int G = FMT == LH_TQ2_0 ? 256 : 32;
+    constexpr int U = steps_in_flight<FMT>(NPOS);
+    uint32_t* xq = reinterpret_cast<uint32_t*>(lds);
+    float* xs = reinterpret_cast<float*>(lds + (size_t)L * K);
+
+    const uint32_t upr = K >> 6;                                  // unit columns per row
+    const uint32_t row_bytes = FMT == LH_TQ2_0 ? (K >> 8) * 66 : (K >> 5) * 18;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lpr = 1u << lpr_log2;                          // lanes per row (NPOS == 1)
+    const uint32_t rpw = NPOS == 1 ? 64u >> lpr_log2 : 1u;        // rows per wave step
+    const uint32_t rsub = NPOS == 1 ? (uint32_t)lane >> lpr_log2 : 0u;
+    const uint32_t col0 = NPOS == 1 ? ((uint32_t)lane & (lpr - 1)) : (uint32_t)lane;
+    const uint32_t steps_per_problem = (rows + rpw - 1) / rpw;
+    const uint64_t total_steps = (uint64_t)steps_per_problem * count;
+    uint64_t g0 = (uint64_t)blockIdx.x * steps_per_wg;
+    const uint64_t g1 = g0 + steps_per_wg < total_steps ? g0 + steps_per_wg : total_steps;
+
+    UnitX<FMT, L> ux[NPOS];
+    const void* staged_vector = nullptr;
+    while (g0 < g1) {
+        const uint32_t prob = (uint32_t)(g0 / steps_per_problem);
+        const uint32_t s_begin = (uint32_t)(g0 - (uint64_t)prob * steps_per_problem);
+        const uint64_t seg_end64 = (uint64_t)(prob + 1) * steps_per_problem;
+        const uint32_t s_end = (uint32_t)((g1 < seg_end64 ? g1 : seg_end64) - (uint64_t)prob * steps_per_problem);
+        const MatvecProblem pb = problems[prob];
+        // this wave's contiguous share of [s_begin, s_end)
+        const uint32_t nseg = s_end - s_begin;
+        const uint32_t per_wave = (nseg + kWaves - 1) / kWaves;
+        uint32_t st = s_begin + wave * per_wave;
+        uint32_t st_end = st + per_wave < s_end ? st + per_wave : s_end;
+        if (st > s_end) st = s_end;
+
+        if (pb.vector != staged_vector) {
+            __syncthreads();   // every wave is done reading the previous vector's limbs
+            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs);
+            __syncthreads();
+#pragma unroll
+            for (int p = 0; p < NPOS; p++) {
+                const uint32_t ucol = col0 + 64u * p;
+                load_unit_x<FMT, L>(ux[p], ucol < upr ? ucol : 0u, K, xq, xs);
+                if (ucol >= upr) {   // a lane without a unit column contributes exactly zero
+#pragma unroll
+                    for (int l = 0; l < L; l++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+#pragma unroll
+                            for (int k = 0; k < 4; k++) ux[p].xl[l][r][k] = 0;
+                    ux[p].scale[0] = ux[p].scale[1] = 0.0f;
+                    ux[p].nsum[0] = ux[p].nsum[1] = 0;
+                }
+            }
+            staged_vector = pb.vector;
+        }
+        YT* y = static_cast<YT*>(pb.output);
+        gptr_t mat = (gptr_t)pb.matrix;
+        const uint32_t last_row = rows - 1;
+        const int red_width = NPOS == 1 ? (int)lpr : 64;
+        const bool writer = NPOS == 1 ? (((uint32_t)lane & (lpr - 1)) == 0) : lane == 0;
+
+        for (; st < st_end; st += U) {
+            UnitW<FMT> w[U][NPOS];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                uint32_t row = (st + u) * rpw + rsub;     // steps past the end re-read the last row (result dropped)
+                row = row < last_row ? row : last_row;
+                gptr_t rp = mat + (size_t)row * row_bytes;
+#pragma unroll
+                for (int p = 0; p < NPOS; p++) {
+                    const uint32_t ucol = col0 + 64u * p;
+                    load_unit_w<FMT>(w[u][p], rp, ucol < upr ? ucol : 0u);
+                }
+            }
+            float part[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                part[u] = 0.0f;
+#pragma unroll
+                for (int p = 0; p < NPOS; p++) part[u] += unit_dot<FMT, L>(w[u][p], ux[p]);
+            }
+            // butterfly over the lanes of a row, all U rows per level
+            if (red_width > 1) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_dpp_f<LH_DPP_QUAD_XOR1>(part[u]);
+            }
+            if (red_width > 2) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_dpp_f<LH_DPP_QUAD_XOR2>(part[u]);
+            }
+            if (red_width > 4) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_dpp_f<LH_DPP_HALF_MIRROR>(part[u]);
+            }
+            if (red_width > 8) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_dpp_f<LH_DPP_ROW_MIRROR>(part[u]);
+            }
+            if (red_width > 16) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_swap16_f(part[u]);
+            }
+            if (red_width > 32) {
+#pragma unroll
+                for (int u = 0; u < U; u++) part[u] += lh_swap32_f(part[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t row = (st + u) * rpw + rsub;
+                if (writer && (st + u) < st_end && row < rows) lh_store_from_f32<YT>(y, row, part[u]);
+            }
+        }
+        g0 = (uint64_t)prob * steps_per_problem + s_end;
+    }
+}
+
+// Fallback for shapes / alignments the fast path does not take (Q4_0 with an
+// odd block count per row, cols > 16384, odd base addresses): one wave per
+// row, byte loads, fp32 FMA on the dequantised value d*(q-zp).
+template <int FMT, typename XT, typename YT>
+__global__ __launch_bounds__(256) void matvec_quant_generic_kernel(const uint8_t* __restrict__ matrix, const XT* __restrict__ x,
+                                                                  YT* __restrict__ y, uint32_t rows, uint32_t K) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    float acc = 0.0f;
+    if constexpr (FMT == LH_Q4_0) {
+        const uint32_t nb = K >> 5;
+        const uint8_t* rp = matrix + (size_t)row * nb * 18;
+        for (uint32_t i = lane; i < nb * 16; i += 64) {     // one quant byte (2 weights) per lane per trip
+            const uint32_t b = i >> 4, j = i & 15;
+            const uint8_t* bp = rp + (size_t)b * 18;
+            const float d = lh_h2f((uint16_t)(bp[0] | (bp[1] << 8)));
+            const uint32_t q = bp[2 + j];
+            acc += d * ((float)(q & 15) - 8.0f) * lh_load_as_f32<XT>(x, b * 32 + j);
+            acc += d * ((float)(q >> 4) - 8.0f) * lh_load_as_f32<XT>(x, b * 32 + 16 + j);
+        }
+    } else {
+        const uint32_t nb = K >> 8;
+        const uint8_t* rp = matrix + (size_t)row * nb * 66;
+        for (uint32_t i = lane; i < nb * 64; i += 64) {     // one qs byte (4 weights) per lane per trip
+            const uint32_t b = i >> 6, j = i & 63;
+            const uint8_t* bp = rp + (size_t)b * 66;
+            const float d = lh_h2f((uint16_t)(bp[64] | (bp[65] << 8)));
+            const uint32_t q = bp[j];
+            const uint32_t e = b * 256 + (j >> 5) * 128 + (j & 31);
+#pragma unroll
+            for (int l = 0; l < 4; l++)
+                acc += d * ((float)((q >> (2 * l)) & 3) - 1.0f) * lh_load_as_f32<XT>(x, e + l * 32);
+        }
+    }
+    acc = lh_group_sum(acc, 64);
+    if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
+}
+
+// SoA TQ2_0 (64-byte aligned qs rows + separate f16 scales): same arithmetic as
+// the generic path with 16-byte loads.
+template <typename XT, typename YT>
+__global__ __launch_bounds__(256) void matvec_tq2_0_soa_kernel(const uint8_t* __restrict__ qs, const uint16_t* __restrict__ scales,
+                                                              const XT* __restrict__ x, YT* __restrict__ y, uint32_t rows, uint32_t K) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint32_t nb = K >> 8;
+    float acc = 0.0f;
+    for (uint32_t u = lane; u < nb * 4; u += 64) {            // 16 qs bytes per lane per trip
+        const uint32_t b = u >> 2, a = u & 3;
+        const uint4 v = *reinterpret_cast<const uint4*>(qs + ((size_t)row * nb + b) * 64 + a * 16);
+        const float d = lh_h2f(scales[(size_t)row * nb + b]);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t e0 = b * 256 + (a >> 1) * 128 + (a & 1) * 16;
+        float s = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 4; m++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t q = (w[m] >> (8 * k)) & 0xFF;
+#pragma unroll
+                for (int l = 0; l < 4; l++)
+                    s += ((float)((q >> (2 * l)) & 3) - 1.0f) * lh_load_as_f32<XT>(x, e0 + l * 32 + m * 4 + k);
+            }
+        acc += d * s;
+    }
+    acc = lh_group_sum(acc, 64);
+    if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
+}
+
+int x_limbs() {
+    static int v = [] {
+        const char* e = getenv("LOCAL_HIP_X_LIMBS");
+        return (e && e[0] == '3') ? 3 : 2;
+    }();
+    return v;
+}
+
+int wg_per_cu() {
+    static int v = [] {
+        const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU");
+        int n = e ? atoi(e) : 2;
+        return n < 1 ? 1 : (n > 8 ? 8 : n);
+    }();
+    return v;
+}
+
+struct LaunchGeom {
+    uint32_t npos, lpr_log2, rpw, grid, steps_per_wg;
+    size_t lds_bytes;
+};
+
+LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_count, int L) {
+    LaunchGeom g{};
+    const uint32_t upr = K / 64;
+    g.npos = (upr + 63) / 64;
+    uint32_t lpr = 1; g.lpr_log2 = 0;
+    if (g.npos == 1) { while (lpr < upr) { lpr <<= 1; g.lpr_log2++; } }
+    else { lpr = 64; g.lpr_log2 = 6; }
+    g.rpw = g.npos == 1 ? 64 / lpr : 1;
+    const uint64_t steps = (uint64_t)((rows + g.rpw - 1) / g.rpw) * count;
+    // two workgroups per CU when there is enough work; never fewer than one step per wave
+    uint64_t want = (steps + kWaves - 1) / kWaves;
+    const uint64_t cap = (uint64_t)cu_count * wg_per_cu();
+    if (want > cap) want = cap;
+    if (want < 1) want = 1;
+    g.steps_per_wg = (uint32_t)((steps + want - 1) / want);
+    g.grid = (uint32_t)((steps + g.steps_per_wg - 1) / g.steps_per_wg);
+    const uint32_t G = fmt == LH_TQ2_0 ? 256 : 32;
+    g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4;
+    return g;
+}
+
+template <int FMT, int L, int NPOS>
+int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, uint32_t count, lh_dtype xt, lh_dtype yt, uint32_t rows,
+                 uint32_t K, const LaunchGeom& g) {
+#define LH_LAUNCH(XT, YT)                                                                                              \
+    hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream, \
+                       dev_problems, count, rows, K, g.lpr_log2, g.steps_per_wg)
+    if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
+    else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
+    else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
+    else LH_LAUNCH(float, uint16_t);
+#undef LH_LAUNCH
+    return lh_check_launch("matvec_quant");
+}
+
+template <int FMT, int L>
+int launch_npos(lh_context* ctx, const MatvecProblem* p, uint32_t count, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K,
+                const LaunchGeom& g) {
+    switch (g.npos) {
+        case 1: return launch_typed<FMT, L, 1>(ctx, p, count, xt, yt, rows, K, g);
+        case 2: return launch_typed<FMT, L, 2>(ctx, p, count, xt, yt, rows, K, g);
+        case 3: return launch_typed<FMT, L, 3>(ctx, p, count, xt, yt, rows, K, g);
+        default: return launch_typed<FMT, L, 4>(ctx, p, count, xt, yt, rows, K, g);
+    }
+}
+
+template <int FMT>
+int launch_generic(lh_context* ctx, const uint8_t* m, const void* x, void* y, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K) {
+    const dim3 grid((rows + 3) / 4), block(256);
+#define LH_LAUNCH(XT, YT) \
+    hipLaunchKernelGGL((matvec_quant_generic_kernel<FMT, XT, YT>), grid, block, 0, ctx->stream, m, (const XT*)x, (YT*)y, rows, K)
+    if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
+    else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
+    else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
+    else LH_LAUNCH(float, uint16_t);
+#undef LH_LAUNCH
+    return lh_check_launch("matvec_quant_generic");
+}
+
+const char* op_name(lh_quant fmt) { return fmt == LH_Q4_0 ? "matvec_q4_0" : "matvec_tq2_0"; }
+
+bool fast_path_ok(lh_quant fmt, const void* matrix, const void* vector, uint32_t K) {
+    if (K > kMaxFastCols) return false;
+    if (((uintptr_t)vector & 15) != 0) return false;
+    if (fmt == LH_Q4_0) return (K % 64) == 0 && ((uintptr_t)matrix & 3) == 0;
+    return ((uintptr_t)matrix & 1) == 0;
+}
+
+// Validates and launches `count` matvecs of one shape.
+int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
+                    const lh_buffer* const* vectors, lh_dtype xt, lh_buffer* const* outputs, lh_dtype yt, uint32_t rows,
+                    uint32_t cols, const char* op) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (xt == LH_BF16 || yt == LH_BF16) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: bf16 vectors are not supported", op);
+    // kernels.rs:5720-5724, 5857-5861: block alignment is checked before anything is encoded.
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    if (cols % blk != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: cols %u not /%u", op, cols, blk);
+    if (count == 0 || rows == 0 || cols == 0) return LH_OK;
+    lh_context* ctx = batch->ctx;
+    const size_t wbytes = (size_t)rows * (cols / blk) * (fmt == LH_Q4_0 ? 18 : 66);
+    bool fast = true;
+    for (uint32_t i = 0; i < count; i++) {
+        LH_NEED(matrices[i], wbytes, op, "matrix");
+        LH_NEED(vectors[i], (size_t)cols * lh_dtype_size(xt), op, "vector");
+        LH_NEED(outputs[i], (size_t)rows * lh_dtype_size(yt), op, "output");
+        fast = fast && fast_path_ok(fmt, matrices[i]->ptr, vectors[i]->ptr, cols);
+    }
+    if (!fast) {
+        for (uint32_t i = 0; i < count; i++) {
+            int r = fmt == LH_Q4_0
+                        ? launch_generic<LH_Q4_0>(ctx, (const uint8_t*)matrices[i]->ptr, vectors[i]->ptr, outputs[i]->ptr, xt, yt, rows, cols)
+                        : launch_generic<LH_TQ2_0>(ctx, (const uint8_t*)matrices[i]->ptr, vectors[i]->ptr, outputs[i]->ptr, xt, yt, rows, cols);
+            if (r != LH_OK) return r;
+            batch->dispatch_count++;
+        }
+        return LH_OK;
+    }
+    // Problem descriptors live in the context's descriptor ring in device memory.
+    const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
+    if (desc_bytes > ctx->workspace_bytes / 4)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u problems exceed the descriptor area", op, count);
+    MatvecProblem stack_desc[8];
+    MatvecProblem* host_desc = count <= 8 ? stack_desc : (MatvecProblem*)malloc(desc_bytes);
+    if (!host_desc) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", desc_bytes);
+    for (uint32_t i = 0; i < count; i++) {
+        host_desc[i].matrix = (const uint8_t*)matrices[i]->ptr;
+        host_desc[i].vector = vectors[i]->ptr;
+        host_desc[i].output = outputs[i]->ptr;
+    }
+    // The descriptor area is the top quarter of the workspace; the copy is stream
+    // ordered, so it cannot overtake a kernel that still reads the previous set.
+    MatvecProblem* dev_desc = (MatvecProblem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
+    hipError_t e = hipMemcpyAsync(dev_desc, host_desc, desc_bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (count > 8) free(host_desc);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
+    const int L = x_limbs();
+    const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L);
+    int r;
+    if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, count, xt, yt, rows, cols, g)
+                                   : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, count, xt, yt, rows, cols, g);
+    else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, count, xt, yt, rows, cols, g)
+                    : launch_npos<LH_TQ2_0, 3>(ctx, dev_desc, count, xt, yt, rows, cols, g);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+int matvec_one(lh_batch* batch, lh_quant fmt, const lh_buffer* m, const lh_buffer* x, lh_dtype xt, lh_buffer* y, lh_dtype yt,
+               uint32_t rows, uint32_t cols) {
+    const lh_buffer* ms[1] = {m};
+    const lh_buffer* xs[1] = {x};
+    lh_buffer* ys[1] = {y};
+    return matvec_dispatch(batch, fmt, 1, ms, xs, xt, ys, yt, rows, cols, op_name(fmt));
+}
+
+int matvec_blocking(lh_context* ctx, lh_quant fmt, const lh_buffer* m, const lh_buffer* x, lh_dtype xt, lh_buffer* y, lh_dtype yt,
+                    uint32_t rows, uint32_t cols) {
+    if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: context is null", op_name(fmt));
+    lh_batch b{ctx, 0};
+    int r = matvec_one(&b, fmt, m, x, xt, y, yt, rows, cols);
+    if (r != LH_OK) return r;
+    return lh_batch_commit_and_wait(&b);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lh_matvec_q4_0(lh_context* ctx, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_blocking(ctx, LH_Q4_0, m, x, LH_F16, y, LH_F16, rows, cols);
+}
+int lh_matvec_q4_0_into(lh_batch* b, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_one(b, LH_Q4_0, m, x, LH_F16, y, LH_F16, rows, cols);
+}
+int lh_matvec_q4_0_f32out(lh_context* ctx, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_blocking(ctx, LH_Q4_0, m, x, LH_F16, y, LH_F32, rows, cols);
+}
+int lh_matvec_q4_0_f32out_into(lh_batch* b, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_one(b, LH_Q4_0, m, x, LH_F16, y, LH_F32, rows, cols);
+}
+int lh_matvec_tq2_0(lh_context* ctx, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_blocking(ctx, LH_TQ2_0, m, x, LH_F16, y, LH_F16, rows, cols);
+}
+int lh_matvec_tq2_0_into(lh_batch* b, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_one(b, LH_TQ2_0, m, x, LH_F16, y, LH_F16, rows, cols);
+}
+int lh_matvec_tq2_0_f32out(lh_context* ctx, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_blocking(ctx, LH_TQ2_0, m, x, LH_F16, y, LH_F32, rows, cols);
+}
+int lh_matvec_tq2_0_f32out_into(lh_batch* b, const lh_buffer* m, const lh_buffer* x, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    return matvec_one(b, LH_TQ2_0, m, x, LH_F16, y, LH_F32, rows, cols);
+}
+
+int lh_matvec_quant_typed_into(lh_batch* b, lh_quant fmt, const lh_buffer* m, const lh_buffer* x, lh_dtype xt, lh_buffer* y,
+                               lh_dtype yt, uint32_t rows, uint32_t cols) {
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
+    return matvec_one(b, fmt, m, x, xt, y, yt, rows, cols);
+}
+
+int lh_matvec_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* const* ms, const lh_buffer* const* xs,
+                                 lh_dtype xt, lh_buffer* const* ys, lh_dtype yt, uint32_t rows, uint32_t cols) {
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
+    if (count && (!ms || !xs || !ys)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null problem arrays", op_name(fmt));
+    return matvec_dispatch(b, fmt, count, ms, xs, xt, ys, yt, rows, cols, op_name(fmt));
+}
+
+int lh_matvec_tq2_0_soa_into(lh_batch* b, const lh_buffer* qs, const lh_buffer* scales, const lh_buffer* x, lh_buffer* y,
+                             uint32_t rows, uint32_t cols) {
+    // kernels.rs:5929-5933
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0_soa: batch is null");
+    if (cols % 256 != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0_soa: cols %u not /256", cols);
+    if (rows == 0 || cols == 0) return LH_OK;
+    const size_t nblk = (size_t)rows * (cols / 256);
+    LH_NEED(qs, nblk * 64, "matvec_tq2_0_soa", "qs");
+    LH_NEED(scales, nblk * 2, "matvec_tq2_0_soa", "scales");
+    LH_NEED(x, (size_t)cols * 2, "matvec_tq2_0_soa", "vector");
+    LH_NEED(y, (size_t)rows * 2, "matvec_tq2_0_soa", "output");
+    LH_REQUIRE(((uintptr_t)qs->ptr & 15) == 0, "matvec_tq2_0_soa: qs must be 16-byte aligned");
+    hipLaunchKernelGGL((matvec_tq2_0_soa_kernel<uint16_t, uint16_t>), dim3((rows + 3) / 4), dim3(256), 0, b->ctx->stream,
+                       (const uint8_t*)qs->ptr, (const uint16_t*)scales->ptr, (const uint16_t*)x->ptr, (uint16_t*)y->ptr, rows, cols);
+    int r = lh_check_launch("matvec_tq2_0_soa");
+    if (r == LH_OK) b->dispatch_count++;
+    return r;
+}
+
+}  // extern "C"

@@ -1,0 +1,279 @@
+// Context, buffer and command-batch plumbing of the C ABI: the HIP stand-ins for
+// local-metal/src/{context.rs, buffer.rs, batch.rs, error.rs}.
+#include "common.hpp"
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+static thread_local char g_last_error[512] = "";
+
+static const char* status_prefix(int code) {
+    switch (code) {  // Display strings of local_metal::Error (error.rs:1-32)
+        case LH_ERR_NO_DEVICE: return "No Metal device found";
+        case LH_ERR_NO_COMMAND_QUEUE: return "Failed to create command queue";
+        case LH_ERR_BUFFER_ALLOCATION: return "Buffer allocation failed";
+        case LH_ERR_LIBRARY_CREATION: return "Failed to create Metal library: ";
+        case LH_ERR_PIPELINE_CREATION: return "Failed to create pipeline state: ";
+        case LH_ERR_SHADER_NOT_FOUND: return "Shader function not found: ";
+        case LH_ERR_COMMAND_BUFFER: return "Command buffer error: ";
+        case LH_ERR_INVALID_ARGUMENT: return "Invalid argument: ";
+        case LH_ERR_IO: return "I/O error: ";
+        default: return "";
+    }
+}
+
+int lh_fail(int code, const char* fmt, ...) {
+    char msg[384];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(msg, sizeof msg, fmt, ap);
+    va_end(ap);
+    if (code == LH_ERR_NO_DEVICE) snprintf(g_last_error, sizeof g_last_error, "No HIP device found (%s)", msg);
+    else if (code == LH_ERR_BUFFER_ALLOCATION) snprintf(g_last_error, sizeof g_last_error, "%s (%s)", status_prefix(code), msg);
+    else snprintf(g_last_error, sizeof g_last_error, "%s%s", status_prefix(code), msg);
+    return code;
+}
+
+int lh_check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s launch failed: %s", what, hipGetErrorString(e));
+    return LH_OK;
+}
+
+extern "C" {
+
+const char* lh_last_error(void) { return g_last_error; }
+const char* lh_version(void) { return "local-hip 0.1 (gfx950)"; }
+
+int lh_context_create(int device_index, lh_context** out) {
+    if (!out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "context_create: out is null");
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return lh_fail(LH_ERR_NO_DEVICE, "hipGetDeviceCount found none");
+    if (device_index < 0 || device_index >= n) return lh_fail(LH_ERR_NO_DEVICE, "device index %d of %d", device_index, n);
+    LH_HIP_TRY(hipSetDevice(device_index), LH_ERR_NO_DEVICE, "hipSetDevice");
+    hipDeviceProp_t prop;
+    LH_HIP_TRY(hipGetDeviceProperties(&prop, device_index), LH_ERR_NO_DEVICE, "hipGetDeviceProperties");
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return lh_fail(LH_ERR_LIBRARY_CREATION, "kernels are built for gfx950 only, device is %s", prop.gcnArchName);
+    lh_context* ctx = new (std::nothrow) lh_context();
+    if (!ctx) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_context));
+    ctx->device = device_index;
+    ctx->cu_count = prop.multiProcessorCount;
+    snprintf(ctx->name, sizeof ctx->name, "%s (%s)", prop.name, prop.gcnArchName);
+    if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+        delete ctx;
+        return lh_fail(LH_ERR_NO_COMMAND_QUEUE, "hipStreamCreate");
+    }
+    ctx->workspace_bytes = (size_t)64 << 20;
+    if (hipMalloc(&ctx->workspace, ctx->workspace_bytes) != hipSuccess) {
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: attention workspace", (size_t)64 << 20);
+    }
+    *out = ctx;
+    return LH_OK;
+}
+
+void lh_context_destroy(lh_context* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->workspace);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+int lh_context_device_name(const lh_context* ctx, char* dst, size_t dst_len) {
+    if (!ctx || !dst || dst_len == 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "device_name: null argument");
+    snprintf(dst, dst_len, "%s", ctx->name);
+    return LH_OK;
+}
+int lh_context_compute_units(const lh_context* ctx) { return ctx ? ctx->cu_count : 0; }
+void* lh_context_stream(const lh_context* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
+
+int lh_context_synchronize(lh_context* ctx) {
+    if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "synchronize: context is null");
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+// ---- events -----------------------------------------------------------------
+struct lh_event { lh_context* ctx; hipEvent_t ev; };
+
+int lh_event_create(lh_context* ctx, lh_event** out) {
+    if (!ctx || !out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "event_create: null argument");
+    lh_event* e = new (std::nothrow) lh_event();
+    if (!e) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_event));
+    e->ctx = ctx;
+    if (hipEventCreate(&e->ev) != hipSuccess) { delete e; return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: hipEventCreate"); }
+    *out = e;
+    return LH_OK;
+}
+void lh_event_destroy(lh_event* ev) { if (ev) { (void)hipEventDestroy(ev->ev); delete ev; } }
+int lh_event_record(lh_event* ev) {
+    if (!ev) return lh_fail(LH_ERR_INVALID_ARGUMENT, "event_record: event is null");
+    hipError_t e = hipEventRecord(ev->ev, ev->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: event_record: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+int lh_event_elapsed_ms(lh_event* start, lh_event* stop, float* ms) {
+    if (!start || !stop || !ms) return lh_fail(LH_ERR_INVALID_ARGUMENT, "event_elapsed_ms: null argument");
+    hipError_t e = hipEventSynchronize(stop->ev);
+    if (e == hipSuccess) e = hipEventElapsedTime(ms, start->ev, stop->ev);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: event_elapsed_ms: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+// ---- buffers ----------------------------------------------------------------
+static int new_buffer(lh_context* ctx, size_t len, lh_buffer** out) {
+    if (!ctx || !out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer: null argument");
+    *out = nullptr;
+    lh_buffer* b = new (std::nothrow) lh_buffer();
+    if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
+    b->ctx = ctx; b->len = len; b->owns = true; b->ptr = nullptr;
+    // Room for one 16-byte over-read past the end keeps vector loads of a
+    // partly filled last unit inside the allocation.
+    hipError_t e = hipMalloc(&b->ptr, (len ? len : 1) + 64);
+    if (e != hipSuccess) { delete b; return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: %s", len, hipGetErrorString(e)); }
+    *out = b;
+    return LH_OK;
+}
+
+int lh_buffer_empty(lh_context* ctx, size_t len, lh_buffer** out) {
+    int r = new_buffer(ctx, len, out);
+    if (r != LH_OK) return r;
+    hipError_t e = hipMemsetAsync((*out)->ptr, 0, len + 64, ctx->stream);
+    if (e != hipSuccess) { lh_buffer_free(*out); *out = nullptr; return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: %s", len, hipGetErrorString(e)); }
+    return LH_OK;
+}
+
+int lh_buffer_from_bytes(lh_context* ctx, const void* src, size_t len, lh_buffer** out) {
+    if (!src && len) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_from_bytes: src is null");
+    int r = new_buffer(ctx, len, out);
+    if (r != LH_OK) return r;
+    hipError_t e = hipMemsetAsync((char*)(*out)->ptr + len, 0, 64, ctx->stream);
+    if (e == hipSuccess && len) e = hipMemcpyAsync((*out)->ptr, src, len, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);  // src may be freed by the caller on return
+    if (e != hipSuccess) { lh_buffer_free(*out); *out = nullptr; return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: %s", len, hipGetErrorString(e)); }
+    return LH_OK;
+}
+
+int lh_buffer_view(lh_buffer* parent, size_t offset, size_t len, lh_buffer** out) {
+    if (!parent || !out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_view: null argument");
+    if (offset > parent->len || len > parent->len - offset)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_view: range %zu+%zu exceeds %zu", offset, len, parent->len);
+    lh_buffer* b = new (std::nothrow) lh_buffer();
+    if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
+    b->ctx = parent->ctx; b->ptr = (char*)parent->ptr + offset; b->len = len; b->owns = false;
+    *out = b;
+    return LH_OK;
+}
+
+int lh_buffer_wrap(lh_context* ctx, void* device_ptr, size_t len, lh_buffer** out) {
+    if (!ctx || !out || (!device_ptr && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_wrap: null argument");
+    lh_buffer* b = new (std::nothrow) lh_buffer();
+    if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
+    b->ctx = ctx; b->ptr = device_ptr; b->len = len; b->owns = false;
+    *out = b;
+    return LH_OK;
+}
+
+void lh_buffer_free(lh_buffer* buf) {
+    if (!buf) return;
+    if (buf->owns && buf->ptr) {
+        (void)hipStreamSynchronize(buf->ctx->stream);
+        (void)hipFree(buf->ptr);
+    }
+    delete buf;
+}
+
+size_t lh_buffer_length(const lh_buffer* buf) { return buf ? buf->len : 0; }
+void* lh_buffer_device_ptr(const lh_buffer* buf) { return buf ? buf->ptr : nullptr; }
+
+int lh_buffer_write(lh_buffer* buf, size_t offset, const void* src, size_t len) {
+    if (!buf || (!src && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_write: null argument");
+    if (offset > buf->len || len > buf->len - offset)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_write: range %zu+%zu exceeds %zu", offset, len, buf->len);
+    if (!len) return LH_OK;
+    hipError_t e = hipMemcpyAsync((char*)buf->ptr + offset, src, len, hipMemcpyHostToDevice, buf->ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(buf->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: buffer_write: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+int lh_buffer_read(const lh_buffer* buf, size_t offset, void* dst, size_t len) {
+    if (!buf || (!dst && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_read: null argument");
+    if (offset > buf->len || len > buf->len - offset)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_read: range %zu+%zu exceeds %zu", offset, len, buf->len);
+    if (!len) return LH_OK;
+    hipError_t e = hipMemcpyAsync(dst, (const char*)buf->ptr + offset, len, hipMemcpyDeviceToHost, buf->ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(buf->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: buffer_read: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+int lh_buffer_fill_zero(lh_buffer* buf) {
+    if (!buf) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_fill_zero: buffer is null");
+    if (!buf->len) return LH_OK;
+    hipError_t e = hipMemsetAsync(buf->ptr, 0, buf->len, buf->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: buffer_fill_zero: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+// ---- command batch ------------------------------------------------------------
+int lh_batch_new(lh_context* ctx, lh_batch** out) {
+    if (!ctx || !out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "batch_new: null argument");
+    lh_batch* b = new (std::nothrow) lh_batch();
+    if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_batch));
+    b->ctx = ctx; b->dispatch_count = 0;
+    *out = b;
+    return LH_OK;
+}
+void lh_batch_free(lh_batch* batch) { delete batch; }
+uint32_t lh_batch_dispatch_count(const lh_batch* batch) { return batch ? batch->dispatch_count : 0; }
+
+int lh_batch_blit_copy(lh_batch* batch, const lh_buffer* src, size_t src_offset, lh_buffer* dst, size_t dst_offset, size_t len) {
+    // batch.rs:46-57: out-of-bounds ranges are rejected before encoding.
+    if (!batch || !src || !dst) return lh_fail(LH_ERR_INVALID_ARGUMENT, "blit_copy: null argument");
+    if (src_offset > src->len || len > src->len - src_offset || dst_offset > dst->len || len > dst->len - dst_offset)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "blit_copy: range out of bounds (src %zu+%zu of %zu, dst %zu+%zu of %zu)",
+                       src_offset, len, src->len, dst_offset, len, dst->len);
+    if (!len) return LH_OK;
+    hipError_t e = hipMemcpyAsync((char*)dst->ptr + dst_offset, (const char*)src->ptr + src_offset, len,
+                                  hipMemcpyDeviceToDevice, batch->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: blit_copy: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+int lh_batch_commit_and_wait(lh_batch* batch) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "commit_and_wait: batch is null");
+    hipError_t e = hipStreamSynchronize(batch->ctx->stream);
+    batch->dispatch_count = 0;
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+int lh_batch_submit_and_renew(lh_batch* batch) {
+    // Work is already on the stream as it is encoded; nothing to flush.
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "submit_and_renew: batch is null");
+    batch->dispatch_count = 0;
+    return LH_OK;
+}
+int lh_batch_commit_and_renew(lh_batch* batch) { return lh_batch_commit_and_wait(batch); }
+
+// kernels.rs:6155-6304
+static int env_flag_default_on(const char* name) {
+    const char* v = getenv(name);
+    return !(v && strcmp(v, "0") == 0);
+}
+uint32_t lh_smallm_max_m(void) { return 8; }
+uint32_t lh_batchm_max_m(void) { return 4; }
+uint32_t lh_multivec_max_m(void) { return 16; }
+int lh_batchm_enabled(void) { static int v = env_flag_default_on("LOCAL_AI_BATCHM"); return v; }
+int lh_mma_enabled(void) { static int v = env_flag_default_on("LOCAL_AI_MMA"); return v; }
+int lh_smallm_enabled(void) { static int v = env_flag_default_on("LOCAL_AI_SMALLM"); return v; }
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+"""``QuantizedKvCache`` (local-engine/src/kv_cache/quant_cache.rs:73-700): TurboQuant KV cache
+in device memory with ring addressing for sliding-window layers."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import Buffer, InvalidArgument, Kernels, lib
+
+TQ_SEED = 0x7459C0DE       # quant_cache.rs:30
+DEFAULT_KV_BITS = 2        # quant_cache.rs:37
+MAX_PREFILL_CHUNK = 256    # quant_cache.rs:43
+
+
+def swa_ring_capacity(window: int, max_positions: int) -> int:
+    """quant_cache.rs:48-54."""
+    f = lib().lh_swa_ring_capacity
+    f.restype = C.c_size_t
+    return int(f(C.c_size_t(window), C.c_size_t(max_positions)))
+
+
+def kv_bits_from_env() -> int:
+    """quant_cache.rs:60-66 (LOCAL_AI_KV_QUANT = tq2 | tq3 | tq4)."""
+    f = lib().lh_kv_bits_from_env
+    f.restype = C.c_uint32
+    return int(f())
+
+
+def turboquant_levels(dim: int, bits: int) -> np.ndarray:
+    out = np.empty(1 << bits, np.float32)
+    rc = lib().lh_turboquant_levels(C.c_uint32(dim), C.c_uint32(bits), C.c_void_p(out.ctypes.data))
+    if rc:
+        raise InvalidArgument(lib().lh_last_error().decode())
+    return out
+
+
+def turboquant_signs(dim: int, seed: int = TQ_SEED) -> np.ndarray:
+    out = np.empty(dim, np.float32)
+    rc = lib().lh_turboquant_signs(C.c_uint32(dim), C.c_uint64(seed), C.c_void_p(out.ctypes.data))
+    if rc:
+        raise InvalidArgument(lib().lh_last_error().decode())
+    return out
+
+
+def code_bytes(dim: int, bits: int) -> int:
+    f = lib().lh_turboquant_code_bytes
+    f.restype = C.c_uint32
+    return int(f(C.c_uint32(dim), C.c_uint32(bits)))
+
+
+class QuantizedKvCache:
+    def __init__(self, ctx, n_kv_heads: int, head_dim: int, max_positions: int, bits: int = DEFAULT_KV_BITS,
+                 physical_positions: int | None = None, sliding_window: int = 0):
+        """quant_cache.rs:182-229 new_with_bits_and_ring."""
+        if not 2 <= bits <= 4:
+            raise InvalidArgument(f"TurboQuant bits must be 2..=4, got {bits}")
+        if head_dim & (head_dim - 1) or head_dim > 512 or head_dim == 0:
+            raise InvalidArgument(f"TurboQuant head_dim must be a power of two <= 512, got {head_dim}")
+        if physical_positions is None:
+            physical_positions = max_positions
+        physical_positions = max(min(physical_positions, max_positions), 1)
+        if physical_positions < max_positions and physical_positions < sliding_window + MAX_PREFILL_CHUNK - 1:
+            raise InvalidArgument(f"ring capacity {physical_positions} too small for window {sliding_window} "
+                                  f"+ prefill slack {MAX_PREFILL_CHUNK - 1}")
+        self.ctx = ctx
+        self.n_kv_heads, self.head_dim, self.bits = n_kv_heads, head_dim, bits
+        self.max_positions, self.physical_positions = max_positions, physical_positions
+        self._cb = code_bytes(head_dim, bits)
+        slots = physical_positions * n_kv_heads
+        self.levels = Buffer.from_slice(ctx, turboquant_levels(head_dim, bits))
+        self.signs = Buffer.from_slice(ctx, turboquant_signs(head_dim, TQ_SEED))
+        self.keys_q = Buffer.empty(ctx, max(slots * self._cb, 1))
+        self.values_q = Buffer.empty(ctx, max(slots * self._cb, 1))
+        self.key_norms = Buffer.empty(ctx, max(slots, 1) * 2)
+        self.value_norms = Buffer.empty(ctx, max(slots, 1) * 2)
+
+    def is_ringed(self) -> bool:
+        return self.physical_positions < self.max_positions
+
+    def ring_capacity(self) -> int:
+        """quant_cache.rs:258-264: physical rows for a ring, 0 for absolute addressing."""
+        return self.physical_positions if self.is_ringed() else 0
+
+    def code_bytes(self) -> int:
+        return self._cb
+
+    def reset(self) -> None:
+        """quant_cache.rs:367-380."""
+        for b in (self.keys_q, self.values_q, self.key_norms, self.value_norms):
+            b.fill_zero()
+
+    def write_kv_gpu_into(self, batch, kernels: Kernels, k_src: Buffer, v_src: Buffer, position: int, n_rows: int):
+        """quant_cache.rs:391-444."""
+        if position + n_rows > self.max_positions:
+            raise InvalidArgument(f"KV write [{position}..{position + n_rows}) exceeds capacity {self.max_positions}")
+        for src, codes, norms in ((k_src, self.keys_q, self.key_norms), (v_src, self.values_q, self.value_norms)):
+            kernels.encode_kv_turboquant_into(batch, src, self.levels, self.signs, codes, norms, self.head_dim,
+                                              self.n_kv_heads, n_rows, self.bits, position, self.ring_capacity())
+
+    def dequantize_into(self, ctx, kernels: Kernels, k_out: Buffer, v_out: Buffer, seq_len: int, token_start: int):
+        """quant_cache.rs:490-532."""
+        for codes, norms, out in ((self.keys_q, self.key_norms, k_out), (self.values_q, self.value_norms, v_out)):
+            kernels.dequantize_kv_turboquant(ctx, codes, norms, self.levels, self.signs, out, self.head_dim,
+                                             self.n_kv_heads, seq_len, self.bits, token_start, self.ring_capacity())
+
+    def fused_attention_into(self, batch, kernels: Kernels, q: Buffer, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                             seq_len: int, current_pos: int, n_q_heads: int, window: int):
+        """quant_cache.rs:548-598: rotate q, attend over codes, inverse-rotate to f16."""
+        hd = self.head_dim
+        kernels.hadamard_rotate_hf_into(batch, q, self.signs, rq, hd, n_q_heads, True, False)
+        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
+                                        self.levels, vacc, hd, seq_len, current_pos, n_q_heads, self.n_kv_heads,
+                                        window, self.bits, self.ring_capacity())
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
+
+    def fused_attention_batch_into(self, batch, kernels: Kernels, q: Buffer, rq: Buffer, vacc: Buffer,
+                                   attn_out: Buffer, kv_len: int, start_pos: int, n_rows: int, n_q_heads: int,
+                                   window: int, tiled: bool = True):
+        """quant_cache.rs:620-700."""
+        hd = self.head_dim
+        vecs = n_rows * n_q_heads
+        kernels.hadamard_rotate_hf_into(batch, q, self.signs, rq, hd, vecs, True, False)
+        fn = kernels.flash_attention_tq_prefill_tiled_into if tiled else kernels.flash_attention_tq_prefill_into
+        fn(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms, self.levels, vacc, hd, kv_len,
+           start_pos, n_rows, n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, vecs, False, True)

@@ -1,0 +1,77 @@
+"""``QuantWeight`` (local-engine/src/layer.rs:18-282): a format-tagged weight in device
+memory that routes matvec / matmul calls to the kernel for its block format."""
+from __future__ import annotations
+
+import numpy as np
+
+from . import Q4_0, TQ2_0, F16, F32, BF16, Buffer, InvalidArgument, Kernels
+
+_BLOCK = {Q4_0: (32, 18), TQ2_0: (256, 66)}
+
+
+class QuantWeight:
+    def __init__(self, buf: Buffer, ty: int, rows: int, cols: int):
+        self.buf, self.ty, self.rows, self.cols = buf, ty, rows, cols
+
+    @classmethod
+    def quantized(cls, buf: Buffer, ty: int, rows: int, cols: int) -> "QuantWeight":
+        """layer.rs:42-66: only Q4_0 and TQ2_0 have device kernels; cols must be block aligned."""
+        if ty not in _BLOCK:
+            raise InvalidArgument(f"QuantWeight: no device kernel for {ty!r}")
+        block = _BLOCK[ty][0]
+        if cols % block != 0:
+            raise InvalidArgument(f"QuantWeight: cols {cols} not a multiple of block {block}")
+        return cls(buf, ty, rows, cols)
+
+    @classmethod
+    def from_bytes(cls, ctx, raw, ty: int, rows: int, cols: int) -> "QuantWeight":
+        """Verbatim GGUF payload upload (local-engine/src/pipeline/init_gemma4_qat.rs:62-66)."""
+        raw = np.ascontiguousarray(raw, np.uint8).reshape(-1)
+        block, nbytes = _BLOCK[ty]
+        if raw.size != rows * (cols // block) * nbytes:
+            raise InvalidArgument(f"QuantWeight: payload of {raw.size} bytes does not match {rows}x{cols}")
+        return cls.quantized(Buffer.from_slice(ctx, raw), ty, rows, cols)
+
+    def device_bytes(self) -> int:
+        return self.buf.length()
+
+    def row_bytes(self) -> int:
+        block, nbytes = _BLOCK[self.ty]
+        return (self.cols // block) * nbytes
+
+    # layer.rs:120-161: out[rows] = self x x[cols]
+    def matvec_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer) -> None:
+        if self.ty == Q4_0:
+            kernels.matvec_q4_0_into(batch, self.buf, x, out, self.rows, self.cols)
+        else:
+            kernels.matvec_tq2_0_into(batch, self.buf, x, out, self.rows, self.cols)
+
+    def matvec_f32out_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer) -> None:
+        if self.ty == Q4_0:
+            kernels.matvec_q4_0_f32out_into(batch, self.buf, x, out, self.rows, self.cols)
+        else:
+            kernels.matvec_tq2_0_f32out_into(batch, self.buf, x, out, self.rows, self.cols)
+
+    def matvec_typed_into(self, batch, kernels: Kernels, x: Buffer, x_dtype: int, out: Buffer, out_dtype: int) -> None:
+        kernels.matvec_quant_typed_into(batch, self.ty, self.buf, x, x_dtype, out, out_dtype, self.rows, self.cols)
+
+    # layer.rs:218-246: out[m, rows] = x[m, cols] . self^T
+    def matmul_nt_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer, m: int) -> None:
+        if self.ty == Q4_0:
+            kernels.matmul_nt_q4_0_into(batch, x, self.buf, out, m, self.cols, self.rows)
+        else:
+            kernels.matmul_nt_tq2_0_into(batch, x, self.buf, out, m, self.cols, self.rows)
+
+    def matmul_nt_typed_into(self, batch, kernels: Kernels, x: Buffer, x_dtype: int, out: Buffer, out_dtype: int,
+                             m: int) -> None:
+        kernels.matmul_nt_quant_typed_into(batch, self.ty, x, x_dtype, self.buf, out, out_dtype, m, self.cols,
+                                           self.rows)
+
+    # layer.rs:269-281: one row dequantised to f16 (embedding gather); row clamps to the last row
+    def dequant_row_into(self, batch, kernels: Kernels, row: int, out: Buffer) -> None:
+        row = min(row, self.rows - 1)
+        off = row * self.row_bytes()
+        if self.ty == Q4_0:
+            kernels.dequant_q4_0_into(batch, self.buf, off, out, self.cols)
+        else:
+            kernels.dequant_tq2_0_into(batch, self.buf, off, out, self.cols)

@@ -17,3 +17,16 @@ def oracle():
     from oracle import oracle as orc
     orc.build()
     return orc
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    import __graft_entry__ as ge
+    return ge.load_package()
+
+
+@pytest.fixture(scope="session")
+def gpu(pkg):
+    """(ctx, kernels) on device 0. The library must be built already: there is no fallback."""
+    ctx = pkg.Context(0)
+    return ctx, pkg.Kernels(ctx)

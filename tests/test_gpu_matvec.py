@@ -1,0 +1,107 @@
+"""GPU parity of the M = 1 fused dequant matvec against the CPU oracle, through the C ABI.
+Mirrors local-metal/src/kernels.rs:9233-9423 (matvec_*_matches_cpu_reference), 9703-9760."""
+import numpy as np
+import pytest
+
+import refgen
+
+pytestmark = pytest.mark.gpu
+
+
+def run_matvec(pkg, gpu, fmt, raw, x, rows, cols, xdt, ydt):
+    ctx, kernels = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    w = pkg.QuantWeight.from_bytes(ctx, raw, ty, rows, cols)
+    xb = pkg.Buffer.from_slice(ctx, x.astype(np.float32) if xdt == pkg.F32 else x.astype(np.float16))
+    yb = pkg.Buffer.empty(ctx, rows * (4 if ydt == pkg.F32 else 2))
+    batch = pkg.CommandBatch(ctx)
+    w.matvec_typed_into(batch, kernels, xb, xdt, yb, ydt)
+    assert batch.dispatch_count() >= 1
+    batch.commit_and_wait()
+    return yb.as_array(np.float32 if ydt == pkg.F32 else np.float16, rows).astype(np.float32)
+
+
+REF_SHAPES = [("q4_0", 5, 96), ("q4_0", 7, 64), ("tq2_0", 4, 512), ("tq2_0", 6, 256),
+              ("q4_0", 33, 1536), ("tq2_0", 37, 1536), ("q4_0", 100, 6144), ("tq2_0", 100, 6144),
+              ("q4_0", 16, 12288), ("tq2_0", 16, 12288), ("tq2_0", 3, 16384), ("q4_0", 3, 16384),
+              ("tq2_0", 2, 32768), ("q4_0", 2, 20480), ("q4_0", 9, 32), ("tq2_0", 1, 256)]
+
+
+@pytest.mark.parametrize("fmt,rows,cols", REF_SHAPES)
+def test_matvec_reference_payloads(pkg, gpu, oracle, fmt, rows, cols):
+    """Reference generators (d in [0.01, 0.11] / [0.05, 0.25], TQ2 codes include 3), f16 x."""
+    print(f"case {fmt} {rows}x{cols}", flush=True)
+    raw = refgen.q4_0_payload(rows, cols, 0xBEEF) if fmt == "q4_0" else refgen.tq2_0_payload(rows, cols, 0xBEEF)
+    expand = oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32
+    v16, v32 = refgen.test_vector(cols)
+    want = oracle.matvec_f32(expand(raw, rows, cols), v32)
+    got32 = run_matvec(pkg, gpu, fmt, raw, v16, rows, cols, pkg.F16, pkg.F32)
+    refgen.assert_close(got32, want, 1e-3, f"{fmt} f32out")      # reference tolerance is 0.01
+    got16 = run_matvec(pkg, gpu, fmt, raw, v16, rows, cols, pkg.F16, pkg.F16)
+    refgen.assert_close(got16, want, 2e-3, f"{fmt} f16out")      # reference tolerance is 0.02 (f16 store)
+    gotf = run_matvec(pkg, gpu, fmt, raw, v32, rows, cols, pkg.F32, pkg.F32)
+    refgen.assert_close(gotf, want, 1e-3, f"{fmt} f32in")
+
+
+@pytest.mark.parametrize("fmt,rows,cols", [("q4_0", 2048, 2048), ("tq2_0", 8192, 2048), ("tq2_0", 2048, 8192),
+                                           ("q4_0", 256, 2048)])
+def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
+    """The measured configurations: fp32 x, fp32 y, against the reference CPU path
+    (block dequant to f16 then a sequential f32 dot), max normalised error <= 1e-3."""
+    print(f"case {fmt} {rows}x{cols}", flush=True)
+    g = pkg.synth.rng(1 if fmt == "q4_0" else 2, rows)
+    raw = pkg.synth.weights(fmt, rows, cols, g)
+    x = pkg.synth.activations(1, cols, g)[0]
+    want = oracle.matvec_quant_ref(fmt, raw, x, rows, cols, threads=8)
+    got = run_matvec(pkg, gpu, fmt, raw, x, rows, cols, pkg.F32, pkg.F32)
+    err = refgen.assert_close(got, want, 1e-3, fmt)
+    # attribution: against an f64 accumulation of the unrounded weights the error is far smaller
+    expand = oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32
+    y64 = oracle.matvec_f64(expand(raw, rows, cols), x)
+    e64 = float(np.max(np.abs(got - y64) / np.maximum(np.abs(y64), 1.0)))
+    print(f"{fmt} {rows}x{cols}: err vs CPU path {err:.2e}, vs f64 {e64:.2e}")
+    assert e64 <= 3e-4   # 16-bit block-fixed-point activations; 24-bit with LOCAL_HIP_X_LIMBS=3
+
+
+def test_matvec_rejects_misaligned_cols(pkg, gpu):
+    """kernels.rs:9752-9760 quant_kernels_reject_misaligned_cols."""
+    ctx, kernels = gpu
+    b = pkg.Buffer.empty(ctx, 4096)
+    batch = pkg.CommandBatch(ctx)
+    with pytest.raises(pkg.InvalidArgument, match=r"matvec_q4_0: cols 100 not /32"):
+        kernels.matvec_q4_0_into(batch, b, b, b, 4, 100)
+    with pytest.raises(pkg.InvalidArgument, match=r"matvec_tq2_0: cols 128 not /256"):
+        kernels.matvec_tq2_0_into(batch, b, b, b, 4, 128)
+    with pytest.raises(pkg.InvalidArgument, match=r"matvec_q4_0: cols 33 not /32"):
+        kernels.matvec_q4_0(ctx, b, b, b, 4, 33)
+    with pytest.raises(pkg.InvalidArgument, match="needs"):
+        kernels.matvec_q4_0_into(batch, b, b, b, 4096, 4096)       # buffers too small for the shape
+    assert batch.dispatch_count() == 0
+
+
+def test_matvec_linearity_and_grouped(pkg, gpu, oracle):
+    """Size-independent properties at full size: y(ax) = a y(x) for a power of two (exact in
+    block fixed point), and a grouped launch equals the separate launches bit for bit."""
+    ctx, kernels = gpu
+    rows, cols = 8192, 2048
+    g = pkg.synth.rng(2, 7)
+    raws = [pkg.synth.weights("tq2_0", rows, cols, g) for _ in range(3)]
+    xs = [pkg.synth.activations(1, cols, g)[0] for _ in range(3)]
+    ws = [pkg.QuantWeight.from_bytes(ctx, r, pkg.TQ2_0, rows, cols) for r in raws]
+    xb = [pkg.Buffer.from_slice(ctx, x) for x in xs]
+    yb = [pkg.Buffer.empty(ctx, rows * 4) for _ in range(3)]
+    yg = [pkg.Buffer.empty(ctx, rows * 4) for _ in range(3)]
+    batch = pkg.CommandBatch(ctx)
+    for w, x, y in zip(ws, xb, yb):
+        w.matvec_typed_into(batch, kernels, x, pkg.F32, y, pkg.F32)
+    kernels.matvec_quant_grouped_into(batch, pkg.TQ2_0, [w.buf for w in ws], xb, pkg.F32, yg, pkg.F32, rows, cols)
+    batch.commit_and_wait()
+    for i in range(3):
+        a, b = yb[i].as_array(np.float32, rows), yg[i].as_array(np.float32, rows)
+        assert np.array_equal(a, b)
+        refgen.assert_close(a, oracle.matvec_quant_ref("tq2_0", raws[i], xs[i], rows, cols, threads=8), 1e-3)
+    x2 = pkg.Buffer.from_slice(ctx, xs[0] * np.float32(4.0))
+    y2 = pkg.Buffer.empty(ctx, rows * 4)
+    ws[0].matvec_typed_into(batch, kernels, x2, pkg.F32, y2, pkg.F32)
+    batch.commit_and_wait()
+    assert np.array_equal(y2.as_array(np.float32, rows), yb[0].as_array(np.float32, rows) * np.float32(4.0))
