@@ -1,0 +1,365 @@
+// Fused flash-decoding attention straight from packed TurboQuant codes.
+//
+// Stands in for shaders/attention_flash_tq.metal:154-690 (flash_attention_tq,
+// _prefill, _prefill_tiled, _batched) and their dispatch in
+// local-metal/src/kernels.rs:5176-5506.
+//
+// Semantics kept from the reference: seq_len = min(kv_len, pos + 1); the window
+// starts at pos + 1 - window when that is positive; logical position t lives in
+// physical row t % ring_capacity when a ring is used; logit_t = f32(norm_k[t]) *
+// sum_i rq_i * levels[Kcode_{t,i}] with no 1/sqrt(d) factor; the output is the
+// softmax-weighted sum of f32(norm_v[t]) * levels[Vcode_{t,i}], normalised, in
+// rotated space; an empty range gives zeros.
+//
+// Structure here (different from the reference's one-threadgroup-per-head scan):
+//  * split-K: the position range of one query is cut into `num_splits` chunks, one
+//    workgroup each; every workgroup serves ALL query heads that share the KV
+//    head (GQA), so each cached position is read and decoded once, not once per
+//    query head;
+//  * per workgroup the partial (max, sum, acc[head_dim]) per head goes to a
+//    workspace and a second small kernel does the log-sum-exp merge; with one
+//    split the workgroup writes the final result itself.
+#include "common.hpp"
+#include <algorithm>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerWG = kThreads / 64;
+constexpr int kMaxDpl = 8;        // head_dim 512 over 64 lanes
+constexpr int kHeadsPerPass = 8;  // query heads served together from one decode of a position
+constexpr int kPosBatch = 8;      // positions whose loads a wave keeps in flight together
+
+enum Mode : uint32_t { kSingle = 0, kPrefill = 1, kBatched = 2 };
+
+struct AttnParams {
+    uint32_t head_dim, bits, code_bytes;
+    uint32_t num_q_heads, num_kv_heads;
+    uint32_t kv_len;          // single / prefill
+    uint32_t pos0;            // single: current_pos; prefill: start_pos
+    uint32_t window, ring_capacity, lane_capacity;
+    uint32_t mode, num_queries, num_splits;
+};
+
+__device__ __forceinline__ void query_range(const AttnParams& p, const uint32_t* positions, uint32_t qi, uint32_t& lo, uint32_t& hi,
+                                            uint32_t& lane_base) {
+    uint32_t pos, kv_len;
+    if (p.mode == kBatched) { pos = positions[qi]; kv_len = pos + 1u; lane_base = qi * p.lane_capacity; }
+    else { pos = p.pos0 + (p.mode == kPrefill ? qi : 0u); kv_len = p.kv_len; lane_base = 0; }
+    hi = kv_len < pos + 1u ? kv_len : pos + 1u;
+    lo = (p.window > 0u && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
+    if (lo > hi) lo = hi;
+}
+
+// The lane's bit window of one code record: `dpl` codes starting at bit lane*dpl*bits.
+__device__ __forceinline__ uint32_t load_window(const uint8_t* rec, uint32_t byte0, uint32_t nbytes) {
+    uint32_t v = 0;
+    for (uint32_t i = 0; i < nbytes; i++) v |= (uint32_t)rec[byte0 + i] << (8 * i);
+    return v;
+}
+
+// Sum each of 8 per-lane values over the 64 lanes; lane l ends with the total of value (l & 7).
+// (Halving butterfly: 7 exchanges instead of 8 full reductions.)
+__device__ __forceinline__ float reduce8(const float (&v)[8], int lane) {
+    float a[4];
+    const bool b0 = lane & 1;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float keep = b0 ? v[2 * j + 1] : v[2 * j];
+        const float give = b0 ? v[2 * j] : v[2 * j + 1];
+        a[j] = keep + lh_dpp_f<LH_DPP_QUAD_XOR1>(give);
+    }
+    float b[2];
+    const bool b1 = lane & 2;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const float keep = b1 ? a[2 * j + 1] : a[2 * j];
+        const float give = b1 ? a[2 * j] : a[2 * j + 1];
+        b[j] = keep + lh_dpp_f<LH_DPP_QUAD_XOR2>(give);
+    }
+    const bool b2 = lane & 4;
+    const float keep = b2 ? b[1] : b[0];
+    const float give = b2 ? b[0] : b[1];
+    // row_half_mirror pairs lane i with 7-i: the partner's bit 2 differs and its low two bits are
+    // complemented, so route through an xor-4 exchange instead.
+    float c = keep + __shfl_xor(give, 4, 64);
+    c += __shfl_xor(c, 8, 64);
+    c += lh_swap16_f(c);
+    c += lh_swap32_f(c);
+    return c;   // total of value index ((lane&1) | (lane&2) | (lane&4)) -> lane & 7
+}
+
+__global__ __launch_bounds__(kThreads) void attention_tq_split_kernel(
+    const float* __restrict__ rq, const uint8_t* __restrict__ k_codes, const uint16_t* __restrict__ k_norms,
+    const uint8_t* __restrict__ v_codes, const uint16_t* __restrict__ v_norms, const float* __restrict__ levels,
+    const uint32_t* __restrict__ positions, float* __restrict__ out, float* __restrict__ ws, AttnParams p) {
+    __shared__ float lds_levels[16];
+    __shared__ float lds_m[kWavesPerWG][kHeadsPerPass];
+    __shared__ float lds_l[kWavesPerWG][kHeadsPerPass];
+    extern __shared__ __align__(16) float lds_acc[];   // [wave][head][head_dim]
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t split = blockIdx.x;
+    const uint32_t qi = blockIdx.y / p.num_kv_heads, kvh = blockIdx.y - qi * p.num_kv_heads;
+    const uint32_t hd = p.head_dim, bits = p.bits;
+    const uint32_t group = p.num_q_heads / p.num_kv_heads;           // query heads per KV head
+    const uint32_t dpl = hd >= 64 ? hd / 64 : 1;                     // dims per lane (contiguous)
+    const bool lane_on = hd >= 64 || (uint32_t)lane < hd;
+    const uint32_t d0 = lane * dpl;
+    const uint32_t bit0 = d0 * bits, byte0 = bit0 >> 3, shift0 = bit0 & 7u;
+    const uint32_t nbytes = lane_on ? (shift0 + dpl * bits + 7u) / 8u : 0u;
+    const uint32_t cmask = (1u << bits) - 1u;
+
+    if (threadIdx.x < (1u << bits)) lds_levels[threadIdx.x] = levels[threadIdx.x];
+    __syncthreads();
+
+    uint32_t lo, hi, lane_base;
+    query_range(p, positions, qi, lo, hi, lane_base);
+    const uint32_t n = hi - lo;
+    const uint32_t chunk = (n + p.num_splits - 1) / p.num_splits;
+    const uint32_t c_lo = lo + std::min(n, split * chunk);
+    const uint32_t c_hi = lo + std::min(n, (split + 1) * chunk);
+
+    for (uint32_t h0 = 0; h0 < group; h0 += kHeadsPerPass) {
+        const uint32_t nh = std::min<uint32_t>(kHeadsPerPass, group - h0);
+        const uint32_t qh0 = kvh * group + h0;
+        float rqr[kHeadsPerPass][kMaxDpl], acc[kHeadsPerPass][kMaxDpl];
+#pragma unroll
+        for (int h = 0; h < kHeadsPerPass; h++)
+#pragma unroll
+            for (int i = 0; i < kMaxDpl; i++) {
+                acc[h][i] = 0.0f;
+                rqr[h][i] = ((uint32_t)h < nh && (uint32_t)i < dpl && lane_on)
+                                ? rq[((size_t)qi * p.num_q_heads + qh0 + h) * hd + d0 + i] : 0.0f;
+            }
+        // lane l tracks the running max / sum of head (l & 7)
+        float run_m = -INFINITY, run_l = 0.0f;
+
+        // each wave takes batches of kPosBatch consecutive positions; all loads of a batch are
+        // issued before any of it is consumed
+        for (uint32_t tb = c_lo + wave * kPosBatch; tb < c_hi; tb += kWavesPerWG * kPosBatch) {
+            uint32_t kw[kPosBatch], vw[kPosBatch];
+            float kn[kPosBatch], vn[kPosBatch];
+#pragma unroll
+            for (int j = 0; j < kPosBatch; j++) {
+                const uint32_t t = std::min(tb + j, c_hi - 1);          // past-the-end entries re-read the last one (unused)
+                const uint32_t pt = p.ring_capacity ? t % p.ring_capacity : t;
+                const size_t slot = (size_t)(lane_base + pt) * p.num_kv_heads + kvh;
+                kw[j] = load_window(k_codes + slot * p.code_bytes, byte0, nbytes) >> shift0;
+                vw[j] = load_window(v_codes + slot * p.code_bytes, byte0, nbytes) >> shift0;
+                kn[j] = lh_h2f(k_norms[slot]);
+                vn[j] = lh_h2f(v_norms[slot]);
+            }
+#pragma unroll
+            for (int j = 0; j < kPosBatch; j++) {
+                if (tb + j >= c_hi) break;
+                float dot[kHeadsPerPass];
+#pragma unroll
+                for (int h = 0; h < kHeadsPerPass; h++) dot[h] = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kMaxDpl; i++) {
+                    if ((uint32_t)i < dpl) {
+                        const float kv = lds_levels[(kw[j] >> (i * bits)) & cmask];
+#pragma unroll
+                        for (int h = 0; h < kHeadsPerPass; h++) dot[h] += rqr[h][i] * kv;
+                    }
+                }
+                const float logit = reduce8(dot, lane) * kn[j];                 // head (lane & 7)
+                const float new_m = fmaxf(run_m, logit);
+                const float rescale = __expf(run_m - new_m);                    // exp(-inf) = 0 on the first position
+                const float w = __expf(logit - new_m);
+                run_l = run_l * rescale + w;
+                run_m = new_m;
+                const float wv = w * vn[j];
+                float vv[kMaxDpl];
+#pragma unroll
+                for (int i = 0; i < kMaxDpl; i++) vv[i] = (uint32_t)i < dpl ? lds_levels[(vw[j] >> (i * bits)) & cmask] : 0.0f;
+#pragma unroll
+                for (int h = 0; h < kHeadsPerPass; h++) {
+                    const float r_h = __shfl(rescale, h, 64), w_h = __shfl(wv, h, 64);
+#pragma unroll
+                    for (int i = 0; i < kMaxDpl; i++)
+                        if ((uint32_t)i < dpl) acc[h][i] = acc[h][i] * r_h + w_h * vv[i];
+                }
+            }
+        }
+
+        // merge the four waves (log-sum-exp), then either finish or hand the partial to the reduce kernel
+        __syncthreads();
+        if (lane < kHeadsPerPass) { lds_m[wave][lane] = run_m; lds_l[wave][lane] = run_l; }
+#pragma unroll
+        for (int h = 0; h < kHeadsPerPass; h++)
+#pragma unroll
+            for (int i = 0; i < kMaxDpl; i++)
+                if ((uint32_t)i < dpl && lane_on) lds_acc[((size_t)wave * kHeadsPerPass + h) * hd + d0 + i] = acc[h][i];
+        __syncthreads();
+        for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += kThreads) {
+            const uint32_t h = idx / hd, d = idx - h * hd;
+            float gm = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < kWavesPerWG; w++) gm = fmaxf(gm, lds_m[w][h]);
+            float gl = 0.0f, o = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWavesPerWG; w++) {
+                const float f = lds_m[w][h] == -INFINITY ? 0.0f : __expf(lds_m[w][h] - gm);
+                gl += f * lds_l[w][h];
+                o += f * lds_acc[((size_t)w * kHeadsPerPass + h) * hd + d];
+            }
+            const uint32_t qh = qh0 + h;
+            if (p.num_splits == 1) {
+                out[((size_t)qi * p.num_q_heads + qh) * hd + d] = gl > 0.0f ? o / gl : 0.0f;
+            } else {
+                // workspace: per (query, head, split): [m, l, pad, pad, acc[hd]]
+                float* rec = ws + (((size_t)qi * p.num_q_heads + qh) * p.num_splits + split) * (hd + 4);
+                if (d == 0) { rec[0] = gm; rec[1] = gl; }
+                rec[4 + d] = o;
+            }
+        }
+    }
+}
+
+// flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.
+__global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
+                                                                 uint32_t num_splits) {
+    const uint32_t qh = blockIdx.x;     // flattened (query, head)
+    const float* base = ws + (size_t)qh * num_splits * (head_dim + 4);
+    float gm = -INFINITY;
+    for (uint32_t s = 0; s < num_splits; s++) gm = fmaxf(gm, base[(size_t)s * (head_dim + 4)]);
+    float gl = 0.0f;
+    for (uint32_t s = 0; s < num_splits; s++) {
+        const float m = base[(size_t)s * (head_dim + 4)];
+        gl += (m == -INFINITY ? 0.0f : __expf(m - gm)) * base[(size_t)s * (head_dim + 4) + 1];
+    }
+    const float inv = gl > 0.0f ? 1.0f / gl : 0.0f;
+    for (uint32_t d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float o = 0.0f;
+        for (uint32_t s = 0; s < num_splits; s++) {
+            const float m = base[(size_t)s * (head_dim + 4)];
+            o += (m == -INFINITY ? 0.0f : __expf(m - gm)) * base[(size_t)s * (head_dim + 4) + 4 + d];
+        }
+        out[(size_t)qh * head_dim + d] = o * inv;
+    }
+}
+
+int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                       const lh_buffer* positions, AttnParams p, uint64_t max_span, uint64_t phys_slots) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (p.bits < 2 || p.bits > 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant bits must be 2..=4, got %u", op, p.bits);
+    if (p.head_dim == 0 || (p.head_dim & (p.head_dim - 1)) || p.head_dim > 512)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant head_dim must be a power of two <= 512, got %u", op, p.head_dim);
+    if (p.num_kv_heads == 0 || p.num_q_heads % p.num_kv_heads != 0)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: num_q_heads %u is not a multiple of num_kv_heads %u", op, p.num_q_heads, p.num_kv_heads);
+    if (p.num_queries == 0 || p.num_q_heads == 0) return LH_OK;
+    lh_context* ctx = batch->ctx;
+    p.code_bytes = (p.head_dim * p.bits + 7) / 8;
+    const size_t qbytes = (size_t)p.num_queries * p.num_q_heads * p.head_dim * 4;
+    LH_NEED(rq, qbytes, op, "rq");
+    LH_NEED(out, qbytes, op, "out");
+    LH_NEED(levels, (size_t)4 << p.bits, op, "levels");
+    LH_NEED(k_codes, (size_t)phys_slots * p.code_bytes, op, "k_codes");
+    LH_NEED(v_codes, (size_t)phys_slots * p.code_bytes, op, "v_codes");
+    LH_NEED(k_norms, (size_t)phys_slots * 2, op, "k_norms");
+    LH_NEED(v_norms, (size_t)phys_slots * 2, op, "v_norms");
+    if (p.mode == kBatched) LH_NEED(positions, (size_t)p.num_queries * 4, op, "positions");
+
+    // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
+    const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
+    uint64_t splits = std::min<uint64_t>(per_query_wgs, (max_span + 31) / 32);
+    splits = std::max<uint64_t>(splits, 1);
+    const size_t rec = (size_t)p.head_dim + 4;
+    const size_t ws_avail = (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
+    while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_avail) splits--;
+    p.num_splits = (uint32_t)splits;
+
+    const size_t lds_bytes = (size_t)kWavesPerWG * kHeadsPerPass * p.head_dim * 4;
+    if (lds_bytes > 48 * 1024) {
+        static bool raised = false;   // one owner thread per context
+        if (!raised) {
+            LH_HIP_TRY(hipFuncSetAttribute((const void*)attention_tq_split_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024),
+                       LH_ERR_PIPELINE_CREATION, op);
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(attention_tq_split_kernel, dim3(p.num_splits, p.num_queries * p.num_kv_heads), dim3(kThreads), lds_bytes, ctx->stream,
+                       (const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr, (const uint8_t*)v_codes->ptr,
+                       (const uint16_t*)v_norms->ptr, (const float*)levels->ptr, positions ? (const uint32_t*)positions->ptr : nullptr,
+                       (float*)out->ptr, (float*)ctx->workspace, p);
+    int r = lh_check_launch(op);
+    if (r != LH_OK) return r;
+    batch->dispatch_count++;
+    if (p.num_splits > 1) {
+        hipLaunchKernelGGL(attention_tq_reduce_kernel, dim3(p.num_queries * p.num_q_heads), dim3(256), 0, ctx->stream,
+                           (const float*)ctx->workspace, (float*)out->ptr, p.head_dim, p.num_splits);
+        r = lh_check_launch(op);
+        if (r == LH_OK) batch->dispatch_count++;
+    }
+    return r;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                               const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                               uint32_t head_dim, uint32_t kv_len, uint32_t current_pos, uint32_t num_q_heads, uint32_t num_kv_heads,
+                               uint32_t window, uint32_t bits, uint32_t ring_capacity) {
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.kv_len = kv_len;
+    p.pos0 = current_pos; p.window = window; p.ring_capacity = ring_capacity; p.mode = kSingle; p.num_queries = 1;
+    const uint64_t seq = std::min<uint64_t>(kv_len, (uint64_t)current_pos + 1);
+    const uint64_t lo = (window > 0 && (uint64_t)current_pos + 1 > window) ? (uint64_t)current_pos + 1 - window : 0;
+    const uint64_t span = seq > lo ? seq - lo : 0;
+    const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
+    return attention_dispatch(batch, "flash_attention_tq", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys);
+}
+
+static int prefill_common(const char* op, lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                          const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                          uint32_t head_dim, uint32_t kv_len, uint32_t start_pos, uint32_t n_rows, uint32_t num_q_heads,
+                          uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t ring_capacity) {
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.kv_len = kv_len;
+    p.pos0 = start_pos; p.window = window; p.ring_capacity = ring_capacity; p.mode = kPrefill; p.num_queries = n_rows;
+    const uint64_t seq = std::min<uint64_t>(kv_len, (uint64_t)start_pos + n_rows);
+    const uint64_t span = window ? std::min<uint64_t>(window, seq) : seq;
+    const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
+    return attention_dispatch(batch, op, rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys);
+}
+
+int lh_flash_attention_tq_prefill_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                       uint32_t head_dim, uint32_t kv_len, uint32_t start_pos, uint32_t n_rows, uint32_t num_q_heads,
+                                       uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t ring_capacity) {
+    return prefill_common("flash_attention_tq_prefill", batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim, kv_len,
+                          start_pos, n_rows, num_q_heads, num_kv_heads, window, bits, ring_capacity);
+}
+
+int lh_flash_attention_tq_prefill_tiled_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                             const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels,
+                                             lh_buffer* out, uint32_t head_dim, uint32_t kv_len, uint32_t start_pos, uint32_t n_rows,
+                                             uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window, uint32_t bits,
+                                             uint32_t ring_capacity) {
+    return prefill_common("flash_attention_tq_prefill_tiled", batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim,
+                          kv_len, start_pos, n_rows, num_q_heads, num_kv_heads, window, bits, ring_capacity);
+}
+
+int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                       const lh_buffer* positions, uint32_t head_dim, uint32_t lane_capacity, uint32_t num_q_heads,
+                                       uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t n_lanes, uint32_t ring_capacity) {
+    const char* op = "flash_attention_tq_batched";
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads;
+    p.window = window; p.ring_capacity = ring_capacity; p.lane_capacity = lane_capacity; p.mode = kBatched; p.num_queries = n_lanes;
+    if (ring_capacity > lane_capacity)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: ring_capacity %u exceeds lane_capacity %u", op, ring_capacity, lane_capacity);
+    // positions are device data: size the split count for the largest possible span
+    const uint64_t cap = ring_capacity ? ring_capacity : lane_capacity;
+    const uint64_t span = window ? std::min<uint64_t>(window, cap) : cap;
+    const uint64_t phys = (uint64_t)n_lanes * lane_capacity * num_kv_heads;
+    return attention_dispatch(batch, op, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions, p, span, phys);
+}
+
+}  // extern "C"

@@ -112,6 +112,10 @@ __device__ __forceinline__ int lh_group_sum_i(int v, int width) {
 
 __device__ __forceinline__ float lh_h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t lh_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// Narrowing of an already rounded f32 value, as f16::from_f32 does it. The empty asm keeps the
+// compiler from folding a preceding multiply into v_fma_mixlo_f16, which rounds the exact
+// product once (a different result in double-rounding cases) and turns -0 into +0.
+__device__ __forceinline__ uint16_t lh_f2h_exact(float f) { asm volatile("" : "+v"(f)); return lh_f2h(f); }
 __device__ __forceinline__ float lh_bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
 
 template <typename T> __device__ __forceinline__ float lh_load_as_f32(const T* p, size_t i);

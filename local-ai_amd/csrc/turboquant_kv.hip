@@ -1,0 +1,388 @@
+// TurboQuant KV cache: codec parameters (host), GPU encode, GPU dequantize and the
+// randomized-Hadamard rotations around the fused attention kernel.
+//
+// Stands in for shaders/dequantize_kv.metal:132-407 (dequantize_kv_turboquant,
+// encode_kv_turboquant{,_batched}), shaders/attention_flash_tq.metal:58-139
+// (hadamard_rotate{,_hf,_fh}) and their dispatch in local-metal/src/kernels.rs:
+// 4641-5163, plus the host-side codec set-up of local-engine/src/turboquant.rs.
+//
+// Bit-exactness contract: codes and f16 norms written by the encode kernels equal
+// the CPU encoder's (turboquant.rs:241-276) for the same levels / signs.  That fixes
+//   - the squared norm as a left-to-right f32 sum of separately rounded squares,
+//   - IEEE sqrt and 1/norm, two separate multiplies (1/norm, then sign),
+//   - butterflies (a+b, a-b) per stage -- the pairing is fixed, so running a stage in
+//     parallel gives the same bits as the sequential loop,
+//   - 1/sqrt(d) computed on the host exactly as the CPU does and passed in,
+//   - nearest level with strict '<' from index 0 (lowest index wins ties).
+// This file is compiled with -ffp-contract=off: no product may be fused into a sum.
+#include "common.hpp"
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <algorithm>
+
+namespace {
+
+constexpr int kMaxHeadDim = 512;
+
+__device__ __forceinline__ uint32_t unpack_code(const uint8_t* codes, uint32_t d, uint32_t bits) {
+    // LSB-first bit stream; a 3-bit code may straddle two bytes (attention_flash_tq.metal:33-47)
+    const uint32_t bit_off = d * bits, byte = bit_off >> 3, shift = bit_off & 7u;
+    uint32_t v = codes[byte];
+    if (shift + bits > 8u) v |= (uint32_t)codes[byte + 1] << 8;
+    return (v >> shift) & ((1u << bits) - 1u);
+}
+
+// In-place unnormalised FWHT over sh[0..d) with one thread per element.
+__device__ __forceinline__ void fwht_lds(float* sh, uint32_t d, uint32_t lane) {
+    for (uint32_t len = 1; len < d; len <<= 1) {
+        __syncthreads();
+        const float self_v = sh[lane], other_v = sh[lane ^ len];
+        __syncthreads();
+        sh[lane] = (lane & len) ? __fsub_rn(other_v, self_v) : __fadd_rn(self_v, other_v);
+    }
+    __syncthreads();
+}
+
+struct EncodeParams {
+    uint32_t head_dim, n_kv_heads, bits, code_bytes;
+    uint32_t position;        // first logical token (single-sequence form)
+    uint32_t ring_capacity;   // 0 = absolute
+    uint32_t lane_capacity;   // batched form: physical tokens per lane region
+    float inv_sqrt_d;
+};
+
+// One workgroup (head_dim threads) per (token, head) vector.  BATCHED: group = (lane, head),
+// slot from positions[lane] (dequantize_kv.metal:327-407); else group = (token, head)
+// (dequantize_kv.metal:216-318).
+template <bool BATCHED>
+__global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* __restrict__ input, const float* __restrict__ levels,
+                                                               const float* __restrict__ signs, uint8_t* __restrict__ packed,
+                                                               uint16_t* __restrict__ norms, const uint32_t* __restrict__ positions,
+                                                               EncodeParams p) {
+    __shared__ __align__(16) float sh[kMaxHeadDim];
+    __shared__ uint32_t code_sh[kMaxHeadDim];
+    const uint32_t d = p.head_dim, lane = threadIdx.x, group = blockIdx.x;
+    const uint32_t tok = group / p.n_kv_heads, head = group - tok * p.n_kv_heads;
+    uint32_t g;
+    if (BATCHED) {
+        const uint32_t pos = positions[tok];
+        const uint32_t ppos = p.ring_capacity ? pos % p.ring_capacity : pos;
+        g = (tok * p.lane_capacity + ppos) * p.n_kv_heads + head;
+    } else {
+        const uint32_t logical = p.position + tok;
+        g = (p.ring_capacity ? logical % p.ring_capacity : logical) * p.n_kv_heads + head;
+    }
+    const float xv = lh_h2f(input[(size_t)group * d + lane]);
+
+    // norm = sqrt(fold(+, x_i * x_i)) in index order; every thread walks the same LDS
+    // words (broadcast reads), so all hold the same value without another barrier.
+    sh[lane] = __fmul_rn(xv, xv);
+    __syncthreads();
+    float sq = 0.0f;
+    if (d >= 4) {
+        for (uint32_t i = 0; i < d; i += 4) {
+            const float4 q = *reinterpret_cast<const float4*>(&sh[i]);
+            sq = __fadd_rn(sq, q.x); sq = __fadd_rn(sq, q.y); sq = __fadd_rn(sq, q.z); sq = __fadd_rn(sq, q.w);
+        }
+    } else {
+        for (uint32_t i = 0; i < d; i++) sq = __fadd_rn(sq, sh[i]);
+    }
+    const float norm = __fsqrt_rn(sq);
+    float v = xv;
+    if (norm > 0.0f) v = __fmul_rn(v, __fdiv_rn(1.0f, norm));
+    v = __fmul_rn(v, signs[lane]);
+    __syncthreads();
+    sh[lane] = v;
+    fwht_lds(sh, d, lane);
+    const float y = __fmul_rn(sh[lane], p.inv_sqrt_d);
+
+    const uint32_t k = 1u << p.bits;
+    uint32_t best = 0;
+    float bd = INFINITY;
+    for (uint32_t i = 0; i < k; ++i) {
+        const float dd = fabsf(__fsub_rn(y, levels[i]));
+        if (dd < bd) { bd = dd; best = i; }
+    }
+    code_sh[lane] = best;
+    if (lane == 0) norms[g] = lh_f2h_exact(norm);
+    __syncthreads();
+    if (lane < p.code_bytes) {     // one thread per output byte
+        uint32_t byte_val = 0;
+        for (uint32_t bitpos = 0; bitpos < 8; ++bitpos) {
+            const uint32_t global_bit = lane * 8 + bitpos, code_idx = global_bit / p.bits;
+            if (code_idx >= d) break;
+            byte_val |= ((code_sh[code_idx] >> (global_bit - code_idx * p.bits)) & 1u) << bitpos;
+        }
+        packed[(size_t)g * p.code_bytes + lane] = (uint8_t)byte_val;
+    }
+}
+
+struct DequantParams {
+    uint32_t head_dim, n_kv_heads, bits, code_bytes, group_offset, ring_capacity;
+    float inv_sqrt_d;
+};
+
+// dequantize_kv.metal:132-189: x^ = sign * (1/sqrt d) * H(levels[code]) * norm -> f16 at the logical slot.
+__global__ __launch_bounds__(kMaxHeadDim) void dequantize_kv_kernel(const uint8_t* __restrict__ packed, const uint16_t* __restrict__ norms,
+                                                                   const float* __restrict__ levels, const float* __restrict__ signs,
+                                                                   uint16_t* __restrict__ output, DequantParams p) {
+    __shared__ __align__(16) float sh[kMaxHeadDim];
+    const uint32_t d = p.head_dim, lane = threadIdx.x;
+    const uint32_t g = blockIdx.x + p.group_offset;
+    uint32_t src_g = g;
+    if (p.ring_capacity) {
+        const uint32_t token = g / p.n_kv_heads, head = g - token * p.n_kv_heads;
+        src_g = (token % p.ring_capacity) * p.n_kv_heads + head;
+    }
+    sh[lane] = levels[unpack_code(packed + (size_t)src_g * p.code_bytes, lane, p.bits)];
+    fwht_lds(sh, d, lane);
+    float val = __fmul_rn(sh[lane], p.inv_sqrt_d);
+    val = __fmul_rn(val, signs[lane]);
+    val = __fmul_rn(val, lh_h2f(norms[src_g]));
+    output[(size_t)g * d + lane] = lh_f2h_exact(val);
+}
+
+// attention_flash_tq.metal:58-90: optional pre-sign, FWHT, 1/sqrt(d), optional post-sign.
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(kMaxHeadDim) void hadamard_rotate_kernel(const TIn* __restrict__ input, const float* __restrict__ signs,
+                                                                     TOut* __restrict__ output, uint32_t head_dim, float inv_sqrt_d,
+                                                                     int pre_sign, int post_sign) {
+    __shared__ __align__(16) float sh[kMaxHeadDim];
+    const uint32_t d = head_dim, lane = threadIdx.x, head = blockIdx.x;
+    const float x = lh_load_as_f32<TIn>(input, (size_t)head * d + lane);
+    sh[lane] = pre_sign ? __fmul_rn(x, signs[lane]) : x;
+    fwht_lds(sh, d, lane);
+    float y = __fmul_rn(sh[lane], inv_sqrt_d);
+    if (post_sign) y = __fmul_rn(y, signs[lane]);
+    if constexpr (sizeof(TOut) == 2) output[(size_t)head * d + lane] = lh_f2h_exact(y);
+    else output[(size_t)head * d + lane] = y;
+}
+
+int check_tq_shape(const char* op, uint32_t head_dim, uint32_t bits) {
+    // quant_cache.rs:191-200 and the debug_assert at kernels.rs:4667
+    if (bits < 2 || bits > 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant bits must be 2..=4, got %u", op, bits);
+    if (head_dim == 0 || (head_dim & (head_dim - 1)) != 0 || head_dim > kMaxHeadDim)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant head_dim must be a power of two <= 512, got %u", op, head_dim);
+    return LH_OK;
+}
+
+inline float host_inv_sqrt(uint32_t d) { return 1.0f / std::sqrt((float)d); }   // turboquant.rs:47
+
+template <typename TIn, typename TOut>
+int hadamard_launch(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs, lh_buffer* output, uint32_t head_dim,
+                    uint32_t num_heads, int pre_sign, int post_sign, const char* op) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    int r = check_tq_shape(op, head_dim, 2);
+    if (r != LH_OK) return r;
+    if (num_heads == 0) return LH_OK;
+    LH_NEED(input, (size_t)num_heads * head_dim * sizeof(TIn), op, "input");
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    LH_NEED(output, (size_t)num_heads * head_dim * sizeof(TOut), op, "output");
+    hipLaunchKernelGGL((hadamard_rotate_kernel<TIn, TOut>), dim3(num_heads), dim3(head_dim), 0, batch->ctx->stream,
+                       (const TIn*)input->ptr, (const float*)signs->ptr, (TOut*)output->ptr, head_dim, host_inv_sqrt(head_dim),
+                       pre_sign, post_sign);
+    r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+// ---- host codec ----------------------------------------------------------------
+// turboquant.rs:114-166, same operation order in f32 (mul_add -> fmaf).
+void lloyd_max_gaussian(uint32_t bits, float* levels) {
+    constexpr int N = 8192;
+    const float LO = -6.0f, HI = 6.0f;
+    const float FRAC_1_SQRT_2 = 0.707106781186547524400844362104849039f;
+    const float FRAC_2_SQRT_PI = 1.12837916709551257389615890312154517f;
+    const size_t k = (size_t)1 << bits;
+    const float dx = (HI - LO) / (float)N;
+    float* xs = (float*)malloc(N * sizeof(float));
+    float* pdf = (float*)malloc(N * sizeof(float));
+    for (int i = 0; i < N; i++) xs[i] = std::fmaf((float)i + 0.5f, dx, LO);
+    for (int i = 0; i < N; i++) {
+        const float x = xs[i];
+        pdf[i] = std::exp(-0.5f * x * x) * FRAC_1_SQRT_2 * FRAC_2_SQRT_PI / 2.0f;
+    }
+    for (size_t i = 0; i < k; i++) {
+        const float t = ((float)i + 0.5f) / (float)k;
+        levels[i] = 6.0f * (t - 0.5f);
+    }
+    float sum[16], wsum[16];
+    for (int it = 0; it < 100; it++) {
+        for (size_t j = 0; j < k; j++) { sum[j] = 0.0f; wsum[j] = 0.0f; }
+        for (int i = 0; i < N; i++) {
+            const float x = xs[i], w = pdf[i];
+            size_t best = 0;
+            float bd = INFINITY;
+            for (size_t j = 0; j < k; j++) {
+                const float dist = std::fabs(x - levels[j]);
+                if (dist < bd) { bd = dist; best = j; }
+            }
+            sum[best] = std::fmaf(w, x, sum[best]);
+            wsum[best] += w;
+        }
+        for (size_t j = 0; j < k; j++)
+            if (wsum[j] > 1e-12f) levels[j] = sum[j] / wsum[j];
+    }
+    std::sort(levels, levels + k);
+    free(xs);
+    free(pdf);
+}
+
+}  // namespace
+
+extern "C" {
+
+int lh_turboquant_levels(uint32_t dim, uint32_t bits, float* levels) {
+    if (!levels) return lh_fail(LH_ERR_INVALID_ARGUMENT, "turboquant_levels: levels is null");
+    if (bits < 1 || bits > 4 || dim == 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "turboquant_levels: bad dim %u / bits %u", dim, bits);
+    lloyd_max_gaussian(bits, levels);
+    const float scale = 1.0f / std::sqrt((float)dim);     // turboquant.rs:187-192
+    for (uint32_t i = 0; i < (1u << bits); i++) levels[i] = levels[i] * scale;
+    return LH_OK;
+}
+
+int lh_turboquant_signs(uint32_t dim, uint64_t seed, float* signs) {
+    if (!signs) return lh_fail(LH_ERR_INVALID_ARGUMENT, "turboquant_signs: signs is null");
+    uint64_t state = seed | 1u;                              // turboquant.rs:66-79
+    for (uint32_t i = 0; i < dim; i++) {
+        state += 0x9E3779B97F4A7C15ull;
+        uint64_t z = state;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        signs[i] = (z & 1u) == 0 ? 1.0f : -1.0f;
+    }
+    return LH_OK;
+}
+
+uint32_t lh_turboquant_code_bytes(uint32_t dim, uint32_t bits) { return (dim * bits + 7) / 8; }
+
+size_t lh_swa_ring_capacity(size_t window, size_t max_positions) {   // quant_cache.rs:48-54
+    const size_t min_safe = window + 256 - 1;
+    size_t v = std::max(window * 2, min_safe), p = 1;
+    while (p < v) p <<= 1;
+    return std::min(p, max_positions);
+}
+
+uint32_t lh_kv_bits_from_env(void) {                                 // quant_cache.rs:60-66
+    const char* v = getenv("LOCAL_AI_KV_QUANT");
+    if (v && strcmp(v, "tq3") == 0) return 3;
+    if (v && strcmp(v, "tq4") == 0) return 4;
+    return LH_DEFAULT_KV_BITS;
+}
+
+int lh_encode_kv_turboquant_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* levels, const lh_buffer* signs,
+                                 lh_buffer* packed, lh_buffer* norms, uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens,
+                                 uint32_t bits, uint32_t position, uint32_t ring_capacity) {
+    const char* op = "encode_kv_turboquant";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    int r = check_tq_shape(op, head_dim, bits);
+    if (r != LH_OK) return r;
+    const uint32_t groups = n_kv_heads * num_tokens;
+    if (groups == 0) return LH_OK;
+    const uint32_t cb = lh_turboquant_code_bytes(head_dim, bits);
+    // highest physical slot written
+    const uint64_t phys_tokens = ring_capacity ? std::min<uint64_t>(ring_capacity, (uint64_t)position + num_tokens)
+                                               : (uint64_t)position + num_tokens;
+    LH_NEED(input, (size_t)groups * head_dim * 2, op, "input");
+    LH_NEED(levels, (size_t)4 << bits, op, "levels");
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    LH_NEED(packed, (size_t)phys_tokens * n_kv_heads * cb, op, "packed");
+    LH_NEED(norms, (size_t)phys_tokens * n_kv_heads * 2, op, "norms");
+    EncodeParams p{head_dim, n_kv_heads, bits, cb, position, ring_capacity, 0, host_inv_sqrt(head_dim)};
+    hipLaunchKernelGGL((encode_kv_kernel<false>), dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
+                       (const float*)levels->ptr, (const float*)signs->ptr, (uint8_t*)packed->ptr, (uint16_t*)norms->ptr,
+                       (const uint32_t*)nullptr, p);
+    r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+int lh_encode_kv_turboquant(lh_context* ctx, const lh_buffer* input, const lh_buffer* levels, const lh_buffer* signs, lh_buffer* packed,
+                            lh_buffer* norms, uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens, uint32_t bits,
+                            uint32_t position, uint32_t ring_capacity) {
+    if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "encode_kv_turboquant: context is null");
+    lh_batch b{ctx, 0};
+    int r = lh_encode_kv_turboquant_into(&b, input, levels, signs, packed, norms, head_dim, n_kv_heads, num_tokens, bits, position,
+                                         ring_capacity);
+    return r != LH_OK ? r : lh_batch_commit_and_wait(&b);
+}
+
+int lh_encode_kv_turboquant_batched_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* levels, const lh_buffer* signs,
+                                         lh_buffer* packed, lh_buffer* norms, const lh_buffer* positions, uint32_t head_dim,
+                                         uint32_t n_kv_heads, uint32_t lane_capacity, uint32_t bits, uint32_t n_lanes,
+                                         uint32_t ring_capacity) {
+    const char* op = "encode_kv_turboquant_batched";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    int r = check_tq_shape(op, head_dim, bits);
+    if (r != LH_OK) return r;
+    const uint32_t groups = n_kv_heads * n_lanes;
+    if (groups == 0) return LH_OK;
+    LH_REQUIRE(ring_capacity <= lane_capacity, "%s: ring_capacity %u exceeds lane_capacity %u", op, ring_capacity, lane_capacity);
+    const uint32_t cb = lh_turboquant_code_bytes(head_dim, bits);
+    LH_NEED(input, (size_t)groups * head_dim * 2, op, "input");
+    LH_NEED(levels, (size_t)4 << bits, op, "levels");
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    LH_NEED(positions, (size_t)n_lanes * 4, op, "positions");
+    // positions live in device memory, so the slot range cannot be checked here beyond the pool size
+    LH_NEED(packed, (size_t)n_lanes * lane_capacity * n_kv_heads * cb, op, "packed");
+    LH_NEED(norms, (size_t)n_lanes * lane_capacity * n_kv_heads * 2, op, "norms");
+    EncodeParams p{head_dim, n_kv_heads, bits, cb, 0, ring_capacity, lane_capacity, host_inv_sqrt(head_dim)};
+    hipLaunchKernelGGL((encode_kv_kernel<true>), dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
+                       (const float*)levels->ptr, (const float*)signs->ptr, (uint8_t*)packed->ptr, (uint16_t*)norms->ptr,
+                       (const uint32_t*)positions->ptr, p);
+    r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+int lh_dequantize_kv_turboquant_into(lh_batch* batch, const lh_buffer* packed, const lh_buffer* norms, const lh_buffer* levels,
+                                     const lh_buffer* signs, lh_buffer* output, uint32_t head_dim, uint32_t n_kv_heads,
+                                     uint32_t num_tokens, uint32_t bits, uint32_t token_start, uint32_t ring_capacity) {
+    const char* op = "dequantize_kv_turboquant";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    int r = check_tq_shape(op, head_dim, bits);
+    if (r != LH_OK) return r;
+    if (token_start > num_tokens) token_start = num_tokens;              // kernels.rs:4668
+    const uint32_t groups = n_kv_heads * (num_tokens - token_start);
+    if (groups == 0) return LH_OK;
+    const uint32_t cb = lh_turboquant_code_bytes(head_dim, bits);
+    const uint64_t phys_tokens = ring_capacity ? std::min<uint64_t>(ring_capacity, num_tokens) : num_tokens;
+    LH_NEED(packed, (size_t)phys_tokens * n_kv_heads * cb, op, "packed");
+    LH_NEED(norms, (size_t)phys_tokens * n_kv_heads * 2, op, "norms");
+    LH_NEED(levels, (size_t)4 << bits, op, "levels");
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    LH_NEED(output, (size_t)num_tokens * n_kv_heads * head_dim * 2, op, "output");
+    DequantParams p{head_dim, n_kv_heads, bits, cb, token_start * n_kv_heads, ring_capacity, host_inv_sqrt(head_dim)};
+    hipLaunchKernelGGL(dequantize_kv_kernel, dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (const uint8_t*)packed->ptr,
+                       (const uint16_t*)norms->ptr, (const float*)levels->ptr, (const float*)signs->ptr, (uint16_t*)output->ptr, p);
+    r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+int lh_dequantize_kv_turboquant(lh_context* ctx, const lh_buffer* packed, const lh_buffer* norms, const lh_buffer* levels,
+                                const lh_buffer* signs, lh_buffer* output, uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens,
+                                uint32_t bits, uint32_t token_start, uint32_t ring_capacity) {
+    if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "dequantize_kv_turboquant: context is null");
+    lh_batch b{ctx, 0};
+    int r = lh_dequantize_kv_turboquant_into(&b, packed, norms, levels, signs, output, head_dim, n_kv_heads, num_tokens, bits,
+                                             token_start, ring_capacity);
+    return r != LH_OK ? r : lh_batch_commit_and_wait(&b);
+}
+
+int lh_hadamard_rotate_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs, lh_buffer* output, uint32_t head_dim,
+                            uint32_t num_heads, int pre_sign, int post_sign) {
+    return hadamard_launch<float, float>(batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign, "hadamard_rotate");
+}
+int lh_hadamard_rotate_hf_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs, lh_buffer* output, uint32_t head_dim,
+                               uint32_t num_heads, int pre_sign, int post_sign) {
+    return hadamard_launch<uint16_t, float>(batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign, "hadamard_rotate_hf");
+}
+int lh_hadamard_rotate_fh_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs, lh_buffer* output, uint32_t head_dim,
+                               uint32_t num_heads, int pre_sign, int post_sign) {
+    return hadamard_launch<float, uint16_t>(batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign, "hadamard_rotate_fh");
+}
+
+}  // extern "C"

@@ -1,0 +1,198 @@
+"""GPU parity of the fused TurboQuant attention kernels against the f64 code-space oracle.
+Mirrors local-metal/src/kernels.rs:9936-10125 (fused vs dequant-then-flash), 10126-10456
+(prefill vs per-row decode, tiled vs non-tiled), 10457 (batched) and
+local-engine/src/kv_cache/quant_cache.rs:1047-1107 (ring == full)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ATTN_TOL = 2e-3   # max |delta| <= tol * max(max|ref|, 1e-3), kernels.rs:10105-10114
+
+
+def build_cache(pkg, oracle, T, n_kv, hd, bits, seed, ring=0, scale=1.0):
+    g = pkg.synth.rng(6, seed)
+    k = (pkg.synth.kv_rows(T, n_kv, hd, g).astype(np.float32) * scale).astype(np.float16)
+    v = pkg.synth.kv_rows(T, n_kv, hd, g)
+    signs, levels = oracle.rotation_signs(hd, oracle.TQ_SEED), oracle.tq_levels(hd, bits)
+    cb = oracle.tq_code_bytes(hd, bits)
+    phys = ring if ring else T
+    kc = np.zeros((phys, n_kv, cb), np.uint8); vc = np.zeros_like(kc)
+    kn = np.zeros((phys, n_kv), np.uint16); vn = np.zeros_like(kn)
+    oracle.tq_write_kv(k.view(np.uint16), n_kv, hd, bits, signs, levels, 0, ring, kc, kn)
+    oracle.tq_write_kv(v.view(np.uint16), n_kv, hd, bits, signs, levels, 0, ring, vc, vn)
+    return signs, levels, kc, kn, vc, vn
+
+
+def check(got, ref, label, tol=ATTN_TOL):
+    err = float(np.max(np.abs(got - ref)))
+    scale = max(float(np.max(np.abs(ref))), 1e-3)
+    assert err <= tol * scale, f"{label}: max|delta| {err:.3e} > {tol} * {scale:.3e}"
+    return err / scale
+
+
+def upload(pkg, ctx, *arrays):
+    return [pkg.Buffer.from_slice(ctx, a) for a in arrays]
+
+
+@pytest.mark.parametrize("hd,nq,nkv,T,bits,window,qscale", [
+    (128, 4, 2, 24, 4, 0, 1.0),        # the reference's own fused-attention test shape
+    (256, 8, 1, 300, 2, 0, 1.0),       # measured configuration, short context
+    (256, 8, 1, 4096, 2, 0, 1.0),
+    (256, 8, 1, 1000, 2, 512, 1.0),    # sliding window
+    (256, 8, 1, 777, 3, 0, 0.3),
+    (512, 8, 1, 200, 2, 0, 0.2),
+    (64, 6, 3, 90, 4, 16, 0.5),
+    (256, 16, 1, 100, 2, 0, 0.3),      # more than 8 query heads per KV head
+    (128, 2, 2, 1, 2, 0, 1.0),         # one position
+])
+def test_decode_attention_matches_oracle(pkg, gpu, oracle, hd, nq, nkv, T, bits, window, qscale):
+    print(f"case hd={hd} nq={nq} nkv={nkv} T={T} bits={bits} window={window}", flush=True)
+    ctx, K = gpu
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, T + bits)
+    q = (pkg.synth.rng(6, 999).standard_normal((nq, hd), dtype=np.float32) * qscale).astype(np.float16)
+    rq_ref = oracle.hadamard_rotate(q.astype(np.float32), signs, hd, nq, True, False)
+    acc_ref = oracle.attention_tq_codespace(rq_ref, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, window, bits, 0)
+    kcb, knb, vcb, vnb, lvb, sgb, qb = upload(pkg, ctx, kc, kn, vc, vn, levels, signs, q)
+    rq, vacc = pkg.Buffer.empty(ctx, nq * hd * 4), pkg.Buffer.empty(ctx, nq * hd * 4)
+    out = pkg.Buffer.empty(ctx, nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+    K.hadamard_rotate_hf_into(batch, qb, sgb, rq, hd, nq, True, False)
+    K.flash_attention_tq_into(batch, rq, kcb, knb, vcb, vnb, lvb, vacc, hd, T, T - 1, nq, nkv, window, bits, 0)
+    K.hadamard_rotate_into(batch, vacc, sgb, out, hd, nq, False, True)
+    batch.commit_and_wait()
+    e1 = check(vacc.as_array(np.float32), acc_ref, "rotated-space accumulation")
+    ref = oracle.hadamard_rotate(acc_ref, signs, hd, nq, False, True)
+    e2 = check(out.as_array(np.float32), ref, "attention output")
+    # element-wise form too: |g - w| <= tol * max(|w|, 1)
+    assert np.max(np.abs(out.as_array(np.float32) - ref) / np.maximum(np.abs(ref), 1.0)) <= ATTN_TOL
+    print(f"  err rotated {e1:.2e}, output {e2:.2e}")
+
+
+def test_decode_attention_vs_reference_cpu_path(pkg, gpu, oracle):
+    """Against the CPU path the reference would run: TurboQuant::decode of every position, then
+    f32 attention in the original space."""
+    ctx, K = gpu
+    hd, nq, nkv, T, bits = 256, 8, 1, 512, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 4242)
+    q = pkg.synth.rng(6, 5).standard_normal((nq, hd), dtype=np.float32).astype(np.float16)
+    cache = pkg.QuantizedKvCache(ctx, nkv, hd, T, bits)
+    cache.keys_q.copy_from_bytes(kc); cache.key_norms.copy_from_bytes(kn)
+    cache.values_q.copy_from_bytes(vc); cache.value_norms.copy_from_bytes(vn)
+    qb = pkg.Buffer.from_slice(ctx, q)
+    rq, vacc = pkg.Buffer.empty(ctx, nq * hd * 4), pkg.Buffer.empty(ctx, nq * hd * 4)
+    out = pkg.Buffer.empty(ctx, nq * hd * 2)
+    batch = pkg.CommandBatch(ctx)
+    cache.fused_attention_into(batch, K, qb, rq, vacc, out, T, T - 1, nq, 0)
+    batch.commit_and_wait()
+    ref = oracle.attention_tq_decode_then_attend(q.astype(np.float32), kc, kn, vc, vn, levels, signs, hd, T, T - 1, nq, nkv,
+                                                 0, bits, 0, threads=8)
+    check(out.as_array(np.float16).astype(np.float32), ref, "fused vs decode-then-attend", tol=ATTN_TOL + 1e-3)  # + f16 store
+
+
+def test_ring_matches_full_cache_bitwise(pkg, gpu, oracle):
+    """quant_cache.rs:1047-1107: attention over a wrapped ring is bit-identical to the full cache."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, T, window, ring = 256, 8, 1, 2, 1500, 512, 512
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 77)
+    _, _, rkc, rkn, rvc, rvn = build_cache(pkg, oracle, T, nkv, hd, bits, 77, ring=ring)
+    rq = pkg.synth.rng(6, 8).standard_normal(nq * hd, dtype=np.float32)
+    lvb, rqb = upload(pkg, ctx, levels, rq)
+    outs = []
+    for (a, b, c, d, r) in ((kc, kn, vc, vn, 0), (rkc, rkn, rvc, rvn, ring)):
+        ab, bb, cb_, db = upload(pkg, ctx, a, b, c, d)
+        o = pkg.Buffer.empty(ctx, nq * hd * 4)
+        batch = pkg.CommandBatch(ctx)
+        K.flash_attention_tq_into(batch, rqb, ab, bb, cb_, db, lvb, o, hd, T, T - 1, nq, nkv, window, bits, r)
+        batch.commit_and_wait()
+        outs.append(o.as_array(np.float32))
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    ref = oracle.attention_tq_codespace(rq, rkc, rkn, rvc, rvn, levels, hd, T, T - 1, nq, nkv, window, bits, ring)
+    check(outs[1], ref, "ring attention")
+
+
+def test_empty_range_gives_zeros(pkg, gpu, oracle):
+    ctx, K = gpu
+    hd, nq, nkv, bits = 128, 4, 2, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, 4, nkv, hd, bits, 1)
+    bufs = upload(pkg, ctx, kc, kn, vc, vn, levels)
+    rq = pkg.Buffer.from_slice(ctx, np.ones(nq * hd, np.float32))
+    out = pkg.Buffer.from_slice(ctx, np.full(nq * hd, 7.0, np.float32))
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rq, bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], out, hd, 0, 0, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    assert np.all(out.as_array(np.float32) == 0)
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("hd,nq,nkv,bits,start,rows,window", [(256, 8, 1, 2, 0, 37, 0), (256, 8, 1, 2, 100, 20, 64),
+                                                              (128, 4, 2, 4, 5, 9, 0)])
+def test_prefill_matches_per_row_decode(pkg, gpu, oracle, tiled, hd, nq, nkv, bits, start, rows, window):
+    """kernels.rs:10126, 10295: every prefill row equals the decode kernel at that position."""
+    print(f"case tiled={tiled} hd={hd} rows={rows} start={start}", flush=True)
+    ctx, K = gpu
+    T = start + rows
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 31 + rows)
+    rq = (pkg.synth.rng(6, 12).standard_normal((rows, nq, hd), dtype=np.float32) * 0.5).astype(np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+    fn = K.flash_attention_tq_prefill_tiled_into if tiled else K.flash_attention_tq_prefill_into
+    fn(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, start, rows, nq, nkv, window, bits, 0)
+    batch.commit_and_wait()
+    got = out.as_array(np.float32).reshape(rows, nq * hd)
+    for r in range(rows):
+        ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, levels, hd, T, start + r, nq, nkv, window, bits, 0)
+        check(got[r], ref, f"row {r}")
+
+
+def test_batched_matches_independent_sequences(pkg, gpu, oracle):
+    """kernels.rs:10457: lanes at different positions in one dispatch == separate single-sequence calls."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, lanes, cap = 256, 8, 1, 2, 4, 600
+    cb = oracle.tq_code_bytes(hd, bits)
+    positions = np.array([599, 0, 123, 300], np.uint32)
+    pool_kc = np.zeros((lanes * cap, nkv, cb), np.uint8); pool_vc = np.zeros_like(pool_kc)
+    pool_kn = np.zeros((lanes * cap, nkv), np.uint16); pool_vn = np.zeros_like(pool_kn)
+    levels = None
+    for l in range(lanes):
+        n = int(positions[l]) + 1
+        signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, n, nkv, hd, bits, 500 + l)
+        pool_kc[l * cap:l * cap + n] = kc; pool_vc[l * cap:l * cap + n] = vc
+        pool_kn[l * cap:l * cap + n] = kn; pool_vn[l * cap:l * cap + n] = vn
+    rq = pkg.synth.rng(6, 13).standard_normal((lanes, nq * hd), dtype=np.float32)
+    bufs = upload(pkg, ctx, pool_kc, pool_kn, pool_vc, pool_vn, levels, rq, positions)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_batched_into(batch, bufs[5], bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], out, bufs[6], hd, cap, nq,
+                                      nkv, 0, bits, lanes, 0)
+    batch.commit_and_wait()
+    got = out.as_array(np.float32).reshape(lanes, nq * hd)
+    for l in range(lanes):
+        ref = oracle.attention_tq_codespace(rq[l], pool_kc, pool_kn, pool_vc, pool_vn, levels, hd, int(positions[l]) + 1,
+                                            int(positions[l]), nq, nkv, 0, bits, 0, lane_base=l * cap)
+        check(got[l], ref, f"lane {l}")
+
+
+def test_split_invariance_at_32k(pkg, gpu, oracle):
+    """Full-size configuration (32768 cached positions, 8 q heads / 1 kv head, hd 256, 2 bits):
+    parity with the f64 oracle, and the SWA-ring configuration (window 512, ring 512, wrapped)."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, T = 256, 8, 1, 2, 32768
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 32768)
+    q = pkg.synth.rng(6, 14).standard_normal((nq, hd), dtype=np.float32).astype(np.float16)
+    rq = oracle.hadamard_rotate(q.astype(np.float32), signs, hd, nq, True, False)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    out = pkg.Buffer.empty(ctx, nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    ref = oracle.attention_tq_codespace(rq, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    e = check(out.as_array(np.float32), ref, "32k full attention")
+    print(f"32k: {e:.2e}")
+    _, _, rkc, rkn, rvc, rvn = build_cache(pkg, oracle, 3000, nkv, hd, bits, 3000, ring=512)
+    bufs = upload(pkg, ctx, rkc, rkn, rvc, rvn)
+    K.flash_attention_tq_into(batch, rqb, bufs[0], bufs[1], bufs[2], bufs[3], lvb, out, hd, 3000, 2999, nq, nkv, 512, bits, 512)
+    batch.commit_and_wait()
+    ref = oracle.attention_tq_codespace(rq, rkc, rkn, rvc, rvn, levels, hd, 3000, 2999, nq, nkv, 512, bits, 512)
+    check(out.as_array(np.float32), ref, "SWA ring 512")
