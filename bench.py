@@ -1,0 +1,374 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+Headline (the JSON line's `value`): HBM GB/s of the fused TQ2_0 dequant matvec at M = 1 on
+the MLP gate/up shape (N = 8192, K = 2048, fp32 activations and outputs), measured the way
+the reference measures its own kernels (local-metal/src/kernels.rs:8883-9020): R distinct
+weight sets totalling >= 1 GiB so nothing is served from cache, GB/s = algorithmic bytes /
+elapsed.  One "step" is one pass over the R weight sets, issued as ONE grouped launch.
+Everything is resident in HBM before the timed region.
+
+Also measured and reported in the same line (`extra`): the Q4_0 matvec (N = K = 2048), the
+TQ2_0 down-projection shape, one logits-sized matvec (262144 x 1536, a single ordinary
+launch), the tq2 flash-decoding attention at 32k context (single query, and a batch of
+independent sequences), the small-batch layer and the prefill matmul.
+
+`roofline` describes the dominant kernel (matvec_quant_kernel, TQ2_0 instantiation): its
+algorithmic bytes per launch over its launch duration from HIP events on the library's
+stream.  `cpu_baseline` times the CPU restatement of the reference's own path (block dequant
+to f16 + sequential f32 dot) on the host cores, on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/matvec_tq2_0_grouped_pmc.md), scaled by the same counters on the library's plain
+# copy kernel; None until that profile has been taken for the current kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def distinct_replicas(pkg, ctx, raw, count, block_bytes):
+    """`count` weight sets of the same shape at distinct addresses (one allocation), each a
+    different rotation of the generated blocks so no two are byte-identical."""
+    wb = raw.size
+    big = pkg.Buffer.empty(ctx, wb * count)
+    for i in range(count):
+        big.copy_from_bytes(np.roll(raw, i * block_bytes * 7), i * wb)
+    return big, [big.view(i * wb, wb) for i in range(count)]
+
+
+def time_steps(pkg, ctx, fn, steps, warmup):
+    """Wall-clock (sync on both sides) and HIP-event time of `steps` calls of fn()."""
+    for _ in range(warmup):
+        fn()
+    ctx.synchronize()
+    e0, e1 = pkg.Event(ctx), pkg.Event(ctx)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    ctx.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_ms(e1)
+    return wall_ms / steps, ev_ms / steps
+
+
+def bound_call(fn, *args):
+    """A zero-argument callable for one C-ABI call with its ctypes arguments converted once:
+    keeps the per-launch host cost of the timing loops near the cost of the launch itself."""
+    import ctypes as C
+    conv = []
+    for a in args:
+        if hasattr(a, "_h"):
+            conv.append(a._h)
+        elif isinstance(a, int):
+            conv.append(C.c_uint32(a))
+        else:
+            conv.append(a)
+    conv = tuple(conv)
+
+    def call():
+        if fn(*conv) != 0:
+            raise RuntimeError("library call failed inside a timing loop")
+    return call
+
+
+def matvec_alg_bytes(pkg, fmt, rows, cols):
+    return pkg.synth.weight_bytes(fmt, rows, cols) + cols * 4 + rows * 4
+
+
+def bench_matvec_grouped(pkg, ctx, K, fmt, rows, cols, steps, warmup, total_bytes=1 << 30):
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(1 if fmt == "q4_0" else 2, rows)
+    raw = pkg.synth.weights(fmt, rows, cols, g)
+    R = max(1, -(-total_bytes // raw.size))
+    big, ws = distinct_replicas(pkg, ctx, raw, R, 18 if fmt == "q4_0" else 66)
+    x = pkg.synth.activations(1, cols, g)[0]
+    xb = pkg.Buffer.from_slice(ctx, x)
+    yall = pkg.Buffer.empty(ctx, R * rows * 4)
+    ys = [yall.view(i * rows * 4, rows * 4) for i in range(R)]
+    xs = [xb] * R
+    batch = pkg.CommandBatch(ctx)
+
+    def step():
+        K.matvec_quant_grouped_into(batch, ty, ws, xs, pkg.F32, ys, pkg.F32, rows, cols)
+
+    wall, ev = time_steps(pkg, ctx, step, steps, warmup)
+    alg = R * matvec_alg_bytes(pkg, fmt, rows, cols)
+    return {"replicas": R, "ms_per_step_wall": wall, "ms_per_launch_events": ev, "alg_bytes_per_launch": alg,
+            "gbs_wall": alg / wall * 1e-6, "gbs_events": alg / ev * 1e-6,
+            "_state": (raw, x, ws, xb, ys, big, yall)}
+
+
+def bench_matvec_single(pkg, ctx, K, fmt, rows, cols, steps, warmup):
+    """One ordinary launch per step (no grouping); replicas rotate so the weights come from HBM."""
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(7, rows)
+    raw = pkg.synth.weights(fmt, rows, cols, g)
+    R = max(2, min(8, (1 << 30) // raw.size))
+    big, ws = distinct_replicas(pkg, ctx, raw, R, 18 if fmt == "q4_0" else 66)
+    xb = pkg.Buffer.from_slice(ctx, pkg.synth.activations(1, cols, g)[0])
+    yb = pkg.Buffer.empty(ctx, rows * 4)
+    batch = pkg.CommandBatch(ctx)
+    import ctypes as C
+    calls = [bound_call(pkg.lib().lh_matvec_quant_typed_into, batch, C.c_int(ty), w, xb, C.c_int(pkg.F32), yb, C.c_int(pkg.F32),
+                        rows, cols) for w in ws]
+    it = [0]
+
+    def step():
+        calls[it[0] % R]()
+        it[0] += 1
+
+    wall, ev = time_steps(pkg, ctx, step, steps, warmup)
+    alg = matvec_alg_bytes(pkg, fmt, rows, cols)
+    return {"us_per_launch": ev * 1e3, "gbs": alg / ev * 1e-6, "alg_bytes": alg}
+
+
+def make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits):
+    """By-lane KV pool [lanes * T] encoded on the GPU from f16 N(0,1) rows (distinct per lane)."""
+    from local_ai_amd import kv_cache
+    cb = kv_cache.code_bytes(hd, bits)
+    levels = pkg.Buffer.from_slice(ctx, kv_cache.turboquant_levels(hd, bits))
+    signs = pkg.Buffer.from_slice(ctx, kv_cache.turboquant_signs(hd))
+    pool = [pkg.Buffer.empty(ctx, lanes * T * nkv * cb), pkg.Buffer.empty(ctx, lanes * T * nkv * 2),
+            pkg.Buffer.empty(ctx, lanes * T * nkv * cb), pkg.Buffer.empty(ctx, lanes * T * nkv * 2)]
+    g = pkg.synth.rng(5, T)
+    batch = pkg.CommandBatch(ctx)
+    chunk = 8192
+    for which in (0, 2):                       # lane 0 is encoded from fresh f16 N(0,1) rows ...
+        for t0 in range(0, T, chunk):
+            n = min(chunk, T - t0)
+            rows = pkg.Buffer.from_slice(ctx, pkg.synth.kv_rows(n, nkv, hd, g))
+            K.encode_kv_turboquant_into(batch, rows, levels, signs, pool[which], pool[which + 1], hd, nkv, n, bits, t0, 0)
+            batch.commit_and_wait()
+    for l in range(1, lanes):                  # ... the others are rotations of it (distinct addresses and contents)
+        r = (l * 997) % T
+        for buf, unit in ((pool[0], nkv * cb), (pool[1], nkv * 2), (pool[2], nkv * cb), (pool[3], nkv * 2)):
+            batch.blit_copy(buf, r * unit, buf, l * T * unit, (T - r) * unit)
+            if r:
+                batch.blit_copy(buf, 0, buf, (l * T + T - r) * unit, r * unit)
+    batch.commit_and_wait()
+    return pool, levels, signs
+
+
+def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits)
+    g = pkg.synth.rng(5, 1)
+    q = g.standard_normal((lanes, nq, hd), dtype=np.float32).astype(np.float16)
+    qb = pkg.Buffer.from_slice(ctx, q)
+    rq = pkg.Buffer.empty(ctx, lanes * nq * hd * 4)
+    out = pkg.Buffer.empty(ctx, lanes * nq * hd * 4)
+    positions = pkg.Buffer.from_slice(ctx, np.full(lanes, T - 1, np.uint32))
+    batch = pkg.CommandBatch(ctx)
+    K.hadamard_rotate_hf_into(batch, qb, signs, rq, hd, lanes * nq, True, False)
+    batch.commit_and_wait()
+    per_pos = nkv * (2 * (hd * bits // 8) + 4)
+
+    def step_batched():
+        K.flash_attention_tq_batched_into(batch, rq, pool[0], pool[1], pool[2], pool[3], levels, out, positions, hd, T, nq, nkv,
+                                          0, bits, lanes, 0)
+
+    _, ev_b = time_steps(pkg, ctx, step_batched, steps, warmup)
+    cb = hd * bits // 8
+    views = [[pool[0].view(l * T * nkv * cb, T * nkv * cb), pool[1].view(l * T * nkv * 2, T * nkv * 2),
+              pool[2].view(l * T * nkv * cb, T * nkv * cb), pool[3].view(l * T * nkv * 2, T * nkv * 2)] for l in range(lanes)]
+    it = [0]
+    calls = [bound_call(pkg.lib().lh_flash_attention_tq_into, batch, rq, v[0], v[1], v[2], v[3], levels, out, hd, T, T - 1, nq, nkv,
+                        0, bits, 0) for v in views]
+
+    def step_single():   # one decode token of one sequence; sequences rotate so the cache comes from HBM
+        calls[it[0] % lanes]()
+        it[0] += 1
+
+    _, ev_s = time_steps(pkg, ctx, step_single, max(steps, 20), warmup)
+    return {"context": T, "bytes_per_position": per_pos,
+            "batched_lanes": lanes, "batched_us_per_launch": ev_b * 1e3,
+            "batched_tokens_per_s": lanes / (ev_b * 1e-3), "batched_gbs": lanes * T * per_pos / ev_b * 1e-6,
+            "single_us_per_token": ev_s * 1e3, "single_tokens_per_s": 1.0 / (ev_s * 1e-3),
+            "single_gbs": T * per_pos / ev_s * 1e-6}
+
+
+def bench_layer(pkg, ctx, K, steps, warmup):
+    """Small-batch decode over one decoder layer's seven projections (mixed Q4_0 / TQ2_0)."""
+    g = pkg.synth.rng(3)
+    ws = []
+    for name, fmt, n, k in pkg.synth.DECODER_LAYER:
+        ws.append((pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k), n, k))
+    wbytes = sum(w.device_bytes() for w, _, _ in ws)
+    res = {"weight_bytes": wbytes}
+    batch = pkg.CommandBatch(ctx)
+    for m in (1, 4, 8, 16):
+        a2k = pkg.Buffer.from_slice(ctx, pkg.synth.activations(m, 2048, g))
+        a8k = pkg.Buffer.from_slice(ctx, pkg.synth.activations(m, 8192, g))
+        outs = [pkg.Buffer.empty(ctx, m * n * 4) for _, n, _ in ws]
+        import ctypes as C
+        calls = [bound_call(pkg.lib().lh_matmul_nt_quant_typed_into, batch, C.c_int(w.ty), a2k if k == 2048 else a8k, C.c_int(pkg.F32),
+                            w.buf, o, C.c_int(pkg.F32), m, k, n) for (w, n, k), o in zip(ws, outs)]
+
+        def step():
+            for c in calls:
+                c()
+
+        _, ev = time_steps(pkg, ctx, step, steps, warmup)
+        res[f"m{m}_us_per_layer"] = ev * 1e3
+        res[f"m{m}_gbs_hot"] = wbytes / ev * 1e-6       # weights stay in the 256 MB last-level cache here
+    return res
+
+
+def bench_prefill(pkg, ctx, K, steps, warmup):
+    m, k, n = 512, 2048, 8192
+    res = {}
+    batch = pkg.CommandBatch(ctx)
+    for fmt in ("tq2_0", "q4_0"):
+        g = pkg.synth.rng(4, 1 if fmt == "q4_0" else 2)
+        w = pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k)
+        ab = pkg.Buffer.from_slice(ctx, pkg.synth.f32_to_bf16_bits(pkg.synth.activations(m, k, g)))
+        cb = pkg.Buffer.empty(ctx, m * n * 4)
+
+        def step():
+            w.matmul_nt_typed_into(batch, K, ab, pkg.BF16, cb, pkg.F32, m)
+
+        _, ev = time_steps(pkg, ctx, step, steps, warmup)
+        tf = 2.0 * m * k * n / (ev * 1e-3) * 1e-12
+        res[fmt] = {"us": ev * 1e3, "tflops": tf, "frac_of_f16_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+    return res
+
+
+def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
+    """CPU restatement of the reference path on the host cores: bounded sample of the same workload."""
+    from oracle import oracle as orc
+    threads = min(orc.max_threads(), os.cpu_count() or 1)
+    alg = matvec_alg_bytes(pkg, "tq2_0", rows, cols)
+    t0 = time.perf_counter()
+    orc.matvec_quant_ref("tq2_0", raw, x, rows, cols, threads=threads)
+    one = time.perf_counter() - t0
+    reps = int(max(1, min(2000, target_s / max(one, 1e-4))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        y = orc.matvec_quant_ref("tq2_0", raw, x, rows, cols, threads=threads)
+    dt = time.perf_counter() - t0
+    t1 = time.perf_counter()
+    orc.matvec_quant_ref("tq2_0", raw, x, rows, cols, threads=1)
+    single = time.perf_counter() - t1
+    return {"value": alg * reps / dt * 1e-9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} repetitions of one 8192x2048 TQ2_0 matvec ({dt:.1f} s, OpenMP over rows); "
+                      f"single thread: {alg / single * 1e-9:.3f} GB/s"}, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--quick", action="store_true", help="headline measurement only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: the hot path is a single-GPU kernel path and no multi-GPU "
+              "figure exists for it; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    ctx = pkg.Context(0)
+    K = pkg.Kernels(ctx)
+    log("[bench] device:", ctx.device_name(), "CUs:", ctx.compute_units())
+
+    # A plain copy of known size first: the reference point for the HBM traffic counters when this
+    # command runs under rocprofv3 --pmc (256 MiB read + 256 MiB written by blit_copy16_kernel).
+    cal_src, cal_dst = pkg.Buffer.empty(ctx, 256 << 20), pkg.Buffer.empty(ctx, 256 << 20)
+    cal_batch = pkg.CommandBatch(ctx)
+    cal_batch.blit_copy(cal_src, 0, cal_dst, 0, 256 << 20)
+    cal_batch.commit_and_wait()
+    cal_src.free(); cal_dst.free()
+
+    rows, cols = 8192, 2048
+    head = bench_matvec_grouped(pkg, ctx, K, "tq2_0", rows, cols, args.steps, args.warmup)
+    raw, x, ws, xb, ys, _, _ = head.pop("_state")
+    log(f"[bench] TQ2_0 {rows}x{cols} x{head['replicas']}: {head['gbs_wall']:.0f} GB/s wall, {head['gbs_events']:.0f} GB/s events")
+
+    # parity of what was just timed: replica 0 against the CPU path
+    extra = {}
+    cpu = None
+    if not args.no_cpu:
+        cpu, y_cpu = cpu_baseline(pkg, raw, x, rows, cols)
+        got = ys[0].as_array(np.float32, rows)
+        err = float(np.max(np.abs(got - y_cpu) / np.maximum(np.abs(y_cpu), 1.0)))
+        extra["parity_max_norm_err_vs_cpu_path"] = err
+        log(f"[bench] CPU baseline {cpu['value']:.2f} GB/s on {cpu['cores']} threads; parity err {err:.2e}")
+        if err > 1e-3:
+            log("[bench] PARITY FAILURE: GPU result differs from the CPU path beyond 1e-3")
+            sys.exit(1)
+
+    if not args.quick:
+        del ws, ys
+        for fmt, r, c in (("q4_0", 2048, 2048), ("tq2_0", 2048, 8192)):
+            res = bench_matvec_grouped(pkg, ctx, K, fmt, r, c, args.steps, args.warmup)
+            res.pop("_state")
+            extra[f"matvec_{fmt}_{r}x{c}_grouped"] = {k: res[k] for k in ("replicas", "ms_per_launch_events", "gbs_events")}
+            extra[f"matvec_{fmt}_{r}x{c}_grouped"]["frac_of_hbm_peak"] = res["gbs_events"] / HBM_PEAK_GBS
+            log(f"[bench] {fmt} {r}x{c} grouped: {res['gbs_events']:.0f} GB/s")
+        for fmt, r, c in (("q4_0", 262144, 1536), ("tq2_0", 8192, 2048), ("q4_0", 2048, 2048)):
+            res = bench_matvec_single(pkg, ctx, K, fmt, r, c, max(args.steps, 50), args.warmup)
+            res["frac_of_hbm_peak"] = res["gbs"] / HBM_PEAK_GBS
+            extra[f"matvec_{fmt}_{r}x{c}_single_launch"] = res
+            log(f"[bench] {fmt} {r}x{c} single launch: {res['us_per_launch']:.1f} us, {res['gbs']:.0f} GB/s")
+        att = bench_attention(pkg, ctx, K, args.steps, args.warmup)
+        att["batched_frac_of_hbm_peak"] = att["batched_gbs"] / HBM_PEAK_GBS
+        extra["tq2_attention_32k"] = att
+        log(f"[bench] tq2 attention 32k: batched {att['batched_tokens_per_s']:.0f} tok/s ({att['batched_gbs']:.0f} GB/s), "
+            f"single {att['single_us_per_token']:.1f} us/token")
+        extra["decoder_layer_small_batch"] = bench_layer(pkg, ctx, K, args.steps, args.warmup)
+        extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
+        log("[bench] layer:", extra["decoder_layer_small_batch"])
+        log("[bench] prefill:", extra["prefill_matmul_512x2048x8192_bf16"])
+
+    achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
+    line = {
+        "metric": "Q4_0/TQ2_0 matvec HBM GB/s (% of peak) at M=1; tq2 KV attn tokens/s @32k",
+        "value": head["gbs_wall"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step_wall"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",   # 2-bit / 4-bit codes x 8-bit activation limbs on v_dot4_i32_i8, f32 block scales
+        "data": "synthetic",
+        "config": {"workload": "TQ2_0 fused dequant-matvec, M=1, N=8192 x K=2048 (MLP gate/up), fp32 x and y",
+                   "replicas_per_step": head["replicas"], "launches_per_step": 1,
+                   "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "matvec_quant_kernel<TQ2_0>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
+                     "launch_ms": head["ms_per_launch_events"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -218,26 +218,47 @@ __global__ __launch_bounds__(kThreads) void attention_tq_split_kernel(
     }
 }
 
-// flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.
+// flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.  One workgroup per
+// (query, head); the per-split factors exp(m_s - max) are computed once into LDS, then every thread
+// folds its output dimension over the splits with coalesced row reads.
+constexpr int kMaxSplits = 1024;
 __global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
                                                                  uint32_t num_splits) {
+    __shared__ float f_s[kMaxSplits];
+    __shared__ float red[8];
     const uint32_t qh = blockIdx.x;     // flattened (query, head)
-    const float* base = ws + (size_t)qh * num_splits * (head_dim + 4);
-    float gm = -INFINITY;
-    for (uint32_t s = 0; s < num_splits; s++) gm = fmaxf(gm, base[(size_t)s * (head_dim + 4)]);
-    float gl = 0.0f;
-    for (uint32_t s = 0; s < num_splits; s++) {
-        const float m = base[(size_t)s * (head_dim + 4)];
-        gl += (m == -INFINITY ? 0.0f : __expf(m - gm)) * base[(size_t)s * (head_dim + 4) + 1];
+    const size_t rec = (size_t)head_dim + 4;
+    const float* base = ws + (size_t)qh * num_splits * rec;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float m_loc = -INFINITY;
+    for (uint32_t s = threadIdx.x; s < num_splits; s += 256) { const float m = base[s * rec]; f_s[s] = m; m_loc = fmaxf(m_loc, m); }
+    m_loc = lh_group_max(m_loc, 64);
+    if (lane == 0) red[wave] = m_loc;
+    __syncthreads();
+    const float gm = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float l_loc = 0.0f;
+    for (uint32_t s = threadIdx.x; s < num_splits; s += 256) {
+        const float m = f_s[s];
+        const float f = m == -INFINITY ? 0.0f : __expf(m - gm);
+        f_s[s] = f;
+        l_loc += f * base[s * rec + 1];
     }
+    l_loc = lh_group_sum(l_loc, 64);
+    if (lane == 0) red[4 + wave] = l_loc;
+    __syncthreads();
+    const float gl = (red[4] + red[5]) + (red[6] + red[7]);
     const float inv = gl > 0.0f ? 1.0f / gl : 0.0f;
-    for (uint32_t d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float o = 0.0f;
-        for (uint32_t s = 0; s < num_splits; s++) {
-            const float m = base[(size_t)s * (head_dim + 4)];
-            o += (m == -INFINITY ? 0.0f : __expf(m - gm)) * base[(size_t)s * (head_dim + 4) + 4 + d];
+    for (uint32_t d = threadIdx.x; d < head_dim; d += 256) {
+        float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+        uint32_t s = 0;
+        for (; s + 4 <= num_splits; s += 4) {
+            o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
+            o1 += f_s[s + 1] * base[(size_t)(s + 1) * rec + 4 + d];
+            o2 += f_s[s + 2] * base[(size_t)(s + 2) * rec + 4 + d];
+            o3 += f_s[s + 3] * base[(size_t)(s + 3) * rec + 4 + d];
         }
-        out[(size_t)qh * head_dim + d] = o * inv;
+        for (; s < num_splits; s++) o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
+        out[(size_t)qh * head_dim + d] = ((o0 + o1) + (o2 + o3)) * inv;
     }
 }
 
@@ -266,7 +287,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
     const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
     uint64_t splits = std::min<uint64_t>(per_query_wgs, (max_span + 31) / 32);
-    splits = std::max<uint64_t>(splits, 1);
+    splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
     const size_t rec = (size_t)p.head_dim + 4;
     const size_t ws_avail = (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_avail) splits--;

@@ -257,8 +257,8 @@ template <int FMT> __host__ __device__ constexpr int steps_in_flight(int npos) {
 
 // One launch serves `count` problems of the same shape (count == 1 for the plain matvec).
 template <int FMT, int L, int NPOS, typename XT, typename YT>
-__global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, uint32_t count,
-                                                             uint32_t rows, uint32_t K, uint32_t lpr_log2,
+__global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, MatvecProblem single,
+                                                             uint32_t count, uint32_t rows, uint32_t K, uint32_t lpr_log2,
                                                              uint32_t steps_per_wg) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int G = FMT == LH_TQ2_0 ? 256 : 32;
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         const uint32_t s_begin = (uint32_t)(g0 - (uint64_t)prob * steps_per_problem);
         const uint64_t seg_end64 = (uint64_t)(prob + 1) * steps_per_problem;
         const uint32_t s_end = (uint32_t)((g1 < seg_end64 ? g1 : seg_end64) - (uint64_t)prob * steps_per_problem);
-        const MatvecProblem pb = problems[prob];
+        const MatvecProblem pb = problems ? problems[prob] : single;   // one problem travels in the kernel arguments
         // this wave's contiguous share of [s_begin, s_end)
         const uint32_t nseg = s_end - s_begin;
         const uint32_t per_wave = (nseg + kWaves - 1) / kWaves;
@@ -490,11 +490,11 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
 }
 
 template <int FMT, int L, int NPOS>
-int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, uint32_t count, lh_dtype xt, lh_dtype yt, uint32_t rows,
-                 uint32_t K, const LaunchGeom& g) {
+int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const MatvecProblem& single, uint32_t count, lh_dtype xt,
+                 lh_dtype yt, uint32_t rows, uint32_t K, const LaunchGeom& g) {
 #define LH_LAUNCH(XT, YT)                                                                                              \
     hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream, \
-                       dev_problems, count, rows, K, g.lpr_log2, g.steps_per_wg)
+                       dev_problems, single, count, rows, K, g.lpr_log2, g.steps_per_wg)
     if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
     else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
@@ -504,13 +504,13 @@ int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, uint32_t co
 }
 
 template <int FMT, int L>
-int launch_npos(lh_context* ctx, const MatvecProblem* p, uint32_t count, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K,
-                const LaunchGeom& g) {
+int launch_npos(lh_context* ctx, const MatvecProblem* p, const MatvecProblem& single, uint32_t count, lh_dtype xt, lh_dtype yt,
+                uint32_t rows, uint32_t K, const LaunchGeom& g) {
     switch (g.npos) {
-        case 1: return launch_typed<FMT, L, 1>(ctx, p, count, xt, yt, rows, K, g);
-        case 2: return launch_typed<FMT, L, 2>(ctx, p, count, xt, yt, rows, K, g);
-        case 3: return launch_typed<FMT, L, 3>(ctx, p, count, xt, yt, rows, K, g);
-        default: return launch_typed<FMT, L, 4>(ctx, p, count, xt, yt, rows, K, g);
+        case 1: return launch_typed<FMT, L, 1>(ctx, p, single, count, xt, yt, rows, K, g);
+        case 2: return launch_typed<FMT, L, 2>(ctx, p, single, count, xt, yt, rows, K, g);
+        case 3: return launch_typed<FMT, L, 3>(ctx, p, single, count, xt, yt, rows, K, g);
+        default: return launch_typed<FMT, L, 4>(ctx, p, single, count, xt, yt, rows, K, g);
     }
 }
 
@@ -565,31 +565,34 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         }
         return LH_OK;
     }
-    // Problem descriptors live in the context's descriptor ring in device memory.
-    const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
-    if (desc_bytes > ctx->workspace_bytes / 4)
-        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u problems exceed the descriptor area", op, count);
-    MatvecProblem stack_desc[8];
-    MatvecProblem* host_desc = count <= 8 ? stack_desc : (MatvecProblem*)malloc(desc_bytes);
-    if (!host_desc) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", desc_bytes);
-    for (uint32_t i = 0; i < count; i++) {
-        host_desc[i].matrix = (const uint8_t*)matrices[i]->ptr;
-        host_desc[i].vector = vectors[i]->ptr;
-        host_desc[i].output = outputs[i]->ptr;
+    // One problem travels in the kernel arguments; several go through a descriptor array in the
+    // top quarter of the context workspace (the copy is stream ordered, so it cannot overtake a
+    // kernel that still reads the previous set).
+    MatvecProblem single{(const uint8_t*)matrices[0]->ptr, vectors[0]->ptr, outputs[0]->ptr};
+    MatvecProblem* dev_desc = nullptr;
+    if (count > 1) {
+        const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
+        if (desc_bytes > ctx->workspace_bytes / 4)
+            return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u problems exceed the descriptor area", op, count);
+        MatvecProblem* host_desc = (MatvecProblem*)malloc(desc_bytes);
+        if (!host_desc) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", desc_bytes);
+        for (uint32_t i = 0; i < count; i++) {
+            host_desc[i].matrix = (const uint8_t*)matrices[i]->ptr;
+            host_desc[i].vector = vectors[i]->ptr;
+            host_desc[i].output = outputs[i]->ptr;
+        }
+        dev_desc = (MatvecProblem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
+        hipError_t e = hipMemcpyAsync(dev_desc, host_desc, desc_bytes, hipMemcpyHostToDevice, ctx->stream);
+        free(host_desc);   // pageable source: the runtime has staged it when the call returns
+        if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
     }
-    // The descriptor area is the top quarter of the workspace; the copy is stream
-    // ordered, so it cannot overtake a kernel that still reads the previous set.
-    MatvecProblem* dev_desc = (MatvecProblem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
-    hipError_t e = hipMemcpyAsync(dev_desc, host_desc, desc_bytes, hipMemcpyHostToDevice, ctx->stream);
-    if (count > 8) free(host_desc);
-    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
     const int L = x_limbs();
     const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L);
     int r;
-    if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, count, xt, yt, rows, cols, g)
-                                   : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, count, xt, yt, rows, cols, g);
-    else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, count, xt, yt, rows, cols, g)
-                    : launch_npos<LH_TQ2_0, 3>(ctx, dev_desc, count, xt, yt, rows, cols, g);
+    if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
+                                   : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
+    else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
+                    : launch_npos<LH_TQ2_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
 }
