@@ -21,6 +21,7 @@ struct lh_buffer {
     void* ptr;
     size_t len;
     bool owns;
+    size_t slack;   // readable bytes behind ptr + len (allocation padding, or the rest of a viewed parent)
 };
 
 struct lh_batch {
@@ -55,6 +56,10 @@ static inline int lh_need(const lh_buffer* b, size_t bytes, const char* op, cons
         int r__ = lh_need((buf), (bytes), (op), (name));     \
         if (r__ != LH_OK) return r__;                        \
     } while (0)
+
+// TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.
+int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
+                              void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K);
 
 static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }
 

@@ -20,6 +20,7 @@
 //  * Row sums use DPP / swizzle butterflies inside the wave (fixed pairing
 //    order, so results are bit-reproducible run to run).
 #include "common.hpp"
+#include "xquant.hpp"
 #include <cstdlib>
 
 namespace {
@@ -33,68 +34,6 @@ struct MatvecProblem {
     const void* vector;
     void* output;
 };
-
-template <int L> struct Limb;
-template <> struct Limb<2> { static constexpr float qmax = 32639.0f; };     // 127*256 + 127
-template <> struct Limb<3> { static constexpr float qmax = 8355711.0f; };   // 127*65536 + 127*256 + 127
-
-// ---- activation quantisation into LDS ----------------------------------------
-// xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
-// xs[K/G]: float scale of each group of G elements (G = weight block size).
-template <int L, int G, typename XT>
-__device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs) {
-    const int tid = threadIdx.x;
-    const uint32_t kq = K >> 2;
-    for (uint32_t base = 0; base < K; base += kWG * 8) {
-        const uint32_t e0 = base + tid * 8;
-        const bool valid = e0 < K;
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.0f;
-        if (valid) {
-            if constexpr (sizeof(XT) == 4) {
-                const float4 a = *reinterpret_cast<const float4*>(x + e0);
-                const float4 b = *reinterpret_cast<const float4*>(x + e0 + 4);
-                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-            } else {
-                const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
-                const uint32_t w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    v[2 * i] = lh_h2f((uint16_t)(w[i] & 0xFFFF));
-                    v[2 * i + 1] = lh_h2f((uint16_t)(w[i] >> 16));
-                }
-            }
-        }
-        float m = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-        m = lh_group_max(m, G / 8);
-        const float inv = m > 0.0f ? Limb<L>::qmax / m : 0.0f;
-        uint32_t packed[L][2];
-#pragma unroll
-        for (int l = 0; l < L; l++) packed[l][0] = packed[l][1] = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            float r = rintf(v[i] * inv);
-            r = fminf(fmaxf(r, -Limb<L>::qmax), Limb<L>::qmax);
-            int n = (int)r;
-#pragma unroll
-            for (int l = 0; l < L; l++) {
-                int limb;
-                if (l == L - 1) limb = n;                       // top limb: what is left, fits a signed byte
-                else { limb = (int)(int8_t)(n & 0xFF); n = (n - limb) >> 8; }
-                packed[l][i >> 2] |= (uint32_t)(limb & 0xFF) << (8 * (i & 3));
-            }
-        }
-        if (valid) {
-#pragma unroll
-            for (int l = 0; l < L; l++)
-                *reinterpret_cast<uint2*>(&xq[l * kq + (e0 >> 2)]) = make_uint2(packed[l][0], packed[l][1]);
-            if ((e0 & (G - 1)) == 0) xs[e0 / G] = m * (1.0f / Limb<L>::qmax);
-        }
-    }
-}
 
 // ---- per-lane activation registers for one unit column -------------------------
 template <int FMT, int L>
@@ -295,7 +234,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
 
         if (pb.vector != staged_vector) {
             __syncthreads();   // every wave is done reading the previous vector's limbs
-            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs);
+            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG);
             __syncthreads();
 #pragma unroll
             for (int p = 0; p < NPOS; p++) {
@@ -454,6 +393,15 @@ int x_limbs() {
     return v;
 }
 
+// LOCAL_HIP_TQ2_KERNEL=valu selects the vector-ALU (v_dot4) TQ2_0 kernel instead of the MFMA one.
+bool tq2_on_matrix_cores() {
+    static bool v = [] {
+        const char* e = getenv("LOCAL_HIP_TQ2_KERNEL");
+        return !(e && e[0] == 'v') && x_limbs() == 2;
+    }();
+    return v;
+}
+
 int wg_per_cu() {
     static int v = [] {
         const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU");
@@ -549,11 +497,14 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     lh_context* ctx = batch->ctx;
     const size_t wbytes = (size_t)rows * (cols / blk) * (fmt == LH_Q4_0 ? 18 : 66);
     bool fast = true;
+    size_t min_slack = ~(size_t)0;   // the staged TQ2_0 kernel reads whole 16-byte chunks: up to 14 bytes past a ragged row
     for (uint32_t i = 0; i < count; i++) {
         LH_NEED(matrices[i], wbytes, op, "matrix");
         LH_NEED(vectors[i], (size_t)cols * lh_dtype_size(xt), op, "vector");
         LH_NEED(outputs[i], (size_t)rows * lh_dtype_size(yt), op, "output");
         fast = fast && fast_path_ok(fmt, matrices[i]->ptr, vectors[i]->ptr, cols);
+        const size_t sl = matrices[i]->len - wbytes + matrices[i]->slack;
+        if (sl < min_slack) min_slack = sl;
     }
     if (!fast) {
         for (uint32_t i = 0; i < count; i++) {
@@ -564,6 +515,18 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
             batch->dispatch_count++;
         }
         return LH_OK;
+    }
+    if (fmt == LH_TQ2_0 && tq2_on_matrix_cores() && cols <= 12288 && ((cols / 256) % 8 == 0 || min_slack >= 16)) {
+        const void* stack_m[8]; const void* stack_x[8]; void* stack_y[8];
+        const void** pm = count <= 8 ? stack_m : (const void**)malloc(sizeof(void*) * 3 * count);
+        if (!pm) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(void*) * 3 * (size_t)count);
+        const void** px = count <= 8 ? stack_x : pm + count;
+        void** py = count <= 8 ? stack_y : (void**)(pm + 2 * (size_t)count);
+        for (uint32_t i = 0; i < count; i++) { pm[i] = matrices[i]->ptr; px[i] = vectors[i]->ptr; py[i] = outputs[i]->ptr; }
+        int r = lh_launch_matvec_tq2_mfma(ctx, count, pm, px, py, xt, yt, rows, cols);
+        if (count > 8) free((void*)pm);
+        if (r == LH_OK) batch->dispatch_count++;
+        return r;
     }
     // One problem travels in the kernel arguments; several go through a descriptor array in the
     // top quarter of the context workspace (the copy is stream ordered, so it cannot overtake a

@@ -1,0 +1,281 @@
+// TQ2_0 fused dequant matvec (M = 1) with the inner products on the matrix cores.
+//
+// Same contract as the TQ2_0 path of matvec_quant.hip (stands in for
+// shaders/matvec_quant.metal:173-312).  At 3.9 weights per byte the 2-bit unpack plus
+// v_dot4 arithmetic of the vector-ALU kernel costs more issue slots than the HBM stream
+// leaves free; here the vector ALU only isolates the 2-bit codes and the integer dot
+// products run as v_mfma_i32_16x16x64_i8.
+//
+// One wave works on tiles of 16 weight rows x (up to) 8 blocks = 2048 columns:
+//   1. The tile's bytes (codes AND the f16 block scales, verbatim GGUF order) are
+//      fetched with fully coalesced 128-bit loads -- consecutive lanes read consecutive
+//      16-byte chunks of a row -- into registers one tile ahead, then parked in a
+//      wave-private LDS image.  (Loading in MFMA operand order straight from global
+//      memory makes every 4-lane group touch 4 different rows, and separate 2-byte
+//      scale loads cost more than the whole code stream: both were measured.)
+//   2. Lane (r = lane % 16, g = lane / 16) takes quarter g of block b of row r from the
+//      image: two aligned ds_read_b128 plus a constant funnel shift (blocks start on
+//      2-byte boundaries).  (codes >> 2f) & 0x03030303 for field f is the MFMA A
+//      operand: 16 rows x 64 k.
+//   3. The B operand holds the activation limbs (16-bit block fixed point, see
+//      xquant.hpp) of those 64 elements in columns 2b (low limb) and 2b + 1 (high limb)
+//      and zeros elsewhere, read from LDS (lanes of other columns read a zero line), so
+//      one accumulator tile D[16 rows][16 cols] collects all 8 blocks x 2 limbs.
+//   4. Per tile the dense accumulator is combined (limbs, zero point), multiplied by
+//      d * s per (row, block) -- the scales come from the same LDS image -- and the 16
+//      columns are summed with DPP.
+#include "common.hpp"
+#include "xquant.hpp"
+#include <cstdlib>
+
+namespace {
+
+constexpr int kL = 2;                        // activation limbs (16-bit block fixed point)
+constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
+constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
+constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+struct Tq2Problem {
+    const uint8_t* matrix;
+    const void* vector;
+    void* output;
+};
+
+__device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p);
+}
+
+// 16 bytes starting `SH` bytes into the 32-byte pair (c0, c1).
+template <int SH>
+__device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uint32_t (&out)[4]) {
+    const uint32_t in[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    constexpr int q = SH >> 2, rem = SH & 3;
+#pragma unroll
+    for (int m = 0; m < 4; m++) out[m] = rem ? __builtin_amdgcn_alignbit(in[m + q + 1], in[m + q], 8 * rem) : in[m + q];
+}
+
+template <typename XT, typename YT>
+__global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Problem single,
+                                                                uint32_t count, uint32_t rows, uint32_t K) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t nb = K >> 8;                                     // blocks per row
+    uint32_t* xq = reinterpret_cast<uint32_t*>(lds);                // [2][K/4] activation limbs
+    float* xs = reinterpret_cast<float*>(lds + (size_t)kL * K);     // [nb] activation scales
+    int* xn = reinterpret_cast<int*>(xs + nb);                      // [nb] sum of the block's integers
+    const uint32_t kq = K >> 2;
+    const uint32_t row_bytes = nb * 66;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const uint32_t r = lane & 15, g = lane >> 4;                    // A layout: row r, quarter g
+    const uint32_t c = lane & 15;                                   // B / D layout: column c, k-group / row-group g
+    const uint32_t cb = c >> 1, cl = c & 1;                         // column's block (within a group of 8) and limb
+    const uint32_t lane_x_off = 4u * (cl * kq + (g >> 1) * 32u + (g & 1) * 4u);
+    const uint32_t zero_off = (uint32_t)((size_t)kL * K + (size_t)nb * 8);      // 128 bytes of zeros behind xs / xn
+    if (threadIdx.x < 32) reinterpret_cast<uint32_t*>(lds + zero_off)[threadIdx.x] = 0;
+    uint8_t* image = lds + zero_off + 128 + (size_t)wave * kImageBytes;         // this wave's tile image
+
+    // Work order: "slots" of nwaves consecutive tiles, dealt round-robin to the workgroups, so that at any moment
+    // the whole grid reads one compact, advancing window of the weight stream.
+    const uint32_t tiles_per_problem = (rows + 15) >> 4;
+    const uint32_t slots_per_problem = (tiles_per_problem + nwaves - 1) / nwaves;
+    const uint64_t total_slots = (uint64_t)slots_per_problem * count;
+    const uint32_t ngroups = (nb + 7) >> 3;
+    const uint64_t my_slots = blockIdx.x < total_slots ? (total_slots - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const uint64_t nitems = my_slots * ngroups;                     // one item = one (tile, block group)
+
+    // Chunk -> (row, chunk-in-row) of the lane's staging loads, precomputed for the two group shapes a row can
+    // have: a full group of 8 blocks (33 chunks per row) and the trailing group of nb % 8 blocks.
+    const uint32_t nbg_tail = (nb & 7) ? (nb & 7) : 8;
+    uint32_t goff_full[kStageLoads], loff_full[kStageLoads], goff_tail[kStageLoads], loff_tail[kStageLoads];
+    {
+        const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
+#pragma unroll
+        for (int i = 0; i < kStageLoads; i++) {
+            const uint32_t ch = lane + 64 * i;
+            const uint32_t cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
+            goff_full[i] = rf * row_bytes + jf * 16;
+            loff_full[i] = ch < 16 * 33 ? rf * (33 * 16) + jf * 16 : 0xFFFFFFFFu;        // surplus lanes do not store
+            const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
+            goff_tail[i] = rt * row_bytes + jt * 16;
+            loff_tail[i] = ch < 16 * nch_t ? rt * ss_t + jt * 16 : 0xFFFFFFFFu;
+        }
+    }
+    auto item_tile_base = [&](uint64_t n, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
+        const uint64_t slot = (uint64_t)blockIdx.x + (n / ngroups) * gridDim.x;
+        grp = (uint32_t)(n % ngroups);
+        const uint32_t prob = (uint32_t)(slot / slots_per_problem);
+        tile = (uint32_t)(slot - (uint64_t)prob * slots_per_problem) * nwaves + wave;
+        pb = problems ? problems[prob] : single;
+    };
+
+    u32x4_t pre[kStageLoads];
+    auto prefetch = [&](uint64_t n) {
+        uint32_t grp, tile; Tq2Problem pb;
+        item_tile_base(n, grp, tile, pb);
+        const bool tail = grp + 1 == ngroups && (nb & 7);
+        if ((tile << 4) + 16 <= rows) {                              // every row of the tile exists: precomputed offsets
+            gptr_t base = (gptr_t)pb.matrix + (size_t)(tile << 4) * row_bytes + (size_t)grp * 528;
+            if (!tail) {
+#pragma unroll
+                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + goff_full[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + goff_tail[i]);
+            }
+        } else {                                                     // last, partial tile (or a surplus wave): clamp the row
+            const uint32_t nbg = tail ? nbg_tail : 8;
+            const uint32_t nch = (nbg * 66 + 15) >> 4;
+            gptr_t base = (gptr_t)pb.matrix + (size_t)grp * 528;
+#pragma unroll
+            for (int i = 0; i < kStageLoads; i++) {
+                uint32_t ch = lane + 64 * i;
+                if (ch >= 16 * nch) ch = 16 * nch - 1;
+                const uint32_t row = ch / nch, j = ch - row * nch;
+                uint32_t grow = (tile << 4) + row;
+                if (grow >= rows) grow = rows - 1;                   // rows past the end re-read the last row (never stored)
+                pre[i] = ld16_align2(base + (size_t)grow * row_bytes + j * 16);
+            }
+        }
+    };
+
+    if (nitems) prefetch(0);
+    const void* staged = nullptr;
+    float rowacc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (uint64_t n = 0; n < nitems; n++) {
+        uint32_t grp, tile; Tq2Problem pb;
+        item_tile_base(n, grp, tile, pb);
+        if (pb.vector != staged) {                                   // uniform over the workgroup
+            __syncthreads();
+            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x);
+            __syncthreads();
+            staged = pb.vector;
+        }
+        const uint32_t b0 = grp << 3;
+        const uint32_t nbg = nb - b0 < 8 ? nb - b0 : 8;
+        const uint32_t nch = (nbg * 66 + 15) >> 4;
+        const uint32_t seg_stride = (nch | 1) * 16;                  // odd number of 16-byte chunks: conflict-free row stride
+        (void)nch;
+
+        // ---- park the prefetched chunks in the wave's LDS image, then start the next item's loads
+        __builtin_amdgcn_wave_barrier();
+        if (nbg == 8) {
+#pragma unroll
+            for (int i = 0; i < kStageLoads; i++)
+                if (loff_full[i] != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + loff_full[i]) = pre[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kStageLoads; i++)
+                if (loff_tail[i] != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + loff_tail[i]) = pre[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (n + 1 < nitems) prefetch(n + 1);
+
+        // ---- column constants of this group
+        const bool col_valid = b0 + cb < nb;
+        const uint32_t dblk = col_valid ? b0 + cb : nb - 1;
+        const float xscale16 = (col_valid && cl == 0) ? xs[dblk] * 0.0625f : 0.0f;   // high-limb columns and padding add nothing
+        const int nsum16 = col_valid ? xn[dblk] << 4 : 0;
+        const uint32_t my_off = col_valid ? lane_x_off + dblk * 256u : zero_off;
+        const uint8_t* arow = image + r * seg_stride + g * 16;
+
+        // accumulators by code scale: fields 0 and 1 arrive as code, field 2 as 4*code, field 3 as 16*code
+        v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0}, acc16 = (v4i){0, 0, 0, 0};
+#define LH_TQ2_BLOCK(B)                                                                                         \
+        if ((B) < nbg) {                                                                                        \
+            constexpr int o = (B) * 66;                                                                         \
+            const u32x4_t c0 = *reinterpret_cast<const u32x4_t*>(arow + (o & ~15));                             \
+            const u32x4_t c1 = *reinterpret_cast<const u32x4_t*>(arow + (o & ~15) + 16);                        \
+            uint32_t wv[4];                                                                                     \
+            take16<(o & 15)>(c0, c1, wv);                                                                       \
+            v4i a0, a1, a2, a3;                                                                                 \
+            _Pragma("unroll") for (int m = 0; m < 4; m++) {                                                     \
+                const uint32_t t = wv[m] >> 2;                                                                  \
+                a0[m] = (int)(wv[m] & 0x03030303u);                                                             \
+                a1[m] = (int)(t & 0x03030303u);                                                                 \
+                a2[m] = (int)(t & 0x0C0C0C0Cu);                                                                 \
+                a3[m] = (int)(t & 0x30303030u);                                                                 \
+            }                                                                                                   \
+            const uint8_t* bp = lds + (cb == (B) ? my_off : zero_off);                                          \
+            const v4i x0 = *reinterpret_cast<const v4i*>(bp);                                                   \
+            const v4i x1 = *reinterpret_cast<const v4i*>(bp + 32);                                              \
+            const v4i x2 = *reinterpret_cast<const v4i*>(bp + 64);                                              \
+            const v4i x3 = *reinterpret_cast<const v4i*>(bp + 96);                                              \
+            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, x0, acc1, 0, 0, 0);                                \
+            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, x1, acc1, 0, 0, 0);                                \
+            acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, x2, acc4, 0, 0, 0);                                \
+            acc16 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a3, x3, acc16, 0, 0, 0);                              \
+        }
+        LH_TQ2_BLOCK(0) LH_TQ2_BLOCK(1) LH_TQ2_BLOCK(2) LH_TQ2_BLOCK(3)
+        LH_TQ2_BLOCK(4) LH_TQ2_BLOCK(5) LH_TQ2_BLOCK(6) LH_TQ2_BLOCK(7)
+#undef LH_TQ2_BLOCK
+
+        // ---- epilogue on the dense accumulator: combine scales and limbs, zero point, block scales
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int t16 = (acc1[i] << 4) + (acc4[i] << 2) + acc16[i];                       // 16 * sum(code * limb)
+            const int hi = __builtin_amdgcn_update_dpp(0, t16, 0xF5, 0xF, 0xF, true);         // quad_perm [1,1,3,3]: odd neighbour
+            const int iq16 = t16 + (hi << 8) - nsum16;                                        // 16 * sum((code - 1) * n), even columns
+            const uint16_t dbits = *reinterpret_cast<const uint16_t*>(image + (4 * g + i) * seg_stride + (col_valid ? cb : nbg - 1) * 66 + 64);
+            rowacc[i] += (float)iq16 * (lh_h2f(dbits) * xscale16);
+        }
+
+        if (grp + 1 == ngroups) {      // tile complete: sum the 16 columns of each row, store 4 rows per lane group
+            YT* y = static_cast<YT*>(pb.output);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float v = rowacc[i];
+                v += lh_dpp_f<LH_DPP_QUAD_XOR1>(v);
+                v += lh_dpp_f<LH_DPP_QUAD_XOR2>(v);
+                v += lh_dpp_f<LH_DPP_HALF_MIRROR>(v);
+                v += lh_dpp_f<LH_DPP_ROW_MIRROR>(v);
+                const uint32_t orow = (tile << 4) + 4 * g + i;
+                if (c == 0 && tile < tiles_per_problem && orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                rowacc[i] = 0.0f;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+// Entry used by matvec_quant.hip's dispatcher. Arrays are host arrays of device pointers.
+int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
+                              void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K) {
+    const uint32_t nb = K >> 8;
+    const uint64_t tiles = (uint64_t)((rows + 15) >> 4) * count;
+    // small jobs: one wave per workgroup so the tiles spread over all CUs; large jobs: four waves share one
+    // quantised activation vector
+    const uint32_t threads = tiles >= (uint64_t)ctx->cu_count * 8 ? 256 : 64;
+    const uint32_t waves = threads / 64;
+    const uint64_t slots = (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
+    static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
+    const uint64_t cap = (uint64_t)ctx->cu_count * (threads == 256 ? wg_cu : 4 * wg_cu);
+    const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
+    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes;
+    if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
+
+    Tq2Problem single{(const uint8_t*)matrices[0], vectors[0], outputs[0]};
+    Tq2Problem* dev = nullptr;
+    if (count > 1) {
+        const size_t bytes = (size_t)count * sizeof(Tq2Problem);
+        if (bytes > ctx->workspace_bytes / 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems exceed the descriptor area", count);
+        Tq2Problem* host = (Tq2Problem*)malloc(bytes);
+        if (!host) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", bytes);
+        for (uint32_t i = 0; i < count; i++) host[i] = Tq2Problem{(const uint8_t*)matrices[i], vectors[i], outputs[i]};
+        dev = (Tq2Problem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
+        hipError_t e = hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream);
+        free(host);
+        if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: descriptor upload: %s", hipGetErrorString(e));
+    }
+#define LH_LAUNCH(XT, YT) \
+    hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K)
+    if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
+    else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
+    else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
+    else LH_LAUNCH(float, uint16_t);
+#undef LH_LAUNCH
+    return lh_check_launch("matvec_tq2_0");
+}

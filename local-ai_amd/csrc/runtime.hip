@@ -145,7 +145,7 @@ static int new_buffer(lh_context* ctx, size_t len, lh_buffer** out) {
     *out = nullptr;
     lh_buffer* b = new (std::nothrow) lh_buffer();
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
-    b->ctx = ctx; b->len = len; b->owns = true; b->ptr = nullptr;
+    b->ctx = ctx; b->len = len; b->owns = true; b->ptr = nullptr; b->slack = 64;
     // Room for one 16-byte over-read past the end keeps vector loads of a
     // partly filled last unit inside the allocation.
     hipError_t e = hipMalloc(&b->ptr, (len ? len : 1) + 64);
@@ -180,6 +180,7 @@ int lh_buffer_view(lh_buffer* parent, size_t offset, size_t len, lh_buffer** out
     lh_buffer* b = new (std::nothrow) lh_buffer();
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
     b->ctx = parent->ctx; b->ptr = (char*)parent->ptr + offset; b->len = len; b->owns = false;
+    b->slack = parent->len - offset - len + parent->slack;
     *out = b;
     return LH_OK;
 }
@@ -188,7 +189,7 @@ int lh_buffer_wrap(lh_context* ctx, void* device_ptr, size_t len, lh_buffer** ou
     if (!ctx || !out || (!device_ptr && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_wrap: null argument");
     lh_buffer* b = new (std::nothrow) lh_buffer();
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
-    b->ctx = ctx; b->ptr = device_ptr; b->len = len; b->owns = false;
+    b->ctx = ctx; b->ptr = device_ptr; b->len = len; b->owns = false; b->slack = 0;
     *out = b;
     return LH_OK;
 }

@@ -1,0 +1,77 @@
+// Activation quantisation shared by the quantized-weight matvec kernels: x -> block fixed point.
+// Per group of G elements (G = weight block size): a float scale s = max|x| / qmax and integers
+// n_i = rint(x_i / s), split into L signed 8-bit limbs (n = sum_l limb_l * 256^l) so that dot
+// products with small unsigned weight codes are exact in v_dot4_i32_i8 / MFMA i8 arithmetic.
+#pragma once
+#include "common.hpp"
+
+template <int L> struct Limb;
+template <> struct Limb<2> { static constexpr float qmax = 32639.0f; };     // 127*256 + 127
+template <> struct Limb<3> { static constexpr float qmax = 8355711.0f; };   // 127*65536 + 127*256 + 127
+
+// ---- activation quantisation into LDS ----------------------------------------
+// xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
+// xs[K/G]: float scale of each group of G elements (G = weight block size).
+// `xn` (optional) receives sum(n_i) per group; `nthreads` = workgroup size (multiple of 64).
+template <int L, int G, typename XT>
+__device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs, int* xn,
+                                                  uint32_t nthreads) {
+    const int tid = threadIdx.x;
+    const uint32_t kq = K >> 2;
+    for (uint32_t base = 0; base < K; base += nthreads * 8) {
+        const uint32_t e0 = base + tid * 8;
+        const bool valid = e0 < K;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        if (valid) {
+            if constexpr (sizeof(XT) == 4) {
+                const float4 a = *reinterpret_cast<const float4*>(x + e0);
+                const float4 b = *reinterpret_cast<const float4*>(x + e0 + 4);
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else {
+                const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
+                const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    v[2 * i] = lh_h2f((uint16_t)(w[i] & 0xFFFF));
+                    v[2 * i + 1] = lh_h2f((uint16_t)(w[i] >> 16));
+                }
+            }
+        }
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+        m = lh_group_max(m, G / 8);
+        const float inv = m > 0.0f ? Limb<L>::qmax / m : 0.0f;
+        uint32_t packed[L][2];
+        int nsum = 0;
+#pragma unroll
+        for (int l = 0; l < L; l++) packed[l][0] = packed[l][1] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float r = rintf(v[i] * inv);
+            r = fminf(fmaxf(r, -Limb<L>::qmax), Limb<L>::qmax);
+            int n = (int)r;
+            nsum += n;
+#pragma unroll
+            for (int l = 0; l < L; l++) {
+                int limb;
+                if (l == L - 1) limb = n;                       // top limb: what is left, fits a signed byte
+                else { limb = (int)(int8_t)(n & 0xFF); n = (n - limb) >> 8; }
+                packed[l][i >> 2] |= (uint32_t)(limb & 0xFF) << (8 * (i & 3));
+            }
+        }
+        if (valid) {
+#pragma unroll
+            for (int l = 0; l < L; l++)
+                *reinterpret_cast<uint2*>(&xq[l * kq + (e0 >> 2)]) = make_uint2(packed[l][0], packed[l][1]);
+            if ((e0 & (G - 1)) == 0) xs[e0 / G] = m * (1.0f / Limb<L>::qmax);
+        }
+        if (xn != nullptr) {
+            nsum = lh_group_sum_i(nsum, G / 8);
+            if (valid && (e0 & (G - 1)) == 0) xn[e0 / G] = nsum;
+        }
+    }
+}
+
