@@ -13,7 +13,7 @@ TQ2_0 down-projection shape, one logits-sized matvec (262144 x 1536, a single or
 launch), the tq2 flash-decoding attention at 32k context (single query, and a batch of
 independent sequences), the small-batch layer and the prefill matmul.
 
-`roofline` describes the dominant kernel (matvec_quant_kernel, TQ2_0 instantiation): its
+`roofline` describes the dominant kernel (matvec_tq2_mfma_kernel, the TQ2_0 matvec): its
 algorithmic bytes per launch over its launch duration from HIP events on the library's
 stream.  `cpu_baseline` times the CPU restatement of the reference's own path (block dequant
 to f16 + sequential f32 dot) on the host cores, on a bounded sample of the same workload.
@@ -36,9 +36,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/matvec_tq2_0_grouped_pmc.md), scaled by the same counters on the library's plain
+# (profiles/matvec_tq2_mfma_grouped_8192x2048.md), scaled by the same counters on the library's plain
 # copy kernel; None until that profile has been taken for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = 1086451302
 
 
 def log(*a):
@@ -355,14 +355,14 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8",   # 2-bit / 4-bit codes x 8-bit activation limbs on v_dot4_i32_i8, f32 block scales
+        "dtype": "int8",   # 2-bit codes x 8-bit activation limbs on v_mfma_i32_16x16x64_i8, f32 block scales
         "data": "synthetic",
         "config": {"workload": "TQ2_0 fused dequant-matvec, M=1, N=8192 x K=2048 (MLP gate/up), fp32 x and y",
                    "replicas_per_step": head["replicas"], "launches_per_step": 1,
                    "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "matvec_quant_kernel<TQ2_0>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
+                     "kernel": "matvec_tq2_mfma_kernel<float, float>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
                      "launch_ms": head["ms_per_launch_events"]},
         "cpu_baseline": cpu,
         "extra": extra,

@@ -276,6 +276,13 @@ def matmul_f16_nt(a_bits, b_bits, m, k, n) -> np.ndarray:
     return c
 
 
+def tensor_bytes(fmt: str, n_elements: int) -> int:
+    """Payload bytes of a GGUF tensor: ceil(n / block elements) * block bytes
+    (local-engine/src/gguf.rs:247-311: Q4_0 32 -> 18, Q8_0 32 -> 34, TQ2_0 256 -> 66)."""
+    elems, size = {"q4_0": (32, 18), "q8_0": (32, 34), "tq2_0": (256, 66)}[fmt]
+    return -(-n_elements // elems) * size
+
+
 def swa_ring_capacity(window: int, max_positions: int) -> int:
     return int(lib().orc_swa_ring_capacity(window, max_positions))
 

@@ -127,10 +127,11 @@ def test_expand_matches_dequant_and_matvec_invariants(oracle, fmt, rows, cols):
     assert np.array_equal(oracle.matvec_quant_ref(fmt, raw, v, rows, cols, threads=3), yr)
 
 
-def test_tensor_byte_sizes():
-    # local-engine/src/gguf.rs:272-311, 524-528
-    assert (1024 // 32) * 18 == 32 * 18
-    assert -(-1024 // 256) * 66 == 4 * 66
+def test_tensor_byte_sizes(oracle):
+    # local-engine/src/gguf.rs:272-311; asserted values from gguf.rs:524-528
+    assert oracle.tensor_bytes("q4_0", 1024) == 32 * 18
+    assert oracle.tensor_bytes("q8_0", 1024) == 32 * 34
+    assert oracle.tensor_bytes("tq2_0", 257) == 2 * 66
 
 
 def test_legacy_tq2_dequant_and_f16_matmul(oracle):
