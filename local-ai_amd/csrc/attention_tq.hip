@@ -19,37 +19,17 @@
 //  * per workgroup the partial (max, sum, acc[head_dim]) per head goes to a
 //    workspace and a second small kernel does the log-sum-exp merge; with one
 //    split the workgroup writes the final result itself.
-#include "common.hpp"
+#include "attention_tq.hpp"
 #include <algorithm>
 
 namespace {
+using namespace lh_attn;
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerWG = kThreads / 64;
 constexpr int kMaxDpl = 8;        // head_dim 512 over 64 lanes
 constexpr int kHeadsPerPass = 8;  // query heads served together from one decode of a position
 constexpr int kPosBatch = 8;      // positions whose loads a wave keeps in flight together
-
-enum Mode : uint32_t { kSingle = 0, kPrefill = 1, kBatched = 2 };
-
-struct AttnParams {
-    uint32_t head_dim, bits, code_bytes;
-    uint32_t num_q_heads, num_kv_heads;
-    uint32_t kv_len;          // single / prefill
-    uint32_t pos0;            // single: current_pos; prefill: start_pos
-    uint32_t window, ring_capacity, lane_capacity;
-    uint32_t mode, num_queries, num_splits;
-};
-
-__device__ __forceinline__ void query_range(const AttnParams& p, const uint32_t* positions, uint32_t qi, uint32_t& lo, uint32_t& hi,
-                                            uint32_t& lane_base) {
-    uint32_t pos, kv_len;
-    if (p.mode == kBatched) { pos = positions[qi]; kv_len = pos + 1u; lane_base = qi * p.lane_capacity; }
-    else { pos = p.pos0 + (p.mode == kPrefill ? qi : 0u); kv_len = p.kv_len; lane_base = 0; }
-    hi = kv_len < pos + 1u ? kv_len : pos + 1u;
-    lo = (p.window > 0u && pos + 1u > p.window) ? pos + 1u - p.window : 0u;
-    if (lo > hi) lo = hi;
-}
 
 // The lane's bit window of one code record: `dpl` codes starting at bit lane*dpl*bits.
 __device__ __forceinline__ uint32_t load_window(const uint8_t* rec, uint32_t byte0, uint32_t nbytes) {
@@ -221,7 +201,6 @@ __global__ __launch_bounds__(kThreads) void attention_tq_split_kernel(
 // flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.  One workgroup per
 // (query, head); the per-split factors exp(m_s - max) are computed once into LDS, then every thread
 // folds its output dimension over the splits with coalesced row reads.
-constexpr int kMaxSplits = 1024;
 __global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
                                                                  uint32_t num_splits) {
     __shared__ float f_s[kMaxSplits];
@@ -284,28 +263,34 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     LH_NEED(v_norms, (size_t)phys_slots * 2, op, "v_norms");
     if (p.mode == kBatched) LH_NEED(positions, (size_t)p.num_queries * 4, op, "positions");
 
-    // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
-    const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
-    uint64_t splits = std::min<uint64_t>(per_query_wgs, (max_span + 31) / 32);
-    splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
-    const size_t rec = (size_t)p.head_dim + 4;
     const size_t ws_avail = (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
-    while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_avail) splits--;
-    p.num_splits = (uint32_t)splits;
+    const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
+                            (const uint8_t*)v_codes->ptr, (const uint16_t*)v_norms->ptr, (const float*)levels->ptr,
+                            positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, (float*)ctx->workspace};
+    if (max_span == 0 || !mfma_supported(p, ptrs)) {
+        // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
+        const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
+        uint64_t splits = std::min<uint64_t>(per_query_wgs, (max_span + 31) / 32);
+        splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
+        const size_t rec = partial_record_floats(p.head_dim);
+        while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_avail) splits--;
+        p.num_splits = (uint32_t)splits;
 
-    const size_t lds_bytes = (size_t)kWavesPerWG * kHeadsPerPass * p.head_dim * 4;
-    if (lds_bytes > 48 * 1024) {
-        static bool raised = false;   // one owner thread per context
-        if (!raised) {
-            LH_HIP_TRY(hipFuncSetAttribute((const void*)attention_tq_split_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024),
-                       LH_ERR_PIPELINE_CREATION, op);
-            raised = true;
+        const size_t lds_bytes = (size_t)kWavesPerWG * kHeadsPerPass * p.head_dim * 4;
+        if (lds_bytes > 48 * 1024) {
+            static bool raised = false;   // one owner thread per context
+            if (!raised) {
+                LH_HIP_TRY(hipFuncSetAttribute((const void*)attention_tq_split_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024),
+                           LH_ERR_PIPELINE_CREATION, op);
+                raised = true;
+            }
         }
+        hipLaunchKernelGGL(attention_tq_split_kernel, dim3(p.num_splits, p.num_queries * p.num_kv_heads), dim3(kThreads), lds_bytes, ctx->stream,
+                           ptrs.rq, ptrs.k_codes, ptrs.k_norms, ptrs.v_codes, ptrs.v_norms, ptrs.levels, ptrs.positions, ptrs.out, ptrs.ws, p);
+    } else {
+        const int rl = launch_mfma(ctx, op, ptrs, p, max_span, ws_avail);
+        if (rl != LH_OK) return rl;
     }
-    hipLaunchKernelGGL(attention_tq_split_kernel, dim3(p.num_splits, p.num_queries * p.num_kv_heads), dim3(kThreads), lds_bytes, ctx->stream,
-                       (const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr, (const uint8_t*)v_codes->ptr,
-                       (const uint16_t*)v_norms->ptr, (const float*)levels->ptr, positions ? (const uint32_t*)positions->ptr : nullptr,
-                       (float*)out->ptr, (float*)ctx->workspace, p);
     int r = lh_check_launch(op);
     if (r != LH_OK) return r;
     batch->dispatch_count++;

@@ -1,0 +1,460 @@
+// Flash-decoding attention over packed 2-bit TurboQuant codes on the matrix cores.
+//
+// Same contract as attention_tq.hip (stands in for shaders/attention_flash_tq.metal:154-690); this
+// kernel takes the common case -- 2-bit codes, head_dim 256, up to 8 query heads per KV head -- and
+// is bound by HBM instead of by the vector ALU.  Per cached position the path moves 132 bytes and
+// needs 8192 multiply-adds (8 heads x 256 dims x {K, V}); decoding every code to a float and
+// multiplying on the vector ALU costs ~40x more issue slots than the memory stream leaves free.
+//
+// The 2-bit level table is written as L[c] = a + b*bit0(c) + g*bit1(c) (+ d*bit0*bit1, which is zero for
+// the symmetric Lloyd-Max tables and costs a third bit plane otherwise).  Bit planes are isolated with
+// one AND per four codes and fed to v_mfma_i32_16x16x64_i8 as they are; what multiplies them is
+// quantised to fixed point and split into signed 8-bit limbs, one MFMA row per (query head, limb):
+//   K side:  rows = 8 heads x 2 limbs of b*rq and g/2*rq (16-bit block fixed point per head), columns =
+//            16 positions, k = 64 code bytes;  logit = norm_k * (scale_h * int + a * sum(rq_h)).
+//   V side:  rows = 4 heads x 4 limbs (two row sets) of w = exp2(logit - R_h) * norm_v in 31-bit fixed
+//            point, columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share one
+//            accumulator because their coefficients are folded into w before quantisation.  The
+//            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
+//            byte transposes.
+// One wave owns a chunk of positions and walks it in aligned groups of 64.  The integer V accumulators
+// persist across groups: the softmax reference R_h is only moved (and the accumulators folded into
+// the float outputs) when a weight would leave the fixed-point range, which the 31-bit width makes
+// rare.  Partials (R, l, acc) per wave chunk go to the workspace for the merge kernel.
+#include "attention_tq.hpp"
+#include <algorithm>
+#include <cstdlib>
+
+namespace {
+using namespace lh_attn;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+
+constexpr int kHeadDim = 256;
+constexpr int kCodeBytes = 64;
+constexpr int kGroup = 64;             // positions per loop step: 4 K-side MFMA tiles, one V-side MFMA k-step
+constexpr int kMaxGroupHeads = 8;      // query heads per KV head served by the 16 MFMA rows
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kQmax = 32639.0f;      // 127 * 256 + 127
+constexpr float kVQ = 2.0e9f;          // V-side weights: fixed point with 4 signed limbs, below 127 * 2^24
+constexpr int kHeadroom = 6;           // log2 of how far a weight may exceed the reference before it is moved
+
+__device__ __forceinline__ u32x4_t ld16(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(4))) u32x4_a4;
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a4*>(p);
+}
+__device__ __forceinline__ uint32_t ld4(gptr_t p) { return *reinterpret_cast<const __attribute__((address_space(1))) uint32_t*>(p); }
+__device__ __forceinline__ float ld_norm(gptr_t p) {
+    return lh_h2f(*reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>(p));
+}
+
+// 4x4 byte transpose: x[q] holds bytes e = 0..3 of position q; y[e] gets byte e of positions 0..3.
+__device__ __forceinline__ void transpose4x4(const uint32_t (&x)[4], uint32_t (&y)[4]) {
+    const uint32_t t0 = __builtin_amdgcn_perm(x[1], x[0], 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(x[1], x[0], 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(x[3], x[2], 0x05010400u);
+    const uint32_t t3 = __builtin_amdgcn_perm(x[3], x[2], 0x07030602u);
+    y[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    y[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    y[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    y[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+struct GroupGeom {
+    uint32_t pb;        // physical slot of the group's first position
+    uint32_t vlo, vhi;  // valid positions of the group: [vlo, vhi) within 0..64
+    bool full;
+};
+
+__global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
+    __shared__ __align__(16) uint8_t s_rqop[12][64][16];          // K-side A operands per (plane, field) and lane
+    __shared__ float s_maxabs[kMaxGroupHeads], s_sum[kMaxGroupHeads];
+    __shared__ __align__(16) float4 s_norm[4][kGroup];            // per wave and group position: (norm_k*log2e, mask bias, norm_v, -)
+    __shared__ __align__(16) uint8_t s_wx[4][3][2][1024];         // per wave, plane, row set: V-side A operands (weights as limbs)
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const uint32_t pcol = lane & 15, g = lane >> 4;               // MFMA column / row group of this lane
+    const uint32_t qi = blockIdx.y / p.num_kv_heads, kvh = blockIdx.y - qi * p.num_kv_heads;
+    const uint32_t group = p.num_q_heads / p.num_kv_heads;
+    const float* rq_base = a.rq + ((size_t)qi * p.num_q_heads + (size_t)kvh * group) * kHeadDim;
+
+    // ---- level table as an affine function of the code bits
+    const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
+    const float alpha = L0, beta = L1 - L0, gam = L2 - L0, delta = (L3 - L2) - (L1 - L0);
+    const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
+    const bool has_delta = fabsf(delta) > 1e-6f * lmax;
+    const int nplanes = has_delta ? 3 : 2;
+    const float cmax_k = fmaxf(fmaxf(fabsf(beta), fabsf(0.5f * gam)), has_delta ? fabsf(delta) : 0.0f);
+    const float cmax_v = fmaxf(fmaxf(fabsf(beta), fabsf(gam)), has_delta ? fabsf(delta) : 0.0f);
+
+    // ---- per head: max |rq| (quantisation scale) and sum(rq) (constant term of the level table)
+    for (uint32_t h = tid >> 5; h < (uint32_t)kMaxGroupHeads; h += blockDim.x >> 5) {
+        const uint32_t sub = tid & 31;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        if (h < group) {
+            const float4 x0 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8);
+            const float4 x1 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8 + 4);
+            v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+        }
+        float m = 0.0f, s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { m = fmaxf(m, fabsf(v[i])); s += v[i]; }
+        m = lh_group_max(m, 32);
+        s = lh_group_sum(s, 32);
+        if (sub == 0) { s_maxabs[h] = m; s_sum[h] = s; }
+    }
+    __syncthreads();
+
+    // ---- K-side A operands.  Row r of the MFMA: head (r / 4) + 4 * ((r / 2) % 2), limb r % 2, so that the lanes of
+    //      row group g end up with heads g and g + 4 on both the K and the V side.  k slot (word m, byte e) of
+    //      row group g is code byte j = 16g + 4m + e, i.e. dim 4j + f for the operand of field f.
+    {
+        const uint32_t h = (pcol >> 2) + 4 * ((pcol >> 1) & 1), limb = pcol & 1;
+        const float ma = s_maxabs[h];
+        const float inv = (ma > 0.0f && cmax_k > 0.0f) ? kQmax / (ma * cmax_k) : 0.0f;
+        for (uint32_t pl = wave; pl < (uint32_t)nplanes; pl += nwaves) {
+            const float mul = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv;
+            uint32_t words[4][4];
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+#pragma unroll
+                for (int m = 0; m < 4; m++) words[f][m] = 0;
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (h < group) x = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + 4 * (16 * g + 4 * m + e));
+                    const float xv[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                    for (int f = 0; f < 4; f++) {
+                        float r = __builtin_rintf(xv[f] * mul);
+                        r = fminf(fmaxf(r, -kQmax), kQmax);
+                        const int n = (int)r;
+                        const int lo = (int)(int8_t)(n & 0xFF);
+                        const int b = limb ? (n - lo) >> 8 : lo;
+                        words[f][m] |= (uint32_t)(b & 0xFF) << (8 * e);
+                    }
+                }
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+                *reinterpret_cast<u32x4_t*>(&s_rqop[pl * 4 + f][lane][0]) = (u32x4_t){words[f][0], words[f][1], words[f][2], words[f][3]};
+        }
+    }
+    __syncthreads();
+    float cs[2], ca[2];   // logit (log2 domain) = norm_k*log2e * (cs * int + ca) for the lane's two heads g, g + 4
+#pragma unroll
+    for (int hs = 0; hs < 2; hs++) {
+        const uint32_t h = g + 4 * hs;
+        cs[hs] = s_maxabs[h] * cmax_k * (0.25f / kQmax);
+        ca[hs] = alpha * s_sum[h];
+    }
+
+    // ---- this wave's chunk of positions
+    uint32_t lo, hi, lane_base;
+    query_range(p, a.positions, qi, lo, hi, lane_base);
+    const uint32_t n = hi - lo, nsplit = p.num_splits;
+    const uint32_t split = blockIdx.x * nwaves + wave;
+    if (split >= nsplit) return;                                  // surplus wave of the last workgroup (no barriers below)
+    const uint32_t chunk = (((n + nsplit - 1) / nsplit) + (kGroup - 1)) & ~(uint32_t)(kGroup - 1);
+    const uint32_t c_lo = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)split * chunk);
+    const uint32_t c_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(split + 1) * chunk);
+
+    const uint32_t stride = p.num_kv_heads * kCodeBytes;          // bytes between positions
+    gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+    gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+    gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
+    gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
+    const uint32_t nstride = p.num_kv_heads * 2;
+
+    auto geom = [&](uint32_t G) {
+        GroupGeom gg;
+        const uint32_t gstart = G << 6;
+        gg.vlo = c_lo > gstart ? c_lo - gstart : 0u;
+        gg.vhi = std::min<uint32_t>(c_hi - gstart, (uint32_t)kGroup);
+        gg.pb = p.ring_capacity ? gstart % p.ring_capacity : gstart;
+        gg.full = gg.vlo == 0 && gg.vhi == (uint32_t)kGroup;
+        return gg;
+    };
+    auto slot_of = [](const GroupGeom& gg, uint32_t idx) {
+        return (size_t)(gg.pb + (gg.full ? idx : std::min(std::max(idx, gg.vlo), gg.vhi - 1u)));
+    };
+
+    v4i acc[4][4][2];      // [code byte e][field f][row set]: integer V accumulators, rows = 4 limbs of head g + 4 * set
+    float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int f = 0; f < 4; f++)
+#pragma unroll
+            for (int hs = 0; hs < 2; hs++) { acc[e][f][hs] = (v4i){0, 0, 0, 0}; outv[e][f][hs] = 0.0f; }
+    float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
+    float vref = 0.0f, wlimit = 0.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
+    uint32_t since_fold = 0;
+
+    // integer accumulators -> float outputs (in the units of the current vref), accumulators cleared
+    auto fold = [&]() {
+        const float unit = wq > 0.0f ? cmax_v / wq : 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    const v4i A = acc[e][f][hs];
+                    const float v = ((float)A[0] + 256.0f * (float)A[1]) + (65536.0f * (float)A[2] + 16777216.0f * (float)A[3]);
+                    outv[e][f][hs] = __builtin_fmaf(v, unit * (1.0f / (float)(1 << (2 * f))), outv[e][f][hs]);
+                    acc[e][f][hs] = (v4i){0, 0, 0, 0};
+                }
+        since_fold = 0;
+    };
+
+    if (c_hi > c_lo) {
+        const uint32_t g_first = c_lo >> 6, g_last = (c_hi - 1) >> 6;
+        GroupGeom gg = geom(g_first);
+        u32x4_t kw[4];
+        uint32_t vx[4][4];
+        float nk, nv;
+        auto load_k = [&](const GroupGeom& G_) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) kw[q] = ld16(krec0 + slot_of(G_, 16 * q + pcol) * stride + 16 * g);
+            const size_t s = slot_of(G_, lane);
+            nk = ld_norm(kn0 + s * nstride);
+            nv = ld_norm(vn0 + s * nstride);
+        };
+        auto load_v = [&](const GroupGeom& G_) {
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+#pragma unroll
+                for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vrec0 + slot_of(G_, 16 * qq + 4 * g + m) * stride + 4 * pcol);
+        };
+        load_k(gg);
+        load_v(gg);
+
+        for (uint32_t G = g_first; G <= g_last; G++) {
+            const bool more = G < g_last;
+            const GroupGeom gnext = geom(more ? G + 1 : G);
+
+            // ---- norms of the group -> LDS
+            {
+                const bool valid = lane >= gg.vlo && lane < gg.vhi;
+                __builtin_amdgcn_wave_barrier();
+                s_norm[wave][lane] = make_float4(nk * kLog2e, valid ? 0.0f : -INFINITY, valid ? nv : 0.0f, 0.0f);
+                __builtin_amdgcn_wave_barrier();
+            }
+
+            // ---- K side: logits of 4 tiles x (this lane's column position, heads g and g + 4)
+            float lg[4][2], vn[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t w[4] = {kw[q].x, kw[q].y, kw[q].z, kw[q].w};
+                v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    const uint32_t u = w[m] >> 4;
+                    b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
+                    b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
+                    b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
+                    b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
+                }
+                const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[0][lane][0]);   // operand pf at rqo[64 * pf]
+                v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
+                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
+                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
+                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
+                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
+                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
+                if (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
+                    v4i d0, d1, d2, d3;
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
+                        d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
+                        d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
+                    }
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
+                }
+                const float4 nrm = s_norm[wave][16 * q + pcol];
+                vn[q] = nrm.z;
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    const int t_lo = (acc1[2 * hs] << 2) + acc4[2 * hs];
+                    const int t_hi = (acc1[2 * hs + 1] << 2) + acc4[2 * hs + 1];
+                    const float inner = (float)(t_lo + (t_hi << 8)) * cs[hs] + ca[hs];
+                    lg[q][hs] = nrm.x * inner + nrm.y;
+                }
+            }
+            if (more) load_k(gnext);   // the K registers are free: fetch the next group's codes and norms
+
+            // ---- softmax weights relative to the running reference R; move R only when the fixed-point range is left
+            float ew[4][2], ww[4][2];
+            auto weights = [&]() {
+                float wm = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        ew[q][hs] = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
+                        ww[q][hs] = ew[q][hs] * vn[q];
+                        wm = fmaxf(wm, ww[q][hs]);
+                    }
+                return lh_group_max(wm, 64);
+            };
+            float wm = weights();
+            if (!(wm <= wlimit) || since_fold >= 256u) {     // uniform; true for the first group (R = -inf gives inf / NaN)
+                fold();
+                float vm = fmaxf(fmaxf(vn[0], vn[1]), fmaxf(vn[2], vn[3]));
+                vm = lh_group_max(vm, 64);
+                vref = fmaxf(vref, vm);
+                wlimit = vref * (float)(1 << kHeadroom);
+                wq = wlimit > 0.0f ? kVQ / wlimit : 0.0f;
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    float m = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
+                    m = lh_group_max(m, 16);
+                    const float rn = fmaxf(R[hs], m);
+                    const float fsc = __builtin_amdgcn_exp2f(R[hs] - rn);   // 0 for the first group
+                    R[hs] = rn;
+                    l_run[hs] *= fsc;
+                    w_run[hs] *= fsc;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+#pragma unroll
+                        for (int f = 0; f < 4; f++) outv[e][f][hs] *= fsc;
+                }
+                wm = weights();
+            }
+            since_fold++;
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) { l_run[hs] += ew[q][hs]; w_run[hs] += ww[q][hs]; }
+
+            // ---- weights -> 31-bit fixed point, one word of 4 signed limbs per (tile, head, plane); byte transpose to
+            //      "limb i over the four tiles" and hand each word to the lane that owns it as an MFMA row:
+            //      lane (column 4A+B, row group g) feeds row 4g + i of k-group A, word B.
+            {
+                const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int pl = 0; pl < 3; pl++) {
+                    if (pl >= nplanes) break;
+                    const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * (wq / cmax_v);
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        uint32_t lw[4], tr[4];
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const int qv = (int)(ww[q][hs] * cq);                 // truncation: |qv| <= kVQ < 127 * 2^24
+                            lw[q] = ((uint32_t)qv + 0x00808080u) ^ 0x00808080u;    // bytes = signed limbs, least significant first
+                        }
+                        transpose4x4(lw, tr);
+                        uint8_t* dst = &s_wx[wave][pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t*>(dst + 16 * i) = tr[i];
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+
+            // ---- V side
+            uint32_t y[4][4];   // [word m][code byte e]: byte e of positions 16qq + 4g + m, qq = 0..3
+#pragma unroll
+            for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
+            if (more) load_v(gnext);   // the V registers are free
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) {
+                if (pl >= nplanes) break;
+                const v4i wop0 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][0][lane * 16]);
+                const v4i wop1 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][1][lane * 16]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    uint32_t yp[4];   // the plane's bit of every field at the even bit positions
+#pragma unroll
+                    for (int m = 0; m < 4; m++) yp[m] = pl == 0 ? y[m][e] : pl == 1 ? y[m][e] >> 1 : y[m][e] & (y[m][e] >> 1);
+#pragma unroll
+                    for (int f = 0; f < 4; f++) {
+                        v4i b;
+#pragma unroll
+                        for (int m = 0; m < 4; m++) b[m] = (int)(yp[m] & (0x01010101u << (2 * f)));
+                        acc[e][f][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop0, b, acc[e][f][0], 0, 0, 0);
+                        acc[e][f][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop1, b, acc[e][f][1], 0, 0, 0);
+                    }
+                }
+            }
+            gg = gnext;
+        }
+        fold();
+    }
+
+    // ---- the wave's result: final output (one split) or a partial record for the merge kernel
+#pragma unroll
+    for (int hs = 0; hs < 2; hs++) {
+        const float l_tot = lh_group_sum(l_run[hs], 16);
+        const float w_tot = lh_group_sum(w_run[hs], 16);
+        const uint32_t h = g + 4 * hs;
+        if (h >= group) continue;
+        const uint32_t qh = kvh * group + h;
+        const float bias = alpha * w_tot;
+        if (nsplit == 1) {
+            float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 16 * pcol;
+            const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                *reinterpret_cast<float4*>(dst + 4 * e) = make_float4((outv[e][0][hs] + bias) * inv, (outv[e][1][hs] + bias) * inv,
+                                                                      (outv[e][2][hs] + bias) * inv, (outv[e][3][hs] + bias) * inv);
+        } else {
+            float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * nsplit + split) * partial_record_floats(kHeadDim);
+            if (pcol == 0) { rec[0] = R[hs] * kLn2; rec[1] = l_tot; }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                *reinterpret_cast<float4*>(rec + 4 + 16 * pcol + 4 * e) =
+                    make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
+        }
+    }
+}
+
+}  // namespace
+
+namespace lh_attn {
+
+bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
+    static const bool off = [] { const char* e = getenv("LOCAL_HIP_ATTN_KERNEL"); return e && e[0] == 'v'; }();   // "valu"
+    if (off) return false;
+    if (p.bits != 2 || p.head_dim != (uint32_t)kHeadDim) return false;
+    if (p.num_q_heads / p.num_kv_heads > (uint32_t)kMaxGroupHeads) return false;
+    if (p.ring_capacity % kGroup != 0) return false;                      // aligned groups must not wrap inside
+    if (((uintptr_t)a.k_codes | (uintptr_t)a.v_codes) & 3) return false;
+    if (((uintptr_t)a.k_norms | (uintptr_t)a.v_norms) & 1) return false;
+    if (((uintptr_t)a.rq | (uintptr_t)a.out) & 15) return false;
+    return true;
+}
+
+int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
+    // One wave per chunk of positions; about one wave per SIMD over the whole launch, at least 128 positions each.
+    const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
+    const uint64_t wave_slots = (uint64_t)ctx->cu_count * 4;
+    uint64_t splits = std::max<uint64_t>(1, wave_slots / pairs);
+    splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
+    splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
+    const size_t rec = partial_record_floats(p.head_dim);
+    while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
+    p.num_splits = (uint32_t)splits;
+    const uint32_t waves = splits * pairs >= wave_slots && splits >= 4 ? 4 : 1;
+    const dim3 grid((uint32_t)((splits + waves - 1) / waves), (uint32_t)pairs);
+    hipLaunchKernelGGL(attention_tq_mfma_kernel, grid, dim3(64 * waves), 0, ctx->stream, a, p);
+    return lh_check_launch(op);
+}
+
+}  // namespace lh_attn

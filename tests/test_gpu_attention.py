@@ -45,6 +45,14 @@ def upload(pkg, ctx, *arrays):
     (64, 6, 3, 90, 4, 16, 0.5),
     (256, 16, 1, 100, 2, 0, 0.3),      # more than 8 query heads per KV head
     (128, 2, 2, 1, 2, 0, 1.0),         # one position
+    (256, 8, 1, 1, 2, 0, 1.0),         # matrix-core path: one position
+    (256, 8, 1, 255, 2, 0, 1.0),       # just under / at / over one 256-position block
+    (256, 8, 1, 256, 2, 0, 1.0),
+    (256, 8, 1, 257, 2, 0, 1.0),
+    (256, 4, 1, 700, 2, 0, 1.0),       # fewer than 8 query heads per KV head (padded MFMA rows)
+    (256, 8, 2, 1300, 2, 300, 1.0),    # two KV heads, window not aligned to the block size
+    (256, 6, 3, 513, 2, 0, 0.5),
+    (256, 8, 1, 20000, 2, 0, 0.25),    # long context, soft attention (many positions carry weight)
 ])
 def test_decode_attention_matches_oracle(pkg, gpu, oracle, hd, nq, nkv, T, bits, window, qscale):
     print(f"case hd={hd} nq={nq} nkv={nkv} T={T} bits={bits} window={window}", flush=True)
@@ -67,6 +75,23 @@ def test_decode_attention_matches_oracle(pkg, gpu, oracle, hd, nq, nkv, T, bits,
     # element-wise form too: |g - w| <= tol * max(|w|, 1)
     assert np.max(np.abs(out.as_array(np.float32) - ref) / np.maximum(np.abs(ref), 1.0)) <= ATTN_TOL
     print(f"  err rotated {e1:.2e}, output {e2:.2e}")
+
+
+@pytest.mark.parametrize("T", [300, 5000])
+def test_decode_attention_with_asymmetric_levels(pkg, gpu, oracle, T):
+    """A level table that is not affine in the code bits (L3 - L2 != L1 - L0) takes the third bit plane."""
+    ctx, K = gpu
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 31 + T)
+    levels = (levels * np.array([1.0, 1.3, 0.8, 1.1], np.float32)).astype(np.float32)
+    rq = pkg.synth.rng(6, 17).standard_normal(nq * hd, dtype=np.float32) * 0.5
+    ref = oracle.attention_tq_codespace(rq, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    out = pkg.Buffer.empty(ctx, nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    check(out.as_array(np.float32), ref, "asymmetric levels")
 
 
 def test_decode_attention_vs_reference_cpu_path(pkg, gpu, oracle):
