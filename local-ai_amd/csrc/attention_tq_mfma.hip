@@ -24,6 +24,7 @@
 #include "attention_tq.hpp"
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 using namespace lh_attn;
@@ -69,24 +70,30 @@ struct GroupGeom {
     bool full;
 };
 
-__global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
-    __shared__ __align__(16) uint8_t s_rqop[12][64][16];          // K-side A operands per (plane, field) and lane
-    __shared__ float s_maxabs[kMaxGroupHeads], s_sum[kMaxGroupHeads];
-    __shared__ __align__(16) float4 s_norm[4][kGroup];            // per wave and group position: (norm_k*log2e, mask bias, norm_v, -)
-    __shared__ __align__(16) uint8_t s_wx[4][3][2][1024];         // per wave, plane, row set: V-side A operands (weights as limbs)
+struct AttnShared {
+    uint8_t rqop[12][64][16];      // K-side A operands per (plane, field) and lane
+    float4 norm[4][kGroup];        // per wave and group position: (norm_k*log2e, mask bias, norm_v, -)
+    uint8_t wx[4][3][2][1024];     // per wave, plane, row set: V-side A operands (weights as limbs)
+    float maxabs[kMaxGroupHeads], sum[kMaxGroupHeads];
+};
 
+// NPL = number of bit planes: 2 when the level table is affine in the code bits, 3 with the bit0*bit1 plane.
+template <int NPL>
+__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared& sh, float alpha, float beta,
+                                               float gam, float delta) {
+    auto& s_rqop = sh.rqop;
+    auto& s_norm = sh.norm;
+    auto& s_wx = sh.wx;
+    auto& s_maxabs = sh.maxabs;
+    auto& s_sum = sh.sum;
+    constexpr bool has_delta = NPL == 3;
+    constexpr int nplanes = NPL;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const uint32_t pcol = lane & 15, g = lane >> 4;               // MFMA column / row group of this lane
     const uint32_t qi = blockIdx.y / p.num_kv_heads, kvh = blockIdx.y - qi * p.num_kv_heads;
     const uint32_t group = p.num_q_heads / p.num_kv_heads;
     const float* rq_base = a.rq + ((size_t)qi * p.num_q_heads + (size_t)kvh * group) * kHeadDim;
 
-    // ---- level table as an affine function of the code bits
-    const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
-    const float alpha = L0, beta = L1 - L0, gam = L2 - L0, delta = (L3 - L2) - (L1 - L0);
-    const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
-    const bool has_delta = fabsf(delta) > 1e-6f * lmax;
-    const int nplanes = has_delta ? 3 : 2;
     const float cmax_k = fmaxf(fmaxf(fabsf(beta), fabsf(0.5f * gam)), has_delta ? fabsf(delta) : 0.0f);
     const float cmax_v = fmaxf(fmaxf(fabsf(beta), fabsf(gam)), has_delta ? fabsf(delta) : 0.0f);
 
@@ -181,9 +188,9 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
         gg.full = gg.vlo == 0 && gg.vhi == (uint32_t)kGroup;
         return gg;
     };
-    auto slot_of = [](const GroupGeom& gg, uint32_t idx) {
-        return (size_t)(gg.pb + (gg.full ? idx : std::min(std::max(idx, gg.vlo), gg.vhi - 1u)));
-    };
+    // Partial groups (chunk ends) load only their valid positions; the others read as zero codes and their
+    // weights are masked to zero.
+    auto is_valid = [](const GroupGeom& gg, uint32_t idx) { return idx - gg.vlo < gg.vhi - gg.vlo; };
 
     v4i acc[4][4][2];      // [code byte e][field f][row set]: integer V accumulators, rows = 4 limbs of head g + 4 * set
     float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
@@ -194,8 +201,9 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
 #pragma unroll
             for (int hs = 0; hs < 2; hs++) { acc[e][f][hs] = (v4i){0, 0, 0, 0}; outv[e][f][hs] = 0.0f; }
     float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
-    float vref = 0.0f, wlimit = 0.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
+    float vref = 0.0f, wlimit = -1.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
     uint32_t since_fold = 0;
+    const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
 
     // integer accumulators -> float outputs (in the units of the current vref), accumulators cleared
     auto fold = [&]() {
@@ -217,28 +225,56 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
     if (c_hi > c_lo) {
         const uint32_t g_first = c_lo >> 6, g_last = (c_hi - 1) >> 6;
         GroupGeom gg = geom(g_first);
-        u32x4_t kw[4];
+        u32x4_t kw[4], kwn[4];   // K codes of the current group and of the next one (a full step of prefetch distance)
         uint32_t vx[4][4];
-        float nk, nv;
-        auto load_k = [&](const GroupGeom& G_) {
+        float nk, nv, nkn = 0.0f, nvn = 0.0f;
+        const uint32_t klane = pcol * stride + 16 * g, vlane = 4 * g * stride + 4 * pcol, nlane = lane * nstride;
+        auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw)[4], float& nk, float& nv) {
+            gptr_t kb = krec0 + (size_t)G_.pb * stride;
+            gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
+            if (G_.full) {
 #pragma unroll
-            for (int q = 0; q < 4; q++) kw[q] = ld16(krec0 + slot_of(G_, 16 * q + pcol) * stride + 16 * g);
-            const size_t s = slot_of(G_, lane);
-            nk = ld_norm(kn0 + s * nstride);
-            nv = ld_norm(vn0 + s * nstride);
+                for (int q = 0; q < 4; q++) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                nk = ld_norm(knb + nlane);
+                nv = ld_norm(vnb + nlane);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    kw[q] = (u32x4_t){0u, 0u, 0u, 0u};
+                    if (is_valid(G_, 16 * q + pcol)) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                }
+                nk = nv = 0.0f;
+                if (is_valid(G_, lane)) { nk = ld_norm(knb + nlane); nv = ld_norm(vnb + nlane); }
+            }
         };
         auto load_v = [&](const GroupGeom& G_) {
+            gptr_t vb = vrec0 + (size_t)G_.pb * stride;
+            if (G_.full) {
 #pragma unroll
-            for (int m = 0; m < 4; m++)
+                for (int m = 0; m < 4; m++)
 #pragma unroll
-                for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vrec0 + slot_of(G_, 16 * qq + 4 * g + m) * stride + 4 * pcol);
+                    for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; m++)
+#pragma unroll
+                    for (int qq = 0; qq < 4; qq++) {
+                        vx[m][qq] = 0u;
+                        if (is_valid(G_, 16 * qq + 4 * g + m)) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
+                    }
+            }
         };
-        load_k(gg);
+        load_k(gg, kw, nk, nv);
         load_v(gg);
 
-        for (uint32_t G = g_first; G <= g_last; G++) {
+        // One group of 64 positions.  MAY_FOLD = false is the steady-state copy: it returns false, with nothing but the
+        // logits computed, when a weight would leave the fixed-point range; the MAY_FOLD = true copy then redoes the
+        // group and moves the reference.  (Keeping the rare path out of the hot loop keeps the accumulators in place.)
+        auto step = [&](auto may_fold_tag, uint32_t G) -> bool {
+            constexpr bool MAY_FOLD = decltype(may_fold_tag)::value;
             const bool more = G < g_last;
             const GroupGeom gnext = geom(more ? G + 1 : G);
+            if (more) load_k(gnext, kwn, nkn, nvn);
 
             // ---- norms of the group -> LDS
             {
@@ -272,7 +308,7 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
                 acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
                 acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
                 acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
-                if (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
+                if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
                     v4i d0, d1, d2, d3;
 #pragma unroll
                     for (int m = 0; m < 4; m++) {
@@ -295,11 +331,10 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
                     lg[q][hs] = nrm.x * inner + nrm.y;
                 }
             }
-            if (more) load_k(gnext);   // the K registers are free: fetch the next group's codes and norms
 
             // ---- softmax weights relative to the running reference R; move R only when the fixed-point range is left
             float ew[4][2], ww[4][2];
-            auto weights = [&]() {
+            auto weights = [&]() {   // returns whether any weight of the wave leaves the fixed-point range (or is NaN)
                 float wm = 0.0f;
 #pragma unroll
                 for (int q = 0; q < 4; q++)
@@ -309,10 +344,11 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
                         ww[q][hs] = ew[q][hs] * vn[q];
                         wm = fmaxf(wm, ww[q][hs]);
                     }
-                return lh_group_max(wm, 64);
+                return __builtin_amdgcn_ballot_w64(!(wm <= wlimit)) != 0;
             };
-            float wm = weights();
-            if (!(wm <= wlimit) || since_fold >= 256u) {     // uniform; true for the first group (R = -inf gives inf / NaN)
+            const bool out_of_range = weights();
+            if (out_of_range || since_fold >= 256u) {     // uniform; true for the first group (wlimit starts negative)
+                if constexpr (!MAY_FOLD) return false;
                 fold();
                 float vm = fmaxf(fmaxf(vn[0], vn[1]), fmaxf(vn[2], vn[3]));
                 vm = lh_group_max(vm, 64);
@@ -333,7 +369,7 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
 #pragma unroll
                         for (int f = 0; f < 4; f++) outv[e][f][hs] *= fsc;
                 }
-                wm = weights();
+                (void)weights();
             }
             since_fold++;
 #pragma unroll
@@ -348,9 +384,8 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
                 const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int pl = 0; pl < 3; pl++) {
-                    if (pl >= nplanes) break;
-                    const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * (wq / cmax_v);
+                for (int pl = 0; pl < nplanes; pl++) {
+                    const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * inv_cmax_v * wq;
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
                         uint32_t lw[4], tr[4];
@@ -374,8 +409,7 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
             for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
             if (more) load_v(gnext);   // the V registers are free
 #pragma unroll
-            for (int pl = 0; pl < 3; pl++) {
-                if (pl >= nplanes) break;
+            for (int pl = 0; pl < nplanes; pl++) {
                 const v4i wop0 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][0][lane * 16]);
                 const v4i wop1 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][1][lane * 16]);
 #pragma unroll
@@ -394,6 +428,17 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
                 }
             }
             gg = gnext;
+#pragma unroll
+            for (int q = 0; q < 4; q++) kw[q] = kwn[q];
+            nk = nkn; nv = nvn;
+            return true;
+        };
+
+        uint32_t G = g_first;
+        while (G <= g_last) {
+            step(std::true_type{}, G);
+            G++;
+            while (G <= g_last && step(std::false_type{}, G)) G++;
         }
         fold();
     }
@@ -425,6 +470,20 @@ __global__ __launch_bounds__(256, 2) void attention_tq_mfma_kernel(AttnPointers 
     }
 }
 
+
+template <int OCC>
+__global__ __launch_bounds__(256, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
+    __shared__ __align__(16) AttnShared sh;
+    // L[c] = alpha + beta*bit0 + gam*bit1 + delta*bit0*bit1.  A delta that is only float noise of a symmetric table
+    // (|delta| <= 1e-5 max|L|) is spread by the least-squares affine fit bit0*bit1 ~ -1/4 + bit0/2 + bit1/2, which
+    // leaves +-delta/4 per code; anything larger gets its own bit plane.
+    const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
+    const float d_raw = (L3 - L2) - (L1 - L0);
+    const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
+    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
+    else attention_body<2>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+}
+
 }  // namespace
 
 namespace lh_attn {
@@ -444,7 +503,9 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
     // One wave per chunk of positions; about one wave per SIMD over the whole launch, at least 128 positions each.
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
-    const uint64_t wave_slots = (uint64_t)ctx->cu_count * 4;
+    static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
+    static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
+    const uint64_t wave_slots = (uint64_t)ctx->cu_count * 4 * wps;
     uint64_t splits = std::max<uint64_t>(1, wave_slots / pairs);
     splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
     splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
@@ -453,7 +514,8 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     p.num_splits = (uint32_t)splits;
     const uint32_t waves = splits * pairs >= wave_slots && splits >= 4 ? 4 : 1;
     const dim3 grid((uint32_t)((splits + waves - 1) / waves), (uint32_t)pairs);
-    hipLaunchKernelGGL(attention_tq_mfma_kernel, grid, dim3(64 * waves), 0, ctx->stream, a, p);
+    if (occ == 1) hipLaunchKernelGGL(attention_tq_mfma_kernel<1>, grid, dim3(64 * waves), 0, ctx->stream, a, p);
+    else hipLaunchKernelGGL(attention_tq_mfma_kernel<2>, grid, dim3(64 * waves), 0, ctx->stream, a, p);
     return lh_check_launch(op);
 }
 
