@@ -17,10 +17,13 @@
 //            accumulator because their coefficients are folded into w before quantisation.  The
 //            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
 //            byte transposes.
-// One wave owns a chunk of positions and walks it in aligned groups of 64.  The integer V accumulators
-// persist across groups: the softmax reference R_h is only moved (and the accumulators folded into
-// the float outputs) when a weight would leave the fixed-point range, which the 31-bit width makes
-// rare.  Partials (R, l, acc) per wave chunk go to the workspace for the merge kernel.
+// One workgroup of two waves owns a chunk of positions and walks it in aligned groups of 64: the K wave
+// produces the softmax weights of a group, the V wave (one group behind, one barrier per group) turns
+// them into limbs and accumulates.  Splitting the roles keeps each wave under 256 registers, so two
+// waves share a SIMD and fill each other's stalls.  The integer V accumulators persist across groups:
+// the softmax reference R_h is only moved (and the accumulators folded into the float outputs) when a
+// weight would leave the fixed-point range, which the 31-bit width makes rare.  Partials (R, l, acc)
+// per chunk go to the workspace for the merge kernel.
 #include "attention_tq.hpp"
 #include <algorithm>
 #include <cstdlib>
@@ -70,10 +73,19 @@ struct GroupGeom {
     bool full;
 };
 
+// One workgroup = two waves on one chunk of positions: the "K wave" turns K codes into softmax weights (as MFMA row
+// operands in LDS), the "V wave" multiplies them with the V codes.  The K wave runs one group ahead; one workgroup
+// barrier per group hands over a double-buffered operand set plus the rare "reference moved" message.
 struct AttnShared {
     uint8_t rqop[12][64][16];      // K-side A operands per (plane, field) and lane
-    float4 norm[4][kGroup];        // per wave and group position: (norm_k*log2e, mask bias, norm_v, -)
-    uint8_t wx[4][3][2][1024];     // per wave, plane, row set: V-side A operands (weights as limbs)
+    float4 norm[kGroup];           // K wave: (norm_k*log2e, mask bias, norm_v, -) per group position
+    float4 ww[2][2][64];           // [buffer][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
+    float wq[2];                   // [buffer]: fixed-point scale of those weights
+    uint8_t wx[3][2][1024];        // V wave: [plane][row set] A operands (weights as limbs)
+    float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
+    float unit_old[2];             // [buffer]: value of one integer step of the accumulators gathered so far
+    uint32_t moved[2];             // [buffer]: the reference moved before this group: fold, then rescale
+    float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads], fin_unit;
     float maxabs[kMaxGroupHeads], sum[kMaxGroupHeads];
 };
 
@@ -82,8 +94,6 @@ template <int NPL>
 __device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared& sh, float alpha, float beta,
                                                float gam, float delta) {
     auto& s_rqop = sh.rqop;
-    auto& s_norm = sh.norm;
-    auto& s_wx = sh.wx;
     auto& s_maxabs = sh.maxabs;
     auto& s_sum = sh.sum;
     constexpr bool has_delta = NPL == 3;
@@ -154,31 +164,20 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         }
     }
     __syncthreads();
-    float cs[2], ca[2];   // logit (log2 domain) = norm_k*log2e * (cs * int + ca) for the lane's two heads g, g + 4
-#pragma unroll
-    for (int hs = 0; hs < 2; hs++) {
-        const uint32_t h = g + 4 * hs;
-        cs[hs] = s_maxabs[h] * cmax_k * (0.25f / kQmax);
-        ca[hs] = alpha * s_sum[h];
-    }
 
-    // ---- this wave's chunk of positions
+    // ---- the workgroup's chunk of positions
     uint32_t lo, hi, lane_base;
     query_range(p, a.positions, qi, lo, hi, lane_base);
     const uint32_t n = hi - lo, nsplit = p.num_splits;
-    const uint32_t split = blockIdx.x * nwaves + wave;
-    if (split >= nsplit) return;                                  // surplus wave of the last workgroup (no barriers below)
+    const uint32_t split = blockIdx.x;
     const uint32_t chunk = (((n + nsplit - 1) / nsplit) + (kGroup - 1)) & ~(uint32_t)(kGroup - 1);
     const uint32_t c_lo = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)split * chunk);
     const uint32_t c_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(split + 1) * chunk);
+    const bool any = c_hi > c_lo;
+    const uint32_t g_first = c_lo >> 6, g_last = any ? (c_hi - 1) >> 6 : 0u;
 
     const uint32_t stride = p.num_kv_heads * kCodeBytes;          // bytes between positions
-    gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
-    gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
-    gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
-    gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
     const uint32_t nstride = p.num_kv_heads * 2;
-
     auto geom = [&](uint32_t G) {
         GroupGeom gg;
         const uint32_t gstart = G << 6;
@@ -191,288 +190,343 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // Partial groups (chunk ends) load only their valid positions; the others read as zero codes and their
     // weights are masked to zero.
     auto is_valid = [](const GroupGeom& gg, uint32_t idx) { return idx - gg.vlo < gg.vhi - gg.vlo; };
-
-    v4i acc[4][4][2];      // [code byte e][field f][row set]: integer V accumulators, rows = 4 limbs of head g + 4 * set
-    float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
-#pragma unroll
-    for (int e = 0; e < 4; e++)
-#pragma unroll
-        for (int f = 0; f < 4; f++)
-#pragma unroll
-            for (int hs = 0; hs < 2; hs++) { acc[e][f][hs] = (v4i){0, 0, 0, 0}; outv[e][f][hs] = 0.0f; }
-    float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
-    float vref = 0.0f, wlimit = -1.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
-    uint32_t since_fold = 0;
     const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
+    const bool k_role = ((wave ^ blockIdx.x) & 1u) == 0;          // alternate, so that both kinds of wave share each SIMD
 
-    // integer accumulators -> float outputs (in the units of the current vref), accumulators cleared
-    auto fold = [&]() {
-        const float unit = wq > 0.0f ? cmax_v / wq : 0.0f;
+    if (k_role) {
+        // =================================================================== K wave
+        float cs[2], ca[2];   // logit (log2 domain) = norm_k*log2e * (cs * int + ca) for the lane's two heads g, g + 4
+#pragma unroll
+        for (int hs = 0; hs < 2; hs++) {
+            const uint32_t h = g + 4 * hs;
+            cs[hs] = s_maxabs[h] * cmax_k * (0.25f / kQmax);
+            ca[hs] = alpha * sh.sum[h];
+        }
+        gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+        gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
+        gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
+        float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
+        float vref = 0.0f, wlimit = -1.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
+        uint32_t since_move = 0;
+
+        if (any) {
+            GroupGeom gg = geom(g_first);
+            u32x4_t kw[4], kwn[4];   // K codes of the current group and of the next one (a full step of prefetch distance)
+            float nk, nv, nkn = 0.0f, nvn = 0.0f;
+            const uint32_t klane = pcol * stride + 16 * g, nlane = lane * nstride;
+            auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw_)[4], float& nk_, float& nv_) {
+                gptr_t kb = krec0 + (size_t)G_.pb * stride;
+                gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
+                if (G_.full) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) kw_[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                    nk_ = ld_norm(knb + nlane);
+                    nv_ = ld_norm(vnb + nlane);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        kw_[q] = (u32x4_t){0u, 0u, 0u, 0u};
+                        if (is_valid(G_, 16 * q + pcol)) kw_[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                    }
+                    nk_ = nv_ = 0.0f;
+                    if (is_valid(G_, lane)) { nk_ = ld_norm(knb + nlane); nv_ = ld_norm(vnb + nlane); }
+                }
+            };
+            load_k(gg, kw, nk, nv);
+
+            for (uint32_t G = g_first; G <= g_last; G++) {
+                const uint32_t buf = (G - g_first) & 1u;
+                const bool more = G < g_last;
+                const GroupGeom gnext = geom(more ? G + 1 : G);
+                if (more) load_k(gnext, kwn, nkn, nvn);
+
+                // ---- norms of the group -> LDS
+                {
+                    const bool valid = lane >= gg.vlo && lane < gg.vhi;
+                    __builtin_amdgcn_wave_barrier();
+                    sh.norm[lane] = make_float4(nk * kLog2e, valid ? 0.0f : -INFINITY, valid ? nv : 0.0f, 0.0f);
+                    __builtin_amdgcn_wave_barrier();
+                }
+
+                // ---- logits of 4 tiles x (this lane's column position, heads g and g + 4)
+                float lg[4][2], vn[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t w[4] = {kw[q].x, kw[q].y, kw[q].z, kw[q].w};
+                    v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        const uint32_t u = w[m] >> 4;
+                        b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
+                        b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
+                        b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
+                        b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
+                    }
+                    const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[0][lane][0]);   // operand pf at rqo[64 * pf]
+                    v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
+                    if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
+                        v4i d0, d1, d2, d3;
+#pragma unroll
+                        for (int m = 0; m < 4; m++) {
+                            const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
+                            d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
+                            d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
+                        }
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
+                    }
+                    const float4 nrm = sh.norm[16 * q + pcol];
+                    vn[q] = nrm.z;
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        const int t_lo = (acc1[2 * hs] << 2) + acc4[2 * hs];
+                        const int t_hi = (acc1[2 * hs + 1] << 2) + acc4[2 * hs + 1];
+                        const float inner = (float)(t_lo + (t_hi << 8)) * cs[hs] + ca[hs];
+                        lg[q][hs] = nrm.x * inner + nrm.y;
+                    }
+                }
+
+                // ---- softmax weights relative to the running reference R; R moves only when the fixed-point range is left
+                float ew[4][2], ww[4][2];
+                auto weights = [&]() {   // returns whether any weight of the wave leaves the fixed-point range (or is NaN)
+                    float wm = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+#pragma unroll
+                        for (int hs = 0; hs < 2; hs++) {
+                            ew[q][hs] = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
+                            ww[q][hs] = ew[q][hs] * vn[q];
+                            wm = fmaxf(wm, ww[q][hs]);
+                        }
+                    return __builtin_amdgcn_ballot_w64(!(wm <= wlimit)) != 0;
+                };
+                const bool out_of_range = weights();
+                const bool move = out_of_range || since_move >= 256u;   // uniform; true for the first group (wlimit starts negative)
+                if (move) {
+                    if (lane == 0) sh.unit_old[buf] = wq > 0.0f ? cmax_v / wq : 0.0f;
+                    float vm = fmaxf(fmaxf(vn[0], vn[1]), fmaxf(vn[2], vn[3]));
+                    vm = lh_group_max(vm, 64);
+                    vref = fmaxf(vref, vm);
+                    wlimit = vref * (float)(1 << kHeadroom);
+                    wq = wlimit > 0.0f ? kVQ / wlimit : 0.0f;
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        float m = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
+                        m = lh_group_max(m, 16);
+                        const float rn = fmaxf(R[hs], m);
+                        const float fsc = __builtin_amdgcn_exp2f(R[hs] - rn);   // 0 for the first group
+                        R[hs] = rn;
+                        l_run[hs] *= fsc;
+                        w_run[hs] *= fsc;
+                        if (pcol == 0) sh.fsc[buf][g + 4 * hs] = fsc;
+                    }
+                    (void)weights();
+                    since_move = 0;
+                }
+                if (lane == 0) sh.moved[buf] = move ? 1u : 0u;
+                since_move++;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) { l_run[hs] += ew[q][hs]; w_run[hs] += ww[q][hs]; }
+
+                // ---- hand the weights to the V wave
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) sh.ww[buf][hs][lane] = make_float4(ww[0][hs], ww[1][hs], ww[2][hs], ww[3][hs]);
+                if (lane == 0) sh.wq[buf] = wq;
+                __syncthreads();   // hand-over of buffer `buf`; also: the V wave is done with the buffer written next
+                gg = gnext;
+#pragma unroll
+                for (int q = 0; q < 4; q++) kw[q] = kwn[q];
+                nk = nkn; nv = nvn;
+            }
+        }
+#pragma unroll
+        for (int hs = 0; hs < 2; hs++) {
+            const float l_tot = lh_group_sum(l_run[hs], 16);
+            const float w_tot = lh_group_sum(w_run[hs], 16);
+            if (pcol == 0) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs]; }
+        }
+        if (lane == 0) sh.fin_unit = wq > 0.0f ? cmax_v / wq : 0.0f;
+        __syncthreads();
+    } else {
+        // =================================================================== V wave
+        gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+        v4i acc[4][4][2];      // [code byte e][field f][row set]: integer accumulators, rows = 4 limbs of head g + 4 * set
+        float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
 #pragma unroll
         for (int e = 0; e < 4; e++)
 #pragma unroll
             for (int f = 0; f < 4; f++)
 #pragma unroll
-                for (int hs = 0; hs < 2; hs++) {
-                    const v4i A = acc[e][f][hs];
-                    const float v = ((float)A[0] + 256.0f * (float)A[1]) + (65536.0f * (float)A[2] + 16777216.0f * (float)A[3]);
-                    outv[e][f][hs] = __builtin_fmaf(v, unit * (1.0f / (float)(1 << (2 * f))), outv[e][f][hs]);
-                    acc[e][f][hs] = (v4i){0, 0, 0, 0};
-                }
-        since_fold = 0;
-    };
-
-    if (c_hi > c_lo) {
-        const uint32_t g_first = c_lo >> 6, g_last = (c_hi - 1) >> 6;
-        GroupGeom gg = geom(g_first);
-        u32x4_t kw[4], kwn[4];   // K codes of the current group and of the next one (a full step of prefetch distance)
-        uint32_t vx[4][4];
-        float nk, nv, nkn = 0.0f, nvn = 0.0f;
-        const uint32_t klane = pcol * stride + 16 * g, vlane = 4 * g * stride + 4 * pcol, nlane = lane * nstride;
-        auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw)[4], float& nk, float& nv) {
-            gptr_t kb = krec0 + (size_t)G_.pb * stride;
-            gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
-            if (G_.full) {
+                for (int hs = 0; hs < 2; hs++) { acc[e][f][hs] = (v4i){0, 0, 0, 0}; outv[e][f][hs] = 0.0f; }
+        // integer accumulators -> float outputs, accumulators cleared
+        auto fold = [&](float unit) {
 #pragma unroll
-                for (int q = 0; q < 4; q++) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
-                nk = ld_norm(knb + nlane);
-                nv = ld_norm(vnb + nlane);
-            } else {
+            for (int e = 0; e < 4; e++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    kw[q] = (u32x4_t){0u, 0u, 0u, 0u};
-                    if (is_valid(G_, 16 * q + pcol)) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
-                }
-                nk = nv = 0.0f;
-                if (is_valid(G_, lane)) { nk = ld_norm(knb + nlane); nv = ld_norm(vnb + nlane); }
-            }
-        };
-        auto load_v = [&](const GroupGeom& G_) {
-            gptr_t vb = vrec0 + (size_t)G_.pb * stride;
-            if (G_.full) {
-#pragma unroll
-                for (int m = 0; m < 4; m++)
-#pragma unroll
-                    for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
-            } else {
-#pragma unroll
-                for (int m = 0; m < 4; m++)
-#pragma unroll
-                    for (int qq = 0; qq < 4; qq++) {
-                        vx[m][qq] = 0u;
-                        if (is_valid(G_, 16 * qq + 4 * g + m)) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
-                    }
-            }
-        };
-        load_k(gg, kw, nk, nv);
-        load_v(gg);
-
-        // One group of 64 positions.  MAY_FOLD = false is the steady-state copy: it returns false, with nothing but the
-        // logits computed, when a weight would leave the fixed-point range; the MAY_FOLD = true copy then redoes the
-        // group and moves the reference.  (Keeping the rare path out of the hot loop keeps the accumulators in place.)
-        auto step = [&](auto may_fold_tag, uint32_t G) -> bool {
-            constexpr bool MAY_FOLD = decltype(may_fold_tag)::value;
-            const bool more = G < g_last;
-            const GroupGeom gnext = geom(more ? G + 1 : G);
-            if (more) load_k(gnext, kwn, nkn, nvn);
-
-            // ---- norms of the group -> LDS
-            {
-                const bool valid = lane >= gg.vlo && lane < gg.vhi;
-                __builtin_amdgcn_wave_barrier();
-                s_norm[wave][lane] = make_float4(nk * kLog2e, valid ? 0.0f : -INFINITY, valid ? nv : 0.0f, 0.0f);
-                __builtin_amdgcn_wave_barrier();
-            }
-
-            // ---- K side: logits of 4 tiles x (this lane's column position, heads g and g + 4)
-            float lg[4][2], vn[4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const uint32_t w[4] = {kw[q].x, kw[q].y, kw[q].z, kw[q].w};
-                v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
-#pragma unroll
-                for (int m = 0; m < 4; m++) {
-                    const uint32_t u = w[m] >> 4;
-                    b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
-                    b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
-                    b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
-                    b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
-                }
-                const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[0][lane][0]);   // operand pf at rqo[64 * pf]
-                v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
-                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
-                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
-                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
-                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
-                acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
-                if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
-                    v4i d0, d1, d2, d3;
-#pragma unroll
-                    for (int m = 0; m < 4; m++) {
-                        const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
-                        d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
-                        d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
-                    }
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
-                }
-                const float4 nrm = s_norm[wave][16 * q + pcol];
-                vn[q] = nrm.z;
-#pragma unroll
-                for (int hs = 0; hs < 2; hs++) {
-                    const int t_lo = (acc1[2 * hs] << 2) + acc4[2 * hs];
-                    const int t_hi = (acc1[2 * hs + 1] << 2) + acc4[2 * hs + 1];
-                    const float inner = (float)(t_lo + (t_hi << 8)) * cs[hs] + ca[hs];
-                    lg[q][hs] = nrm.x * inner + nrm.y;
-                }
-            }
-
-            // ---- softmax weights relative to the running reference R; move R only when the fixed-point range is left
-            float ew[4][2], ww[4][2];
-            auto weights = [&]() {   // returns whether any weight of the wave leaves the fixed-point range (or is NaN)
-                float wm = 0.0f;
-#pragma unroll
-                for (int q = 0; q < 4; q++)
+                for (int f = 0; f < 4; f++)
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        ew[q][hs] = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
-                        ww[q][hs] = ew[q][hs] * vn[q];
-                        wm = fmaxf(wm, ww[q][hs]);
+                        const v4i A = acc[e][f][hs];
+                        const float v = ((float)A[0] + 256.0f * (float)A[1]) + (65536.0f * (float)A[2] + 16777216.0f * (float)A[3]);
+                        outv[e][f][hs] = __builtin_fmaf(v, unit * (1.0f / (float)(1 << (2 * f))), outv[e][f][hs]);
+                        acc[e][f][hs] = (v4i){0, 0, 0, 0};
                     }
-                return __builtin_amdgcn_ballot_w64(!(wm <= wlimit)) != 0;
-            };
-            const bool out_of_range = weights();
-            if (out_of_range || since_fold >= 256u) {     // uniform; true for the first group (wlimit starts negative)
-                if constexpr (!MAY_FOLD) return false;
-                fold();
-                float vm = fmaxf(fmaxf(vn[0], vn[1]), fmaxf(vn[2], vn[3]));
-                vm = lh_group_max(vm, 64);
-                vref = fmaxf(vref, vm);
-                wlimit = vref * (float)(1 << kHeadroom);
-                wq = wlimit > 0.0f ? kVQ / wlimit : 0.0f;
-#pragma unroll
-                for (int hs = 0; hs < 2; hs++) {
-                    float m = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
-                    m = lh_group_max(m, 16);
-                    const float rn = fmaxf(R[hs], m);
-                    const float fsc = __builtin_amdgcn_exp2f(R[hs] - rn);   // 0 for the first group
-                    R[hs] = rn;
-                    l_run[hs] *= fsc;
-                    w_run[hs] *= fsc;
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-#pragma unroll
-                        for (int f = 0; f < 4; f++) outv[e][f][hs] *= fsc;
-                }
-                (void)weights();
-            }
-            since_fold++;
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-#pragma unroll
-                for (int hs = 0; hs < 2; hs++) { l_run[hs] += ew[q][hs]; w_run[hs] += ww[q][hs]; }
+        };
 
-            // ---- weights -> 31-bit fixed point, one word of 4 signed limbs per (tile, head, plane); byte transpose to
-            //      "limb i over the four tiles" and hand each word to the lane that owns it as an MFMA row:
-            //      lane (column 4A+B, row group g) feeds row 4g + i of k-group A, word B.
-            {
-                const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
-                __builtin_amdgcn_wave_barrier();
+        if (any) {
+            GroupGeom gg = geom(g_first);
+            uint32_t vx[4][4];
+            const uint32_t vlane = 4 * g * stride + 4 * pcol;
+            auto load_v = [&](const GroupGeom& G_) {
+                gptr_t vb = vrec0 + (size_t)G_.pb * stride;
+                if (G_.full) {
+#pragma unroll
+                    for (int m = 0; m < 4; m++)
+#pragma unroll
+                        for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
+                } else {
+#pragma unroll
+                    for (int m = 0; m < 4; m++)
+#pragma unroll
+                        for (int qq = 0; qq < 4; qq++) {
+                            vx[m][qq] = 0u;
+                            if (is_valid(G_, 16 * qq + 4 * g + m)) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
+                        }
+                }
+            };
+            load_v(gg);
+
+            // One group.  The MAY_FOLD = false copy is the steady state: it returns false right after the barrier when the
+            // K wave moved the reference; the MAY_FOLD = true copy then handles that group without a second barrier.
+            // (Keeping the rare path out of the hot loop keeps the accumulators in place.)
+            auto step = [&](auto may_fold_tag, uint32_t G, bool wait) -> bool {
+                constexpr bool MAY_FOLD = decltype(may_fold_tag)::value;
+                const uint32_t buf = (G - g_first) & 1u;
+                const bool more = G < g_last;
+                if (wait) __syncthreads();
+                const bool moved = __builtin_amdgcn_readfirstlane(sh.moved[buf]) != 0;
+                if (moved) {
+                    if constexpr (!MAY_FOLD) return false;
+                    fold(sh.unit_old[buf]);
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        const float fsc = sh.fsc[buf][g + 4 * hs];
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+#pragma unroll
+                            for (int f = 0; f < 4; f++) outv[e][f][hs] *= fsc;
+                    }
+                }
+                // ---- weights -> 31-bit fixed point, one word of 4 signed limbs per (tile, head, plane); byte transpose to
+                //      "limb i over the four tiles" and hand each word to the lane that owns it as an MFMA row:
+                //      lane (column 4A+B, row group g) feeds row 4g + i of k-group A, word B.
+                {
+                    const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
+                    const float wqv = sh.wq[buf] * inv_cmax_v;
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        const float4 wv = sh.ww[buf][hs][lane];
+                        const float wws[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+                        for (int pl = 0; pl < nplanes; pl++) {
+                            const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * wqv;
+                            uint32_t lw[4], tr[4];
+#pragma unroll
+                            for (int q = 0; q < 4; q++) {
+                                const int qv = (int)(wws[q] * cq);                    // truncation: |qv| <= kVQ < 127 * 2^24
+                                lw[q] = ((uint32_t)qv + 0x00808080u) ^ 0x00808080u;    // bytes = signed limbs, least significant first
+                            }
+                            transpose4x4(lw, tr);
+                            uint8_t* dst = &sh.wx[pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
+#pragma unroll
+                            for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t*>(dst + 16 * i) = tr[i];
+                        }
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+                uint32_t y[4][4];   // [word m][code byte e]: byte e of positions 16qq + 4g + m, qq = 0..3
+#pragma unroll
+                for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
+                if (more) load_v(geom(G + 1));   // the V registers are free
 #pragma unroll
                 for (int pl = 0; pl < nplanes; pl++) {
-                    const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * inv_cmax_v * wq;
+                    const v4i wop0 = *reinterpret_cast<const v4i*>(&sh.wx[pl][0][lane * 16]);
+                    const v4i wop1 = *reinterpret_cast<const v4i*>(&sh.wx[pl][1][lane * 16]);
 #pragma unroll
-                    for (int hs = 0; hs < 2; hs++) {
-                        uint32_t lw[4], tr[4];
+                    for (int e = 0; e < 4; e++) {
+                        uint32_t yp[4];   // the plane's bit of every field at the even bit positions
 #pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            const int qv = (int)(ww[q][hs] * cq);                 // truncation: |qv| <= kVQ < 127 * 2^24
-                            lw[q] = ((uint32_t)qv + 0x00808080u) ^ 0x00808080u;    // bytes = signed limbs, least significant first
+                        for (int m = 0; m < 4; m++) yp[m] = pl == 0 ? y[m][e] : pl == 1 ? y[m][e] >> 1 : y[m][e] & (y[m][e] >> 1);
+#pragma unroll
+                        for (int f = 0; f < 4; f++) {
+                            v4i b;
+#pragma unroll
+                            for (int m = 0; m < 4; m++) b[m] = (int)(yp[m] & (0x01010101u << (2 * f)));
+                            acc[e][f][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop0, b, acc[e][f][0], 0, 0, 0);
+                            acc[e][f][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop1, b, acc[e][f][1], 0, 0, 0);
                         }
-                        transpose4x4(lw, tr);
-                        uint8_t* dst = &s_wx[wave][pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
-#pragma unroll
-                        for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t*>(dst + 16 * i) = tr[i];
                     }
                 }
-                __builtin_amdgcn_wave_barrier();
-            }
+                return true;
+            };
 
-            // ---- V side
-            uint32_t y[4][4];   // [word m][code byte e]: byte e of positions 16qq + 4g + m, qq = 0..3
-#pragma unroll
-            for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
-            if (more) load_v(gnext);   // the V registers are free
-#pragma unroll
-            for (int pl = 0; pl < nplanes; pl++) {
-                const v4i wop0 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][0][lane * 16]);
-                const v4i wop1 = *reinterpret_cast<const v4i*>(&s_wx[wave][pl][1][lane * 16]);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    uint32_t yp[4];   // the plane's bit of every field at the even bit positions
-#pragma unroll
-                    for (int m = 0; m < 4; m++) yp[m] = pl == 0 ? y[m][e] : pl == 1 ? y[m][e] >> 1 : y[m][e] & (y[m][e] >> 1);
-#pragma unroll
-                    for (int f = 0; f < 4; f++) {
-                        v4i b;
-#pragma unroll
-                        for (int m = 0; m < 4; m++) b[m] = (int)(yp[m] & (0x01010101u << (2 * f)));
-                        acc[e][f][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop0, b, acc[e][f][0], 0, 0, 0);
-                        acc[e][f][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop1, b, acc[e][f][1], 0, 0, 0);
-                    }
+            uint32_t G = g_first;
+            bool wait = true;
+            while (G <= g_last) {
+                step(std::true_type{}, G, wait);
+                G++;
+                wait = true;
+                while (G <= g_last) {
+                    if (!step(std::false_type{}, G, true)) { wait = false; break; }
+                    G++;
                 }
             }
-            gg = gnext;
-#pragma unroll
-            for (int q = 0; q < 4; q++) kw[q] = kwn[q];
-            nk = nkn; nv = nvn;
-            return true;
-        };
-
-        uint32_t G = g_first;
-        while (G <= g_last) {
-            step(std::true_type{}, G);
-            G++;
-            while (G <= g_last && step(std::false_type{}, G)) G++;
         }
-        fold();
-    }
+        __syncthreads();   // the K wave's totals
+        fold(sh.fin_unit);
 
-    // ---- the wave's result: final output (one split) or a partial record for the merge kernel
+        // ---- the workgroup's result: final output (one split) or a partial record for the merge kernel
 #pragma unroll
-    for (int hs = 0; hs < 2; hs++) {
-        const float l_tot = lh_group_sum(l_run[hs], 16);
-        const float w_tot = lh_group_sum(w_run[hs], 16);
-        const uint32_t h = g + 4 * hs;
-        if (h >= group) continue;
-        const uint32_t qh = kvh * group + h;
-        const float bias = alpha * w_tot;
-        if (nsplit == 1) {
-            float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 16 * pcol;
-            const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+        for (int hs = 0; hs < 2; hs++) {
+            const uint32_t h = g + 4 * hs;
+            if (h >= group) continue;
+            const float l_tot = sh.fin_l[h], w_tot = sh.fin_w[h];
+            const uint32_t qh = kvh * group + h;
+            const float bias = alpha * w_tot;
+            if (nsplit == 1) {
+                float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 16 * pcol;
+                const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                *reinterpret_cast<float4*>(dst + 4 * e) = make_float4((outv[e][0][hs] + bias) * inv, (outv[e][1][hs] + bias) * inv,
-                                                                      (outv[e][2][hs] + bias) * inv, (outv[e][3][hs] + bias) * inv);
-        } else {
-            float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * nsplit + split) * partial_record_floats(kHeadDim);
-            if (pcol == 0) { rec[0] = R[hs] * kLn2; rec[1] = l_tot; }
+                for (int e = 0; e < 4; e++)
+                    *reinterpret_cast<float4*>(dst + 4 * e) = make_float4((outv[e][0][hs] + bias) * inv, (outv[e][1][hs] + bias) * inv,
+                                                                          (outv[e][2][hs] + bias) * inv, (outv[e][3][hs] + bias) * inv);
+            } else {
+                float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * nsplit + split) * partial_record_floats(kHeadDim);
+                if (pcol == 0) { rec[0] = sh.fin_r[h] * kLn2; rec[1] = l_tot; }
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                *reinterpret_cast<float4*>(rec + 4 + 16 * pcol + 4 * e) =
-                    make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
+                for (int e = 0; e < 4; e++)
+                    *reinterpret_cast<float4*>(rec + 4 + 16 * pcol + 4 * e) =
+                        make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
+            }
         }
     }
 }
 
-
 template <int OCC>
-__global__ __launch_bounds__(256, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
+__global__ __launch_bounds__(128, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
     __shared__ __align__(16) AttnShared sh;
     // L[c] = alpha + beta*bit0 + gam*bit1 + delta*bit0*bit1.  A delta that is only float noise of a symmetric table
     // (|delta| <= 1e-5 max|L|) is spread by the least-squares affine fit bit0*bit1 ~ -1/4 + bit0/2 + bit1/2, which
@@ -501,21 +555,21 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
 }
 
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
-    // One wave per chunk of positions; about one wave per SIMD over the whole launch, at least 128 positions each.
-    const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
+    // One workgroup (a K wave and a V wave) per chunk of positions; about `wps` waves per SIMD over the whole launch,
+    // at least 128 positions per chunk.
     static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
     static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
-    const uint64_t wave_slots = (uint64_t)ctx->cu_count * 4 * wps;
-    uint64_t splits = std::max<uint64_t>(1, wave_slots / pairs);
+    const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
+    const uint64_t wg_slots = (uint64_t)ctx->cu_count * 2 * wps;
+    uint64_t splits = std::max<uint64_t>(1, wg_slots / pairs);
     splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
     splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
     const size_t rec = partial_record_floats(p.head_dim);
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
-    const uint32_t waves = splits * pairs >= wave_slots && splits >= 4 ? 4 : 1;
-    const dim3 grid((uint32_t)((splits + waves - 1) / waves), (uint32_t)pairs);
-    if (occ == 1) hipLaunchKernelGGL(attention_tq_mfma_kernel<1>, grid, dim3(64 * waves), 0, ctx->stream, a, p);
-    else hipLaunchKernelGGL(attention_tq_mfma_kernel<2>, grid, dim3(64 * waves), 0, ctx->stream, a, p);
+    const dim3 grid((uint32_t)splits, (uint32_t)pairs);
+    if (occ == 1) hipLaunchKernelGGL(attention_tq_mfma_kernel<1>, grid, dim3(128), 0, ctx->stream, a, p);
+    else hipLaunchKernelGGL(attention_tq_mfma_kernel<2>, grid, dim3(128), 0, ctx->stream, a, p);
     return lh_check_launch(op);
 }
 
