@@ -199,14 +199,17 @@ __global__ __launch_bounds__(kThreads) void attention_tq_split_kernel(
 }
 
 // flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.  One workgroup per
-// (query, head); the per-split factors exp(m_s - max) are computed once into LDS, then every thread
-// folds its output dimension over the splits with coalesced row reads.
+// (query, head, slab of 32 output dims): the per-split factors exp(m_s - max) are computed once into LDS,
+// then 8 thread groups fold interleaved subsets of the splits (coalesced 128-byte row reads) and are
+// summed through LDS.
+constexpr int kReduceDims = 32;
 __global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
                                                                  uint32_t num_splits) {
     __shared__ float f_s[kMaxSplits];
     __shared__ float red[8];
+    __shared__ float part[8][kReduceDims];
     const uint32_t qh = blockIdx.x;     // flattened (query, head)
-    const size_t rec = (size_t)head_dim + 4;
+    const size_t rec = partial_record_floats(head_dim);
     const float* base = ws + (size_t)qh * num_splits * rec;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     float m_loc = -INFINITY;
@@ -227,17 +230,22 @@ __global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* _
     __syncthreads();
     const float gl = (red[4] + red[5]) + (red[6] + red[7]);
     const float inv = gl > 0.0f ? 1.0f / gl : 0.0f;
-    for (uint32_t d = threadIdx.x; d < head_dim; d += 256) {
-        float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
-        uint32_t s = 0;
-        for (; s + 4 <= num_splits; s += 4) {
+    const uint32_t dl = threadIdx.x & (kReduceDims - 1), slice = threadIdx.x / kReduceDims;   // 8 slices of the splits
+    const uint32_t d = blockIdx.y * kReduceDims + dl;
+    float o0 = 0.0f, o1 = 0.0f;
+    if (d < head_dim) {
+        uint32_t s = slice;
+        for (; s + 8 < num_splits; s += 16) {
             o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
-            o1 += f_s[s + 1] * base[(size_t)(s + 1) * rec + 4 + d];
-            o2 += f_s[s + 2] * base[(size_t)(s + 2) * rec + 4 + d];
-            o3 += f_s[s + 3] * base[(size_t)(s + 3) * rec + 4 + d];
+            o1 += f_s[s + 8] * base[(size_t)(s + 8) * rec + 4 + d];
         }
-        for (; s < num_splits; s++) o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
-        out[(size_t)qh * head_dim + d] = ((o0 + o1) + (o2 + o3)) * inv;
+        if (s < num_splits) o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
+    }
+    part[slice][dl] = o0 + o1;
+    __syncthreads();
+    if (slice == 0 && d < head_dim) {
+        const float o = ((part[0][dl] + part[1][dl]) + (part[2][dl] + part[3][dl])) + ((part[4][dl] + part[5][dl]) + (part[6][dl] + part[7][dl]));
+        out[(size_t)qh * head_dim + d] = o * inv;
     }
 }
 
@@ -295,7 +303,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     if (r != LH_OK) return r;
     batch->dispatch_count++;
     if (p.num_splits > 1) {
-        hipLaunchKernelGGL(attention_tq_reduce_kernel, dim3(p.num_queries * p.num_q_heads), dim3(256), 0, ctx->stream,
+        hipLaunchKernelGGL(attention_tq_reduce_kernel, dim3(p.num_queries * p.num_q_heads, (p.head_dim + kReduceDims - 1) / kReduceDims), dim3(256), 0, ctx->stream,
                            (const float*)ctx->workspace, (float*)out->ptr, p.head_dim, p.num_splits);
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
