@@ -26,6 +26,7 @@
 //      columns are summed with DPP.
 #include "common.hpp"
 #include "xquant.hpp"
+#include <algorithm>
 #include <cstdlib>
 
 namespace {
@@ -86,10 +87,12 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
     const uint64_t my_slots = blockIdx.x < total_slots ? (total_slots - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
     const uint64_t nitems = my_slots * ngroups;                     // one item = one (tile, block group)
 
-    // Chunk -> (row, chunk-in-row) of the lane's staging loads, precomputed for the two group shapes a row can
-    // have: a full group of 8 blocks (33 chunks per row) and the trailing group of nb % 8 blocks.
+    // Chunk -> (row, chunk-in-row) of the lane's staging loads.  Full groups of 8 blocks (33 chunks per row): the global
+    // offsets live in registers and the image offsets are linear in the chunk index.  The trailing group of nb % 8
+    // blocks: both tables live in LDS (one per workgroup), read back when such a group comes up.
     const uint32_t nbg_tail = (nb & 7) ? (nb & 7) : 8;
-    uint32_t goff_full[kStageLoads], loff_full[kStageLoads], goff_tail[kStageLoads], loff_tail[kStageLoads];
+    uint32_t goff_full[kStageLoads];
+    uint32_t* tail_tab = reinterpret_cast<uint32_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [2][kStageLoads][64]
     {
         const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
 #pragma unroll
@@ -97,24 +100,37 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
             const uint32_t ch = lane + 64 * i;
             const uint32_t cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
             goff_full[i] = rf * row_bytes + jf * 16;
-            loff_full[i] = ch < 16 * 33 ? rf * (33 * 16) + jf * 16 : 0xFFFFFFFFu;        // surplus lanes do not store
-            const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
-            goff_tail[i] = rt * row_bytes + jt * 16;
-            loff_tail[i] = ch < 16 * nch_t ? rt * ss_t + jt * 16 : 0xFFFFFFFFu;
+            if (wave == 0) {
+                const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
+                tail_tab[i * 64 + lane] = rt * row_bytes + jt * 16;
+                tail_tab[(kStageLoads + i) * 64 + lane] = ch < 16 * nch_t ? rt * ss_t + jt * 16 : 0xFFFFFFFFu;   // surplus lanes do not store
+            }
         }
     }
-    auto item_tile_base = [&](uint64_t n, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
-        const uint64_t slot = (uint64_t)blockIdx.x + (n / ngroups) * gridDim.x;
-        grp = (uint32_t)(n % ngroups);
-        const uint32_t prob = (uint32_t)(slot / slots_per_problem);
-        tile = (uint32_t)(slot - (uint64_t)prob * slots_per_problem) * nwaves + wave;
-        pb = problems ? problems[prob] : single;
+    __syncthreads();
+    // Position in the work order, advanced incrementally (all scalar, no division in the loop).
+    struct Item { uint32_t grp, sip, prob; };                       // block group, slot within the problem, problem
+    const uint32_t step_prob = gridDim.x / slots_per_problem, step_sip = gridDim.x % slots_per_problem;
+    auto advance = [&](Item it) {
+        if (++it.grp == ngroups) {
+            it.grp = 0;
+            it.sip += step_sip;
+            it.prob += step_prob;
+            if (it.sip >= slots_per_problem) { it.sip -= slots_per_problem; it.prob++; }
+        }
+        return it;
     };
+    auto item_tile_base = [&](const Item& it, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
+        grp = it.grp;
+        tile = it.sip * nwaves + wave;
+        pb = problems ? problems[it.prob] : single;
+    };
+    Item cur{0u, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
 
     u32x4_t pre[kStageLoads];
-    auto prefetch = [&](uint64_t n) {
+    auto prefetch = [&](const Item& it) {
         uint32_t grp, tile; Tq2Problem pb;
-        item_tile_base(n, grp, tile, pb);
+        item_tile_base(it, grp, tile, pb);
         const bool tail = grp + 1 == ngroups && (nb & 7);
         if ((tile << 4) + 16 <= rows) {                              // every row of the tile exists: precomputed offsets
             gptr_t base = (gptr_t)pb.matrix + (size_t)(tile << 4) * row_bytes + (size_t)grp * 528;
@@ -123,7 +139,7 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
                 for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + goff_full[i]);
             } else {
 #pragma unroll
-                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + goff_tail[i]);
+                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + tail_tab[i * 64 + lane]);
             }
         } else {                                                     // last, partial tile (or a surplus wave): clamp the row
             const uint32_t nbg = tail ? nbg_tail : 8;
@@ -141,12 +157,13 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
         }
     };
 
-    if (nitems) prefetch(0);
+    if (nitems) prefetch(cur);
     const void* staged = nullptr;
     float rowacc[4] = {0.f, 0.f, 0.f, 0.f};
     for (uint64_t n = 0; n < nitems; n++) {
         uint32_t grp, tile; Tq2Problem pb;
-        item_tile_base(n, grp, tile, pb);
+        item_tile_base(cur, grp, tile, pb);
+        const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
             quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x);
@@ -164,14 +181,18 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
         if (nbg == 8) {
 #pragma unroll
             for (int i = 0; i < kStageLoads; i++)
-                if (loff_full[i] != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + loff_full[i]) = pre[i];
+                if (i < kStageLoads - 1 || lane < 16 * 33 - 64 * (kStageLoads - 1))   // 528 chunks: the last round is partial
+                    *reinterpret_cast<u32x4_t*>(image + lane * 16 + 1024 * i) = pre[i];
         } else {
 #pragma unroll
-            for (int i = 0; i < kStageLoads; i++)
-                if (loff_tail[i] != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + loff_tail[i]) = pre[i];
+            for (int i = 0; i < kStageLoads; i++) {
+                const uint32_t lo = tail_tab[(kStageLoads + i) * 64 + lane];
+                if (lo != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + lo) = pre[i];
+            }
         }
         __builtin_amdgcn_wave_barrier();
-        if (n + 1 < nitems) prefetch(n + 1);
+        if (n + 1 < nitems) prefetch(nxt);
+        cur = nxt;
 
         // ---- column constants of this group
         const bool col_valid = b0 + cb < nb;
@@ -183,8 +204,8 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
 
         // accumulators by code scale: fields 0 and 1 arrive as code, field 2 as 4*code, field 3 as 16*code
         v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0}, acc16 = (v4i){0, 0, 0, 0};
-#define LH_TQ2_BLOCK(B)                                                                                         \
-        if ((B) < nbg) {                                                                                        \
+#define LH_TQ2_BLOCK(B, GUARD)                                                                                         \
+        if (!(GUARD) || (B) < nbg) {                                                                                        \
             constexpr int o = (B) * 66;                                                                         \
             const u32x4_t c0 = *reinterpret_cast<const u32x4_t*>(arow + (o & ~15));                             \
             const u32x4_t c1 = *reinterpret_cast<const u32x4_t*>(arow + (o & ~15) + 16);                        \
@@ -198,18 +219,23 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
                 a2[m] = (int)(t & 0x0C0C0C0Cu);                                                                 \
                 a3[m] = (int)(t & 0x30303030u);                                                                 \
             }                                                                                                   \
-            const uint8_t* bp = lds + (cb == (B) ? my_off : zero_off);                                          \
-            const v4i x0 = *reinterpret_cast<const v4i*>(bp);                                                   \
-            const v4i x1 = *reinterpret_cast<const v4i*>(bp + 32);                                              \
-            const v4i x2 = *reinterpret_cast<const v4i*>(bp + 64);                                              \
-            const v4i x3 = *reinterpret_cast<const v4i*>(bp + 96);                                              \
+            const uint8_t* bq = lds + (cb == (B) ? my_off : zero_off);                                          \
+            const v4i x0 = *reinterpret_cast<const v4i*>(bq);                                                   \
+            const v4i x1 = *reinterpret_cast<const v4i*>(bq + 32);                                              \
+            const v4i x2 = *reinterpret_cast<const v4i*>(bq + 64);                                              \
+            const v4i x3 = *reinterpret_cast<const v4i*>(bq + 96);                                              \
             acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, x0, acc1, 0, 0, 0);                                \
             acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, x1, acc1, 0, 0, 0);                                \
             acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, x2, acc4, 0, 0, 0);                                \
             acc16 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a3, x3, acc16, 0, 0, 0);                              \
         }
-        LH_TQ2_BLOCK(0) LH_TQ2_BLOCK(1) LH_TQ2_BLOCK(2) LH_TQ2_BLOCK(3)
-        LH_TQ2_BLOCK(4) LH_TQ2_BLOCK(5) LH_TQ2_BLOCK(6) LH_TQ2_BLOCK(7)
+        if (nbg == 8) {   // full group: no branches between the blocks, so their LDS reads and MFMAs interleave
+            LH_TQ2_BLOCK(0, false) LH_TQ2_BLOCK(1, false) LH_TQ2_BLOCK(2, false) LH_TQ2_BLOCK(3, false)
+            LH_TQ2_BLOCK(4, false) LH_TQ2_BLOCK(5, false) LH_TQ2_BLOCK(6, false) LH_TQ2_BLOCK(7, false)
+        } else {
+            LH_TQ2_BLOCK(0, true) LH_TQ2_BLOCK(1, true) LH_TQ2_BLOCK(2, true) LH_TQ2_BLOCK(3, true)
+            LH_TQ2_BLOCK(4, true) LH_TQ2_BLOCK(5, true) LH_TQ2_BLOCK(6, true) LH_TQ2_BLOCK(7, true)
+        }
 #undef LH_TQ2_BLOCK
 
         // ---- epilogue on the dense accumulator: combine scales and limbs, zero point, block scales
@@ -252,9 +278,12 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const uint32_t waves = threads / 64;
     const uint64_t slots = (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
     static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    const uint64_t cap = (uint64_t)ctx->cu_count * (threads == 256 ? wg_cu : 4 * wg_cu);
+    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4;
+    const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_guess);          // workgroups per CU that LDS allows
+    const int wg_eff = threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu;
+    const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
-    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes;
+    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4;
     if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
 
     Tq2Problem single{(const uint8_t*)matrices[0], vectors[0], outputs[0]};
