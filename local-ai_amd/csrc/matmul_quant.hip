@@ -262,6 +262,15 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
     LH_REQUIRE(((uintptr_t)input->ptr & 15) == 0, "%s: input must be 16-byte aligned", op);
     LH_REQUIRE(((uintptr_t)weight->ptr & 1) == 0, "%s: weight must be 2-byte aligned", op);
     const bool mfma = kind == kF16W || (!force_multivec && m > (uint32_t)kMaxMultivecM);
+    if (!mfma) {
+        // up to 16 activation rows: m matvecs against the same matrix in one launch of the M = 1 kernels (the weights
+        // of one call stay cache resident between the rows); shapes they do not take fall through to multivec_kernel
+        const int rr = lh_matvec_rows(batch, kind == kQ4 ? LH_Q4_0 : LH_TQ2_0, m, weight, input, at, output, ct, n, k, op);
+        if (rr != -1) {
+            if (rr == LH_OK) batch->dispatch_count++;
+            return rr;
+        }
+    }
     hipStream_t s = batch->ctx->stream;
     const uint8_t* W = (const uint8_t*)weight->ptr;
     if (kind == kQ4) launch_by_in<kQ4>(mfma, s, input->ptr, at, W, output->ptr, ct, m, k, n);

@@ -34,6 +34,12 @@ struct MatvecProblem {
     const void* vector;
     void* output;
 };
+// The problem that travels in the kernel arguments.  With a descriptor table absent and count > 1, problem i is this
+// one with its vector and output advanced by i strides (the rows of a small activation batch against one matrix).
+struct MatvecBase {
+    MatvecProblem p;
+    uint32_t xstride, ystride;   // bytes
+};
 
 // ---- per-lane activation registers for one unit column -------------------------
 template <int FMT, int L>
@@ -196,7 +202,7 @@ template <int FMT> __host__ __device__ constexpr int steps_in_flight(int npos) {
 
 // One launch serves `count` problems of the same shape (count == 1 for the plain matvec).
 template <int FMT, int L, int NPOS, typename XT, typename YT>
-__global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, MatvecProblem single,
+__global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, MatvecBase single,
                                                              uint32_t count, uint32_t rows, uint32_t K, uint32_t lpr_log2,
                                                              uint32_t steps_per_wg) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -224,7 +230,9 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         const uint32_t s_begin = (uint32_t)(g0 - (uint64_t)prob * steps_per_problem);
         const uint64_t seg_end64 = (uint64_t)(prob + 1) * steps_per_problem;
         const uint32_t s_end = (uint32_t)((g1 < seg_end64 ? g1 : seg_end64) - (uint64_t)prob * steps_per_problem);
-        const MatvecProblem pb = problems ? problems[prob] : single;   // one problem travels in the kernel arguments
+        const MatvecProblem pb = problems ? problems[prob]
+                                          : MatvecProblem{single.p.matrix, (const char*)single.p.vector + (size_t)prob * single.xstride,
+                                                          (char*)single.p.output + (size_t)prob * single.ystride};
         // this wave's contiguous share of [s_begin, s_end)
         const uint32_t nseg = s_end - s_begin;
         const uint32_t per_wave = (nseg + kWaves - 1) / kWaves;
@@ -438,7 +446,7 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
 }
 
 template <int FMT, int L, int NPOS>
-int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const MatvecProblem& single, uint32_t count, lh_dtype xt,
+int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const MatvecBase& single, uint32_t count, lh_dtype xt,
                  lh_dtype yt, uint32_t rows, uint32_t K, const LaunchGeom& g) {
 #define LH_LAUNCH(XT, YT)                                                                                              \
     hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream, \
@@ -452,7 +460,7 @@ int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const Matve
 }
 
 template <int FMT, int L>
-int launch_npos(lh_context* ctx, const MatvecProblem* p, const MatvecProblem& single, uint32_t count, lh_dtype xt, lh_dtype yt,
+int launch_npos(lh_context* ctx, const MatvecProblem* p, const MatvecBase& single, uint32_t count, lh_dtype xt, lh_dtype yt,
                 uint32_t rows, uint32_t K, const LaunchGeom& g) {
     switch (g.npos) {
         case 1: return launch_typed<FMT, L, 1>(ctx, p, single, count, xt, yt, rows, K, g);
@@ -523,7 +531,7 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         const void** px = count <= 8 ? stack_x : pm + count;
         void** py = count <= 8 ? stack_y : (void**)(pm + 2 * (size_t)count);
         for (uint32_t i = 0; i < count; i++) { pm[i] = matrices[i]->ptr; px[i] = vectors[i]->ptr; py[i] = outputs[i]->ptr; }
-        int r = lh_launch_matvec_tq2_mfma(ctx, count, pm, px, py, xt, yt, rows, cols);
+        int r = lh_launch_matvec_tq2_mfma(ctx, count, pm, px, py, xt, yt, rows, cols, 0, 0);
         if (count > 8) free((void*)pm);
         if (r == LH_OK) batch->dispatch_count++;
         return r;
@@ -531,7 +539,7 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     // One problem travels in the kernel arguments; several go through a descriptor array in the
     // top quarter of the context workspace (the copy is stream ordered, so it cannot overtake a
     // kernel that still reads the previous set).
-    MatvecProblem single{(const uint8_t*)matrices[0]->ptr, vectors[0]->ptr, outputs[0]->ptr};
+    MatvecBase single{MatvecProblem{(const uint8_t*)matrices[0]->ptr, vectors[0]->ptr, outputs[0]->ptr}, 0, 0};
     MatvecProblem* dev_desc = nullptr;
     if (count > 1) {
         const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
@@ -577,7 +585,40 @@ int matvec_blocking(lh_context* ctx, lh_quant fmt, const lh_buffer* m, const lh_
     return lh_batch_commit_and_wait(&b);
 }
 
+
+int matvec_rows_impl(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer* weight, const lh_buffer* input, lh_dtype at,
+                     lh_buffer* output, lh_dtype ct, uint32_t n, uint32_t k, const char* op) {
+    if (at == LH_BF16 || ct == LH_BF16) return -1;
+    if (!fast_path_ok(fmt, weight->ptr, input->ptr, k)) return -1;
+    const size_t xstride = (size_t)k * lh_dtype_size(at), ystride = (size_t)n * lh_dtype_size(ct);
+    if ((xstride & 15) != 0 || xstride > 0xFFFFFFFFull || ystride > 0xFFFFFFFFull) return -1;
+    lh_context* ctx = batch->ctx;
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    const size_t wbytes = (size_t)n * (k / blk) * (fmt == LH_Q4_0 ? 18 : 66);
+    const size_t slack = weight->len - wbytes + weight->slack;
+    int r;
+    if (fmt == LH_TQ2_0 && tq2_on_matrix_cores() && k <= 12288 && ((k / 256) % 8 == 0 || slack >= 16)) {
+        const void* pm[1] = {weight->ptr}; const void* px[1] = {input->ptr}; void* py[1] = {output->ptr};
+        r = lh_launch_matvec_tq2_mfma(ctx, m, pm, px, py, at, ct, n, k, (uint32_t)xstride, (uint32_t)ystride);
+    } else {
+        MatvecBase single{MatvecProblem{(const uint8_t*)weight->ptr, input->ptr, output->ptr}, (uint32_t)xstride, (uint32_t)ystride};
+        const int L = x_limbs();
+        const LaunchGeom g = plan(fmt, m, n, k, ctx->cu_count, L);
+        if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
+                                       : launch_npos<LH_Q4_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
+        else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
+                        : launch_npos<LH_TQ2_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
+    }
+    (void)op;
+    return r;
+}
+
 }  // namespace
+
+int lh_matvec_rows(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer* weight, const lh_buffer* input, lh_dtype at,
+                   lh_buffer* output, lh_dtype ct, uint32_t n, uint32_t k, const char* op) {
+    return matvec_rows_impl(batch, fmt, m, weight, input, at, output, ct, n, k, op);
+}
 
 extern "C" {
 

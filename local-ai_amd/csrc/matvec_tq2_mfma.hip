@@ -44,6 +44,12 @@ struct Tq2Problem {
     const void* vector;
     void* output;
 };
+// The problem that travels in the kernel arguments.  With a descriptor table absent and count > 1, problem i is this
+// one with its vector and output advanced by i strides (the rows of a small activation batch against one matrix).
+struct Tq2Base {
+    Tq2Problem p;
+    uint32_t xstride, ystride;   // bytes
+};
 
 __device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
     typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
@@ -60,7 +66,7 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
 }
 
 template <typename XT, typename YT>
-__global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Problem single,
+__global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t nb = K >> 8;                                     // blocks per row
@@ -123,7 +129,9 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
     auto item_tile_base = [&](const Item& it, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
         grp = it.grp;
         tile = it.sip * nwaves + wave;
-        pb = problems ? problems[it.prob] : single;
+        if (problems) pb = problems[it.prob];
+        else pb = Tq2Problem{single.p.matrix, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
+                             (char*)single.p.output + (size_t)it.prob * single.ystride};
     };
     Item cur{0u, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
 
@@ -269,7 +277,9 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
 
 // Entry used by matvec_quant.hip's dispatcher. Arrays are host arrays of device pointers.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
-                              void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K) {
+                              void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K, uint32_t xstride,
+                              uint32_t ystride) {
+    const bool strided = xstride != 0 || ystride != 0;   // problem i = problem 0 advanced by i strides: no descriptor table
     const uint32_t nb = K >> 8;
     const uint64_t tiles = (uint64_t)((rows + 15) >> 4) * count;
     // small jobs: one wave per workgroup so the tiles spread over all CUs; large jobs: four waves share one
@@ -286,9 +296,9 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4;
     if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
 
-    Tq2Problem single{(const uint8_t*)matrices[0], vectors[0], outputs[0]};
+    Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
     Tq2Problem* dev = nullptr;
-    if (count > 1) {
+    if (count > 1 && !strided) {
         const size_t bytes = (size_t)count * sizeof(Tq2Problem);
         if (bytes > ctx->workspace_bytes / 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems exceed the descriptor area", count);
         Tq2Problem* host = (Tq2Problem*)malloc(bytes);
