@@ -208,6 +208,48 @@ def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
             "single_gbs": T * per_pos / ev_s * 1e-6}
 
 
+def bench_attention_sweep(pkg, ctx, K, steps, warmup):
+    """Context sweep (single decode token, sequences rotating so the cache comes from HBM) and the
+    sliding-window layer: window 512 over a 512-slot ring that has wrapped many times."""
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    per_pos = nkv * (2 * (hd * bits // 8) + 4)
+    res = {}
+    for T, lanes in ((4096, 64), (16384, 32), (131072, 8)):
+        r = bench_attention(pkg, ctx, K, steps, warmup, T=T, lanes=lanes)
+        res[f"ctx_{T}"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"],
+                           "batched_lanes": lanes, "batched_us_per_launch": r["batched_us_per_launch"], "batched_gbs": r["batched_gbs"]}
+    # sliding window: every lane is a 512-slot ring; logical position far beyond the ring size
+    ring, lanes, pos = 512, 4096, 100000
+    pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, ring, hd, nkv, bits)
+    g = pkg.synth.rng(9, 1)
+    rq = pkg.Buffer.from_slice(ctx, g.standard_normal((lanes, nq, hd), dtype=np.float32))
+    out = pkg.Buffer.empty(ctx, lanes * nq * hd * 4)
+    positions = pkg.Buffer.from_slice(ctx, np.full(lanes, pos, np.uint32))
+    batch = pkg.CommandBatch(ctx)
+
+    def step_batched():
+        K.flash_attention_tq_batched_into(batch, rq, pool[0], pool[1], pool[2], pool[3], levels, out, positions, hd, ring, nq, nkv,
+                                          ring, bits, lanes, ring)
+
+    _, ev_b = time_steps(pkg, ctx, step_batched, steps, warmup)
+    cb = hd * bits // 8
+    views = [[pool[0].view(l * ring * nkv * cb, ring * nkv * cb), pool[1].view(l * ring * nkv * 2, ring * nkv * 2),
+              pool[2].view(l * ring * nkv * cb, ring * nkv * cb), pool[3].view(l * ring * nkv * 2, ring * nkv * 2)] for l in range(64)]
+    calls = [bound_call(pkg.lib().lh_flash_attention_tq_into, batch, rq, v[0], v[1], v[2], v[3], levels, out, hd, pos + 1, pos, nq, nkv,
+                        ring, bits, ring) for v in views]
+    it = [0]
+
+    def step_single():
+        calls[it[0] % len(calls)]()
+        it[0] += 1
+
+    _, ev_s = time_steps(pkg, ctx, step_single, max(steps, 50), warmup)
+    res["swa_window512_ring512"] = {"batched_lanes": lanes, "batched_us_per_launch": ev_b * 1e3,
+                                    "batched_tokens_per_s": lanes / (ev_b * 1e-3), "batched_gbs": lanes * ring * per_pos / ev_b * 1e-6,
+                                    "single_us_per_token": ev_s * 1e3}
+    return res
+
+
 def bench_layer(pkg, ctx, K, steps, warmup):
     """Small-batch decode over one decoder layer's seven projections (mixed Q4_0 / TQ2_0)."""
     g = pkg.synth.rng(3)
@@ -245,8 +287,9 @@ def bench_prefill(pkg, ctx, K, steps, warmup):
         ab = pkg.Buffer.from_slice(ctx, pkg.synth.f32_to_bf16_bits(pkg.synth.activations(m, k, g)))
         cb = pkg.Buffer.empty(ctx, m * n * 4)
 
-        def step():
-            w.matmul_nt_typed_into(batch, K, ab, pkg.BF16, cb, pkg.F32, m)
+        import ctypes as C
+        step = bound_call(pkg.lib().lh_matmul_nt_quant_typed_into, batch, C.c_int(w.ty), ab, C.c_int(pkg.BF16), w.buf, cb,
+                          C.c_int(pkg.F32), m, k, n)
 
         _, ev = time_steps(pkg, ctx, step, steps, warmup)
         tf = 2.0 * m * k * n / (ev * 1e-3) * 1e-12
@@ -338,6 +381,8 @@ def main():
         extra["tq2_attention_32k"] = att
         log(f"[bench] tq2 attention 32k: batched {att['batched_tokens_per_s']:.0f} tok/s ({att['batched_gbs']:.0f} GB/s), "
             f"single {att['single_us_per_token']:.1f} us/token")
+        extra["tq2_attention_sweep"] = bench_attention_sweep(pkg, ctx, K, args.steps, args.warmup)
+        log("[bench] attention sweep:", extra["tq2_attention_sweep"])
         extra["decoder_layer_small_batch"] = bench_layer(pkg, ctx, K, args.steps, args.warmup)
         extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] layer:", extra["decoder_layer_small_batch"])

@@ -89,142 +89,223 @@ __global__ __launch_bounds__(256) void multivec_kernel(const void* __restrict__ 
 }
 
 // -------------------------------------------------------------------- MFMA ----
-constexpr int BM = 128, BN = 128, BK = 32, LDK = BK + 8;   // LDS row stride in f16 (80 bytes)
+// C[M, N] = A[M, K] . W[N, K]^T with f16 MFMA: BM x 128 output tile per workgroup (BM = 64 or 128), 128-wide k steps.
+// Weight tiles are dequantised to exactly the f16 values of the CPU path (qat_recover.rs:23-97) with packed f16
+// arithmetic -- (1024 + code) is built by a byte permute, then (x - 1025) * d for TQ2_0 or (x - 1032) * d for Q4_0,
+// whose single rounding equals f16::from_f32 of the f32 product -- and staged through LDS together with the
+// activations (converted to f16); the next step's global loads fly during the MFMAs.
+constexpr int BN = 128, BK = 128, LDK = BK + 8;   // LDS row stride in f16 (272 bytes: conflict-free 16-byte reads)
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-struct Frag16 { uint32_t w[8]; };   // 16 f16 values
-
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) { return (uint32_t)lh_f2h(a) | ((uint32_t)lh_f2h(b) << 16); }
+__device__ __forceinline__ uint32_t h2_sub_mul(uint32_t x, uint32_t bias, uint32_t d2) {
+    const f16x2 r = (__builtin_bit_cast(f16x2, x) - __builtin_bit_cast(f16x2, bias)) * __builtin_bit_cast(f16x2, d2);
+    return __builtin_bit_cast(uint32_t, r);
+}
 
-// 16 consecutive activations of one row as f16 (zero past row M).
+// Raw global data of one staging run (32 consecutive k of one row), kept in registers across two k steps so that the
+// loads have two steps of MFMA work to arrive; converted to f16 words just before they go to LDS.
+template <int ADT> struct RawA { uint4 v[ADT == LH_F32 ? 8 : 4]; };
+template <int FMT> struct RawB { uint4 q[FMT == kF16W ? 4 : 2]; uint32_t d; };
+
 template <int ADT>
-__device__ __forceinline__ void load_a16(Frag16& f, const void* A, uint32_t row, uint32_t M, uint32_t K, uint32_t k0) {
-    if (row >= M) {
+__device__ __forceinline__ void load_raw_a(RawA<ADT>& r, const void* A, uint32_t row, uint32_t M, uint32_t K, uint32_t k0) {
+    constexpr int NV = ADT == LH_F32 ? 8 : 4;
+    if (row >= M || k0 >= K) {   // K is a multiple of 32: a run that starts inside a row ends inside it
 #pragma unroll
-        for (int i = 0; i < 8; i++) f.w[i] = 0;
+        for (int i = 0; i < NV; i++) r.v[i] = make_uint4(0u, 0u, 0u, 0u);
         return;
     }
-    if constexpr (ADT == LH_F32) {
-        const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(A) + (size_t)row * K + k0);
+    const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(A) + ((size_t)row * K + k0) * (ADT == LH_F32 ? 4 : 2));
 #pragma unroll
-        for (int i = 0; i < 4; i++) { const float4 v = p[i]; f.w[2 * i] = pack_h2(v.x, v.y); f.w[2 * i + 1] = pack_h2(v.z, v.w); }
-    } else {
-        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(A) + (size_t)row * K + k0);
-        const uint4 a = p[0], b = p[1];
-        const uint32_t r[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    for (int i = 0; i < NV; i++) r.v[i] = p[i];
+}
+
+template <int ADT>
+__device__ __forceinline__ void convert_a(uint32_t (&f)[16], const RawA<ADT>& r) {
+    if constexpr (ADT == LH_F32) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            if constexpr (ADT == LH_F16) f.w[i] = r[i];
-            else f.w[i] = pack_h2(lh_bf2f((uint16_t)(r[i] & 0xFFFF)), lh_bf2f((uint16_t)(r[i] >> 16)));   // bf16 -> f16
-        }
-    }
-}
-
-// 16 consecutive dequantised weights of one row: elements k0 + half*16 .. +16 of weight row `row`.
-template <int FMT>
-__device__ __forceinline__ void load_b16(Frag16& f, const uint8_t* W, uint32_t row, uint32_t K, uint32_t k0, uint32_t half) {
-    if constexpr (FMT == kF16W) {
-        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(W) + (size_t)row * K + k0 + half * 16);
-        const uint4 a = p[0], b = p[1];
-        f.w[0] = a.x; f.w[1] = a.y; f.w[2] = a.z; f.w[3] = a.w; f.w[4] = b.x; f.w[5] = b.y; f.w[6] = b.z; f.w[7] = b.w;
-    } else if constexpr (FMT == kQ4) {
-        const uint8_t* bp = W + ((size_t)row * (K >> 5) + (k0 >> 5)) * 18;
-        const float d = lh_h2f(*reinterpret_cast<const uint16_t*>(bp));
-        uint4 qv; __builtin_memcpy(&qv, __builtin_assume_aligned(bp + 2, 2), 16);
-        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
-        const uint32_t sh = half * 4;    // low nibbles -> elements 0..15, high nibbles -> 16..31
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t v = q[i] >> sh;
-            f.w[2 * i] = pack_h2(((float)(v & 15) - 8.0f) * d, ((float)((v >> 8) & 15) - 8.0f) * d);
-            f.w[2 * i + 1] = pack_h2(((float)((v >> 16) & 15) - 8.0f) * d, ((float)((v >> 24) & 15) - 8.0f) * d);
+            f[2 * i] = pack_h2(__builtin_bit_cast(float, r.v[i].x), __builtin_bit_cast(float, r.v[i].y));
+            f[2 * i + 1] = pack_h2(__builtin_bit_cast(float, r.v[i].z), __builtin_bit_cast(float, r.v[i].w));
         }
     } else {
-        const uint32_t blk = k0 >> 8, s = (k0 >> 5) & 7;               // 32-element slice s of the block
-        const uint8_t* bp = W + ((size_t)row * (K >> 8) + blk) * 66;
-        const float d = lh_h2f(*reinterpret_cast<const uint16_t*>(bp + 64));
-        uint4 qv; __builtin_memcpy(&qv, __builtin_assume_aligned(bp + (s >> 2) * 32 + half * 16, 2), 16);
-        const uint32_t q[4] = {qv.x, qv.y, qv.z, qv.w};
-        const uint32_t sh = (s & 3) * 2;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t v = q[i] >> sh;
-            f.w[2 * i] = pack_h2(d * ((float)(v & 3) - 1.0f), d * ((float)((v >> 8) & 3) - 1.0f));
-            f.w[2 * i + 1] = pack_h2(d * ((float)((v >> 16) & 3) - 1.0f), d * ((float)((v >> 24) & 3) - 1.0f));
+            const uint32_t w[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (ADT == LH_F16) f[4 * i + j] = w[j];
+                else f[4 * i + j] = pack_h2(lh_bf2f((uint16_t)(w[j] & 0xFFFF)), lh_bf2f((uint16_t)(w[j] >> 16)));   // bf16 -> f16
+            }
         }
     }
 }
 
-__device__ __forceinline__ void store_frag(_Float16* dst, const Frag16& f) {
-    *reinterpret_cast<uint4*>(dst) = make_uint4(f.w[0], f.w[1], f.w[2], f.w[3]);
-    *reinterpret_cast<uint4*>(dst + 8) = make_uint4(f.w[4], f.w[5], f.w[6], f.w[7]);
+// Elements k0 .. k0 + 32 of weight row `row` (k0 a multiple of 32).
+template <int FMT>
+__device__ __forceinline__ void load_raw_b(RawB<FMT>& r, const uint8_t* W, uint32_t row, uint32_t K, uint32_t k0) {
+    if (k0 >= K) {   // past the end of the row in the last k step: scale 0 (and zero words for f16 weights)
+        r.d = 0;
+#pragma unroll
+        for (int i = 0; i < (FMT == kF16W ? 4 : 2); i++) r.q[i] = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
+    if constexpr (FMT == kF16W) {
+        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(W) + (size_t)row * K + k0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.q[i] = p[i];
+        r.d = 0;
+    } else if constexpr (FMT == kQ4) {
+        const uint8_t* bp = W + ((size_t)row * (K >> 5) + (k0 >> 5)) * 18;
+        r.d = *reinterpret_cast<const uint16_t*>(bp);
+        __builtin_memcpy(&r.q[0], __builtin_assume_aligned(bp + 2, 2), 16);
+        r.q[1] = make_uint4(0u, 0u, 0u, 0u);
+    } else {
+        const uint32_t blk = k0 >> 8, s = (k0 >> 5) & 7;               // 32-element slice s of the block: bytes (s/4)*32.., field s%4
+        const uint8_t* bp = W + ((size_t)row * (K >> 8) + blk) * 66;
+        r.d = *reinterpret_cast<const uint16_t*>(bp + 64) | (((s & 3) * 2) << 16);   // scale bits and the field's shift
+        __builtin_memcpy(&r.q[0], __builtin_assume_aligned(bp + (s >> 2) * 32, 2), 16);
+        __builtin_memcpy(&r.q[1], __builtin_assume_aligned(bp + (s >> 2) * 32 + 16, 2), 16);
+    }
 }
 
-template <int FMT, int ADT, int CDT>
+template <int FMT>
+__device__ __forceinline__ void convert_b(uint32_t (&f)[16], const RawB<FMT>& r) {
+    if constexpr (FMT == kF16W) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) { f[4 * i] = r.q[i].x; f[4 * i + 1] = r.q[i].y; f[4 * i + 2] = r.q[i].z; f[4 * i + 3] = r.q[i].w; }
+    } else if constexpr (FMT == kQ4) {
+        const uint32_t d2 = (r.d & 0xFFFFu) | (r.d << 16);
+        const uint32_t q[4] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w};
+        // byte j: low nibble = element j, high nibble = element 16 + j
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t lo = q[i] & 0x0F0F0F0Fu, hi = (q[i] >> 4) & 0x0F0F0F0Fu;
+            f[2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u), 0x64086408u, d2);          // 1024 + q - 1032
+            f[2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u), 0x64086408u, d2);
+            f[8 + 2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u), 0x64086408u, d2);
+            f[8 + 2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u), 0x64086408u, d2);
+        }
+    } else {
+        const uint32_t d2 = (r.d & 0xFFFFu) | (r.d << 16), sh = r.d >> 16;
+        const uint32_t q[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t c = (q[i] >> sh) & 0x03030303u;
+            f[2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04010400u), 0x64016401u, d2);            // 1024 + c - 1025
+            f[2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04030402u), 0x64016401u, d2);
+        }
+    }
+}
+
+template <int NW>
+__device__ __forceinline__ void store_words(_Float16* dst, const uint32_t (&f)[NW]) {
+#pragma unroll
+    for (int i = 0; i < NW / 4; i++) *reinterpret_cast<uint4*>(dst + 8 * i) = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+}
+
+template <int FMT, int ADT, int CDT, int BM>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
                                                          uint32_t M, uint32_t K, uint32_t N) {
+    constexpr int TI = BM / 32;                              // 16-row MFMA tiles per wave along M (2 x 2 waves)
+    constexpr int AR = BM / 64;                              // 32-element activation runs staged per thread
     __shared__ __align__(16) _Float16 As[BM * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;                 // 2 x 2 waves, 64 x 64 each
+    const int wm = wave >> 1, wn = wave & 1;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const uint32_t ld_row = tid >> 1, ld_half = tid & 1;     // staging: one 16-element run per thread
-    const uint32_t a_row = m0 + ld_row;
-    const uint32_t b_row = n0 + ld_row < N ? n0 + ld_row : N - 1;   // past-the-end rows re-read the last (never stored)
+    const uint32_t a_ld_row = BM == 128 ? tid >> 1 : tid >> 2, a_ld_k = BM == 128 ? (tid & 1) * 64 : (tid & 3) * 32;
+    const uint32_t b_ld_row = tid >> 1, b_ld_k = (tid & 1) * 64;
+    const uint32_t a_row = m0 + a_ld_row;
+    const uint32_t b_row = n0 + b_ld_row < N ? n0 + b_ld_row : N - 1;   // past-the-end rows re-read the last (never stored)
 
-    f32x4 acc[4][4];
+    f32x4 acc[TI][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    Frag16 ra, rb;
-    load_a16<ADT>(ra, A, a_row, M, K, ld_half * 16);
-    load_b16<FMT>(rb, W, b_row, K, 0, ld_half);
-    const uint32_t nk = K / BK;
-    for (uint32_t kt = 0; kt < nk; kt++) {
-        store_frag(&As[ld_row * LDK + ld_half * 16], ra);
-        store_frag(&Bs[ld_row * LDK + ld_half * 16], rb);
-        __syncthreads();
-        if (kt + 1 < nk) {      // next tile's global loads fly during the MFMAs
-            load_a16<ADT>(ra, A, a_row, M, K, (kt + 1) * BK + ld_half * 16);
-            load_b16<FMT>(rb, W, b_row, K, (kt + 1) * BK, ld_half);
+    RawA<ADT> ra[2][AR];   // [k step parity][run]
+    RawB<FMT> rb[2][2];
+    auto load_step = [&](int set, uint32_t kt) {
+#pragma unroll
+        for (int i = 0; i < AR; i++) load_raw_a<ADT>(ra[set][i], A, a_row, M, K, kt * BK + a_ld_k + 32 * i);
+#pragma unroll
+        for (int i = 0; i < 2; i++) load_raw_b<FMT>(rb[set][i], W, b_row, K, kt * BK + b_ld_k + 32 * i);
+    };
+    auto stage_step = [&](int set) {
+        uint32_t f[16];
+#pragma unroll
+        for (int i = 0; i < AR; i++) { convert_a<ADT>(f, ra[set][i]); store_words<16>(&As[a_ld_row * LDK + a_ld_k + 32 * i], f); }
+#pragma unroll
+        for (int i = 0; i < 2; i++) { convert_b<FMT>(f, rb[set][i]); store_words<16>(&Bs[b_ld_row * LDK + b_ld_k + 32 * i], f); }
+    };
+    auto mfma_step = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ks++) {
+            f16x8 fa[TI], fb[4];
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+                fa[i] = *reinterpret_cast<const f16x8*>(&As[(wm * (BM / 2) + i * 16 + (lane & 15)) * LDK + ks * 32 + (lane >> 4) * 8]);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                fb[j] = *reinterpret_cast<const f16x8*>(&Bs[(wn * 64 + j * 16 + (lane & 15)) * LDK + ks * 32 + (lane >> 4) * 8]);
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
-        f16x8 fa[4], fb[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            fa[i] = *reinterpret_cast<const f16x8*>(&As[(wm * 64 + i * 16 + (lane & 15)) * LDK + (lane >> 4) * 8]);
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            fb[j] = *reinterpret_cast<const f16x8*>(&Bs[(wn * 64 + j * 16 + (lane & 15)) * LDK + (lane >> 4) * 8]);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    const uint32_t nk = (K + BK - 1) / BK;
+    load_step(0, 0);
+    if (nk > 1) load_step(1, 1);
+    for (uint32_t kt = 0; kt < nk; kt += 2) {   // two k steps per trip: the register sets alternate without copies
+        stage_step(0);
         __syncthreads();
+        if (kt + 2 < nk) load_step(0, kt + 2);
+        mfma_step();
+        __syncthreads();
+        if (kt + 1 < nk) {
+            stage_step(1);
+            __syncthreads();
+            if (kt + 3 < nk) load_step(1, kt + 3);
+            mfma_step();
+            __syncthreads();
+        }
     }
     // D tile: lane holds column (lane & 15), rows 4*(lane >> 4) .. +4
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const uint32_t n = n0 + wn * 64 + j * 16 + (lane & 15);
             if (n >= N) continue;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const uint32_t m = m0 + wm * 64 + i * 16 + (lane >> 4) * 4 + r;
+                const uint32_t m = m0 + wm * (BM / 2) + i * 16 + (lane >> 4) * 4 + r;
                 if (m < M) store_elem<CDT>(C, (size_t)m * N + n, acc[i][j][r]);
             }
         }
 }
 
 template <int FMT, int ADT>
-int launch_by_out(bool mfma, hipStream_t s, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n) {
+int launch_by_out(bool mfma, hipStream_t s, int cus, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
+                  uint32_t n) {
     if (mfma) {
-        const dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
-        if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32>), grid, dim3(256), 0, s, A, W, C, m, k, n);
-        else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+        // 128-row tiles reuse each dequantised weight tile twice as often; 64-row tiles when that leaves CUs idle
+        const uint64_t tiles128 = (uint64_t)((n + BN - 1) / BN) * ((m + 127) / 128);
+        if (tiles128 >= 2ull * (uint64_t)cus) {
+            const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+        } else {
+            const dim3 grid((n + BN - 1) / BN, (m + 63) / 64);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+        }
     } else {
         if constexpr (FMT != kF16W) {
             const dim3 grid((n + 3) / 4);
@@ -236,12 +317,12 @@ int launch_by_out(bool mfma, hipStream_t s, const void* A, const uint8_t* W, voi
 }
 
 template <int FMT>
-int launch_by_in(bool mfma, hipStream_t s, const void* A, lh_dtype at, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
+int launch_by_in(bool mfma, hipStream_t s, int cus, const void* A, lh_dtype at, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
                  uint32_t n) {
     switch (at) {
-        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, s, A, W, C, ct, m, k, n);
-        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, s, A, W, C, ct, m, k, n);
-        default: return launch_by_out<FMT, LH_F16>(mfma, s, A, W, C, ct, m, k, n);
+        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, s, cus, A, W, C, ct, m, k, n);
+        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, s, cus, A, W, C, ct, m, k, n);
+        default: return launch_by_out<FMT, LH_F16>(mfma, s, cus, A, W, C, ct, m, k, n);
     }
 }
 
@@ -273,9 +354,9 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
     }
     hipStream_t s = batch->ctx->stream;
     const uint8_t* W = (const uint8_t*)weight->ptr;
-    if (kind == kQ4) launch_by_in<kQ4>(mfma, s, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, s, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else launch_by_in<kF16W>(true, s, input->ptr, at, W, output->ptr, ct, m, k, n);
+    if (kind == kQ4) launch_by_in<kQ4>(mfma, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
+    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
+    else launch_by_in<kF16W>(true, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
     int r = lh_check_launch(op);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
