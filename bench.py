@@ -38,7 +38,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/matvec_tq2_mfma_grouped_8192x2048.md), scaled by the same counters on the library's plain
 # copy kernel; None until that profile has been taken for the current kernel.
-MEASURED_TRAFFIC_BYTES = 1086451302
+MEASURED_TRAFFIC_BYTES = 1086334464
 
 
 def log(*a):
@@ -325,6 +325,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill",
+                    help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: the hot path is a single-GPU kernel path and no multi-GPU "
@@ -363,8 +365,9 @@ def main():
             log("[bench] PARITY FAILURE: GPU result differs from the CPU path beyond 1e-3")
             sys.exit(1)
 
-    if not args.quick:
-        del ws, ys
+    legs = set() if args.quick else set(args.legs.split(","))
+    del ws, ys
+    if "matvec" in legs:
         for fmt, r, c in (("q4_0", 2048, 2048), ("tq2_0", 2048, 8192)):
             res = bench_matvec_grouped(pkg, ctx, K, fmt, r, c, args.steps, args.warmup)
             res.pop("_state")
@@ -376,16 +379,20 @@ def main():
             res["frac_of_hbm_peak"] = res["gbs"] / HBM_PEAK_GBS
             extra[f"matvec_{fmt}_{r}x{c}_single_launch"] = res
             log(f"[bench] {fmt} {r}x{c} single launch: {res['us_per_launch']:.1f} us, {res['gbs']:.0f} GB/s")
+    if "attention" in legs:
         att = bench_attention(pkg, ctx, K, args.steps, args.warmup)
         att["batched_frac_of_hbm_peak"] = att["batched_gbs"] / HBM_PEAK_GBS
         extra["tq2_attention_32k"] = att
         log(f"[bench] tq2 attention 32k: batched {att['batched_tokens_per_s']:.0f} tok/s ({att['batched_gbs']:.0f} GB/s), "
             f"single {att['single_us_per_token']:.1f} us/token")
+    if "sweep" in legs:
         extra["tq2_attention_sweep"] = bench_attention_sweep(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] attention sweep:", extra["tq2_attention_sweep"])
+    if "layer" in legs:
         extra["decoder_layer_small_batch"] = bench_layer(pkg, ctx, K, args.steps, args.warmup)
-        extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] layer:", extra["decoder_layer_small_batch"])
+    if "prefill" in legs:
+        extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] prefill:", extra["prefill_matmul_512x2048x8192_bf16"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
