@@ -65,9 +65,10 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
     for (int m = 0; m < 4; m++) out[m] = rem ? __builtin_amdgcn_alignbit(in[m + q + 1], in[m + q], 8 * rem) : in[m + q];
 }
 
-template <typename XT, typename YT>
+template <typename XT, typename YT, bool SPLITK>
 __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
+    constexpr bool splitk = SPLITK;
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t nb = K >> 8;                                     // blocks per row
     uint32_t* xq = reinterpret_cast<uint32_t*>(lds);                // [2][K/4] activation limbs
@@ -87,11 +88,15 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
     // Work order: "slots" of nwaves consecutive tiles, dealt round-robin to the workgroups, so that at any moment
     // the whole grid reads one compact, advancing window of the weight stream.
     const uint32_t tiles_per_problem = (rows + 15) >> 4;
-    const uint32_t slots_per_problem = (tiles_per_problem + nwaves - 1) / nwaves;
+    // Normally a slot is nwaves consecutive tiles, one per wave, each wave walking all block groups of its tile.  With
+    // `splitk` (few tiles, long rows) a slot is ONE tile whose block groups are dealt to the waves (nwaves divides their
+    // number) and the waves' partial row sums are added through LDS in a fixed order.
+    const uint32_t slots_per_problem = splitk ? tiles_per_problem : (tiles_per_problem + nwaves - 1) / nwaves;
     const uint64_t total_slots = (uint64_t)slots_per_problem * count;
     const uint32_t ngroups = (nb + 7) >> 3;
     const uint64_t my_slots = blockIdx.x < total_slots ? (total_slots - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
-    const uint64_t nitems = my_slots * ngroups;                     // one item = one (tile, block group)
+    const uint32_t grp0 = splitk ? (uint32_t)wave : 0u, grp_step = splitk ? (uint32_t)nwaves : 1u;
+    const uint64_t nitems = my_slots * (ngroups / grp_step);        // one item = one (tile, block group)
 
     // Chunk -> (row, chunk-in-row) of the lane's staging loads.  Full groups of 8 blocks (33 chunks per row): the global
     // offsets live in registers and the image offsets are linear in the chunk index.  The trailing group of nb % 8
@@ -118,8 +123,9 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
     struct Item { uint32_t grp, sip, prob; };                       // block group, slot within the problem, problem
     const uint32_t step_prob = gridDim.x / slots_per_problem, step_sip = gridDim.x % slots_per_problem;
     auto advance = [&](Item it) {
-        if (++it.grp == ngroups) {
-            it.grp = 0;
+        it.grp += grp_step;
+        if (it.grp >= ngroups) {
+            it.grp = grp0;
             it.sip += step_sip;
             it.prob += step_prob;
             if (it.sip >= slots_per_problem) { it.sip -= slots_per_problem; it.prob++; }
@@ -128,12 +134,12 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
     };
     auto item_tile_base = [&](const Item& it, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
         grp = it.grp;
-        tile = it.sip * nwaves + wave;
+        tile = splitk ? it.sip : it.sip * nwaves + wave;
         if (problems) pb = problems[it.prob];
         else pb = Tq2Problem{single.p.matrix, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
                              (char*)single.p.output + (size_t)it.prob * single.ystride};
     };
-    Item cur{0u, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
+    Item cur{grp0, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
 
     u32x4_t pre[kStageLoads];
     auto prefetch = [&](const Item& it) {
@@ -256,8 +262,9 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
             rowacc[i] += (float)iq16 * (lh_h2f(dbits) * xscale16);
         }
 
-        if (grp + 1 == ngroups) {      // tile complete: sum the 16 columns of each row, store 4 rows per lane group
+        if (grp + grp_step >= ngroups) {      // tile complete for this wave: sum the 16 columns of each row (4 rows per lane group)
             YT* y = static_cast<YT*>(pb.output);
+            float* part = reinterpret_cast<float*>(tail_tab + 2 * kStageLoads * 64);   // [nwaves][16] partial rows (splitk)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float v = rowacc[i];
@@ -266,8 +273,22 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
                 v += lh_dpp_f<LH_DPP_HALF_MIRROR>(v);
                 v += lh_dpp_f<LH_DPP_ROW_MIRROR>(v);
                 const uint32_t orow = (tile << 4) + 4 * g + i;
-                if (c == 0 && tile < tiles_per_problem && orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                if (!splitk) {
+                    if (c == 0 && tile < tiles_per_problem && orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                } else if (c == 0) {
+                    part[wave * 16 + 4 * g + i] = v;
+                }
                 rowacc[i] = 0.0f;
+            }
+            if (splitk) {   // every wave of the workgroup reaches this point once per slot
+                __syncthreads();
+                if (wave == 0 && lane < 16) {
+                    float v = part[lane];
+                    for (int w = 1; w < nwaves; w++) v += part[w * 16 + lane];
+                    const uint32_t orow = (tile << 4) + lane;
+                    if (orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                }
+                __syncthreads();
             }
         }
     }
@@ -283,17 +304,22 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const uint32_t nb = K >> 8;
     const uint64_t tiles = (uint64_t)((rows + 15) >> 4) * count;
     // small jobs: one wave per workgroup so the tiles spread over all CUs; large jobs: four waves share one
-    // quantised activation vector
-    const uint32_t threads = tiles >= (uint64_t)ctx->cu_count * 8 ? 256 : 64;
+    // quantised activation vector; few tiles with long rows: the block groups of a tile are split over 2-4 waves
+    const uint32_t ngroups = (nb + 7) >> 3;
+    uint32_t split_waves = 1;
+    if (tiles < (uint64_t)ctx->cu_count * 2)
+        for (uint32_t w = 4; w >= 2; w--) if (ngroups % w == 0) { split_waves = w; break; }
+    const uint32_t splitk = split_waves > 1 ? 1u : 0u;
+    const uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * 8 ? 256 : 64);
     const uint32_t waves = threads / 64;
-    const uint64_t slots = (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
+    const uint64_t slots = splitk ? tiles : (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
     static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4;
+    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 4 * 16 * 4;
     const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_guess);          // workgroups per CU that LDS allows
     const int wg_eff = threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu;
     const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
-    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4;
+    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 4 * 16 * 4;
     if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
@@ -309,8 +335,11 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         free(host);
         if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: descriptor upload: %s", hipGetErrorString(e));
     }
-#define LH_LAUNCH(XT, YT) \
-    hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K)
+#define LH_LAUNCH(XT, YT)                                                                                                          \
+    do {                                                                                                                           \
+        if (splitk) hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, true>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
+        else hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, false>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
+    } while (0)
     if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
     else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
