@@ -94,6 +94,35 @@ def test_prefill_config_bf16(pkg, gpu, oracle, fmt):
     print(f"prefill {fmt}: max normalised err {err:.2e}")
 
 
+@pytest.mark.parametrize("fmt", ["tq2_0", "q4_0"])
+def test_prefill_weight_tiles_are_the_cpu_f16_values(pkg, gpu, oracle, fmt):
+    """One-hot activation rows make the prefill matmul return the weight tile it staged: every sampled
+    column must equal the CPU path's dequantised f16 value bit for bit (incl. TQ2 code 3, subnormal and
+    zero scales from the reference's payload generators)."""
+    ctx, K = gpu
+    m, k, n = 96, 1024 + 32 * (fmt == "q4_0"), 200          # m > 16: the MFMA kernel; ragged n; k not a multiple of 128 for Q4_0
+    if fmt == "tq2_0":
+        k = 1280
+    raw = payload(fmt, n, k, 0x51DE).copy()
+    blk = 18 if fmt == "q4_0" else 66
+    doff = 0 if fmt == "q4_0" else 64
+    raw.reshape(-1, blk)[3, doff:doff + 2] = np.array([6e-8], np.float16).view(np.uint8)    # subnormal scale
+    raw.reshape(-1, blk)[5, doff:doff + 2] = 0                                               # zero scale
+    deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).reshape(n, k)
+    cols = (np.arange(m) * 37 + 5) % k
+    a = np.zeros((m, k), np.float16)
+    a[np.arange(m), cols] = 1.0
+    w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k)
+    ab, cb = pkg.Buffer.from_slice(ctx, a), pkg.Buffer.empty(ctx, m * n * 4)
+    batch = pkg.CommandBatch(ctx)
+    w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32, m)
+    batch.commit_and_wait()
+    got = cb.as_array(np.float32).reshape(m, n)
+    want = deq[:, cols].T.astype(np.float32)
+    assert np.array_equal(got.view(np.uint32) & 0x7FFFFFFF, want.view(np.uint32) & 0x7FFFFFFF)   # sign of zero aside
+    assert np.array_equal(got, want)
+
+
 def test_small_batch_layer_config_f32(pkg, gpu, oracle):
     """One decoder layer's seven projections with fp32 activations at M in {1, 4, 8, 16}."""
     ctx, K = gpu
