@@ -200,52 +200,92 @@ __global__ __launch_bounds__(kThreads) void attention_tq_split_kernel(
 
 // flash_decoding.metal:148-189 applied to the TQ partials: LSE merge over splits.  One workgroup per
 // (query, head, slab of 32 output dims): the per-split factors exp(m_s - max) are computed once into LDS,
-// then 8 thread groups fold interleaved subsets of the splits (coalesced 128-byte row reads) and are
-// summed through LDS.
-constexpr int kReduceDims = 32;
-__global__ __launch_bounds__(256) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
-                                                                 uint32_t num_splits) {
+// then thread groups fold interleaved subsets of the splits (coalesced 128-byte row reads, a batch of
+// them in flight per thread, the first batch requested before the factors are known) and are summed through LDS.
+constexpr int kReduceDims = 32;     // dims per workgroup
+constexpr int kReduceBatch = 16;    // records per thread whose loads are in flight together
+// kReduceSlices thread groups fold interleaved subsets of the splits: 16 for many splits (one long query), 2 for few
+// (many queries, each with its own small merge).
+template <int kReduceSlices>
+__global__ __launch_bounds__(kReduceDims * kReduceSlices) void attention_tq_reduce_kernel(const float* __restrict__ ws, float* __restrict__ out,
+                                                                                          uint32_t head_dim, uint32_t num_splits) {
+    constexpr int kThreads = kReduceDims * kReduceSlices, kWaves = kThreads / 64;
+    constexpr int kMl = kMaxSplits / kThreads;   // (m, l) pairs per thread
     __shared__ float f_s[kMaxSplits];
-    __shared__ float red[8];
-    __shared__ float part[8][kReduceDims];
+    __shared__ float red[2 * kWaves];
+    __shared__ float part[kReduceSlices][kReduceDims];
     const uint32_t qh = blockIdx.x;     // flattened (query, head)
     const size_t rec = partial_record_floats(head_dim);
     const float* base = ws + (size_t)qh * num_splits * rec;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t dl = threadIdx.x & (kReduceDims - 1), slice = threadIdx.x / kReduceDims;
+    const uint32_t d = blockIdx.y * kReduceDims + dl;
+    const bool d_ok = d < head_dim;
+
+    // The first batch of accumulator rows does not depend on the split weights: request it before anything else.
+    float v[kReduceBatch];
+#pragma unroll
+    for (int i = 0; i < kReduceBatch; i++) {
+        const uint32_t sp = slice + kReduceSlices * i;
+        v[i] = (d_ok && sp < num_splits) ? base[(size_t)sp * rec + 4 + d] : 0.0f;
+    }
+    // (m, l) of every split, kMl per thread
+    float2 ml[kMl];
+#pragma unroll
+    for (int i = 0; i < kMl; i++) {
+        const uint32_t sp = threadIdx.x + kThreads * i;
+        ml[i] = sp < num_splits ? *reinterpret_cast<const float2*>(base + (size_t)sp * rec) : make_float2(-INFINITY, 0.0f);
+    }
     float m_loc = -INFINITY;
-    for (uint32_t s = threadIdx.x; s < num_splits; s += 256) { const float m = base[s * rec]; f_s[s] = m; m_loc = fmaxf(m_loc, m); }
+#pragma unroll
+    for (int i = 0; i < kMl; i++) m_loc = fmaxf(m_loc, ml[i].x);
     m_loc = lh_group_max(m_loc, 64);
     if (lane == 0) red[wave] = m_loc;
     __syncthreads();
-    const float gm = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float gm = red[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) gm = fmaxf(gm, red[w]);
     float l_loc = 0.0f;
-    for (uint32_t s = threadIdx.x; s < num_splits; s += 256) {
-        const float m = f_s[s];
-        const float f = m == -INFINITY ? 0.0f : __expf(m - gm);
-        f_s[s] = f;
-        l_loc += f * base[s * rec + 1];
+#pragma unroll
+    for (int i = 0; i < kMl; i++) {
+        const uint32_t sp = threadIdx.x + kThreads * i;
+        const float f = ml[i].x == -INFINITY ? 0.0f : __expf(ml[i].x - gm);
+        if (sp < num_splits) f_s[sp] = f;
+        l_loc += f * ml[i].y;
     }
     l_loc = lh_group_sum(l_loc, 64);
-    if (lane == 0) red[4 + wave] = l_loc;
+    if (lane == 0) red[kWaves + wave] = l_loc;
     __syncthreads();
-    const float gl = (red[4] + red[5]) + (red[6] + red[7]);
+    float gl = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) gl += red[kWaves + w];
     const float inv = gl > 0.0f ? 1.0f / gl : 0.0f;
-    const uint32_t dl = threadIdx.x & (kReduceDims - 1), slice = threadIdx.x / kReduceDims;   // 8 slices of the splits
-    const uint32_t d = blockIdx.y * kReduceDims + dl;
-    float o0 = 0.0f, o1 = 0.0f;
-    if (d < head_dim) {
-        uint32_t s = slice;
-        for (; s + 8 < num_splits; s += 16) {
-            o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
-            o1 += f_s[s + 8] * base[(size_t)(s + 8) * rec + 4 + d];
-        }
-        if (s < num_splits) o0 += f_s[s] * base[(size_t)s * rec + 4 + d];
+
+    float o = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kReduceBatch; i++) {
+        const uint32_t sp = slice + kReduceSlices * i;
+        if (sp < num_splits) o = __builtin_fmaf(f_s[sp], v[i], o);
     }
-    part[slice][dl] = o0 + o1;
+    for (uint32_t s0 = kReduceSlices * kReduceBatch; s0 < num_splits; s0 += kReduceSlices * kReduceBatch) {   // more than 256 splits
+#pragma unroll
+        for (int i = 0; i < kReduceBatch; i++) {
+            const uint32_t sp = s0 + slice + kReduceSlices * i;
+            v[i] = (d_ok && sp < num_splits) ? base[(size_t)sp * rec + 4 + d] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < kReduceBatch; i++) {
+            const uint32_t sp = s0 + slice + kReduceSlices * i;
+            if (sp < num_splits) o = __builtin_fmaf(f_s[sp], v[i], o);
+        }
+    }
+    part[slice][dl] = o;
     __syncthreads();
-    if (slice == 0 && d < head_dim) {
-        const float o = ((part[0][dl] + part[1][dl]) + (part[2][dl] + part[3][dl])) + ((part[4][dl] + part[5][dl]) + (part[6][dl] + part[7][dl]));
-        out[(size_t)qh * head_dim + d] = o * inv;
+    if (slice == 0 && d_ok) {
+        float t = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kReduceSlices; i++) t += part[i][dl];
+        out[(size_t)qh * head_dim + d] = t * inv;
     }
 }
 
@@ -303,8 +343,13 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     if (r != LH_OK) return r;
     batch->dispatch_count++;
     if (p.num_splits > 1) {
-        hipLaunchKernelGGL(attention_tq_reduce_kernel, dim3(p.num_queries * p.num_q_heads, (p.head_dim + kReduceDims - 1) / kReduceDims), dim3(256), 0, ctx->stream,
-                           (const float*)ctx->workspace, (float*)out->ptr, p.head_dim, p.num_splits);
+        const dim3 rgrid(p.num_queries * p.num_q_heads, (p.head_dim + kReduceDims - 1) / kReduceDims);
+        if (p.num_splits <= 2 * kReduceBatch)
+            hipLaunchKernelGGL(attention_tq_reduce_kernel<2>, rgrid, dim3(kReduceDims * 2), 0, ctx->stream, (const float*)ctx->workspace,
+                               (float*)out->ptr, p.head_dim, p.num_splits);
+        else
+            hipLaunchKernelGGL(attention_tq_reduce_kernel<16>, rgrid, dim3(kReduceDims * 16), 0, ctx->stream, (const float*)ctx->workspace,
+                               (float*)out->ptr, p.head_dim, p.num_splits);
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
     }

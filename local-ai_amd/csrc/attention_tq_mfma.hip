@@ -107,64 +107,6 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     const float cmax_k = fmaxf(fmaxf(fabsf(beta), fabsf(0.5f * gam)), has_delta ? fabsf(delta) : 0.0f);
     const float cmax_v = fmaxf(fmaxf(fabsf(beta), fabsf(gam)), has_delta ? fabsf(delta) : 0.0f);
 
-    // ---- per head: max |rq| (quantisation scale) and sum(rq) (constant term of the level table)
-    for (uint32_t h = tid >> 5; h < (uint32_t)kMaxGroupHeads; h += blockDim.x >> 5) {
-        const uint32_t sub = tid & 31;
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.0f;
-        if (h < group) {
-            const float4 x0 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8);
-            const float4 x1 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8 + 4);
-            v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
-        }
-        float m = 0.0f, s = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) { m = fmaxf(m, fabsf(v[i])); s += v[i]; }
-        m = lh_group_max(m, 32);
-        s = lh_group_sum(s, 32);
-        if (sub == 0) { s_maxabs[h] = m; s_sum[h] = s; }
-    }
-    __syncthreads();
-
-    // ---- K-side A operands.  Row r of the MFMA: head (r / 4) + 4 * ((r / 2) % 2), limb r % 2, so that the lanes of
-    //      row group g end up with heads g and g + 4 on both the K and the V side.  k slot (word m, byte e) of
-    //      row group g is code byte j = 16g + 4m + e, i.e. dim 4j + f for the operand of field f.
-    {
-        const uint32_t h = (pcol >> 2) + 4 * ((pcol >> 1) & 1), limb = pcol & 1;
-        const float ma = s_maxabs[h];
-        const float inv = (ma > 0.0f && cmax_k > 0.0f) ? kQmax / (ma * cmax_k) : 0.0f;
-        for (uint32_t pl = wave; pl < (uint32_t)nplanes; pl += nwaves) {
-            const float mul = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv;
-            uint32_t words[4][4];
-#pragma unroll
-            for (int f = 0; f < 4; f++)
-#pragma unroll
-                for (int m = 0; m < 4; m++) words[f][m] = 0;
-#pragma unroll
-            for (int m = 0; m < 4; m++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (h < group) x = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + 4 * (16 * g + 4 * m + e));
-                    const float xv[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-                    for (int f = 0; f < 4; f++) {
-                        float r = __builtin_rintf(xv[f] * mul);
-                        r = fminf(fmaxf(r, -kQmax), kQmax);
-                        const int n = (int)r;
-                        const int lo = (int)(int8_t)(n & 0xFF);
-                        const int b = limb ? (n - lo) >> 8 : lo;
-                        words[f][m] |= (uint32_t)(b & 0xFF) << (8 * e);
-                    }
-                }
-#pragma unroll
-            for (int f = 0; f < 4; f++)
-                *reinterpret_cast<u32x4_t*>(&s_rqop[pl * 4 + f][lane][0]) = (u32x4_t){words[f][0], words[f][1], words[f][2], words[f][3]};
-        }
-    }
-    __syncthreads();
-
     // ---- the workgroup's chunk of positions
     uint32_t lo, hi, lane_base;
     query_range(p, a.positions, qi, lo, hi, lane_base);
@@ -192,6 +134,96 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     auto is_valid = [](const GroupGeom& gg, uint32_t idx) { return idx - gg.vlo < gg.vhi - gg.vlo; };
     const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
     const bool k_role = ((wave ^ blockIdx.x) & 1u) == 0;          // alternate, so that both kinds of wave share each SIMD
+
+    // ---- touch the first group's codes (one 64-byte record per lane) so that they are on their way into the cache
+    //      while the set-up below runs; the value is only consumed (and waited for) after the set-up
+    uint32_t touched = 0;
+    if (any) {
+        const GroupGeom g0 = geom(g_first);
+        const uint8_t* rec0 = (k_role ? a.k_codes : a.v_codes) + (((size_t)lane_base + g0.pb + lane) * p.num_kv_heads + kvh) * kCodeBytes;
+        if (is_valid(g0, lane)) touched = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(rec0));
+    }
+
+    // ---- this lane's share of the rotated queries for the K-side operands, requested together with the values for
+    //      the statistics (one round trip to memory instead of two).  The lanes pcol, pcol ^ 1 serve the two limbs of
+    //      one head; each quantises half of the code bytes 16g .. 16g + 15 (words m = 2 * limb, 2 * limb + 1) and
+    //      they swap the limb the other one needs.
+    const uint32_t h_op = (pcol >> 2) + 4 * ((pcol >> 1) & 1), limb_op = pcol & 1;
+    float4 xq[2][4];
+#pragma unroll
+    for (int mm = 0; mm < 2; mm++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            xq[mm][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (h_op < group) xq[mm][e] = *reinterpret_cast<const float4*>(rq_base + (size_t)h_op * kHeadDim + 4 * (16 * g + 4 * (2 * limb_op + mm) + e));
+        }
+
+    // ---- per head: max |rq| (quantisation scale) and sum(rq) (constant term of the level table)
+    for (uint32_t h = tid >> 5; h < (uint32_t)kMaxGroupHeads; h += blockDim.x >> 5) {
+        const uint32_t sub = tid & 31;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        if (h < group) {
+            const float4 x0 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8);
+            const float4 x1 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8 + 4);
+            v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+        }
+        float m = 0.0f, s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { m = fmaxf(m, fabsf(v[i])); s += v[i]; }
+        m = lh_group_max(m, 32);
+        s = lh_group_sum(s, 32);
+        if (sub == 0) { s_maxabs[h] = m; s_sum[h] = s; }
+    }
+    __syncthreads();
+
+    // ---- K-side A operands.  Row r of the MFMA: head (r / 4) + 4 * ((r / 2) % 2), limb r % 2, so that the lanes of
+    //      row group g end up with heads g and g + 4 on both the K and the V side.  k slot (word m, byte e) of
+    //      row group g is code byte j = 16g + 4m + e, i.e. dim 4j + f for the operand of field f.
+    {
+        const float ma = s_maxabs[h_op];
+        const float inv = (ma > 0.0f && cmax_k > 0.0f) ? kQmax / (ma * cmax_k) : 0.0f;
+        for (uint32_t pl = wave; pl < (uint32_t)nplanes; pl += nwaves) {
+            const float mul = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv;
+            uint32_t wlo[4][2], whi[4][2];   // [field][word mm]: low / high limbs of this lane's half, byte e = code byte 4m + e
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+#pragma unroll
+                for (int mm = 0; mm < 2; mm++) wlo[f][mm] = whi[f][mm] = 0;
+#pragma unroll
+            for (int mm = 0; mm < 2; mm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float xv[4] = {xq[mm][e].x, xq[mm][e].y, xq[mm][e].z, xq[mm][e].w};
+#pragma unroll
+                    for (int f = 0; f < 4; f++) {
+                        float r = __builtin_rintf(xv[f] * mul);
+                        r = fminf(fmaxf(r, -kQmax), kQmax);
+                        const int n = (int)r;
+                        const int lo = (int)(int8_t)(n & 0xFF);
+                        wlo[f][mm] |= (uint32_t)(lo & 0xFF) << (8 * e);
+                        whi[f][mm] |= (uint32_t)(((n - lo) >> 8) & 0xFF) << (8 * e);
+                    }
+                }
+            uint32_t words[4][4];
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+#pragma unroll
+                for (int mm = 0; mm < 2; mm++) {
+                    const uint32_t mine = limb_op ? whi[f][mm] : wlo[f][mm];
+                    const uint32_t give = limb_op ? wlo[f][mm] : whi[f][mm];
+                    const uint32_t got = (uint32_t)__builtin_amdgcn_mov_dpp((int)give, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]: lane ^ 1
+                    words[f][mm] = limb_op ? got : mine;        // words 0, 1 were quantised by the limb-0 lane
+                    words[f][2 + mm] = limb_op ? mine : got;    // words 2, 3 by the limb-1 lane
+                }
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+                *reinterpret_cast<u32x4_t*>(&s_rqop[pl * 4 + f][lane][0]) = (u32x4_t){words[f][0], words[f][1], words[f][2], words[f][3]};
+        }
+    }
+    __syncthreads();
+    asm volatile("" :: "v"(touched));
 
     if (k_role) {
         // =================================================================== K wave
@@ -555,14 +587,19 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
 }
 
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
-    // One workgroup (a K wave and a V wave) per chunk of positions; about `wps` waves per SIMD over the whole launch,
-    // at least 128 positions per chunk.
+    // One workgroup (a K wave and a V wave) per chunk of positions.  Short jobs (the chunks of one workgroup per CU
+    // stay within 128 positions) are latency bound: they get chunks down to one group of 64 and never share a CU.
+    // Everything else gets about `wps` waves per SIMD over the whole launch and at least 128 positions per chunk.
     static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
     static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
     const uint64_t wg_slots = (uint64_t)ctx->cu_count * 2 * wps;
-    uint64_t splits = std::max<uint64_t>(1, wg_slots / pairs);
-    splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
+    uint64_t splits = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)ctx->cu_count / pairs));
+    splits = std::max<uint64_t>(splits, 1);
+    if ((max_span + splits - 1) / splits > 128) {
+        splits = std::max<uint64_t>(1, wg_slots / pairs);
+        splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
+    }
     splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
     const size_t rec = partial_record_floats(p.head_dim);
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
