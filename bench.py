@@ -170,8 +170,8 @@ def make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits):
     return pool, levels, signs
 
 
-def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
-    hd, nq, nkv, bits = 256, 8, 1, 2
+def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64, hd=256):
+    nq, nkv, bits = 8, 1, 2
     pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits)
     g = pkg.synth.rng(5, 1)
     q = g.standard_normal((lanes, nq, hd), dtype=np.float32).astype(np.float16)
@@ -218,6 +218,10 @@ def bench_attention_sweep(pkg, ctx, K, steps, warmup):
         r = bench_attention(pkg, ctx, K, steps, warmup, T=T, lanes=lanes)
         res[f"ctx_{T}"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"],
                            "batched_lanes": lanes, "batched_us_per_launch": r["batched_us_per_launch"], "batched_gbs": r["batched_gbs"]}
+    # the reference model's full-attention layers: head_dim 512 (260 bytes per position)
+    r = bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=32, hd=512)
+    res["ctx_32768_head_dim_512"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"],
+                                     "batched_lanes": 32, "batched_us_per_launch": r["batched_us_per_launch"], "batched_gbs": r["batched_gbs"]}
     # sliding window: every lane is a 512-slot ring; logical position far beyond the ring size
     ring, lanes, pos = 512, 4096, 100000
     pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, ring, hd, nkv, bits)

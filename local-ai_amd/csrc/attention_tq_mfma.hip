@@ -36,8 +36,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
 
-constexpr int kHeadDim = 256;
-constexpr int kCodeBytes = 64;
 constexpr int kGroup = 64;             // positions per loop step: 4 K-side MFMA tiles, one V-side MFMA k-step
 constexpr int kMaxGroupHeads = 8;      // query heads per KV head served by the 16 MFMA rows
 constexpr float kLog2e = 1.4426950408889634f;
@@ -76,12 +74,13 @@ struct GroupGeom {
 // One workgroup = two waves on one chunk of positions: the "K wave" turns K codes into softmax weights (as MFMA row
 // operands in LDS), the "V wave" multiplies them with the V codes.  The K wave runs one group ahead; one workgroup
 // barrier per group hands over a double-buffered operand set plus the rare "reference moved" message.
+template <int NH>   // NH = 64-byte halves of a position's code (head_dim / 256) = number of V waves
 struct AttnShared {
-    uint8_t rqop[12][64][16];      // K-side A operands per (plane, field) and lane
+    uint8_t rqop[12 * NH][64][16]; // K-side A operands per (code half, plane, field) and lane
     float4 norm[kGroup];           // K wave: (norm_k*log2e, mask bias, norm_v, -) per group position
     float4 ww[2][2][64];           // [buffer][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
     float wq[2];                   // [buffer]: fixed-point scale of those weights
-    uint8_t wx[3][2][1024];        // V wave: [plane][row set] A operands (weights as limbs)
+    uint8_t wx[NH][3][2][1024];    // [V wave][plane][row set]: that wave's A operands (weights as limbs)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
     float unit_old[2];             // [buffer]: value of one integer step of the accumulators gathered so far
     uint32_t moved[2];             // [buffer]: the reference moved before this group: fold, then rescale
@@ -90,12 +89,14 @@ struct AttnShared {
 };
 
 // NPL = number of bit planes: 2 when the level table is affine in the code bits, 3 with the bit0*bit1 plane.
-template <int NPL>
-__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared& sh, float alpha, float beta,
+// HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
+template <int NPL, int HD>
+__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256)>& sh, float alpha, float beta,
                                                float gam, float delta) {
     auto& s_rqop = sh.rqop;
     auto& s_maxabs = sh.maxabs;
     auto& s_sum = sh.sum;
+    constexpr int kHeadDim = HD, kCodeBytes = HD / 4, NH = HD / 256;   // NH: 64-byte halves of a code
     constexpr bool has_delta = NPL == 3;
     constexpr int nplanes = NPL;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
@@ -133,14 +134,17 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // weights are masked to zero.
     auto is_valid = [](const GroupGeom& gg, uint32_t idx) { return idx - gg.vlo < gg.vhi - gg.vlo; };
     const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
-    const bool k_role = ((wave ^ blockIdx.x) & 1u) == 0;          // alternate, so that both kinds of wave share each SIMD
+    // Roles rotate with the workgroup index, so that the kinds of wave mix on every SIMD.
+    const uint32_t role = NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) % 3u;   // 0: K wave; 1, 2: V wave of code half role - 1
+    const bool k_role = role == 0;
+    const uint32_t vhalf = k_role ? 0u : role - 1u;
 
     // ---- touch the first group's codes (one 64-byte record per lane) so that they are on their way into the cache
     //      while the set-up below runs; the value is only consumed (and waited for) after the set-up
     uint32_t touched = 0;
     if (any) {
         const GroupGeom g0 = geom(g_first);
-        const uint8_t* rec0 = (k_role ? a.k_codes : a.v_codes) + (((size_t)lane_base + g0.pb + lane) * p.num_kv_heads + kvh) * kCodeBytes;
+        const uint8_t* rec0 = (k_role ? a.k_codes : a.v_codes) + (((size_t)lane_base + g0.pb + lane) * p.num_kv_heads + kvh) * kCodeBytes + 64 * vhalf;
         if (is_valid(g0, lane)) touched = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(rec0));
     }
 
@@ -150,28 +154,37 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     //      they swap the limb the other one needs.
     const uint32_t h_op = (pcol >> 2) + 4 * ((pcol >> 1) & 1), limb_op = pcol & 1;
     float4 xq[2][4];
+    auto load_xq = [&](uint32_t half) {   // code bytes 64 * half + 16g + 4 * (2 * limb + mm) + e
 #pragma unroll
-    for (int mm = 0; mm < 2; mm++)
+        for (int mm = 0; mm < 2; mm++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            xq[mm][e] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (h_op < group) xq[mm][e] = *reinterpret_cast<const float4*>(rq_base + (size_t)h_op * kHeadDim + 4 * (16 * g + 4 * (2 * limb_op + mm) + e));
-        }
+            for (int e = 0; e < 4; e++) {
+                xq[mm][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (h_op < group)
+                    xq[mm][e] = *reinterpret_cast<const float4*>(rq_base + (size_t)h_op * kHeadDim + 256 * half + 4 * (16 * g + 4 * (2 * limb_op + mm) + e));
+            }
+    };
+    // Operand units (code half, plane) are dealt to the waves round robin; the first unit's queries are requested here.
+    uint32_t xq_half = wave / (uint32_t)nplanes;
+    if (wave < (uint32_t)(nplanes * NH)) load_xq(xq_half);
 
     // ---- per head: max |rq| (quantisation scale) and sum(rq) (constant term of the level table)
     for (uint32_t h = tid >> 5; h < (uint32_t)kMaxGroupHeads; h += blockDim.x >> 5) {
         const uint32_t sub = tid & 31;
-        float v[8];
+        constexpr int NV = HD / 32;   // values per thread: 32 threads per head
+        float v[NV];
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        for (int i = 0; i < NV; i++) v[i] = 0.0f;
         if (h < group) {
-            const float4 x0 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8);
-            const float4 x1 = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * 8 + 4);
-            v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+#pragma unroll
+            for (int i = 0; i < NV / 4; i++) {
+                const float4 x = *reinterpret_cast<const float4*>(rq_base + (size_t)h * kHeadDim + sub * NV + 4 * i);
+                v[4 * i] = x.x; v[4 * i + 1] = x.y; v[4 * i + 2] = x.z; v[4 * i + 3] = x.w;
+            }
         }
         float m = 0.0f, s = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) { m = fmaxf(m, fabsf(v[i])); s += v[i]; }
+        for (int i = 0; i < NV; i++) { m = fmaxf(m, fabsf(v[i])); s += v[i]; }
         m = lh_group_max(m, 32);
         s = lh_group_sum(s, 32);
         if (sub == 0) { s_maxabs[h] = m; s_sum[h] = s; }
@@ -180,11 +193,13 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 
     // ---- K-side A operands.  Row r of the MFMA: head (r / 4) + 4 * ((r / 2) % 2), limb r % 2, so that the lanes of
     //      row group g end up with heads g and g + 4 on both the K and the V side.  k slot (word m, byte e) of
-    //      row group g is code byte j = 16g + 4m + e, i.e. dim 4j + f for the operand of field f.
+    //      row group g is code byte j = 64 * half + 16g + 4m + e, i.e. dim 4j + f for the operand of field f.
     {
         const float ma = s_maxabs[h_op];
         const float inv = (ma > 0.0f && cmax_k > 0.0f) ? kQmax / (ma * cmax_k) : 0.0f;
-        for (uint32_t pl = wave; pl < (uint32_t)nplanes; pl += nwaves) {
+        for (uint32_t unit = wave; unit < (uint32_t)(nplanes * NH); unit += nwaves) {
+            const uint32_t half = unit / (uint32_t)nplanes, pl = unit - half * (uint32_t)nplanes;
+            if (half != xq_half) { load_xq(half); xq_half = half; }
             const float mul = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv;
             uint32_t wlo[4][2], whi[4][2];   // [field][word mm]: low / high limbs of this lane's half, byte e = code byte 4m + e
 #pragma unroll
@@ -219,7 +234,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 }
 #pragma unroll
             for (int f = 0; f < 4; f++)
-                *reinterpret_cast<u32x4_t*>(&s_rqop[pl * 4 + f][lane][0]) = (u32x4_t){words[f][0], words[f][1], words[f][2], words[f][3]};
+                *reinterpret_cast<u32x4_t*>(&s_rqop[(half * nplanes + pl) * 4 + f][lane][0]) = (u32x4_t){words[f][0], words[f][1], words[f][2], words[f][3]};
         }
     }
     __syncthreads();
@@ -243,23 +258,27 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 
         if (any) {
             GroupGeom gg = geom(g_first);
-            u32x4_t kw[4], kwn[4];   // K codes of the current group and of the next one (a full step of prefetch distance)
+            u32x4_t kw[NH][4], kwn[NH][4];   // K codes of the current group and of the next one (a full step of prefetch distance)
             float nk, nv, nkn = 0.0f, nvn = 0.0f;
             const uint32_t klane = pcol * stride + 16 * g, nlane = lane * nstride;
-            auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw_)[4], float& nk_, float& nv_) {
+            auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw_)[NH][4], float& nk_, float& nv_) {
                 gptr_t kb = krec0 + (size_t)G_.pb * stride;
                 gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
                 if (G_.full) {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) kw_[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                    for (int hf = 0; hf < NH; hf++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) kw_[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
                     nk_ = ld_norm(knb + nlane);
                     nv_ = ld_norm(vnb + nlane);
                 } else {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        kw_[q] = (u32x4_t){0u, 0u, 0u, 0u};
-                        if (is_valid(G_, 16 * q + pcol)) kw_[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
-                    }
+                    for (int hf = 0; hf < NH; hf++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            kw_[hf][q] = (u32x4_t){0u, 0u, 0u, 0u};
+                            if (is_valid(G_, 16 * q + pcol)) kw_[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
+                        }
                     nk_ = nv_ = 0.0f;
                     if (is_valid(G_, lane)) { nk_ = ld_norm(knb + nlane); nv_ = ld_norm(vnb + nlane); }
                 }
@@ -284,38 +303,42 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 float lg[4][2], vn[4];
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const uint32_t w[4] = {kw[q].x, kw[q].y, kw[q].z, kw[q].w};
-                    v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
-#pragma unroll
-                    for (int m = 0; m < 4; m++) {
-                        const uint32_t u = w[m] >> 4;
-                        b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
-                        b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
-                        b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
-                        b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
-                    }
-                    const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[0][lane][0]);   // operand pf at rqo[64 * pf]
                     v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
-                    if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
-                        v4i d0, d1, d2, d3;
+#pragma unroll
+                    for (int hf = 0; hf < NH; hf++) {
+                        const uint32_t w[4] = {kw[hf][q].x, kw[hf][q].y, kw[hf][q].z, kw[hf][q].w};
+                        v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
 #pragma unroll
                         for (int m = 0; m < 4; m++) {
-                            const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
-                            d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
-                            d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
+                            const uint32_t u = w[m] >> 4;
+                            b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
+                            b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
+                            b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
+                            b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
                         }
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
+                        // operand (plane pl, field f) of this code half at rqo[64 * (4 * pl + f)]
+                        const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[hf * nplanes * 4][lane][0]);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
+                        if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
+                            v4i d0, d1, d2, d3;
+#pragma unroll
+                            for (int m = 0; m < 4; m++) {
+                                const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
+                                d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
+                                d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
+                            }
+                            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
+                            acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
+                            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
+                            acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
+                        }
                     }
                     const float4 nrm = sh.norm[16 * q + pcol];
                     vn[q] = nrm.z;
@@ -379,7 +402,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 __syncthreads();   // hand-over of buffer `buf`; also: the V wave is done with the buffer written next
                 gg = gnext;
 #pragma unroll
-                for (int q = 0; q < 4; q++) kw[q] = kwn[q];
+                for (int hf = 0; hf < NH; hf++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) kw[hf][q] = kwn[hf][q];
                 nk = nkn; nv = nvn;
             }
         }
@@ -393,7 +418,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         __syncthreads();
     } else {
         // =================================================================== V wave
-        gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+        gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * vhalf;
         v4i acc[4][4][2];      // [code byte e][field f][row set]: integer accumulators, rows = 4 limbs of head g + 4 * set
         float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
 #pragma unroll
@@ -482,7 +507,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                                 lw[q] = ((uint32_t)qv + 0x00808080u) ^ 0x00808080u;    // bytes = signed limbs, least significant first
                             }
                             transpose4x4(lw, tr);
-                            uint8_t* dst = &sh.wx[pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
+                            uint8_t* dst = &sh.wx[vhalf][pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
 #pragma unroll
                             for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t*>(dst + 16 * i) = tr[i];
                         }
@@ -495,8 +520,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 if (more) load_v(geom(G + 1));   // the V registers are free
 #pragma unroll
                 for (int pl = 0; pl < nplanes; pl++) {
-                    const v4i wop0 = *reinterpret_cast<const v4i*>(&sh.wx[pl][0][lane * 16]);
-                    const v4i wop1 = *reinterpret_cast<const v4i*>(&sh.wx[pl][1][lane * 16]);
+                    const v4i wop0 = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][0][lane * 16]);
+                    const v4i wop1 = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][1][lane * 16]);
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         uint32_t yp[4];   // the plane's bit of every field at the even bit positions
@@ -539,7 +564,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             const uint32_t qh = kvh * group + h;
             const float bias = alpha * w_tot;
             if (nsplit == 1) {
-                float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 16 * pcol;
+                float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 16 * pcol;
                 const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
@@ -547,27 +572,27 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                                                                           (outv[e][2][hs] + bias) * inv, (outv[e][3][hs] + bias) * inv);
             } else {
                 float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * nsplit + split) * partial_record_floats(kHeadDim);
-                if (pcol == 0) { rec[0] = sh.fin_r[h] * kLn2; rec[1] = l_tot; }
+                if (pcol == 0 && vhalf == 0) { rec[0] = sh.fin_r[h] * kLn2; rec[1] = l_tot; }
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    *reinterpret_cast<float4*>(rec + 4 + 16 * pcol + 4 * e) =
+                    *reinterpret_cast<float4*>(rec + 4 + 256 * vhalf + 16 * pcol + 4 * e) =
                         make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
             }
         }
     }
 }
 
-template <int OCC>
-__global__ __launch_bounds__(128, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {
-    __shared__ __align__(16) AttnShared sh;
+template <int OCC, int HD>
+__global__ __launch_bounds__(64 + HD / 4, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {   // 128 / 192 threads
+    __shared__ __align__(16) AttnShared<HD / 256> sh;
     // L[c] = alpha + beta*bit0 + gam*bit1 + delta*bit0*bit1.  A delta that is only float noise of a symmetric table
     // (|delta| <= 1e-5 max|L|) is spread by the least-squares affine fit bit0*bit1 ~ -1/4 + bit0/2 + bit1/2, which
     // leaves +-delta/4 per code; anything larger gets its own bit plane.
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
-    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
-    else attention_body<2>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
+    else attention_body<2, HD>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
@@ -577,7 +602,7 @@ namespace lh_attn {
 bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
     static const bool off = [] { const char* e = getenv("LOCAL_HIP_ATTN_KERNEL"); return e && e[0] == 'v'; }();   // "valu"
     if (off) return false;
-    if (p.bits != 2 || p.head_dim != (uint32_t)kHeadDim) return false;
+    if (p.bits != 2 || (p.head_dim != 256 && p.head_dim != 512)) return false;
     if (p.num_q_heads / p.num_kv_heads > (uint32_t)kMaxGroupHeads) return false;
     if (p.ring_capacity % kGroup != 0) return false;                      // aligned groups must not wrap inside
     if (((uintptr_t)a.k_codes | (uintptr_t)a.v_codes) & 3) return false;
@@ -587,13 +612,14 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
 }
 
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
-    // One workgroup (a K wave and a V wave) per chunk of positions.  Short jobs (the chunks of one workgroup per CU
+    // One workgroup (a K wave and one V wave per 256 dims) per chunk of positions.  Short jobs (the chunks of one workgroup per CU
     // stay within 128 positions) are latency bound: they get chunks down to one group of 64 and never share a CU.
     // Everything else gets about `wps` waves per SIMD over the whole launch and at least 128 positions per chunk.
     static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
     static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
-    const uint64_t wg_slots = (uint64_t)ctx->cu_count * 2 * wps;
+    const uint32_t wg_waves = p.head_dim == 512 ? 3 : 2;
+    const uint64_t wg_slots = (uint64_t)ctx->cu_count * std::max(1u, 4u * (uint32_t)wps / wg_waves);
     uint64_t splits = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)ctx->cu_count / pairs));
     splits = std::max<uint64_t>(splits, 1);
     if ((max_span + splits - 1) / splits > 128) {
@@ -605,8 +631,13 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
-    if (occ == 1) hipLaunchKernelGGL(attention_tq_mfma_kernel<1>, grid, dim3(128), 0, ctx->stream, a, p);
-    else hipLaunchKernelGGL(attention_tq_mfma_kernel<2>, grid, dim3(128), 0, ctx->stream, a, p);
+    if (p.head_dim == 512) {
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512>), grid, dim3(192), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512>), grid, dim3(192), 0, ctx->stream, a, p);
+    } else {
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256>), grid, dim3(128), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256>), grid, dim3(128), 0, ctx->stream, a, p);
+    }
     return lh_check_launch(op);
 }
 

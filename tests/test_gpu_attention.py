@@ -53,6 +53,12 @@ def upload(pkg, ctx, *arrays):
     (256, 8, 2, 1300, 2, 300, 1.0),    # two KV heads, window not aligned to the block size
     (256, 6, 3, 513, 2, 0, 0.5),
     (256, 8, 1, 20000, 2, 0, 0.25),    # long context, soft attention (many positions carry weight)
+    (512, 8, 1, 1, 2, 0, 1.0),         # head_dim 512 (full-attention layers): two V waves per workgroup
+    (512, 8, 1, 257, 2, 0, 0.3),
+    (512, 8, 1, 2500, 2, 0, 0.3),
+    (512, 8, 2, 1300, 2, 300, 0.3),
+    (512, 4, 1, 700, 2, 512, 0.3),
+    (512, 8, 1, 20000, 2, 0, 0.15),
 ])
 def test_decode_attention_matches_oracle(pkg, gpu, oracle, hd, nq, nkv, T, bits, window, qscale):
     print(f"case hd={hd} nq={nq} nkv={nkv} T={T} bits={bits} window={window}", flush=True)
@@ -151,7 +157,7 @@ def test_empty_range_gives_zeros(pkg, gpu, oracle):
 
 @pytest.mark.parametrize("tiled", [False, True])
 @pytest.mark.parametrize("hd,nq,nkv,bits,start,rows,window", [(256, 8, 1, 2, 0, 37, 0), (256, 8, 1, 2, 100, 20, 64),
-                                                              (128, 4, 2, 4, 5, 9, 0)])
+                                                              (128, 4, 2, 4, 5, 9, 0), (512, 8, 1, 2, 70, 11, 0)])
 def test_prefill_matches_per_row_decode(pkg, gpu, oracle, tiled, hd, nq, nkv, bits, start, rows, window):
     """kernels.rs:10126, 10295: every prefill row equals the decode kernel at that position."""
     print(f"case tiled={tiled} hd={hd} rows={rows} start={start}", flush=True)
@@ -171,10 +177,11 @@ def test_prefill_matches_per_row_decode(pkg, gpu, oracle, tiled, hd, nq, nkv, bi
         check(got[r], ref, f"row {r}")
 
 
-def test_batched_matches_independent_sequences(pkg, gpu, oracle):
+@pytest.mark.parametrize("hd", [256, 512])
+def test_batched_matches_independent_sequences(pkg, gpu, oracle, hd):
     """kernels.rs:10457: lanes at different positions in one dispatch == separate single-sequence calls."""
     ctx, K = gpu
-    hd, nq, nkv, bits, lanes, cap = 256, 8, 1, 2, 4, 600
+    nq, nkv, bits, lanes, cap = 8, 1, 2, 4, 600
     cb = oracle.tq_code_bytes(hd, bits)
     positions = np.array([599, 0, 123, 300], np.uint32)
     pool_kc = np.zeros((lanes * cap, nkv, cb), np.uint8); pool_vc = np.zeros_like(pool_kc)
