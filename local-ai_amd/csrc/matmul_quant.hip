@@ -13,6 +13,7 @@
 //    d*(q-1) is exact in f16 -- and staged in LDS next to the activation tile
 //    (converted to f16), then v_mfma_f32_16x16x32_f16 with fp32 accumulate.
 #include "common.hpp"
+#include <cstdlib>
 
 namespace {
 
@@ -105,54 +106,71 @@ __device__ __forceinline__ uint32_t h2_sub_mul(uint32_t x, uint32_t bias, uint32
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// Raw global data of one staging run (32 consecutive k of one row), kept in registers across two k steps so that the
+// Raw global data of one weight staging run (32 consecutive k of one row), kept in registers across two k steps so that the
 // loads have two steps of MFMA work to arrive; converted to f16 words just before they go to LDS.
-template <int ADT> struct RawA { uint4 v[ADT == LH_F32 ? 8 : 4]; };
-template <int FMT> struct RawB { uint4 q[FMT == kF16W ? 4 : 2]; uint32_t d; };
+template <int FMT> struct RawB { uint4 q[FMT == kF16W ? 4 : (FMT == kQ4 ? 1 : 2)]; uint32_t d; };
 
+// Activations are staged in chunks of 8 consecutive k: the 16 lanes that share a row read 256 contiguous bytes (f16 / bf16).
+template <int ADT> struct RawA8 { uint4 v[ADT == LH_F32 ? 2 : 1]; };
+
+// Branch-free (the compiler can then count the loads in flight instead of waiting for all of them): rows past the end
+// re-read the last row (their products are never stored), chunks past the end of a row re-read its last chunk and are
+// zeroed by convert_a8.
 template <int ADT>
-__device__ __forceinline__ void load_raw_a(RawA<ADT>& r, const void* A, uint32_t row, uint32_t M, uint32_t K, uint32_t k0) {
-    constexpr int NV = ADT == LH_F32 ? 8 : 4;
-    if (row >= M || k0 >= K) {   // K is a multiple of 32: a run that starts inside a row ends inside it
-#pragma unroll
-        for (int i = 0; i < NV; i++) r.v[i] = make_uint4(0u, 0u, 0u, 0u);
-        return;
-    }
-    const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(A) + ((size_t)row * K + k0) * (ADT == LH_F32 ? 4 : 2));
+__device__ __forceinline__ void load_raw_a8(RawA8<ADT>& r, const void* A, uint32_t row, uint32_t M, uint32_t K, uint32_t k0) {
+    constexpr int NV = ADT == LH_F32 ? 2 : 1;
+    const uint32_t rc = row < M ? row : M - 1, kc = k0 < K ? k0 : K - 8;
+    const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(A) + ((size_t)rc * K + kc) * (ADT == LH_F32 ? 4 : 2));
 #pragma unroll
     for (int i = 0; i < NV; i++) r.v[i] = p[i];
 }
 
 template <int ADT>
-__device__ __forceinline__ void convert_a(uint32_t (&f)[16], const RawA<ADT>& r) {
+__device__ __forceinline__ uint4 convert_a8(const RawA8<ADT>& r) {
     if constexpr (ADT == LH_F32) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            f[2 * i] = pack_h2(__builtin_bit_cast(float, r.v[i].x), __builtin_bit_cast(float, r.v[i].y));
-            f[2 * i + 1] = pack_h2(__builtin_bit_cast(float, r.v[i].z), __builtin_bit_cast(float, r.v[i].w));
-        }
+        return make_uint4(pack_h2(__builtin_bit_cast(float, r.v[0].x), __builtin_bit_cast(float, r.v[0].y)),
+                          pack_h2(__builtin_bit_cast(float, r.v[0].z), __builtin_bit_cast(float, r.v[0].w)),
+                          pack_h2(__builtin_bit_cast(float, r.v[1].x), __builtin_bit_cast(float, r.v[1].y)),
+                          pack_h2(__builtin_bit_cast(float, r.v[1].z), __builtin_bit_cast(float, r.v[1].w)));
+    } else if constexpr (ADT == LH_F16) {
+        return r.v[0];
     } else {
+        const uint32_t w[4] = {r.v[0].x, r.v[0].y, r.v[0].z, r.v[0].w};
+        uint32_t f[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t w[4] = {r.v[i].x, r.v[i].y, r.v[i].z, r.v[i].w};
+        for (int j = 0; j < 4; j++) f[j] = pack_h2(lh_bf2f((uint16_t)(w[j] & 0xFFFF)), lh_bf2f((uint16_t)(w[j] >> 16)));   // bf16 -> f16
+        return make_uint4(f[0], f[1], f[2], f[3]);
+    }
+}
+
+// TQ2_0 weights of one k step (128 k = half a block = 32 code bytes of a row): a thread takes 16 of the bytes, i.e.
+// elements 32f + 16 * part + j (field f = 0..3, j = 0..15) of the half block.
+struct RawBT { uint4 q; uint32_t d; };
+__device__ __forceinline__ void load_raw_bt(RawBT& r, const uint8_t* W, uint32_t row, uint32_t K, uint32_t k0, uint32_t part) {
+    if (k0 >= K) k0 = K - 128;   // a step past the end re-reads the last one; convert_bt zeroes it
+    const uint8_t* bp = W + ((size_t)row * (K >> 8) + (k0 >> 8)) * 66;
+    r.d = *reinterpret_cast<const uint16_t*>(bp + 64);
+    __builtin_memcpy(&r.q, __builtin_assume_aligned(bp + ((k0 >> 7) & 1) * 32 + 16 * part, 2), 16);
+}
+// f16 values of field f: 16 consecutive k as 8 words
+__device__ __forceinline__ void convert_bt(uint32_t (&w)[8], const RawBT& r, int f, bool valid) {
+    const uint32_t d = valid ? r.d : 0u;
+    const uint32_t d2 = (d & 0xFFFFu) | (d << 16);
+    const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if constexpr (ADT == LH_F16) f[4 * i + j] = w[j];
-                else f[4 * i + j] = pack_h2(lh_bf2f((uint16_t)(w[j] & 0xFFFF)), lh_bf2f((uint16_t)(w[j] >> 16)));   // bf16 -> f16
-            }
-        }
+    for (int i = 0; i < 4; i++) {
+        const uint32_t c = (q[i] >> (2 * f)) & 0x03030303u;
+        w[2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04010400u), 0x64016401u, d2);            // 1024 + c - 1025
+        w[2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04030402u), 0x64016401u, d2);
     }
 }
 
 // Elements k0 .. k0 + 32 of weight row `row` (k0 a multiple of 32).
 template <int FMT>
 __device__ __forceinline__ void load_raw_b(RawB<FMT>& r, const uint8_t* W, uint32_t row, uint32_t K, uint32_t k0) {
-    if (k0 >= K) {   // past the end of the row in the last k step: scale 0 (and zero words for f16 weights)
-        r.d = 0;
-#pragma unroll
-        for (int i = 0; i < (FMT == kF16W ? 4 : 2); i++) r.q[i] = make_uint4(0u, 0u, 0u, 0u);
-        return;
-    }
+    // Past the end of the row in the last k step the last run is read again; convert_b zeroes it.  Nothing here may
+    // compute on a loaded value: that would wait for the load right where it is issued.
+    if (k0 >= K) k0 = K - 32;
     if constexpr (FMT == kF16W) {
         const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(W) + (size_t)row * K + k0);
 #pragma unroll
@@ -162,23 +180,26 @@ __device__ __forceinline__ void load_raw_b(RawB<FMT>& r, const uint8_t* W, uint3
         const uint8_t* bp = W + ((size_t)row * (K >> 5) + (k0 >> 5)) * 18;
         r.d = *reinterpret_cast<const uint16_t*>(bp);
         __builtin_memcpy(&r.q[0], __builtin_assume_aligned(bp + 2, 2), 16);
-        r.q[1] = make_uint4(0u, 0u, 0u, 0u);
     } else {
         const uint32_t blk = k0 >> 8, s = (k0 >> 5) & 7;               // 32-element slice s of the block: bytes (s/4)*32.., field s%4
         const uint8_t* bp = W + ((size_t)row * (K >> 8) + blk) * 66;
-        r.d = *reinterpret_cast<const uint16_t*>(bp + 64) | (((s & 3) * 2) << 16);   // scale bits and the field's shift
+        r.d = *reinterpret_cast<const uint16_t*>(bp + 64);
         __builtin_memcpy(&r.q[0], __builtin_assume_aligned(bp + (s >> 2) * 32, 2), 16);
         __builtin_memcpy(&r.q[1], __builtin_assume_aligned(bp + (s >> 2) * 32 + 16, 2), 16);
     }
 }
 
+// k0 = first element of the run; `valid` = false past the end of the row (the run becomes zeros).
 template <int FMT>
-__device__ __forceinline__ void convert_b(uint32_t (&f)[16], const RawB<FMT>& r) {
+__device__ __forceinline__ void convert_b(uint32_t (&f)[16], const RawB<FMT>& r, uint32_t k0, bool valid) {
     if constexpr (FMT == kF16W) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) { f[4 * i] = r.q[i].x; f[4 * i + 1] = r.q[i].y; f[4 * i + 2] = r.q[i].z; f[4 * i + 3] = r.q[i].w; }
+        for (int i = 0; i < 4; i++) {
+            f[4 * i] = valid ? r.q[i].x : 0u; f[4 * i + 1] = valid ? r.q[i].y : 0u; f[4 * i + 2] = valid ? r.q[i].z : 0u; f[4 * i + 3] = valid ? r.q[i].w : 0u;
+        }
     } else if constexpr (FMT == kQ4) {
-        const uint32_t d2 = (r.d & 0xFFFFu) | (r.d << 16);
+        const uint32_t d = valid ? r.d : 0u;
+        const uint32_t d2 = (d & 0xFFFFu) | (d << 16);
         const uint32_t q[4] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w};
         // byte j: low nibble = element j, high nibble = element 16 + j
 #pragma unroll
@@ -190,7 +211,8 @@ __device__ __forceinline__ void convert_b(uint32_t (&f)[16], const RawB<FMT>& r)
             f[8 + 2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u), 0x64086408u, d2);
         }
     } else {
-        const uint32_t d2 = (r.d & 0xFFFFu) | (r.d << 16), sh = r.d >> 16;
+        const uint32_t d = valid ? r.d : 0u;
+        const uint32_t d2 = (d & 0xFFFFu) | (d << 16), sh = ((k0 >> 5) & 3) * 2;
         const uint32_t q[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -211,15 +233,13 @@ template <int FMT, int ADT, int CDT, int BM>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
                                                          uint32_t M, uint32_t K, uint32_t N) {
     constexpr int TI = BM / 32;                              // 16-row MFMA tiles per wave along M (2 x 2 waves)
-    constexpr int AR = BM / 64;                              // 32-element activation runs staged per thread
+    constexpr int NCH = BM / 16;                             // 8-element activation chunks staged per thread
     __shared__ __align__(16) _Float16 As[BM * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const uint32_t a_ld_row = BM == 128 ? tid >> 1 : tid >> 2, a_ld_k = BM == 128 ? (tid & 1) * 64 : (tid & 3) * 32;
     const uint32_t b_ld_row = tid >> 1, b_ld_k = (tid & 1) * 64;
-    const uint32_t a_row = m0 + a_ld_row;
     const uint32_t b_row = n0 + b_ld_row < N ? n0 + b_ld_row : N - 1;   // past-the-end rows re-read the last (never stored)
 
     f32x4 acc[TI][4];
@@ -228,20 +248,46 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    RawA<ADT> ra[2][AR];   // [k step parity][run]
-    RawB<FMT> rb[2][2];
+    RawA8<ADT> ra[2][NCH];   // [k step parity][chunk]: chunk c = tid + 256 i is row c / 16, k offset 8 * (c % 16)
+    RawB<FMT> rb[2][FMT == kTQ2 ? 1 : 2];
+    RawBT rbt[2];
     auto load_step = [&](int set, uint32_t kt) {
 #pragma unroll
-        for (int i = 0; i < AR; i++) load_raw_a<ADT>(ra[set][i], A, a_row, M, K, kt * BK + a_ld_k + 32 * i);
+        for (int i = 0; i < NCH; i++) {
+            const uint32_t c = tid + 256 * i;
+            load_raw_a8<ADT>(ra[set][i], A, m0 + (c >> 4), M, K, kt * BK + 8 * (c & 15));
+        }
+        if constexpr (FMT == kTQ2) {
+            load_raw_bt(rbt[set], W, b_row, K, kt * BK, tid & 1);
+        } else {
 #pragma unroll
-        for (int i = 0; i < 2; i++) load_raw_b<FMT>(rb[set][i], W, b_row, K, kt * BK + b_ld_k + 32 * i);
+            for (int i = 0; i < 2; i++) load_raw_b<FMT>(rb[set][i], W, b_row, K, kt * BK + b_ld_k + 32 * i);
+        }
     };
-    auto stage_step = [&](int set) {
-        uint32_t f[16];
+    auto stage_step = [&](int set, uint32_t kt) {
 #pragma unroll
-        for (int i = 0; i < AR; i++) { convert_a<ADT>(f, ra[set][i]); store_words<16>(&As[a_ld_row * LDK + a_ld_k + 32 * i], f); }
+        for (int i = 0; i < NCH; i++) {
+            const uint32_t c = tid + 256 * i;
+            uint4 v = convert_a8<ADT>(ra[set][i]);
+            if (kt * BK + BK > K && kt * BK + 8 * (c & 15) >= K) v = make_uint4(0u, 0u, 0u, 0u);   // only in a partial last k step
+            *reinterpret_cast<uint4*>(&As[(c >> 4) * LDK + 8 * (c & 15)]) = v;
+        }
+        if constexpr (FMT == kTQ2) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) { convert_b<FMT>(f, rb[set][i]); store_words<16>(&Bs[b_ld_row * LDK + b_ld_k + 32 * i], f); }
+            for (int f = 0; f < 4; f++) {
+                uint32_t w[8];
+                convert_bt(w, rbt[set], f, kt * BK < K);
+                store_words<8>(&Bs[b_ld_row * LDK + 32 * f + 16 * (tid & 1)], w);
+            }
+        } else {
+            uint32_t f[16];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const uint32_t k0 = kt * BK + b_ld_k + 32 * i;
+                convert_b<FMT>(f, rb[set][i], k0, k0 < K);
+                store_words<16>(&Bs[b_ld_row * LDK + b_ld_k + 32 * i], f);
+            }
+        }
     };
     auto mfma_step = [&]() {
 #pragma unroll
@@ -259,22 +305,23 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
                 for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
     };
+    // Two k steps per trip (the register sets alternate without copies).  Every trip issues the same loads in the same
+    // order, also past the end of K (those re-read the last step and are staged as zeros): a fixed number of loads in
+    // flight lets the waits before staging leave the newer set outstanding.
     const uint32_t nk = (K + BK - 1) / BK;
     load_step(0, 0);
-    if (nk > 1) load_step(1, 1);
-    for (uint32_t kt = 0; kt < nk; kt += 2) {   // two k steps per trip: the register sets alternate without copies
-        stage_step(0);
+    load_step(1, 1);
+    for (uint32_t kt = 0; kt < nk; kt += 2) {
+        stage_step(0, kt);
         __syncthreads();
-        if (kt + 2 < nk) load_step(0, kt + 2);
+        load_step(0, kt + 2);
         mfma_step();
         __syncthreads();
-        if (kt + 1 < nk) {
-            stage_step(1);
-            __syncthreads();
-            if (kt + 3 < nk) load_step(1, kt + 3);
-            mfma_step();
-            __syncthreads();
-        }
+        stage_step(1, kt + 1);
+        __syncthreads();
+        load_step(1, kt + 3);
+        mfma_step();
+        __syncthreads();
     }
     // D tile: lane holds column (lane & 15), rows 4*(lane >> 4) .. +4
 #pragma unroll
@@ -291,13 +338,224 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
         }
 }
 
+// ---- 128 x 128 tiles for large M: f16 activations (converted once by a pre-pass when they arrive as bf16 / f32),
+//      double-buffered LDS (one barrier per k step), four staging waves next to four multiplying waves, global data two
+//      steps ahead in registers, and load addresses formed as uniform base + constant lane offset so that a staging
+//      step spends its vector ALU time on the dequantisation.  The LDS traffic per step (128 KB of fragment reads, 64 KB
+//      of staging writes against 1024 MFMA cycles per SIMD) is what bounds this tile shape.
+template <int ADT>
+__global__ __launch_bounds__(256) void convert_to_f16_kernel(const void* __restrict__ src, uint16_t* __restrict__ dst, size_t n8) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;   // 8 elements each
+    if (i >= n8) return;
+    RawA8<ADT> r;
+    const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint8_t*>(src) + i * 8 * (ADT == LH_F32 ? 4 : 2));
+#pragma unroll
+    for (int j = 0; j < (ADT == LH_F32 ? 2 : 1); j++) r.v[j] = p[j];
+    reinterpret_cast<uint4*>(dst)[i] = convert_a8<ADT>(r);
+}
+
+// Global loads whose completion the kernel waits for itself: the two register sets in flight need "wait until only
+// the newer set is outstanding", which the compiler's own wait insertion turns into a wait for everything.  The value
+// of a destination is undefined until wait_loads<N>() has run and the destination has passed through settle().
+typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void async_load16(u32x4v& dst, const uint8_t* uniform_base, uint32_t lane_offset) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(lane_offset), "s"(uniform_base) : "memory");
+}
+__device__ __forceinline__ void async_load2(uint32_t& dst, const uint8_t* uniform_base, uint32_t lane_offset) {
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(dst) : "v"(lane_offset), "s"(uniform_base) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+__device__ __forceinline__ void settle(u32x4v& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(uint32_t& v) { asm volatile("" : "+v"(v)); }
+
+template <int FMT, int CDT>
+__global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
+                                                            uint32_t M, uint32_t K, uint32_t N) {
+    static_assert(FMT == kQ4 || FMT == kTQ2, "quantised weights only");
+    constexpr int BM = 128, NCH = 8;
+    constexpr int NB = FMT == kQ4 ? 2 : 1;                        // weight pieces per staging thread and step
+    constexpr int kLoadsPerStep = NCH + 2 * NB;
+    __shared__ __align__(16) _Float16 As[2][BM * LDK];
+    __shared__ __align__(16) _Float16 Bs[2][BN * LDK];
+    // Waves 0-3 multiply (2 x 2 waves, 64 x 64 outputs each), waves 4-7 stage: every SIMD holds one of each kind, so the
+    // staging waves' memory and LDS waits are filled by the other wave's MFMAs.  One barrier per k step hands over a buffer.
+    const bool producer = threadIdx.x >= 256;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const uint32_t nk = K / BK;                                   // K is a multiple of 128 here
+
+    if (producer) {
+        const uint32_t row_bytes = FMT == kQ4 ? (K >> 5) * 18 : (K >> 8) * 66;
+        // lane-constant byte offsets from the tile bases; rows past the end re-read the last row (their products are not stored)
+        uint32_t a_off[NCH], a_lds[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const uint32_t c = tid + 256 * i, row = c >> 4, kc = c & 15;
+            const uint32_t rc = m0 + row < M ? row : M - 1 - m0;
+            a_off[i] = (rc * K + 8 * kc) * 2;
+            a_lds[i] = row * LDK + 8 * kc;
+        }
+        const uint32_t b_ld_row = tid >> 1, part = tid & 1;
+        const uint32_t b_rc = n0 + b_ld_row < N ? b_ld_row : N - 1 - n0;
+        // Q4_0: 4 blocks of 18 bytes per step and row, this thread takes blocks 2 * part, 2 * part + 1.
+        // TQ2_0: one 66-byte block per two steps and row, this thread takes 16 of the step's 32 code bytes.
+        const uint32_t b_off = b_rc * row_bytes + (FMT == kQ4 ? part * 36 : part * 16);
+        const uint8_t* a_tile = reinterpret_cast<const uint8_t*>(A) + (size_t)m0 * K * 2;
+        const uint8_t* w_tile = W + (size_t)n0 * row_bytes;
+
+        u32x4v ra[2][NCH], rq[2][NB];
+        uint32_t rd[2][NB];
+        auto load_step = [&](int set, uint32_t kt) {
+            if (kt >= nk) kt = nk - 1;                            // over-issued steps re-read the last one (staged into a buffer that is not read again)
+            const uint8_t* ab = a_tile + (size_t)kt * (BK * 2);
+#pragma unroll
+            for (int i = 0; i < NCH; i++) async_load16(ra[set][i], ab, a_off[i]);
+            if constexpr (FMT == kQ4) {
+                const uint8_t* wb = w_tile + (size_t)kt * 72;
+#pragma unroll
+                for (int i = 0; i < NB; i++) {
+                    async_load2(rd[set][i], wb, b_off + 18 * i);
+                    async_load16(rq[set][i], wb, b_off + 18 * i + 2);
+                }
+            } else {
+                const uint8_t* wb = w_tile + (size_t)(kt >> 1) * 66;
+                async_load2(rd[set][0], wb, b_rc * row_bytes + 64);
+                async_load16(rq[set][0], wb + (kt & 1) * 32, b_off);
+            }
+        };
+        auto stage_step = [&](int set, int buf) {
+            wait_loads<kLoadsPerStep>();                          // everything but the newer set has arrived
+#pragma unroll
+            for (int i = 0; i < NCH; i++) settle(ra[set][i]);
+#pragma unroll
+            for (int i = 0; i < NB; i++) { settle(rq[set][i]); settle(rd[set][i]); }
+#pragma unroll
+            for (int i = 0; i < NCH; i++)
+                *reinterpret_cast<uint4*>(&As[buf][a_lds[i]]) = make_uint4(ra[set][i].x, ra[set][i].y, ra[set][i].z, ra[set][i].w);
+            if constexpr (FMT == kQ4) {
+                uint32_t f[16];
+#pragma unroll
+                for (int i = 0; i < NB; i++) {
+                    RawB<kQ4> r;
+                    r.q[0] = make_uint4(rq[set][i].x, rq[set][i].y, rq[set][i].z, rq[set][i].w);
+                    r.d = rd[set][i];
+                    convert_b<kQ4>(f, r, 0, true);
+                    store_words<16>(&Bs[buf][b_ld_row * LDK + 64 * part + 32 * i], f);
+                }
+            } else {
+                RawBT r;
+                r.q = make_uint4(rq[set][0].x, rq[set][0].y, rq[set][0].z, rq[set][0].w);
+                r.d = rd[set][0];
+#pragma unroll
+                for (int f = 0; f < 4; f++) {
+                    uint32_t w[8];
+                    convert_bt(w, r, f, true);
+                    store_words<8>(&Bs[buf][b_ld_row * LDK + 32 * f + 16 * part], w);
+                }
+            }
+        };
+        // Step kt is multiplied from LDS buffer kt & 1 while step kt + 1 is staged into the other buffer from register
+        // set (kt + 1) & 1, whose registers then take the loads of step kt + 3.  Every stage finds exactly two sets in
+        // flight, the one it needs being the older.
+        load_step(0, 0);
+        load_step(1, 1);
+        stage_step(0, 0);
+        load_step(0, 2);
+        __syncthreads();
+        for (uint32_t kt = 0; kt < nk; kt += 2) {
+            stage_step(1, 1);
+            load_step(1, kt + 3);
+            __syncthreads();
+            if (kt + 1 < nk) {
+                stage_step(0, 0);
+                load_step(0, kt + 4);
+                __syncthreads();
+            }
+        }
+        wait_loads<0>();             // the over-issued loads must not outlive their destination registers
+        return;
+    }
+
+    const int wm = wave >> 1, wn = wave & 1;
+    // acc[i][j] holds the transposed 16 x 16 tile (weights as the MFMA row operand): lane = output row m (lane & 15) and
+    // four consecutive output columns 4 * (lane >> 4) .. + 3, i.e. one 16-byte store per tile.
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto mfma_step = [&](int buf) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ks++) {
+            f16x8 fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                fa[i] = *reinterpret_cast<const f16x8*>(&As[buf][(wm * 64 + i * 16 + (lane & 15)) * LDK + ks * 32 + (lane >> 4) * 8]);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                fb[j] = *reinterpret_cast<const f16x8*>(&Bs[buf][(wn * 64 + j * 16 + (lane & 15)) * LDK + ks * 32 + (lane >> 4) * 8]);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        }
+    };
+    __syncthreads();
+    for (uint32_t kt = 0; kt < nk; kt += 2) {
+        mfma_step(0);
+        __syncthreads();
+        if (kt + 1 < nk) {
+            mfma_step(1);
+            __syncthreads();
+        }
+    }
+
+    const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t m = m0 + wm * 64 + i * 16 + (lane & 15);
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t n = n0 + wn * 64 + j * 16 + (lane >> 4) * 4;
+            const f32x4 v = acc[i][j];
+            if (vec_ok && n + 3 < N) {
+                if constexpr (CDT == LH_F32) *reinterpret_cast<float4*>(static_cast<float*>(C) + (size_t)m * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+                else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(C) + (size_t)m * N + n) = make_uint2(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (n + r < N) store_elem<CDT>(C, (size_t)m * N + n + r, v[r]);
+            }
+        }
+    }
+}
+
 template <int FMT, int ADT>
-int launch_by_out(bool mfma, hipStream_t s, int cus, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
-                  uint32_t n) {
+int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n) {
+    hipStream_t s = ctx->stream;
+    const int cus = ctx->cu_count;
     if (mfma) {
-        // 128-row tiles reuse each dequantised weight tile twice as often; 64-row tiles when that leaves CUs idle
+        static const int force_bm = [] { const char* e = getenv("LOCAL_HIP_PREFILL_BM"); return e ? atoi(e) : 0; }();
+        // 128-row tiles reuse each dequantised weight tile twice as often; 64-row tiles when that would leave most CUs idle
         const uint64_t tiles128 = (uint64_t)((n + BN - 1) / BN) * ((m + 127) / 128);
-        if (tiles128 >= 2ull * (uint64_t)cus) {
+        const bool big = force_bm == 128 || (force_bm == 0 && m > 64 && tiles128 * 2 >= (uint64_t)cus);
+        if constexpr (FMT != kF16W) {
+            const size_t a16_bytes = (size_t)m * k * 2;
+            if (big && k % BK == 0 && (ADT == LH_F16 || a16_bytes <= ctx->workspace_bytes)) {
+                const uint16_t* a16 = static_cast<const uint16_t*>(A);
+                if constexpr (ADT != LH_F16) {   // one pass over the activations instead of a conversion in every column tile
+                    const size_t n8 = (size_t)m * k / 8;
+                    hipLaunchKernelGGL((convert_to_f16_kernel<ADT>), dim3((uint32_t)((n8 + 255) / 256)), dim3(256), 0, s, A, (uint16_t*)ctx->workspace, n8);
+                    a16 = static_cast<const uint16_t*>(ctx->workspace);
+                }
+                const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
+                if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32>), grid, dim3(512), 0, s, a16, W, C, m, k, n);
+                else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16>), grid, dim3(512), 0, s, a16, W, C, m, k, n);
+                return LH_OK;
+            }
+        }
+        if (force_bm == 128 || (force_bm == 0 && tiles128 >= 2ull * (uint64_t)cus)) {
             const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
             if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
             else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
@@ -317,12 +575,12 @@ int launch_by_out(bool mfma, hipStream_t s, int cus, const void* A, const uint8_
 }
 
 template <int FMT>
-int launch_by_in(bool mfma, hipStream_t s, int cus, const void* A, lh_dtype at, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
+int launch_by_in(bool mfma, lh_context* ctx, const void* A, lh_dtype at, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
                  uint32_t n) {
     switch (at) {
-        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, s, cus, A, W, C, ct, m, k, n);
-        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, s, cus, A, W, C, ct, m, k, n);
-        default: return launch_by_out<FMT, LH_F16>(mfma, s, cus, A, W, C, ct, m, k, n);
+        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, ctx, A, W, C, ct, m, k, n);
+        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, ctx, A, W, C, ct, m, k, n);
+        default: return launch_by_out<FMT, LH_F16>(mfma, ctx, A, W, C, ct, m, k, n);
     }
 }
 
@@ -352,11 +610,10 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
             return rr;
         }
     }
-    hipStream_t s = batch->ctx->stream;
     const uint8_t* W = (const uint8_t*)weight->ptr;
-    if (kind == kQ4) launch_by_in<kQ4>(mfma, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else launch_by_in<kF16W>(true, s, batch->ctx->cu_count, input->ptr, at, W, output->ptr, ct, m, k, n);
+    if (kind == kQ4) launch_by_in<kQ4>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
+    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
+    else launch_by_in<kF16W>(true, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
     int r = lh_check_launch(op);
     if (r == LH_OK) batch->dispatch_count++;
     return r;

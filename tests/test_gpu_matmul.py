@@ -66,6 +66,35 @@ def test_mfma_matmul_tile_boundaries(pkg, gpu, oracle, fmt):
         refgen.assert_close(cb.as_array(np.float32), want_unrounded, 1e-2, f"{fmt} mfma {m}x{k}x{n} vs f32 weights")
 
 
+@pytest.mark.parametrize("adt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_mfma_matmul_large_tiles(pkg, gpu, oracle, fmt, adt):
+    """Shapes that take the 128 x 128 tile kernel (many column tiles, M > 64): ragged M and N, one / odd / even
+    numbers of k steps, every activation type (bf16 and f32 go through the f16 pre-pass), f32 and f16 outputs."""
+    ctx, K = gpu
+    for (m, k, n, ct) in ((130, 256, 8200, "f32"), (200, 768 if fmt == "tq2_0" else 384, 8192, "f16"), (129, 2048, 8300, "f32")):
+        print(f"case {fmt} {adt} m={m} k={k} n={n} out={ct}", flush=True)
+        raw = payload(fmt, n, k, 0xBEEF + m)
+        deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+        a = pkg.synth.rng(4, m + k).standard_normal((m, k), dtype=np.float32) * 0.5
+        if adt == "f16":
+            a_in = a.astype(np.float16); a_eff = a_in.astype(np.float32); dt = pkg.F16
+        elif adt == "bf16":
+            a_in = pkg.synth.f32_to_bf16_bits(a); dt = pkg.BF16
+            a_eff = (a_in.astype(np.uint32) << 16).view(np.float32).astype(np.float16).astype(np.float32)   # bf16 -> f16 as staged
+        else:
+            a_in = a; a_eff = a.astype(np.float16).astype(np.float32); dt = pkg.F32
+        want = oracle.matmul_nt_f32(a_eff, deq)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k)
+        ab = pkg.Buffer.from_slice(ctx, a_in)
+        cb = pkg.Buffer.empty(ctx, m * n * (4 if ct == "f32" else 2))
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, dt, cb, pkg.F32 if ct == "f32" else pkg.F16, m)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float32) if ct == "f32" else cb.as_array(np.float16).astype(np.float32)
+        refgen.assert_close(got, want, 1e-3 if ct == "f32" else 2e-3, f"{fmt} {adt} 128x128 tiles {m}x{k}x{n}")
+
+
 @pytest.mark.parametrize("fmt", ["tq2_0", "q4_0"])
 def test_prefill_config_bf16(pkg, gpu, oracle, fmt):
     """M = 512, K = 2048, N = 8192 with bf16 activations: max normalised error <= 1e-3 against the
@@ -94,8 +123,9 @@ def test_prefill_config_bf16(pkg, gpu, oracle, fmt):
     print(f"prefill {fmt}: max normalised err {err:.2e}")
 
 
+@pytest.mark.parametrize("large", [False, True])
 @pytest.mark.parametrize("fmt", ["tq2_0", "q4_0"])
-def test_prefill_weight_tiles_are_the_cpu_f16_values(pkg, gpu, oracle, fmt):
+def test_prefill_weight_tiles_are_the_cpu_f16_values(pkg, gpu, oracle, fmt, large):
     """One-hot activation rows make the prefill matmul return the weight tile it staged: every sampled
     column must equal the CPU path's dequantised f16 value bit for bit (incl. TQ2 code 3, subnormal and
     zero scales from the reference's payload generators)."""
@@ -103,6 +133,8 @@ def test_prefill_weight_tiles_are_the_cpu_f16_values(pkg, gpu, oracle, fmt):
     m, k, n = 96, 1024 + 32 * (fmt == "q4_0"), 200          # m > 16: the MFMA kernel; ragged n; k not a multiple of 128 for Q4_0
     if fmt == "tq2_0":
         k = 1280
+    if large:                                                # enough tiles for the 128 x 128 kernel; odd number of k steps for Q4_0
+        m, k, n = 160, 1152 if fmt == "q4_0" else 1280, 8200
     raw = payload(fmt, n, k, 0x51DE).copy()
     blk = 18 if fmt == "q4_0" else 66
     doff = 0 if fmt == "q4_0" else 64
