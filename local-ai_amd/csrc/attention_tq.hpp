@@ -1,6 +1,6 @@
 // Shared between the two implementations of attention over packed TurboQuant codes
 // (attention_tq.hip: any bits / head_dim on the vector ALU; attention_tq_mfma.hip: 2-bit codes,
-// head_dim 256 on the matrix cores).
+// head_dim 256 or 512 on the matrix cores).
 #pragma once
 #include "common.hpp"
 
@@ -46,7 +46,7 @@ struct AttnPointers {
     float* ws;
 };
 
-// True when the matrix-core kernel can take this call (2-bit codes, head_dim 256, at most 8 query heads per
+// True when the matrix-core kernel can take this call (2-bit codes, head_dim 256 or 512, at most 8 query heads per
 // KV head, ring absent or a multiple of 64 slots, 4-byte aligned code buffers).
 bool mfma_supported(const AttnParams& p, const AttnPointers& a);
 // Chooses p.num_splits (wave chunks per query and KV head) and launches the split kernel; the caller

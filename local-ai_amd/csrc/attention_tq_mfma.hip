@@ -1,7 +1,7 @@
 // Flash-decoding attention over packed 2-bit TurboQuant codes on the matrix cores.
 //
 // Same contract as attention_tq.hip (stands in for shaders/attention_flash_tq.metal:154-690); this
-// kernel takes the common case -- 2-bit codes, head_dim 256, up to 8 query heads per KV head -- and
+// kernel takes the common case -- 2-bit codes, head_dim 256 or 512, up to 8 query heads per KV head -- and
 // is bound by HBM instead of by the vector ALU.  Per cached position the path moves 132 bytes and
 // needs 8192 multiply-adds (8 heads x 256 dims x {K, V}); decoding every code to a float and
 // multiplying on the vector ALU costs ~40x more issue slots than the memory stream leaves free.
@@ -17,10 +17,10 @@
 //            accumulator because their coefficients are folded into w before quantisation.  The
 //            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
 //            byte transposes.
-// One workgroup of two waves owns a chunk of positions and walks it in aligned groups of 64: the K wave
-// produces the softmax weights of a group, the V wave (one group behind, one barrier per group) turns
-// them into limbs and accumulates.  Splitting the roles keeps each wave under 256 registers, so two
-// waves share a SIMD and fill each other's stalls.  The integer V accumulators persist across groups:
+// One workgroup owns a chunk of positions and walks it in aligned groups of 64: the K wave produces the
+// softmax weights of a group, a V wave per 256 output dims (one group behind, one barrier per group)
+// turns them into limbs and accumulates.  Splitting the roles keeps each wave under 256 registers, so
+// two waves share a SIMD and fill each other's stalls.  The integer V accumulators persist across groups:
 // the softmax reference R_h is only moved (and the accumulators folded into the float outputs) when a
 // weight would leave the fixed-point range, which the 31-bit width makes rare.  Partials (R, l, acc)
 // per chunk go to the workspace for the merge kernel.
