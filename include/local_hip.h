@@ -165,6 +165,12 @@ LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh
 /* kernels.rs:5517-5568 matmul_nt_into: FP16 weights, shaders/matmul_f16.metal:74-114. */
 LH_API int lh_matmul_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, lh_buffer* output,
                              uint32_t m, uint32_t k, uint32_t n);
+/* kernels.rs:3244-3330 clipped_linear_tiled_nt_into (shaders/matmul_f16.metal:121-170):
+ * output = clamp(clamp(input, input_min, input_max) . weight^T + bias, output_min, output_max), all f16,
+ * input [m, k], weight [n, k], bias [n] or NULL. */
+LH_API int lh_clipped_linear_tiled_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                           const lh_buffer* bias, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n,
+                                           float input_min, float input_max, float output_min, float output_max);
 /* kernels.rs:6155, 6160, 6362 constants and 6277-6304 env-flag getters
  * (LOCAL_AI_BATCHM / LOCAL_AI_MMA / LOCAL_AI_SMALLM, read once per process). */
 LH_API uint32_t lh_smallm_max_m(void);

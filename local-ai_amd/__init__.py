@@ -356,6 +356,13 @@ class Kernels:
     def matmul_nt_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
 
+    def clipped_linear_tiled_nt_into(self, batch, input, weight, bias, output, m, k, n, input_min, input_max,
+                                     output_min, output_max):
+        """kernels.rs:3244-3330: clamp(clamp(x) @ W^T + bias); `bias` may be None."""
+        _check(self._l.lh_clipped_linear_tiled_nt_into(batch._h, input._h, weight._h, bias._h if bias is not None else None,
+                                                       output._h, _u32(m), _u32(k), _u32(n), C.c_float(input_min),
+                                                       C.c_float(input_max), C.c_float(output_min), C.c_float(output_max)))
+
     # -- block dequant (qat_recover.rs:23-97) and legacy unpack (kernels.rs:6753-6802) --
     def dequant_q4_0_into(self, batch, data, byte_offset, output, num_elements):
         _check(self._l.lh_dequant_q4_0_into(batch._h, data._h, C.c_size_t(byte_offset), output._h,

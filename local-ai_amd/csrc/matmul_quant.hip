@@ -229,9 +229,22 @@ __device__ __forceinline__ void store_words(_Float16* dst, const uint32_t (&f)[N
     for (int i = 0; i < NW / 4; i++) *reinterpret_cast<uint4*>(dst + 8 * i) = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
 }
 
+// Optional fused clamp / bias of the clipped linear layer (shaders/matmul_f16.metal:121-170):
+// C = clamp(clamp(A, in_lo, in_hi) . W^T + bias, out_lo, out_hi).  Inactive for every other entry point.
+struct ClipArgs {
+    const uint16_t* bias;   // f16 [N] or null
+    float in_lo, in_hi, out_lo, out_hi;
+    uint32_t enabled;
+};
+
+__device__ __forceinline__ uint32_t clamp_h2(uint32_t w, float lo, float hi) {
+    const float a = fminf(fmaxf(lh_h2f((uint16_t)(w & 0xFFFF)), lo), hi), b = fminf(fmaxf(lh_h2f((uint16_t)(w >> 16)), lo), hi);
+    return pack_h2(a, b);
+}
+
 template <int FMT, int ADT, int CDT, int BM>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
-                                                         uint32_t M, uint32_t K, uint32_t N) {
+                                                         uint32_t M, uint32_t K, uint32_t N, ClipArgs clip) {
     constexpr int TI = BM / 32;                              // 16-row MFMA tiles per wave along M (2 x 2 waves)
     constexpr int NCH = BM / 16;                             // 8-element activation chunks staged per thread
     __shared__ __align__(16) _Float16 As[BM * LDK];
@@ -269,6 +282,8 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
         for (int i = 0; i < NCH; i++) {
             const uint32_t c = tid + 256 * i;
             uint4 v = convert_a8<ADT>(ra[set][i]);
+            if (clip.enabled) v = make_uint4(clamp_h2(v.x, clip.in_lo, clip.in_hi), clamp_h2(v.y, clip.in_lo, clip.in_hi),
+                                             clamp_h2(v.z, clip.in_lo, clip.in_hi), clamp_h2(v.w, clip.in_lo, clip.in_hi));
             if (kt * BK + BK > K && kt * BK + 8 * (c & 15) >= K) v = make_uint4(0u, 0u, 0u, 0u);   // only in a partial last k step
             *reinterpret_cast<uint4*>(&As[(c >> 4) * LDK + 8 * (c & 15)]) = v;
         }
@@ -330,10 +345,13 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
         for (int j = 0; j < 4; j++) {
             const uint32_t n = n0 + wn * 64 + j * 16 + (lane & 15);
             if (n >= N) continue;
+            const float bias = (clip.enabled && clip.bias) ? lh_h2f(clip.bias[n]) : 0.0f;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const uint32_t m = m0 + wm * (BM / 2) + i * 16 + (lane >> 4) * 4 + r;
-                if (m < M) store_elem<CDT>(C, (size_t)m * N + n, acc[i][j][r]);
+                float v = acc[i][j][r];
+                if (clip.enabled) v = fminf(fmaxf(v + bias, clip.out_lo), clip.out_hi);
+                if (m < M) store_elem<CDT>(C, (size_t)m * N + n, v);
             }
         }
 }
@@ -532,7 +550,8 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
 }
 
 template <int FMT, int ADT>
-int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n) {
+int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n,
+                  const ClipArgs& clip) {
     hipStream_t s = ctx->stream;
     const int cus = ctx->cu_count;
     if (mfma) {
@@ -557,12 +576,12 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
         }
         if (force_bm == 128 || (force_bm == 0 && tiles128 >= 2ull * (uint64_t)cus)) {
             const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
         } else {
             const dim3 grid((n + BN - 1) / BN, (m + 63) / 64);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
         }
     } else {
         if constexpr (FMT != kF16W) {
@@ -576,17 +595,18 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
 
 template <int FMT>
 int launch_by_in(bool mfma, lh_context* ctx, const void* A, lh_dtype at, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k,
-                 uint32_t n) {
+                 uint32_t n, const ClipArgs& clip) {
     switch (at) {
-        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, ctx, A, W, C, ct, m, k, n);
-        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, ctx, A, W, C, ct, m, k, n);
-        default: return launch_by_out<FMT, LH_F16>(mfma, ctx, A, W, C, ct, m, k, n);
+        case LH_F32: return launch_by_out<FMT, LH_F32>(mfma, ctx, A, W, C, ct, m, k, n, clip);
+        case LH_BF16: return launch_by_out<FMT, LH_BF16>(mfma, ctx, A, W, C, ct, m, k, n, clip);
+        default: return launch_by_out<FMT, LH_F16>(mfma, ctx, A, W, C, ct, m, k, n, clip);
     }
 }
 
 // kind: kQ4 / kTQ2 / kF16W. `force_multivec` is the multivec_nt_* entry (m <= 16 enforced by the caller).
 int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* input, lh_dtype at, const lh_buffer* weight,
-                    lh_buffer* output, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n, bool force_multivec) {
+                    lh_buffer* output, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n, bool force_multivec,
+                    const ClipArgs& clip = ClipArgs{nullptr, 0.f, 0.f, 0.f, 0.f, 0u}) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     if (ct == LH_BF16) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: bf16 output is not supported", op);
     const uint32_t blk = kind == kQ4 ? 32 : (kind == kTQ2 ? 256 : 32);
@@ -611,9 +631,9 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
         }
     }
     const uint8_t* W = (const uint8_t*)weight->ptr;
-    if (kind == kQ4) launch_by_in<kQ4>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
-    else launch_by_in<kF16W>(true, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n);
+    if (kind == kQ4) launch_by_in<kQ4>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n, clip);
+    else if (kind == kTQ2) launch_by_in<kTQ2>(mfma, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n, clip);
+    else launch_by_in<kF16W>(true, batch->ctx, input->ptr, at, W, output->ptr, ct, m, k, n, clip);
     int r = lh_check_launch(op);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
@@ -649,6 +669,12 @@ int lh_matmul_nt_quant_typed_into(lh_batch* b, lh_quant fmt, const lh_buffer* in
 }
 int lh_matmul_nt_into(lh_batch* b, const lh_buffer* in, const lh_buffer* w, lh_buffer* out, uint32_t m, uint32_t k, uint32_t n) {
     return matmul_dispatch(b, "matmul_nt", kF16W, in, LH_F16, w, out, LH_F16, m, k, n, false);
+}
+int lh_clipped_linear_tiled_nt_into(lh_batch* b, const lh_buffer* in, const lh_buffer* w, const lh_buffer* bias, lh_buffer* out, uint32_t m,
+                                    uint32_t k, uint32_t n, float input_min, float input_max, float output_min, float output_max) {
+    if (bias) LH_NEED(bias, (size_t)n * 2, "clipped_linear_tiled_nt", "bias");
+    const ClipArgs clip{bias ? (const uint16_t*)bias->ptr : nullptr, input_min, input_max, output_min, output_max, 1u};
+    return matmul_dispatch(b, "clipped_linear_tiled_nt", kF16W, in, LH_F16, w, out, LH_F16, m, k, n, false, clip);
 }
 
 }  // extern "C"

@@ -203,6 +203,36 @@ def test_matmul_f16_nt(pkg, gpu, oracle):
         refgen.assert_close(cb.as_array(np.float16).astype(np.float32), want, 2e-3, f"f16 nt {m}x{k}x{n}")
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_clipped_linear_tiled_nt(pkg, gpu, oracle, with_bias):
+    """kernels.rs:3244-3330 / shaders/matmul_f16.metal:121-170: clamp(clamp(x) @ W^T + bias), f16 in and out.
+    The checker is the f32 matmul of the oracle over the clamped input plus numpy clamps (bounds chosen
+    f16-exact; both clamps are active on part of the data)."""
+    ctx, K = gpu
+    for (m, k, n) in ((5, 64, 7), (70, 256, 100), (130, 512, 129)):
+        g = pkg.synth.rng(4, 3 * m + n)
+        a = (g.standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+        b = (g.standard_normal((n, k), dtype=np.float32) * 0.5).astype(np.float16)
+        bias = (g.standard_normal(n, dtype=np.float32)).astype(np.float16)
+        in_lo, in_hi, out_lo, out_hi = -0.75, 0.5, -2.0, 3.0
+        ac = np.clip(a.astype(np.float32), in_lo, in_hi)
+        assert (ac != a.astype(np.float32)).any()
+        want = oracle.matmul_nt_f32(ac, b.astype(np.float32))
+        if with_bias:
+            want = want.reshape(m, n) + bias.astype(np.float32)[None, :]
+        unclipped = want
+        want = np.clip(want, out_lo, out_hi).astype(np.float16).astype(np.float32)
+        assert (np.clip(unclipped, out_lo, out_hi) != unclipped).any()
+        ab, bb, cb = pkg.Buffer.from_slice(ctx, a), pkg.Buffer.from_slice(ctx, b), pkg.Buffer.empty(ctx, m * n * 2)
+        biasb = pkg.Buffer.from_slice(ctx, bias) if with_bias else None
+        batch = pkg.CommandBatch(ctx)
+        K.clipped_linear_tiled_nt_into(batch, ab, bb, biasb, cb, m, k, n, in_lo, in_hi, out_lo, out_hi)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float16).astype(np.float32)
+        refgen.assert_close(got, want, 2e-3, f"clipped linear {m}x{k}x{n} bias={with_bias}")
+        assert got.min() >= out_lo and got.max() <= out_hi
+
+
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_block_dequant_bit_exact(pkg, gpu, oracle, fmt):
     """Dequantised weights equal the CPU path's f16 bits for every element, incl. subnormal scales."""
