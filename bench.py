@@ -301,6 +301,38 @@ def bench_prefill(pkg, ctx, K, steps, warmup):
     return res
 
 
+def bench_glue(pkg, ctx, K, steps, warmup):
+    """Decoder-layer glue kernels: latency at the decode shapes (one row of hidden 2048, 8 heads x 256, FFN 8192, the
+    262144 logits) and streaming rate on a large batch of rows (algorithmic bytes = reads + writes)."""
+    g = pkg.synth.rng(11, 1)
+    res = {}
+    batch = pkg.CommandBatch(ctx)
+
+    def f16buf(n):
+        return pkg.Buffer.from_slice(ctx, g.standard_normal(n, dtype=np.float32).astype(np.float16))
+
+    dim, rows = 2048, 49152          # 201 MB per tensor: beyond the 256 MB last-level cache
+    x, w, r, o = f16buf(rows * dim), f16buf(dim), f16buf(rows * dim), pkg.Buffer.empty(ctx, rows * dim * 2)
+    _, ev = time_steps(pkg, ctx, lambda: K.rms_norm_add_into(batch, x, w, r, o, dim, 1, 1e-6), max(steps, 20), warmup)
+    res["rms_norm_add_1x2048_us"] = ev * 1e3
+    _, ev = time_steps(pkg, ctx, lambda: K.rms_norm_add_into(batch, x, w, r, o, dim, rows, 1e-6), steps, warmup)
+    res["rms_norm_add_49152x2048_gbs"] = rows * dim * 2 * 3 / ev * 1e-6
+    hd, nh = 256, 8
+    q, qw = f16buf(nh * hd), f16buf(hd)
+    _, ev = time_steps(pkg, ctx, lambda: K.qk_norm_rope_into(batch, q, q, qw, hd, nh, 1e-6, 1234, 1e6, 1.0), max(steps, 20), warmup)
+    res["qk_norm_rope_8x256_us"] = ev * 1e3
+    n, big = 8192, 1 << 26
+    a, b, go = f16buf(big), f16buf(big), pkg.Buffer.empty(ctx, big * 2)
+    _, ev = time_steps(pkg, ctx, lambda: K.gelu_mul_into(batch, a, b, go, n), max(steps, 20), warmup)
+    res["gelu_mul_8192_us"] = ev * 1e3
+    _, ev = time_steps(pkg, ctx, lambda: K.gelu_mul_into(batch, a, b, go, big), steps, warmup)
+    res["gelu_mul_64M_gbs"] = big * 2 * 3 / ev * 1e-6
+    logits = pkg.Buffer.from_slice(ctx, g.standard_normal(262144, dtype=np.float32))
+    _, ev = time_steps(pkg, ctx, lambda: K.logit_softcap_gpu_into(batch, logits, 30.0, 262144), max(steps, 20), warmup)
+    res["logit_softcap_262144_us"] = ev * 1e3
+    return res
+
+
 def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
     """CPU restatement of the reference path on the host cores: bounded sample of the same workload."""
     from oracle import oracle as orc
@@ -329,7 +361,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill",
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -398,6 +430,9 @@ def main():
     if "prefill" in legs:
         extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] prefill:", extra["prefill_matmul_512x2048x8192_bf16"])
+    if "glue" in legs:
+        extra["layer_glue_kernels"] = bench_glue(pkg, ctx, K, args.steps, args.warmup)
+        log("[bench] glue:", extra["layer_glue_kernels"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
     line = {

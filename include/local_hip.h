@@ -171,6 +171,42 @@ LH_API int lh_matmul_nt_into(lh_batch* batch, const lh_buffer* input, const lh_b
 LH_API int lh_clipped_linear_tiled_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
                                            const lh_buffer* bias, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n,
                                            float input_min, float input_max, float output_min, float output_max);
+/* ---- decoder-layer glue around the hot path (TransformerLayer::forward_decode, layer.rs:354-523) ----
+ * All tensors f16 unless stated; argument order follows the Kernels method named on each line. */
+/* kernels.rs:2142-2152 rms_norm_into (shaders/rms_norm.metal:4-46): out[r] = in[r] * rsqrt(mean(in[r]^2) + eps) * weight */
+LH_API int lh_rms_norm_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, lh_buffer* output,
+                            uint32_t dim, uint32_t rows, float eps);
+/* kernels.rs:6663-6673 rms_norm_add_into (rms_norm.metal:48-88): the same plus residual[r] */
+LH_API int lh_rms_norm_add_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, const lh_buffer* residual,
+                                lh_buffer* output, uint32_t dim, uint32_t rows, float eps);
+/* kernels.rs:2215-2280 qk_norm_gpu_into / qk_norm_offset_into (shaders/qk_norm.metal:6-56): per-head RMSNorm in place;
+ * weight_offset in bytes into the weight buffer */
+LH_API int lh_qk_norm_gpu_into(lh_batch* batch, lh_buffer* qk_data, const lh_buffer* weight, uint32_t head_dim,
+                               uint32_t num_heads, float eps);
+LH_API int lh_qk_norm_offset_into(lh_batch* batch, lh_buffer* qk_data, const lh_buffer* weight, size_t weight_offset,
+                                  uint32_t head_dim, uint32_t num_heads, float eps);
+/* kernels.rs:2282-2392 qk_norm_rope_available / qk_norm_rope_into (qk_norm.metal:70-140): fused norm + NEOX RoPE,
+ * bit-identical to qk_norm followed by rope; input may be output.  Honours LOCAL_AI_NO_FUSE_QKROPE=1. */
+LH_API int lh_qk_norm_rope_available(uint32_t head_dim);
+LH_API int lh_qk_norm_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, const lh_buffer* weight,
+                                uint32_t head_dim, uint32_t num_heads, float eps, uint32_t position, float theta,
+                                float partial_rotary_factor);
+/* kernels.rs:509-580 rope_into (shaders/rope.metal:14-61): NEOX pairs (i, i + head_dim/2), proportional partial rotary;
+ * input may be output */
+LH_API int lh_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, uint32_t head_dim, uint32_t position,
+                        float theta, float partial_rotary_factor, uint32_t num_heads);
+/* kernels.rs:6648-6660 gelu_mul_into (shaders/gelu.metal:23-41): out = gelu_tanh(a) * b */
+LH_API int lh_gelu_mul_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* out, uint32_t count);
+/* kernels.rs:2592-2637 residual_add_into (shaders/residual_add.metal:5-15) */
+LH_API int lh_residual_add_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* output, uint32_t count);
+/* kernels.rs:2845-2890 scale_in_place_gpu_into (shaders/scale_in_place.metal:5-14) */
+LH_API int lh_scale_in_place_gpu_into(lh_batch* batch, lh_buffer* data, float scalar, uint32_t count);
+/* kernels.rs:2801-2843 gather_strided_f16_into (scale_in_place.metal:21-35): dst[i*pld + p] = src[i*row_stride + base_off + p] */
+LH_API int lh_gather_strided_f16_into(lh_batch* batch, const lh_buffer* src, lh_buffer* dst, uint32_t row_stride,
+                                      uint32_t base_off, uint32_t pld, uint32_t n_rows);
+/* kernels.rs:2749-2799 logit_softcap_gpu_into (scale_in_place.metal:39-49): f32 data[i] = cap * tanh(data[i] / cap) */
+LH_API int lh_logit_softcap_gpu_into(lh_batch* batch, lh_buffer* data, float cap, uint32_t count);
+
 /* kernels.rs:6155, 6160, 6362 constants and 6277-6304 env-flag getters
  * (LOCAL_AI_BATCHM / LOCAL_AI_MMA / LOCAL_AI_SMALLM, read once per process). */
 LH_API uint32_t lh_smallm_max_m(void);

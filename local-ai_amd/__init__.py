@@ -363,6 +363,50 @@ class Kernels:
                                                        output._h, _u32(m), _u32(k), _u32(n), C.c_float(input_min),
                                                        C.c_float(input_max), C.c_float(output_min), C.c_float(output_max)))
 
+    # -- decoder-layer glue (kernels.rs:509, 2142-2392, 2592-2890, 6648-6673) --
+    def rms_norm_into(self, batch, input, weight, output, dim, rows, eps):
+        _check(self._l.lh_rms_norm_into(batch._h, input._h, weight._h, output._h, _u32(dim), _u32(rows), C.c_float(eps)))
+
+    def rms_norm_add_into(self, batch, input, weight, residual, output, dim, rows, eps):
+        _check(self._l.lh_rms_norm_add_into(batch._h, input._h, weight._h, residual._h, output._h, _u32(dim), _u32(rows),
+                                            C.c_float(eps)))
+
+    def qk_norm_gpu_into(self, batch, qk_data, weight, head_dim, num_heads, eps):
+        _check(self._l.lh_qk_norm_gpu_into(batch._h, qk_data._h, weight._h, _u32(head_dim), _u32(num_heads), C.c_float(eps)))
+
+    def qk_norm_offset_into(self, batch, qk_data, weight, weight_offset, head_dim, num_heads, eps):
+        _check(self._l.lh_qk_norm_offset_into(batch._h, qk_data._h, weight._h, C.c_size_t(weight_offset), _u32(head_dim),
+                                              _u32(num_heads), C.c_float(eps)))
+
+    def qk_norm_rope_available(self, head_dim):
+        return bool(self._l.lh_qk_norm_rope_available(_u32(head_dim)))
+
+    def qk_norm_rope_into(self, batch, input, output, weight, head_dim, num_heads, eps, position, theta,
+                          partial_rotary_factor):
+        _check(self._l.lh_qk_norm_rope_into(batch._h, input._h, output._h, weight._h, _u32(head_dim), _u32(num_heads),
+                                            C.c_float(eps), _u32(position), C.c_float(theta),
+                                            C.c_float(partial_rotary_factor)))
+
+    def rope_into(self, batch, input, output, head_dim, position, theta, partial_rotary_factor, num_heads):
+        _check(self._l.lh_rope_into(batch._h, input._h, output._h, _u32(head_dim), _u32(position), C.c_float(theta),
+                                    C.c_float(partial_rotary_factor), _u32(num_heads)))
+
+    def gelu_mul_into(self, batch, a, b, out, count):
+        _check(self._l.lh_gelu_mul_into(batch._h, a._h, b._h, out._h, _u32(count)))
+
+    def residual_add_into(self, batch, a, b, output, count):
+        _check(self._l.lh_residual_add_into(batch._h, a._h, b._h, output._h, _u32(count)))
+
+    def scale_in_place_gpu_into(self, batch, data, scalar, count):
+        _check(self._l.lh_scale_in_place_gpu_into(batch._h, data._h, C.c_float(scalar), _u32(count)))
+
+    def gather_strided_f16_into(self, batch, src, dst, row_stride, base_off, pld, n_rows):
+        _check(self._l.lh_gather_strided_f16_into(batch._h, src._h, dst._h, _u32(row_stride), _u32(base_off), _u32(pld),
+                                                  _u32(n_rows)))
+
+    def logit_softcap_gpu_into(self, batch, data, cap, count):
+        _check(self._l.lh_logit_softcap_gpu_into(batch._h, data._h, C.c_float(cap), _u32(count)))
+
     # -- block dequant (qat_recover.rs:23-97) and legacy unpack (kernels.rs:6753-6802) --
     def dequant_q4_0_into(self, batch, data, byte_offset, output, num_elements):
         _check(self._l.lh_dequant_q4_0_into(batch._h, data._h, C.c_size_t(byte_offset), output._h,

@@ -1,0 +1,341 @@
+// Decoder-layer glue kernels around the matvec / attention hot path: RMSNorm (+ residual), per-head QK norm
+// (+ RoPE), NEOX RoPE with proportional partial rotary, GeGLU elementwise, residual add, in-place scale,
+// strided f16 gather, final-logit soft cap.  Stand in for shaders/rms_norm.metal:4-88, qk_norm.metal:6-140,
+// rope.metal:14-61, gelu.metal:23-41, residual_add.metal:5-15, scale_in_place.metal:5-52 and their dispatchers
+// in local-metal/src/kernels.rs.  At decode these touch a few KB per call: they are latency bound, one small
+// workgroup per row / head, f32 math, f16 storage with the same rounding points as the reference kernels.
+#include "common.hpp"
+#include <cstdlib>
+
+namespace {
+
+__device__ __forceinline__ float h_at(const uint16_t* p, size_t i) { return lh_h2f(p[i]); }
+
+// One NEOX pair at `position` (rope.metal:46-58).  The same instruction sequence serves the stand-alone and the fused
+// kernel, so that qk_norm + rope and qk_norm_rope agree bit for bit (kernels.rs:7873).
+__device__ __forceinline__ void rotate_pair(float x0, float x1, uint32_t i, uint32_t head_dim, uint32_t position, float theta, uint16_t& o0, uint16_t& o1) {
+    const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)head_dim);
+    const float angle = (float)position * freq;
+    const float c = cosf(angle), sn = sinf(angle);
+    o0 = lh_f2h(__builtin_fmaf(x0, c, -(x1 * sn)));
+    o1 = lh_f2h(__builtin_fmaf(x0, sn, x1 * c));
+}
+
+// Sum over a workgroup of up to 256 threads (4 waves).
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    v = lh_group_sum(v, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = (blockDim.x + 63) >> 6;
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nwaves; w++) t += scratch[w];
+    __syncthreads();
+    return t;
+}
+
+// rms_norm.metal:4-46 / 48-88: out[r, i] = in[r, i] * rsqrt(mean(in[r]^2) + eps) * w[i] (+ residual[r, i]).
+// VEC = 8: 16-byte accesses (dim a multiple of 8, 16-byte aligned rows); VEC = 1 otherwise.
+template <bool ADD, int VEC>
+__global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const uint16_t* __restrict__ w, const uint16_t* res, uint16_t* out,   // out may be in or res
+                                                      uint32_t dim, float eps) {
+    __shared__ float scratch[4];
+    const size_t row = (size_t)blockIdx.x * dim;
+    float s = 0.0f;
+    if constexpr (VEC == 8) {
+        for (uint32_t i = threadIdx.x * 8; i < dim; i += blockDim.x * 8) {
+            const uint4 v = *reinterpret_cast<const uint4*>(in + row + i);
+            const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) { const float a = lh_h2f((uint16_t)(wv[j] & 0xFFFF)), b = lh_h2f((uint16_t)(wv[j] >> 16)); s += a * a; s += b * b; }
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) { const float v = h_at(in, row + i); s += v * v; }
+    }
+    const float rms = rsqrtf(block_sum(s, scratch) / (float)dim + eps);
+    if constexpr (VEC == 8) {
+        for (uint32_t i = threadIdx.x * 8; i < dim; i += blockDim.x * 8) {
+            const uint4 v = *reinterpret_cast<const uint4*>(in + row + i), g = *reinterpret_cast<const uint4*>(w + i);
+            uint4 r = v;
+            if (ADD) r = *reinterpret_cast<const uint4*>(res + row + i);
+            const uint32_t wv[4] = {v.x, v.y, v.z, v.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
+            uint32_t wo[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float lo = lh_h2f((uint16_t)(wv[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
+                float hi = lh_h2f((uint16_t)(wv[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
+                if (ADD) { lo += lh_h2f((uint16_t)(wr[j] & 0xFFFF)); hi += lh_h2f((uint16_t)(wr[j] >> 16)); }
+                wo[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
+            }
+            *reinterpret_cast<uint4*>(out + row + i) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
+            float v = h_at(in, row + i) * rms * h_at(w, i);
+            if (ADD) v += h_at(res, row + i);
+            out[row + i] = lh_f2h(v);
+        }
+    }
+}
+
+template <bool ADD>
+void launch_rms_norm(hipStream_t stream, const void* in, const void* w, const void* res, void* out, uint32_t dim, uint32_t rows, float eps) {
+    const bool vec = (dim & 7) == 0 && (((uintptr_t)in | (uintptr_t)w | (uintptr_t)(res ? res : in) | (uintptr_t)out) & 15) == 0;
+    const uint32_t threads = vec ? (dim >= 2048 ? 256u : (dim >= 1024 ? 128u : 64u)) : (dim >= 256 ? 256u : (dim > 64 ? 128u : 64u));
+    if (vec) hipLaunchKernelGGL((rms_norm_kernel<ADD, 8>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps);
+    else hipLaunchKernelGGL((rms_norm_kernel<ADD, 1>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps);
+}
+
+// qk_norm.metal:6-56 (in place; head h of `qk`), and 70-140 with the NEOX rotation fused: the normalised values are
+// rounded to f16 before they are rotated, exactly as when qk_norm and rope run as two kernels.
+template <bool ROPE>
+__global__ __launch_bounds__(256) void qk_norm_kernel(const uint16_t* in, uint16_t* out, const uint16_t* __restrict__ w,   // in may be out
+                                                     uint32_t head_dim, float eps, uint32_t position, float theta, float prf) {
+    __shared__ float scratch[4];
+    __shared__ uint16_t normed[512];
+    const size_t base = (size_t)blockIdx.x * head_dim;
+    float s = 0.0f;
+    for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) { const float v = h_at(in, base + j); s += v * v; }
+    const float rms = rsqrtf(block_sum(s, scratch) / (float)head_dim + eps);
+    if (!ROPE) {
+        for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) out[base + j] = lh_f2h(h_at(in, base + j) * rms * h_at(w, j));
+        return;
+    }
+    for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) normed[j] = lh_f2h(h_at(in, base + j) * rms * h_at(w, j));
+    __syncthreads();
+    const uint32_t half_dim = head_dim / 2;
+    const uint32_t rope_angles = (uint32_t)((float)head_dim * prf) / 2;
+    for (uint32_t i = threadIdx.x; i < half_dim; i += blockDim.x) {
+        const float x0 = lh_h2f(normed[i]), x1 = lh_h2f(normed[i + half_dim]);
+        if (i >= rope_angles) {
+            out[base + i] = lh_f2h(x0);
+            out[base + i + half_dim] = lh_f2h(x1);
+        } else {
+            uint16_t o0, o1;
+            rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
+            out[base + i] = o0;
+            out[base + i + half_dim] = o1;
+        }
+    }
+}
+
+// rope.metal:14-61: NEOX pairing (i, i + head_dim / 2); only the first prf * head_dim / 2 pairs rotate, with the
+// frequencies of the full head.
+__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* in, uint16_t* out, uint32_t head_dim, uint32_t position,   // in may be out
+                                                  float theta, float prf, uint32_t num_heads) {
+    const uint32_t half_dim = head_dim / 2;
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= half_dim * num_heads) return;
+    const uint32_t head = t / half_dim, i = t - head * half_dim;
+    const size_t idx0 = (size_t)head * head_dim + i, idx1 = idx0 + half_dim;
+    const uint32_t rope_angles = (uint32_t)((float)head_dim * prf) / 2;
+    if (i >= rope_angles) { out[idx0] = in[idx0]; out[idx1] = in[idx1]; return; }
+    const float x0 = h_at(in, idx0), x1 = h_at(in, idx1);
+    uint16_t o0, o1;
+    rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
+    out[idx0] = o0;
+    out[idx1] = o1;
+}
+
+// Elementwise f16 kernels: a thread takes 8 consecutive elements with 16-byte accesses; the launcher sends a
+// count that is not a multiple of 8, or pointers that are not 16-byte aligned, to the one-element form (VEC = 1).
+__device__ __forceinline__ float gelu_tanh_f32(float x) {   // gelu.metal:31-35
+    const float x3 = x * x * x;
+    const float inner = 0.7978845608f * (x + 0.044715f * x3);
+    const float t = tanhf(fminf(fmaxf(inner, -10.0f), 10.0f));
+    return 0.5f * x * (1.0f + t);
+}
+
+enum { kGeluMul = 0, kResidualAdd = 1, kScale = 2 };
+
+// gelu.metal:23-41 (out = gelu(a) * b), residual_add.metal:5-15 (an f16 addition: one rounding of the exact sum),
+// scale_in_place.metal:5-14 (out = half(float(a) * scalar), a may be out)
+template <int OP>
+__device__ __forceinline__ uint16_t elementwise_one(uint16_t a, uint16_t b, float scalar) {
+    if constexpr (OP == kGeluMul) return lh_f2h(gelu_tanh_f32(lh_h2f(a)) * lh_h2f(b));
+    else if constexpr (OP == kResidualAdd) return __builtin_bit_cast(uint16_t, (_Float16)(__builtin_bit_cast(_Float16, a) + __builtin_bit_cast(_Float16, b)));
+    else return lh_f2h(lh_h2f(a) * scalar);
+}
+
+template <int OP, int VEC>
+__global__ __launch_bounds__(256) void elementwise_kernel(const uint16_t* a, const uint16_t* b, uint16_t* out, float scalar, uint32_t count) {
+    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (i >= count) return;
+    if constexpr (VEC == 8) {
+        const uint4 va = *reinterpret_cast<const uint4*>(a + i);
+        uint4 vb = va;
+        if constexpr (OP != kScale) vb = *reinterpret_cast<const uint4*>(b + i);
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+        uint32_t wo[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            wo[j] = (uint32_t)elementwise_one<OP>((uint16_t)(wa[j] & 0xFFFF), (uint16_t)(wb[j] & 0xFFFF), scalar) |
+                    ((uint32_t)elementwise_one<OP>((uint16_t)(wa[j] >> 16), (uint16_t)(wb[j] >> 16), scalar) << 16);
+        *reinterpret_cast<uint4*>(out + i) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+    } else {
+        out[i] = elementwise_one<OP>(a[i], OP != kScale ? b[i] : a[i], scalar);
+    }
+}
+
+template <int OP>
+void launch_elementwise(hipStream_t stream, const void* a, const void* b, void* out, float scalar, uint32_t count) {
+    const bool vec = (count & 7) == 0 && (((uintptr_t)a | (uintptr_t)(b ? b : a) | (uintptr_t)out) & 15) == 0;
+    if (vec) hipLaunchKernelGGL((elementwise_kernel<OP, 8>), dim3((count / 8 + 255) / 256), dim3(256), 0, stream, (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, scalar, count);
+    else hipLaunchKernelGGL((elementwise_kernel<OP, 1>), dim3((count + 255) / 256), dim3(256), 0, stream, (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, scalar, count);
+}
+
+// scale_in_place.metal:21-35: dst[i * pld + p] = src[i * row_stride + base_off + p]
+__global__ __launch_bounds__(256) void gather_strided_f16_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, uint32_t row_stride, uint32_t base_off,
+                                                                uint32_t pld, uint32_t n_rows) {
+    const uint32_t g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= n_rows * pld) return;
+    const uint32_t i = g / pld, p = g - i * pld;
+    dst[g] = src[(size_t)i * row_stride + base_off + p];
+}
+
+// scale_in_place.metal:39-49
+__global__ __launch_bounds__(256) void logit_softcap_kernel(float* __restrict__ data, float cap, uint32_t count) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) data[i] = cap * tanhf(data[i] / cap);
+}
+
+inline uint32_t blocks_for(uint64_t n) { return (uint32_t)((n + 255) / 256); }
+inline uint32_t norm_threads(uint32_t dim) { return dim >= 256 ? 256u : (dim > 64 ? 128u : 64u); }
+
+int finish(lh_batch* batch, const char* op) {
+    const int r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lh_rms_norm_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, lh_buffer* output, uint32_t dim, uint32_t rows, float eps) {
+    const char* op = "rms_norm";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (dim == 0 || rows == 0) return LH_OK;
+    LH_NEED(input, (size_t)rows * dim * 2, op, "input");
+    LH_NEED(weight, (size_t)dim * 2, op, "weight");
+    LH_NEED(output, (size_t)rows * dim * 2, op, "output");
+    launch_rms_norm<false>(batch->ctx->stream, input->ptr, weight->ptr, nullptr, output->ptr, dim, rows, eps);
+    return finish(batch, op);
+}
+
+int lh_rms_norm_add_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, const lh_buffer* residual, lh_buffer* output,
+                         uint32_t dim, uint32_t rows, float eps) {
+    const char* op = "rms_norm_add";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (dim == 0 || rows == 0) return LH_OK;
+    LH_NEED(input, (size_t)rows * dim * 2, op, "input");
+    LH_NEED(weight, (size_t)dim * 2, op, "weight");
+    LH_NEED(residual, (size_t)rows * dim * 2, op, "residual");
+    LH_NEED(output, (size_t)rows * dim * 2, op, "output");
+    launch_rms_norm<true>(batch->ctx->stream, input->ptr, weight->ptr, residual->ptr, output->ptr, dim, rows, eps);
+    return finish(batch, op);
+}
+
+int lh_qk_norm_offset_into(lh_batch* batch, lh_buffer* qk_data, const lh_buffer* weight, size_t weight_offset, uint32_t head_dim,
+                           uint32_t num_heads, float eps) {
+    const char* op = "qk_norm";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (head_dim == 0 || num_heads == 0) return LH_OK;
+    LH_REQUIRE((weight_offset & 1) == 0, "%s: weight offset %zu is not 2-byte aligned", op, weight_offset);
+    LH_NEED(qk_data, (size_t)num_heads * head_dim * 2, op, "qk_data");
+    LH_NEED(weight, weight_offset + (size_t)head_dim * 2, op, "weight");
+    const uint16_t* w = (const uint16_t*)((const uint8_t*)weight->ptr + weight_offset);
+    hipLaunchKernelGGL(qk_norm_kernel<false>, dim3(num_heads), dim3(norm_threads(head_dim)), 0, batch->ctx->stream, (const uint16_t*)qk_data->ptr,
+                       (uint16_t*)qk_data->ptr, w, head_dim, eps, 0u, 0.0f, 0.0f);
+    return finish(batch, op);
+}
+
+int lh_qk_norm_gpu_into(lh_batch* batch, lh_buffer* qk_data, const lh_buffer* weight, uint32_t head_dim, uint32_t num_heads, float eps) {
+    return lh_qk_norm_offset_into(batch, qk_data, weight, 0, head_dim, num_heads, eps);
+}
+
+int lh_qk_norm_rope_available(uint32_t head_dim) {
+    static const bool disabled = [] { const char* e = getenv("LOCAL_AI_NO_FUSE_QKROPE"); return e && e[0] == '1' && e[1] == 0; }();
+    return (!disabled && head_dim <= 512) ? 1 : 0;
+}
+
+int lh_qk_norm_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, const lh_buffer* weight, uint32_t head_dim,
+                         uint32_t num_heads, float eps, uint32_t position, float theta, float partial_rotary_factor) {
+    const char* op = "qk_norm_rope";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (head_dim == 0 || num_heads == 0) return LH_OK;
+    LH_REQUIRE(head_dim <= 512 && (head_dim & 1) == 0, "%s: head_dim %u must be even and at most 512", op, head_dim);
+    LH_NEED(input, (size_t)num_heads * head_dim * 2, op, "input");
+    LH_NEED(output, (size_t)num_heads * head_dim * 2, op, "output");
+    LH_NEED(weight, (size_t)head_dim * 2, op, "weight");
+    hipLaunchKernelGGL(qk_norm_kernel<true>, dim3(num_heads), dim3(norm_threads(head_dim)), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
+                       (uint16_t*)output->ptr, (const uint16_t*)weight->ptr, head_dim, eps, position, theta, partial_rotary_factor);
+    return finish(batch, op);
+}
+
+int lh_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, uint32_t head_dim, uint32_t position, float theta,
+                 float partial_rotary_factor, uint32_t num_heads) {
+    const char* op = "rope";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (head_dim == 0 || num_heads == 0) return LH_OK;
+    LH_REQUIRE((head_dim & 1) == 0, "%s: head_dim %u must be even", op, head_dim);
+    LH_NEED(input, (size_t)num_heads * head_dim * 2, op, "input");
+    LH_NEED(output, (size_t)num_heads * head_dim * 2, op, "output");
+    hipLaunchKernelGGL(rope_kernel, dim3(blocks_for((uint64_t)num_heads * head_dim / 2)), dim3(256), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
+                       (uint16_t*)output->ptr, head_dim, position, theta, partial_rotary_factor, num_heads);
+    return finish(batch, op);
+}
+
+int lh_gelu_mul_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* out, uint32_t count) {
+    const char* op = "gelu_mul";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (count == 0) return LH_OK;
+    LH_NEED(a, (size_t)count * 2, op, "a");
+    LH_NEED(b, (size_t)count * 2, op, "b");
+    LH_NEED(out, (size_t)count * 2, op, "out");
+    launch_elementwise<kGeluMul>(batch->ctx->stream, a->ptr, b->ptr, out->ptr, 0.0f, count);
+    return finish(batch, op);
+}
+
+int lh_residual_add_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* output, uint32_t count) {
+    const char* op = "residual_add";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (count == 0) return LH_OK;
+    LH_NEED(a, (size_t)count * 2, op, "a");
+    LH_NEED(b, (size_t)count * 2, op, "b");
+    LH_NEED(output, (size_t)count * 2, op, "output");
+    launch_elementwise<kResidualAdd>(batch->ctx->stream, a->ptr, b->ptr, output->ptr, 0.0f, count);
+    return finish(batch, op);
+}
+
+int lh_scale_in_place_gpu_into(lh_batch* batch, lh_buffer* data, float scalar, uint32_t count) {
+    const char* op = "scale_in_place";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (count == 0) return LH_OK;
+    LH_NEED(data, (size_t)count * 2, op, "data");
+    launch_elementwise<kScale>(batch->ctx->stream, data->ptr, nullptr, data->ptr, scalar, count);
+    return finish(batch, op);
+}
+
+int lh_gather_strided_f16_into(lh_batch* batch, const lh_buffer* src, lh_buffer* dst, uint32_t row_stride, uint32_t base_off, uint32_t pld,
+                               uint32_t n_rows) {
+    const char* op = "gather_strided_f16";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (pld == 0 || n_rows == 0) return LH_OK;
+    LH_REQUIRE((uint64_t)n_rows * pld <= 0xFFFFFFFFull, "%s: %u rows x %u elements do not fit 32 bits", op, n_rows, pld);
+    LH_NEED(src, ((size_t)(n_rows - 1) * row_stride + base_off + pld) * 2, op, "src");
+    LH_NEED(dst, (size_t)n_rows * pld * 2, op, "dst");
+    hipLaunchKernelGGL(gather_strided_f16_kernel, dim3(blocks_for((uint64_t)n_rows * pld)), dim3(256), 0, batch->ctx->stream, (const uint16_t*)src->ptr,
+                       (uint16_t*)dst->ptr, row_stride, base_off, pld, n_rows);
+    return finish(batch, op);
+}
+
+int lh_logit_softcap_gpu_into(lh_batch* batch, lh_buffer* data, float cap, uint32_t count) {
+    const char* op = "logit_softcap";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (count == 0) return LH_OK;
+    LH_NEED(data, (size_t)count * 4, op, "data");
+    hipLaunchKernelGGL(logit_softcap_kernel, dim3(blocks_for(count)), dim3(256), 0, batch->ctx->stream, (float*)data->ptr, cap, count);
+    return finish(batch, op);
+}
+
+}  // extern "C"
