@@ -327,6 +327,17 @@ def bench_glue(pkg, ctx, K, steps, warmup):
     res["gelu_mul_8192_us"] = ev * 1e3
     _, ev = time_steps(pkg, ctx, lambda: K.gelu_mul_into(batch, a, b, go, big), steps, warmup)
     res["gelu_mul_64M_gbs"] = big * 2 * 3 / ev * 1e-6
+    # FP16-weight matvec (the QuantWeight fallback): 131072 x 2048 f16 = 537 MB streamed once
+    frows, fcols = 131072, 2048
+    fw = pkg.Buffer.empty(ctx, frows * fcols * 2)
+    seed_rows = g.standard_normal(4096 * fcols, dtype=np.float32).astype(np.float16)
+    for i in range(frows // 4096):
+        fw.copy_from_bytes(seed_rows, i * 4096 * fcols * 2)
+    fx, fy = f16buf(fcols), pkg.Buffer.empty(ctx, frows * 4)
+    _, ev = time_steps(pkg, ctx, lambda: K.matvec_f32out_offset_into(batch, fw, 0, fx, fy, frows, fcols), steps, warmup)
+    res["matvec_f16_131072x2048_gbs"] = (frows * fcols * 2 + fcols * 2 + frows * 4) / ev * 1e-6
+    _, ev = time_steps(pkg, ctx, lambda: K.matvec_f32out_offset_into(batch, fw, 0, fx, fy, 2048, fcols), max(steps, 20), warmup)
+    res["matvec_f16_2048x2048_us"] = ev * 1e3
     logits = pkg.Buffer.from_slice(ctx, g.standard_normal(262144, dtype=np.float32))
     _, ev = time_steps(pkg, ctx, lambda: K.logit_softcap_gpu_into(batch, logits, 30.0, 262144), max(steps, 20), warmup)
     res["logit_softcap_262144_us"] = ev * 1e3

@@ -171,6 +171,24 @@ LH_API int lh_matmul_nt_into(lh_batch* batch, const lh_buffer* input, const lh_b
 LH_API int lh_clipped_linear_tiled_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
                                            const lh_buffer* bias, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n,
                                            float input_min, float input_max, float output_min, float output_max);
+/* ---- FP16-weight matvec family (shaders/matvec_f16.metal:14-133), the QuantWeight fallbacks for tensors kept as
+ * F16 (layer.rs:134, 158, 182).  matrix [rows, cols] f16 starting matrix_offset bytes into its buffer; f32 accumulate. */
+/* kernels.rs:582-640 matvec (f16 x, f16 y; enqueue and wait) and 1710-1764 matvec_offset_into */
+LH_API int lh_matvec(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
+                     uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector,
+                                 lh_buffer* output, uint32_t rows, uint32_t cols);
+/* kernels.rs:1766-1874 matvec_f32out_offset{,_into} (matvec_f16w_f32out: f16 x, f32 y) */
+LH_API int lh_matvec_f32out_offset(lh_context* ctx, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector,
+                                   lh_buffer* output, uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_f32out_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset,
+                                        const lh_buffer* vector, lh_buffer* output, uint32_t rows, uint32_t cols);
+/* kernels.rs:1876-1930 matvec_f32in_offset (matvec_f16w_f32in: f32 x, f16 y); the _into form is this library's */
+LH_API int lh_matvec_f32in_offset(lh_context* ctx, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector,
+                                  lh_buffer* output, uint32_t rows, uint32_t cols);
+LH_API int lh_matvec_f32in_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset,
+                                       const lh_buffer* vector, lh_buffer* output, uint32_t rows, uint32_t cols);
+
 /* ---- decoder-layer glue around the hot path (TransformerLayer::forward_decode, layer.rs:354-523) ----
  * All tensors f16 unless stated; argument order follows the Kernels method named on each line. */
 /* kernels.rs:2142-2152 rms_norm_into (shaders/rms_norm.metal:4-46): out[r] = in[r] * rsqrt(mean(in[r]^2) + eps) * weight */

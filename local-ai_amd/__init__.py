@@ -363,6 +363,30 @@ class Kernels:
                                                        output._h, _u32(m), _u32(k), _u32(n), C.c_float(input_min),
                                                        C.c_float(input_max), C.c_float(output_min), C.c_float(output_max)))
 
+    # -- FP16-weight matvec family (kernels.rs:582, 1710-1930) --
+    def matvec(self, ctx, matrix, vector, output, rows, cols):
+        _check(self._l.lh_matvec(ctx._h, matrix._h, vector._h, output._h, _u32(rows), _u32(cols)))
+
+    def matvec_offset_into(self, batch, matrix, matrix_offset, vector, output, rows, cols):
+        _check(self._l.lh_matvec_offset_into(batch._h, matrix._h, C.c_size_t(matrix_offset), vector._h, output._h, _u32(rows),
+                                             _u32(cols)))
+
+    def matvec_f32out_offset(self, ctx, matrix, matrix_offset, vector, output, rows, cols):
+        _check(self._l.lh_matvec_f32out_offset(ctx._h, matrix._h, C.c_size_t(matrix_offset), vector._h, output._h, _u32(rows),
+                                               _u32(cols)))
+
+    def matvec_f32out_offset_into(self, batch, matrix, matrix_offset, vector, output, rows, cols):
+        _check(self._l.lh_matvec_f32out_offset_into(batch._h, matrix._h, C.c_size_t(matrix_offset), vector._h, output._h,
+                                                    _u32(rows), _u32(cols)))
+
+    def matvec_f32in_offset(self, ctx, matrix, matrix_offset, vector, output, rows, cols):
+        _check(self._l.lh_matvec_f32in_offset(ctx._h, matrix._h, C.c_size_t(matrix_offset), vector._h, output._h, _u32(rows),
+                                              _u32(cols)))
+
+    def matvec_f32in_offset_into(self, batch, matrix, matrix_offset, vector, output, rows, cols):
+        _check(self._l.lh_matvec_f32in_offset_into(batch._h, matrix._h, C.c_size_t(matrix_offset), vector._h, output._h,
+                                                   _u32(rows), _u32(cols)))
+
     # -- decoder-layer glue (kernels.rs:509, 2142-2392, 2592-2890, 6648-6673) --
     def rms_norm_into(self, batch, input, weight, output, dim, rows, eps):
         _check(self._l.lh_rms_norm_into(batch._h, input._h, weight._h, output._h, _u32(dim), _u32(rows), C.c_float(eps)))

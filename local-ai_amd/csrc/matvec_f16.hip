@@ -1,0 +1,128 @@
+// FP16-weight matvec family: y[rows] = W[rows, cols] . x[cols], f32 accumulation; x and y f16 or f32.
+// Stands in for shaders/matvec_f16.metal:14-133 (matvec_f16, matvec_f16w_f32out, matvec_f16w_f32in) and their
+// dispatchers (local-metal/src/kernels.rs:582, 1710-1930), the fallbacks of QuantWeight for tensors that are kept
+// as F16 (local-engine/src/layer.rs:134, 158, 182).  Pure weight streaming: 2 bytes per multiply-add, HBM-bound.
+// One wave per row at a time, 16 bytes per lane and load, the activation vector staged once per workgroup in LDS
+// as f32; rows are dealt to the waves of the whole grid round robin so that the grid reads one advancing window.
+#include "common.hpp"
+#include <algorithm>
+
+namespace {
+
+constexpr int kMaxLdsCols = 12288;   // 48 KB of f32 activations
+
+template <typename XT> __device__ __forceinline__ float x_at(const XT* x, uint32_t i);
+template <> __device__ __forceinline__ float x_at<uint16_t>(const uint16_t* x, uint32_t i) { return lh_h2f(x[i]); }
+template <> __device__ __forceinline__ float x_at<float>(const float* x, uint32_t i) { return x[i]; }
+
+template <typename XT, typename YT, bool VEC, bool XLDS>
+__global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restrict__ W, const XT* __restrict__ x, YT* __restrict__ y, uint32_t rows,
+                                                        uint32_t cols) {
+    extern __shared__ float xs[];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    if (XLDS) {
+        for (uint32_t i = threadIdx.x; i < cols; i += blockDim.x) xs[i] = x_at<XT>(x, i);
+        __syncthreads();
+    }
+    auto xv = [&](uint32_t i) { return XLDS ? xs[i] : x_at<XT>(x, i); };
+    for (uint32_t row = blockIdx.x * nwaves + wave; row < rows; row += gridDim.x * nwaves) {
+        const uint16_t* wr = W + (size_t)row * cols;
+        float acc = 0.0f;
+        if (VEC) {   // cols a multiple of 8 and 16-byte aligned rows; up to 8 loads of 16 bytes in flight per lane
+            for (uint32_t k0 = lane * 8; k0 < cols; k0 += 8 * 512) {
+                uint4 v[8];
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const uint32_t k = k0 + 512 * c;
+                    v[c] = k < cols ? *reinterpret_cast<const uint4*>(wr + k) : make_uint4(0u, 0u, 0u, 0u);
+                }
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    const uint32_t k = k0 + 512 * c;
+                    if (k >= cols) break;
+                    const uint32_t wv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), xv(k + 2 * j), acc);
+                        acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] >> 16)), xv(k + 2 * j + 1), acc);
+                    }
+                }
+            }
+        } else {
+            for (uint32_t k = lane; k < cols; k += 64) acc = __builtin_fmaf(lh_h2f(wr[k]), xv(k), acc);
+        }
+        acc = lh_group_sum(acc, 64);
+        if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
+    }
+}
+
+template <typename XT, typename YT>
+int launch(lh_context* ctx, const uint16_t* W, const void* x, void* y, uint32_t rows, uint32_t cols) {
+    const bool vec = (cols & 7) == 0 && ((uintptr_t)W & 15) == 0;
+    const bool xlds = cols <= (uint32_t)kMaxLdsCols;
+    const uint32_t waves = 4;
+    const uint64_t want = ((uint64_t)rows + waves - 1) / waves;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>(want, (uint64_t)ctx->cu_count * 8);
+    const size_t lds = xlds ? (size_t)cols * 4 : 0;
+#define LH_F16MV(V, L) hipLaunchKernelGGL((matvec_f16_kernel<XT, YT, V, L>), dim3(grid), dim3(64 * waves), lds, ctx->stream, W, (const XT*)x, (YT*)y, rows, cols)
+    if (vec && xlds) LH_F16MV(true, true);
+    else if (vec) LH_F16MV(true, false);
+    else if (xlds) LH_F16MV(false, true);
+    else LH_F16MV(false, false);
+#undef LH_F16MV
+    return LH_OK;
+}
+
+int matvec_f16_dispatch(lh_context* ctx, lh_batch* batch, const char* op, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector,
+                        lh_buffer* output, uint32_t rows, uint32_t cols, bool x_f32, bool y_f32) {
+    if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: context is null", op);
+    if (rows == 0 || cols == 0) return LH_OK;
+    LH_REQUIRE((matrix_offset & 1) == 0, "%s: matrix offset %zu is not 2-byte aligned", op, matrix_offset);
+    LH_NEED(matrix, matrix_offset + (size_t)rows * cols * 2, op, "matrix");
+    LH_NEED(vector, (size_t)cols * (x_f32 ? 4 : 2), op, "vector");
+    LH_NEED(output, (size_t)rows * (y_f32 ? 4 : 2), op, "output");
+    const uint16_t* W = (const uint16_t*)((const uint8_t*)matrix->ptr + matrix_offset);
+    if (!x_f32 && !y_f32) launch<uint16_t, uint16_t>(ctx, W, vector->ptr, output->ptr, rows, cols);
+    else if (!x_f32) launch<uint16_t, float>(ctx, W, vector->ptr, output->ptr, rows, cols);
+    else if (!y_f32) launch<float, uint16_t>(ctx, W, vector->ptr, output->ptr, rows, cols);
+    else launch<float, float>(ctx, W, vector->ptr, output->ptr, rows, cols);
+    const int r = lh_check_launch(op);
+    if (r != LH_OK) return r;
+    if (batch) { batch->dispatch_count++; return LH_OK; }
+    lh_batch one_shot{ctx, 1};
+    return lh_batch_commit_and_wait(&one_shot);
+}
+
+}  // namespace
+
+extern "C" {
+
+// kernels.rs:582-640 matvec (one-shot: enqueue and wait)
+int lh_matvec(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output, uint32_t rows, uint32_t cols) {
+    return matvec_f16_dispatch(ctx, nullptr, "matvec", matrix, 0, vector, output, rows, cols, false, false);
+}
+int lh_matvec_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector, lh_buffer* output, uint32_t rows,
+                          uint32_t cols) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec: batch is null");
+    return matvec_f16_dispatch(batch->ctx, batch, "matvec", matrix, matrix_offset, vector, output, rows, cols, false, false);
+}
+int lh_matvec_f32out_offset(lh_context* ctx, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector, lh_buffer* output, uint32_t rows,
+                            uint32_t cols) {
+    return matvec_f16_dispatch(ctx, nullptr, "matvec_f32out", matrix, matrix_offset, vector, output, rows, cols, false, true);
+}
+int lh_matvec_f32out_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector, lh_buffer* output,
+                                 uint32_t rows, uint32_t cols) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_f32out: batch is null");
+    return matvec_f16_dispatch(batch->ctx, batch, "matvec_f32out", matrix, matrix_offset, vector, output, rows, cols, false, true);
+}
+int lh_matvec_f32in_offset(lh_context* ctx, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector, lh_buffer* output, uint32_t rows,
+                           uint32_t cols) {
+    return matvec_f16_dispatch(ctx, nullptr, "matvec_f32in", matrix, matrix_offset, vector, output, rows, cols, true, false);
+}
+int lh_matvec_f32in_offset_into(lh_batch* batch, const lh_buffer* matrix, size_t matrix_offset, const lh_buffer* vector, lh_buffer* output,
+                                uint32_t rows, uint32_t cols) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_f32in: batch is null");
+    return matvec_f16_dispatch(batch->ctx, batch, "matvec_f32in", matrix, matrix_offset, vector, output, rows, cols, true, false);
+}
+
+}  // extern "C"

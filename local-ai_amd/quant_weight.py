@@ -7,11 +7,17 @@ import numpy as np
 from . import Q4_0, TQ2_0, F16, F32, BF16, Buffer, InvalidArgument, Kernels
 
 _BLOCK = {Q4_0: (32, 18), TQ2_0: (256, 66)}
+W_F16 = "f16"   # GGUFType::F16: plain f16 rows, served by the FP16 matvec / matmul kernels (layer.rs:27-34)
 
 
 class QuantWeight:
     def __init__(self, buf: Buffer, ty: int, rows: int, cols: int):
         self.buf, self.ty, self.rows, self.cols = buf, ty, rows, cols
+
+    @classmethod
+    def f16(cls, buf: Buffer, rows: int, cols: int) -> "QuantWeight":
+        """layer.rs:27-34: an FP16 tensor (also what Q8_0 / F32 tensors are expanded to at load time)."""
+        return cls(buf, W_F16, rows, cols)
 
     @classmethod
     def quantized(cls, buf: Buffer, ty: int, rows: int, cols: int) -> "QuantWeight":
@@ -36,6 +42,8 @@ class QuantWeight:
         return self.buf.length()
 
     def row_bytes(self) -> int:
+        if self.ty == W_F16:
+            return self.cols * 2
         block, nbytes = _BLOCK[self.ty]
         return (self.cols // block) * nbytes
 
@@ -43,14 +51,18 @@ class QuantWeight:
     def matvec_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer) -> None:
         if self.ty == Q4_0:
             kernels.matvec_q4_0_into(batch, self.buf, x, out, self.rows, self.cols)
-        else:
+        elif self.ty == TQ2_0:
             kernels.matvec_tq2_0_into(batch, self.buf, x, out, self.rows, self.cols)
+        else:
+            kernels.matvec_offset_into(batch, self.buf, 0, x, out, self.rows, self.cols)
 
     def matvec_f32out_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer) -> None:
         if self.ty == Q4_0:
             kernels.matvec_q4_0_f32out_into(batch, self.buf, x, out, self.rows, self.cols)
-        else:
+        elif self.ty == TQ2_0:
             kernels.matvec_tq2_0_f32out_into(batch, self.buf, x, out, self.rows, self.cols)
+        else:
+            kernels.matvec_f32out_offset_into(batch, self.buf, 0, x, out, self.rows, self.cols)
 
     def matvec_typed_into(self, batch, kernels: Kernels, x: Buffer, x_dtype: int, out: Buffer, out_dtype: int) -> None:
         kernels.matvec_quant_typed_into(batch, self.ty, self.buf, x, x_dtype, out, out_dtype, self.rows, self.cols)
@@ -59,8 +71,10 @@ class QuantWeight:
     def matmul_nt_into(self, batch, kernels: Kernels, x: Buffer, out: Buffer, m: int) -> None:
         if self.ty == Q4_0:
             kernels.matmul_nt_q4_0_into(batch, x, self.buf, out, m, self.cols, self.rows)
-        else:
+        elif self.ty == TQ2_0:
             kernels.matmul_nt_tq2_0_into(batch, x, self.buf, out, m, self.cols, self.rows)
+        else:
+            kernels.matmul_nt_into(batch, x, self.buf, out, m, self.cols, self.rows)
 
     def matmul_nt_typed_into(self, batch, kernels: Kernels, x: Buffer, x_dtype: int, out: Buffer, out_dtype: int,
                              m: int) -> None:
@@ -73,5 +87,7 @@ class QuantWeight:
         off = row * self.row_bytes()
         if self.ty == Q4_0:
             kernels.dequant_q4_0_into(batch, self.buf, off, out, self.cols)
-        else:
+        elif self.ty == TQ2_0:
             kernels.dequant_tq2_0_into(batch, self.buf, off, out, self.cols)
+        else:
+            batch.blit_copy(self.buf, off, out, 0, self.cols * 2)   # an f16 row is its own dequantisation

@@ -96,3 +96,12 @@ def logit_softcap(data, cap: float) -> np.ndarray:
     """shaders/scale_in_place.metal:39-49: cap * tanh(x / cap) in f32."""
     x = np.asarray(data, F32)
     return (F32(cap) * np.tanh((x / F32(cap)).astype(np.float64))).astype(F32)
+
+
+def matvec_f16(w, x, rows: int, cols: int, out_f32: bool = False) -> np.ndarray:
+    """shaders/matvec_f16.metal:14-133: y = W . x with f16 weights, f16 or f32 x, f32 accumulation (summed here in
+    float64), y rounded to f16 unless `out_f32`."""
+    w = np.asarray(w, F16).reshape(rows, cols).astype(np.float64)
+    xv = np.asarray(x).astype(np.float64).reshape(cols)
+    y = w @ xv
+    return y.astype(F32) if out_f32 else y.astype(F32).astype(F16)
