@@ -85,3 +85,18 @@ def test_elementwise_closed_forms():
     out = lg.logit_softcap(data, 30.0)
     for i in (0, 1000, 2048, 2049, 4095):
         assert abs(out[i] - 30.0 * math.tanh(float(data[i]) / 30.0)) < 1e-4
+
+
+def test_matvec_f16_known_products():
+    """kernels.rs:7294-7360: identity x [5,7,9]; [[1,2],[3,4]] x [5,6] = [17,39]; [[1..4],[5..8]] x ones = [10,26]."""
+    h = np.float16
+    assert np.array_equal(lg.matvec_f16(np.eye(3, dtype=h), np.array([5, 7, 9], h), 3, 3), np.array([5, 7, 9], h))
+    assert np.array_equal(lg.matvec_f16(np.array([1, 2, 3, 4], h), np.array([5, 6], h), 2, 2), np.array([17, 39], h))
+    assert np.array_equal(lg.matvec_f16(np.arange(1, 9).astype(h), np.ones(4, h), 2, 4, out_f32=True), np.array([10, 26], np.float32))
+    # linear in x, and rows are independent
+    g = np.random.default_rng(5)
+    w = g.standard_normal((6, 40)).astype(h)
+    x1, x2 = g.standard_normal(40).astype(np.float32), g.standard_normal(40).astype(np.float32)
+    y = lg.matvec_f16(w, x1 + x2, 6, 40, out_f32=True)
+    assert np.allclose(y, lg.matvec_f16(w, x1, 6, 40, out_f32=True) + lg.matvec_f16(w, x2, 6, 40, out_f32=True), atol=1e-4)
+    assert np.array_equal(lg.matvec_f16(w[2:3], x1, 1, 40, out_f32=True), lg.matvec_f16(w, x1, 6, 40, out_f32=True)[2:3])
