@@ -213,6 +213,12 @@ LH_API int lh_qk_norm_rope_into(lh_batch* batch, const lh_buffer* input, lh_buff
  * input may be output */
 LH_API int lh_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, uint32_t head_dim, uint32_t position,
                         float theta, float partial_rotary_factor, uint32_t num_heads);
+/* kernels.rs:4228-4300 rope_batch_into (rope.metal:105-150): in place over qk [seq_len, num_heads, head_dim], row r at
+ * position start_pos + r; kernels.rs:4311-4385 rope_batch_decode_into (rope.metal:157-200): row r at positions[r] (u32) */
+LH_API int lh_rope_batch_into(lh_batch* batch, lh_buffer* qk, uint32_t start_pos, float theta, uint32_t head_dim,
+                              uint32_t num_heads, uint32_t seq_len, float partial_rotary_factor);
+LH_API int lh_rope_batch_decode_into(lh_batch* batch, lh_buffer* qk, const lh_buffer* positions, float theta,
+                                     uint32_t head_dim, uint32_t num_heads, uint32_t seq_len, float partial_rotary_factor);
 /* kernels.rs:6648-6660 gelu_mul_into (shaders/gelu.metal:23-41): out = gelu_tanh(a) * b */
 LH_API int lh_gelu_mul_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* out, uint32_t count);
 /* kernels.rs:2592-2637 residual_add_into (shaders/residual_add.metal:5-15) */

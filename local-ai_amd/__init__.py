@@ -415,6 +415,14 @@ class Kernels:
         _check(self._l.lh_rope_into(batch._h, input._h, output._h, _u32(head_dim), _u32(position), C.c_float(theta),
                                     C.c_float(partial_rotary_factor), _u32(num_heads)))
 
+    def rope_batch_into(self, batch, qk, start_pos, theta, head_dim, num_heads, seq_len, partial_rotary_factor):
+        _check(self._l.lh_rope_batch_into(batch._h, qk._h, _u32(start_pos), C.c_float(theta), _u32(head_dim), _u32(num_heads),
+                                          _u32(seq_len), C.c_float(partial_rotary_factor)))
+
+    def rope_batch_decode_into(self, batch, qk, positions, theta, head_dim, num_heads, seq_len, partial_rotary_factor):
+        _check(self._l.lh_rope_batch_decode_into(batch._h, qk._h, positions._h, C.c_float(theta), _u32(head_dim), _u32(num_heads),
+                                                 _u32(seq_len), C.c_float(partial_rotary_factor)))
+
     def gelu_mul_into(self, batch, a, b, out, count):
         _check(self._l.lh_gelu_mul_into(batch._h, a._h, b._h, out._h, _u32(count)))
 

@@ -136,6 +136,25 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* in, uint16_t*
     out[idx1] = o1;
 }
 
+// rope.metal:105-200 rope_batch / rope_batch_decode: in place over qk [seq_len, num_heads, head_dim]; row r sits at
+// position start_pos + r, or at positions[r] when a table is given (independent sequences of a batched decode).
+__global__ __launch_bounds__(256) void rope_batch_kernel(uint16_t* qk, const uint32_t* __restrict__ positions, uint32_t start_pos, float theta, uint32_t head_dim,
+                                                        uint32_t num_heads, uint32_t seq_len, float prf) {
+    const uint32_t half_dim = head_dim / 2;
+    const uint32_t rope_angles = (uint32_t)((float)head_dim * prf) / 2;
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (rope_angles == 0 || t >= (uint64_t)rope_angles * num_heads * seq_len) return;
+    const uint32_t i = (uint32_t)(t % rope_angles);
+    const uint32_t flat = (uint32_t)(t / rope_angles);          // (row, head), head fastest: rows of qk are contiguous
+    const uint32_t seq_idx = flat / num_heads, head = flat - seq_idx * num_heads;
+    const uint32_t position = positions ? positions[seq_idx] : start_pos + seq_idx;
+    const size_t idx0 = ((size_t)seq_idx * num_heads + head) * head_dim + i, idx1 = idx0 + half_dim;
+    uint16_t o0, o1;
+    rotate_pair(h_at(qk, idx0), h_at(qk, idx1), i, head_dim, position, theta, o0, o1);
+    qk[idx0] = o0;
+    qk[idx1] = o1;
+}
+
 // Elementwise f16 kernels: a thread takes 8 consecutive elements with 16-byte accesses; the launcher sends a
 // count that is not a multiple of 8, or pointers that are not 16-byte aligned, to the one-element form (VEC = 1).
 __device__ __forceinline__ float gelu_tanh_f32(float x) {   // gelu.metal:31-35
@@ -283,6 +302,31 @@ int lh_rope_into(lh_batch* batch, const lh_buffer* input, lh_buffer* output, uin
     hipLaunchKernelGGL(rope_kernel, dim3(blocks_for((uint64_t)num_heads * head_dim / 2)), dim3(256), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
                        (uint16_t*)output->ptr, head_dim, position, theta, partial_rotary_factor, num_heads);
     return finish(batch, op);
+}
+
+static int rope_batch_common(const char* op, lh_batch* batch, lh_buffer* qk, const lh_buffer* positions, uint32_t start_pos, float theta, uint32_t head_dim,
+                             uint32_t num_heads, uint32_t seq_len, float partial_rotary_factor) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (head_dim == 0 || num_heads == 0 || seq_len == 0) return LH_OK;
+    LH_REQUIRE((head_dim & 1) == 0, "%s: head_dim %u must be even", op, head_dim);
+    LH_NEED(qk, (size_t)seq_len * num_heads * head_dim * 2, op, "qk");
+    if (positions) LH_NEED(positions, (size_t)seq_len * 4, op, "positions");
+    const uint32_t rope_angles = (uint32_t)((float)head_dim * partial_rotary_factor) / 2;
+    if (rope_angles == 0) return LH_OK;
+    hipLaunchKernelGGL(rope_batch_kernel, dim3(blocks_for((uint64_t)rope_angles * num_heads * seq_len)), dim3(256), 0, batch->ctx->stream, (uint16_t*)qk->ptr,
+                       positions ? (const uint32_t*)positions->ptr : nullptr, start_pos, theta, head_dim, num_heads, seq_len, partial_rotary_factor);
+    return finish(batch, op);
+}
+
+int lh_rope_batch_into(lh_batch* batch, lh_buffer* qk, uint32_t start_pos, float theta, uint32_t head_dim, uint32_t num_heads, uint32_t seq_len,
+                       float partial_rotary_factor) {
+    return rope_batch_common("rope_batch", batch, qk, nullptr, start_pos, theta, head_dim, num_heads, seq_len, partial_rotary_factor);
+}
+
+int lh_rope_batch_decode_into(lh_batch* batch, lh_buffer* qk, const lh_buffer* positions, float theta, uint32_t head_dim, uint32_t num_heads,
+                              uint32_t seq_len, float partial_rotary_factor) {
+    if (!positions) return lh_fail(LH_ERR_INVALID_ARGUMENT, "rope_batch_decode: positions is null");
+    return rope_batch_common("rope_batch_decode", batch, qk, positions, 0, theta, head_dim, num_heads, seq_len, partial_rotary_factor);
 }
 
 int lh_gelu_mul_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh_buffer* out, uint32_t count) {

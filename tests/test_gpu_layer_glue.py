@@ -76,6 +76,34 @@ def test_qk_norm_rope_family(pkg, gpu, hd, nh, prf, pos, theta):
     assert np.array_equal(got[:, ra:hd // 2], src[:, ra:hd // 2]) and np.array_equal(got[:, hd // 2 + ra:], src[:, hd // 2 + ra:])
 
 
+@pytest.mark.parametrize("hd,nh,rows,prf", [(256, 8, 5, 1.0), (512, 2, 3, 0.25), (64, 4, 17, 0.5)])
+def test_rope_batch_forms(pkg, gpu, hd, nh, rows, prf):
+    """kernels.rs:8079-8190: rope_batch == rope per row at consecutive positions (bit for bit: same rotation code),
+    rope_batch_decode == rope_batch for contiguous positions and applies independent positions per row."""
+    ctx, K = gpu
+    n = rows * nh * hd
+    data = (np.sin(np.arange(n, dtype=np.float32) * np.float32(0.017)) * np.float32(0.9)).astype(np.float16)
+    start, theta = 731, 1e6
+    per_row = pkg.Buffer.from_slice(ctx, data)
+    batched, dec_contig, dec_indep = (pkg.Buffer.from_slice(ctx, data) for _ in range(3))
+    pos_indep = np.array([(r * 7919 + 13) % 50000 for r in range(rows)], np.uint32)
+    pc, pi = pkg.Buffer.from_slice(ctx, np.arange(start, start + rows, dtype=np.uint32)), pkg.Buffer.from_slice(ctx, pos_indep)
+    batch = pkg.CommandBatch(ctx)
+    for r in range(rows):
+        v = per_row.view(r * nh * hd * 2, nh * hd * 2)
+        K.rope_into(batch, v, v, hd, start + r, theta, prf, nh)
+    K.rope_batch_into(batch, batched, start, theta, hd, nh, rows, prf)
+    K.rope_batch_decode_into(batch, dec_contig, pc, theta, hd, nh, rows, prf)
+    K.rope_batch_decode_into(batch, dec_indep, pi, theta, hd, nh, rows, prf)
+    batch.commit_and_wait()
+    assert np.array_equal(batched.as_array(np.uint16), per_row.as_array(np.uint16))
+    assert np.array_equal(dec_contig.as_array(np.uint16), batched.as_array(np.uint16))
+    got = dec_indep.as_array(np.float16).reshape(rows, nh * hd)
+    for r in range(rows):
+        want = lg.rope(data.reshape(rows, nh * hd)[r], hd, int(pos_indep[r]), theta, prf, nh)
+        close(got[r], want, 2e-3 + 2.5e-7 * int(pos_indep[r]), f"rope_batch_decode row {r}")
+
+
 @pytest.mark.parametrize("n", [8192 + 37, 8192, 8])
 def test_elementwise_glue(pkg, gpu, n):
     """kernels.rs:7076-7117, 7693-7815: gelu_mul, residual_add, scale_in_place, gather_strided_f16, logit_softcap
