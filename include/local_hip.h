@@ -62,6 +62,10 @@ LH_API const char* lh_version(void);
 
 /* ---- context: MetalContext::new / device_name / caps (context.rs:38-86) ---- */
 LH_API int lh_context_create(int device_index, lh_context** out);
+/* Waits for the stream and drops the creator's handle.  Buffers, batches and events made from the
+ * context keep its stream and workspace alive until the last of them is freed, so handles may be
+ * released in any order (as Rust's drop order lets the reference's owners do); `ctx` itself must not
+ * be passed to any call afterwards. */
 LH_API void lh_context_destroy(lh_context* ctx);
 LH_API int lh_context_device_name(const lh_context* ctx, char* dst, size_t dst_len);
 LH_API int lh_context_compute_units(const lh_context* ctx);

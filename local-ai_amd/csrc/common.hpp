@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <atomic>
 #include "../../include/local_hip.h"
 
 struct lh_context {
@@ -14,6 +15,9 @@ struct lh_context {
     // per (query head, split). Allocated once with the context.
     void* workspace;
     size_t workspace_bytes;
+    // The creator's handle plus one per live buffer, batch and event: the stream and the workspace are
+    // released when the last of them goes, so handles may be freed in any order.
+    std::atomic<int> refs;
 };
 
 struct lh_buffer {

@@ -58,6 +58,17 @@ extern "C" {
 const char* lh_last_error(void) { return g_last_error; }
 const char* lh_version(void) { return "local-hip 0.1 (gfx950)"; }
 
+static void ctx_retain(lh_context* ctx) { ctx->refs.fetch_add(1, std::memory_order_relaxed); }
+
+static void ctx_release(lh_context* ctx) {
+    if (ctx->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->workspace);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
 int lh_context_create(int device_index, lh_context** out) {
     if (!out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "context_create: out is null");
     *out = nullptr;
@@ -72,6 +83,7 @@ int lh_context_create(int device_index, lh_context** out) {
     lh_context* ctx = new (std::nothrow) lh_context();
     if (!ctx) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_context));
     ctx->device = device_index;
+    ctx->refs.store(1, std::memory_order_relaxed);
     ctx->cu_count = prop.multiProcessorCount;
     snprintf(ctx->name, sizeof ctx->name, "%s (%s)", prop.name, prop.gcnArchName);
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
@@ -92,9 +104,7 @@ void lh_context_destroy(lh_context* ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree(ctx->workspace);
-    (void)hipStreamDestroy(ctx->stream);
-    delete ctx;
+    ctx_release(ctx);
 }
 
 int lh_context_device_name(const lh_context* ctx, char* dst, size_t dst_len) {
@@ -121,10 +131,16 @@ int lh_event_create(lh_context* ctx, lh_event** out) {
     if (!e) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_event));
     e->ctx = ctx;
     if (hipEventCreate(&e->ev) != hipSuccess) { delete e; return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: hipEventCreate"); }
+    ctx_retain(ctx);
     *out = e;
     return LH_OK;
 }
-void lh_event_destroy(lh_event* ev) { if (ev) { (void)hipEventDestroy(ev->ev); delete ev; } }
+void lh_event_destroy(lh_event* ev) {
+    if (!ev) return;
+    (void)hipEventDestroy(ev->ev);
+    ctx_release(ev->ctx);
+    delete ev;
+}
 int lh_event_record(lh_event* ev) {
     if (!ev) return lh_fail(LH_ERR_INVALID_ARGUMENT, "event_record: event is null");
     hipError_t e = hipEventRecord(ev->ev, ev->ctx->stream);
@@ -150,6 +166,7 @@ static int new_buffer(lh_context* ctx, size_t len, lh_buffer** out) {
     // partly filled last unit inside the allocation.
     hipError_t e = hipMalloc(&b->ptr, (len ? len : 1) + 64);
     if (e != hipSuccess) { delete b; return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: %s", len, hipGetErrorString(e)); }
+    ctx_retain(ctx);
     *out = b;
     return LH_OK;
 }
@@ -181,6 +198,7 @@ int lh_buffer_view(lh_buffer* parent, size_t offset, size_t len, lh_buffer** out
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
     b->ctx = parent->ctx; b->ptr = (char*)parent->ptr + offset; b->len = len; b->owns = false;
     b->slack = parent->len - offset - len + parent->slack;
+    ctx_retain(b->ctx);
     *out = b;
     return LH_OK;
 }
@@ -190,6 +208,7 @@ int lh_buffer_wrap(lh_context* ctx, void* device_ptr, size_t len, lh_buffer** ou
     lh_buffer* b = new (std::nothrow) lh_buffer();
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", len);
     b->ctx = ctx; b->ptr = device_ptr; b->len = len; b->owns = false; b->slack = 0;
+    ctx_retain(ctx);
     *out = b;
     return LH_OK;
 }
@@ -200,6 +219,7 @@ void lh_buffer_free(lh_buffer* buf) {
         (void)hipStreamSynchronize(buf->ctx->stream);
         (void)hipFree(buf->ptr);
     }
+    ctx_release(buf->ctx);
     delete buf;
 }
 
@@ -242,10 +262,15 @@ int lh_batch_new(lh_context* ctx, lh_batch** out) {
     lh_batch* b = new (std::nothrow) lh_batch();
     if (!b) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_batch));
     b->ctx = ctx; b->dispatch_count = 0;
+    ctx_retain(ctx);
     *out = b;
     return LH_OK;
 }
-void lh_batch_free(lh_batch* batch) { delete batch; }
+void lh_batch_free(lh_batch* batch) {
+    if (!batch) return;
+    ctx_release(batch->ctx);
+    delete batch;
+}
 uint32_t lh_batch_dispatch_count(const lh_batch* batch) { return batch ? batch->dispatch_count : 0; }
 
 int lh_batch_blit_copy(lh_batch* batch, const lh_buffer* src, size_t src_offset, lh_buffer* dst, size_t dst_offset, size_t len) {

@@ -125,3 +125,86 @@ class QuantizedKvCache:
         fn(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms, self.levels, vacc, hd, kv_len,
            start_pos, n_rows, n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
         kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, vecs, False, True)
+
+
+class QuantizedUnifiedKvPool:
+    """``QuantizedUnifiedKvPool`` (local-engine/src/kv_cache/quant_unified_pool.rs:33-345): one layer's
+    TurboQuant KV for ``n_lanes`` independent sequences, laid out
+    ``[n_lanes, lane rows, n_kv_heads, code_bytes]``; a device ``positions[n_lanes]`` u32 buffer carries
+    every lane's current position so one encode launch and one attention launch serve all lanes."""
+
+    def __init__(self, ctx, n_lanes: int, lane_capacity: int, n_kv_heads: int, head_dim: int, bits: int,
+                 lane_ring_capacity: int = 0):
+        """quant_unified_pool.rs:69-104: a ringed lane keeps only its first ``lane_ring_capacity`` rows."""
+        if not 2 <= bits <= 4:
+            raise InvalidArgument(f"TurboQuant bits must be 2..=4, got {bits}")
+        lane_ring_capacity = min(lane_ring_capacity, lane_capacity)
+        self.ctx = ctx
+        self.n_lanes, self.lane_capacity, self.lane_ring_capacity = n_lanes, lane_capacity, lane_ring_capacity
+        self.n_kv_heads, self.head_dim, self.bits = n_kv_heads, head_dim, bits
+        self._cb = code_bytes(head_dim, bits)
+        slots = max(n_lanes * self.lane_stride() * n_kv_heads, 1)
+        self.levels = Buffer.from_slice(ctx, turboquant_levels(head_dim, bits))
+        self.signs = Buffer.from_slice(ctx, turboquant_signs(head_dim, TQ_SEED))
+        self.keys_q = Buffer.empty(ctx, slots * self._cb)
+        self.values_q = Buffer.empty(ctx, slots * self._cb)
+        self.key_norms = Buffer.empty(ctx, slots * 2)
+        self.value_norms = Buffer.empty(ctx, slots * 2)
+
+    def lane_stride(self) -> int:
+        """quant_unified_pool.rs:116-122: physical rows per lane, the lane base stride of the batched kernels."""
+        return self.lane_ring_capacity if self.lane_ring_capacity else self.lane_capacity
+
+    def write_kv_into(self, batch, kernels: Kernels, k_src: Buffer, v_src: Buffer, positions: Buffer,
+                      active_lanes: int) -> None:
+        """quant_unified_pool.rs:138-181: encode one K and one V row per lane at ``positions[lane]``."""
+        lanes = min(active_lanes, self.n_lanes)
+        for src, codes, norms in ((k_src, self.keys_q, self.key_norms), (v_src, self.values_q, self.value_norms)):
+            kernels.encode_kv_turboquant_batched_into(batch, src, self.levels, self.signs, codes, norms, positions,
+                                                      self.head_dim, self.n_kv_heads, self.lane_stride(), self.bits,
+                                                      lanes, self.lane_ring_capacity)
+
+    def attention_into(self, batch, kernels: Kernels, q: Buffer, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                       positions: Buffer, n_q_heads: int, window: int, active_lanes: int) -> None:
+        """quant_unified_pool.rs:194-256: rotate every lane's query heads, attend over the lane's codes up to its
+        own position, rotate back to f16."""
+        hd = self.head_dim
+        lanes = min(active_lanes, self.n_lanes)
+        total_heads = lanes * n_q_heads
+        kernels.hadamard_rotate_hf_into(batch, q, self.signs, rq, hd, total_heads, True, False)
+        kernels.flash_attention_tq_batched_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
+                                                self.value_norms, self.levels, vacc, positions, hd, self.lane_stride(),
+                                                n_q_heads, self.n_kv_heads, window, self.bits, lanes,
+                                                self.lane_ring_capacity)
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, total_heads, False, True)
+
+    def copy_prefill_from(self, batch, cache: QuantizedKvCache, lane: int, positions: int) -> None:
+        """quant_unified_pool.rs:269-315: seed ``lane`` with the first ``positions`` rows of a single-sequence
+        cache that shares the codec (a ringed pair copies the whole physical ring once it has wrapped).  Both
+        sides live in device memory here, so the four copies are device-to-device and ordered in ``batch``."""
+        if positions > self.lane_capacity:
+            raise InvalidArgument(f"prefill {positions} positions exceeds lane_capacity {self.lane_capacity}")
+        if lane >= self.n_lanes or positions == 0:
+            return
+        if self.lane_ring_capacity and self.lane_ring_capacity != cache.physical_positions:
+            raise InvalidArgument(f"pool ring {self.lane_ring_capacity} must match staging cache ring "
+                                  f"{cache.physical_positions}")
+        rows = (min(positions, self.lane_ring_capacity) if self.lane_ring_capacity else positions) * self.n_kv_heads
+        lane_row0 = lane * self.lane_stride() * self.n_kv_heads
+        for src, dst, stride in ((cache.keys_q, self.keys_q, self._cb), (cache.values_q, self.values_q, self._cb),
+                                 (cache.key_norms, self.key_norms, 2), (cache.value_norms, self.value_norms, 2)):
+            batch.blit_copy(src, 0, dst, lane_row0 * stride, rows * stride)
+
+    def reset(self) -> None:
+        """quant_unified_pool.rs:318-328: a zero norm annihilates whatever the codes say."""
+        for b in (self.keys_q, self.values_q, self.key_norms, self.value_norms):
+            b.fill_zero()
+
+    def reset_lane(self, lane: int) -> None:
+        """quant_unified_pool.rs:331-345."""
+        if lane >= self.n_lanes:
+            return
+        rows = self.lane_stride() * self.n_kv_heads
+        for b, stride in ((self.keys_q, self._cb), (self.values_q, self._cb), (self.key_norms, 2),
+                          (self.value_norms, 2)):
+            b.view(lane * rows * stride, rows * stride).fill_zero()

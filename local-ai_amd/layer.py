@@ -1,0 +1,317 @@
+"""``TransformerLayer`` (local-engine/src/layer.rs:284-873): one Gemma decoder layer encoded into a
+command batch -- single-token decode, multi-row prefill / batched decode over one sequence, and
+continuous-batching decode over independent lanes -- plus its scratch arenas
+(``ScratchBuffers`` layer.rs:951-1037, ``BatchScratch`` layer.rs:878-948).
+
+Every dispatch is one of the HIP kernels behind the C ABI; this file only orders them the way the
+reference does and owns no arithmetic.  One addition over the reference's call sequence: when two
+projections read the same input and share format and shape (K/V, gate/up), the single-token path
+launches them as one grouped matvec so both weight streams are in flight together; the results are
+the same values the separate launches produce.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+from . import F16, Q4_0, TQ2_0, Buffer, InvalidArgument, Kernels
+from .kv_cache import QuantizedKvCache, QuantizedUnifiedKvPool
+from .quant_weight import W_F16, QuantWeight
+
+MAX_FLASH_SPLITS = 16   # layer.rs:979
+
+
+@dataclass
+class LayerParams:
+    """layer.rs:291-308."""
+    layer_idx: int
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    per_layer_dim: int = 0
+    rope_theta: float = 10000.0
+    partial_rotary_factor: float = 1.0
+    sliding_window: int = 0
+    rms_norm_eps: float = 1e-6
+    is_kv_shared: bool = False
+
+
+@dataclass
+class LayerWeights:
+    """layer.rs:310-328: norm vectors are f16 buffers, projections are ``QuantWeight``."""
+    attn_norm: Buffer
+    attn_q: QuantWeight
+    attn_output: QuantWeight
+    attn_post_norm: Buffer
+    ffn_norm: Buffer
+    ffn_gate: QuantWeight
+    ffn_up: QuantWeight
+    ffn_down: QuantWeight
+    ffn_post_norm: Buffer
+    attn_k: Optional[QuantWeight] = None
+    attn_v: Optional[QuantWeight] = None
+    q_norm: Optional[Buffer] = None
+    k_norm: Optional[Buffer] = None
+    per_layer_inp_gate: Optional[QuantWeight] = None
+    per_layer_proj: Optional[QuantWeight] = None
+    per_layer_post_norm: Optional[Buffer] = None
+    layer_output_scale: Optional[Buffer] = None
+
+    @classmethod
+    def from_host(cls, ctx, tensors: dict) -> "LayerWeights":
+        """Upload host tensors keyed by field name: a projection is ``(format, rows, cols, payload)`` with
+        format "q4_0" / "tq2_0" (GGUF block bytes, uploaded verbatim) or "f16"; anything else is an f16 vector."""
+        fields = {}
+        for name, t in tensors.items():
+            if isinstance(t, tuple):
+                fmt, rows, cols, payload = t
+                if fmt == "f16":
+                    fields[name] = QuantWeight.f16(Buffer.from_slice(ctx, np.asarray(payload, np.float16)), rows, cols)
+                else:
+                    fields[name] = QuantWeight.from_bytes(ctx, payload, {"q4_0": Q4_0, "tq2_0": TQ2_0}[fmt], rows, cols)
+            else:
+                fields[name] = Buffer.from_slice(ctx, np.asarray(t, np.float16))
+        return cls(**fields)
+
+
+def _alloc_f16(ctx, elems: int) -> Buffer:
+    return Buffer.empty(ctx, max(elems, 1) * 2)
+
+
+def _alloc_f32(ctx, elems: int) -> Buffer:
+    return Buffer.empty(ctx, max(elems, 1) * 4)
+
+
+class ScratchBuffers:
+    """layer.rs:951-1037: single-token scratch sized for the widest layer."""
+
+    def __init__(self, ctx, hidden_size: int, intermediate_size: int, num_attention_heads: int,
+                 num_key_value_heads: int, head_dim: int, per_layer_dim: int):
+        q_elems = num_attention_heads * head_dim
+        kv_elems = num_key_value_heads * head_dim
+        self.normed = _alloc_f16(ctx, hidden_size)
+        self.q = _alloc_f16(ctx, q_elems)
+        self.k = _alloc_f16(ctx, kv_elems)
+        self.v = _alloc_f16(ctx, kv_elems)
+        self.rq = _alloc_f32(ctx, q_elems)
+        self.vacc = _alloc_f32(ctx, q_elems)
+        self.attn_out = _alloc_f16(ctx, q_elems)
+        self.attn_resid = _alloc_f16(ctx, hidden_size)
+        self.gate = _alloc_f16(ctx, intermediate_size)
+        self.up = _alloc_f16(ctx, intermediate_size)
+        self.ffn_out = _alloc_f16(ctx, hidden_size)
+        self.ple = _alloc_f16(ctx, per_layer_dim)
+        self.ple_h = _alloc_f16(ctx, hidden_size)
+        self.ones = Buffer.from_slice(ctx, np.ones(head_dim, np.float16))
+        self.fa_pmax = _alloc_f32(ctx, num_attention_heads * MAX_FLASH_SPLITS)
+        self.fa_psum = _alloc_f32(ctx, num_attention_heads * MAX_FLASH_SPLITS)
+        self.fa_pacc = _alloc_f32(ctx, num_attention_heads * MAX_FLASH_SPLITS * head_dim)
+
+
+class BatchScratch:
+    """layer.rs:878-948: multi-row scratch sized for ``max_batch`` rows at the widest layer."""
+
+    def __init__(self, ctx, max_batch: int, hidden_size: int, intermediate_size: int, num_attention_heads: int,
+                 num_key_value_heads: int, head_dim: int, per_layer_dim: int, num_layers: int):
+        mb = max_batch
+        ple_total = mb * num_layers * per_layer_dim
+        self.max_batch = max_batch
+        self.hidden_a = _alloc_f16(ctx, mb * hidden_size)
+        self.hidden_b = _alloc_f16(ctx, mb * hidden_size)
+        self.normed = _alloc_f16(ctx, mb * hidden_size)
+        self.q = _alloc_f16(ctx, mb * num_attention_heads * head_dim)
+        self.k = _alloc_f16(ctx, mb * num_key_value_heads * head_dim)
+        self.v = _alloc_f16(ctx, mb * num_key_value_heads * head_dim)
+        self.attn_out = _alloc_f16(ctx, mb * num_attention_heads * head_dim)
+        self.rq = _alloc_f32(ctx, mb * num_attention_heads * head_dim)
+        self.vacc = _alloc_f32(ctx, mb * num_attention_heads * head_dim)
+        self.attn_resid = _alloc_f16(ctx, mb * hidden_size)
+        self.gate = _alloc_f16(ctx, mb * intermediate_size)
+        self.up = _alloc_f16(ctx, mb * intermediate_size)
+        self.ffn_out = _alloc_f16(ctx, mb * hidden_size)
+        self.ple_tok = _alloc_f16(ctx, ple_total)
+        self.ple_proj = _alloc_f16(ctx, ple_total)
+        self.ple_all = _alloc_f16(ctx, ple_total)
+        self.ple_g = _alloc_f16(ctx, mb * max(per_layer_dim, 1))
+        self.ple_slice = _alloc_f16(ctx, mb * max(per_layer_dim, 1))
+
+
+def _groupable(a: Optional[QuantWeight], b: Optional[QuantWeight]) -> bool:
+    return (a is not None and b is not None and a.ty == b.ty and a.ty != W_F16
+            and a.rows == b.rows and a.cols == b.cols)
+
+
+class TransformerLayer:
+    """layer.rs:330-873."""
+
+    def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True):
+        self.params, self.weights = params, weights
+        self.group_projections = group_projections
+        # layer.rs:515-520 reads the scalar out of shared memory at every encode; the buffer lives in device
+        # memory here, so it is fetched once.
+        self._output_scale = None
+        if weights.layer_output_scale is not None and weights.layer_output_scale.length() >= 2:
+            self._output_scale = float(weights.layer_output_scale.as_array(np.float16, 1)[0])
+
+    # ------------------------------------------------------------------ helpers
+    def _pair_matvec(self, batch, kernels: Kernels, wa: QuantWeight, wb: QuantWeight, x: Buffer, out_a: Buffer,
+                     out_b: Buffer) -> None:
+        if self.group_projections and _groupable(wa, wb):
+            kernels.matvec_quant_grouped_into(batch, wa.ty, [wa.buf, wb.buf], [x, x], F16, [out_a, out_b], F16,
+                                              wa.rows, wa.cols)
+        else:
+            wa.matvec_into(batch, kernels, x, out_a)
+            wb.matvec_into(batch, kernels, x, out_b)
+
+    def _scale_output(self, batch, kernels: Kernels, output: Buffer, count: int) -> None:
+        if self._output_scale is not None:
+            kernels.scale_in_place_gpu_into(batch, output, self._output_scale, count)
+
+    # ----------------------------------------------------- single-token decode
+    def forward_decode(self, kernels: Kernels, batch, input: Buffer, output: Buffer, position: int,
+                       scratch: ScratchBuffers, kv_cache: QuantizedKvCache, per_layer_input: Optional[Buffer] = None,
+                       n_layer_total: int = 0) -> None:
+        """layer.rs:354-523.  ``kv_cache`` is this layer's cache, or for a KV-shared layer the source layer's
+        (already written earlier in the same step)."""
+        p, w, s = self.params, self.weights, scratch
+        h, hd, n_head, n_kv, eps = p.hidden_size, p.head_dim, p.num_attention_heads, p.num_key_value_heads, p.rms_norm_eps
+        pos, seq_len = position, position + 1
+
+        # 1. input_layernorm -> Q projection -> q_norm -> RoPE
+        kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
+        w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
+        if w.q_norm is not None:
+            kernels.qk_norm_gpu_into(batch, s.q, w.q_norm, hd, n_head, eps)
+        kernels.rope_into(batch, s.q, s.q, hd, pos, p.rope_theta, p.partial_rotary_factor, n_head)
+
+        # 2. own K/V into the TurboQuant cache, then attention over the codes
+        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
+            self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
+            if w.k_norm is not None:
+                kernels.qk_norm_gpu_into(batch, s.k, w.k_norm, hd, n_kv, eps)
+            kernels.rms_norm_into(batch, s.v, s.ones, s.v, hd, n_kv, eps)   # V: RMS norm with unit weight
+            kernels.rope_into(batch, s.k, s.k, hd, pos, p.rope_theta, p.partial_rotary_factor, n_kv)
+            kv_cache.write_kv_gpu_into(batch, kernels, s.k, s.v, position, 1)
+        kv_cache.fused_attention_into(batch, kernels, s.q, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
+                                      p.sliding_window)
+
+        # 3. output projection -> post_attention_norm + residual #1
+        w.attn_output.matvec_into(batch, kernels, s.attn_out, s.ffn_out)
+        kernels.rms_norm_add_into(batch, s.ffn_out, w.attn_post_norm, input, s.attn_resid, h, 1, eps)
+
+        # 4. GeGLU feed-forward -> post_feedforward_norm + residual #2
+        inter = p.intermediate_size
+        kernels.rms_norm_into(batch, s.attn_resid, w.ffn_norm, s.normed, h, 1, eps)
+        self._pair_matvec(batch, kernels, w.ffn_gate, w.ffn_up, s.normed, s.gate, s.up)
+        kernels.gelu_mul_into(batch, s.gate, s.up, s.gate, inter)
+        w.ffn_down.matvec_into(batch, kernels, s.gate, s.ffn_out)
+        kernels.rms_norm_add_into(batch, s.ffn_out, w.ffn_post_norm, s.attn_resid, output, h, 1, eps)
+
+        # 5. per-layer input injection -> residual #3
+        if (w.per_layer_inp_gate is not None and w.per_layer_proj is not None and w.per_layer_post_norm is not None
+                and per_layer_input is not None):
+            pld = p.per_layer_dim
+            batch.blit_copy(per_layer_input, p.layer_idx * pld * 2, s.ple, 0, pld * 2)
+            w.per_layer_inp_gate.matvec_into(batch, kernels, output, s.ple_h)
+            kernels.gelu_mul_into(batch, s.ple_h, s.ple, s.ple_h, pld)
+            w.per_layer_proj.matvec_into(batch, kernels, s.ple_h, s.ffn_out)
+            kernels.rms_norm_into(batch, s.ffn_out, w.per_layer_post_norm, s.normed, h, 1, eps)
+            kernels.residual_add_into(batch, output, s.normed, output, h)
+
+        # 6. per-layer output scale
+        self._scale_output(batch, kernels, output, h)
+
+    # ------------------------------------------------ shared multi-row tail
+    def _attention_tail(self, kernels: Kernels, batch, rows: int, input: Buffer, output: Buffer, bs: BatchScratch,
+                        ple_all) -> None:
+        """Everything after attention, identical in layer.rs:640-716 and layer.rs:808-870."""
+        p, w = self.params, self.weights
+        h, eps, inter = p.hidden_size, p.rms_norm_eps, p.intermediate_size
+        w.attn_output.matmul_nt_into(batch, kernels, bs.attn_out, bs.ffn_out, rows)
+        kernels.rms_norm_add_into(batch, bs.ffn_out, w.attn_post_norm, input, bs.attn_resid, h, rows, eps)
+        kernels.rms_norm_into(batch, bs.attn_resid, w.ffn_norm, bs.normed, h, rows, eps)
+        w.ffn_gate.matmul_nt_into(batch, kernels, bs.normed, bs.gate, rows)
+        w.ffn_up.matmul_nt_into(batch, kernels, bs.normed, bs.up, rows)
+        kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
+        w.ffn_down.matmul_nt_into(batch, kernels, bs.gate, bs.ffn_out, rows)
+        kernels.rms_norm_add_into(batch, bs.ffn_out, w.ffn_post_norm, bs.attn_resid, output, h, rows, eps)
+        if (w.per_layer_inp_gate is not None and w.per_layer_proj is not None and w.per_layer_post_norm is not None
+                and ple_all is not None):
+            ple_buf, n_layer_total = ple_all
+            pld = p.per_layer_dim
+            kernels.gather_strided_f16_into(batch, ple_buf, bs.ple_slice, n_layer_total * pld, p.layer_idx * pld, pld,
+                                            rows)
+            w.per_layer_inp_gate.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
+            kernels.gelu_mul_into(batch, bs.ple_g, bs.ple_slice, bs.ple_g, rows * pld)
+            w.per_layer_proj.matmul_nt_into(batch, kernels, bs.ple_g, bs.ffn_out, rows)
+            kernels.rms_norm_add_into(batch, bs.ffn_out, w.per_layer_post_norm, output, output, h, rows, eps)
+        self._scale_output(batch, kernels, output, rows * h)
+
+    def _check_rows(self, rows: int, bs: BatchScratch) -> None:
+        if rows == 0 or rows > bs.max_batch:
+            raise InvalidArgument(f"rows {rows} outside 1..={bs.max_batch} (BatchScratch capacity)")
+
+    # -------------------------------------- n consecutive rows of one sequence
+    def forward_batch(self, kernels: Kernels, batch, n_rows: int, start_pos: int, input: Buffer, output: Buffer,
+                      bs: BatchScratch, ones: Buffer, kv_cache: QuantizedKvCache, ple_all=None) -> None:
+        """layer.rs:542-718: rows at positions ``start_pos .. start_pos + n_rows``; ``ple_all`` is
+        ``(buffer [n_rows, n_layer_total, per_layer_dim] f16, n_layer_total)``."""
+        self._check_rows(n_rows, bs)
+        p, w = self.params, self.weights
+        rows, h, hd, n_head, n_kv, eps = n_rows, p.hidden_size, p.head_dim, p.num_attention_heads, \
+            p.num_key_value_heads, p.rms_norm_eps
+        kv_len = start_pos + n_rows
+
+        kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
+        if w.q_norm is not None:
+            kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
+        kernels.rope_batch_into(batch, bs.q, start_pos, p.rope_theta, hd, n_head, rows, p.partial_rotary_factor)
+
+        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
+            w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
+            w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
+            if w.k_norm is not None:
+                kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
+            kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
+            kernels.rope_batch_into(batch, bs.k, start_pos, p.rope_theta, hd, n_kv, rows, p.partial_rotary_factor)
+            kv_cache.write_kv_gpu_into(batch, kernels, bs.k, bs.v, start_pos, n_rows)
+
+        kv_cache.fused_attention_batch_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
+                                            n_head, p.sliding_window)
+        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)
+
+    # ---------------------------- one row per independent lane (continuous batching)
+    def forward_decode_batch_turbo(self, batch, kernels: Kernels, n_lanes: int, positions: Buffer, input: Buffer,
+                                   output: Buffer, bs: BatchScratch, ones: Buffer, pool: QuantizedUnifiedKvPool,
+                                   ple_all=None) -> None:
+        """layer.rs:731-873: ``positions`` is a device ``[n_lanes]`` u32 buffer shared by rope, the KV scatter
+        and attention."""
+        self._check_rows(n_lanes, bs)
+        p, w = self.params, self.weights
+        rows, h, hd, n_head, n_kv, eps = n_lanes, p.hidden_size, p.head_dim, p.num_attention_heads, \
+            p.num_key_value_heads, p.rms_norm_eps
+
+        kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
+        if w.q_norm is not None:
+            kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
+        kernels.rope_batch_decode_into(batch, bs.q, positions, p.rope_theta, hd, n_head, rows, p.partial_rotary_factor)
+
+        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
+            w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
+            w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
+            if w.k_norm is not None:
+                kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
+            kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
+            kernels.rope_batch_decode_into(batch, bs.k, positions, p.rope_theta, hd, n_kv, rows,
+                                           p.partial_rotary_factor)
+            pool.write_kv_into(batch, kernels, bs.k, bs.v, positions, n_lanes)
+
+        pool.attention_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, positions, n_head, p.sliding_window,
+                            n_lanes)
+        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)

@@ -72,3 +72,39 @@ DECODER_LAYER = (
 def kv_rows(t: int, n_kv: int, head_dim: int, g: np.random.Generator) -> np.ndarray:
     """K or V rows [t, n_kv, head_dim] as f16 N(0, 1)."""
     return g.standard_normal((t, n_kv, head_dim), dtype=np.float32).astype(np.float16)
+
+
+def decoder_layer_tensors(hidden: int, inter: int, n_head: int, n_kv: int, head_dim: int, per_layer_dim: int,
+                          g: np.random.Generator, attn_fmt: str = "q4_0", ffn_fmt: str = "tq2_0",
+                          output_scale: float | None = None, kv_shared: bool = False) -> dict:
+    """Every tensor of one decoder layer (names of local-engine/src/layer.rs:310-328): projections as
+    ``(format, rows, cols, payload bytes)``, norm vectors as f16 arrays c * (1 + N(0, 0.1)) with c = 1 except
+    for q_norm / k_norm, where c = head_dim^-1/4: normalised q and k then have length head_dim^1/4, so the
+    unscaled scores q . k of attention are about N(0, 1) rather than N(0, head_dim)."""
+    def proj(fmt, rows, cols):
+        return (fmt, rows, cols, weights(fmt, rows, cols, g))
+
+    def norm(n, c=1.0):
+        return (np.float32(c) * (np.float32(1.0) + np.float32(0.1) * g.standard_normal(n, dtype=np.float32))) \
+            .astype(np.float16)
+
+    qk_scale = float(head_dim) ** -0.25
+
+    t = {
+        "attn_norm": norm(hidden), "attn_q": proj(attn_fmt, n_head * head_dim, hidden),
+        "q_norm": norm(head_dim, qk_scale), "attn_output": proj(attn_fmt, hidden, n_head * head_dim),
+        "attn_post_norm": norm(hidden), "ffn_norm": norm(hidden),
+        "ffn_gate": proj(ffn_fmt, inter, hidden), "ffn_up": proj(ffn_fmt, inter, hidden),
+        "ffn_down": proj(ffn_fmt, hidden, inter), "ffn_post_norm": norm(hidden),
+    }
+    if not kv_shared:
+        t["attn_k"] = proj(attn_fmt, n_kv * head_dim, hidden)
+        t["attn_v"] = proj(attn_fmt, n_kv * head_dim, hidden)
+        t["k_norm"] = norm(head_dim, qk_scale)
+    if per_layer_dim:
+        t["per_layer_inp_gate"] = proj(attn_fmt, per_layer_dim, hidden)
+        t["per_layer_proj"] = proj(attn_fmt, hidden, per_layer_dim)
+        t["per_layer_post_norm"] = norm(hidden)
+    if output_scale is not None:
+        t["layer_output_scale"] = np.array([output_scale], np.float16)
+    return t
