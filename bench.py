@@ -344,6 +344,125 @@ def bench_glue(pkg, ctx, K, steps, warmup):
     return res
 
 
+def fill_kv(pkg, ctx, K, cache, lanes, T, g):
+    """Fill a KV cache / lane pool ([lanes * T] rows) with TurboQuant codes: lane 0 encoded on the GPU from f16
+    N(0, 1) rows, the other lanes rotations of it (distinct addresses and contents)."""
+    hd, nkv, bits = cache.head_dim, cache.n_kv_heads, cache.bits
+    cb = hd * bits // 8
+    batch = pkg.CommandBatch(ctx)
+    for codes, norms in ((cache.keys_q, cache.key_norms), (cache.values_q, cache.value_norms)):
+        for t0 in range(0, T, 8192):
+            n = min(8192, T - t0)
+            rows = pkg.Buffer.from_slice(ctx, pkg.synth.kv_rows(n, nkv, hd, g))
+            K.encode_kv_turboquant_into(batch, rows, cache.levels, cache.signs, codes, norms, hd, nkv, n, bits, t0, 0)
+            batch.commit_and_wait()
+    for l in range(1, lanes):
+        r = (l * 997) % T
+        for buf, unit in ((cache.keys_q, nkv * cb), (cache.key_norms, nkv * 2), (cache.values_q, nkv * cb),
+                          (cache.value_norms, nkv * 2)):
+            batch.blit_copy(buf, r * unit, buf, l * T * unit, (T - r) * unit)
+            if r:
+                batch.blit_copy(buf, 0, buf, (l * T + T - r) * unit, r * unit)
+    batch.commit_and_wait()
+
+
+def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3):
+    """Whole decoder layers end to end (norms, Q/K/V projections, RoPE, KV encode, attention over the tq2 cache,
+    output projection, GeGLU feed-forward, per-layer input injection) at hidden 2048, FFN 8192, 8 query heads over
+    1 KV head of 256, Q4_0 attention and TQ2_0 feed-forward weights, context T.  A step runs `n_layers` distinct
+    layers back to back (18.9 MB of weights and a cache of their own each, so nothing is served from the last-level
+    cache twice), the output of one feeding the next, as a model's decode step does.  `which`: "single" (one
+    sequence, one token per step) and / or "lanes" (continuous batching, one token of each of `lanes` sequences)."""
+    L = pkg.layer
+    dims = dict(hidden_size=2048, intermediate_size=8192, num_attention_heads=8, num_key_value_heads=1, head_dim=256)
+    pld = 256
+    g = pkg.synth.rng(12, 0)
+
+    def make_layer(i):
+        t = pkg.synth.decoder_layer_tensors(2048, 8192, 8, 1, 256, pld, g)
+        params = L.LayerParams(layer_idx=i, per_layer_dim=pld, rope_theta=1e6, **dims)
+        return L.TransformerLayer(params, L.LayerWeights.from_host(ctx, t))
+
+    res = {"context": T}
+    scratch = L.ScratchBuffers(ctx, 2048, 8192, 8, 1, 256, pld)
+    batch = pkg.CommandBatch(ctx)
+    kv_bytes = T * (2 * 64 + 4)
+    if "single" in which:
+        res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes)
+    if "lanes" in which:
+        res["lanes"] = _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g,
+                                     kv_bytes)
+    return res
+
+
+def _layer_weight_bytes(pkg, layer):
+    return sum(w.device_bytes() for w in vars(layer.weights).values() if isinstance(w, pkg.QuantWeight))
+
+
+def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes):
+    pld = 256
+    layers = [make_layer(i) for i in range(n_layers)]
+    wbytes = _layer_weight_bytes(pkg, layers[0])
+    caches = []
+    for i in range(n_layers):
+        c = pkg.QuantizedKvCache(ctx, 1, 256, T)
+        fill_kv(pkg, ctx, K, c, 1, T, pkg.synth.rng(12, 100 + i))
+        caches.append(c)
+    hidden = [pkg.Buffer.from_slice(ctx, g.standard_normal(2048, dtype=np.float32).astype(np.float16)),
+              pkg.Buffer.empty(ctx, 2048 * 2)]
+    x0 = pkg.Buffer.from_slice(ctx, hidden[0].as_array(np.float16, 2048))
+    ple = pkg.Buffer.from_slice(ctx, g.standard_normal(n_layers * pld, dtype=np.float32).astype(np.float16))
+
+    def step_single():
+        batch.blit_copy(x0, 0, hidden[0], 0, 4096)
+        for i, layer in enumerate(layers):
+            layer.forward_decode(K, batch, hidden[i & 1], hidden[(i + 1) & 1], T - 1, scratch, caches[i], ple, n_layers)
+
+    d0 = batch.dispatch_count()
+    step_single()
+    per_layer = (batch.dispatch_count() - d0 - 1) // n_layers
+    wall, ev = time_steps(pkg, ctx, step_single, max(steps, 20), warmup)
+    out = hidden[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
+    if not np.isfinite(out).all():
+        raise RuntimeError("decode step produced non-finite hidden state")
+    return {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
+                     "dispatches_per_layer": per_layer,
+                     "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
+                     "gbs_events": (wbytes + kv_bytes) / (ev / n_layers) * 1e-6,
+                     "tokens_per_s_35_layers": 1.0 / (ev * 1e-3 / n_layers * 35)}
+
+
+def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g, kv_bytes):
+    pld = 256
+    layers = [make_layer(i) for i in range(lane_layers)]
+    wbytes = _layer_weight_bytes(pkg, layers[0])
+    pools = []
+    for i in range(lane_layers):
+        pool = pkg.QuantizedUnifiedKvPool(ctx, lanes, T, 1, 256, 2, 0)
+        fill_kv(pkg, ctx, K, pool, lanes, T, pkg.synth.rng(12, 200 + i))
+        pools.append(pool)
+    bs = pkg.layer.BatchScratch(ctx, lanes, 2048, 8192, 8, 1, 256, pld, lane_layers)
+    xin = pkg.Buffer.from_slice(ctx, g.standard_normal(lanes * 2048, dtype=np.float32).astype(np.float16))
+    ple_all = pkg.Buffer.from_slice(ctx, g.standard_normal(lanes * lane_layers * pld, dtype=np.float32).astype(np.float16))
+    positions = pkg.Buffer.from_slice(ctx, np.full(lanes, T - 1, np.uint32))
+
+    def step_lanes():
+        batch.blit_copy(xin, 0, bs.hidden_a, 0, lanes * 4096)
+        bufs = (bs.hidden_a, bs.hidden_b)
+        for i, layer in enumerate(layers):
+            layer.forward_decode_batch_turbo(batch, K, lanes, positions, bufs[i & 1], bufs[(i + 1) & 1], bs, scratch.ones,
+                                             pools[i], (ple_all, lane_layers))
+
+    wall, ev = time_steps(pkg, ctx, step_lanes, steps, warmup)
+    out = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
+    if not np.isfinite(out).all():
+        raise RuntimeError("batched decode step produced non-finite hidden state")
+    return {"lanes": lanes, "layers_per_step": lane_layers, "us_per_layer_events": ev * 1e3 / lane_layers,
+                    "us_per_layer_wall": wall * 1e3 / lane_layers, "kv_bytes_per_layer": lanes * kv_bytes,
+                    "gbs_events": (wbytes + lanes * kv_bytes) / (ev / lane_layers) * 1e-6,
+                    "tokens_per_s_35_layers": lanes / (ev * 1e-3 / lane_layers * 35)}
+
+
 def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
     """CPU restatement of the reference path on the host cores: bounded sample of the same workload."""
     from oracle import oracle as orc
@@ -372,7 +491,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue",
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -444,6 +563,11 @@ def main():
     if "glue" in legs:
         extra["layer_glue_kernels"] = bench_glue(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] glue:", extra["layer_glue_kernels"])
+
+    if legs & {"decode", "lanes"}:
+        which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else [])
+        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which)
+        log("[bench] decode step:", extra["decode_step_end_to_end"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
     line = {

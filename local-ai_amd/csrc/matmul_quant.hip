@@ -244,7 +244,8 @@ __device__ __forceinline__ uint32_t clamp_h2(uint32_t w, float lo, float hi) {
 
 template <int FMT, int ADT, int CDT, int BM>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
-                                                         uint32_t M, uint32_t K, uint32_t N, ClipArgs clip) {
+                                                         uint32_t M, uint32_t K, uint32_t N, ClipArgs clip,
+                                                         float* __restrict__ partial, uint32_t steps_per_split) {
     constexpr int TI = BM / 32;                              // 16-row MFMA tiles per wave along M (2 x 2 waves)
     constexpr int NCH = BM / 16;                             // 8-element activation chunks staged per thread
     __shared__ __align__(16) _Float16 As[BM * LDK];
@@ -254,6 +255,13 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const uint32_t b_ld_row = tid >> 1, b_ld_k = (tid & 1) * 64;
     const uint32_t b_row = n0 + b_ld_row < N ? n0 + b_ld_row : N - 1;   // past-the-end rows re-read the last (never stored)
+
+    // Split k (gridDim.z > 1, few output tiles): this workgroup multiplies k steps [kt_begin, kt_end) only and leaves
+    // its f32 tile in `partial[z]`; splitk_reduce_kernel sums the splits.  Steps at or past Kend are staged as zeros.
+    const uint32_t nk = (K + BK - 1) / BK;
+    const uint32_t kt_begin = blockIdx.z * steps_per_split;
+    const uint32_t kt_end = kt_begin + steps_per_split < nk ? kt_begin + steps_per_split : nk;
+    const uint32_t Kend = kt_end * BK < K ? kt_end * BK : K;
 
     f32x4 acc[TI][4];
 #pragma unroll
@@ -284,14 +292,14 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
             uint4 v = convert_a8<ADT>(ra[set][i]);
             if (clip.enabled) v = make_uint4(clamp_h2(v.x, clip.in_lo, clip.in_hi), clamp_h2(v.y, clip.in_lo, clip.in_hi),
                                              clamp_h2(v.z, clip.in_lo, clip.in_hi), clamp_h2(v.w, clip.in_lo, clip.in_hi));
-            if (kt * BK + BK > K && kt * BK + 8 * (c & 15) >= K) v = make_uint4(0u, 0u, 0u, 0u);   // only in a partial last k step
+            if (kt * BK + BK > Kend && kt * BK + 8 * (c & 15) >= Kend) v = make_uint4(0u, 0u, 0u, 0u);   // only past the last k step
             *reinterpret_cast<uint4*>(&As[(c >> 4) * LDK + 8 * (c & 15)]) = v;
         }
         if constexpr (FMT == kTQ2) {
 #pragma unroll
             for (int f = 0; f < 4; f++) {
                 uint32_t w[8];
-                convert_bt(w, rbt[set], f, kt * BK < K);
+                convert_bt(w, rbt[set], f, kt * BK < Kend);
                 store_words<8>(&Bs[b_ld_row * LDK + 32 * f + 16 * (tid & 1)], w);
             }
         } else {
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const uint32_t k0 = kt * BK + b_ld_k + 32 * i;
-                convert_b<FMT>(f, rb[set][i], k0, k0 < K);
+                convert_b<FMT>(f, rb[set][i], k0, k0 < Kend);
                 store_words<16>(&Bs[b_ld_row * LDK + b_ld_k + 32 * i], f);
             }
         }
@@ -323,10 +331,9 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
     // Two k steps per trip (the register sets alternate without copies).  Every trip issues the same loads in the same
     // order, also past the end of K (those re-read the last step and are staged as zeros): a fixed number of loads in
     // flight lets the waits before staging leave the newer set outstanding.
-    const uint32_t nk = (K + BK - 1) / BK;
-    load_step(0, 0);
-    load_step(1, 1);
-    for (uint32_t kt = 0; kt < nk; kt += 2) {
+    load_step(0, kt_begin);
+    load_step(1, kt_begin + 1);
+    for (uint32_t kt = kt_begin; kt < kt_end; kt += 2) {
         stage_step(0, kt);
         __syncthreads();
         load_step(0, kt + 2);
@@ -345,6 +352,14 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
         for (int j = 0; j < 4; j++) {
             const uint32_t n = n0 + wn * 64 + j * 16 + (lane & 15);
             if (n >= N) continue;
+            if (partial) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const uint32_t m = m0 + wm * (BM / 2) + i * 16 + (lane >> 4) * 4 + r;
+                    if (m < M) partial[((size_t)blockIdx.z * M + m) * N + n] = acc[i][j][r];
+                }
+                continue;
+            }
             const float bias = (clip.enabled && clip.bias) ? lh_h2f(clip.bias[n]) : 0.0f;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
@@ -354,6 +369,21 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
                 if (m < M) store_elem<CDT>(C, (size_t)m * N + n, v);
             }
         }
+}
+
+// Sum of the split-k partial tiles, with the bias / clamp of the clipped linear layer, stored in the output type.
+template <int CDT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ C, uint32_t M, uint32_t N,
+                                                           uint32_t splits, ClipArgs clip) {
+    const size_t total = (size_t)M * N, i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float v = 0.0f;
+    for (uint32_t z = 0; z < splits; z++) v += partial[(size_t)z * total + i];
+    if (clip.enabled) {
+        const float bias = clip.bias ? lh_h2f(clip.bias[i % N]) : 0.0f;
+        v = fminf(fmaxf(v + bias, clip.out_lo), clip.out_hi);
+    }
+    store_elem<CDT>(C, i, v);
 }
 
 // ---- 128 x 128 tiles for large M: f16 activations (converted once by a pre-pass when they arrive as bf16 / f32),
@@ -574,14 +604,33 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
                 return LH_OK;
             }
         }
+        const uint32_t nk = (k + BK - 1) / BK;
         if (force_bm == 128 || (force_bm == 0 && tiles128 >= 2ull * (uint64_t)cus)) {
             const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk);
         } else {
-            const dim3 grid((n + BN - 1) / BN, (m + 63) / 64);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip);
+            // Few output tiles (a decode batch of some tens of rows): split k so that every CU gets a workgroup, at least
+            // two k steps per split, partial tiles within the lower half of the context workspace.
+            static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
+            const uint64_t tiles64 = (uint64_t)((n + BN - 1) / BN) * ((m + 63) / 64);
+            uint32_t splits = 1;
+            if (!no_splitk && tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
+                splits = (uint32_t)std::min<uint64_t>(nk / 2, ((uint64_t)cus + tiles64 - 1) / tiles64);
+                const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * n * 4);
+                splits = (uint32_t)std::min<uint64_t>(splits, fit);
+            }
+            const uint32_t steps = splits > 1 ? (nk + splits - 1) / splits : nk;
+            if (splits > 1) splits = (nk + steps - 1) / steps;
+            float* partial = splits > 1 ? static_cast<float*>(ctx->workspace) : nullptr;
+            const dim3 grid((n + BN - 1) / BN, (m + 63) / 64, splits > 1 ? splits : 1);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps);
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps);
+            if (splits > 1) {
+                const uint32_t rgrid = (uint32_t)(((size_t)m * n + 255) / 256);
+                if (ct == LH_F32) hipLaunchKernelGGL((splitk_reduce_kernel<LH_F32>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, splits, clip);
+                else hipLaunchKernelGGL((splitk_reduce_kernel<LH_F16>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, splits, clip);
+            }
         }
     } else {
         if constexpr (FMT != kF16W) {

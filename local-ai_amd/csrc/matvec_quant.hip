@@ -39,6 +39,10 @@ struct MatvecProblem {
 struct MatvecBase {
     MatvecProblem p;
     uint32_t xstride, ystride;   // bytes
+    // A pair of unrelated problems (K and V, gate and up) also travels here, so the common grouped launch
+    // needs no descriptor upload ahead of it.
+    MatvecProblem second = {nullptr, nullptr, nullptr};
+    uint32_t pair = 0;
 };
 
 // ---- per-lane activation registers for one unit column -------------------------
@@ -231,6 +235,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         const uint64_t seg_end64 = (uint64_t)(prob + 1) * steps_per_problem;
         const uint32_t s_end = (uint32_t)((g1 < seg_end64 ? g1 : seg_end64) - (uint64_t)prob * steps_per_problem);
         const MatvecProblem pb = problems ? problems[prob]
+                                 : (single.pair && prob == 1) ? single.second
                                           : MatvecProblem{single.p.matrix, (const char*)single.p.vector + (size_t)prob * single.xstride,
                                                           (char*)single.p.output + (size_t)prob * single.ystride};
         // this wave's contiguous share of [s_begin, s_end)
@@ -541,7 +546,10 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     // kernel that still reads the previous set).
     MatvecBase single{MatvecProblem{(const uint8_t*)matrices[0]->ptr, vectors[0]->ptr, outputs[0]->ptr}, 0, 0};
     MatvecProblem* dev_desc = nullptr;
-    if (count > 1) {
+    if (count == 2) {
+        single.second = MatvecProblem{(const uint8_t*)matrices[1]->ptr, vectors[1]->ptr, outputs[1]->ptr};
+        single.pair = 1;
+    } else if (count > 2) {
         const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
         if (desc_bytes > ctx->workspace_bytes / 4)
             return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u problems exceed the descriptor area", op, count);

@@ -49,6 +49,10 @@ struct Tq2Problem {
 struct Tq2Base {
     Tq2Problem p;
     uint32_t xstride, ystride;   // bytes
+    // A pair of unrelated problems (gate and up) also travels here, so the common grouped launch needs no
+    // descriptor upload ahead of it.
+    Tq2Problem second = {nullptr, nullptr, nullptr};
+    uint32_t pair = 0;
 };
 
 __device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
@@ -136,6 +140,7 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
         grp = it.grp;
         tile = splitk ? it.sip : it.sip * nwaves + wave;
         if (problems) pb = problems[it.prob];
+        else if (single.pair && it.prob == 1) pb = single.second;
         else pb = Tq2Problem{single.p.matrix, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
                              (char*)single.p.output + (size_t)it.prob * single.ystride};
     };
@@ -324,7 +329,10 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
     Tq2Problem* dev = nullptr;
-    if (count > 1 && !strided) {
+    if (count == 2 && !strided) {
+        single.second = Tq2Problem{(const uint8_t*)matrices[1], vectors[1], outputs[1]};
+        single.pair = 1;
+    } else if (count > 2 && !strided) {
         const size_t bytes = (size_t)count * sizeof(Tq2Problem);
         if (bytes > ctx->workspace_bytes / 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems exceed the descriptor area", count);
         Tq2Problem* host = (Tq2Problem*)malloc(bytes);

@@ -148,9 +148,10 @@ def _groupable(a: Optional[QuantWeight], b: Optional[QuantWeight]) -> bool:
 class TransformerLayer:
     """layer.rs:330-873."""
 
-    def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True):
+    def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True,
+                 fuse_norm_rope: bool = True):
         self.params, self.weights = params, weights
-        self.group_projections = group_projections
+        self.group_projections, self.fuse_norm_rope = group_projections, fuse_norm_rope
         # layer.rs:515-520 reads the scalar out of shared memory at every encode; the buffer lives in device
         # memory here, so it is fetched once.
         self._output_scale = None
@@ -166,6 +167,17 @@ class TransformerLayer:
         else:
             wa.matvec_into(batch, kernels, x, out_a)
             wb.matvec_into(batch, kernels, x, out_b)
+
+    def _norm_rope(self, batch, kernels: Kernels, qk: Buffer, norm_w: Optional[Buffer], heads: int, pos: int) -> None:
+        """layer.rs:393-404 / 415-428: per-head RMS norm (when the layer has one) then RoPE, in place."""
+        p = self.params
+        if norm_w is not None and self.fuse_norm_rope and kernels.qk_norm_rope_available(p.head_dim):
+            kernels.qk_norm_rope_into(batch, qk, qk, norm_w, p.head_dim, heads, p.rms_norm_eps, pos, p.rope_theta,
+                                      p.partial_rotary_factor)
+            return
+        if norm_w is not None:
+            kernels.qk_norm_gpu_into(batch, qk, norm_w, p.head_dim, heads, p.rms_norm_eps)
+        kernels.rope_into(batch, qk, qk, p.head_dim, pos, p.rope_theta, p.partial_rotary_factor, heads)
 
     def _scale_output(self, batch, kernels: Kernels, output: Buffer, count: int) -> None:
         if self._output_scale is not None:
@@ -184,17 +196,13 @@ class TransformerLayer:
         # 1. input_layernorm -> Q projection -> q_norm -> RoPE
         kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
         w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
-        if w.q_norm is not None:
-            kernels.qk_norm_gpu_into(batch, s.q, w.q_norm, hd, n_head, eps)
-        kernels.rope_into(batch, s.q, s.q, hd, pos, p.rope_theta, p.partial_rotary_factor, n_head)
+        self._norm_rope(batch, kernels, s.q, w.q_norm, n_head, pos)
 
         # 2. own K/V into the TurboQuant cache, then attention over the codes
         if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
             self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
-            if w.k_norm is not None:
-                kernels.qk_norm_gpu_into(batch, s.k, w.k_norm, hd, n_kv, eps)
             kernels.rms_norm_into(batch, s.v, s.ones, s.v, hd, n_kv, eps)   # V: RMS norm with unit weight
-            kernels.rope_into(batch, s.k, s.k, hd, pos, p.rope_theta, p.partial_rotary_factor, n_kv)
+            self._norm_rope(batch, kernels, s.k, w.k_norm, n_kv, pos)
             kv_cache.write_kv_gpu_into(batch, kernels, s.k, s.v, position, 1)
         kv_cache.fused_attention_into(batch, kernels, s.q, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
                                       p.sliding_window)

@@ -149,12 +149,12 @@ def test_forward_decode_sliding_window_ring_and_shared_kv(pkg, gpu, oracle):
     _same_cache(cache, kv, cap)
 
 
-def test_grouped_projections_change_nothing(pkg, gpu, oracle):
+def test_grouped_and_fused_dispatches_change_nothing(pkg, gpu, oracle):
     ctx, kernels = gpu
     g = pkg.synth.rng(902, 0)
     dims = _dims()
     dev, _, _ = _make(pkg, gpu, g, dims)
-    plain = pkg.layer.TransformerLayer(dev.params, dev.weights, group_projections=False)
+    plain = pkg.layer.TransformerLayer(dev.params, dev.weights, group_projections=False, fuse_norm_rope=False)
     x = g.standard_normal(512, dtype=np.float32).astype(np.float16)
     res = []
     for layer in (dev, plain):
@@ -163,7 +163,7 @@ def test_grouped_projections_change_nothing(pkg, gpu, oracle):
         scratch = pkg.layer.ScratchBuffers(ctx, 512, 1024, 4, 1, 256, 0)
         inp, out = pkg.Buffer.from_slice(ctx, x), pkg.Buffer.empty(ctx, 1024)
         batch = pkg.CommandBatch(ctx)
-        layer.forward_decode(kernels, batch, inp, out, 0, scratch, cache)
+        layer.forward_decode(kernels, batch, inp, out, 5, scratch, cache)
         batch.commit_and_wait()
         res.append((out.as_array(np.uint16, 512), cache.keys_q.as_array(np.uint8), cache.values_q.as_array(np.uint8)))
     for a, b in zip(*res):

@@ -66,6 +66,30 @@ def test_mfma_matmul_tile_boundaries(pkg, gpu, oracle, fmt):
         refgen.assert_close(cb.as_array(np.float32), want_unrounded, 1e-2, f"{fmt} mfma {m}x{k}x{n} vs f32 weights")
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_mfma_matmul_split_k(pkg, gpu, oracle, fmt):
+    """A decode batch of some tens of rows against the layer's projections: few output tiles, so the k range is split
+    over several workgroups whose partial tiles a second kernel sums -- even and odd numbers of k steps per split, a
+    ragged last split, ragged M and N, f16 and f32 outputs."""
+    ctx, K = gpu
+    shapes = ((64, 2048, 2048, "f16"), (33, 2048, 8192, "f16"), (64, 8192, 2048, "f16"), (100, 1280, 200, "f32"),
+              (17, 2304, 130, "f32"))
+    for (m, k, n, ct) in shapes:
+        print(f"case {fmt} m={m} k={k} n={n} out={ct}", flush=True)
+        raw = payload(fmt, n, k, 0x5117 + m)
+        deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+        a16 = (pkg.synth.rng(4, m + k).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+        want = oracle.matmul_nt_f32(a16.astype(np.float32), deq)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k)
+        ab = pkg.Buffer.from_slice(ctx, a16)
+        cb = pkg.Buffer.empty(ctx, m * n * (4 if ct == "f32" else 2))
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32 if ct == "f32" else pkg.F16, m)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float32) if ct == "f32" else cb.as_array(np.float16).astype(np.float32)
+        refgen.assert_close(got, want, 1e-3 if ct == "f32" else 2e-3, f"{fmt} split k {m}x{k}x{n}")
+
+
 @pytest.mark.parametrize("adt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_large_tiles(pkg, gpu, oracle, fmt, adt):
