@@ -425,8 +425,39 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
     out = hidden[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("decode step produced non-finite hidden state")
+    # The same step through the position-in-a-buffer path (one lane of forward_decode_batch_turbo), recorded once into a
+    # graph and replayed: one host call per step instead of one per dispatch.
+    L = pkg.layer
+    pools = []
+    for i in range(n_layers):
+        pool = pkg.QuantizedUnifiedKvPool(ctx, 1, T, 1, 256, 2, 0)
+        for name in ("keys_q", "values_q", "key_norms", "value_norms"):
+            src = getattr(caches[i], name)
+            batch.blit_copy(src, 0, getattr(pool, name), 0, src.length())
+        pools.append(pool)
+    batch.commit_and_wait()
+    bs = L.BatchScratch(ctx, 1, 2048, 8192, 8, 1, 256, pld, n_layers)
+    positions = pkg.Buffer.from_slice(ctx, np.full(1, T - 1, np.uint32))
+    gbufs = (bs.hidden_a, bs.hidden_b)
+
+    def encode_lane_step(b):
+        b.blit_copy(x0, 0, bs.hidden_a, 0, 4096)
+        for i, layer in enumerate(layers):
+            layer.forward_decode_batch_turbo(b, K, 1, positions, gbufs[i & 1], gbufs[(i + 1) & 1], bs, scratch.ones, pools[i],
+                                             (ple, n_layers))
+
+    batch.begin_capture()
+    encode_lane_step(batch)
+    graph = batch.end_capture()
+    gwall, gev = time_steps(pkg, ctx, graph.launch, max(steps, 20), warmup)
+    gout = gbufs[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
+    if not np.isfinite(gout).all() or np.abs(gout - out).max() > 0.05 * max(1.0, np.abs(out).max()):
+        raise RuntimeError("graph replay of the decode step disagrees with the eager step")
     return {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
                      "dispatches_per_layer": per_layer,
+                     "graph_us_per_layer_events": gev * 1e3 / n_layers, "graph_us_per_layer_wall": gwall * 1e3 / n_layers,
+                     "graph_dispatches_per_layer": graph.dispatch_count() // n_layers,
+                     "graph_tokens_per_s_35_layers": 1.0 / (gev * 1e-3 / n_layers * 35),
                      "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
                      "gbs_events": (wbytes + kv_bytes) / (ev / n_layers) * 1e-6,
                      "tokens_per_s_35_layers": 1.0 / (ev * 1e-3 / n_layers * 35)}
@@ -457,8 +488,18 @@ def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer,
     out = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("batched decode step produced non-finite hidden state")
+    batch.commit_and_wait()
+    batch.begin_capture()
+    step_lanes()
+    graph = batch.end_capture()
+    gwall, gev = time_steps(pkg, ctx, graph.launch, steps, warmup)
+    gout = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
+    if not np.array_equal(gout, out):
+        raise RuntimeError("graph replay of the batched decode step disagrees with the eager step")
     return {"lanes": lanes, "layers_per_step": lane_layers, "us_per_layer_events": ev * 1e3 / lane_layers,
                     "us_per_layer_wall": wall * 1e3 / lane_layers, "kv_bytes_per_layer": lanes * kv_bytes,
+                    "graph_us_per_layer_events": gev * 1e3 / lane_layers,
+                    "graph_tokens_per_s_35_layers": lanes / (gev * 1e-3 / lane_layers * 35),
                     "gbs_events": (wbytes + lanes * kv_bytes) / (ev / lane_layers) * 1e-6,
                     "tokens_per_s_35_layers": lanes / (ev * 1e-3 / lane_layers * 35)}
 

@@ -107,6 +107,22 @@ LH_API int lh_batch_commit_and_wait(lh_batch* batch);
 LH_API int lh_batch_submit_and_renew(lh_batch* batch);
 LH_API int lh_batch_commit_and_renew(lh_batch* batch);
 
+/* ---- recorded batches (no counterpart in the reference: a Metal command buffer is encoded anew for
+ *      every commit, batch.rs:240-291).  A decode step is a fixed sequence of some hundreds of short
+ *      dispatches, and issuing them one by one costs more host time than the GPU needs to run them; the
+ *      sequence is recorded once into a HIP graph and replayed with one call per step.  Between
+ *      begin_capture and end_capture every `*_into` call on the context is recorded instead of run; calls
+ *      that wait, allocate, copy from host memory or clear a buffer return LH_ERR_INVALID_ARGUMENT (and so
+ *      does a grouped matvec of more than two problems).  Whatever changes from step to step must live in
+ *      device buffers the recorded kernels read (positions: rope_batch_decode, encode_kv_turboquant_batched,
+ *      flash_attention_tq_batched; inputs: write them into the same buffers before each replay). ---- */
+typedef struct lh_graph lh_graph;
+LH_API int lh_batch_begin_capture(lh_batch* batch);
+LH_API int lh_batch_end_capture(lh_batch* batch, lh_graph** out);
+LH_API int lh_graph_launch(lh_graph* graph);                    /* enqueues one replay on the context stream */
+LH_API uint32_t lh_graph_dispatch_count(const lh_graph* graph);
+LH_API void lh_graph_free(lh_graph* graph);
+
 /* ---- M = 1 fused dequant matvec: y[rows] = W[rows, cols] . x[cols] ----------
  * kernels.rs:5711-5838 matvec_q4_0{,_into,_f32out,_f32out_into};
  * kernels.rs:5848-6038 matvec_tq2_0{,_into,_f32out,_f32out_into};
@@ -148,6 +164,18 @@ LH_API int lh_matvec_quant_grouped_into(lh_batch* batch, lh_quant fmt, uint32_t 
                                         const lh_buffer* const* matrices, const lh_buffer* const* vectors,
                                         lh_dtype vector_dtype, lh_buffer* const* outputs, lh_dtype output_dtype,
                                         uint32_t rows, uint32_t cols);
+/* 1..8 matvecs of one shape against ONE f16 vector that is transformed while it is staged, so the
+ * kernel that would have produced the transformed vector is not dispatched (a single-token decode
+ * step is bound by the number of dispatches).  Replaces, in layer.rs:387-392 / 468-482,
+ *   LH_PROLOGUE_RMS_NORM: rms_norm_into(x, aux = weight, eps) followed by matvec_*_into      (attn_norm -> Q, K, V;
+ *                         ffn_norm -> gate, up)
+ *   LH_PROLOGUE_GELU_MUL: gelu_mul_into(x = gate, aux = up) followed by matvec_*_into       (-> down)
+ * The transformed value is rounded to f16 exactly where the separate kernel would have stored it.
+ * f16 vector and outputs; cols a multiple of 64 and 16-byte aligned operands, else INVALID_ARGUMENT. */
+typedef enum lh_prologue { LH_PROLOGUE_RMS_NORM = 1, LH_PROLOGUE_GELU_MUL = 2 } lh_prologue;
+LH_API int lh_matvec_quant_fused_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
+                                      const lh_buffer* vector, int prologue, const lh_buffer* aux, float eps,
+                                      lh_buffer* const* outputs, uint32_t rows, uint32_t cols);
 
 /* ---- small-M / prefill quantized matmul: C[m,n] = A[m,k] . W[n,k]^T ----------
  * kernels.rs:6459-6563 matmul_nt_{q4_0,tq2_0}_into (routes by m:
@@ -201,6 +229,13 @@ LH_API int lh_rms_norm_into(lh_batch* batch, const lh_buffer* input, const lh_bu
 /* kernels.rs:6663-6673 rms_norm_add_into (rms_norm.metal:48-88): the same plus residual[r] */
 LH_API int lh_rms_norm_add_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, const lh_buffer* residual,
                                 lh_buffer* output, uint32_t dim, uint32_t rows, float eps);
+/* The tail of the single-token layer step in one dispatch (layer.rs:507-520 issues rms_norm_into, residual_add_into and,
+ * when the layer has an output scale, scale_in_place_gpu_into): out = f16(f16(f16(norm(in) * weight) + residual) * scale),
+ * i.e. with the f16 rounding after each of the three steps that the separate kernels apply; `scale` is used only when
+ * `apply_scale` is non-zero.  `output` may alias `residual`. */
+LH_API int lh_rms_norm_residual_scale_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight,
+                                           const lh_buffer* residual, lh_buffer* output, uint32_t dim, uint32_t rows,
+                                           float eps, int apply_scale, float scale);
 /* kernels.rs:2215-2280 qk_norm_gpu_into / qk_norm_offset_into (shaders/qk_norm.metal:6-56): per-head RMSNorm in place;
  * weight_offset in bytes into the weight buffer */
 LH_API int lh_qk_norm_gpu_into(lh_batch* batch, lh_buffer* qk_data, const lh_buffer* weight, uint32_t head_dim,

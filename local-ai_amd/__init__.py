@@ -255,11 +255,46 @@ class CommandBatch:
     def commit_and_renew(self) -> None:
         _check(lib().lh_batch_commit_and_renew(self._h))
 
+    def begin_capture(self) -> None:
+        """Record the following ``*_into`` calls into a graph instead of running them."""
+        _check(lib().lh_batch_begin_capture(self._h))
+
+    def end_capture(self) -> "Graph":
+        h = C.c_void_p()
+        _check(lib().lh_batch_end_capture(self._h, C.byref(h)))
+        return Graph(h, self.ctx)
+
     def __del__(self):
         try:
             if self._h:
                 lib().lh_batch_free(self._h)
                 self._h = C.c_void_p()
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded batch: ``launch()`` enqueues one replay of every dispatch captured between
+    ``CommandBatch.begin_capture`` and ``end_capture``."""
+
+    def __init__(self, handle, ctx):
+        self._h, self.ctx = handle, ctx
+
+    def launch(self) -> None:
+        _check(lib().lh_graph_launch(self._h))
+
+    def dispatch_count(self) -> int:
+        lib().lh_graph_dispatch_count.restype = C.c_uint32
+        return int(lib().lh_graph_dispatch_count(self._h))
+
+    def free(self) -> None:
+        if self._h:
+            lib().lh_graph_free(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
         except Exception:
             pass
 
@@ -335,6 +370,17 @@ class Kernels:
                                                     _handles(vectors), C.c_int(vector_dtype), _handles(outputs),
                                                     C.c_int(output_dtype), _u32(rows), _u32(cols)))
 
+    PROLOGUE_RMS_NORM, PROLOGUE_GELU_MUL = 1, 2
+
+    def matvec_quant_fused_into(self, batch, fmt, matrices, vector, prologue, aux, eps, outputs, rows, cols):
+        """1..8 matvecs of one shape against one f16 vector transformed while it is staged: rms_norm(vector) * aux
+        (PROLOGUE_RMS_NORM) or gelu(vector) * aux (PROLOGUE_GELU_MUL), rounded to f16 as the separate kernel would."""
+        n = len(matrices)
+        assert len(outputs) == n
+        _check(self._l.lh_matvec_quant_fused_into(batch._h, C.c_int(fmt), _u32(n), _handles(matrices), vector._h,
+                                                  C.c_int(prologue), aux._h, C.c_float(eps), _handles(outputs),
+                                                  _u32(rows), _u32(cols)))
+
     # -- small-M / prefill matmul (kernels.rs:6378-6563, 5517-5568) --
     def matmul_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
@@ -394,6 +440,13 @@ class Kernels:
     def rms_norm_add_into(self, batch, input, weight, residual, output, dim, rows, eps):
         _check(self._l.lh_rms_norm_add_into(batch._h, input._h, weight._h, residual._h, output._h, _u32(dim), _u32(rows),
                                             C.c_float(eps)))
+
+    def rms_norm_residual_scale_into(self, batch, input, weight, residual, output, dim, rows, eps, scale=None):
+        """rms_norm_into + residual_add_into (+ scale_in_place_gpu_into when `scale` is given) in one dispatch, with the
+        f16 rounding after each step that the separate kernels apply."""
+        _check(self._l.lh_rms_norm_residual_scale_into(batch._h, input._h, weight._h, residual._h, output._h, _u32(dim),
+                                                       _u32(rows), C.c_float(eps), C.c_int(scale is not None),
+                                                       C.c_float(scale if scale is not None else 1.0)))
 
     def qk_norm_gpu_into(self, batch, qk_data, weight, head_dim, num_heads, eps):
         _check(self._l.lh_qk_norm_gpu_into(batch._h, qk_data._h, weight._h, _u32(head_dim), _u32(num_heads), C.c_float(eps)))

@@ -18,6 +18,11 @@ struct lh_context {
     // The creator's handle plus one per live buffer, batch and event: the stream and the workspace are
     // released when the last of them goes, so handles may be freed in any order.
     std::atomic<int> refs;
+    // True between lh_batch_begin_capture and lh_batch_end_capture: dispatches are recorded into a graph instead
+    // of running, and calls that would wait, allocate, copy from host memory or record a memset are refused.
+    bool capturing;
+    void* deferred_free[64];    // owning buffers released during a capture: freed when the capture ends
+    int deferred_count;
 };
 
 struct lh_buffer {
@@ -61,12 +66,23 @@ static inline int lh_need(const lh_buffer* b, size_t bytes, const char* op, cons
         if (r__ != LH_OK) return r__;                        \
     } while (0)
 
+// Optional transform applied to an f16 activation vector while a matvec stages it (saves the dispatch of the kernel
+// that would otherwise have produced it): the value that is quantised is the f16 the separate kernel would have stored.
+//   kXProRmsNorm: x_i * rsqrt(mean(x^2) + eps) * aux_i   (rms_norm.metal:4-46; aux = norm weight, f16[K])
+//   kXProGeluMul: gelu_tanh(x_i) * aux_i                 (gelu.metal:23-41; x = gate, aux = up, f16[K])
+enum : uint32_t { kXProNone = 0, kXProRmsNorm = 1, kXProGeluMul = 2 };
+struct XPrologue {
+    uint32_t kind;
+    const uint16_t* aux;
+    float eps;
+};
+
 // TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.
 // With a non-zero stride only entry 0 of the arrays is used: problem i is problem 0 with its vector / output advanced by
 // i * xstride / i * ystride bytes.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
                               void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K, uint32_t xstride,
-                              uint32_t ystride);
+                              uint32_t ystride, const XPrologue& pro = XPrologue{kXProNone, nullptr, 0.0f});
 // The m rows of a small activation batch against one quantized matrix, as m matvecs in one launch (matvec_quant.hip).
 // Returns LH_OK, an error, or -1 when the fast kernels do not take the shape (the caller then uses its own kernel).
 int lh_matvec_rows(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer* weight, const lh_buffer* input, lh_dtype at,

@@ -5,6 +5,7 @@
 // in local-metal/src/kernels.rs.  At decode these touch a few KB per call: they are latency bound, one small
 // workgroup per row / head, f32 math, f16 storage with the same rounding points as the reference kernels.
 #include "common.hpp"
+#include "xquant.hpp"
 #include <cstdlib>
 
 namespace {
@@ -35,9 +36,17 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 
 // rms_norm.metal:4-46 / 48-88: out[r, i] = in[r, i] * rsqrt(mean(in[r]^2) + eps) * w[i] (+ residual[r, i]).
 // VEC = 8: 16-byte accesses (dim a multiple of 8, 16-byte aligned rows); VEC = 1 otherwise.
+// ADD with `tail` != 0 is the three-kernel tail of the single-token layer in one dispatch (layer.rs:507-520: rms_norm,
+// residual_add, scale_in_place): the normalised value is rounded to f16, added to the residual as an f16 addition, and,
+// with tail == 2, scaled and rounded once more -- the roundings of the three separate kernels.
+__device__ __forceinline__ float norm_tail(float normed, float res, uint32_t tail, float scale) {
+    const _Float16 sum = (_Float16)normed + (_Float16)res;
+    return tail == 2 ? (float)sum * scale : (float)sum;
+}
+
 template <bool ADD, int VEC>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const uint16_t* __restrict__ w, const uint16_t* res, uint16_t* out,   // out may be in or res
-                                                      uint32_t dim, float eps) {
+                                                      uint32_t dim, float eps, uint32_t tail = 0, float scale = 1.0f) {
     __shared__ float scratch[4];
     const size_t row = (size_t)blockIdx.x * dim;
     float s = 0.0f;
@@ -63,7 +72,11 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const
             for (int j = 0; j < 4; j++) {
                 float lo = lh_h2f((uint16_t)(wv[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
                 float hi = lh_h2f((uint16_t)(wv[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
-                if (ADD) { lo += lh_h2f((uint16_t)(wr[j] & 0xFFFF)); hi += lh_h2f((uint16_t)(wr[j] >> 16)); }
+                if (ADD) {
+                    const float rlo = lh_h2f((uint16_t)(wr[j] & 0xFFFF)), rhi = lh_h2f((uint16_t)(wr[j] >> 16));
+                    if (tail) { lo = norm_tail(lo, rlo, tail, scale); hi = norm_tail(hi, rhi, tail, scale); }
+                    else { lo += rlo; hi += rhi; }
+                }
                 wo[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
             }
             *reinterpret_cast<uint4*>(out + row + i) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
@@ -71,18 +84,19 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const
     } else {
         for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
             float v = h_at(in, row + i) * rms * h_at(w, i);
-            if (ADD) v += h_at(res, row + i);
+            if (ADD) v = tail ? norm_tail(v, h_at(res, row + i), tail, scale) : v + h_at(res, row + i);
             out[row + i] = lh_f2h(v);
         }
     }
 }
 
 template <bool ADD>
-void launch_rms_norm(hipStream_t stream, const void* in, const void* w, const void* res, void* out, uint32_t dim, uint32_t rows, float eps) {
+void launch_rms_norm(hipStream_t stream, const void* in, const void* w, const void* res, void* out, uint32_t dim, uint32_t rows, float eps,
+                     uint32_t tail = 0, float scale = 1.0f) {
     const bool vec = (dim & 7) == 0 && (((uintptr_t)in | (uintptr_t)w | (uintptr_t)(res ? res : in) | (uintptr_t)out) & 15) == 0;
     const uint32_t threads = vec ? (dim >= 2048 ? 256u : (dim >= 1024 ? 128u : 64u)) : (dim >= 256 ? 256u : (dim > 64 ? 128u : 64u));
-    if (vec) hipLaunchKernelGGL((rms_norm_kernel<ADD, 8>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps);
-    else hipLaunchKernelGGL((rms_norm_kernel<ADD, 1>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps);
+    if (vec) hipLaunchKernelGGL((rms_norm_kernel<ADD, 8>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps, tail, scale);
+    else hipLaunchKernelGGL((rms_norm_kernel<ADD, 1>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps, tail, scale);
 }
 
 // qk_norm.metal:6-56 (in place; head h of `qk`), and 70-140 with the NEOX rotation fused: the normalised values are
@@ -157,12 +171,6 @@ __global__ __launch_bounds__(256) void rope_batch_kernel(uint16_t* qk, const uin
 
 // Elementwise f16 kernels: a thread takes 8 consecutive elements with 16-byte accesses; the launcher sends a
 // count that is not a multiple of 8, or pointers that are not 16-byte aligned, to the one-element form (VEC = 1).
-__device__ __forceinline__ float gelu_tanh_f32(float x) {   // gelu.metal:31-35
-    const float x3 = x * x * x;
-    const float inner = 0.7978845608f * (x + 0.044715f * x3);
-    const float t = tanhf(fminf(fmaxf(inner, -10.0f), 10.0f));
-    return 0.5f * x * (1.0f + t);
-}
 
 enum { kGeluMul = 0, kResidualAdd = 1, kScale = 2 };
 
@@ -170,7 +178,7 @@ enum { kGeluMul = 0, kResidualAdd = 1, kScale = 2 };
 // scale_in_place.metal:5-14 (out = half(float(a) * scalar), a may be out)
 template <int OP>
 __device__ __forceinline__ uint16_t elementwise_one(uint16_t a, uint16_t b, float scalar) {
-    if constexpr (OP == kGeluMul) return lh_f2h(gelu_tanh_f32(lh_h2f(a)) * lh_h2f(b));
+    if constexpr (OP == kGeluMul) return lh_f2h(lh_gelu_tanh_f32(lh_h2f(a)) * lh_h2f(b));
     else if constexpr (OP == kResidualAdd) return __builtin_bit_cast(uint16_t, (_Float16)(__builtin_bit_cast(_Float16, a) + __builtin_bit_cast(_Float16, b)));
     else return lh_f2h(lh_h2f(a) * scalar);
 }
@@ -251,6 +259,19 @@ int lh_rms_norm_add_into(lh_batch* batch, const lh_buffer* input, const lh_buffe
     LH_NEED(residual, (size_t)rows * dim * 2, op, "residual");
     LH_NEED(output, (size_t)rows * dim * 2, op, "output");
     launch_rms_norm<true>(batch->ctx->stream, input->ptr, weight->ptr, residual->ptr, output->ptr, dim, rows, eps);
+    return finish(batch, op);
+}
+
+int lh_rms_norm_residual_scale_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, const lh_buffer* residual,
+                                    lh_buffer* output, uint32_t dim, uint32_t rows, float eps, int apply_scale, float scale) {
+    const char* op = "rms_norm_residual_scale";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (dim == 0 || rows == 0) return LH_OK;
+    LH_NEED(input, (size_t)rows * dim * 2, op, "input");
+    LH_NEED(weight, (size_t)dim * 2, op, "weight");
+    LH_NEED(residual, (size_t)rows * dim * 2, op, "residual");
+    LH_NEED(output, (size_t)rows * dim * 2, op, "output");
+    launch_rms_norm<true>(batch->ctx->stream, input->ptr, weight->ptr, residual->ptr, output->ptr, dim, rows, eps, apply_scale ? 2u : 1u, scale);
     return finish(batch, op);
 }
 

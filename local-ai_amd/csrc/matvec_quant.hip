@@ -43,6 +43,7 @@ struct MatvecBase {
     // needs no descriptor upload ahead of it.
     MatvecProblem second = {nullptr, nullptr, nullptr};
     uint32_t pair = 0;
+    XPrologue pro = {kXProNone, nullptr, 0.0f};   // applied to every problem's vector while it is staged
 };
 
 // ---- per-lane activation registers for one unit column -------------------------
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
 
         if (pb.vector != staged_vector) {
             __syncthreads();   // every wave is done reading the previous vector's limbs
-            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG);
+            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG, single.pro);
             __syncthreads();
 #pragma unroll
             for (int p = 0; p < NPOS; p++) {
@@ -500,7 +501,7 @@ bool fast_path_ok(lh_quant fmt, const void* matrix, const void* vector, uint32_t
 // Validates and launches `count` matvecs of one shape.
 int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
                     const lh_buffer* const* vectors, lh_dtype xt, lh_buffer* const* outputs, lh_dtype yt, uint32_t rows,
-                    uint32_t cols, const char* op) {
+                    uint32_t cols, const char* op, const XPrologue& pro = XPrologue{kXProNone, nullptr, 0.0f}) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     if (xt == LH_BF16 || yt == LH_BF16) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: bf16 vectors are not supported", op);
     // kernels.rs:5720-5724, 5857-5861: block alignment is checked before anything is encoded.
@@ -519,6 +520,8 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         const size_t sl = matrices[i]->len - wbytes + matrices[i]->slack;
         if (sl < min_slack) min_slack = sl;
     }
+    if (!fast && pro.kind != kXProNone)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: a fused activation prologue needs 16-byte aligned vectors and cols a multiple of 64", op);
     if (!fast) {
         for (uint32_t i = 0; i < count; i++) {
             int r = fmt == LH_Q4_0
@@ -536,7 +539,7 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         const void** px = count <= 8 ? stack_x : pm + count;
         void** py = count <= 8 ? stack_y : (void**)(pm + 2 * (size_t)count);
         for (uint32_t i = 0; i < count; i++) { pm[i] = matrices[i]->ptr; px[i] = vectors[i]->ptr; py[i] = outputs[i]->ptr; }
-        int r = lh_launch_matvec_tq2_mfma(ctx, count, pm, px, py, xt, yt, rows, cols, 0, 0);
+        int r = lh_launch_matvec_tq2_mfma(ctx, count, pm, px, py, xt, yt, rows, cols, 0, 0, pro);
         if (count > 8) free((void*)pm);
         if (r == LH_OK) batch->dispatch_count++;
         return r;
@@ -545,11 +548,13 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     // top quarter of the context workspace (the copy is stream ordered, so it cannot overtake a
     // kernel that still reads the previous set).
     MatvecBase single{MatvecProblem{(const uint8_t*)matrices[0]->ptr, vectors[0]->ptr, outputs[0]->ptr}, 0, 0};
+    single.pro = pro;
     MatvecProblem* dev_desc = nullptr;
     if (count == 2) {
         single.second = MatvecProblem{(const uint8_t*)matrices[1]->ptr, vectors[1]->ptr, outputs[1]->ptr};
         single.pair = 1;
     } else if (count > 2) {
+        if (ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: more than two grouped problems need a descriptor upload, which a captured graph cannot hold", op);
         const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);
         if (desc_bytes > ctx->workspace_bytes / 4)
             return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u problems exceed the descriptor area", op, count);
@@ -666,6 +671,24 @@ int lh_matvec_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, cons
     if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
     if (count && (!ms || !xs || !ys)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null problem arrays", op_name(fmt));
     return matvec_dispatch(b, fmt, count, ms, xs, xt, ys, yt, rows, cols, op_name(fmt));
+}
+
+int lh_matvec_quant_fused_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* const* ms, const lh_buffer* x, int prologue,
+                               const lh_buffer* aux, float eps, lh_buffer* const* ys, uint32_t rows, uint32_t cols) {
+    const char* op = fmt == LH_Q4_0 ? "matvec_q4_0 (fused prologue)" : "matvec_tq2_0 (fused prologue)";
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
+    if (prologue != LH_PROLOGUE_RMS_NORM && prologue != LH_PROLOGUE_GELU_MUL)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: unknown prologue %d", op, prologue);
+    if (count == 0 || rows == 0 || cols == 0) return LH_OK;
+    if (count > 8) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: at most 8 matrices share one staged vector, got %u", op, count);
+    if (!ms || !ys || !x) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null problem arrays", op);
+    if (cols % 8 != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: cols %u not /8", op, cols);
+    LH_NEED(aux, (size_t)cols * 2, op, prologue == LH_PROLOGUE_RMS_NORM ? "norm weight" : "second factor");
+    LH_REQUIRE(((uintptr_t)aux->ptr & 15) == 0, "%s: the prologue operand must be 16-byte aligned", op);
+    const lh_buffer* xs[8];
+    for (uint32_t i = 0; i < count; i++) xs[i] = x;
+    const XPrologue pro{prologue == LH_PROLOGUE_RMS_NORM ? kXProRmsNorm : kXProGeluMul, (const uint16_t*)aux->ptr, eps};
+    return matvec_dispatch(b, fmt, count, ms, xs, LH_F16, ys, LH_F16, rows, cols, op, pro);
 }
 
 int lh_matvec_tq2_0_soa_into(lh_batch* b, const lh_buffer* qs, const lh_buffer* scales, const lh_buffer* x, lh_buffer* y,

@@ -53,6 +53,7 @@ struct Tq2Base {
     // descriptor upload ahead of it.
     Tq2Problem second = {nullptr, nullptr, nullptr};
     uint32_t pair = 0;
+    XPrologue pro = {kXProNone, nullptr, 0.0f};   // applied to every problem's vector while it is staged
 };
 
 __device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
         const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
-            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x);
+            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro);
             __syncthreads();
             staged = pb.vector;
         }
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Proble
 // Entry used by matvec_quant.hip's dispatcher. Arrays are host arrays of device pointers.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
                               void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K, uint32_t xstride,
-                              uint32_t ystride) {
+                              uint32_t ystride, const XPrologue& pro) {
     const bool strided = xstride != 0 || ystride != 0;   // problem i = problem 0 advanced by i strides: no descriptor table
     const uint32_t nb = K >> 8;
     const uint64_t tiles = (uint64_t)((rows + 15) >> 4) * count;
@@ -328,11 +329,13 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
+    single.pro = pro;
     Tq2Problem* dev = nullptr;
     if (count == 2 && !strided) {
         single.second = Tq2Problem{(const uint8_t*)matrices[1], vectors[1], outputs[1]};
         single.pair = 1;
     } else if (count > 2 && !strided) {
+        if (ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: more than two grouped problems need a descriptor upload, which a captured graph cannot hold");
         const size_t bytes = (size_t)count * sizeof(Tq2Problem);
         if (bytes > ctx->workspace_bytes / 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems exceed the descriptor area", count);
         Tq2Problem* host = (Tq2Problem*)malloc(bytes);

@@ -84,6 +84,8 @@ int lh_context_create(int device_index, lh_context** out) {
     if (!ctx) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_context));
     ctx->device = device_index;
     ctx->refs.store(1, std::memory_order_relaxed);
+    ctx->capturing = false;
+    ctx->deferred_count = 0;
     ctx->cu_count = prop.multiProcessorCount;
     snprintf(ctx->name, sizeof ctx->name, "%s (%s)", prop.name, prop.gcnArchName);
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
@@ -116,6 +118,7 @@ int lh_context_compute_units(const lh_context* ctx) { return ctx ? ctx->cu_count
 void* lh_context_stream(const lh_context* ctx) { return ctx ? (void*)ctx->stream : nullptr; }
 
 int lh_context_synchronize(lh_context* ctx) {
+    if (ctx && ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "context_synchronize: not while a graph is being captured");
     if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "synchronize: context is null");
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
@@ -172,6 +175,7 @@ static int new_buffer(lh_context* ctx, size_t len, lh_buffer** out) {
 }
 
 int lh_buffer_empty(lh_context* ctx, size_t len, lh_buffer** out) {
+    if (ctx && ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_empty: not while a graph is being captured");
     int r = new_buffer(ctx, len, out);
     if (r != LH_OK) return r;
     hipError_t e = hipMemsetAsync((*out)->ptr, 0, len + 64, ctx->stream);
@@ -180,6 +184,7 @@ int lh_buffer_empty(lh_context* ctx, size_t len, lh_buffer** out) {
 }
 
 int lh_buffer_from_bytes(lh_context* ctx, const void* src, size_t len, lh_buffer** out) {
+    if (ctx && ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_from_bytes: not while a graph is being captured");
     if (!src && len) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_from_bytes: src is null");
     int r = new_buffer(ctx, len, out);
     if (r != LH_OK) return r;
@@ -216,8 +221,13 @@ int lh_buffer_wrap(lh_context* ctx, void* device_ptr, size_t len, lh_buffer** ou
 void lh_buffer_free(lh_buffer* buf) {
     if (!buf) return;
     if (buf->owns && buf->ptr) {
-        (void)hipStreamSynchronize(buf->ctx->stream);
-        (void)hipFree(buf->ptr);
+        lh_context* ctx = buf->ctx;
+        if (ctx->capturing && ctx->deferred_count < 64) {
+            ctx->deferred_free[ctx->deferred_count++] = buf->ptr;   // neither a wait nor a free may happen inside a capture
+        } else if (!ctx->capturing) {
+            (void)hipStreamSynchronize(ctx->stream);
+            (void)hipFree(buf->ptr);
+        }   // (a 65th release inside one capture leaks its allocation rather than break the capture)
     }
     ctx_release(buf->ctx);
     delete buf;
@@ -228,6 +238,7 @@ void* lh_buffer_device_ptr(const lh_buffer* buf) { return buf ? buf->ptr : nullp
 
 int lh_buffer_write(lh_buffer* buf, size_t offset, const void* src, size_t len) {
     if (!buf || (!src && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_write: null argument");
+    if (buf->ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_write: not while a graph is being captured");
     if (offset > buf->len || len > buf->len - offset)
         return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_write: range %zu+%zu exceeds %zu", offset, len, buf->len);
     if (!len) return LH_OK;
@@ -239,6 +250,7 @@ int lh_buffer_write(lh_buffer* buf, size_t offset, const void* src, size_t len) 
 
 int lh_buffer_read(const lh_buffer* buf, size_t offset, void* dst, size_t len) {
     if (!buf || (!dst && len)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_read: null argument");
+    if (buf->ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_read: not while a graph is being captured");
     if (offset > buf->len || len > buf->len - offset)
         return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_read: range %zu+%zu exceeds %zu", offset, len, buf->len);
     if (!len) return LH_OK;
@@ -251,6 +263,7 @@ int lh_buffer_read(const lh_buffer* buf, size_t offset, void* dst, size_t len) {
 int lh_buffer_fill_zero(lh_buffer* buf) {
     if (!buf) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_fill_zero: buffer is null");
     if (!buf->len) return LH_OK;
+    if (buf->ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "buffer_fill_zero: not while a graph is being captured");
     hipError_t e = hipMemsetAsync(buf->ptr, 0, buf->len, buf->ctx->stream);
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: buffer_fill_zero: %s", hipGetErrorString(e));
     return LH_OK;
@@ -300,6 +313,7 @@ int lh_batch_blit_copy(lh_batch* batch, const lh_buffer* src, size_t src_offset,
 
 int lh_batch_commit_and_wait(lh_batch* batch) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "commit_and_wait: batch is null");
+    if (batch->ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "commit_and_wait: not while a graph is being captured");
     hipError_t e = hipStreamSynchronize(batch->ctx->stream);
     batch->dispatch_count = 0;
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
@@ -312,6 +326,72 @@ int lh_batch_submit_and_renew(lh_batch* batch) {
     return LH_OK;
 }
 int lh_batch_commit_and_renew(lh_batch* batch) { return lh_batch_commit_and_wait(batch); }
+
+// ---- recorded batches ----------------------------------------------------------
+struct lh_graph { lh_context* ctx; hipGraph_t graph; hipGraphExec_t exec; uint32_t dispatch_count; };
+
+int lh_batch_begin_capture(lh_batch* batch) {
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "begin_capture: batch is null");
+    lh_context* ctx = batch->ctx;
+    if (ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "begin_capture: a capture is already open on this context");
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: begin_capture: %s", hipGetErrorString(e));
+    ctx->capturing = true;
+    batch->dispatch_count = 0;
+    return LH_OK;
+}
+
+int lh_batch_end_capture(lh_batch* batch, lh_graph** out) {
+    if (!batch || !out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "end_capture: null argument");
+    *out = nullptr;
+    lh_context* ctx = batch->ctx;
+    if (!ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "end_capture: no capture is open on this context");
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (ctx->deferred_count) {
+        (void)hipStreamSynchronize(ctx->stream);
+        for (int i = 0; i < ctx->deferred_count; i++) (void)hipFree(ctx->deferred_free[i]);
+        ctx->deferred_count = 0;
+    }
+    if (e != hipSuccess || !graph) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: end_capture: %s", hipGetErrorString(e));
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: graph instantiation: %s", hipGetErrorString(e));
+    }
+    lh_graph* g = new (std::nothrow) lh_graph();
+    if (!g) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_graph));
+    }
+    g->ctx = ctx; g->graph = graph; g->exec = exec; g->dispatch_count = batch->dispatch_count;
+    ctx_retain(ctx);
+    batch->dispatch_count = 0;
+    *out = g;
+    return LH_OK;
+}
+
+int lh_graph_launch(lh_graph* graph) {
+    if (!graph) return lh_fail(LH_ERR_INVALID_ARGUMENT, "graph_launch: graph is null");
+    if (graph->ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "graph_launch: not while a graph is being captured");
+    hipError_t e = hipGraphLaunch(graph->exec, graph->ctx->stream);
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: graph_launch: %s", hipGetErrorString(e));
+    return LH_OK;
+}
+
+uint32_t lh_graph_dispatch_count(const lh_graph* graph) { return graph ? graph->dispatch_count : 0; }
+
+void lh_graph_free(lh_graph* graph) {
+    if (!graph) return;
+    (void)hipStreamSynchronize(graph->ctx->stream);   // a replay may still be running
+    (void)hipGraphExecDestroy(graph->exec);
+    (void)hipGraphDestroy(graph->graph);
+    ctx_release(graph->ctx);
+    delete graph;
+}
 
 // kernels.rs:6155-6304
 static int env_flag_default_on(const char* name) {

@@ -9,15 +9,45 @@ template <int L> struct Limb;
 template <> struct Limb<2> { static constexpr float qmax = 32639.0f; };     // 127*256 + 127
 template <> struct Limb<3> { static constexpr float qmax = 8355711.0f; };   // 127*65536 + 127*256 + 127
 
+__device__ __forceinline__ float lh_gelu_tanh_f32(float x) {   // gelu.metal:31-35
+    const float x3 = x * x * x;
+    const float inner = 0.7978845608f * (x + 0.044715f * x3);
+    const float t = tanhf(fminf(fmaxf(inner, -10.0f), 10.0f));
+    return 0.5f * x * (1.0f + t);
+}
+
 // ---- activation quantisation into LDS ----------------------------------------
 // xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
 // xs[K/G]: float scale of each group of G elements (G = weight block size).
 // `xn` (optional) receives sum(n_i) per group; `nthreads` = workgroup size (multiple of 64).
 template <int L, int G, typename XT>
 __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs, int* xn,
-                                                  uint32_t nthreads) {
+                                                  uint32_t nthreads, const XPrologue pro = XPrologue{kXProNone, nullptr, 0.0f}) {
     const int tid = threadIdx.x;
     const uint32_t kq = K >> 2;
+    float rms = 1.0f;
+    if constexpr (sizeof(XT) == 2) {
+        if (pro.kind == kXProRmsNorm) {   // uniform over the workgroup; xs doubles as the reduction scratch before it is filled
+            float s = 0.0f;
+            for (uint32_t e0 = tid * 8; e0 < K; e0 += nthreads * 8) {
+                const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
+                const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float lo = lh_h2f((uint16_t)(w[i] & 0xFFFF)), hi = lh_h2f((uint16_t)(w[i] >> 16));
+                    s += lo * lo;
+                    s += hi * hi;
+                }
+            }
+            s = lh_group_sum(s, 64);
+            if ((tid & 63) == 0) xs[tid >> 6] = s;
+            __syncthreads();
+            float t = 0.0f;
+            for (uint32_t w = 0; w < nthreads / 64; w++) t += xs[w];
+            __syncthreads();
+            rms = rsqrtf(t / (float)K + pro.eps);
+        }
+    }
     for (uint32_t base = 0; base < K; base += nthreads * 8) {
         const uint32_t e0 = base + tid * 8;
         const bool valid = e0 < K;
@@ -36,6 +66,18 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                 for (int i = 0; i < 4; i++) {
                     v[2 * i] = lh_h2f((uint16_t)(w[i] & 0xFFFF));
                     v[2 * i + 1] = lh_h2f((uint16_t)(w[i] >> 16));
+                }
+                if (pro.kind != kXProNone) {
+                    const uint4 b = *reinterpret_cast<const uint4*>(pro.aux + e0);
+                    const uint32_t wb[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float g = lh_h2f((uint16_t)((wb[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
+                        float t;
+                        if (pro.kind == kXProRmsNorm) t = v[i] * rms * g;
+                        else t = lh_gelu_tanh_f32(v[i]) * g;
+                        v[i] = lh_h2f(lh_f2h(t));
+                    }
                 }
             }
         }

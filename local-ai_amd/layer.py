@@ -149,9 +149,10 @@ class TransformerLayer:
     """layer.rs:330-873."""
 
     def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True,
-                 fuse_norm_rope: bool = True):
+                 fuse_norm_rope: bool = True, fuse_prologues: bool = True):
         self.params, self.weights = params, weights
         self.group_projections, self.fuse_norm_rope = group_projections, fuse_norm_rope
+        self.fuse_prologues = fuse_prologues
         # layer.rs:515-520 reads the scalar out of shared memory at every encode; the buffer lives in device
         # memory here, so it is fetched once.
         self._output_scale = None
@@ -167,6 +168,28 @@ class TransformerLayer:
         else:
             wa.matvec_into(batch, kernels, x, out_a)
             wb.matvec_into(batch, kernels, x, out_b)
+
+    def _ple_slice(self, per_layer_input: Buffer) -> Buffer:
+        """This layer's [per_layer_dim] slice of the per-layer input buffer, as a view (cached per buffer)."""
+        cached = getattr(self, "_ple_view", None)
+        if cached is None or cached[0] is not per_layer_input:
+            pld = self.params.per_layer_dim
+            cached = (per_layer_input, per_layer_input.view(self.params.layer_idx * pld * 2, pld * 2))
+            self._ple_view = cached
+        return cached[1]
+
+    def _fusable(self, *ws: Optional[QuantWeight]) -> bool:
+        return self.fuse_prologues and all(w is not None and w.ty != W_F16 and w.cols % 64 == 0 for w in ws)
+
+    def _fused_matvecs(self, batch, kernels: Kernels, prologue: int, x: Buffer, aux: Buffer, ws, outs) -> None:
+        """Every weight in `ws` against prologue(x, aux); weights of one format and shape share a launch."""
+        eps = self.params.rms_norm_eps
+        if len(ws) == 2 and self.group_projections and _groupable(ws[0], ws[1]):
+            kernels.matvec_quant_fused_into(batch, ws[0].ty, [w.buf for w in ws], x, prologue, aux, eps, list(outs),
+                                            ws[0].rows, ws[0].cols)
+            return
+        for w, out in zip(ws, outs):
+            kernels.matvec_quant_fused_into(batch, w.ty, [w.buf], x, prologue, aux, eps, [out], w.rows, w.cols)
 
     def _norm_rope(self, batch, kernels: Kernels, qk: Buffer, norm_w: Optional[Buffer], heads: int, pos: int) -> None:
         """layer.rs:393-404 / 415-428: per-head RMS norm (when the layer has one) then RoPE, in place."""
@@ -194,13 +217,22 @@ class TransformerLayer:
         pos, seq_len = position, position + 1
 
         # 1. input_layernorm -> Q projection -> q_norm -> RoPE
-        kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
-        w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
+        own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
+        fused_in = self._fusable(w.attn_q) and (not own_kv or self._fusable(w.attn_k, w.attn_v))
+        if fused_in:
+            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [w.attn_q], [s.q])
+        else:
+            kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
+            w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
         self._norm_rope(batch, kernels, s.q, w.q_norm, n_head, pos)
 
         # 2. own K/V into the TurboQuant cache, then attention over the codes
-        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
-            self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
+        if own_kv:
+            if fused_in:
+                self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm,
+                                    [w.attn_k, w.attn_v], [s.k, s.v])
+            else:
+                self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
             kernels.rms_norm_into(batch, s.v, s.ones, s.v, hd, n_kv, eps)   # V: RMS norm with unit weight
             self._norm_rope(batch, kernels, s.k, w.k_norm, n_kv, pos)
             kv_cache.write_kv_gpu_into(batch, kernels, s.k, s.v, position, 1)
@@ -213,20 +245,36 @@ class TransformerLayer:
 
         # 4. GeGLU feed-forward -> post_feedforward_norm + residual #2
         inter = p.intermediate_size
-        kernels.rms_norm_into(batch, s.attn_resid, w.ffn_norm, s.normed, h, 1, eps)
-        self._pair_matvec(batch, kernels, w.ffn_gate, w.ffn_up, s.normed, s.gate, s.up)
-        kernels.gelu_mul_into(batch, s.gate, s.up, s.gate, inter)
-        w.ffn_down.matvec_into(batch, kernels, s.gate, s.ffn_out)
+        if self._fusable(w.ffn_gate, w.ffn_up):
+            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, s.attn_resid, w.ffn_norm,
+                                [w.ffn_gate, w.ffn_up], [s.gate, s.up])
+        else:
+            kernels.rms_norm_into(batch, s.attn_resid, w.ffn_norm, s.normed, h, 1, eps)
+            self._pair_matvec(batch, kernels, w.ffn_gate, w.ffn_up, s.normed, s.gate, s.up)
+        if self._fusable(w.ffn_down):
+            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_GELU_MUL, s.gate, s.up, [w.ffn_down], [s.ffn_out])
+        else:
+            kernels.gelu_mul_into(batch, s.gate, s.up, s.gate, inter)
+            w.ffn_down.matvec_into(batch, kernels, s.gate, s.ffn_out)
         kernels.rms_norm_add_into(batch, s.ffn_out, w.ffn_post_norm, s.attn_resid, output, h, 1, eps)
 
         # 5. per-layer input injection -> residual #3
         if (w.per_layer_inp_gate is not None and w.per_layer_proj is not None and w.per_layer_post_norm is not None
                 and per_layer_input is not None):
             pld = p.per_layer_dim
-            batch.blit_copy(per_layer_input, p.layer_idx * pld * 2, s.ple, 0, pld * 2)
             w.per_layer_inp_gate.matvec_into(batch, kernels, output, s.ple_h)
-            kernels.gelu_mul_into(batch, s.ple_h, s.ple, s.ple_h, pld)
-            w.per_layer_proj.matvec_into(batch, kernels, s.ple_h, s.ffn_out)
+            if self._fusable(w.per_layer_proj):
+                # this layer's slice is read in place (no copy into scratch) while the projection stages its input
+                self._fused_matvecs(batch, kernels, kernels.PROLOGUE_GELU_MUL, s.ple_h, self._ple_slice(per_layer_input),
+                                    [w.per_layer_proj], [s.ffn_out])
+            else:
+                batch.blit_copy(per_layer_input, p.layer_idx * pld * 2, s.ple, 0, pld * 2)
+                kernels.gelu_mul_into(batch, s.ple_h, s.ple, s.ple_h, pld)
+                w.per_layer_proj.matvec_into(batch, kernels, s.ple_h, s.ffn_out)
+            if self.fuse_prologues:   # norm, residual #3 and the output scale (step 6) in one dispatch
+                kernels.rms_norm_residual_scale_into(batch, s.ffn_out, w.per_layer_post_norm, output, output, h, 1, eps,
+                                                     self._output_scale)
+                return
             kernels.rms_norm_into(batch, s.ffn_out, w.per_layer_post_norm, s.normed, h, 1, eps)
             kernels.residual_add_into(batch, output, s.normed, output, h)
 

@@ -148,3 +148,27 @@ def test_glue_argument_errors(pkg, gpu):
         K.rope_into(batch, small, small, 7, 0, 1e4, 1.0, 1)
     with pytest.raises(pkg.InvalidArgument):
         K.logit_softcap_gpu_into(batch, small, 30.0, 17)
+
+
+@pytest.mark.parametrize("dim,rows", [(2048, 1), (512, 3), (100, 2)])
+@pytest.mark.parametrize("scale", [None, 0.75])
+def test_rms_norm_residual_scale_equals_the_three_kernels(pkg, gpu, dim, rows, scale):
+    """One dispatch for rms_norm_into -> residual_add_into (-> scale_in_place_gpu_into), layer.rs:507-520: the same
+    bits as the separate kernels, which the tests above hold to the oracle."""
+    ctx, K = gpu
+    g = pkg.synth.rng(77, dim + rows)
+    x = (g.standard_normal(rows * dim, dtype=np.float32) * 3).astype(np.float16)
+    w = (1 + 0.1 * g.standard_normal(dim, dtype=np.float32)).astype(np.float16)
+    r = g.standard_normal(rows * dim, dtype=np.float32).astype(np.float16)
+    xb, wb, rb = (pkg.Buffer.from_slice(ctx, a) for a in (x, w, r))
+    tmp, want, got = (pkg.Buffer.empty(ctx, rows * dim * 2) for _ in range(3))
+    batch = pkg.CommandBatch(ctx)
+    K.rms_norm_into(batch, xb, wb, tmp, dim, rows, 1e-6)
+    K.residual_add_into(batch, rb, tmp, want, rows * dim)
+    if scale is not None:
+        K.scale_in_place_gpu_into(batch, want, scale, rows * dim)
+    K.rms_norm_residual_scale_into(batch, xb, wb, rb, got, dim, rows, 1e-6, scale)
+    K.rms_norm_residual_scale_into(batch, xb, wb, rb, rb, dim, rows, 1e-6, scale)      # in place over the residual
+    batch.commit_and_wait()
+    assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16))
+    assert np.array_equal(rb.as_array(np.uint16), want.as_array(np.uint16))

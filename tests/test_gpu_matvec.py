@@ -106,3 +106,49 @@ def test_matvec_linearity_and_grouped(pkg, gpu, oracle):
     ws[0].matvec_typed_into(batch, kernels, x2, pkg.F32, y2, pkg.F32)
     batch.commit_and_wait()
     assert np.array_equal(y2.as_array(np.float32, rows), yb[0].as_array(np.float32, rows) * np.float32(4.0))
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+@pytest.mark.parametrize("rows,cols,count", [(2048, 2048, 1), (256, 2048, 2), (8192, 2048, 2), (2048, 8192, 1),
+                                             (40, 512, 3), (17, 10240, 1)])
+def test_matvec_fused_prologues(pkg, gpu, oracle, fmt, rows, cols, count):
+    """matvec_quant_fused_into: rms_norm(x) * w or gelu(gate) * up computed while the matvec stages its vector
+    (layer.rs:387-392, 468-482 as one dispatch).  Against the oracle (glue restatement, then the f64 dot over the f32
+    weight expansion, f16 result) and against the two separate kernels: GeGLU must agree bit for bit (same formula
+    per element); the RMS variant may differ by an f16 ulp of the normalised vector (its sum of squares runs in
+    another order), so it is only held to the oracle."""
+    from oracle import layer_glue as G
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(31, rows + cols + count)
+    raws = [refgen.q4_0_payload(rows, cols, 0x77 + i) if fmt == "q4_0" else refgen.tq2_0_payload(rows, cols, 0x77 + i)
+            for i in range(count)]
+    dqs = [(oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32)(r, rows, cols) for r in raws]
+    ws = [pkg.QuantWeight.from_bytes(ctx, r, ty, rows, cols) for r in raws]
+    x = (g.standard_normal(cols, dtype=np.float32) * 1.5).astype(np.float16)
+    aux = (1.0 + 0.2 * g.standard_normal(cols, dtype=np.float32)).astype(np.float16)
+    xb, ab = pkg.Buffer.from_slice(ctx, x), pkg.Buffer.from_slice(ctx, aux)
+    for kind in (K.PROLOGUE_RMS_NORM, K.PROLOGUE_GELU_MUL):
+        eps = 1e-6
+        staged = G.rms_norm(x, aux, cols, 1, eps) if kind == K.PROLOGUE_RMS_NORM else G.gelu_mul(x, aux)
+        outs = [pkg.Buffer.empty(ctx, rows * 2) for _ in range(count)]
+        batch = pkg.CommandBatch(ctx)
+        K.matvec_quant_fused_into(batch, ty, [w.buf for w in ws], xb, kind, ab, eps, outs, rows, cols)
+        assert batch.dispatch_count() == 1
+        tmp = pkg.Buffer.empty(ctx, cols * 2)
+        if kind == K.PROLOGUE_RMS_NORM:
+            K.rms_norm_into(batch, xb, ab, tmp, cols, 1, eps)
+        else:
+            K.gelu_mul_into(batch, xb, ab, tmp, cols)
+        sep = [pkg.Buffer.empty(ctx, rows * 2) for _ in range(count)]
+        for w, o in zip(ws, sep):
+            w.matvec_into(batch, K, tmp, o)
+        batch.commit_and_wait()
+        for i in range(count):
+            got = outs[i].as_array(np.float16, rows)
+            want = oracle.matvec_f64(dqs[i], staged.astype(np.float32)).astype(np.float32)
+            refgen.assert_close(got.astype(np.float32), want, 2e-3, f"{fmt} fused prologue {kind} {rows}x{cols} #{i}")
+            if kind == K.PROLOGUE_GELU_MUL:
+                assert np.array_equal(got.view(np.uint16), sep[i].as_array(np.uint16, rows))
+    with pytest.raises(pkg.InvalidArgument):
+        K.matvec_quant_fused_into(pkg.CommandBatch(ctx), ty, [ws[0].buf], xb, 7, ab, 1e-6, [outs[0]], rows, cols)
