@@ -338,6 +338,20 @@ LH_API int lh_dequantize_kv_turboquant_into(lh_batch* batch, const lh_buffer* pa
                                             const lh_buffer* levels, const lh_buffer* signs, lh_buffer* output,
                                             uint32_t head_dim, uint32_t n_kv_heads, uint32_t num_tokens,
                                             uint32_t bits, uint32_t token_start, uint32_t ring_capacity);
+/* Single-token Q / K / V preparation in one dispatch (no single counterpart in the reference: it replaces the eight
+ * dispatches of layer.rs:393-450 + quant_cache.rs:391-444, 560-570 -- qk_norm_gpu_into and rope_into on Q and on K,
+ * rms_norm_into with unit weight on V, encode_kv_turboquant_into for K and for V, hadamard_rotate_hf_into on Q):
+ *   q [n_q_heads, head_dim] f16, in place: per-head RMS norm (when `q_norm` is given), NEOX RoPE at `position`;
+ *      rq [n_q_heads, head_dim] f32 = FWHT(signs * q) / sqrt(head_dim), the query of flash_attention_tq_into;
+ *   k, v [n_kv_heads, head_dim] f16, in place: K as Q with `k_norm`, V RMS-normalised with unit weight; both encoded
+ *      into the cache row of `position` (ring addressing as in encode_kv_turboquant_into).
+ * Pass k = v = NULL for a layer that shares another layer's cache (only Q is prepared).  Values are rounded to f16
+ * wherever the separate kernels store f16; codes and norms equal the CPU encoder's for the k / v rows left behind. */
+LH_API int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm,
+                                      const lh_buffer* k_norm, const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq,
+                                      lh_buffer* k_codes, lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms,
+                                      uint32_t head_dim, uint32_t n_q_heads, uint32_t n_kv_heads, float eps, uint32_t position,
+                                      float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity);
 /* kernels.rs:5032-5163 hadamard_rotate{,_hf,_fh}_into,
  * shaders/attention_flash_tq.metal:58-139: per head optional sign flip, FWHT,
  * 1/sqrt(d), optional sign flip.  f32->f32, f16->f32, f32->f16. */

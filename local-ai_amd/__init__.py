@@ -536,6 +536,19 @@ class Kernels:
                                                         _u32(head_dim), _u32(n_kv_heads), _u32(num_tokens), _u32(bits),
                                                         _u32(token_start), _u32(ring_capacity)))
 
+    def decode_qkv_prepare_into(self, batch, q, k, v, q_norm, k_norm, levels, signs, rq, k_codes, k_norms, v_codes, v_norms,
+                                head_dim, n_q_heads, n_kv_heads, eps, position, theta, partial_rotary_factor, bits,
+                                ring_capacity):
+        """Head norms, RoPE, unit-weight V norm, both KV encodes and the query rotation of one decoded token in one
+        dispatch; k = v = None prepares the query only (a layer reading another layer's cache)."""
+        def h(b):
+            return b._h if b is not None else None
+        _check(self._l.lh_decode_qkv_prepare_into(batch._h, q._h, h(k), h(v), h(q_norm), h(k_norm), levels._h, signs._h, rq._h,
+                                                  h(k_codes), h(k_norms), h(v_codes), h(v_norms), _u32(head_dim),
+                                                  _u32(n_q_heads), _u32(n_kv_heads), C.c_float(eps), _u32(position),
+                                                  C.c_float(theta), C.c_float(partial_rotary_factor), _u32(bits),
+                                                  _u32(ring_capacity)))
+
     def hadamard_rotate_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
         _check(self._l.lh_hadamard_rotate_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
                                                _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))

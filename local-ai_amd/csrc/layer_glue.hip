@@ -12,16 +12,6 @@ namespace {
 
 __device__ __forceinline__ float h_at(const uint16_t* p, size_t i) { return lh_h2f(p[i]); }
 
-// One NEOX pair at `position` (rope.metal:46-58).  The same instruction sequence serves the stand-alone and the fused
-// kernel, so that qk_norm + rope and qk_norm_rope agree bit for bit (kernels.rs:7873).
-__device__ __forceinline__ void rotate_pair(float x0, float x1, uint32_t i, uint32_t head_dim, uint32_t position, float theta, uint16_t& o0, uint16_t& o1) {
-    const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)head_dim);
-    const float angle = (float)position * freq;
-    const float c = cosf(angle), sn = sinf(angle);
-    o0 = lh_f2h(__builtin_fmaf(x0, c, -(x1 * sn)));
-    o1 = lh_f2h(__builtin_fmaf(x0, sn, x1 * c));
-}
-
 // Sum over a workgroup of up to 256 threads (4 waves).
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
     v = lh_group_sum(v, 64);
@@ -125,7 +115,7 @@ __global__ __launch_bounds__(256) void qk_norm_kernel(const uint16_t* in, uint16
             out[base + i + half_dim] = lh_f2h(x1);
         } else {
             uint16_t o0, o1;
-            rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
+            lh_rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
             out[base + i] = o0;
             out[base + i + half_dim] = o1;
         }
@@ -145,7 +135,7 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* in, uint16_t*
     if (i >= rope_angles) { out[idx0] = in[idx0]; out[idx1] = in[idx1]; return; }
     const float x0 = h_at(in, idx0), x1 = h_at(in, idx1);
     uint16_t o0, o1;
-    rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
+    lh_rotate_pair(x0, x1, i, head_dim, position, theta, o0, o1);
     out[idx0] = o0;
     out[idx1] = o1;
 }
@@ -164,7 +154,7 @@ __global__ __launch_bounds__(256) void rope_batch_kernel(uint16_t* qk, const uin
     const uint32_t position = positions ? positions[seq_idx] : start_pos + seq_idx;
     const size_t idx0 = ((size_t)seq_idx * num_heads + head) * head_dim + i, idx1 = idx0 + half_dim;
     uint16_t o0, o1;
-    rotate_pair(h_at(qk, idx0), h_at(qk, idx1), i, head_dim, position, theta, o0, o1);
+    lh_rotate_pair(h_at(qk, idx0), h_at(qk, idx1), i, head_dim, position, theta, o0, o1);
     qk[idx0] = o0;
     qk[idx1] = o1;
 }

@@ -52,6 +52,56 @@ struct EncodeParams {
     float inv_sqrt_d;
 };
 
+// TurboQuant encode of one vector held one coordinate per thread (turboquant.rs:241-276): norm, unit vector, signs,
+// FWHT, 1/sqrt(d), nearest level, bit packing.  `sh` and `code_sh` are workgroup arrays of at least d entries; the
+// calling kernel runs d threads.
+__device__ __forceinline__ void encode_vector(float xv, uint32_t lane, uint32_t d, float* sh, uint32_t* code_sh,
+                                              const float* __restrict__ signs, const float* __restrict__ levels, uint32_t bits,
+                                              uint32_t code_bytes, float inv_sqrt_d, uint8_t* __restrict__ packed_slot,
+                                              uint16_t* __restrict__ norm_slot) {
+    // norm = sqrt(fold(+, x_i * x_i)) in index order; every thread walks the same LDS
+    // words (broadcast reads), so all hold the same value without another barrier.
+    sh[lane] = __fmul_rn(xv, xv);
+    __syncthreads();
+    float sq = 0.0f;
+    if (d >= 4) {
+        for (uint32_t i = 0; i < d; i += 4) {
+            const float4 q = *reinterpret_cast<const float4*>(&sh[i]);
+            sq = __fadd_rn(sq, q.x); sq = __fadd_rn(sq, q.y); sq = __fadd_rn(sq, q.z); sq = __fadd_rn(sq, q.w);
+        }
+    } else {
+        for (uint32_t i = 0; i < d; i++) sq = __fadd_rn(sq, sh[i]);
+    }
+    const float norm = __fsqrt_rn(sq);
+    float v = xv;
+    if (norm > 0.0f) v = __fmul_rn(v, __fdiv_rn(1.0f, norm));
+    v = __fmul_rn(v, signs[lane]);
+    __syncthreads();
+    sh[lane] = v;
+    fwht_lds(sh, d, lane);
+    const float y = __fmul_rn(sh[lane], inv_sqrt_d);
+
+    const uint32_t k = 1u << bits;
+    uint32_t best = 0;
+    float bd = INFINITY;
+    for (uint32_t i = 0; i < k; ++i) {
+        const float dd = fabsf(__fsub_rn(y, levels[i]));
+        if (dd < bd) { bd = dd; best = i; }
+    }
+    code_sh[lane] = best;
+    if (lane == 0) *norm_slot = lh_f2h_exact(norm);
+    __syncthreads();
+    if (lane < code_bytes) {     // one thread per output byte
+        uint32_t byte_val = 0;
+        for (uint32_t bitpos = 0; bitpos < 8; ++bitpos) {
+            const uint32_t global_bit = lane * 8 + bitpos, code_idx = global_bit / bits;
+            if (code_idx >= d) break;
+            byte_val |= ((code_sh[code_idx] >> (global_bit - code_idx * bits)) & 1u) << bitpos;
+        }
+        packed_slot[lane] = (uint8_t)byte_val;
+    }
+}
+
 // One workgroup (head_dim threads) per (token, head) vector.  BATCHED: group = (lane, head),
 // slot from positions[lane] (dequantize_kv.metal:327-407); else group = (token, head)
 // (dequantize_kv.metal:216-318).
@@ -73,49 +123,78 @@ __global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* 
         const uint32_t logical = p.position + tok;
         g = (p.ring_capacity ? logical % p.ring_capacity : logical) * p.n_kv_heads + head;
     }
-    const float xv = lh_h2f(input[(size_t)group * d + lane]);
+    encode_vector(lh_h2f(input[(size_t)group * d + lane]), lane, d, sh, code_sh, signs, levels, p.bits, p.code_bytes, p.inv_sqrt_d,
+                  packed + (size_t)g * p.code_bytes, norms + g);
+}
 
-    // norm = sqrt(fold(+, x_i * x_i)) in index order; every thread walks the same LDS
-    // words (broadcast reads), so all hold the same value without another barrier.
-    sh[lane] = __fmul_rn(xv, xv);
-    __syncthreads();
-    float sq = 0.0f;
-    if (d >= 4) {
-        for (uint32_t i = 0; i < d; i += 4) {
-            const float4 q = *reinterpret_cast<const float4*>(&sh[i]);
-            sq = __fadd_rn(sq, q.x); sq = __fadd_rn(sq, q.y); sq = __fadd_rn(sq, q.z); sq = __fadd_rn(sq, q.w);
-        }
-    } else {
-        for (uint32_t i = 0; i < d; i++) sq = __fadd_rn(sq, sh[i]);
-    }
-    const float norm = __fsqrt_rn(sq);
-    float v = xv;
-    if (norm > 0.0f) v = __fmul_rn(v, __fdiv_rn(1.0f, norm));
-    v = __fmul_rn(v, signs[lane]);
-    __syncthreads();
-    sh[lane] = v;
-    fwht_lds(sh, d, lane);
-    const float y = __fmul_rn(sh[lane], p.inv_sqrt_d);
+// ---- single-token Q / K / V preparation in one dispatch ---------------------------------------------------------
+// What layer.rs:393-450 issues as qk_norm (Q), rope (Q), qk_norm (K), rms_norm with unit weight (V), rope (K), two KV
+// encodes and the query rotation of quant_cache.rs:560-570 -- eight dispatches of a few hundred bytes each -- as one
+// kernel: workgroup b < n_q prepares query head b (norm, RoPE, f16 store, signs + FWHT -> f32 rq), the next n_kv
+// workgroups one K head each (norm, RoPE, f16 store, encode into the cache slot), the last n_kv one V head each
+// (unit-weight RMS norm, f16 store, encode).  Every value is rounded to f16 where the separate kernels store f16, and
+// the encode is the same code as encode_kv_kernel, so the codes are exactly those of the CPU encoder for the f16 rows
+// this kernel leaves in k / v.
+struct PrepareParams {
+    uint32_t head_dim, n_q_heads, n_kv_heads, bits, code_bytes, position, ring_capacity, write_kv;
+    float eps, theta, prf, inv_sqrt_d;
+};
 
-    const uint32_t k = 1u << p.bits;
-    uint32_t best = 0;
-    float bd = INFINITY;
-    for (uint32_t i = 0; i < k; ++i) {
-        const float dd = fabsf(__fsub_rn(y, levels[i]));
-        if (dd < bd) { bd = dd; best = i; }
+__global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k,
+                                                                        uint16_t* __restrict__ v, const uint16_t* __restrict__ q_norm_w,
+                                                                        const uint16_t* __restrict__ k_norm_w, const float* __restrict__ signs,
+                                                                        const float* __restrict__ levels, float* __restrict__ rq,
+                                                                        uint8_t* __restrict__ k_codes, uint16_t* __restrict__ k_norms,
+                                                                        uint8_t* __restrict__ v_codes, uint16_t* __restrict__ v_norms,
+                                                                        PrepareParams p) {
+    __shared__ __align__(16) float sh[kMaxHeadDim];
+    __shared__ uint32_t code_sh[kMaxHeadDim];
+    __shared__ uint16_t hbuf[kMaxHeadDim];
+    __shared__ float wsum[kMaxHeadDim / 64];
+    const uint32_t d = p.head_dim, lane = threadIdx.x, b = blockIdx.x;
+    const bool is_q = b < p.n_q_heads, is_k = !is_q && b < p.n_q_heads + p.n_kv_heads;
+    const uint32_t head = is_q ? b : (is_k ? b - p.n_q_heads : b - p.n_q_heads - p.n_kv_heads);
+    uint16_t* vec = (is_q ? q : (is_k ? k : v)) + (size_t)head * d;
+    const uint16_t* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+    const bool normalise = !(is_q || is_k) || norm_w != nullptr;          // V always (unit weight); Q / K when the layer has the weight
+
+    const uint16_t raw = vec[lane];
+    uint16_t h = raw;
+    if (normalise) {
+        const float x = lh_h2f(raw);
+        const float part = lh_group_sum(x * x, 64);
+        if ((lane & 63) == 0) wsum[lane >> 6] = part;
+        __syncthreads();
+        float ss = 0.0f;
+        for (uint32_t w = 0; w < d / 64; w++) ss += wsum[w];
+        const float rms = rsqrtf(ss / (float)d + p.eps);
+        h = lh_f2h(x * rms * (norm_w ? lh_h2f(norm_w[lane]) : 1.0f));
     }
-    code_sh[lane] = best;
-    if (lane == 0) norms[g] = lh_f2h_exact(norm);
-    __syncthreads();
-    if (lane < p.code_bytes) {     // one thread per output byte
-        uint32_t byte_val = 0;
-        for (uint32_t bitpos = 0; bitpos < 8; ++bitpos) {
-            const uint32_t global_bit = lane * 8 + bitpos, code_idx = global_bit / p.bits;
-            if (code_idx >= d) break;
-            byte_val |= ((code_sh[code_idx] >> (global_bit - code_idx * p.bits)) & 1u) << bitpos;
+    if (is_q || is_k) {                                                    // NEOX RoPE on the f16-rounded head (rope.metal:14-61)
+        hbuf[lane] = h;
+        __syncthreads();
+        const uint32_t half_dim = d / 2, rope_angles = (uint32_t)((float)d * p.prf) / 2;
+        if (lane < rope_angles) {
+            uint16_t o0, o1;
+            lh_rotate_pair(lh_h2f(hbuf[lane]), lh_h2f(hbuf[lane + half_dim]), lane, d, p.position, p.theta, o0, o1);
+            hbuf[lane] = o0;
+            hbuf[lane + half_dim] = o1;
         }
-        packed[(size_t)g * p.code_bytes + lane] = (uint8_t)byte_val;
+        __syncthreads();
+        h = hbuf[lane];
     }
+    vec[lane] = h;
+    const float xv = lh_h2f(h);
+    if (is_q) {                                                            // hadamard_rotate_hf with pre-sign (attention_flash_tq.metal:58-90)
+        sh[lane] = __fmul_rn(xv, signs[lane]);
+        fwht_lds(sh, d, lane);
+        rq[(size_t)head * d + lane] = __fmul_rn(sh[lane], p.inv_sqrt_d);
+        return;
+    }
+    if (!p.write_kv) return;
+    const uint32_t g = (p.ring_capacity ? p.position % p.ring_capacity : p.position) * p.n_kv_heads + head;
+    encode_vector(xv, lane, d, sh, code_sh, signs, levels, p.bits, p.code_bytes, p.inv_sqrt_d,
+                  (is_k ? k_codes : v_codes) + (size_t)g * p.code_bytes, (is_k ? k_norms : v_norms) + g);
 }
 
 struct DequantParams {
@@ -332,6 +411,47 @@ int lh_encode_kv_turboquant_batched_into(lh_batch* batch, const lh_buffer* input
     hipLaunchKernelGGL((encode_kv_kernel<true>), dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (const uint16_t*)input->ptr,
                        (const float*)levels->ptr, (const float*)signs->ptr, (uint8_t*)packed->ptr, (uint16_t*)norms->ptr,
                        (const uint32_t*)positions->ptr, p);
+    r = lh_check_launch(op);
+    if (r == LH_OK) batch->dispatch_count++;
+    return r;
+}
+
+int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm, const lh_buffer* k_norm,
+                               const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes, lh_buffer* k_norms,
+                               lh_buffer* v_codes, lh_buffer* v_norms, uint32_t head_dim, uint32_t n_q_heads, uint32_t n_kv_heads, float eps,
+                               uint32_t position, float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity) {
+    const char* op = "decode_qkv_prepare";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    int r = check_tq_shape(op, head_dim, bits);
+    if (r != LH_OK) return r;
+    LH_REQUIRE(head_dim >= 64, "%s: head_dim %u below 64", op, head_dim);
+    if (n_q_heads == 0) return LH_OK;
+    const bool write_kv = k != nullptr && v != nullptr && n_kv_heads != 0;
+    const uint32_t cb = lh_turboquant_code_bytes(head_dim, bits);
+    LH_NEED(q, (size_t)n_q_heads * head_dim * 2, op, "q");
+    LH_NEED(rq, (size_t)n_q_heads * head_dim * 4, op, "rq");
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    if (q_norm) LH_NEED(q_norm, (size_t)head_dim * 2, op, "q_norm");
+    if (write_kv) {
+        const uint64_t phys = (ring_capacity ? position % ring_capacity : position) + 1ull;
+        LH_NEED(k, (size_t)n_kv_heads * head_dim * 2, op, "k");
+        LH_NEED(v, (size_t)n_kv_heads * head_dim * 2, op, "v");
+        LH_NEED(levels, (size_t)4 << bits, op, "levels");
+        if (k_norm) LH_NEED(k_norm, (size_t)head_dim * 2, op, "k_norm");
+        LH_NEED(k_codes, (size_t)phys * n_kv_heads * cb, op, "k_codes");
+        LH_NEED(v_codes, (size_t)phys * n_kv_heads * cb, op, "v_codes");
+        LH_NEED(k_norms, (size_t)phys * n_kv_heads * 2, op, "k_norms");
+        LH_NEED(v_norms, (size_t)phys * n_kv_heads * 2, op, "v_norms");
+    }
+    PrepareParams p{head_dim, n_q_heads, write_kv ? n_kv_heads : 0u, bits, cb, position, ring_capacity, write_kv ? 1u : 0u,
+                    eps, theta, partial_rotary_factor, host_inv_sqrt(head_dim)};
+    const uint32_t groups = n_q_heads + (write_kv ? 2 * n_kv_heads : 0);
+    hipLaunchKernelGGL(decode_qkv_prepare_kernel, dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (uint16_t*)q->ptr,
+                       write_kv ? (uint16_t*)k->ptr : nullptr, write_kv ? (uint16_t*)v->ptr : nullptr,
+                       q_norm ? (const uint16_t*)q_norm->ptr : nullptr, (write_kv && k_norm) ? (const uint16_t*)k_norm->ptr : nullptr,
+                       (const float*)signs->ptr, write_kv ? (const float*)levels->ptr : nullptr, (float*)rq->ptr,
+                       write_kv ? (uint8_t*)k_codes->ptr : nullptr, write_kv ? (uint16_t*)k_norms->ptr : nullptr,
+                       write_kv ? (uint8_t*)v_codes->ptr : nullptr, write_kv ? (uint16_t*)v_norms->ptr : nullptr, p);
     r = lh_check_launch(op);
     if (r == LH_OK) batch->dispatch_count++;
     return r;

@@ -114,6 +114,28 @@ class QuantizedKvCache:
                                         window, self.bits, self.ring_capacity())
         kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
 
+    def prepare_token_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, position: int,
+                           n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:
+        """One dispatch for a decoded token's head norms, RoPE, V norm, ``write_kv_gpu_into`` (quant_cache.rs:391-444)
+        and the query rotation that opens ``fused_attention_into`` (quant_cache.rs:560-570); ``k = v = None`` leaves
+        the cache alone (a KV-shared layer)."""
+        if k is not None and position + 1 > self.max_positions:
+            raise InvalidArgument(f"KV write [{position}..{position + 1}) exceeds capacity {self.max_positions}")
+        kernels.decode_qkv_prepare_into(batch, q, k, v, q_norm, k_norm, self.levels, self.signs, rq,
+                                        self.keys_q, self.key_norms, self.values_q, self.value_norms, self.head_dim,
+                                        n_q_heads, self.n_kv_heads, eps, position, theta, partial_rotary_factor, self.bits,
+                                        self.ring_capacity())
+
+    def attention_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                                    seq_len: int, current_pos: int, n_q_heads: int, window: int) -> None:
+        """quant_cache.rs:571-598: the attend and rotate-back steps of ``fused_attention_into`` for a query that
+        ``prepare_token_into`` has already rotated."""
+        hd = self.head_dim
+        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
+                                        self.levels, vacc, hd, seq_len, current_pos, n_q_heads, self.n_kv_heads,
+                                        window, self.bits, self.ring_capacity())
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
+
     def fused_attention_batch_into(self, batch, kernels: Kernels, q: Buffer, rq: Buffer, vacc: Buffer,
                                    attn_out: Buffer, kv_len: int, start_pos: int, n_rows: int, n_q_heads: int,
                                    window: int, tiled: bool = True):

@@ -224,7 +224,9 @@ class TransformerLayer:
         else:
             kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
             w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
-        self._norm_rope(batch, kernels, s.q, w.q_norm, n_head, pos)
+        one_prepare = self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
+        if not one_prepare:
+            self._norm_rope(batch, kernels, s.q, w.q_norm, n_head, pos)
 
         # 2. own K/V into the TurboQuant cache, then attention over the codes
         if own_kv:
@@ -233,11 +235,18 @@ class TransformerLayer:
                                     [w.attn_k, w.attn_v], [s.k, s.v])
             else:
                 self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
+        if one_prepare:   # head norms, RoPE, V norm, both encodes and the query rotation in one dispatch
+            kv_cache.prepare_token_into(batch, kernels, s.q, s.k if own_kv else None, s.v if own_kv else None, w.q_norm,
+                                        w.k_norm, s.rq, position, n_head, eps, p.rope_theta, p.partial_rotary_factor)
+            kv_cache.attention_from_rotated_into(batch, kernels, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
+                                                 p.sliding_window)
+        elif own_kv:
             kernels.rms_norm_into(batch, s.v, s.ones, s.v, hd, n_kv, eps)   # V: RMS norm with unit weight
             self._norm_rope(batch, kernels, s.k, w.k_norm, n_kv, pos)
             kv_cache.write_kv_gpu_into(batch, kernels, s.k, s.v, position, 1)
-        kv_cache.fused_attention_into(batch, kernels, s.q, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
-                                      p.sliding_window)
+        if not one_prepare:
+            kv_cache.fused_attention_into(batch, kernels, s.q, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
+                                          p.sliding_window)
 
         # 3. output projection -> post_attention_norm + residual #1
         w.attn_output.matvec_into(batch, kernels, s.attn_out, s.ffn_out)

@@ -189,3 +189,79 @@ def test_bad_shapes_are_rejected(pkg, gpu):
     with pytest.raises(pkg.InvalidArgument):
         pkg.QuantizedKvCache(ctx, 1, 256, 100000, 2, physical_positions=600, sliding_window=512)   # ring too small
     assert batch.dispatch_count() == 0
+
+
+@pytest.mark.parametrize("hd,n_q,n_kv,bits,prf,with_norms,ring", [(256, 8, 1, 2, 1.0, True, 0), (512, 4, 2, 2, 0.25, True, 0),
+                                                                 (128, 4, 4, 4, 1.0, False, 0), (64, 2, 1, 3, 0.5, True, 0),
+                                                                 (256, 8, 1, 2, 1.0, True, 512)])
+def test_decode_qkv_prepare_equals_the_separate_kernels(pkg, gpu, oracle, hd, n_q, n_kv, bits, prf, with_norms, ring):
+    """One dispatch for qk_norm + rope on Q and K, unit-weight rms_norm on V, both KV encodes and the query rotation.
+    Checked stage by stage: q / k / v left behind against the glue oracle (f16 ulps), the codes and norms against the
+    CPU encoder applied to exactly those k / v rows (bit for bit), rq against the oracle's rotation of that q; and the
+    whole against the eight separate dispatches (q, k, v within an f16 ulp -- the RMS sums run in another order)."""
+    from oracle import layer_glue as G
+    ctx, K = gpu
+    g = pkg.synth.rng(61, hd + n_q + bits)
+    position, eps, theta = 777, 1e-6, 1e4
+    cap = ring if ring else 1024
+    q0 = (g.standard_normal(n_q * hd, dtype=np.float32) * 2).astype(np.float16)
+    k0 = (g.standard_normal(n_kv * hd, dtype=np.float32) * 2).astype(np.float16)
+    v0 = (g.standard_normal(n_kv * hd, dtype=np.float32) * 2).astype(np.float16)
+    qw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    kw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    levels, signs = oracle.tq_levels(hd, bits), oracle.rotation_signs(hd)
+    cb = oracle.tq_code_bytes(hd, bits)
+    lv, sg = pkg.Buffer.from_slice(ctx, levels), pkg.Buffer.from_slice(ctx, signs)
+    qwb, kwb = (pkg.Buffer.from_slice(ctx, qw), pkg.Buffer.from_slice(ctx, kw)) if with_norms else (None, None)
+
+    def fresh():
+        return dict(q=pkg.Buffer.from_slice(ctx, q0), k=pkg.Buffer.from_slice(ctx, k0), v=pkg.Buffer.from_slice(ctx, v0),
+                    rq=pkg.Buffer.empty(ctx, n_q * hd * 4), kc=pkg.Buffer.empty(ctx, cap * n_kv * cb),
+                    kn=pkg.Buffer.empty(ctx, cap * n_kv * 2), vc=pkg.Buffer.empty(ctx, cap * n_kv * cb),
+                    vn=pkg.Buffer.empty(ctx, cap * n_kv * 2))
+
+    a, b = fresh(), fresh()
+    batch = pkg.CommandBatch(ctx)
+    K.decode_qkv_prepare_into(batch, a["q"], a["k"], a["v"], qwb, kwb, lv, sg, a["rq"], a["kc"], a["kn"], a["vc"], a["vn"],
+                              hd, n_q, n_kv, eps, position, theta, prf, bits, ring)
+    assert batch.dispatch_count() == 1
+    ones = pkg.Buffer.from_slice(ctx, np.ones(hd, np.float16))
+    if with_norms:
+        K.qk_norm_gpu_into(batch, b["q"], qwb, hd, n_q, eps)
+        K.qk_norm_gpu_into(batch, b["k"], kwb, hd, n_kv, eps)
+    K.rope_into(batch, b["q"], b["q"], hd, position, theta, prf, n_q)
+    K.rope_into(batch, b["k"], b["k"], hd, position, theta, prf, n_kv)
+    K.rms_norm_into(batch, b["v"], ones, b["v"], hd, n_kv, eps)
+    K.encode_kv_turboquant_into(batch, b["k"], lv, sg, b["kc"], b["kn"], hd, n_kv, 1, bits, position, ring)
+    K.encode_kv_turboquant_into(batch, b["v"], lv, sg, b["vc"], b["vn"], hd, n_kv, 1, bits, position, ring)
+    K.hadamard_rotate_hf_into(batch, b["q"], sg, b["rq"], hd, n_q, True, False)
+    batch.commit_and_wait()
+
+    got = {n: a[n].as_array(np.float16) for n in ("q", "k", "v")}
+    want_q = G.rope(G.qk_norm(q0, qw, hd, n_q, eps) if with_norms else q0, hd, position, theta, prf, n_q)
+    want_k = G.rope(G.qk_norm(k0, kw, hd, n_kv, eps) if with_norms else k0, hd, position, theta, prf, n_kv)
+    want_v = G.rms_norm(v0, np.ones(hd, np.float16), hd, n_kv, eps)
+    for name, want in (("q", want_q), ("k", want_k), ("v", want_v)):
+        d = np.abs(got[name].astype(np.float32) - want.astype(np.float32))
+        assert d.max() <= 4e-3 * max(1.0, np.abs(want.astype(np.float32)).max()), (name, d.max())
+        sep = b[name].as_array(np.float16).astype(np.float32)
+        assert np.abs(got[name].astype(np.float32) - sep).max() <= 2e-3 * max(1.0, np.abs(sep).max()), name
+    # encode: bit exact for the rows this kernel left in k / v
+    slot = position % ring if ring else position
+    for rows, codes, norms in ((got["k"], a["kc"], a["kn"]), (got["v"], a["vc"], a["vn"])):
+        packed, nrm = np.zeros(cap * n_kv * cb, np.uint8), np.zeros(cap * n_kv, np.uint16)
+        oracle.tq_write_kv(rows.view(np.uint16), n_kv, hd, bits, signs, levels, position, ring, packed, nrm)
+        assert packed[slot * n_kv * cb:(slot + 1) * n_kv * cb].any()
+        assert np.array_equal(codes.as_array(np.uint8, cap * n_kv * cb), packed)
+        assert np.array_equal(norms.as_array(np.uint16, cap * n_kv), nrm)
+    want_rq = oracle.hadamard_rotate(got["q"].astype(np.float32), signs, hd, n_q, True, False)
+    assert np.abs(a["rq"].as_array(np.float32) - want_rq).max() <= 1e-5 * max(1.0, np.abs(want_rq).max())
+    # query only (a layer that reads another layer's cache): caches untouched
+    c = fresh()
+    batch = pkg.CommandBatch(ctx)
+    K.decode_qkv_prepare_into(batch, c["q"], None, None, qwb, None, lv, sg, c["rq"], None, None, None, None, hd, n_q, n_kv, eps,
+                              position, theta, prf, bits, ring)
+    batch.commit_and_wait()
+    assert np.array_equal(c["q"].as_array(np.uint16), a["q"].as_array(np.uint16))
+    assert np.array_equal(c["rq"].as_array(np.uint32), a["rq"].as_array(np.uint32))
+    assert not c["kc"].as_array(np.uint8).any()
