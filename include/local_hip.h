@@ -173,6 +173,14 @@ LH_API int lh_matvec_quant_grouped_into(lh_batch* batch, lh_quant fmt, uint32_t 
  * The transformed value is rounded to f16 exactly where the separate kernel would have stored it.
  * f16 vector and outputs; cols a multiple of 64 and 16-byte aligned operands, else INVALID_ARGUMENT. */
 typedef enum lh_prologue { LH_PROLOGUE_RMS_NORM = 1, LH_PROLOGUE_GELU_MUL = 2 } lh_prologue;
+/* The same for the norm chain between two sub-blocks of a layer (layer.rs:452-475, 484-510): the staged vector is
+ *   t = f16(rms_norm(vector) * weight + residual)           as rms_norm_add_into computes it (residual may be NULL),
+ *   then, when `next_weight` is given, f16(rms_norm(t) * next_weight)   as the following rms_norm_into would;
+ * `store` (optional) receives t, written once, for the later residual.  It may alias none of the other operands. */
+LH_API int lh_matvec_quant_norm_chain_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
+                                           const lh_buffer* vector, const lh_buffer* weight, const lh_buffer* residual,
+                                           const lh_buffer* next_weight, lh_buffer* store, float eps,
+                                           lh_buffer* const* outputs, uint32_t rows, uint32_t cols);
 LH_API int lh_matvec_quant_fused_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
                                       const lh_buffer* vector, int prologue, const lh_buffer* aux, float eps,
                                       lh_buffer* const* outputs, uint32_t rows, uint32_t cols);

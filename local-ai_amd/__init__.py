@@ -381,6 +381,16 @@ class Kernels:
                                                   C.c_int(prologue), aux._h, C.c_float(eps), _handles(outputs),
                                                   _u32(rows), _u32(cols)))
 
+    def matvec_quant_norm_chain_into(self, batch, fmt, matrices, vector, weight, residual, next_weight, store, eps, outputs,
+                                     rows, cols):
+        """Matvecs against t = rms_norm(vector) * weight + residual (as rms_norm_add_into rounds it), or against
+        rms_norm(t) * next_weight when that is given; `store` receives t.  `residual`, `next_weight`, `store` may be None."""
+        def h(b):
+            return b._h if b is not None else None
+        _check(self._l.lh_matvec_quant_norm_chain_into(batch._h, C.c_int(fmt), _u32(len(matrices)), _handles(matrices),
+                                                       vector._h, weight._h, h(residual), h(next_weight), h(store),
+                                                       C.c_float(eps), _handles(outputs), _u32(rows), _u32(cols)))
+
     # -- small-M / prefill matmul (kernels.rs:6378-6563, 5517-5568) --
     def matmul_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))

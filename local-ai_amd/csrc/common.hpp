@@ -68,13 +68,19 @@ static inline int lh_need(const lh_buffer* b, size_t bytes, const char* op, cons
 
 // Optional transform applied to an f16 activation vector while a matvec stages it (saves the dispatch of the kernel
 // that would otherwise have produced it): the value that is quantised is the f16 the separate kernel would have stored.
-//   kXProRmsNorm: x_i * rsqrt(mean(x^2) + eps) * aux_i   (rms_norm.metal:4-46; aux = norm weight, f16[K])
+//   kXProRmsNorm: t_i = x_i * rsqrt(mean(x^2) + eps) * aux_i (rms_norm.metal:4-46; aux = norm weight, f16[K]); with
+//                 `res` the residual is added before the one rounding (rms_norm.metal:48-88), the workgroup with
+//                 blockIdx.x == 0 stores that vector to `store` when given, and with `aux2` the staged vector is the
+//                 RMS norm of it with weight aux2 -- post-norm + residual followed by the next pre-norm.
 //   kXProGeluMul: gelu_tanh(x_i) * aux_i                 (gelu.metal:23-41; x = gate, aux = up, f16[K])
 enum : uint32_t { kXProNone = 0, kXProRmsNorm = 1, kXProGeluMul = 2 };
 struct XPrologue {
     uint32_t kind;
     const uint16_t* aux;
     float eps;
+    const uint16_t* res = nullptr;
+    const uint16_t* aux2 = nullptr;
+    uint16_t* store = nullptr;
 };
 
 // TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.

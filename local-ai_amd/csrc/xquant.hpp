@@ -16,6 +16,22 @@ __device__ __forceinline__ float lh_gelu_tanh_f32(float x) {   // gelu.metal:31-
     return 0.5f * x * (1.0f + t);
 }
 
+// Elements e0 .. e0 + 8 of f16(x * rms * aux (+ res)) as four packed words: the arithmetic of rms_norm_kernel<ADD>.
+__device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& pro, uint32_t e0, float rms, uint32_t (&packed)[4]) {
+    const uint16_t* x = static_cast<const uint16_t*>(xv);
+    const uint4 a = *reinterpret_cast<const uint4*>(x + e0), g = *reinterpret_cast<const uint4*>(pro.aux + e0);
+    uint4 r = make_uint4(0u, 0u, 0u, 0u);
+    if (pro.res != nullptr) r = *reinterpret_cast<const uint4*>(pro.res + e0);
+    const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float lo = lh_h2f((uint16_t)(wa[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
+        float hi = lh_h2f((uint16_t)(wa[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
+        if (pro.res != nullptr) { lo += lh_h2f((uint16_t)(wr[j] & 0xFFFF)); hi += lh_h2f((uint16_t)(wr[j] >> 16)); }
+        packed[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
+    }
+}
+
 // ---- activation quantisation into LDS ----------------------------------------
 // xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
 // xs[K/G]: float scale of each group of G elements (G = weight block size).
@@ -25,9 +41,18 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                                                   uint32_t nthreads, const XPrologue pro = XPrologue{kXProNone, nullptr, 0.0f}) {
     const int tid = threadIdx.x;
     const uint32_t kq = K >> 2;
-    float rms = 1.0f;
+    float rms = 1.0f, rms2 = 1.0f;
     if constexpr (sizeof(XT) == 2) {
         if (pro.kind == kXProRmsNorm) {   // uniform over the workgroup; xs doubles as the reduction scratch before it is filled
+            auto block_total = [&](float s) {
+                s = lh_group_sum(s, 64);
+                if ((tid & 63) == 0) xs[tid >> 6] = s;
+                __syncthreads();
+                float t = 0.0f;
+                for (uint32_t w = 0; w < nthreads / 64; w++) t += xs[w];
+                __syncthreads();
+                return t;
+            };
             float s = 0.0f;
             for (uint32_t e0 = tid * 8; e0 < K; e0 += nthreads * 8) {
                 const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
@@ -39,13 +64,23 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                     s += hi * hi;
                 }
             }
-            s = lh_group_sum(s, 64);
-            if ((tid & 63) == 0) xs[tid >> 6] = s;
-            __syncthreads();
-            float t = 0.0f;
-            for (uint32_t w = 0; w < nthreads / 64; w++) t += xs[w];
-            __syncthreads();
-            rms = rsqrtf(t / (float)K + pro.eps);
+            rms = rsqrtf(block_total(s) / (float)K + pro.eps);
+            if (pro.aux2 != nullptr || pro.store != nullptr) {   // the normalised (+ residual) vector: its mean square, and the one stored copy
+                float s2 = 0.0f;
+                for (uint32_t e0 = tid * 8; e0 < K; e0 += nthreads * 8) {
+                    uint32_t packed[4];
+                    xpro_norm_add8(x, pro, e0, rms, packed);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float lo = lh_h2f((uint16_t)(packed[i] & 0xFFFF)), hi = lh_h2f((uint16_t)(packed[i] >> 16));
+                        s2 += lo * lo;
+                        s2 += hi * hi;
+                    }
+                    if (pro.store != nullptr && blockIdx.x == 0)
+                        *reinterpret_cast<uint4*>(pro.store + e0) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+                }
+                if (pro.aux2 != nullptr) rms2 = rsqrtf(block_total(s2) / (float)K + pro.eps);
+            }
         }
     }
     for (uint32_t base = 0; base < K; base += nthreads * 8) {
@@ -67,16 +102,25 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                     v[2 * i] = lh_h2f((uint16_t)(w[i] & 0xFFFF));
                     v[2 * i + 1] = lh_h2f((uint16_t)(w[i] >> 16));
                 }
-                if (pro.kind != kXProNone) {
+                if (pro.kind == kXProRmsNorm) {
+                    uint32_t packed[4];
+                    xpro_norm_add8(x, pro, e0, rms, packed);
+                    uint4 g2 = make_uint4(0u, 0u, 0u, 0u);
+                    if (pro.aux2 != nullptr) g2 = *reinterpret_cast<const uint4*>(pro.aux2 + e0);
+                    const uint32_t wg2[4] = {g2.x, g2.y, g2.z, g2.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float t = lh_h2f((uint16_t)((packed[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
+                        if (pro.aux2 != nullptr) v[i] = lh_h2f(lh_f2h(t * rms2 * lh_h2f((uint16_t)((wg2[i >> 1] >> (16 * (i & 1))) & 0xFFFF))));
+                        else v[i] = t;
+                    }
+                } else if (pro.kind == kXProGeluMul) {
                     const uint4 b = *reinterpret_cast<const uint4*>(pro.aux + e0);
                     const uint32_t wb[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
                         const float g = lh_h2f((uint16_t)((wb[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
-                        float t;
-                        if (pro.kind == kXProRmsNorm) t = v[i] * rms * g;
-                        else t = lh_gelu_tanh_f32(v[i]) * g;
-                        v[i] = lh_h2f(lh_f2h(t));
+                        v[i] = lh_h2f(lh_f2h(lh_gelu_tanh_f32(v[i]) * g));
                     }
                 }
             }

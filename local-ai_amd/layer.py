@@ -94,9 +94,12 @@ class ScratchBuffers:
         q_elems = num_attention_heads * head_dim
         kv_elems = num_key_value_heads * head_dim
         self.normed = _alloc_f16(ctx, hidden_size)
-        self.q = _alloc_f16(ctx, q_elems)
-        self.k = _alloc_f16(ctx, kv_elems)
-        self.v = _alloc_f16(ctx, kv_elems)
+        # q, k, v are consecutive pieces of one allocation: a layer whose three projections were stacked into one
+        # matrix writes them with a single matvec (at that layer's own sizes, see TransformerLayer._qkv_views)
+        self.qkv = _alloc_f16(ctx, q_elems + 2 * kv_elems)
+        self.q = self.qkv.view(0, q_elems * 2)
+        self.k = self.qkv.view(q_elems * 2, kv_elems * 2)
+        self.v = self.qkv.view((q_elems + kv_elems) * 2, kv_elems * 2)
         self.rq = _alloc_f32(ctx, q_elems)
         self.vacc = _alloc_f32(ctx, q_elems)
         self.attn_out = _alloc_f16(ctx, q_elems)
@@ -149,15 +152,55 @@ class TransformerLayer:
     """layer.rs:330-873."""
 
     def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True,
-                 fuse_norm_rope: bool = True, fuse_prologues: bool = True):
+                 fuse_norm_rope: bool = True, fuse_prologues: bool = True, fuse_norm_chain: bool = True,
+                 stack_qkv: bool = True):
         self.params, self.weights = params, weights
         self.group_projections, self.fuse_norm_rope = group_projections, fuse_norm_rope
-        self.fuse_prologues = fuse_prologues
+        self.fuse_prologues, self.fuse_norm_chain = fuse_prologues, fuse_prologues and fuse_norm_chain
         # layer.rs:515-520 reads the scalar out of shared memory at every encode; the buffer lives in device
         # memory here, so it is fetched once.
         self._output_scale = None
         if weights.layer_output_scale is not None and weights.layer_output_scale.length() >= 2:
             self._output_scale = float(weights.layer_output_scale.as_array(np.float16, 1)[0])
+        self._qkv = None
+        if stack_qkv:
+            self._stack_qkv()
+
+    def _stack_qkv(self) -> None:
+        """Q, K and V projections of one format over the same input become the row blocks of one matrix (one
+        allocation, the three weights rebound to views of it), so a decoded token needs one matvec for all three."""
+        w = self.weights
+        q, k, v = w.attn_q, w.attn_k, w.attn_v
+        if self.params.is_kv_shared or k is None or v is None or q.ty == W_F16:
+            return
+        if not (q.ty == k.ty == v.ty and q.cols == k.cols == v.cols and q.cols % 64 == 0):
+            return
+        ctx = q.buf.ctx
+        sizes = [x.rows * x.row_bytes() for x in (q, k, v)]
+        stacked = Buffer.empty(ctx, sum(sizes))
+        from . import CommandBatch
+        batch = CommandBatch(ctx)
+        off = 0
+        for x, n in zip((q, k, v), sizes):
+            batch.blit_copy(x.buf, 0, stacked, off, n)
+            off += n
+        batch.commit_and_wait()
+        off = 0
+        for x, n in zip((q, k, v), sizes):
+            x.buf = stacked.view(off, n)
+            off += n
+        self._qkv = QuantWeight.quantized(stacked, q.ty, q.rows + k.rows + v.rows, q.cols)
+
+    def _qkv_views(self, scratch: "ScratchBuffers"):
+        """(q, k, v) views of scratch.qkv at this layer's sizes, consecutive (cached per scratch object)."""
+        cached = getattr(self, "_qkv_view_cache", None)
+        if cached is None or cached[0] is not scratch:
+            p = self.params
+            nq, nkv = p.num_attention_heads * p.head_dim * 2, p.num_key_value_heads * p.head_dim * 2
+            cached = (scratch, scratch.qkv.view(0, nq), scratch.qkv.view(nq, nkv), scratch.qkv.view(nq + nkv, nkv),
+                      scratch.qkv.view(0, nq + 2 * nkv))
+            self._qkv_view_cache = cached
+        return cached[1:]
 
     # ------------------------------------------------------------------ helpers
     def _pair_matvec(self, batch, kernels: Kernels, wa: QuantWeight, wb: QuantWeight, x: Buffer, out_a: Buffer,
@@ -219,42 +262,55 @@ class TransformerLayer:
         # 1. input_layernorm -> Q projection -> q_norm -> RoPE
         own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
         fused_in = self._fusable(w.attn_q) and (not own_kv or self._fusable(w.attn_k, w.attn_v))
-        if fused_in:
+        q_buf, k_buf, v_buf = s.q, s.k, s.v
+        stacked = fused_in and own_kv and self._qkv is not None
+        if stacked:   # one matvec over the stacked [Wq; Wk; Wv] writes q | k | v side by side
+            q_buf, k_buf, v_buf, qkv_out = self._qkv_views(s)
+            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [self._qkv], [qkv_out])
+        elif fused_in:
             self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [w.attn_q], [s.q])
         else:
             kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
             w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
         one_prepare = self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
         if not one_prepare:
-            self._norm_rope(batch, kernels, s.q, w.q_norm, n_head, pos)
+            self._norm_rope(batch, kernels, q_buf, w.q_norm, n_head, pos)
 
         # 2. own K/V into the TurboQuant cache, then attention over the codes
-        if own_kv:
+        if own_kv and not stacked:
             if fused_in:
                 self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm,
                                     [w.attn_k, w.attn_v], [s.k, s.v])
             else:
                 self._pair_matvec(batch, kernels, w.attn_k, w.attn_v, s.normed, s.k, s.v)
         if one_prepare:   # head norms, RoPE, V norm, both encodes and the query rotation in one dispatch
-            kv_cache.prepare_token_into(batch, kernels, s.q, s.k if own_kv else None, s.v if own_kv else None, w.q_norm,
-                                        w.k_norm, s.rq, position, n_head, eps, p.rope_theta, p.partial_rotary_factor)
+            kv_cache.prepare_token_into(batch, kernels, q_buf, k_buf if own_kv else None, v_buf if own_kv else None,
+                                        w.q_norm, w.k_norm, s.rq, position, n_head, eps, p.rope_theta,
+                                        p.partial_rotary_factor)
             kv_cache.attention_from_rotated_into(batch, kernels, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
                                                  p.sliding_window)
         elif own_kv:
-            kernels.rms_norm_into(batch, s.v, s.ones, s.v, hd, n_kv, eps)   # V: RMS norm with unit weight
-            self._norm_rope(batch, kernels, s.k, w.k_norm, n_kv, pos)
-            kv_cache.write_kv_gpu_into(batch, kernels, s.k, s.v, position, 1)
+            kernels.rms_norm_into(batch, v_buf, s.ones, v_buf, hd, n_kv, eps)   # V: RMS norm with unit weight
+            self._norm_rope(batch, kernels, k_buf, w.k_norm, n_kv, pos)
+            kv_cache.write_kv_gpu_into(batch, kernels, k_buf, v_buf, position, 1)
         if not one_prepare:
-            kv_cache.fused_attention_into(batch, kernels, s.q, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
+            kv_cache.fused_attention_into(batch, kernels, q_buf, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
                                           p.sliding_window)
 
         # 3. output projection -> post_attention_norm + residual #1
         w.attn_output.matvec_into(batch, kernels, s.attn_out, s.ffn_out)
-        kernels.rms_norm_add_into(batch, s.ffn_out, w.attn_post_norm, input, s.attn_resid, h, 1, eps)
+        chain_ffn = (self.fuse_norm_chain and self._fusable(w.ffn_gate, w.ffn_up) and self.group_projections
+                     and _groupable(w.ffn_gate, w.ffn_up))
+        if not chain_ffn:
+            kernels.rms_norm_add_into(batch, s.ffn_out, w.attn_post_norm, input, s.attn_resid, h, 1, eps)
 
         # 4. GeGLU feed-forward -> post_feedforward_norm + residual #2
         inter = p.intermediate_size
-        if self._fusable(w.ffn_gate, w.ffn_up):
+        if chain_ffn:   # residual #1 and the feed-forward pre-norm while gate / up stage their input; attn_resid kept
+            kernels.matvec_quant_norm_chain_into(batch, w.ffn_gate.ty, [w.ffn_gate.buf, w.ffn_up.buf], s.ffn_out,
+                                                 w.attn_post_norm, input, w.ffn_norm, s.attn_resid, eps, [s.gate, s.up],
+                                                 w.ffn_gate.rows, w.ffn_gate.cols)
+        elif self._fusable(w.ffn_gate, w.ffn_up):
             self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, s.attn_resid, w.ffn_norm,
                                 [w.ffn_gate, w.ffn_up], [s.gate, s.up])
         else:
@@ -265,13 +321,21 @@ class TransformerLayer:
         else:
             kernels.gelu_mul_into(batch, s.gate, s.up, s.gate, inter)
             w.ffn_down.matvec_into(batch, kernels, s.gate, s.ffn_out)
-        kernels.rms_norm_add_into(batch, s.ffn_out, w.ffn_post_norm, s.attn_resid, output, h, 1, eps)
+        has_ple = (w.per_layer_inp_gate is not None and w.per_layer_proj is not None
+                   and w.per_layer_post_norm is not None and per_layer_input is not None)
+        chain_ple = self.fuse_norm_chain and has_ple and self._fusable(w.per_layer_inp_gate) and output is not s.ffn_out
+        if not chain_ple:
+            kernels.rms_norm_add_into(batch, s.ffn_out, w.ffn_post_norm, s.attn_resid, output, h, 1, eps)
 
         # 5. per-layer input injection -> residual #3
-        if (w.per_layer_inp_gate is not None and w.per_layer_proj is not None and w.per_layer_post_norm is not None
-                and per_layer_input is not None):
+        if has_ple:
             pld = p.per_layer_dim
-            w.per_layer_inp_gate.matvec_into(batch, kernels, output, s.ple_h)
+            if chain_ple:   # residual #2 while the per-layer gate stages its input; `output` written once by that kernel
+                g = w.per_layer_inp_gate
+                kernels.matvec_quant_norm_chain_into(batch, g.ty, [g.buf], s.ffn_out, w.ffn_post_norm, s.attn_resid, None,
+                                                     output, eps, [s.ple_h], g.rows, g.cols)
+            else:
+                w.per_layer_inp_gate.matvec_into(batch, kernels, output, s.ple_h)
             if self._fusable(w.per_layer_proj):
                 # this layer's slice is read in place (no copy into scratch) while the projection stages its input
                 self._fused_matvecs(batch, kernels, kernels.PROLOGUE_GELU_MUL, s.ple_h, self._ple_slice(per_layer_input),

@@ -152,3 +152,42 @@ def test_matvec_fused_prologues(pkg, gpu, oracle, fmt, rows, cols, count):
                 assert np.array_equal(got.view(np.uint16), sep[i].as_array(np.uint16, rows))
     with pytest.raises(pkg.InvalidArgument):
         K.matvec_quant_fused_into(pkg.CommandBatch(ctx), ty, [ws[0].buf], xb, 7, ab, 1e-6, [outs[0]], rows, cols)
+
+
+@pytest.mark.parametrize("fmt,rows,cols,count", [("q4_0", 256, 2048, 1), ("tq2_0", 8192, 2048, 2), ("tq2_0", 300, 512, 2),
+                                                 ("q4_0", 64, 8192, 1)])
+@pytest.mark.parametrize("second_norm", [True, False])
+def test_matvec_norm_chain(pkg, gpu, oracle, fmt, rows, cols, count, second_norm):
+    """matvec_quant_norm_chain_into: t = rms_norm(x) * w1 + residual (stored once), then optionally rms_norm(t) * w2,
+    staged by the matvec itself (layer.rs:452-475 / 484-510 as one dispatch).  The stored vector and the products are
+    held to the oracle's composition of the glue restatements and the f64 dot."""
+    from oracle import layer_glue as G
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(33, rows + cols + count)
+    raws = [refgen.q4_0_payload(rows, cols, 0x91 + i) if fmt == "q4_0" else refgen.tq2_0_payload(rows, cols, 0x91 + i)
+            for i in range(count)]
+    dqs = [(oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32)(r, rows, cols) for r in raws]
+    ws = [pkg.QuantWeight.from_bytes(ctx, r, ty, rows, cols) for r in raws]
+    x = (g.standard_normal(cols, dtype=np.float32) * 0.7).astype(np.float16)
+    res = g.standard_normal(cols, dtype=np.float32).astype(np.float16)
+    w1 = (1.0 + 0.2 * g.standard_normal(cols, dtype=np.float32)).astype(np.float16)
+    w2 = (1.0 + 0.2 * g.standard_normal(cols, dtype=np.float32)).astype(np.float16)
+    xb, rb, w1b, w2b = (pkg.Buffer.from_slice(ctx, a) for a in (x, res, w1, w2))
+    store = pkg.Buffer.empty(ctx, cols * 2)
+    outs = [pkg.Buffer.empty(ctx, rows * 2) for _ in range(count)]
+    batch = pkg.CommandBatch(ctx)
+    K.matvec_quant_norm_chain_into(batch, ty, [w.buf for w in ws], xb, w1b, rb, w2b if second_norm else None, store, 1e-6,
+                                   outs, rows, cols)
+    assert batch.dispatch_count() == 1
+    batch.commit_and_wait()
+    t = G.rms_norm(x, w1, cols, 1, 1e-6, residual=res)
+    got_t = store.as_array(np.float16, cols)
+    assert np.abs(got_t.astype(np.float32) - t.astype(np.float32)).max() <= 4e-3 * max(1.0, np.abs(t.astype(np.float32)).max())
+    # continue from the vector the kernel stored (what it staged is a function of exactly these f16 values)
+    staged = G.rms_norm(got_t, w2, cols, 1, 1e-6) if second_norm else got_t
+    for i in range(count):
+        want = oracle.matvec_f64(dqs[i], staged.astype(np.float32)).astype(np.float32)
+        refgen.assert_close(outs[i].as_array(np.float16, rows).astype(np.float32), want, 2e-3, f"{fmt} norm chain #{i}")
+    with pytest.raises(pkg.InvalidArgument):     # the stored vector may not alias an input
+        K.matvec_quant_norm_chain_into(pkg.CommandBatch(ctx), ty, [ws[0].buf], xb, w1b, rb, None, xb, 1e-6, [outs[0]], rows, cols)
