@@ -366,7 +366,7 @@ def fill_kv(pkg, ctx, K, cache, lanes, T, g):
     batch.commit_and_wait()
 
 
-def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3):
+def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3, graphs=True):
     """Whole decoder layers end to end (norms, Q/K/V projections, RoPE, KV encode, attention over the tq2 cache,
     output projection, GeGLU feed-forward, per-layer input injection) at hidden 2048, FFN 8192, 8 query heads over
     1 KV head of 256, Q4_0 attention and TQ2_0 feed-forward weights, context T.  A step runs `n_layers` distinct
@@ -388,10 +388,10 @@ def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, l
     batch = pkg.CommandBatch(ctx)
     kv_bytes = T * (2 * 64 + 4)
     if "single" in which:
-        res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes)
+        res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs)
     if "lanes" in which:
         res["lanes"] = _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g,
-                                     kv_bytes)
+                                     kv_bytes, graphs)
     return res
 
 
@@ -399,7 +399,7 @@ def _layer_weight_bytes(pkg, layer):
     return sum(w.device_bytes() for w in vars(layer.weights).values() if isinstance(w, pkg.QuantWeight))
 
 
-def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes):
+def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs):
     pld = 256
     layers = [make_layer(i) for i in range(n_layers)]
     wbytes = _layer_weight_bytes(pkg, layers[0])
@@ -425,6 +425,12 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
     out = hidden[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("decode step produced non-finite hidden state")
+    res = {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
+           "dispatches_per_layer": per_layer, "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
+           "gbs_events": (wbytes + kv_bytes) / (ev / n_layers) * 1e-6,
+           "tokens_per_s_35_layers": 1.0 / (ev * 1e-3 / n_layers * 35)}
+    if not graphs:
+        return res
     # The same step through the position-in-a-buffer path (one lane of forward_decode_batch_turbo), recorded once into a
     # graph and replayed: one host call per step instead of one per dispatch.
     L = pkg.layer
@@ -453,17 +459,13 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
     gout = gbufs[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
     if not np.isfinite(gout).all() or np.abs(gout - out).max() > 0.05 * max(1.0, np.abs(out).max()):
         raise RuntimeError("graph replay of the decode step disagrees with the eager step")
-    return {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
-                     "dispatches_per_layer": per_layer,
-                     "graph_us_per_layer_events": gev * 1e3 / n_layers, "graph_us_per_layer_wall": gwall * 1e3 / n_layers,
-                     "graph_dispatches_per_layer": graph.dispatch_count() // n_layers,
-                     "graph_tokens_per_s_35_layers": 1.0 / (gev * 1e-3 / n_layers * 35),
-                     "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
-                     "gbs_events": (wbytes + kv_bytes) / (ev / n_layers) * 1e-6,
-                     "tokens_per_s_35_layers": 1.0 / (ev * 1e-3 / n_layers * 35)}
+    res.update({"graph_us_per_layer_events": gev * 1e3 / n_layers, "graph_us_per_layer_wall": gwall * 1e3 / n_layers,
+                "graph_dispatches_per_layer": graph.dispatch_count() // n_layers,
+                "graph_tokens_per_s_35_layers": 1.0 / (gev * 1e-3 / n_layers * 35)})
+    return res
 
 
-def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g, kv_bytes):
+def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g, kv_bytes, graphs):
     pld = 256
     layers = [make_layer(i) for i in range(lane_layers)]
     wbytes = _layer_weight_bytes(pkg, layers[0])
@@ -488,6 +490,12 @@ def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer,
     out = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("batched decode step produced non-finite hidden state")
+    res = {"lanes": lanes, "layers_per_step": lane_layers, "us_per_layer_events": ev * 1e3 / lane_layers,
+           "us_per_layer_wall": wall * 1e3 / lane_layers, "kv_bytes_per_layer": lanes * kv_bytes,
+           "gbs_events": (wbytes + lanes * kv_bytes) / (ev / lane_layers) * 1e-6,
+           "tokens_per_s_35_layers": lanes / (ev * 1e-3 / lane_layers * 35)}
+    if not graphs:
+        return res
     batch.commit_and_wait()
     batch.begin_capture()
     step_lanes()
@@ -496,12 +504,9 @@ def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer,
     gout = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
     if not np.array_equal(gout, out):
         raise RuntimeError("graph replay of the batched decode step disagrees with the eager step")
-    return {"lanes": lanes, "layers_per_step": lane_layers, "us_per_layer_events": ev * 1e3 / lane_layers,
-                    "us_per_layer_wall": wall * 1e3 / lane_layers, "kv_bytes_per_layer": lanes * kv_bytes,
-                    "graph_us_per_layer_events": gev * 1e3 / lane_layers,
-                    "graph_tokens_per_s_35_layers": lanes / (gev * 1e-3 / lane_layers * 35),
-                    "gbs_events": (wbytes + lanes * kv_bytes) / (ev / lane_layers) * 1e-6,
-                    "tokens_per_s_35_layers": lanes / (ev * 1e-3 / lane_layers * 35)}
+    res.update({"graph_us_per_layer_events": gev * 1e3 / lane_layers,
+                "graph_tokens_per_s_35_layers": lanes / (gev * 1e-3 / lane_layers * 35)})
+    return res
 
 
 def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
@@ -531,6 +536,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
+    ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
@@ -607,7 +613,7 @@ def main():
 
     if legs & {"decode", "lanes"}:
         which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else [])
-        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which)
+        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
