@@ -38,7 +38,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/matvec_tq2_mfma_grouped_8192x2048.md), scaled by the same counters on the library's plain
 # copy kernel; None until that profile has been taken for the current kernel.
-MEASURED_TRAFFIC_BYTES = 1086338150
+MEASURED_TRAFFIC_BYTES = 1089494324
 
 
 def log(*a):
@@ -372,7 +372,8 @@ def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, l
     1 KV head of 256, Q4_0 attention and TQ2_0 feed-forward weights, context T.  A step runs `n_layers` distinct
     layers back to back (18.9 MB of weights and a cache of their own each, so nothing is served from the last-level
     cache twice), the output of one feeding the next, as a model's decode step does.  `which`: "single" (one
-    sequence, one token per step) and / or "lanes" (continuous batching, one token of each of `lanes` sequences)."""
+    sequence, one token per step), "lanes" (continuous batching, one token of each of `lanes` sequences) and / or
+    "chunk" (a 256-token prefill chunk through forward_batch)."""
     L = pkg.layer
     dims = dict(hidden_size=2048, intermediate_size=8192, num_attention_heads=8, num_key_value_heads=1, head_dim=256)
     pld = 256
@@ -389,9 +390,42 @@ def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, l
     kv_bytes = T * (2 * 64 + 4)
     if "single" in which:
         res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs)
+    if "chunk" in which:
+        res["prefill_chunk"] = _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g)
     if "lanes" in which:
         res["lanes"] = _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer, scratch, batch, g,
                                      kv_bytes, graphs)
+    return res
+
+
+def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g, rows=256, n_layers=4):
+    """forward_batch over one prefill chunk (`rows` prompt tokens, the reference's MAX_PREFILL_CHUNK) through
+    `n_layers` distinct layers: at the start of a prompt, and as the last chunk of a T-token prompt (attention over the
+    whole cache)."""
+    pld = 256
+    layers = [make_layer(i) for i in range(n_layers)]
+    caches = []
+    for i in range(n_layers):
+        c = pkg.QuantizedKvCache(ctx, 1, 256, T)
+        fill_kv(pkg, ctx, K, c, 1, T, pkg.synth.rng(12, 300 + i))
+        caches.append(c)
+    bs = pkg.layer.BatchScratch(ctx, rows, 2048, 8192, 8, 1, 256, pld, n_layers)
+    xin = pkg.Buffer.from_slice(ctx, g.standard_normal(rows * 2048, dtype=np.float32).astype(np.float16))
+    ple_all = pkg.Buffer.from_slice(ctx, g.standard_normal(rows * n_layers * pld, dtype=np.float32).astype(np.float16))
+    bufs = (bs.hidden_a, bs.hidden_b)
+    res = {"rows": rows, "layers_per_step": n_layers}
+    for name, start in (("first_chunk", 0), ("last_chunk_of_%d" % T, T - rows)):
+        def step():
+            batch.blit_copy(xin, 0, bs.hidden_a, 0, rows * 4096)
+            for i, layer in enumerate(layers):
+                layer.forward_batch(K, batch, rows, start, bufs[i & 1], bufs[(i + 1) & 1], bs, scratch.ones, caches[i],
+                                    (ple_all, n_layers))
+        wall, ev = time_steps(pkg, ctx, step, steps, warmup)
+        out = bufs[n_layers & 1].as_array(np.float16, rows * 2048).astype(np.float32)
+        if not np.isfinite(out).all():
+            raise RuntimeError("prefill chunk produced non-finite hidden state")
+        res[name] = {"us_per_layer_events": ev * 1e3 / n_layers,
+                     "prompt_tokens_per_s_35_layers": rows / (ev * 1e-3 / n_layers * 35)}
     return res
 
 
@@ -538,7 +572,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes",
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -611,8 +645,9 @@ def main():
         extra["layer_glue_kernels"] = bench_glue(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] glue:", extra["layer_glue_kernels"])
 
-    if legs & {"decode", "lanes"}:
-        which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else [])
+    if legs & {"decode", "lanes", "chunk"}:
+        which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else []) + \
+            (["chunk"] if "chunk" in legs else [])
         extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
