@@ -58,7 +58,8 @@ struct Tq2Base {
 
 __device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
     typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
-    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p);
+    // weights are read once per launch: a streaming load keeps them from displacing the activations in the caches
+    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p));
 }
 
 // 16 bytes starting `SH` bytes into the 32-byte pair (c0, c1).
