@@ -9,6 +9,14 @@
 
 namespace {
 
+// Weights are read once per launch: a streaming (non-temporal) 16-byte load.
+__device__ __forceinline__ uint4 lh_ld16_stream(const uint16_t* p) {
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+
 constexpr int kMaxLdsCols = 12288;   // 48 KB of f32 activations
 
 template <typename XT> __device__ __forceinline__ float x_at(const XT* x, uint32_t i);
@@ -34,7 +42,7 @@ __global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restr
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
                     const uint32_t k = k0 + 512 * c;
-                    v[c] = k < cols ? *reinterpret_cast<const uint4*>(wr + k) : make_uint4(0u, 0u, 0u, 0u);
+                    v[c] = k < cols ? lh_ld16_stream(wr + k) : make_uint4(0u, 0u, 0u, 0u);
                 }
 #pragma unroll
                 for (int c = 0; c < 8; c++) {
