@@ -360,6 +360,19 @@ LH_API int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* 
                                       lh_buffer* k_codes, lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms,
                                       uint32_t head_dim, uint32_t n_q_heads, uint32_t n_kv_heads, float eps, uint32_t position,
                                       float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity);
+/* The same for `rows` tokens at once (the eight dispatches of layer.rs:568-616 / 763-800 + quant_cache.rs:620-660 /
+ * quant_unified_pool.rs:138-230): q [rows, n_q_heads, head_dim], k / v [rows, n_kv_heads, head_dim], rq [rows, n_q_heads,
+ * head_dim] f32.  With `positions` == NULL (and lane_capacity 0) row r is the token at start_position + r of one
+ * sequence (rope_batch_into / encode_kv_turboquant_into addressing); with a device table `positions[rows]` row r is one
+ * token of lane r at positions[r], written into the lane's region of `lane_capacity` rows (rope_batch_decode_into /
+ * encode_kv_turboquant_batched_into addressing). */
+LH_API int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm,
+                                           const lh_buffer* k_norm, const lh_buffer* levels, const lh_buffer* signs,
+                                           lh_buffer* rq, lh_buffer* k_codes, lh_buffer* k_norms, lh_buffer* v_codes,
+                                           lh_buffer* v_norms, const lh_buffer* positions, uint32_t head_dim,
+                                           uint32_t n_q_heads, uint32_t n_kv_heads, uint32_t rows, float eps,
+                                           uint32_t start_position, float theta, float partial_rotary_factor, uint32_t bits,
+                                           uint32_t ring_capacity, uint32_t lane_capacity);
 /* kernels.rs:5032-5163 hadamard_rotate{,_hf,_fh}_into,
  * shaders/attention_flash_tq.metal:58-139: per head optional sign flip, FWHT,
  * 1/sqrt(d), optional sign flip.  f32->f32, f16->f32, f32->f16. */

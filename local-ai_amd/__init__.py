@@ -559,6 +559,20 @@ class Kernels:
                                                   C.c_float(theta), C.c_float(partial_rotary_factor), _u32(bits),
                                                   _u32(ring_capacity)))
 
+    def decode_qkv_prepare_rows_into(self, batch, q, k, v, q_norm, k_norm, levels, signs, rq, k_codes, k_norms, v_codes,
+                                     v_norms, positions, head_dim, n_q_heads, n_kv_heads, rows, eps, start_position, theta,
+                                     partial_rotary_factor, bits, ring_capacity, lane_capacity):
+        """decode_qkv_prepare_into for `rows` tokens: consecutive positions of one sequence from `start_position`
+        (positions None, lane_capacity 0), or one token per lane at the device table `positions`."""
+        def h(b):
+            return b._h if b is not None else None
+        _check(self._l.lh_decode_qkv_prepare_rows_into(batch._h, q._h, h(k), h(v), h(q_norm), h(k_norm), levels._h, signs._h,
+                                                       rq._h, h(k_codes), h(k_norms), h(v_codes), h(v_norms), h(positions),
+                                                       _u32(head_dim), _u32(n_q_heads), _u32(n_kv_heads), _u32(rows),
+                                                       C.c_float(eps), _u32(start_position), C.c_float(theta),
+                                                       C.c_float(partial_rotary_factor), _u32(bits), _u32(ring_capacity),
+                                                       _u32(lane_capacity)))
+
     def hadamard_rotate_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
         _check(self._l.lh_hadamard_rotate_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
                                                _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))

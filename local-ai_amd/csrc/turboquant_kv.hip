@@ -135,8 +135,11 @@ __global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* 
 // (unit-weight RMS norm, f16 store, encode).  Every value is rounded to f16 where the separate kernels store f16, and
 // the encode is the same code as encode_kv_kernel, so the codes are exactly those of the CPU encoder for the f16 rows
 // this kernel leaves in k / v.
+// Several rows at once: row r is the token at position `position + r` of one sequence (lane_capacity == 0; a prefill
+// chunk or a verify batch), or one token of lane r at positions[r], whose cache region starts lane_capacity rows
+// after the previous lane's (continuous batching; the addressing of encode_kv_turboquant_batched).
 struct PrepareParams {
-    uint32_t head_dim, n_q_heads, n_kv_heads, bits, code_bytes, position, ring_capacity, write_kv;
+    uint32_t head_dim, n_q_heads, n_kv_heads, bits, code_bytes, position, ring_capacity, write_kv, lane_capacity;
     float eps, theta, prf, inv_sqrt_d;
 };
 
@@ -146,15 +149,18 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
                                                                         const float* __restrict__ levels, float* __restrict__ rq,
                                                                         uint8_t* __restrict__ k_codes, uint16_t* __restrict__ k_norms,
                                                                         uint8_t* __restrict__ v_codes, uint16_t* __restrict__ v_norms,
-                                                                        PrepareParams p) {
+                                                                        const uint32_t* __restrict__ positions, PrepareParams p) {
     __shared__ __align__(16) float sh[kMaxHeadDim];
     __shared__ uint32_t code_sh[kMaxHeadDim];
     __shared__ uint16_t hbuf[kMaxHeadDim];
     __shared__ float wsum[kMaxHeadDim / 64];
-    const uint32_t d = p.head_dim, lane = threadIdx.x, b = blockIdx.x;
+    const uint32_t d = p.head_dim, lane = threadIdx.x;
+    const uint32_t per_row = p.n_q_heads + 2 * p.n_kv_heads;            // n_kv_heads is 0 when the cache is not written
+    const uint32_t row = blockIdx.x / per_row, b = blockIdx.x - row * per_row;
+    const uint32_t position = positions ? positions[row] : p.position + row;
     const bool is_q = b < p.n_q_heads, is_k = !is_q && b < p.n_q_heads + p.n_kv_heads;
     const uint32_t head = is_q ? b : (is_k ? b - p.n_q_heads : b - p.n_q_heads - p.n_kv_heads);
-    uint16_t* vec = (is_q ? q : (is_k ? k : v)) + (size_t)head * d;
+    uint16_t* vec = (is_q ? q : (is_k ? k : v)) + ((size_t)row * (is_q ? p.n_q_heads : p.n_kv_heads) + head) * d;
     const uint16_t* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
     const bool normalise = !(is_q || is_k) || norm_w != nullptr;          // V always (unit weight); Q / K when the layer has the weight
 
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
         const uint32_t half_dim = d / 2, rope_angles = (uint32_t)((float)d * p.prf) / 2;
         if (lane < rope_angles) {
             uint16_t o0, o1;
-            lh_rotate_pair(lh_h2f(hbuf[lane]), lh_h2f(hbuf[lane + half_dim]), lane, d, p.position, p.theta, o0, o1);
+            lh_rotate_pair(lh_h2f(hbuf[lane]), lh_h2f(hbuf[lane + half_dim]), lane, d, position, p.theta, o0, o1);
             hbuf[lane] = o0;
             hbuf[lane + half_dim] = o1;
         }
@@ -188,11 +194,12 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     if (is_q) {                                                            // hadamard_rotate_hf with pre-sign (attention_flash_tq.metal:58-90)
         sh[lane] = __fmul_rn(xv, signs[lane]);
         fwht_lds(sh, d, lane);
-        rq[(size_t)head * d + lane] = __fmul_rn(sh[lane], p.inv_sqrt_d);
+        rq[((size_t)row * p.n_q_heads + head) * d + lane] = __fmul_rn(sh[lane], p.inv_sqrt_d);
         return;
     }
     if (!p.write_kv) return;
-    const uint32_t g = (p.ring_capacity ? p.position % p.ring_capacity : p.position) * p.n_kv_heads + head;
+    const uint32_t slot = p.ring_capacity ? position % p.ring_capacity : position;
+    const uint32_t g = (row * p.lane_capacity + slot) * p.n_kv_heads + head;   // lane_capacity == 0: one sequence, slot alone
     encode_vector(xv, lane, d, sh, code_sh, signs, levels, p.bits, p.code_bytes, p.inv_sqrt_d,
                   (is_k ? k_codes : v_codes) + (size_t)g * p.code_bytes, (is_k ? k_norms : v_norms) + g);
 }
@@ -416,26 +423,33 @@ int lh_encode_kv_turboquant_batched_into(lh_batch* batch, const lh_buffer* input
     return r;
 }
 
-int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm, const lh_buffer* k_norm,
-                               const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes, lh_buffer* k_norms,
-                               lh_buffer* v_codes, lh_buffer* v_norms, uint32_t head_dim, uint32_t n_q_heads, uint32_t n_kv_heads, float eps,
-                               uint32_t position, float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity) {
+int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm,
+                                    const lh_buffer* k_norm, const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes,
+                                    lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms, const lh_buffer* positions, uint32_t head_dim,
+                                    uint32_t n_q_heads, uint32_t n_kv_heads, uint32_t rows, float eps, uint32_t start_position, float theta,
+                                    float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity, uint32_t lane_capacity) {
     const char* op = "decode_qkv_prepare";
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     int r = check_tq_shape(op, head_dim, bits);
     if (r != LH_OK) return r;
     LH_REQUIRE(head_dim >= 64, "%s: head_dim %u below 64", op, head_dim);
-    if (n_q_heads == 0) return LH_OK;
+    if (n_q_heads == 0 || rows == 0) return LH_OK;
+    LH_REQUIRE((positions != nullptr) == (lane_capacity != 0), "%s: a positions table and a lane capacity go together", op);
+    LH_REQUIRE(ring_capacity <= lane_capacity || lane_capacity == 0, "%s: ring_capacity %u exceeds lane_capacity %u", op, ring_capacity, lane_capacity);
     const bool write_kv = k != nullptr && v != nullptr && n_kv_heads != 0;
     const uint32_t cb = lh_turboquant_code_bytes(head_dim, bits);
-    LH_NEED(q, (size_t)n_q_heads * head_dim * 2, op, "q");
-    LH_NEED(rq, (size_t)n_q_heads * head_dim * 4, op, "rq");
+    LH_NEED(q, (size_t)rows * n_q_heads * head_dim * 2, op, "q");
+    LH_NEED(rq, (size_t)rows * n_q_heads * head_dim * 4, op, "rq");
     LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
     if (q_norm) LH_NEED(q_norm, (size_t)head_dim * 2, op, "q_norm");
+    if (positions) LH_NEED(positions, (size_t)rows * 4, op, "positions");
     if (write_kv) {
-        const uint64_t phys = (ring_capacity ? position % ring_capacity : position) + 1ull;
-        LH_NEED(k, (size_t)n_kv_heads * head_dim * 2, op, "k");
-        LH_NEED(v, (size_t)n_kv_heads * head_dim * 2, op, "v");
+        // one sequence: rows land at start_position .. + rows (modulo the ring); lanes: positions live in device memory,
+        // so the slot range cannot be checked here beyond the pool size
+        const uint64_t last = (uint64_t)start_position + rows;
+        const uint64_t phys = lane_capacity ? (uint64_t)rows * lane_capacity : (ring_capacity ? std::min<uint64_t>(ring_capacity, last) : last);
+        LH_NEED(k, (size_t)rows * n_kv_heads * head_dim * 2, op, "k");
+        LH_NEED(v, (size_t)rows * n_kv_heads * head_dim * 2, op, "v");
         LH_NEED(levels, (size_t)4 << bits, op, "levels");
         if (k_norm) LH_NEED(k_norm, (size_t)head_dim * 2, op, "k_norm");
         LH_NEED(k_codes, (size_t)phys * n_kv_heads * cb, op, "k_codes");
@@ -443,18 +457,28 @@ int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_b
         LH_NEED(k_norms, (size_t)phys * n_kv_heads * 2, op, "k_norms");
         LH_NEED(v_norms, (size_t)phys * n_kv_heads * 2, op, "v_norms");
     }
-    PrepareParams p{head_dim, n_q_heads, write_kv ? n_kv_heads : 0u, bits, cb, position, ring_capacity, write_kv ? 1u : 0u,
+    PrepareParams p{head_dim, n_q_heads, write_kv ? n_kv_heads : 0u, bits, cb, start_position, ring_capacity, write_kv ? 1u : 0u, lane_capacity,
                     eps, theta, partial_rotary_factor, host_inv_sqrt(head_dim)};
-    const uint32_t groups = n_q_heads + (write_kv ? 2 * n_kv_heads : 0);
-    hipLaunchKernelGGL(decode_qkv_prepare_kernel, dim3(groups), dim3(head_dim), 0, batch->ctx->stream, (uint16_t*)q->ptr,
+    const uint64_t groups = (uint64_t)rows * (n_q_heads + (write_kv ? 2 * n_kv_heads : 0));
+    LH_REQUIRE(groups <= 0x7FFFFFFFull, "%s: %u rows are too many for one launch", op, rows);
+    hipLaunchKernelGGL(decode_qkv_prepare_kernel, dim3((uint32_t)groups), dim3(head_dim), 0, batch->ctx->stream, (uint16_t*)q->ptr,
                        write_kv ? (uint16_t*)k->ptr : nullptr, write_kv ? (uint16_t*)v->ptr : nullptr,
                        q_norm ? (const uint16_t*)q_norm->ptr : nullptr, (write_kv && k_norm) ? (const uint16_t*)k_norm->ptr : nullptr,
                        (const float*)signs->ptr, write_kv ? (const float*)levels->ptr : nullptr, (float*)rq->ptr,
                        write_kv ? (uint8_t*)k_codes->ptr : nullptr, write_kv ? (uint16_t*)k_norms->ptr : nullptr,
-                       write_kv ? (uint8_t*)v_codes->ptr : nullptr, write_kv ? (uint16_t*)v_norms->ptr : nullptr, p);
+                       write_kv ? (uint8_t*)v_codes->ptr : nullptr, write_kv ? (uint16_t*)v_norms->ptr : nullptr,
+                       positions ? (const uint32_t*)positions->ptr : nullptr, p);
     r = lh_check_launch(op);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
+}
+
+int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm, const lh_buffer* k_norm,
+                               const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes, lh_buffer* k_norms,
+                               lh_buffer* v_codes, lh_buffer* v_norms, uint32_t head_dim, uint32_t n_q_heads, uint32_t n_kv_heads, float eps,
+                               uint32_t position, float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity) {
+    return lh_decode_qkv_prepare_rows_into(batch, q, k, v, q_norm, k_norm, levels, signs, rq, k_codes, k_norms, v_codes, v_norms, nullptr,
+                                           head_dim, n_q_heads, n_kv_heads, 1, eps, position, theta, partial_rotary_factor, bits, ring_capacity, 0);
 }
 
 int lh_dequantize_kv_turboquant_into(lh_batch* batch, const lh_buffer* packed, const lh_buffer* norms, const lh_buffer* levels,

@@ -136,6 +136,25 @@ class QuantizedKvCache:
                                         window, self.bits, self.ring_capacity())
         kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
 
+    def prepare_rows_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, start_pos: int,
+                          n_rows: int, n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:
+        """``prepare_token_into`` for the ``n_rows`` consecutive tokens of a prefill chunk."""
+        if k is not None and start_pos + n_rows > self.max_positions:
+            raise InvalidArgument(f"KV write [{start_pos}..{start_pos + n_rows}) exceeds capacity {self.max_positions}")
+        kernels.decode_qkv_prepare_rows_into(batch, q, k, v, q_norm, k_norm, self.levels, self.signs, rq, self.keys_q,
+                                             self.key_norms, self.values_q, self.value_norms, None, self.head_dim,
+                                             n_q_heads, self.n_kv_heads, n_rows, eps, start_pos, theta,
+                                             partial_rotary_factor, self.bits, self.ring_capacity(), 0)
+
+    def attention_rows_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                                         kv_len: int, start_pos: int, n_rows: int, n_q_heads: int, window: int) -> None:
+        """quant_cache.rs:660-700: the attend and rotate-back steps of ``fused_attention_batch_into``."""
+        hd = self.head_dim
+        kernels.flash_attention_tq_prefill_tiled_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
+                                                      self.value_norms, self.levels, vacc, hd, kv_len, start_pos, n_rows,
+                                                      n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_rows * n_q_heads, False, True)
+
     def fused_attention_batch_into(self, batch, kernels: Kernels, q: Buffer, rq: Buffer, vacc: Buffer,
                                    attn_out: Buffer, kv_len: int, start_pos: int, n_rows: int, n_q_heads: int,
                                    window: int, tiled: bool = True):
@@ -199,6 +218,28 @@ class QuantizedUnifiedKvPool:
                                                 n_q_heads, self.n_kv_heads, window, self.bits, lanes,
                                                 self.lane_ring_capacity)
         kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, total_heads, False, True)
+
+    def prepare_lanes_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, positions: Buffer,
+                           active_lanes: int, n_q_heads: int, eps: float, theta: float,
+                           partial_rotary_factor: float) -> None:
+        """One dispatch for every lane's head norms, RoPE, V norm, ``write_kv_into`` and the query rotation that opens
+        ``attention_into``; ``k = v = None`` leaves the pool alone (a KV-shared layer)."""
+        lanes = min(active_lanes, self.n_lanes)
+        kernels.decode_qkv_prepare_rows_into(batch, q, k, v, q_norm, k_norm, self.levels, self.signs, rq, self.keys_q,
+                                             self.key_norms, self.values_q, self.value_norms, positions, self.head_dim,
+                                             n_q_heads, self.n_kv_heads, lanes, eps, 0, theta, partial_rotary_factor,
+                                             self.bits, self.lane_ring_capacity, self.lane_stride())
+
+    def attention_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                                    positions: Buffer, n_q_heads: int, window: int, active_lanes: int) -> None:
+        """quant_unified_pool.rs:225-256: the attend and rotate-back steps of ``attention_into``."""
+        hd = self.head_dim
+        lanes = min(active_lanes, self.n_lanes)
+        kernels.flash_attention_tq_batched_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
+                                                self.value_norms, self.levels, vacc, positions, hd, self.lane_stride(),
+                                                n_q_heads, self.n_kv_heads, window, self.bits, lanes,
+                                                self.lane_ring_capacity)
+        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, lanes * n_q_heads, False, True)
 
     def copy_prefill_from(self, batch, cache: QuantizedKvCache, lane: int, positions: int) -> None:
         """quant_unified_pool.rs:269-315: seed ``lane`` with the first ``positions`` rows of a single-sequence

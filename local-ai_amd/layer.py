@@ -221,6 +221,10 @@ class TransformerLayer:
             self._ple_view = cached
         return cached[1]
 
+    def _one_prepare(self) -> bool:
+        hd = self.params.head_dim
+        return self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
+
     def _fusable(self, *ws: Optional[QuantWeight]) -> bool:
         return self.fuse_prologues and all(w is not None and w.ty != W_F16 and w.cols % 64 == 0 for w in ws)
 
@@ -272,7 +276,7 @@ class TransformerLayer:
         else:
             kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
             w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
-        one_prepare = self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
+        one_prepare = self._one_prepare()
         if not one_prepare:
             self._norm_rope(batch, kernels, q_buf, w.q_norm, n_head, pos)
 
@@ -395,23 +399,31 @@ class TransformerLayer:
             p.num_key_value_heads, p.rms_norm_eps
         kv_len = start_pos + n_rows
 
+        own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
+        one_prepare = self._one_prepare()
         kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
         w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
-        if w.q_norm is not None:
-            kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
-        kernels.rope_batch_into(batch, bs.q, start_pos, p.rope_theta, hd, n_head, rows, p.partial_rotary_factor)
-
-        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
+        if own_kv:
             w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
             w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
-            if w.k_norm is not None:
-                kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
-            kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
-            kernels.rope_batch_into(batch, bs.k, start_pos, p.rope_theta, hd, n_kv, rows, p.partial_rotary_factor)
-            kv_cache.write_kv_gpu_into(batch, kernels, bs.k, bs.v, start_pos, n_rows)
-
-        kv_cache.fused_attention_batch_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
-                                            n_head, p.sliding_window)
+        if one_prepare:   # head norms, RoPE, V norm, both encodes and the query rotation of all rows in one dispatch
+            kv_cache.prepare_rows_into(batch, kernels, bs.q, bs.k if own_kv else None, bs.v if own_kv else None, w.q_norm,
+                                       w.k_norm, bs.rq, start_pos, n_rows, n_head, eps, p.rope_theta,
+                                       p.partial_rotary_factor)
+            kv_cache.attention_rows_from_rotated_into(batch, kernels, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
+                                                      n_head, p.sliding_window)
+        else:
+            if w.q_norm is not None:
+                kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
+            kernels.rope_batch_into(batch, bs.q, start_pos, p.rope_theta, hd, n_head, rows, p.partial_rotary_factor)
+            if own_kv:
+                if w.k_norm is not None:
+                    kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
+                kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
+                kernels.rope_batch_into(batch, bs.k, start_pos, p.rope_theta, hd, n_kv, rows, p.partial_rotary_factor)
+                kv_cache.write_kv_gpu_into(batch, kernels, bs.k, bs.v, start_pos, n_rows)
+            kv_cache.fused_attention_batch_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
+                                                n_head, p.sliding_window)
         self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)
 
     # ---------------------------- one row per independent lane (continuous batching)
@@ -425,22 +437,31 @@ class TransformerLayer:
         rows, h, hd, n_head, n_kv, eps = n_lanes, p.hidden_size, p.head_dim, p.num_attention_heads, \
             p.num_key_value_heads, p.rms_norm_eps
 
+        own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
+        one_prepare = self._one_prepare()
         kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
         w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
-        if w.q_norm is not None:
-            kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
-        kernels.rope_batch_decode_into(batch, bs.q, positions, p.rope_theta, hd, n_head, rows, p.partial_rotary_factor)
-
-        if not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None:
+        if own_kv:
             w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
             w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
-            if w.k_norm is not None:
-                kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
-            kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
-            kernels.rope_batch_decode_into(batch, bs.k, positions, p.rope_theta, hd, n_kv, rows,
+        if one_prepare:   # every lane's head norms, RoPE, V norm, encodes and query rotation in one dispatch
+            pool.prepare_lanes_into(batch, kernels, bs.q, bs.k if own_kv else None, bs.v if own_kv else None, w.q_norm,
+                                    w.k_norm, bs.rq, positions, n_lanes, n_head, eps, p.rope_theta,
+                                    p.partial_rotary_factor)
+            pool.attention_from_rotated_into(batch, kernels, bs.rq, bs.vacc, bs.attn_out, positions, n_head,
+                                             p.sliding_window, n_lanes)
+        else:
+            if w.q_norm is not None:
+                kernels.qk_norm_gpu_into(batch, bs.q, w.q_norm, hd, rows * n_head, eps)
+            kernels.rope_batch_decode_into(batch, bs.q, positions, p.rope_theta, hd, n_head, rows,
                                            p.partial_rotary_factor)
-            pool.write_kv_into(batch, kernels, bs.k, bs.v, positions, n_lanes)
-
-        pool.attention_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, positions, n_head, p.sliding_window,
-                            n_lanes)
+            if own_kv:
+                if w.k_norm is not None:
+                    kernels.qk_norm_gpu_into(batch, bs.k, w.k_norm, hd, rows * n_kv, eps)
+                kernels.rms_norm_into(batch, bs.v, ones, bs.v, hd, rows * n_kv, eps)
+                kernels.rope_batch_decode_into(batch, bs.k, positions, p.rope_theta, hd, n_kv, rows,
+                                               p.partial_rotary_factor)
+                pool.write_kv_into(batch, kernels, bs.k, bs.v, positions, n_lanes)
+            pool.attention_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, positions, n_head, p.sliding_window,
+                                n_lanes)
         self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)

@@ -191,14 +191,18 @@ def test_forward_decode_one_kernel_per_op_matches_oracle(pkg, gpu, oracle):
     _same_cache(cache, kv, 12)
 
 
-@pytest.mark.parametrize("n_rows,start", [(1, 0), (5, 0), (16, 7), (48, 20), (130, 3)])
-def test_forward_batch_matches_decode_row_by_row(pkg, gpu, oracle, n_rows, start):
+@pytest.mark.parametrize("n_rows,start,fused", [(1, 0, True), (5, 0, True), (16, 7, True), (48, 20, True), (130, 3, True),
+                                                (5, 0, False), (48, 20, False)])
+def test_forward_batch_matches_decode_row_by_row(pkg, gpu, oracle, n_rows, start, fused):
     """layer.rs:542-718 over rows start..start+n equals n single-token steps (oracle) -- with per-layer input
     injection and the output scale on."""
     ctx, kernels = gpu
     g = pkg.synth.rng(903, n_rows)
     dims, pld, n_layers, layer_idx = _dims(), 256, 2, 1
     dev, ora, _ = _make(pkg, gpu, g, dims, pld, n_layers, layer_idx, output_scale=1.25)
+    if not fused:    # the reference's literal sequence: one kernel per operation
+        dev = pkg.layer.TransformerLayer(dev.params, dev.weights, group_projections=False, fuse_norm_rope=False,
+                                         fuse_prologues=False)
     total = start + n_rows
     cache = pkg.kv_cache.QuantizedKvCache(ctx, 1, 256, 256)
     cache.reset()
@@ -231,8 +235,8 @@ def test_forward_batch_matches_decode_row_by_row(pkg, gpu, oracle, n_rows, start
         dev.forward_batch(kernels, pkg.CommandBatch(ctx), n_rows + 1, 0, inp, out, bs, scratch.ones, cache)
 
 
-@pytest.mark.parametrize("window", [0, 32])
-def test_forward_decode_batch_turbo_matches_single_sequence(pkg, gpu, oracle, window):
+@pytest.mark.parametrize("window,fused", [(0, True), (32, True), (0, False), (32, False)])
+def test_forward_decode_batch_turbo_matches_single_sequence(pkg, gpu, oracle, window, fused):
     """layer.rs:731-873: lanes at different positions, each equal to its own single-sequence decode
     (pipeline/batched.rs:649-735 checks the same over greedy steps on the real model)."""
     ctx, kernels = gpu
@@ -241,6 +245,9 @@ def test_forward_decode_batch_turbo_matches_single_sequence(pkg, gpu, oracle, wi
     ring = pkg.kv_cache.swa_ring_capacity(window, lane_cap) if window else 0
     assert ring in (0, 512)
     dev, ora, _ = _make(pkg, gpu, g, dims, extra=dict(sliding_window=window))
+    if not fused:
+        dev = pkg.layer.TransformerLayer(dev.params, dev.weights, group_projections=False, fuse_norm_rope=False,
+                                         fuse_prologues=False)
     pool = pkg.kv_cache.QuantizedUnifiedKvPool(ctx, n_lanes, lane_cap, 1, 256, 2, ring)
     pool.reset()
     kvs = [OL.KvState(1, 256, 2, lane_cap, ring_capacity=ring) for _ in range(n_lanes)]

@@ -265,3 +265,59 @@ def test_decode_qkv_prepare_equals_the_separate_kernels(pkg, gpu, oracle, hd, n_
     assert np.array_equal(c["q"].as_array(np.uint16), a["q"].as_array(np.uint16))
     assert np.array_equal(c["rq"].as_array(np.uint32), a["rq"].as_array(np.uint32))
     assert not c["kc"].as_array(np.uint8).any()
+
+
+@pytest.mark.parametrize("lanes_mode", [False, True])
+def test_decode_qkv_prepare_rows_equals_row_by_row(pkg, gpu, oracle, lanes_mode):
+    """Several tokens in one dispatch -- consecutive positions of one sequence on a ring that wraps inside the call, or
+    one token per lane at positions from a device table -- give the bits of one single-token call per row (the
+    single-token form is checked against the oracle and the separate kernels above)."""
+    ctx, K = gpu
+    hd, n_q, n_kv, bits, rows, eps, theta, prf = 256, 4, 2, 2, 7, 1e-6, 1e4, 1.0
+    g = pkg.synth.rng(62, int(lanes_mode))
+    cb = oracle.tq_code_bytes(hd, bits)
+    ring = 512
+    lane_cap = 600 if lanes_mode else 0
+    start = 509                                            # rows 509..515 wrap the 512-slot ring
+    positions = np.array([3, 700, 511, 512, 0, 1023, 77], np.uint32)
+    q0 = (g.standard_normal(rows * n_q * hd, dtype=np.float32) * 2).astype(np.float16)
+    k0 = (g.standard_normal(rows * n_kv * hd, dtype=np.float32) * 2).astype(np.float16)
+    v0 = (g.standard_normal(rows * n_kv * hd, dtype=np.float32) * 2).astype(np.float16)
+    qw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    kw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    lv = pkg.Buffer.from_slice(ctx, oracle.tq_levels(hd, bits))
+    sg = pkg.Buffer.from_slice(ctx, oracle.rotation_signs(hd))
+    qwb, kwb = pkg.Buffer.from_slice(ctx, qw), pkg.Buffer.from_slice(ctx, kw)
+    phys = rows * lane_cap if lanes_mode else ring
+
+    def fresh():
+        return dict(q=pkg.Buffer.from_slice(ctx, q0), k=pkg.Buffer.from_slice(ctx, k0), v=pkg.Buffer.from_slice(ctx, v0),
+                    rq=pkg.Buffer.empty(ctx, rows * n_q * hd * 4), kc=pkg.Buffer.empty(ctx, phys * n_kv * cb),
+                    kn=pkg.Buffer.empty(ctx, phys * n_kv * 2), vc=pkg.Buffer.empty(ctx, phys * n_kv * cb),
+                    vn=pkg.Buffer.empty(ctx, phys * n_kv * 2))
+
+    a, b = fresh(), fresh()
+    pos_buf = pkg.Buffer.from_slice(ctx, positions) if lanes_mode else None
+    batch = pkg.CommandBatch(ctx)
+    K.decode_qkv_prepare_rows_into(batch, a["q"], a["k"], a["v"], qwb, kwb, lv, sg, a["rq"], a["kc"], a["kn"], a["vc"], a["vn"],
+                                   pos_buf, hd, n_q, n_kv, rows, eps, 0 if lanes_mode else start, theta, prf, bits, ring, lane_cap)
+    assert batch.dispatch_count() == 1
+    for r in range(rows):
+        pos = int(positions[r]) if lanes_mode else start + r
+        lane_bytes = lane_cap * n_kv
+        view = {n: b[n].view(r * w, w) for n, w in (("q", n_q * hd * 2), ("k", n_kv * hd * 2), ("v", n_kv * hd * 2),
+                                                     ("rq", n_q * hd * 4))}
+        if lanes_mode:                                     # lane r's own region of the pool, addressed like a one-lane cache
+            caches = {n: b[n].view(r * lane_bytes * u, lane_bytes * u) for n, u in (("kc", cb), ("kn", 2), ("vc", cb), ("vn", 2))}
+        else:
+            caches = {n: b[n] for n in ("kc", "kn", "vc", "vn")}
+        K.decode_qkv_prepare_into(batch, view["q"], view["k"], view["v"], qwb, kwb, lv, sg, view["rq"], caches["kc"], caches["kn"],
+                                  caches["vc"], caches["vn"], hd, n_q, n_kv, eps, pos, theta, prf, bits, ring)
+    batch.commit_and_wait()
+    for n in ("q", "k", "v", "rq", "kc", "kn", "vc", "vn"):
+        assert np.array_equal(a[n].as_array(np.uint8), b[n].as_array(np.uint8)), n
+    assert a["kc"].as_array(np.uint8).any()
+    with pytest.raises(pkg.InvalidArgument):               # a positions table needs a lane capacity and the reverse
+        K.decode_qkv_prepare_rows_into(pkg.CommandBatch(ctx), a["q"], a["k"], a["v"], qwb, kwb, lv, sg, a["rq"], a["kc"], a["kn"],
+                                       a["vc"], a["vn"], None if lanes_mode else pkg.Buffer.from_slice(ctx, positions), hd, n_q,
+                                       n_kv, rows, eps, 0, theta, prf, bits, ring, lane_cap if lanes_mode else 0)
