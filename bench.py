@@ -38,7 +38,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/matvec_tq2_mfma_grouped_8192x2048.md), scaled by the same counters on the library's plain
 # copy kernel; None until that profile has been taken for the current kernel.
-MEASURED_TRAFFIC_BYTES = 1089494324
+MEASURED_TRAFFIC_BYTES = 1088685363
 
 
 def log(*a):
