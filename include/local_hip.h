@@ -202,6 +202,12 @@ LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, co
 LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, lh_dtype input_dtype,
                                          const lh_buffer* weight, lh_buffer* output, lh_dtype output_dtype,
                                          uint32_t m, uint32_t k, uint32_t n);
+/* Up to four weight matrices of one format and one k against the same activations as one launch (what layer.rs:570-590 /
+ * 658-662 issue back to back: Q, K and V, or gate and up), f16 in and out; output i is [m, ns[i]].  Shapes the separate
+ * calls would send to other kernels (m <= 16, or enough 128-row tiles to fill the chip) are issued as those calls. */
+LH_API int lh_matmul_nt_quant_grouped_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* input,
+                                           const lh_buffer* const* weights, lh_buffer* const* outputs, const uint32_t* ns,
+                                           uint32_t m, uint32_t k);
 /* kernels.rs:5517-5568 matmul_nt_into: FP16 weights, shaders/matmul_f16.metal:74-114. */
 LH_API int lh_matmul_nt_into(lh_batch* batch, const lh_buffer* input, const lh_buffer* weight, lh_buffer* output,
                              uint32_t m, uint32_t k, uint32_t n);

@@ -409,6 +409,14 @@ class Kernels:
                                                      weight._h, output._h, C.c_int(output_dtype), _u32(m), _u32(k),
                                                      _u32(n)))
 
+    def matmul_nt_quant_grouped_into(self, batch, fmt, input, weights, outputs, m, k, ns):
+        """Up to four matrices of one format against the same activations in one launch; output i is [m, ns[i]] f16."""
+        n = len(weights)
+        assert len(outputs) == n and len(ns) == n
+        _check(self._l.lh_matmul_nt_quant_grouped_into(batch._h, C.c_int(fmt), _u32(n), input._h, _handles(weights),
+                                                       _handles(outputs), (C.c_uint32 * n)(*[int(v) for v in ns]),
+                                                       _u32(m), _u32(k)))
+
     def matmul_nt_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
 

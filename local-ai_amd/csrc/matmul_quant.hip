@@ -229,6 +229,22 @@ __device__ __forceinline__ void store_words(_Float16* dst, const uint32_t (&f)[N
     for (int i = 0; i < NW / 4; i++) *reinterpret_cast<uint4*>(dst + 8 * i) = make_uint4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
 }
 
+// Up to four weight matrices of one format and one K that multiply the same activations (Q / K / V, gate / up) as one
+// launch: their column tiles are laid side by side, tile0[i] being the first tile of matrix i (tile0[count] = all).
+struct GroupArgs {
+    const uint8_t* W[4];
+    void* C[4];
+    uint32_t N[4];
+    uint32_t tile0[5];
+    uint32_t count;          // 0: the single matrix of the kernel arguments
+};
+__device__ __forceinline__ uint32_t group_of_tile(const GroupArgs& g, uint32_t tile) {
+    uint32_t i = 0;
+#pragma unroll
+    for (uint32_t j = 1; j < 4; j++) if (j < g.count && tile >= g.tile0[j]) i = j;
+    return i;
+}
+
 // Optional fused clamp / bias of the clipped linear layer (shaders/matmul_f16.metal:121-170):
 // C = clamp(clamp(A, in_lo, in_hi) . W^T + bias, out_lo, out_hi).  Inactive for every other entry point.
 struct ClipArgs {
@@ -243,16 +259,24 @@ __device__ __forceinline__ uint32_t clamp_h2(uint32_t w, float lo, float hi) {
 }
 
 template <int FMT, int ADT, int CDT, int BM>
-__global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
-                                                         uint32_t M, uint32_t K, uint32_t N, ClipArgs clip,
-                                                         float* __restrict__ partial, uint32_t steps_per_split) {
+__global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict__ A, const uint8_t* __restrict__ W_one, void* __restrict__ C_one,
+                                                         uint32_t M, uint32_t K, uint32_t N_one, ClipArgs clip,
+                                                         float* __restrict__ partial, uint32_t steps_per_split, GroupArgs grp) {
+    const uint8_t* __restrict__ W = W_one;
+    void* __restrict__ C = C_one;
+    uint32_t N = N_one, col_tile = blockIdx.x;
+    if (grp.count) {   // uniform over the workgroup
+        const uint32_t gi = group_of_tile(grp, col_tile);
+        W = grp.W[gi]; C = grp.C[gi]; N = grp.N[gi];
+        col_tile -= grp.tile0[gi];
+    }
     constexpr int TI = BM / 32;                              // 16-row MFMA tiles per wave along M (2 x 2 waves)
     constexpr int NCH = BM / 16;                             // 8-element activation chunks staged per thread
     __shared__ __align__(16) _Float16 As[BM * LDK];
     __shared__ __align__(16) _Float16 Bs[BN * LDK];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const uint32_t m0 = blockIdx.y * BM, n0 = col_tile * BN;
     const uint32_t b_ld_row = tid >> 1, b_ld_k = (tid & 1) * 64;
     const uint32_t b_row = n0 + b_ld_row < N ? n0 + b_ld_row : N - 1;   // past-the-end rows re-read the last (never stored)
 
@@ -356,7 +380,8 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const uint32_t m = m0 + wm * (BM / 2) + i * 16 + (lane >> 4) * 4 + r;
-                    if (m < M) partial[((size_t)blockIdx.z * M + m) * N + n] = acc[i][j][r];
+                    // partial tiles keep the launch's tile grid: row stride gridDim.x * BN, column = tile * BN + offset
+                    if (m < M) partial[((size_t)blockIdx.z * M + m) * (gridDim.x * BN) + blockIdx.x * BN + (n - n0)] = acc[i][j][r];
                 }
                 continue;
             }
@@ -371,19 +396,29 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(const void* __restrict
         }
 }
 
-// Sum of the split-k partial tiles, with the bias / clamp of the clipped linear layer, stored in the output type.
+// Sum of the split-k partial tiles (laid out on the launch's tile grid, `tiles` column tiles wide), with the bias / clamp
+// of the clipped linear layer, stored in the output type of the matrix the column belongs to.
 template <int CDT>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ C, uint32_t M, uint32_t N,
-                                                           uint32_t splits, ClipArgs clip) {
-    const size_t total = (size_t)M * N, i = (size_t)blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ C_one, uint32_t M, uint32_t N_one,
+                                                           uint32_t tiles, uint32_t splits, ClipArgs clip, GroupArgs grp) {
+    const size_t nv_total = (size_t)tiles * BN, total = (size_t)M * nv_total, i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
+    const uint32_t m = (uint32_t)(i / nv_total), nv = (uint32_t)(i - (size_t)m * nv_total);
+    void* C = C_one;
+    uint32_t N = N_one, n = nv;
+    if (grp.count) {
+        const uint32_t gi = group_of_tile(grp, nv / BN);
+        C = grp.C[gi]; N = grp.N[gi];
+        n = nv - grp.tile0[gi] * BN;
+    }
+    if (n >= N) return;
     float v = 0.0f;
     for (uint32_t z = 0; z < splits; z++) v += partial[(size_t)z * total + i];
     if (clip.enabled) {
-        const float bias = clip.bias ? lh_h2f(clip.bias[i % N]) : 0.0f;
+        const float bias = clip.bias ? lh_h2f(clip.bias[n]) : 0.0f;
         v = fminf(fmaxf(v + bias, clip.out_lo), clip.out_hi);
     }
-    store_elem<CDT>(C, i, v);
+    store_elem<CDT>(C, (size_t)m * N + n, v);
 }
 
 // ---- 128 x 128 tiles for large M: f16 activations (converted once by a pre-pass when they arrive as bf16 / f32),
@@ -579,6 +614,37 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
     }
 }
 
+// The 64-row-tile kernel over `tiles_n` column tiles (one matrix, or the matrices of `grp` side by side).  Few output
+// tiles (a decode batch of some tens of rows): k is split so that every CU gets a workgroup, at least two k steps per
+// split, partial tiles within the lower half of the context workspace, summed by splitk_reduce_kernel.
+template <int FMT, int ADT>
+void launch_tiles64(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n, const ClipArgs& clip,
+                    const GroupArgs& grp) {
+    hipStream_t s = ctx->stream;
+    const int cus = ctx->cu_count;
+    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
+    const uint32_t nk = (k + BK - 1) / BK;
+    const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
+    const uint64_t tiles64 = (uint64_t)tiles_n * ((m + 63) / 64);
+    uint32_t splits = 1;
+    if (!no_splitk && tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
+        splits = (uint32_t)std::min<uint64_t>(nk / 2, ((uint64_t)cus + tiles64 - 1) / tiles64);
+        const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * tiles_n * BN * 4);
+        splits = (uint32_t)std::min<uint64_t>(splits, fit);
+    }
+    const uint32_t steps = splits > 1 ? (nk + splits - 1) / splits : nk;
+    if (splits > 1) splits = (nk + steps - 1) / steps;
+    float* partial = splits > 1 ? static_cast<float*>(ctx->workspace) : nullptr;
+    const dim3 grid(tiles_n, (m + 63) / 64, splits > 1 ? splits : 1);
+    if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps, grp);
+    else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps, grp);
+    if (splits > 1) {
+        const uint32_t rgrid = (uint32_t)(((size_t)m * tiles_n * BN + 255) / 256);
+        if (ct == LH_F32) hipLaunchKernelGGL((splitk_reduce_kernel<LH_F32>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+        else hipLaunchKernelGGL((splitk_reduce_kernel<LH_F16>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+    }
+}
+
 template <int FMT, int ADT>
 int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n,
                   const ClipArgs& clip) {
@@ -607,30 +673,10 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
         const uint32_t nk = (k + BK - 1) / BK;
         if (force_bm == 128 || (force_bm == 0 && tiles128 >= 2ull * (uint64_t)cus)) {
             const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk, GroupArgs{});
+            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk, GroupArgs{});
         } else {
-            // Few output tiles (a decode batch of some tens of rows): split k so that every CU gets a workgroup, at least
-            // two k steps per split, partial tiles within the lower half of the context workspace.
-            static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
-            const uint64_t tiles64 = (uint64_t)((n + BN - 1) / BN) * ((m + 63) / 64);
-            uint32_t splits = 1;
-            if (!no_splitk && tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
-                splits = (uint32_t)std::min<uint64_t>(nk / 2, ((uint64_t)cus + tiles64 - 1) / tiles64);
-                const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * n * 4);
-                splits = (uint32_t)std::min<uint64_t>(splits, fit);
-            }
-            const uint32_t steps = splits > 1 ? (nk + splits - 1) / splits : nk;
-            if (splits > 1) splits = (nk + steps - 1) / steps;
-            float* partial = splits > 1 ? static_cast<float*>(ctx->workspace) : nullptr;
-            const dim3 grid((n + BN - 1) / BN, (m + 63) / 64, splits > 1 ? splits : 1);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps);
-            else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 64>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, partial, steps);
-            if (splits > 1) {
-                const uint32_t rgrid = (uint32_t)(((size_t)m * n + 255) / 256);
-                if (ct == LH_F32) hipLaunchKernelGGL((splitk_reduce_kernel<LH_F32>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, splits, clip);
-                else hipLaunchKernelGGL((splitk_reduce_kernel<LH_F16>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, splits, clip);
-            }
+            launch_tiles64<FMT, ADT>(ctx, A, W, C, ct, m, k, n, clip, GroupArgs{});
         }
     } else {
         if constexpr (FMT != kF16W) {
@@ -716,6 +762,55 @@ int lh_matmul_nt_quant_typed_into(lh_batch* b, lh_quant fmt, const lh_buffer* in
     return matmul_dispatch(b, fmt == LH_Q4_0 ? "matmul_nt_q4_0" : "matmul_nt_tq2_0", fmt == LH_Q4_0 ? kQ4 : kTQ2, in, at, w, out, ct, m,
                            k, n, false);
 }
+int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* in, const lh_buffer* const* ws,
+                                    lh_buffer* const* outs, const uint32_t* ns, uint32_t m, uint32_t k) {
+    const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 (grouped)" : "matmul_nt_tq2_0 (grouped)";
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
+    if (count == 0 || m == 0 || k == 0) return LH_OK;
+    if (count > 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: at most 4 matrices share one launch, got %u", op, count);
+    if (!in || !ws || !outs || !ns) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null argument", op);
+    const int kind = fmt == LH_Q4_0 ? kQ4 : kTQ2;
+    lh_context* ctx = b->ctx;
+    // The shapes the 64-row-tile kernel takes (some tens to a few hundred rows, not enough 128-row tiles to fill the
+    // chip) go out as one launch; everything else as the separate calls this entry point stands for.
+    uint64_t tiles_n = 0;
+    for (uint32_t i = 0; i < count; i++) tiles_n += (ns[i] + BN - 1) / BN;
+    const uint64_t tiles128 = tiles_n * ((m + 127) / 128);
+    const bool together = m > (uint32_t)kMaxMultivecM && !(m > 64 && tiles128 * 2 >= (uint64_t)ctx->cu_count);
+    if (!together) {
+        for (uint32_t i = 0; i < count; i++) {
+            int r = matmul_dispatch(b, op, kind, in, LH_F16, ws[i], outs[i], LH_F16, m, k, ns[i], false);
+            if (r != LH_OK) return r;
+        }
+        return LH_OK;
+    }
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    if (k % blk != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: k %u not /%u", op, k, blk);
+    LH_NEED(in, (size_t)m * k * 2, op, "input");
+    LH_REQUIRE(((uintptr_t)in->ptr & 15) == 0, "%s: input must be 16-byte aligned", op);
+    GroupArgs grp{};
+    grp.count = count;
+    uint32_t tile = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (ns[i] == 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: matrix %u has no rows", op, i);
+        const size_t wbytes = fmt == LH_Q4_0 ? (size_t)ns[i] * (k / 32) * 18 : (size_t)ns[i] * (k / 256) * 66;
+        LH_NEED(ws[i], wbytes, op, "weight");
+        LH_NEED(outs[i], (size_t)m * ns[i] * 2, op, "output");
+        LH_REQUIRE(((uintptr_t)ws[i]->ptr & 1) == 0, "%s: weight must be 2-byte aligned", op);
+        grp.W[i] = (const uint8_t*)ws[i]->ptr; grp.C[i] = outs[i]->ptr; grp.N[i] = ns[i];
+        grp.tile0[i] = tile;
+        tile += (ns[i] + BN - 1) / BN;
+    }
+    for (uint32_t i = count; i <= 4; i++) grp.tile0[i] = tile;
+    const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
+    if (fmt == LH_Q4_0) launch_tiles64<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
+    else launch_tiles64<kTQ2, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
+    int r = lh_check_launch(op);
+    if (r == LH_OK) b->dispatch_count++;
+    return r;
+}
+
 int lh_matmul_nt_into(lh_batch* b, const lh_buffer* in, const lh_buffer* w, lh_buffer* out, uint32_t m, uint32_t k, uint32_t n) {
     return matmul_dispatch(b, "matmul_nt", kF16W, in, LH_F16, w, out, LH_F16, m, k, n, false);
 }

@@ -221,6 +221,17 @@ class TransformerLayer:
             self._ple_view = cached
         return cached[1]
 
+    def _matmuls(self, batch, kernels: Kernels, ws, x: Buffer, outs, rows: int) -> None:
+        """out_i[rows, w_i.rows] = x . w_i^T for projections that read the same rows; weights of one quantized format
+        and width go out as one launch."""
+        if (self.group_projections and len(ws) > 1 and all(w.ty == ws[0].ty and w.cols == ws[0].cols for w in ws)
+                and ws[0].ty != W_F16):
+            kernels.matmul_nt_quant_grouped_into(batch, ws[0].ty, x, [w.buf for w in ws], list(outs), rows, ws[0].cols,
+                                                 [w.rows for w in ws])
+            return
+        for w, out in zip(ws, outs):
+            w.matmul_nt_into(batch, kernels, x, out, rows)
+
     def _one_prepare(self) -> bool:
         hd = self.params.head_dim
         return self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
@@ -367,8 +378,7 @@ class TransformerLayer:
         w.attn_output.matmul_nt_into(batch, kernels, bs.attn_out, bs.ffn_out, rows)
         kernels.rms_norm_add_into(batch, bs.ffn_out, w.attn_post_norm, input, bs.attn_resid, h, rows, eps)
         kernels.rms_norm_into(batch, bs.attn_resid, w.ffn_norm, bs.normed, h, rows, eps)
-        w.ffn_gate.matmul_nt_into(batch, kernels, bs.normed, bs.gate, rows)
-        w.ffn_up.matmul_nt_into(batch, kernels, bs.normed, bs.up, rows)
+        self._matmuls(batch, kernels, [w.ffn_gate, w.ffn_up], bs.normed, [bs.gate, bs.up], rows)
         kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
         w.ffn_down.matmul_nt_into(batch, kernels, bs.gate, bs.ffn_out, rows)
         kernels.rms_norm_add_into(batch, bs.ffn_out, w.ffn_post_norm, bs.attn_resid, output, h, rows, eps)
@@ -402,10 +412,10 @@ class TransformerLayer:
         own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
         one_prepare = self._one_prepare()
         kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
-        w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
         if own_kv:
-            w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
-            w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
+            self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
+        else:
+            w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
         if one_prepare:   # head norms, RoPE, V norm, both encodes and the query rotation of all rows in one dispatch
             kv_cache.prepare_rows_into(batch, kernels, bs.q, bs.k if own_kv else None, bs.v if own_kv else None, w.q_norm,
                                        w.k_norm, bs.rq, start_pos, n_rows, n_head, eps, p.rope_theta,
@@ -440,10 +450,10 @@ class TransformerLayer:
         own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
         one_prepare = self._one_prepare()
         kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
-        w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
         if own_kv:
-            w.attn_k.matmul_nt_into(batch, kernels, bs.normed, bs.k, rows)
-            w.attn_v.matmul_nt_into(batch, kernels, bs.normed, bs.v, rows)
+            self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
+        else:
+            w.attn_q.matmul_nt_into(batch, kernels, bs.normed, bs.q, rows)
         if one_prepare:   # every lane's head norms, RoPE, V norm, encodes and query rotation in one dispatch
             pool.prepare_lanes_into(batch, kernels, bs.q, bs.k if own_kv else None, bs.v if own_kv else None, w.q_norm,
                                     w.k_norm, bs.rq, positions, n_lanes, n_head, eps, p.rope_theta,

@@ -90,6 +90,34 @@ def test_mfma_matmul_split_k(pkg, gpu, oracle, fmt):
         refgen.assert_close(got, want, 1e-3 if ct == "f32" else 2e-3, f"{fmt} split k {m}x{k}x{n}")
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+@pytest.mark.parametrize("m,k,ns", [(64, 2048, (2048, 256, 256)), (64, 2048, (8192, 8192)), (40, 512, (100, 257, 33, 128)),
+                                    (256, 2048, (2048, 256, 256)), (300, 2048, (8192, 8192)), (8, 512, (64, 200))])
+def test_matmul_grouped(pkg, gpu, oracle, fmt, m, k, ns):
+    """matmul_nt_quant_grouped_into: Q / K / V or gate / up against the same rows in one launch (column tiles of the
+    matrices side by side, ragged last tiles, with and without the k split), and the shapes it passes on to the
+    separate calls (m <= 16; enough 128-row tiles to fill the chip).  Each output against the oracle."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    raws = [payload(fmt, n, k, 0x6A0 + i) for i, n in enumerate(ns)]
+    ws = [pkg.QuantWeight.from_bytes(ctx, r, ty, n, k) for r, n in zip(raws, ns)]
+    a16 = (pkg.synth.rng(4, m + k + len(ns)).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+    ab = pkg.Buffer.from_slice(ctx, a16)
+    outs = [pkg.Buffer.empty(ctx, m * n * 2) for n in ns]
+    batch = pkg.CommandBatch(ctx)
+    K.matmul_nt_quant_grouped_into(batch, ty, ab, [w.buf for w in ws], outs, m, k, list(ns))
+    batch.commit_and_wait()
+    for i, n in enumerate(ns):
+        if m > 16:   # MFMA path: the weights are the CPU path's f16 values (qat_recover.rs:84-93)
+            deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raws[i]).view(np.float16).astype(np.float32).reshape(n, k)
+        else:        # rows as matvecs: the unrounded f32 products of the fused matvec kernels
+            deq = expand(oracle, fmt, raws[i], n, k)
+        want = oracle.matmul_nt_f32(a16.astype(np.float32), deq)
+        refgen.assert_close(outs[i].as_array(np.float16).astype(np.float32), want, 2e-3, f"{fmt} grouped {m}x{k}x{n} #{i}")
+    with pytest.raises(pkg.InvalidArgument):
+        K.matmul_nt_quant_grouped_into(pkg.CommandBatch(ctx), ty, ab, [w.buf for w in ws] * 3, outs * 3, m, k, list(ns) * 3)
+
+
 @pytest.mark.parametrize("adt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_large_tiles(pkg, gpu, oracle, fmt, adt):
