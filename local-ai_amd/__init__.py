@@ -649,4 +649,5 @@ from .quant_weight import QuantWeight  # noqa: E402
 from .kv_cache import QuantizedKvCache, QuantizedUnifiedKvPool, swa_ring_capacity, kv_bits_from_env, TQ_SEED, DEFAULT_KV_BITS  # noqa: E402
 from . import gguf, weights  # noqa: E402  (GGUF reader and weight loader: gguf.rs, init_gemma4_qat.rs)
 from . import layer  # noqa: E402  (decoder layer: layer.rs)
+from . import pipeline  # noqa: E402  (decode core of the token loop: pipeline.rs)
 from .layer import LayerParams, LayerWeights, ScratchBuffers, BatchScratch, TransformerLayer  # noqa: E402

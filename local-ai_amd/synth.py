@@ -108,3 +108,31 @@ def decoder_layer_tensors(hidden: int, inter: int, n_head: int, n_kv: int, head_
     if output_scale is not None:
         t["layer_output_scale"] = np.array([output_scale], np.float16)
     return t
+
+
+def decode_model_tensors(config, g: np.random.Generator, intermediate_size, attn_fmt: str = "q4_0", ffn_fmt: str = "tq2_0",
+                         table_rows: int | None = None) -> dict:
+    """Every tensor of a decode stack shaped by `config` (a pipeline.Gemma4QATConfig): one dict of layer tensors per
+    layer (head_dim and KV sharing by layer type; `intermediate_size` an int or one value per layer), the tied
+    Q4_0 embedding table, the output norm and, when the configuration has per-layer inputs, their table, projection
+    and norm.  `table_rows` distinct rows are generated for the two vocabulary-sized tables and repeated to
+    vocab_size (the decode step reads one row of each, so the repetition is invisible to it)."""
+    h, n_layer, pld, vocab = config.hidden_size, config.num_hidden_layers, config.hidden_size_per_layer_input, config.vocab_size
+    inters = [intermediate_size] * n_layer if isinstance(intermediate_size, int) else list(intermediate_size)
+    layers = [decoder_layer_tensors(h, inters[i], config.num_attention_heads, config.num_key_value_heads,
+                                    config.attn_head_dim(i), pld, g, attn_fmt, ffn_fmt, kv_shared=config.is_kv_shared(i))
+              for i in range(n_layer)]
+
+    def table(cols):
+        rows = min(table_rows or vocab, vocab)
+        block = q4_0_weights(rows, cols, g).reshape(rows, -1)
+        reps = -(-vocab // rows)
+        return ("q4_0", vocab, cols, np.tile(block, (reps, 1))[:vocab].reshape(-1))
+
+    t = {"layers": layers, "token_embd": table(h),
+         "output_norm": (np.float32(1.0) + np.float32(0.1) * g.standard_normal(h, dtype=np.float32)).astype(np.float16)}
+    if pld:
+        t["ple_table"] = table(pld * n_layer)
+        t["per_layer_model_proj"] = (attn_fmt, pld * n_layer, h, weights(attn_fmt, pld * n_layer, h, g))
+        t["per_layer_proj_norm"] = (np.float32(1.0) + np.float32(0.1) * g.standard_normal(pld, dtype=np.float32)).astype(np.float16)
+    return t

@@ -73,6 +73,29 @@ class KvState:
             O.tq_write_kv(np.asarray(src, F16).view(np.uint16), self.n_kv, self.head_dim, self.bits, self.signs,
                           self.levels, position, self.ring_capacity, codes, norms)
 
+    def row_slices(self, position: int):
+        """(code bytes, norm entries) of the cache row that holds `position`."""
+        cb = len(self.k_codes) // len(self.k_norms)
+        slot = position % self.ring_capacity if self.ring_capacity else position
+        return slice(slot * self.n_kv * cb, (slot + 1) * self.n_kv * cb), slice(slot * self.n_kv, (slot + 1) * self.n_kv)
+
+    def replace_row(self, position: int, k_codes, k_norms, v_codes, v_norms) -> float:
+        """Overwrite the row of `position`; returns the fraction of its code fields (of the given bit width, byte
+        aligned widths only) that differed from what was there."""
+        cs, ns = self.row_slices(position)
+        new_k, new_v = np.asarray(k_codes, np.uint8).reshape(-1), np.asarray(v_codes, np.uint8).reshape(-1)
+        diff, fields = 0, 0
+        if 8 % self.bits == 0:
+            mask = (1 << self.bits) - 1
+            for old, new in ((self.k_codes[cs], new_k), (self.v_codes[cs], new_v)):
+                x = np.bitwise_xor(old, new)
+                for sh in range(0, 8, self.bits):
+                    diff += int((((x >> sh) & mask) != 0).sum())
+                fields += x.size * (8 // self.bits)
+        self.k_codes[cs], self.v_codes[cs] = new_k, new_v
+        self.k_norms[ns], self.v_norms[ns] = np.asarray(k_norms, np.uint16).reshape(-1), np.asarray(v_norms, np.uint16).reshape(-1)
+        return diff / fields if fields else 0.0
+
     def attend(self, q, seq_len: int, current_pos: int, n_q_heads: int, window: int) -> np.ndarray:
         """quant_cache.rs:548-598: rotate q (f16 -> f32), attend in code space, rotate back (f32 -> f16)."""
         hd = self.head_dim
@@ -133,13 +156,17 @@ class Layer:
         return cls(**fields, **dims)
 
 
-def decode_layer(L: Layer, x, position: int, kv: KvState, per_layer_input=None, kv_rows=None, trace=None) -> np.ndarray:
+def decode_layer(L: Layer, x, position: int, kv: KvState, per_layer_input=None, kv_rows=None, trace=None,
+                 kv_codes=None) -> np.ndarray:
     """layer.rs:354-523: hidden state [hidden_size] f16 in and out; ``kv`` is updated in place.
 
     ``trace``, a dict, receives the intermediates (normed, q, k, v, attn_out, attn_resid).  ``kv_rows = (k, v)``
     encodes those f16 rows into the cache in place of the layer's own (still computed and traced): a 2-bit
     code is a discontinuous function of its input, so a checker that wants tight bounds downstream of the
-    cache compares k / v first and then continues from the rows of the implementation under test."""
+    cache compares k / v first and then continues from the rows of the implementation under test.  ``kv_codes =
+    (k_codes, k_norms, v_codes, v_norms)`` (the cache row of this position as the implementation under test wrote it)
+    does the same one stage later, for a checker that cannot see the rows: the layer's own codes are still computed,
+    the fraction of 2-bit codes that differ goes to ``trace["code_flips"]``, and the given row replaces them."""
     trace = {} if trace is None else trace
     h, hd, n_head, n_kv, eps = L.hidden_size, L.head_dim, L.num_attention_heads, L.num_key_value_heads, L.rms_norm_eps
     x = np.asarray(x, F16).reshape(h)
@@ -163,6 +190,8 @@ def decode_layer(L: Layer, x, position: int, kv: KvState, per_layer_input=None, 
         if kv_rows is not None:
             k, v = kv_rows
         kv.write(k, v, position)
+        if kv_codes is not None:
+            trace["code_flips"] = kv.replace_row(position, *kv_codes)
     trace["normed"], trace["q"] = normed, q
     attn_out = kv.attend(q, position + 1, position, n_head, L.sliding_window)
 
@@ -189,3 +218,87 @@ def decode_layer(L: Layer, x, position: int, kv: KvState, per_layer_input=None, 
     if L.layer_output_scale is not None:
         out = G.scale_in_place(out, L.layer_output_scale)
     return out
+
+
+@dataclass
+class Model:
+    """Host-side state of the decode core of the reference's Pipeline (local-engine/src/pipeline.rs:714-953)."""
+    hidden_size: int
+    vocab_size: int
+    layers: list                      # [Layer]
+    kv_index_map: list                # layer -> index into the list of KvState (pipeline.rs:379-437)
+    token_embd: Weight                # [vocab, hidden]: the f16 values of the stored rows, as f32
+    output_norm: np.ndarray
+    per_layer_dim: int = 0
+    ple_table: Optional[Weight] = None          # [vocab, n_layer * pld]
+    per_layer_model_proj: Optional[Weight] = None
+    per_layer_proj_norm: Optional[np.ndarray] = None
+    rms_norm_eps: float = 1e-6
+    logit_softcap: float = 30.0
+
+
+def model_from_host(config, tensors: dict, logit_softcap: float = 30.0) -> Model:
+    """The host tensors of ``synth.decode_model_tensors`` for a ``pipeline.Gemma4QATConfig``-shaped `config`, with the
+    cache-slot map of pipeline.rs:379-437."""
+    n_layer = config.num_hidden_layers
+    layers = []
+    for i, lt in enumerate(tensors["layers"]):
+        inter = lt["ffn_gate"][1]
+        layers.append(Layer.from_host(lt, hidden_size=config.hidden_size, intermediate_size=inter,
+                                      num_attention_heads=config.num_attention_heads,
+                                      num_key_value_heads=config.num_key_value_heads, head_dim=config.attn_head_dim(i),
+                                      layer_idx=i, per_layer_dim=config.hidden_size_per_layer_input,
+                                      rope_theta=config.rope_theta(i), partial_rotary_factor=config.partial_rotary_factor(i),
+                                      sliding_window=0 if config.is_full_attention(i) else config.sliding_window,
+                                      rms_norm_eps=config.rms_norm_eps, is_kv_shared=config.is_kv_shared(i)))
+    slot_of, kv_index_map, n_slots = {}, [0] * n_layer, 0
+    for i in range(n_layer):
+        if config.is_kv_shared(i):
+            kv_index_map[i] = slot_of[config.kv_source_layer(i)]
+        else:
+            slot_of[i] = kv_index_map[i] = n_slots
+            n_slots += 1
+
+    def weight(t):
+        fmt, rows, cols, payload = t
+        return Weight.from_quant(fmt, payload, rows, cols)
+
+    m = Model(hidden_size=config.hidden_size, vocab_size=config.vocab_size, layers=layers, kv_index_map=kv_index_map,
+              token_embd=weight(tensors["token_embd"]), output_norm=np.asarray(tensors["output_norm"], F16),
+              per_layer_dim=config.hidden_size_per_layer_input, rms_norm_eps=config.rms_norm_eps, logit_softcap=logit_softcap)
+    if "ple_table" in tensors:
+        m.ple_table = weight(tensors["ple_table"])
+        m.per_layer_model_proj = weight(tensors["per_layer_model_proj"])
+        m.per_layer_proj_norm = np.asarray(tensors["per_layer_proj_norm"], F16)
+    return m
+
+
+def per_layer_inputs(M: Model, token: int, hidden) -> Optional[np.ndarray]:
+    """pipeline.rs:725-776."""
+    if M.ple_table is None or M.per_layer_model_proj is None or M.per_layer_proj_norm is None:
+        return None
+    pld, n_layer = M.per_layer_dim, len(M.layers)
+    tok = G.scale_in_place(M.ple_table.dq[min(token, M.vocab_size - 1)].astype(F16), float(F32(np.sqrt(F32(pld)))))
+    proj = G.scale_in_place(M.per_layer_model_proj.matvec(hidden), float(F32(1.0) / np.sqrt(F32(M.hidden_size))))
+    proj = G.rms_norm(proj, M.per_layer_proj_norm, pld, n_layer, M.rms_norm_eps)
+    return G.scale_in_place(G.residual_add(proj, tok), float(F32(np.sqrt(0.5))))
+
+
+def decode_token(M: Model, token: int, position: int, kvs: list, layer_kv_codes=None, trace=None) -> np.ndarray:
+    """pipeline.rs:834-953: the f32 logits of `token` at `position`; `kvs` are the KvStates of the cache slots.
+    `layer_kv_codes[i]`, when given for a layer that owns its KV, is passed to decode_layer as `kv_codes`."""
+    trace = {} if trace is None else trace
+    hidden = M.token_embd.dq[min(token, M.vocab_size - 1)].astype(F16)
+    hidden = G.scale_in_place(hidden, float(F32(np.sqrt(F32(M.hidden_size)))))
+    ple = per_layer_inputs(M, token, hidden)
+    flips = []
+    for i, layer in enumerate(M.layers):
+        tr = {}
+        hidden = decode_layer(layer, hidden, position, kvs[M.kv_index_map[i]], ple, trace=tr,
+                              kv_codes=None if layer_kv_codes is None else layer_kv_codes[i])
+        if "code_flips" in tr:
+            flips.append(tr["code_flips"])
+    trace["code_flips"] = flips
+    final = G.rms_norm(hidden, M.output_norm, M.hidden_size, 1, M.rms_norm_eps)
+    logits = O.matvec_f64(M.token_embd.dq, final.astype(F32)).astype(F32)
+    return G.logit_softcap(logits, M.logit_softcap) if M.logit_softcap > 0 else logits
