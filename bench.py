@@ -429,6 +429,57 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     return res
 
 
+def bench_model(pkg, ctx, K, steps, warmup, T=32768):
+    """End-to-end decode of a synthetic model with the geometry of the reference's Gemma 4 E2B configuration
+    (local-core/src/config/gemma4_qat.rs:262-283: vocabulary 262144, hidden 1536, 35 layers in a sliding x4 / full
+    pattern with head_dim 256 / 512, window 512, the last 20 layers sharing KV, per-layer inputs of 256; Q4_0
+    attention and embedding tables, TQ2_0 feed-forward, 6144 wide and 12288 in the KV-shared layers) with T cached
+    positions: embedding gather, per-layer inputs, 35 layers, output norm, 262144-row logits, soft cap -- one batch and
+    one wait per token."""
+    P = pkg.pipeline
+    types = ["full_attention" if i % 5 == 4 else "sliding_attention" for i in range(35)]
+    cfg = P.Gemma4QATConfig(vocab_size=262144, hidden_size=1536, num_hidden_layers=35, num_attention_heads=8,
+                            num_key_value_heads=1, head_dim=256, global_head_dim=512, sliding_window=512,
+                            num_kv_shared_layers=20, hidden_size_per_layer_input=256, layer_types=types,
+                            sliding_rope_theta=10000.0, full_rope_theta=1000000.0, full_partial_rotary_factor=0.25)
+    g = pkg.synth.rng(13, 0)
+    # one generated tensor set per kind of layer, uploaded once per layer (distinct addresses, nothing shared in HBM)
+    kinds = {}
+    for full in (False, True):
+        for shared in (False, True):
+            kinds[(full, shared)] = pkg.synth.decoder_layer_tensors(1536, 12288 if shared else 6144, 8, 1, 512 if full else 256,
+                                                                   256, g, kv_shared=shared)
+    one = pkg.synth.decode_model_tensors(P.Gemma4QATConfig(vocab_size=262144, hidden_size=1536, num_hidden_layers=35,
+                                                           num_attention_heads=8, num_key_value_heads=1, head_dim=256,
+                                                           hidden_size_per_layer_input=256, layer_types=[]),
+                                         g, 256, table_rows=2048)
+    tensors = {k: v for k, v in one.items() if k != "layers"}
+    tensors["layers"] = [kinds[(cfg.is_full_attention(i), cfg.is_kv_shared(i))] for i in range(35)]
+    max_ctx = T + 256
+    pipe = P.DecodePipeline.from_host(ctx, K, cfg, tensors, max_ctx)
+    del tensors, one, kinds
+    for i, c in enumerate(pipe.kv_caches):
+        fill_kv(pkg, ctx, K, c, 1, min(T, c.physical_positions), pkg.synth.rng(13, 10 + i))
+    pipe.position = T - 1
+    weight_bytes = sum(_layer_weight_bytes(pkg, l) for l in pipe.layers) + pipe.token_embd.device_bytes() \
+        + pipe.per_layer_model_proj.device_bytes()
+    kv_bytes = sum(min(T, c.physical_positions) * (2 * c.code_bytes() + 4) for c in pipe.kv_caches)
+    tokens = [int(v) for v in g.integers(0, cfg.vocab_size, steps + warmup)]
+    for t in tokens[:warmup]:
+        pipe.decode_step(t)
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for t in tokens[warmup:]:
+        pipe.decode_step(t)
+    dt = (time.perf_counter() - t0) / steps
+    logits = pipe.logits()
+    if not np.isfinite(logits).all() or np.abs(logits).max() > 30.001:
+        raise RuntimeError("model decode produced logits outside the soft cap")
+    return {"context": T, "layers": 35, "us_per_token_wall": dt * 1e6, "tokens_per_s": 1.0 / dt,
+            "weight_bytes_read_per_token": weight_bytes, "kv_bytes_read_per_token": kv_bytes,
+            "gbs_wall": (weight_bytes + kv_bytes) / dt * 1e-9}
+
+
 def _layer_weight_bytes(pkg, layer):
     return sum(w.device_bytes() for w in vars(layer.weights).values() if isinstance(w, pkg.QuantWeight))
 
@@ -572,7 +623,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk",
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -650,6 +701,10 @@ def main():
             (["chunk"] if "chunk" in legs else [])
         extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
+
+    if "model" in legs:
+        extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup)
+        log("[bench] model decode:", extra["model_decode_e2b_geometry"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
     line = {
