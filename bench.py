@@ -429,7 +429,7 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     return res
 
 
-def bench_model(pkg, ctx, K, steps, warmup, T=32768):
+def bench_model(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
     """End-to-end decode of a synthetic model with the geometry of the reference's Gemma 4 E2B configuration
     (local-core/src/config/gemma4_qat.rs:262-283: vocabulary 262144, hidden 1536, 35 layers in a sliding x4 / full
     pattern with head_dim 256 / 512, window 512, the last 20 layers sharing KV, per-layer inputs of 256; Q4_0
@@ -463,7 +463,17 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768):
     pipe.position = T - 1
     weight_bytes = sum(_layer_weight_bytes(pkg, l) for l in pipe.layers) + pipe.token_embd.device_bytes() \
         + pipe.per_layer_model_proj.device_bytes()
-    kv_bytes = sum(min(T, c.physical_positions) * (2 * c.code_bytes() + 4) for c in pipe.kv_caches)
+    def kv_read_bytes(kv_len):
+        """Codes and norms the 35 layers' attention reads for one token at kv_len cached positions: the window of a
+        sliding layer, everything for a full layer; KV-shared layers read their source layer's rows again."""
+        total = 0
+        for i in range(cfg.num_hidden_layers):
+            c = pipe.kv_caches[pipe.kv_index_map[i]]
+            span = kv_len if cfg.is_full_attention(i) else min(kv_len, cfg.sliding_window)
+            total += span * c.n_kv_heads * (2 * c.code_bytes() + 4)
+        return total
+
+    kv_bytes = kv_read_bytes(T)
     tokens = [int(v) for v in g.integers(0, cfg.vocab_size, steps + warmup)]
     for t in tokens[:warmup]:
         pipe.decode_step(t)
@@ -475,9 +485,33 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768):
     logits = pipe.logits()
     if not np.isfinite(logits).all() or np.abs(logits).max() > 30.001:
         raise RuntimeError("model decode produced logits outside the soft cap")
-    return {"context": T, "layers": 35, "us_per_token_wall": dt * 1e6, "tokens_per_s": 1.0 / dt,
-            "weight_bytes_read_per_token": weight_bytes, "kv_bytes_read_per_token": kv_bytes,
-            "gbs_wall": (weight_bytes + kv_bytes) / dt * 1e-9}
+    res = {"context": T, "layers": 35, "us_per_token_wall": dt * 1e6, "tokens_per_s": 1.0 / dt,
+           "weight_bytes_read_per_token": weight_bytes, "kv_bytes_read_per_token": kv_bytes,
+           "gbs_wall": (weight_bytes + kv_bytes) / dt * 1e-9}
+    if lanes:
+        # continuous batching (local-engine/src/pipeline/batched.rs:271-478): `lanes` sequences, each with about T cached
+        # positions in by-lane pools, one token each per step; logits of every lane stay in device memory
+        state = pipe.new_batched_decode_state(lanes, max_ctx)
+        for i, pool in enumerate(state.pools):
+            fill_kv(pkg, ctx, K, pool, lanes, pool.lane_stride(), pkg.synth.rng(13, 40 + i))
+        positions = [T - 1 - l for l in range(lanes)]
+        lane_steps = max(steps // 2, 5)
+        toks = g.integers(0, cfg.vocab_size, (lane_steps + warmup, lanes))
+        for row in toks[:warmup]:
+            pipe.decode_batch_step(state, [int(v) for v in row], [int(v) for v in row], positions, read_logits=False)
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        for row in toks[warmup:]:
+            pipe.decode_batch_step(state, [int(v) for v in row], [int(v) for v in row], positions, read_logits=False)
+        dl = (time.perf_counter() - t0) / lane_steps
+        lg = state.logits(2)
+        if not np.isfinite(lg).all() or np.abs(lg).max() > 30.001:
+            raise RuntimeError("batched model decode produced logits outside the soft cap")
+        lane_kv = sum(kv_read_bytes(p_ + 1) for p_ in positions)
+        res["lanes"] = {"lanes": lanes, "ms_per_step_wall": dl * 1e3, "tokens_per_s": lanes / dl,
+                        "kv_bytes_read_per_step": lane_kv, "weight_bytes_read_per_step": weight_bytes,
+                        "gbs_wall": (lane_kv + weight_bytes) / dl * 1e-9}
+    return res
 
 
 def _layer_weight_bytes(pkg, layer):

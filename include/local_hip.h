@@ -301,6 +301,15 @@ LH_API int lh_dequant_q4_0_into(lh_batch* batch, const lh_buffer* data, size_t b
                                 size_t num_elements);
 LH_API int lh_dequant_tq2_0_into(lh_batch* batch, const lh_buffer* data, size_t byte_offset, lh_buffer* output,
                                  size_t num_elements);
+/* Rows `rows[0 .. n_rows)` (a device u32 list; an index past the end reads the last row, init_gemma4_qat.rs:152)
+ * of a packed [table_rows, cols] table decoded to a dense f16 [n_rows, cols] matrix in one dispatch: the embedding
+ * gather of local-engine/src/pipeline.rs:781-832 (gather_embeddings, which decodes on the CPU one row at a time)
+ * and the per-layer-embedding rows of pipeline.rs:1011-1019.  `fmt` is an lh_quant value or LH_ROWS_F16 for a
+ * table of plain f16 rows.  With scale != 1 every value is multiplied by it and rounded to f16 once more, exactly
+ * what scale_in_place_gpu_into (pipeline.rs:999-1001) does to the gathered rows. */
+#define LH_ROWS_F16 2
+LH_API int lh_dequant_rows_into(lh_batch* batch, int fmt, const lh_buffer* table, uint32_t table_rows, uint32_t cols,
+                                const lh_buffer* rows, uint32_t n_rows, float scale, lh_buffer* output);
 /* kernels.rs:6753-6802 tq2_dequant (legacy 2-bit unpack, shaders/tq2_dequant.metal:4-16). */
 LH_API int lh_tq2_dequant(lh_context* ctx, const lh_buffer* packed, const lh_buffer* scales, lh_buffer* output,
                           uint32_t num_elements);

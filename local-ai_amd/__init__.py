@@ -22,6 +22,7 @@ LIB_PATH = os.path.join(_HERE, "liblocal_hip.so")
 
 F16, F32, BF16 = 0, 1, 2
 Q4_0, TQ2_0 = 0, 1
+ROWS_F16 = 2          # lh_dequant_rows_into: a table of plain f16 rows
 _DTYPE_SIZE = {F16: 2, F32: 4, BF16: 2}
 
 SMALLM_MAX_M = 8      # local-metal/src/kernels.rs:6155
@@ -518,6 +519,12 @@ class Kernels:
     def dequant_tq2_0_into(self, batch, data, byte_offset, output, num_elements):
         _check(self._l.lh_dequant_tq2_0_into(batch._h, data._h, C.c_size_t(byte_offset), output._h,
                                              C.c_size_t(num_elements)))
+
+    def dequant_rows_into(self, batch, fmt, table, table_rows, cols, rows, n_rows, output, scale=1.0):
+        """Rows `rows[0 .. n_rows)` (device u32 indices, clamped to the last row) of a packed table as a dense f16
+        [n_rows, cols] matrix; `fmt` is Q4_0, TQ2_0 or ROWS_F16."""
+        _check(self._l.lh_dequant_rows_into(batch._h, C.c_int(fmt), table._h, _u32(table_rows), _u32(cols), rows._h,
+                                            _u32(n_rows), C.c_float(scale), output._h))
 
     def tq2_dequant(self, ctx, packed, scales, output, num_elements):
         _check(self._l.lh_tq2_dequant(ctx._h, packed._h, scales._h, output._h, _u32(num_elements)))

@@ -2,12 +2,16 @@
 (local-core/src/config/gemma4_qat.rs:170-252), the KV-cache slots with their sharing map
 (local-engine/src/pipeline.rs:379-437) and the decode core of ``Pipeline`` -- embedding gather and
 scale, per-layer inputs, the layer stack in one command batch, final norm + logits + soft cap
-(pipeline.rs:714-953).  Tokenizer, sampling, prompt caches and the multimodal front ends of the
-reference's ``Pipeline`` are not part of the hot path and are not here.
+(pipeline.rs:714-953), chunked prompt prefill (pipeline.rs:969-1100, 1332-1367) and the continuous-batching
+step over by-lane KV pools (local-engine/src/pipeline/batched.rs:72-478).  Tokenizer, sampling, prompt
+caches and the multimodal front ends of the reference's ``Pipeline`` are not part of the hot path and
+are not here.
 
-Two differences from the reference, both because buffers live in device memory: embedding rows are
-decoded by the device dequant kernels instead of by the CPU out of shared memory, and the whole token
-(set-up, layers, logits tail) is encoded into one batch with a single wait at the end.
+Differences from the reference, all because buffers live in device memory: embedding rows are decoded
+by the device dequant kernels instead of by the CPU out of shared memory; a token (set-up, layers,
+logits tail) or a batched step is encoded into one batch with a single wait at the end; and the logits
+of a batched step come from one [lanes, hidden] x table^T product that reads the embedding table once,
+where the reference runs one matvec per lane.
 """
 from __future__ import annotations
 
@@ -18,11 +22,13 @@ from typing import List, Optional
 import numpy as np
 
 from . import Buffer, CommandBatch, InvalidArgument, Kernels
-from .kv_cache import QuantizedKvCache, kv_bits_from_env, swa_ring_capacity
-from .layer import ScratchBuffers, TransformerLayer
+from . import F16, F32
+from .kv_cache import QuantizedKvCache, QuantizedUnifiedKvPool, kv_bits_from_env, swa_ring_capacity
+from .layer import BatchScratch, ScratchBuffers, TransformerLayer
 from .quant_weight import QuantWeight
 
 DEFAULT_LOGIT_SOFTCAP = 30.0   # local-engine/src/sampler.rs:30
+DEFAULT_MAX_BATCH = 256         # local-engine/src/pipeline.rs:620-622: rows of the shared multi-row scratch
 
 
 @dataclass
@@ -112,13 +118,32 @@ def build_kv_caches(config: Gemma4QATConfig, layers: List[TransformerLayer], ctx
     return caches, kv_index_map
 
 
+class BatchedDecodeState:
+    """batched.rs:25-60: one by-lane KV pool per cache slot, the lanes' device-resident positions and logits."""
+
+    def __init__(self, ctx, pools: List[QuantizedUnifiedKvPool], n_lanes: int, lane_capacity: int, vocab_size: int):
+        self.pools, self.n_lanes, self.lane_capacity = pools, n_lanes, lane_capacity
+        self.pos_buf = Buffer.empty(ctx, n_lanes * 4)
+        self.logits_buf = Buffer.empty(ctx, n_lanes * vocab_size * 4)   # [n_lanes, vocab] f32
+        self._vocab = vocab_size
+
+    def reset_lane(self, lane: int) -> None:
+        """batched.rs:55-59."""
+        for pool in self.pools:
+            pool.reset_lane(lane)
+
+    def logits(self, n: Optional[int] = None) -> np.ndarray:
+        n = self.n_lanes if n is None else n
+        return self.logits_buf.as_array(np.float32, n * self._vocab).reshape(n, self._vocab)
+
+
 class DecodePipeline:
     """The decode core of ``Pipeline`` (pipeline.rs:714-953)."""
 
     def __init__(self, ctx, kernels: Kernels, config: Gemma4QATConfig, layers: List[TransformerLayer],
                  token_embd: QuantWeight, output_norm: Buffer, max_context_length: int, ple_table=None,
                  per_layer_model_proj: Optional[QuantWeight] = None, per_layer_proj_norm: Optional[Buffer] = None,
-                 logit_softcap: float = DEFAULT_LOGIT_SOFTCAP):
+                 logit_softcap: float = DEFAULT_LOGIT_SOFTCAP, max_batch: int = DEFAULT_MAX_BATCH):
         if len(layers) != config.num_hidden_layers:
             raise InvalidArgument(f"{len(layers)} layers for a {config.num_hidden_layers}-layer configuration")
         if token_embd.rows != config.vocab_size or token_embd.cols != config.hidden_size:
@@ -137,12 +162,30 @@ class DecodePipeline:
         self.per_layer_input = self.ple_tok = self.ple_proj = None
         if ple_table is not None and per_layer_model_proj is not None and per_layer_proj_norm is not None:
             self.per_layer_input, self.ple_tok, self.ple_proj = (Buffer.empty(ctx, ple_total * 2) for _ in range(3))
+        self.max_batch = max_batch
+        self._batch_scratch: Optional[BatchScratch] = None
+        self._tokens_buf = self._ple_tokens_buf = None
         self.position = 0
         self.reset()
 
+    @property
+    def batch_scratch(self) -> BatchScratch:
+        """pipeline.rs:619-630: the shared multi-row scratch of prefill chunks and batched steps (built on first use)."""
+        if self._batch_scratch is None:
+            cfg = self.config
+            self._batch_scratch = BatchScratch(self.ctx, self.max_batch, cfg.hidden_size,
+                                               max(l.params.intermediate_size for l in self.layers),
+                                               cfg.num_attention_heads, cfg.num_key_value_heads,
+                                               max(l.params.head_dim for l in self.layers),
+                                               cfg.hidden_size_per_layer_input, cfg.num_hidden_layers)
+            self._tokens_buf = Buffer.empty(self.ctx, self.max_batch * 4)
+            self._ple_tokens_buf = Buffer.empty(self.ctx, self.max_batch * 4)
+        return self._batch_scratch
+
     @classmethod
     def from_host(cls, ctx, kernels: Kernels, config: Gemma4QATConfig, tensors: dict, max_context_length: int,
-                  logit_softcap: float = DEFAULT_LOGIT_SOFTCAP, **layer_options) -> "DecodePipeline":
+                  logit_softcap: float = DEFAULT_LOGIT_SOFTCAP, max_batch: int = DEFAULT_MAX_BATCH,
+                  **layer_options) -> "DecodePipeline":
         """Upload host tensors laid out as ``synth.decode_model_tensors`` returns them: ``layers`` (one dict of layer
         tensors each), ``token_embd`` / ``ple_table`` / ``per_layer_model_proj`` as ``(format, rows, cols, payload)``,
         the norms as f16 vectors."""
@@ -173,7 +216,7 @@ class DecodePipeline:
             model_proj = QuantWeight.from_bytes(ctx, payload, fmt_id[fmt], rows, cols)
             proj_norm = Buffer.from_slice(ctx, np.asarray(tensors["per_layer_proj_norm"], np.float16))
         return cls(ctx, kernels, config, layers, token_embd, output_norm, max_context_length, ple_table, model_proj,
-                   proj_norm, logit_softcap)
+                   proj_norm, logit_softcap, max_batch)
 
     def reset(self) -> None:
         """pipeline.rs:714-717."""
@@ -246,3 +289,138 @@ class DecodePipeline:
 
     def logits(self) -> np.ndarray:
         return self.logits_buf.as_array(np.float32, self.config.vocab_size)
+
+    # ---- multi-row paths: prefill chunks and continuous batching ---------------------------------------------------
+
+    def _embed_rows(self, batch, tokens, ple_tokens) -> bool:
+        """pipeline.rs:994-1060 / batched.rs:305-368: rows of the embedding table scaled by sqrt(hidden) into hidden_a,
+        and the per-layer inputs of every row into ple_all.  Returns whether per-layer inputs exist."""
+        cfg, K, bs = self.config, self.kernels, self.batch_scratch
+        n, h = len(tokens), cfg.hidden_size
+        self._tokens_buf.copy_from_bytes(np.asarray(tokens, np.uint32))
+        self.token_embd.dequant_rows_into(batch, K, self._tokens_buf, n, bs.hidden_a, math.sqrt(h))
+        if self.per_layer_input is None:
+            return False
+        pld, nl = cfg.hidden_size_per_layer_input, cfg.num_hidden_layers
+        total = n * pld * nl
+        self._ple_tokens_buf.copy_from_bytes(np.asarray(ple_tokens, np.uint32))
+        self.ple_table.dequant_rows_into(batch, K, self._ple_tokens_buf, n, bs.ple_tok, math.sqrt(pld))
+        self.per_layer_model_proj.matmul_nt_into(batch, K, bs.hidden_a, bs.ple_proj, n)
+        K.scale_in_place_gpu_into(batch, bs.ple_proj, 1.0 / math.sqrt(h), total)
+        K.rms_norm_into(batch, bs.ple_proj, self.per_layer_proj_norm, bs.ple_proj, pld, n * nl, cfg.rms_norm_eps)
+        K.residual_add_into(batch, bs.ple_proj, bs.ple_tok, bs.ple_all, total)
+        K.scale_in_place_gpu_into(batch, bs.ple_all, math.sqrt(0.5), total)
+        return True
+
+    def forward_tokens_batch(self, tokens, start_pos: int, ple_tokens=None, batch=None) -> bool:
+        """pipeline.rs:969-1100: one prefill chunk, rows at positions start_pos .. start_pos + len(tokens), through every
+        layer's batch path into the single-sequence caches.  Returns True when the result is in batch_scratch.hidden_a."""
+        n = len(tokens)
+        ple_tokens = tokens if ple_tokens is None else ple_tokens
+        if len(ple_tokens) != n:
+            raise InvalidArgument(f"PLE token count {len(ple_tokens)} does not match token count {n}")
+        if n < 1 or n > self.max_batch:
+            raise InvalidArgument(f"chunk of {n} rows must be in 1..={self.max_batch}")
+        if start_pos + n > self.max_context:
+            raise InvalidArgument(f"positions up to {start_pos + n} beyond the context of {self.max_context}")
+        own = batch is None
+        batch = batch or CommandBatch(self.ctx)
+        bs = self.batch_scratch
+        ple_arg = (bs.ple_all, self.config.num_hidden_layers) if self._embed_rows(batch, tokens, ple_tokens) else None
+        cur_in_a = True
+        for i, layer in enumerate(self.layers):
+            inp, out = (bs.hidden_a, bs.hidden_b) if cur_in_a else (bs.hidden_b, bs.hidden_a)
+            layer.forward_batch(self.kernels, batch, n, start_pos, inp, out, bs, self.scratch.ones,
+                                self.kv_caches[self.kv_index_map[i]], ple_arg)
+            cur_in_a = not cur_in_a
+        if own:
+            batch.commit_and_wait()
+        return cur_in_a
+
+    def prefill_prompt(self, tokens, chunk_len: Optional[int] = None) -> bool:
+        """pipeline.rs:1332-1367 without the prompt cache: all tokens but the last in chunks of at most max_batch rows,
+        the last through forward_token so that its hidden state is where write_logits reads it."""
+        if len(tokens) == 0:
+            raise InvalidArgument("prefill prompt is empty")
+        chunk_len = min(chunk_len or self.max_batch, self.max_batch)
+        last_idx = len(tokens) - 1
+        pos = 0
+        while pos < last_idx:
+            chunk = tokens[pos:min(pos + chunk_len, last_idx)]
+            self.forward_tokens_batch(chunk, pos)
+            pos += len(chunk)
+        self.position = last_idx
+        return self.forward_token(tokens[last_idx], last_idx)
+
+    def new_batched_decode_state(self, n_lanes: int, lane_capacity: int) -> BatchedDecodeState:
+        """batched.rs:72-151: one pool per cache slot with the slot's head_dim; a sliding-window slot's lanes are rings of
+        the staging cache's size so that a wrapped prefill copies slot for slot."""
+        if n_lanes == 0:
+            raise InvalidArgument("n_lanes must be >= 1")
+        if n_lanes > self.max_batch:
+            raise InvalidArgument(f"n_lanes {n_lanes} exceeds batch scratch capacity {self.max_batch}")
+        bits = kv_bits_from_env()
+        pools = []
+        for staging in self.kv_caches:
+            lane_ring = 0
+            if staging.is_ringed():
+                lane_ring = staging.physical_positions
+                if lane_capacity < lane_ring:
+                    raise InvalidArgument(f"lane_capacity {lane_capacity} below sliding-window ring {lane_ring}")
+            pools.append(QuantizedUnifiedKvPool(self.ctx, n_lanes, lane_capacity, self.config.num_key_value_heads,
+                                                staging.head_dim, bits, lane_ring))
+        return BatchedDecodeState(self.ctx, pools, n_lanes, lane_capacity, self.config.vocab_size)
+
+    def prefill_lane(self, state: BatchedDecodeState, lane: int, tokens) -> np.ndarray:
+        """batched.rs:162-197: prefill on the single-sequence caches, keep the last token's logits, copy the encoded
+        rows into the lane's region of every pool."""
+        if len(tokens) == 0:
+            raise InvalidArgument("prefill prompt is empty")
+        if lane >= state.n_lanes:
+            raise InvalidArgument(f"lane {lane} out of range (n_lanes {state.n_lanes})")
+        if len(tokens) > state.lane_capacity:
+            raise InvalidArgument(f"prompt length {len(tokens)} exceeds lane_capacity {state.lane_capacity}")
+        self.reset()
+        final_in_a = self.prefill_prompt(tokens)
+        batch = CommandBatch(self.ctx)
+        self.write_logits(final_in_a, batch=batch)
+        for slot, pool in enumerate(state.pools):
+            pool.copy_prefill_from(batch, self.kv_caches[slot], lane, len(tokens))
+        batch.commit_and_wait()
+        return self.logits().copy()
+
+    def encode_batch_step(self, batch, state: BatchedDecodeState, n: int) -> None:
+        """The device work of decode_batch_step for the tokens and positions already uploaded: layers at M = n over the
+        lanes' pools (batched.rs:371-409), then output norm, logits and soft cap of every lane (batched.rs:411-455)."""
+        cfg, K, bs = self.config, self.kernels, self.batch_scratch
+        h = cfg.hidden_size
+        ple_arg = (bs.ple_all, cfg.num_hidden_layers) if self.per_layer_input is not None else None
+        cur_in_a = True
+        for i, layer in enumerate(self.layers):
+            inp, out = (bs.hidden_a, bs.hidden_b) if cur_in_a else (bs.hidden_b, bs.hidden_a)
+            layer.forward_decode_batch_turbo(batch, K, n, state.pos_buf, inp, out, bs, self.scratch.ones,
+                                             state.pools[self.kv_index_map[i]], ple_arg)
+            cur_in_a = not cur_in_a
+        final_hidden = bs.hidden_a if cur_in_a else bs.hidden_b
+        K.rms_norm_into(batch, final_hidden, self.output_norm, bs.normed, h, n, cfg.rms_norm_eps)
+        self.token_embd.matmul_nt_typed_into(batch, K, bs.normed, F16, state.logits_buf, F32, n)
+        if self.logit_softcap > 0.0:
+            K.logit_softcap_gpu_into(batch, state.logits_buf, self.logit_softcap, n * cfg.vocab_size)
+
+    def decode_batch_step(self, state: BatchedDecodeState, tokens, ple_tokens, positions, read_logits: bool = True):
+        """batched.rs:271-478: one token for each of len(tokens) active lanes (lane l is row l), lane l at
+        positions[l]; returns the [n, vocab] logits (or leaves them in state.logits_buf with read_logits=False)."""
+        n = len(tokens)
+        if n == 0 or n > state.n_lanes:
+            raise InvalidArgument(f"active lanes {n} must be in 1..={state.n_lanes}")
+        if len(ple_tokens) != n or len(positions) != n:
+            raise InvalidArgument("tokens, ple_tokens and positions must have equal length")
+        for lane, pos in enumerate(positions):
+            if pos >= state.lane_capacity:
+                raise InvalidArgument(f"lane {lane} position {pos} exceeds capacity {state.lane_capacity}")
+        state.pos_buf.copy_from_bytes(np.asarray(positions, np.uint32))
+        batch = CommandBatch(self.ctx)
+        self._embed_rows(batch, tokens, ple_tokens)
+        self.encode_batch_step(batch, state, n)
+        batch.commit_and_wait()
+        return state.logits(n).copy() if read_logits else None

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from . import Q4_0, TQ2_0, F16, F32, BF16, Buffer, InvalidArgument, Kernels
+from . import Q4_0, TQ2_0, ROWS_F16, F16, F32, BF16, Buffer, InvalidArgument, Kernels
 
 _BLOCK = {Q4_0: (32, 18), TQ2_0: (256, 66)}
 W_F16 = "f16"   # GGUFType::F16: plain f16 rows, served by the FP16 matvec / matmul kernels (layer.rs:27-34)
@@ -91,3 +91,9 @@ class QuantWeight:
             kernels.dequant_tq2_0_into(batch, self.buf, off, out, self.cols)
         else:
             batch.blit_copy(self.buf, off, out, 0, self.cols * 2)   # an f16 row is its own dequantisation
+
+    def dequant_rows_into(self, batch, kernels: Kernels, rows: Buffer, n_rows: int, out: Buffer, scale: float = 1.0) -> None:
+        """The rows listed in the device u32 buffer `rows` as a dense f16 [n_rows, cols] matrix, optionally scaled: the
+        embedding gather of a chunk or of a step over many lanes (local-engine/src/pipeline.rs:781-832) in one dispatch."""
+        fmt = ROWS_F16 if self.ty == W_F16 else self.ty
+        kernels.dequant_rows_into(batch, fmt, self.buf, self.rows, self.cols, rows, n_rows, out, scale)

@@ -124,6 +124,10 @@ class QuantRowTable:
         """Row `row` (clamped to the last row, init_gemma4_qat.rs:152) as cols f16 values into `out`."""
         self._w.dequant_row_into(batch, kernels, row, out)
 
+    def dequant_rows_into(self, batch, kernels: Kernels, rows: Buffer, n_rows: int, out: Buffer, scale: float = 1.0) -> None:
+        """Rows listed in a device u32 buffer, decoded side by side (pipeline.rs:1011-1019 loops over the tokens)."""
+        self._w.dequant_rows_into(batch, kernels, rows, n_rows, out, scale)
+
     def dequant_row(self, ctx, kernels: Kernels, row: int) -> np.ndarray:
         out = Buffer.empty(ctx, self._w.cols * 2)
         batch = CommandBatch(ctx)

@@ -325,6 +325,44 @@ def test_block_dequant_bit_exact(pkg, gpu, oracle, fmt):
         assert np.array_equal(got3[~nan], want3[~nan]) and np.all(np.isnan(got3.view(np.float16)[nan]))
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0", "f16"])
+def test_dequant_rows_gather_bit_exact(pkg, gpu, oracle, fmt):
+    """Rows picked by a device index list (an index past the end reads the last row), decoded side by side, equal the CPU
+    path's row-by-row dequant (pipeline.rs:781-832) bit for bit; with a scale, its scale_in_place on top."""
+    from oracle import layer_glue as G
+    ctx, K = gpu
+    n, k = 37, 1536
+    g = pkg.synth.rng(61, 7)
+    if fmt == "f16":
+        table = g.standard_normal((n, k)).astype(np.float16)
+        w = pkg.QuantWeight.f16(pkg.Buffer.from_slice(ctx, table), n, k)
+        want = table.view(np.uint16)
+    else:
+        raw = pkg.synth.weights(fmt, n, k, g)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0, n, k)
+        want = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).reshape(n, k)
+    idx = np.array([0, 36, 5, 5, 400, 17, 2 ** 32 - 1], np.uint32)
+    src = np.minimum(idx, n - 1)
+    rows = pkg.Buffer.from_slice(ctx, idx)
+    out = pkg.Buffer.empty(ctx, idx.size * k * 2)
+    for scale in (1.0, float(np.sqrt(np.float32(k)))):
+        batch = pkg.CommandBatch(ctx)
+        w.dequant_rows_into(batch, K, rows, idx.size, out, scale)
+        batch.commit_and_wait()
+        expect = want[src]
+        if scale != 1.0:
+            expect = G.scale_in_place(expect.view(np.float16), scale).view(np.uint16)
+        assert np.array_equal(out.as_array(np.uint16).reshape(idx.size, k), expect.reshape(idx.size, k)), scale
+    batch = pkg.CommandBatch(ctx)
+    with pytest.raises(pkg.InvalidArgument):
+        K.dequant_rows_into(batch, 7, w.buf, n, k, rows, idx.size, out)
+    with pytest.raises(pkg.InvalidArgument):
+        K.dequant_rows_into(batch, pkg.ROWS_F16, w.buf, n, k, rows, idx.size + 1, out)        # index list too short
+    with pytest.raises(pkg.InvalidArgument):
+        K.dequant_rows_into(batch, pkg.Q4_0, w.buf, n, 48, rows, 1, out)                      # not block aligned
+    K.dequant_rows_into(batch, pkg.Q4_0, w.buf, n, k, rows, 0, out)                           # nothing to do
+
+
 def test_legacy_tq2_dequant(pkg, gpu, oracle):
     ctx, K = gpu
     g = pkg.synth.rng(9)
