@@ -429,7 +429,7 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     return res
 
 
-def bench_model(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
+def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64):
     """End-to-end decode of a synthetic model with the geometry of the reference's Gemma 4 E2B configuration
     (local-core/src/config/gemma4_qat.rs:262-283: vocabulary 262144, hidden 1536, 35 layers in a sliding x4 / full
     pattern with head_dim 256 / 512, window 512, the last 20 layers sharing KV, per-layer inputs of 256; Q4_0
@@ -458,8 +458,9 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
     max_ctx = T + 256
     pipe = P.DecodePipeline.from_host(ctx, K, cfg, tensors, max_ctx)
     del tensors, one, kinds
-    for i, c in enumerate(pipe.kv_caches):
-        fill_kv(pkg, ctx, K, c, 1, min(T, c.physical_positions), pkg.synth.rng(13, 10 + i))
+    if single:
+        for i, c in enumerate(pipe.kv_caches):
+            fill_kv(pkg, ctx, K, c, 1, min(T, c.physical_positions), pkg.synth.rng(13, 10 + i))
     pipe.position = T - 1
     weight_bytes = sum(_layer_weight_bytes(pkg, l) for l in pipe.layers) + pipe.token_embd.device_bytes() \
         + pipe.per_layer_model_proj.device_bytes()
@@ -474,20 +475,21 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768, lanes=64):
         return total
 
     kv_bytes = kv_read_bytes(T)
-    tokens = [int(v) for v in g.integers(0, cfg.vocab_size, steps + warmup)]
-    for t in tokens[:warmup]:
-        pipe.decode_step(t)
-    ctx.synchronize()
-    t0 = time.perf_counter()
-    for t in tokens[warmup:]:
-        pipe.decode_step(t)
-    dt = (time.perf_counter() - t0) / steps
-    logits = pipe.logits()
-    if not np.isfinite(logits).all() or np.abs(logits).max() > 30.001:
-        raise RuntimeError("model decode produced logits outside the soft cap")
-    res = {"context": T, "layers": 35, "us_per_token_wall": dt * 1e6, "tokens_per_s": 1.0 / dt,
-           "weight_bytes_read_per_token": weight_bytes, "kv_bytes_read_per_token": kv_bytes,
-           "gbs_wall": (weight_bytes + kv_bytes) / dt * 1e-9}
+    res = {"context": T, "layers": 35}
+    if single:
+        tokens = [int(v) for v in g.integers(0, cfg.vocab_size, steps + warmup)]
+        for t in tokens[:warmup]:
+            pipe.decode_step(t)
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        for t in tokens[warmup:]:
+            pipe.decode_step(t)
+        dt = (time.perf_counter() - t0) / steps
+        logits = pipe.logits()
+        if not np.isfinite(logits).all() or np.abs(logits).max() > 30.001:
+            raise RuntimeError("model decode produced logits outside the soft cap")
+        res.update({"us_per_token_wall": dt * 1e6, "tokens_per_s": 1.0 / dt, "weight_bytes_read_per_token": weight_bytes,
+                    "kv_bytes_read_per_token": kv_bytes, "gbs_wall": (weight_bytes + kv_bytes) / dt * 1e-9})
     if lanes:
         # continuous batching (local-engine/src/pipeline/batched.rs:271-478): `lanes` sequences, each with about T cached
         # positions in by-lane pools, one token each per step; logits of every lane stay in device memory
@@ -657,7 +659,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model",
+    ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model,model_lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -736,8 +738,9 @@ def main():
         extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
-    if "model" in legs:
-        extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup)
+    if legs & {"model", "model_lanes"}:
+        extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup, single="model" in legs,
+                                                         lanes=64 if "model_lanes" in legs else 0)
         log("[bench] model decode:", extra["model_decode_e2b_geometry"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6

@@ -202,6 +202,19 @@ LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, co
 LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, lh_dtype input_dtype,
                                          const lh_buffer* weight, lh_buffer* output, lh_dtype output_dtype,
                                          uint32_t m, uint32_t k, uint32_t n);
+/* A product followed by the row-wise norm that consumes it, as one encoded step: out = rms_norm(in[m, k] . w^T,
+ * norm_weight) (+ residual) (* scale), and with norm2_weight also out2 = rms_norm(out, norm2_weight).  This is the
+ * sequence matmul_nt_into -> rms_norm_add_into (-> scale_in_place_gpu_into) (-> rms_norm_into) of the multi-row layer
+ * paths -- local-engine/src/layer.rs:640-652 (attention output, post-attention norm + residual, feed-forward norm),
+ * 664-672 (down projection, post-feed-forward norm + residual), 699-716 (per-layer projection, its norm + residual,
+ * the layer's output scale) -- with the roundings of the separate kernels, so the results are theirs bit for bit.  For
+ * a decode batch (17 .. 64 rows) the norm kernel sums the product's k-split partial tiles itself, which removes the
+ * reduction pass as well.  residual / norm2_weight / out2 may be NULL; out may alias residual; n must be a multiple
+ * of 8, at most 8192, and every buffer 16-byte aligned. */
+LH_API int lh_matmul_nt_quant_norm_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* weight,
+                                        uint32_t m, uint32_t k, uint32_t n, const lh_buffer* norm_weight,
+                                        const lh_buffer* residual, lh_buffer* output, float eps, int apply_scale,
+                                        float scale, const lh_buffer* norm2_weight, lh_buffer* output2);
 /* Up to four weight matrices of one format and one k against the same activations as one launch (what layer.rs:570-590 /
  * 658-662 issue back to back: Q, K and V, or gate and up), f16 in and out; output i is [m, ns[i]].  Shapes the separate
  * calls would send to other kernels (m <= 16, or enough 128-row tiles to fill the chip) are issued as those calls. */

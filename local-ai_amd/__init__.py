@@ -418,6 +418,17 @@ class Kernels:
                                                        _handles(outputs), (C.c_uint32 * n)(*[int(v) for v in ns]),
                                                        _u32(m), _u32(k)))
 
+    def matmul_nt_quant_norm_into(self, batch, fmt, input, weight, m, k, n, norm_weight, residual, output, eps, scale=None,
+                                  norm2_weight=None, output2=None):
+        """matmul_nt -> rms_norm(_add) (-> scale_in_place) (-> rms_norm) of the multi-row layer paths as one step, bit for
+        bit the separate kernels' result; `residual`, `scale`, `norm2_weight` / `output2` are optional."""
+        _check(self._l.lh_matmul_nt_quant_norm_into(batch._h, C.c_int(fmt), input._h, weight._h, _u32(m), _u32(k), _u32(n),
+                                                    norm_weight._h, residual._h if residual is not None else None, output._h,
+                                                    C.c_float(eps), C.c_int(0 if scale is None else 1),
+                                                    C.c_float(0.0 if scale is None else scale),
+                                                    norm2_weight._h if norm2_weight is not None else None,
+                                                    output2._h if output2 is not None else None))
+
     def matmul_nt_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))
 

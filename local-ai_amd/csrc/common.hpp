@@ -94,6 +94,27 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
 int lh_matvec_rows(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer* weight, const lh_buffer* input, lh_dtype at,
                    lh_buffer* output, lh_dtype ct, uint32_t n, uint32_t k, const char* op);
 
+// A row-wise RMS norm whose input is f16 rows (`in`) or the f32 partial tiles of a k-split product (`partial`: split z
+// of row r starts at partial[(z * part_rows + r) * part_cols]), with the optional residual, output scale and second
+// norm of a decoder layer's tail; defined beside the stand-alone norm kernels, launched by the fused product entry.
+struct LhNormFused {
+    const uint16_t* in;
+    const float* partial;
+    uint32_t splits, part_rows, part_cols;
+    const uint16_t* w;
+    const uint16_t* res;      // null: no residual
+    uint16_t* out;
+    uint32_t dim, rows;
+    float eps;
+    uint32_t apply_scale;
+    float scale;
+    uint32_t tail;            // 0 here: the residual is added in f32 (rms_norm_add); passed through to the shared chunk arithmetic
+    const uint16_t* w2;       // null: no second norm
+    uint16_t* out2;
+};
+bool lh_norm_fused_supported(uint32_t dim);
+void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
+
 static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }
 
 // ---- device helpers -------------------------------------------------------

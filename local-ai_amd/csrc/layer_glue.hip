@@ -34,6 +34,30 @@ __device__ __forceinline__ float norm_tail(float normed, float res, uint32_t tai
     return tail == 2 ? (float)sum * scale : (float)sum;
 }
 
+// The arithmetic of one 8-element chunk, shared by every kernel that must reproduce the stand-alone norm bit for bit.
+__device__ __forceinline__ void rms_sumsq8(const uint4& v, float& s) {
+    const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) { const float a = lh_h2f((uint16_t)(wv[j] & 0xFFFF)), b = lh_h2f((uint16_t)(wv[j] >> 16)); s += a * a; s += b * b; }
+}
+template <bool ADD>
+__device__ __forceinline__ uint4 rms_apply8(const uint4& v, const uint4& g, const uint4& r, float rms, uint32_t tail, float scale) {
+    const uint32_t wv[4] = {v.x, v.y, v.z, v.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
+    uint32_t wo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float lo = lh_h2f((uint16_t)(wv[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
+        float hi = lh_h2f((uint16_t)(wv[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
+        if (ADD) {
+            const float rlo = lh_h2f((uint16_t)(wr[j] & 0xFFFF)), rhi = lh_h2f((uint16_t)(wr[j] >> 16));
+            if (tail) { lo = norm_tail(lo, rlo, tail, scale); hi = norm_tail(hi, rhi, tail, scale); }
+            else { lo += rlo; hi += rhi; }
+        }
+        wo[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
+    }
+    return make_uint4(wo[0], wo[1], wo[2], wo[3]);
+}
+
 template <bool ADD, int VEC>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const uint16_t* __restrict__ w, const uint16_t* res, uint16_t* out,   // out may be in or res
                                                       uint32_t dim, float eps, uint32_t tail = 0, float scale = 1.0f) {
@@ -43,9 +67,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const
     if constexpr (VEC == 8) {
         for (uint32_t i = threadIdx.x * 8; i < dim; i += blockDim.x * 8) {
             const uint4 v = *reinterpret_cast<const uint4*>(in + row + i);
-            const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) { const float a = lh_h2f((uint16_t)(wv[j] & 0xFFFF)), b = lh_h2f((uint16_t)(wv[j] >> 16)); s += a * a; s += b * b; }
+            rms_sumsq8(v, s);
         }
     } else {
         for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) { const float v = h_at(in, row + i); s += v * v; }
@@ -56,20 +78,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const
             const uint4 v = *reinterpret_cast<const uint4*>(in + row + i), g = *reinterpret_cast<const uint4*>(w + i);
             uint4 r = v;
             if (ADD) r = *reinterpret_cast<const uint4*>(res + row + i);
-            const uint32_t wv[4] = {v.x, v.y, v.z, v.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
-            uint32_t wo[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float lo = lh_h2f((uint16_t)(wv[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
-                float hi = lh_h2f((uint16_t)(wv[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
-                if (ADD) {
-                    const float rlo = lh_h2f((uint16_t)(wr[j] & 0xFFFF)), rhi = lh_h2f((uint16_t)(wr[j] >> 16));
-                    if (tail) { lo = norm_tail(lo, rlo, tail, scale); hi = norm_tail(hi, rhi, tail, scale); }
-                    else { lo += rlo; hi += rhi; }
-                }
-                wo[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
-            }
-            *reinterpret_cast<uint4*>(out + row + i) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+            *reinterpret_cast<uint4*>(out + row + i) = rms_apply8<ADD>(v, g, r, rms, tail, scale);
         }
     } else {
         for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
@@ -87,6 +96,69 @@ void launch_rms_norm(hipStream_t stream, const void* in, const void* w, const vo
     const uint32_t threads = vec ? (dim >= 2048 ? 256u : (dim >= 1024 ? 128u : 64u)) : (dim >= 256 ? 256u : (dim > 64 ? 128u : 64u));
     if (vec) hipLaunchKernelGGL((rms_norm_kernel<ADD, 8>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps, tail, scale);
     else hipLaunchKernelGGL((rms_norm_kernel<ADD, 1>), dim3(rows), dim3(threads), 0, stream, (const uint16_t*)in, (const uint16_t*)w, (const uint16_t*)res, (uint16_t*)out, dim, eps, tail, scale);
+}
+
+// rms_norm_kernel<ADD, 8> with its input taken either from f16 rows or from the f32 partial tiles of a k-split product
+// (summed in split order and rounded to f16, which is what the product's own reduction would have stored), optionally
+// followed by the output scale (scale_in_place.metal:5-14) and by a second plain norm of the row just produced
+// (layer.rs:640-652: post-attention norm + residual, then the feed-forward norm): up to four dispatches of a decode
+// batch's layer in one.  Same thread count, accumulation order and rounding points as the separate kernels, so the
+// results are theirs bit for bit.  A thread keeps its (up to four) 8-element chunks in registers between the passes.
+template <bool PART, bool ADD>
+__global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a) {
+    __shared__ float scratch[4];
+    const uint32_t dim = a.dim, rowi = blockIdx.x;
+    const size_t row = (size_t)rowi * dim;
+    uint4 x[4], o[4];
+    float s = 0.0f;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
+        if (i >= dim) break;
+        if constexpr (PART) {
+            float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (uint32_t z = 0; z < a.splits; z++) {
+                const float* p = a.partial + ((size_t)z * a.part_rows + rowi) * a.part_cols + i;
+                const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
+                v[0] += lo.x; v[1] += lo.y; v[2] += lo.z; v[3] += lo.w; v[4] += hi.x; v[5] += hi.y; v[6] += hi.z; v[7] += hi.w;
+            }
+            x[it] = make_uint4((uint32_t)lh_f2h(v[0]) | ((uint32_t)lh_f2h(v[1]) << 16), (uint32_t)lh_f2h(v[2]) | ((uint32_t)lh_f2h(v[3]) << 16),
+                               (uint32_t)lh_f2h(v[4]) | ((uint32_t)lh_f2h(v[5]) << 16), (uint32_t)lh_f2h(v[6]) | ((uint32_t)lh_f2h(v[7]) << 16));
+        } else {
+            x[it] = *reinterpret_cast<const uint4*>(a.in + row + i);
+        }
+        rms_sumsq8(x[it], s);
+    }
+    const float rms = rsqrtf(block_sum(s, scratch) / (float)dim + a.eps);
+    float s2 = 0.0f;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
+        if (i >= dim) break;
+        const uint4 g = *reinterpret_cast<const uint4*>(a.w + i);
+        uint4 r = x[it];
+        if (ADD) r = *reinterpret_cast<const uint4*>(a.res + row + i);
+        uint4 w = rms_apply8<ADD>(x[it], g, r, rms, a.tail, 1.0f);
+        if (a.apply_scale) {
+            uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                ws[j] = (uint32_t)lh_f2h(lh_h2f((uint16_t)(ws[j] & 0xFFFF)) * a.scale) | ((uint32_t)lh_f2h(lh_h2f((uint16_t)(ws[j] >> 16)) * a.scale) << 16);
+            w = make_uint4(ws[0], ws[1], ws[2], ws[3]);
+        }
+        o[it] = w;
+        rms_sumsq8(w, s2);
+        *reinterpret_cast<uint4*>(a.out + row + i) = w;
+    }
+    if (a.w2 == nullptr) return;
+    const float rms2 = rsqrtf(block_sum(s2, scratch) / (float)dim + a.eps);
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
+        if (i >= dim) break;
+        const uint4 g = *reinterpret_cast<const uint4*>(a.w2 + i);
+        *reinterpret_cast<uint4*>(a.out2 + row + i) = rms_apply8<false>(o[it], g, o[it], rms2, a.tail, 1.0f);
+    }
 }
 
 // qk_norm.metal:6-56 (in place; head h of `qk`), and 70-140 with the NEOX rotation fused: the normalised values are
@@ -225,6 +297,21 @@ int finish(lh_batch* batch, const char* op) {
 }
 
 }  // namespace
+
+bool lh_norm_fused_supported(uint32_t dim) { return (dim & 7) == 0 && dim <= 8192; }
+
+void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a) {
+    // the thread count launch_rms_norm picks for 16-byte accesses: the partial sums of the squares add up in the same order
+    const uint32_t threads = a.dim >= 2048 ? 256u : (a.dim >= 1024 ? 128u : 64u);
+    const bool part = a.partial != nullptr, add = a.res != nullptr;
+    if (part) {
+        if (add) hipLaunchKernelGGL((rms_norm_fused_kernel<true, true>), dim3(a.rows), dim3(threads), 0, stream, a);
+        else hipLaunchKernelGGL((rms_norm_fused_kernel<true, false>), dim3(a.rows), dim3(threads), 0, stream, a);
+    } else {
+        if (add) hipLaunchKernelGGL((rms_norm_fused_kernel<false, true>), dim3(a.rows), dim3(threads), 0, stream, a);
+        else hipLaunchKernelGGL((rms_norm_fused_kernel<false, false>), dim3(a.rows), dim3(threads), 0, stream, a);
+    }
+}
 
 extern "C" {
 

@@ -614,6 +614,211 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
     }
 }
 
+// ---- a decode batch of 17 .. 64 rows: weights straight from global memory into MFMA operands ---------------------------------
+// At these row counts a product is a few microseconds of matrix-core time and what counts is latency, so this kernel
+// has no staging phase and one barrier.  A workgroup owns 64 weight rows (four 16-row MFMA tiles) and a k range; its
+// four waves split that range in quarters, every wave multiplying all four tiles against all activation rows for its
+// quarter (one B fragment feeds four MFMAs, which keeps the activation reads -- straight from L2, 16 bytes a lane -- at
+// what a CU's vector memory path delivers), and the four partial tiles are added through LDS at the end.
+//
+// A lane fetches the codes it turns into its own A fragments, 8 bytes at a time, one "unit" ahead:
+//   Q4_0  unit = 2 blocks (64 k).  Lane (row r, g) reads qs bytes 8(g&1) .. +8 of block (g>>1): the low nibbles are
+//         elements 8(g&1) .. +8 of that block (fragment 0), the high nibbles elements 16 + 8(g&1) .. +8 (fragment 1).
+//   TQ2_0 unit = half a block (128 k).  Lane (r, g) reads bytes 8g .. +8 of the half: field f of those bytes is
+//         elements 32 f + 8g .. +8 of the half (fragment f, 0 .. 3).
+// A code byte c becomes the f16 value 1024 + c by byte permutation (0x6400 | c), the zero point is subtracted exactly
+// and the result multiplied by the block scale in f16: the CPU path's dequantised weight f16((q - 8) d) / d (q - 1)
+// (qat_recover.rs:39-47, 84-93) bit for bit, as in the LDS-tiled kernels.  The B fragment of a k step holds the
+// activations of the same eight k indices, read from the row-major f16 matrix.
+template <int FMT> struct Skinny;
+template <> struct Skinny<kQ4> { static constexpr int unit_k = 64, frags = 2; };
+template <> struct Skinny<kTQ2> { static constexpr int unit_k = 128, frags = 4; };
+
+struct SkinnyRaw { uint32_t w0, w1, d; };
+
+__device__ __forceinline__ uint2 ld8_align2(const uint8_t* p) {
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    typedef u32x2_t __attribute__((aligned(2))) u32x2_a2;
+    const u32x2_t v = *reinterpret_cast<const u32x2_a2*>(p);
+    return make_uint2(v.x, v.y);
+}
+
+template <int FMT>
+__device__ __forceinline__ f16x8 skinny_fragment(const SkinnyRaw& raw, int f) {
+    uint32_t c0, c1;
+    f16x2 zp;
+    if constexpr (FMT == kQ4) { c0 = (raw.w0 >> (4 * f)) & 0x0F0F0F0Fu; c1 = (raw.w1 >> (4 * f)) & 0x0F0F0F0Fu; zp = (f16x2){(_Float16)1032.0f, (_Float16)1032.0f}; }
+    else { c0 = (raw.w0 >> (2 * f)) & 0x03030303u; c1 = (raw.w1 >> (2 * f)) & 0x03030303u; zp = (f16x2){(_Float16)1025.0f, (_Float16)1025.0f}; }
+    const f16x2 dd = __builtin_bit_cast(f16x2, raw.d);
+    const uint32_t p[4] = {__builtin_amdgcn_perm(0x64646464u, c0, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, c0, 0x04030402u),
+                           __builtin_amdgcn_perm(0x64646464u, c1, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, c1, 0x04030402u)};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(f16x2, p[i]) - zp) * dd);
+    struct { uint32_t v[4]; } t = {{o[0], o[1], o[2], o[3]}};
+    return __builtin_bit_cast(f16x8, t);
+}
+
+template <int FMT, int CDT>
+__global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W_one, void* __restrict__ C_one,
+                                                              uint32_t M, uint32_t K, uint32_t N_one, float* __restrict__ partial,
+                                                              uint32_t units_per_wave, GroupArgs grp) {
+    constexpr int UK = Skinny<FMT>::unit_k, NF = Skinny<FMT>::frags;
+    __shared__ float4 red[4][4][4][64];                       // [wave][tile][activation group][lane]
+    const uint8_t* __restrict__ W = W_one;
+    void* __restrict__ C = C_one;
+    uint32_t N = N_one, tile = blockIdx.x >> 1;               // blockIdx.x counts 64-row halves of the 128-row tile grid
+    if (grp.count) {
+        const uint32_t gi = group_of_tile(grp, tile);
+        W = grp.W[gi]; C = grp.C[gi]; N = grp.N[gi];
+        tile -= grp.tile0[gi];
+    }
+    const uint32_t n0 = tile * BN + (blockIdx.x & 1) * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = FMT == kQ4 ? (size_t)(K >> 5) * 18 : (size_t)(K >> 8) * 66;
+    const uint32_t k_begin = (blockIdx.z * 4 + wave) * units_per_wave * UK;
+
+    const uint8_t* wrow = W + (size_t)(n0 + r) * row_bytes;   // tile t starts 16 rows further on
+    const size_t tile_bytes = 16 * row_bytes;
+    const uint16_t* xrow[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t m = 16 * j + r;
+        xrow[j] = X + (size_t)(m < M ? m : M - 1) * K;        // rows past M repeat the last one and are never stored
+    }
+
+    auto load_a = [&](SkinnyRaw (&raw)[4], uint32_t k0) {
+        size_t off, doff;
+        if constexpr (FMT == kQ4) { const size_t b = (k0 >> 5) + (g >> 1); doff = b * 18; off = doff + 2 + 8 * (g & 1); }
+        else { const size_t b = k0 >> 8; doff = b * 66 + 64; off = b * 66 + 32 * ((k0 >> 7) & 1) + 8 * g; }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint8_t* p = wrow + t * tile_bytes;
+            const uint2 w = ld8_align2(p + off);
+            const uint32_t d = *reinterpret_cast<const uint16_t*>(p + doff);
+            raw[t].w0 = w.x; raw[t].w1 = w.y; raw[t].d = d | (d << 16);
+        }
+    };
+    auto load_b = [&](f16x8 (&b)[NF][4], uint32_t k0) {
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            uint32_t kf;
+            if constexpr (FMT == kQ4) kf = k0 + 32 * (g >> 1) + 8 * (g & 1) + 16 * f;
+            else kf = k0 + 32 * f + 8 * g;
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[f][j] = *reinterpret_cast<const f16x8*>(xrow[j] + kf);
+        }
+    };
+
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const SkinnyRaw (&raw)[4], const f16x8 (&b)[NF][4]) {
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const f16x8 a = skinny_fragment<FMT>(raw[t], f);
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[f][j], acc[t][j], 0, 0, 0);
+            }
+    };
+
+    // two register sets, the unit after the one being multiplied always in flight; the load past the end re-reads the last unit
+    SkinnyRaw ra0[4], ra1[4];
+    f16x8 rb0[NF][4], rb1[NF][4];
+    const uint32_t last = k_begin + (units_per_wave - 1) * UK;
+    load_a(ra0, k_begin);
+    load_b(rb0, k_begin);
+    for (uint32_t u = 0; u < units_per_wave; u += 2) {
+        const uint32_t k1 = k_begin + (u + 1) * UK, k2 = k_begin + (u + 2) * UK;
+        load_a(ra1, k1 < last ? k1 : last);
+        load_b(rb1, k1 < last ? k1 : last);
+        multiply(ra0, rb0);
+        if (u + 1 < units_per_wave) {
+            load_a(ra0, k2 < last ? k2 : last);
+            load_b(rb0, k2 < last ? k2 : last);
+            multiply(ra1, rb1);
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) red[wave][t][j][lane] = make_float4(acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]);
+    __syncthreads();
+    // wave w finishes tile w: D[row 4g + i][activation row r] of each group j
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float4 v = red[0][wave][j][lane];
+#pragma unroll
+        for (int w = 1; w < 4; w++) {
+            const float4 o = red[w][wave][j][lane];
+            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+        }
+        const uint32_t m = 16 * j + r;
+        if (m >= M) continue;
+        const uint32_t nl = 16 * wave + 4 * g;
+        if (partial) {
+            const size_t cols = (size_t)gridDim.x * 64;
+            *reinterpret_cast<float4*>(partial + ((size_t)blockIdx.z * M + m) * cols + (size_t)blockIdx.x * 64 + nl) = v;
+        } else if constexpr (CDT == LH_F32) {
+            *reinterpret_cast<float4*>(static_cast<float*>(C) + (size_t)m * N + n0 + nl) = v;
+        } else {
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(C) + (size_t)m * N + n0 + nl) = make_uint2(pack_h2(v.x, v.y), pack_h2(v.z, v.w));
+        }
+    }
+}
+
+// The skinny kernel when the shape allows it (f16 activations, 17 .. 64 rows, whole 128-row tiles, at least one unit of k
+// per wave, at most two workgroups per CU -- with more, the activations every workgroup re-reads outweigh what the
+// LDS-tiled kernel spends on staging); false leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
+// tiles (one split included) stay in the workspace for a consumer that sums them itself.
+struct SkinnyPartials { const float* partial; uint32_t splits, cols; };
+template <int FMT, int ADT>
+bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n, const ClipArgs& clip,
+                const GroupArgs& grp, SkinnyPartials* keep = nullptr) {
+    hipStream_t s = ctx->stream;
+    const int cus = ctx->cu_count;
+    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
+    const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
+    if constexpr (FMT != kF16W && ADT == LH_F16) {
+        static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
+        bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
+        for (uint32_t i = 0; i < grp.count; i++) whole = whole && grp.N[i] % BN == 0;
+        const uint32_t units = k / Skinny<FMT>::unit_k;
+        if (!no_skinny && !clip.enabled && m > (uint32_t)kMaxMultivecM && m <= 64 && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+            2 * tiles_n <= 2 * (uint32_t)cus) {
+            // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
+            const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
+            uint32_t splits = 1;
+            const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
+            if (keep && fit == 0) return false;
+            if (!no_splitk && blocks < (uint32_t)cus) {
+                const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)cus + blocks - 1) / blocks, fit);
+                for (uint32_t c = 1; c <= want && c <= per_wg; c++) if (per_wg % c == 0) splits = c;
+            }
+            float* partial = (splits > 1 || keep) ? static_cast<float*>(ctx->workspace) : nullptr;
+            const dim3 grid(blocks, 1, splits);
+            const uint16_t* X = static_cast<const uint16_t*>(A);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F32>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
+            else hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F16>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
+            if (keep) {
+                *keep = SkinnyPartials{partial, splits, blocks * 64};
+            } else if (splits > 1) {
+                const uint32_t rgrid = (uint32_t)(((size_t)m * tiles_n * BN + 255) / 256);
+                if (ct == LH_F32) hipLaunchKernelGGL((splitk_reduce_kernel<LH_F32>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+                else hipLaunchKernelGGL((splitk_reduce_kernel<LH_F16>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+            }
+            return true;
+        }
+    }
+    return false;
+}
+
 // The 64-row-tile kernel over `tiles_n` column tiles (one matrix, or the matrices of `grp` side by side).  Few output
 // tiles (a decode batch of some tens of rows): k is split so that every CU gets a workgroup, at least two k steps per
 // split, partial tiles within the lower half of the context workspace, summed by splitk_reduce_kernel.
@@ -625,6 +830,7 @@ void launch_tiles64(lh_context* ctx, const void* A, const uint8_t* W, void* C, l
     static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
     const uint32_t nk = (k + BK - 1) / BK;
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
+    if (try_skinny<FMT, ADT>(ctx, A, W, C, ct, m, k, n, clip, grp)) return;
     const uint64_t tiles64 = (uint64_t)tiles_n * ((m + 63) / 64);
     uint32_t splits = 1;
     if (!no_splitk && tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
@@ -651,6 +857,7 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
     hipStream_t s = ctx->stream;
     const int cus = ctx->cu_count;
     if (mfma) {
+        if (try_skinny<FMT, ADT>(ctx, A, W, C, ct, m, k, n, clip, GroupArgs{})) return LH_OK;
         static const int force_bm = [] { const char* e = getenv("LOCAL_HIP_PREFILL_BM"); return e ? atoi(e) : 0; }();
         // 128-row tiles reuse each dequantised weight tile twice as often; 64-row tiles when that would leave most CUs idle
         const uint64_t tiles128 = (uint64_t)((n + BN - 1) / BN) * ((m + 127) / 128);
@@ -761,6 +968,59 @@ int lh_matmul_nt_quant_typed_into(lh_batch* b, lh_quant fmt, const lh_buffer* in
     if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
     return matmul_dispatch(b, fmt == LH_Q4_0 ? "matmul_nt_q4_0" : "matmul_nt_tq2_0", fmt == LH_Q4_0 ? kQ4 : kTQ2, in, at, w, out, ct, m,
                            k, n, false);
+}
+int lh_matmul_nt_quant_norm_into(lh_batch* b, lh_quant fmt, const lh_buffer* in, const lh_buffer* w, uint32_t m, uint32_t k, uint32_t n,
+                                 const lh_buffer* norm_weight, const lh_buffer* residual, lh_buffer* out, float eps, int apply_scale,
+                                 float scale, const lh_buffer* norm2_weight, lh_buffer* out2) {
+    const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 + rms_norm" : "matmul_nt_tq2_0 + rms_norm";
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    if (k % blk != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: k %u not /%u", op, k, blk);
+    if (m == 0 || n == 0 || k == 0) return LH_OK;
+    if (!lh_norm_fused_supported(n)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: n %u must be a multiple of 8, at most 8192", op, n);
+    if ((norm2_weight == nullptr) != (out2 == nullptr)) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: the second norm needs both its weight and its output", op);
+    lh_context* ctx = b->ctx;
+    const size_t wbytes = fmt == LH_Q4_0 ? (size_t)n * (k / 32) * 18 : (size_t)n * (k / 256) * 66;
+    LH_NEED(in, (size_t)m * k * 2, op, "input");
+    LH_NEED(w, wbytes, op, "weight");
+    LH_NEED(norm_weight, (size_t)n * 2, op, "norm weight");
+    LH_NEED(out, (size_t)m * n * 2, op, "output");
+    if (residual) LH_NEED(residual, (size_t)m * n * 2, op, "residual");
+    if (norm2_weight) { LH_NEED(norm2_weight, (size_t)n * 2, op, "second norm weight"); LH_NEED(out2, (size_t)m * n * 2, op, "second output"); }
+    const uintptr_t align = (uintptr_t)in->ptr | (uintptr_t)norm_weight->ptr | (uintptr_t)out->ptr | (uintptr_t)(residual ? residual->ptr : nullptr) |
+                            (uintptr_t)(norm2_weight ? norm2_weight->ptr : nullptr) | (uintptr_t)(out2 ? out2->ptr : nullptr);
+    LH_REQUIRE((align & 15) == 0, "%s: buffers must be 16-byte aligned", op);
+    LH_REQUIRE(((uintptr_t)w->ptr & 1) == 0, "%s: weight must be 2-byte aligned", op);
+
+    LhNormFused a{};
+    a.w = (const uint16_t*)norm_weight->ptr; a.res = residual ? (const uint16_t*)residual->ptr : nullptr; a.out = (uint16_t*)out->ptr;
+    a.dim = n; a.rows = m; a.eps = eps; a.apply_scale = apply_scale ? 1u : 0u; a.scale = scale;
+    a.w2 = norm2_weight ? (const uint16_t*)norm2_weight->ptr : nullptr; a.out2 = out2 ? (uint16_t*)out2->ptr : nullptr;
+    const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
+    SkinnyPartials kept{nullptr, 0, 0};
+    const uint8_t* W = (const uint8_t*)w->ptr;
+    const bool skinny = fmt == LH_Q4_0 ? try_skinny<kQ4, LH_F16>(ctx, in->ptr, W, nullptr, LH_F16, m, k, n, none, GroupArgs{}, &kept)
+                                       : try_skinny<kTQ2, LH_F16>(ctx, in->ptr, W, nullptr, LH_F16, m, k, n, none, GroupArgs{}, &kept);
+    if (skinny) {
+        a.partial = kept.partial; a.splits = kept.splits; a.part_rows = m; a.part_cols = kept.cols;
+    } else {
+        // any other shape: the product as matmul_nt_quant_typed_into computes it, into the third quarter of the workspace
+        // (the lower half holds partial tiles, the top quarter descriptor tables), then the same norm kernel over those rows
+        const size_t half = ctx->workspace_bytes / 2, quarter = ctx->workspace_bytes / 4;
+        if ((size_t)m * n * 2 > quarter) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u x %u product exceeds the %zu-byte staging area", op, m, n, quarter);
+        lh_buffer tmp{};
+        tmp.ptr = static_cast<uint8_t*>(ctx->workspace) + half; tmp.len = quarter; tmp.ctx = ctx;
+        const uint32_t d0 = b->dispatch_count;
+        int r = matmul_dispatch(b, op, fmt == LH_Q4_0 ? kQ4 : kTQ2, in, LH_F16, w, &tmp, LH_F16, m, k, n, false);
+        if (r != LH_OK) return r;
+        b->dispatch_count = d0;
+        a.in = (const uint16_t*)tmp.ptr;
+    }
+    lh_launch_norm_fused(ctx->stream, a);
+    int r = lh_check_launch(op);
+    if (r == LH_OK) b->dispatch_count++;
+    return r;
 }
 int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* in, const lh_buffer* const* ws,
                                     lh_buffer* const* outs, const uint32_t* ns, uint32_t m, uint32_t k) {

@@ -375,24 +375,35 @@ class TransformerLayer:
         """Everything after attention, identical in layer.rs:640-716 and layer.rs:808-870."""
         p, w = self.params, self.weights
         h, eps, inter = p.hidden_size, p.rms_norm_eps, p.intermediate_size
-        w.attn_output.matmul_nt_into(batch, kernels, bs.attn_out, bs.ffn_out, rows)
-        kernels.rms_norm_add_into(batch, bs.ffn_out, w.attn_post_norm, input, bs.attn_resid, h, rows, eps)
-        kernels.rms_norm_into(batch, bs.attn_resid, w.ffn_norm, bs.normed, h, rows, eps)
+        has_ple = (w.per_layer_inp_gate is not None and w.per_layer_proj is not None
+                   and w.per_layer_post_norm is not None and ple_all is not None)
+
+        def product_norm(weight, x, norm_w, residual, out, scale=None, norm2_w=None, out2=None):
+            """matmul_nt -> rms_norm_add (-> output scale) (-> rms_norm): one fused step where the weight format has
+            one, the separate kernels otherwise (same result either way)."""
+            if self.fuse_norm_chain and weight.ty != W_F16 and h % 8 == 0 and h <= 8192:
+                kernels.matmul_nt_quant_norm_into(batch, weight.ty, x, weight.buf, rows, weight.cols, weight.rows, norm_w,
+                                                  residual, out, eps, scale, norm2_w, out2)
+                return
+            weight.matmul_nt_into(batch, kernels, x, bs.ffn_out, rows)
+            kernels.rms_norm_add_into(batch, bs.ffn_out, norm_w, residual, out, h, rows, eps)
+            if scale is not None:
+                kernels.scale_in_place_gpu_into(batch, out, scale, rows * h)
+            if norm2_w is not None:
+                kernels.rms_norm_into(batch, out, norm2_w, out2, h, rows, eps)
+
+        product_norm(w.attn_output, bs.attn_out, w.attn_post_norm, input, bs.attn_resid, None, w.ffn_norm, bs.normed)
         self._matmuls(batch, kernels, [w.ffn_gate, w.ffn_up], bs.normed, [bs.gate, bs.up], rows)
         kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
-        w.ffn_down.matmul_nt_into(batch, kernels, bs.gate, bs.ffn_out, rows)
-        kernels.rms_norm_add_into(batch, bs.ffn_out, w.ffn_post_norm, bs.attn_resid, output, h, rows, eps)
-        if (w.per_layer_inp_gate is not None and w.per_layer_proj is not None and w.per_layer_post_norm is not None
-                and ple_all is not None):
+        product_norm(w.ffn_down, bs.gate, w.ffn_post_norm, bs.attn_resid, output, None if has_ple else self._output_scale)
+        if has_ple:
             ple_buf, n_layer_total = ple_all
             pld = p.per_layer_dim
             kernels.gather_strided_f16_into(batch, ple_buf, bs.ple_slice, n_layer_total * pld, p.layer_idx * pld, pld,
                                             rows)
             w.per_layer_inp_gate.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
             kernels.gelu_mul_into(batch, bs.ple_g, bs.ple_slice, bs.ple_g, rows * pld)
-            w.per_layer_proj.matmul_nt_into(batch, kernels, bs.ple_g, bs.ffn_out, rows)
-            kernels.rms_norm_add_into(batch, bs.ffn_out, w.per_layer_post_norm, output, output, h, rows, eps)
-        self._scale_output(batch, kernels, output, rows * h)
+            product_norm(w.per_layer_proj, bs.ple_g, w.per_layer_post_norm, output, output, self._output_scale)
 
     def _check_rows(self, rows: int, bs: BatchScratch) -> None:
         if rows == 0 or rows > bs.max_batch:

@@ -67,6 +67,104 @@ def test_mfma_matmul_tile_boundaries(pkg, gpu, oracle, fmt):
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_decode_batch_matmul(pkg, gpu, oracle, fmt):
+    """17 .. 64 activation rows against whole 128-row tiles (a continuous-batching step): the kernel that feeds the
+    matrix cores straight from global memory -- one and many units of k per wave, with and without the k split, ragged
+    row counts, f16 and f32 outputs -- against the oracle's product with the CPU path's f16 weights; then one-hot rows,
+    which must return those weights bit for bit (subnormal and zero scales, TQ2 code 3 included)."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    kmin = 256 if fmt == "q4_0" else 512
+    shapes = ((64, kmin, 128, "f32"), (17, kmin, 1536, "f16"), (33, 1536, 256, "f16"), (48, 1536, 12288, "f16"),
+              (64, 6144, 1536, "f32"), (50, 3 * kmin, 4096, "f32"), (64, 1536, 32768, "f32"))
+    for (m, k, n, ct) in shapes:
+        print(f"case {fmt} m={m} k={k} n={n} out={ct}", flush=True)
+        raw = payload(fmt, n, k, 0x5C1 + m)
+        deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+        a16 = (pkg.synth.rng(4, m + k + n).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+        want = oracle.matmul_nt_f32(a16.astype(np.float32), deq)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, ty, n, k)
+        ab = pkg.Buffer.from_slice(ctx, a16)
+        guard = 64                                             # bytes behind the output stay untouched
+        cb = pkg.Buffer.from_slice(ctx, np.full(m * n * (4 if ct == "f32" else 2) + guard, 0xA5, np.uint8))
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32 if ct == "f32" else pkg.F16, m)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float32, m * n) if ct == "f32" else cb.as_array(np.float16, m * n).astype(np.float32)
+        refgen.assert_close(got, want, 1e-3 if ct == "f32" else 2e-3, f"{fmt} decode batch {m}x{k}x{n}")
+        assert (cb.as_array(np.uint8)[-guard:] == 0xA5).all()
+    for (m, k, n) in ((64, 2 * kmin, 256), (40, 6 * kmin, 128)):
+        raw = payload(fmt, n, k, 0x51DF).copy()
+        blk, doff = (18, 0) if fmt == "q4_0" else (66, 64)
+        raw.reshape(-1, blk)[3, doff:doff + 2] = np.array([6e-8], np.float16).view(np.uint8)
+        raw.reshape(-1, blk)[5, doff:doff + 2] = 0
+        deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).reshape(n, k)
+        cols = (np.arange(m) * 37 + 5) % k
+        a = np.zeros((m, k), np.float16)
+        a[np.arange(m), cols] = 1.0
+        w = pkg.QuantWeight.from_bytes(ctx, raw, ty, n, k)
+        ab, cb = pkg.Buffer.from_slice(ctx, a), pkg.Buffer.empty(ctx, m * n * 4)
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32, m)
+        batch.commit_and_wait()
+        assert np.array_equal(cb.as_array(np.float32).reshape(m, n), deq[:, cols].T.astype(np.float32)), (fmt, m, k, n)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_matmul_norm_fused_equals_separate_kernels(pkg, gpu, fmt):
+    """matmul_nt_quant_norm_into against the sequence it stands for -- matmul_nt, rms_norm(_add), scale_in_place, a second
+    rms_norm -- bit for bit: decode batches (the norm kernel sums the k-split partial tiles), rows served as matvecs and
+    prefill chunks (the product staged in the workspace); with and without residual, scale and second norm; the output
+    written over the residual."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    kq = 256 if fmt == "q4_0" else 512
+    cases = [(64, 2048, 1536, True, None, True), (33, 12 * kq, 1536, True, 0.37, False), (17, kq, 256, False, None, False),
+             (64, 1536, 2048, True, 1.7, True), (48, 1536, 8192, False, 0.5, True), (8, 1024, 1536, True, 0.9, True),
+             (200, 2048, 1536, True, None, True), (40, 1280, 200, True, 2.0, False)]
+    for (m, k, n, add, scale, second) in cases:
+        print(f"case {fmt} m={m} k={k} n={n} add={add} scale={scale} second={second}", flush=True)
+        g = pkg.synth.rng(77, m + k + n)
+        w = pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), ty, n, k)
+        x = pkg.Buffer.from_slice(ctx, (g.standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16))
+        nw = pkg.Buffer.from_slice(ctx, (1.0 + 0.1 * g.standard_normal(n, dtype=np.float32)).astype(np.float16))
+        nw2 = pkg.Buffer.from_slice(ctx, (1.0 + 0.1 * g.standard_normal(n, dtype=np.float32)).astype(np.float16))
+        res_host = g.standard_normal((m, n), dtype=np.float32).astype(np.float16)
+        eps = 1e-6
+        # the separate kernels
+        tmp, want, want2 = (pkg.Buffer.empty(ctx, m * n * 2) for _ in range(3))
+        res = pkg.Buffer.from_slice(ctx, res_host)
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_into(batch, K, x, tmp, m)
+        if add:
+            K.rms_norm_add_into(batch, tmp, nw, res, want, n, m, eps)
+        else:
+            K.rms_norm_into(batch, tmp, nw, want, n, m, eps)
+        if scale is not None:
+            K.scale_in_place_gpu_into(batch, want, scale, m * n)
+        if second:
+            K.rms_norm_into(batch, want, nw2, want2, n, m, eps)
+        batch.commit_and_wait()
+        # one step; the output lands on the residual when there is one
+        got = pkg.Buffer.from_slice(ctx, res_host) if add else pkg.Buffer.empty(ctx, m * n * 2)
+        got2 = pkg.Buffer.empty(ctx, m * n * 2)
+        batch = pkg.CommandBatch(ctx)
+        d0 = batch.dispatch_count()
+        K.matmul_nt_quant_norm_into(batch, ty, x, w.buf, m, k, n, nw, got if add else None, got, eps, scale,
+                                    nw2 if second else None, got2 if second else None)
+        assert batch.dispatch_count() == d0 + 1
+        batch.commit_and_wait()
+        assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16)), (fmt, m, k, n)
+        if second:
+            assert np.array_equal(got2.as_array(np.uint16), want2.as_array(np.uint16)), (fmt, m, k, n)
+    batch = pkg.CommandBatch(ctx)
+    with pytest.raises(pkg.InvalidArgument):
+        K.matmul_nt_quant_norm_into(batch, ty, x, w.buf, m, k, 12, nw, None, got, eps)               # n not a multiple of 8
+    with pytest.raises(pkg.InvalidArgument):
+        K.matmul_nt_quant_norm_into(batch, ty, x, w.buf, m, k, n, nw, None, got, eps, None, nw2, None)   # second norm without its output
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_split_k(pkg, gpu, oracle, fmt):
     """A decode batch of some tens of rows against the layer's projections: few output tiles, so the k range is split
     over several workgroups whose partial tiles a second kernel sums -- even and odd numbers of k steps per split, a
