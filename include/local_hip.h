@@ -294,6 +294,11 @@ LH_API int lh_scale_in_place_gpu_into(lh_batch* batch, lh_buffer* data, float sc
 /* kernels.rs:2801-2843 gather_strided_f16_into (scale_in_place.metal:21-35): dst[i*pld + p] = src[i*row_stride + base_off + p] */
 LH_API int lh_gather_strided_f16_into(lh_batch* batch, const lh_buffer* src, lh_buffer* dst, uint32_t row_stride,
                                       uint32_t base_off, uint32_t pld, uint32_t n_rows);
+/* gather_strided_f16_into followed by gelu_mul_into on the gathered rows (the per-layer-input gate of the multi-row
+ * layer paths, local-engine/src/layer.rs:690-700) as one dispatch without the gathered copy:
+ * out[r*dim + i] = half(gelu(a[r*dim + i]) * b[r*b_row_stride + b_offset + i]); out may be a. */
+LH_API int lh_gelu_mul_strided_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, uint32_t b_row_stride,
+                                    uint32_t b_offset, lh_buffer* out, uint32_t dim, uint32_t rows);
 /* kernels.rs:2749-2799 logit_softcap_gpu_into (scale_in_place.metal:39-49): f32 data[i] = cap * tanh(data[i] / cap) */
 LH_API int lh_logit_softcap_gpu_into(lh_batch* batch, lh_buffer* data, float cap, uint32_t count);
 

@@ -519,6 +519,11 @@ class Kernels:
         _check(self._l.lh_gather_strided_f16_into(batch._h, src._h, dst._h, _u32(row_stride), _u32(base_off), _u32(pld),
                                                   _u32(n_rows)))
 
+    def gelu_mul_strided_into(self, batch, a, b, b_row_stride, b_offset, out, dim, rows):
+        """gather_strided_f16 + gelu_mul in one dispatch: out[r, i] = gelu(a[r, i]) * b[r * b_row_stride + b_offset + i]."""
+        _check(self._l.lh_gelu_mul_strided_into(batch._h, a._h, b._h, _u32(b_row_stride), _u32(b_offset), out._h, _u32(dim),
+                                                _u32(rows)))
+
     def logit_softcap_gpu_into(self, batch, data, cap, count):
         _check(self._l.lh_logit_softcap_gpu_into(batch._h, data._h, C.c_float(cap), _u32(count)))
 

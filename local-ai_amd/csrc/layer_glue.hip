@@ -117,10 +117,21 @@ __global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a
         if (i >= dim) break;
         if constexpr (PART) {
             float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            for (uint32_t z = 0; z < a.splits; z++) {
-                const float* p = a.partial + ((size_t)z * a.part_rows + rowi) * a.part_cols + i;
-                const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
-                v[0] += lo.x; v[1] += lo.y; v[2] += lo.z; v[3] += lo.w; v[4] += hi.x; v[5] += hi.y; v[6] += hi.z; v[7] += hi.w;
+            const size_t zstride = (size_t)a.part_rows * a.part_cols;
+            const float* p0 = a.partial + (size_t)rowi * a.part_cols + i;
+            for (uint32_t z0 = 0; z0 < a.splits; z0 += 4) {      // four splits' loads in flight, added in split order
+                float4 lo[4], hi[4];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    const float* p = p0 + (size_t)(z0 + u < a.splits ? z0 + u : a.splits - 1) * zstride;
+                    lo[u] = *reinterpret_cast<const float4*>(p); hi[u] = *reinterpret_cast<const float4*>(p + 4);
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 4; u++) {
+                    if (z0 + u >= a.splits) break;
+                    v[0] += lo[u].x; v[1] += lo[u].y; v[2] += lo[u].z; v[3] += lo[u].w;
+                    v[4] += hi[u].x; v[5] += hi[u].y; v[6] += hi[u].z; v[7] += hi[u].w;
+                }
             }
             x[it] = make_uint4((uint32_t)lh_f2h(v[0]) | ((uint32_t)lh_f2h(v[1]) << 16), (uint32_t)lh_f2h(v[2]) | ((uint32_t)lh_f2h(v[3]) << 16),
                                (uint32_t)lh_f2h(v[4]) | ((uint32_t)lh_f2h(v[5]) << 16), (uint32_t)lh_f2h(v[6]) | ((uint32_t)lh_f2h(v[7]) << 16));
@@ -262,6 +273,30 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const uint16_t* a, con
         *reinterpret_cast<uint4*>(out + i) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
     } else {
         out[i] = elementwise_one<OP>(a[i], OP != kScale ? b[i] : a[i], scalar);
+    }
+}
+
+// gelu_mul whose second operand is read through gather_strided_f16's addressing (row r of `b` starts at
+// r * b_row_stride + b_off): out[r, i] = half(gelu(a[r, i]) * b[r * b_row_stride + b_off + i]) -- the slice gather and the
+// gate of the per-layer input (layer.rs:690-700) in one dispatch, without the gathered copy.
+template <int VEC>
+__global__ __launch_bounds__(256) void gelu_mul_strided_kernel(const uint16_t* a, const uint16_t* __restrict__ b, uint16_t* out, uint32_t dim,
+                                                              uint32_t rows, uint32_t b_row_stride, uint32_t b_off) {
+    const uint32_t per_row = dim / VEC, idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per_row * rows) return;
+    const uint32_t r = idx / per_row, i = (idx - r * per_row) * VEC;
+    const size_t ia = (size_t)r * dim + i, ib = (size_t)r * b_row_stride + b_off + i;
+    if constexpr (VEC == 8) {
+        const uint4 va = *reinterpret_cast<const uint4*>(a + ia), vb = *reinterpret_cast<const uint4*>(b + ib);
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+        uint32_t wo[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            wo[j] = (uint32_t)elementwise_one<kGeluMul>((uint16_t)(wa[j] & 0xFFFF), (uint16_t)(wb[j] & 0xFFFF), 0.0f) |
+                    ((uint32_t)elementwise_one<kGeluMul>((uint16_t)(wa[j] >> 16), (uint16_t)(wb[j] >> 16), 0.0f) << 16);
+        *reinterpret_cast<uint4*>(out + ia) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+    } else {
+        out[ia] = elementwise_one<kGeluMul>(a[ia], b[ib], 0.0f);
     }
 }
 
@@ -435,6 +470,23 @@ int lh_gelu_mul_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, lh
     LH_NEED(b, (size_t)count * 2, op, "b");
     LH_NEED(out, (size_t)count * 2, op, "out");
     launch_elementwise<kGeluMul>(batch->ctx->stream, a->ptr, b->ptr, out->ptr, 0.0f, count);
+    return finish(batch, op);
+}
+
+int lh_gelu_mul_strided_into(lh_batch* batch, const lh_buffer* a, const lh_buffer* b, uint32_t b_row_stride, uint32_t b_offset, lh_buffer* out,
+                             uint32_t dim, uint32_t rows) {
+    const char* op = "gelu_mul_strided";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (dim == 0 || rows == 0) return LH_OK;
+    LH_NEED(a, (size_t)rows * dim * 2, op, "a");
+    LH_NEED(b, ((size_t)(rows - 1) * b_row_stride + b_offset + dim) * 2, op, "b");
+    LH_NEED(out, (size_t)rows * dim * 2, op, "out");
+    const bool vec = ((dim | b_row_stride | b_offset) & 7) == 0 && (((uintptr_t)a->ptr | (uintptr_t)b->ptr | (uintptr_t)out->ptr) & 15) == 0;
+    const uint32_t items = rows * (dim / (vec ? 8 : 1));
+    if (vec) hipLaunchKernelGGL(gelu_mul_strided_kernel<8>, dim3((items + 255) / 256), dim3(256), 0, batch->ctx->stream, (const uint16_t*)a->ptr,
+                                (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset);
+    else hipLaunchKernelGGL(gelu_mul_strided_kernel<1>, dim3((items + 255) / 256), dim3(256), 0, batch->ctx->stream, (const uint16_t*)a->ptr,
+                            (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset);
     return finish(batch, op);
 }
 

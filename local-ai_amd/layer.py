@@ -371,8 +371,10 @@ class TransformerLayer:
 
     # ------------------------------------------------ shared multi-row tail
     def _attention_tail(self, kernels: Kernels, batch, rows: int, input: Buffer, output: Buffer, bs: BatchScratch,
-                        ple_all) -> None:
-        """Everything after attention, identical in layer.rs:640-716 and layer.rs:808-870."""
+                        ple_all, next_norm: Optional[Buffer] = None) -> None:
+        """Everything after attention, identical in layer.rs:640-716 and layer.rs:808-870.  With ``next_norm`` (the next
+        layer's attention-norm weight) the last step also leaves rms_norm(output, next_norm) in ``bs.normed``, which is
+        that layer's first dispatch."""
         p, w = self.params, self.weights
         h, eps, inter = p.hidden_size, p.rms_norm_eps, p.intermediate_size
         has_ple = (w.per_layer_inp_gate is not None and w.per_layer_proj is not None
@@ -395,15 +397,24 @@ class TransformerLayer:
         product_norm(w.attn_output, bs.attn_out, w.attn_post_norm, input, bs.attn_resid, None, w.ffn_norm, bs.normed)
         self._matmuls(batch, kernels, [w.ffn_gate, w.ffn_up], bs.normed, [bs.gate, bs.up], rows)
         kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
-        product_norm(w.ffn_down, bs.gate, w.ffn_post_norm, bs.attn_resid, output, None if has_ple else self._output_scale)
+        if has_ple:
+            product_norm(w.ffn_down, bs.gate, w.ffn_post_norm, bs.attn_resid, output)
+        else:
+            product_norm(w.ffn_down, bs.gate, w.ffn_post_norm, bs.attn_resid, output, self._output_scale, next_norm,
+                         bs.normed if next_norm is not None else None)
         if has_ple:
             ple_buf, n_layer_total = ple_all
             pld = p.per_layer_dim
-            kernels.gather_strided_f16_into(batch, ple_buf, bs.ple_slice, n_layer_total * pld, p.layer_idx * pld, pld,
-                                            rows)
             w.per_layer_inp_gate.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
-            kernels.gelu_mul_into(batch, bs.ple_g, bs.ple_slice, bs.ple_g, rows * pld)
-            product_norm(w.per_layer_proj, bs.ple_g, w.per_layer_post_norm, output, output, self._output_scale)
+            if self.fuse_norm_chain:   # this layer's slice of every row's per-layer inputs is read in place
+                kernels.gelu_mul_strided_into(batch, bs.ple_g, ple_buf, n_layer_total * pld, p.layer_idx * pld, bs.ple_g, pld,
+                                              rows)
+            else:
+                kernels.gather_strided_f16_into(batch, ple_buf, bs.ple_slice, n_layer_total * pld, p.layer_idx * pld, pld,
+                                                rows)
+                kernels.gelu_mul_into(batch, bs.ple_g, bs.ple_slice, bs.ple_g, rows * pld)
+            product_norm(w.per_layer_proj, bs.ple_g, w.per_layer_post_norm, output, output, self._output_scale,
+                         next_norm, bs.normed if next_norm is not None else None)
 
     def _check_rows(self, rows: int, bs: BatchScratch) -> None:
         if rows == 0 or rows > bs.max_batch:
@@ -411,9 +422,12 @@ class TransformerLayer:
 
     # -------------------------------------- n consecutive rows of one sequence
     def forward_batch(self, kernels: Kernels, batch, n_rows: int, start_pos: int, input: Buffer, output: Buffer,
-                      bs: BatchScratch, ones: Buffer, kv_cache: QuantizedKvCache, ple_all=None) -> None:
+                      bs: BatchScratch, ones: Buffer, kv_cache: QuantizedKvCache, ple_all=None, prenormed: bool = False,
+                      next_norm: Optional[Buffer] = None) -> None:
         """layer.rs:542-718: rows at positions ``start_pos .. start_pos + n_rows``; ``ple_all`` is
-        ``(buffer [n_rows, n_layer_total, per_layer_dim] f16, n_layer_total)``."""
+        ``(buffer [n_rows, n_layer_total, per_layer_dim] f16, n_layer_total)``.  ``prenormed``: ``bs.normed`` already
+        holds this layer's attention norm of ``input`` (the previous layer was given this layer's norm weight as its
+        ``next_norm``)."""
         self._check_rows(n_rows, bs)
         p, w = self.params, self.weights
         rows, h, hd, n_head, n_kv, eps = n_rows, p.hidden_size, p.head_dim, p.num_attention_heads, \
@@ -422,7 +436,8 @@ class TransformerLayer:
 
         own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
         one_prepare = self._one_prepare()
-        kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        if not prenormed:
+            kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
         if own_kv:
             self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
         else:
@@ -445,14 +460,14 @@ class TransformerLayer:
                 kv_cache.write_kv_gpu_into(batch, kernels, bs.k, bs.v, start_pos, n_rows)
             kv_cache.fused_attention_batch_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
                                                 n_head, p.sliding_window)
-        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)
+        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all, next_norm)
 
     # ---------------------------- one row per independent lane (continuous batching)
     def forward_decode_batch_turbo(self, batch, kernels: Kernels, n_lanes: int, positions: Buffer, input: Buffer,
                                    output: Buffer, bs: BatchScratch, ones: Buffer, pool: QuantizedUnifiedKvPool,
-                                   ple_all=None) -> None:
+                                   ple_all=None, prenormed: bool = False, next_norm: Optional[Buffer] = None) -> None:
         """layer.rs:731-873: ``positions`` is a device ``[n_lanes]`` u32 buffer shared by rope, the KV scatter
-        and attention."""
+        and attention; ``prenormed`` / ``next_norm`` as in ``forward_batch``."""
         self._check_rows(n_lanes, bs)
         p, w = self.params, self.weights
         rows, h, hd, n_head, n_kv, eps = n_lanes, p.hidden_size, p.head_dim, p.num_attention_heads, \
@@ -460,7 +475,8 @@ class TransformerLayer:
 
         own_kv = not p.is_kv_shared and w.attn_k is not None and w.attn_v is not None
         one_prepare = self._one_prepare()
-        kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        if not prenormed:
+            kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
         if own_kv:
             self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
         else:
@@ -485,4 +501,4 @@ class TransformerLayer:
                 pool.write_kv_into(batch, kernels, bs.k, bs.v, positions, n_lanes)
             pool.attention_into(batch, kernels, bs.q, bs.rq, bs.vacc, bs.attn_out, positions, n_head, p.sliding_window,
                                 n_lanes)
-        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all)
+        self._attention_tail(kernels, batch, rows, input, output, bs, ple_all, next_norm)

@@ -292,6 +292,13 @@ class DecodePipeline:
 
     # ---- multi-row paths: prefill chunks and continuous batching ---------------------------------------------------
 
+    def _next_norm(self, i: int) -> Optional[Buffer]:
+        """Layer i + 1's attention-norm weight when layer i can apply it in its last dispatch (the norm is then layer
+        i + 1's first step, layer.rs:556 / 745, moved across the layer boundary); None for the last layer."""
+        if i + 1 < len(self.layers) and self.layers[i].fuse_norm_chain and self.layers[i + 1].fuse_norm_chain:
+            return self.layers[i + 1].weights.attn_norm
+        return None
+
     def _embed_rows(self, batch, tokens, ple_tokens) -> bool:
         """pipeline.rs:994-1060 / batched.rs:305-368: rows of the embedding table scaled by sqrt(hidden) into hidden_a,
         and the per-layer inputs of every row into ple_all.  Returns whether per-layer inputs exist."""
@@ -327,12 +334,13 @@ class DecodePipeline:
         batch = batch or CommandBatch(self.ctx)
         bs = self.batch_scratch
         ple_arg = (bs.ple_all, self.config.num_hidden_layers) if self._embed_rows(batch, tokens, ple_tokens) else None
-        cur_in_a = True
+        cur_in_a, prenormed = True, False
         for i, layer in enumerate(self.layers):
             inp, out = (bs.hidden_a, bs.hidden_b) if cur_in_a else (bs.hidden_b, bs.hidden_a)
+            next_norm = self._next_norm(i)
             layer.forward_batch(self.kernels, batch, n, start_pos, inp, out, bs, self.scratch.ones,
-                                self.kv_caches[self.kv_index_map[i]], ple_arg)
-            cur_in_a = not cur_in_a
+                                self.kv_caches[self.kv_index_map[i]], ple_arg, prenormed, next_norm)
+            cur_in_a, prenormed = not cur_in_a, next_norm is not None
         if own:
             batch.commit_and_wait()
         return cur_in_a
@@ -395,12 +403,13 @@ class DecodePipeline:
         cfg, K, bs = self.config, self.kernels, self.batch_scratch
         h = cfg.hidden_size
         ple_arg = (bs.ple_all, cfg.num_hidden_layers) if self.per_layer_input is not None else None
-        cur_in_a = True
+        cur_in_a, prenormed = True, False
         for i, layer in enumerate(self.layers):
             inp, out = (bs.hidden_a, bs.hidden_b) if cur_in_a else (bs.hidden_b, bs.hidden_a)
+            next_norm = self._next_norm(i)
             layer.forward_decode_batch_turbo(batch, K, n, state.pos_buf, inp, out, bs, self.scratch.ones,
-                                             state.pools[self.kv_index_map[i]], ple_arg)
-            cur_in_a = not cur_in_a
+                                             state.pools[self.kv_index_map[i]], ple_arg, prenormed, next_norm)
+            cur_in_a, prenormed = not cur_in_a, next_norm is not None
         final_hidden = bs.hidden_a if cur_in_a else bs.hidden_b
         K.rms_norm_into(batch, final_hidden, self.output_norm, bs.normed, h, n, cfg.rms_norm_eps)
         self.token_embd.matmul_nt_typed_into(batch, K, bs.normed, F16, state.logits_buf, F32, n)

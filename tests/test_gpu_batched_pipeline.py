@@ -27,12 +27,12 @@ def _config(pkg, pld=64):
                                         full_partial_rotary_factor=0.25)
 
 
-def _pipe(pkg, gpu, pld=64, seed=0, max_batch=8, max_ctx=1024):
+def _pipe(pkg, gpu, pld=64, seed=0, max_batch=8, max_ctx=1024, **layer_options):
     ctx, K = gpu
     cfg = _config(pkg, pld)
     g = pkg.synth.rng(981, seed)
     t = pkg.synth.decode_model_tensors(cfg, g, [512, 512, 512, 1024, 1024, 1024])
-    pipe = pkg.pipeline.DecodePipeline.from_host(ctx, K, cfg, t, max_ctx, max_batch=max_batch)
+    pipe = pkg.pipeline.DecodePipeline.from_host(ctx, K, cfg, t, max_ctx, max_batch=max_batch, **layer_options)
     return cfg, g, pipe, OL.model_from_host(cfg, t)
 
 
@@ -121,6 +121,28 @@ def test_batched_step_matches_single_sequence_at_pos0(pkg, gpu):
     rev = pipe.decode_batch_step(state, tokens[::-1], tokens[::-1], zeros)
     for lane in range(4):                          # results follow the token, not the lane index
         assert np.array_equal(rev[lane], got[3 - lane])
+
+
+@pytest.mark.parametrize("pld,lanes", [(64, 40), (0, 24), (64, 5)])
+def test_fused_tail_equals_separate_kernels(pkg, gpu, pld, lanes):
+    """The fused steps of the multi-row layer tail (product + norm + residual (+ scale) (+ the next layer's attention
+    norm), the per-layer-input gate read in place) against the reference's kernel-by-kernel sequence: the same logits bit
+    for bit, for a prefilled lane and for batched steps -- a decode batch whose products take the direct-to-MFMA kernel
+    and one small enough to run as matvecs."""
+    runs = []
+    for fused in (True, False):
+        cfg, g, pipe, _ = _pipe(pkg, gpu, pld, seed=11, max_batch=64, fuse_norm_chain=fused)
+        state = pipe.new_batched_decode_state(lanes, 1024)
+        out = [pipe.prefill_lane(state, 1, [int(v) for v in g.integers(0, cfg.vocab_size, 19)])]
+        positions = [0] * lanes
+        positions[1] = 19
+        for _ in range(3):
+            tokens = [int(v) for v in g.integers(0, cfg.vocab_size, lanes)]
+            out.append(pipe.decode_batch_step(state, tokens, tokens, positions))
+            positions = [p + 1 for p in positions]
+        runs.append(out)
+    for a, b in zip(*runs):
+        assert np.array_equal(a, b)
 
 
 def test_batched_step_arguments(pkg, gpu):

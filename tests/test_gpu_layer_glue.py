@@ -172,3 +172,24 @@ def test_rms_norm_residual_scale_equals_the_three_kernels(pkg, gpu, dim, rows, s
     batch.commit_and_wait()
     assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16))
     assert np.array_equal(rb.as_array(np.uint16), want.as_array(np.uint16))
+
+
+def test_gelu_mul_strided_equals_gather_then_gelu_mul(pkg, gpu):
+    """gelu_mul_strided_into against gather_strided_f16_into + gelu_mul_into, bit for bit, on the vector and scalar paths."""
+    ctx, K = gpu
+    g = pkg.synth.rng(44, 1)
+    for rows, dim, stride, off in ((64, 256, 35 * 256, 7 * 256), (5, 24, 100, 3), (1, 256, 256, 0), (33, 40, 48, 8)):
+        a_host = (g.standard_normal((rows, dim), dtype=np.float32) * 2).astype(np.float16)
+        b_host = g.standard_normal(rows * stride + dim, dtype=np.float32).astype(np.float16)
+        a, b = pkg.Buffer.from_slice(ctx, a_host), pkg.Buffer.from_slice(ctx, b_host)
+        sl, want, got = (pkg.Buffer.empty(ctx, rows * dim * 2) for _ in range(3))
+        batch = pkg.CommandBatch(ctx)
+        K.gather_strided_f16_into(batch, b, sl, stride, off, dim, rows)
+        K.gelu_mul_into(batch, a, sl, want, rows * dim)
+        K.gelu_mul_strided_into(batch, a, b, stride, off, got, dim, rows)
+        K.gelu_mul_strided_into(batch, a, b, stride, off, a, dim, rows)          # in place
+        batch.commit_and_wait()
+        assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16)), (rows, dim, stride, off)
+        assert np.array_equal(a.as_array(np.uint16), want.as_array(np.uint16))
+    with pytest.raises(pkg.InvalidArgument):
+        K.gelu_mul_strided_into(pkg.CommandBatch(ctx), a, b, stride, off + 64, got, dim, rows)     # last row past the end of b

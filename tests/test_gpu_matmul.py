@@ -93,7 +93,7 @@ def test_decode_batch_matmul(pkg, gpu, oracle, fmt):
         got = cb.as_array(np.float32, m * n) if ct == "f32" else cb.as_array(np.float16, m * n).astype(np.float32)
         refgen.assert_close(got, want, 1e-3 if ct == "f32" else 2e-3, f"{fmt} decode batch {m}x{k}x{n}")
         assert (cb.as_array(np.uint8)[-guard:] == 0xA5).all()
-    for (m, k, n) in ((64, 2 * kmin, 256), (40, 6 * kmin, 128)):
+    for (m, k, n) in ((64, 2 * kmin, 256), (40, 6 * kmin, 128), (64, 2 * kmin, 12288)):   # the last: whole 128-row tiles per workgroup
         raw = payload(fmt, n, k, 0x51DF).copy()
         blk, doff = (18, 0) if fmt == "q4_0" else (66, 64)
         raw.reshape(-1, blk)[3, doff:doff + 2] = np.array([6e-8], np.float16).view(np.uint8)
