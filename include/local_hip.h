@@ -202,6 +202,13 @@ LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, co
 LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, lh_dtype input_dtype,
                                          const lh_buffer* weight, lh_buffer* output, lh_dtype output_dtype,
                                          uint32_t m, uint32_t k, uint32_t n);
+/* The feed-forward gate and up projections and their gelu_mul as one encoded step:
+ * out[m, n] = half(gelu(half(in . w_gate^T)) * half(in . w_up^T)) -- matmul_nt_into twice and gelu_mul_into of the
+ * multi-row layer paths (local-engine/src/layer.rs:652-662), with their roundings, so the result is theirs bit for
+ * bit.  For a decode batch (17 .. 64 rows) whose pair fills the chip without a k split this is a single kernel that
+ * pairs gate and up rows in one workgroup; other shapes run the grouped product into the workspace and gelu_mul. */
+LH_API int lh_matmul_nt_quant_gelu_mul_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* w_gate,
+                                            const lh_buffer* w_up, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
 /* A product followed by the row-wise norm that consumes it, as one encoded step: out = rms_norm(in[m, k] . w^T,
  * norm_weight) (+ residual) (* scale), and with norm2_weight also out2 = rms_norm(out, norm2_weight).  This is the
  * sequence matmul_nt_into -> rms_norm_add_into (-> scale_in_place_gpu_into) (-> rms_norm_into) of the multi-row layer

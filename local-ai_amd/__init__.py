@@ -418,6 +418,11 @@ class Kernels:
                                                        _handles(outputs), (C.c_uint32 * n)(*[int(v) for v in ns]),
                                                        _u32(m), _u32(k)))
 
+    def matmul_nt_quant_gelu_mul_into(self, batch, fmt, input, w_gate, w_up, output, m, k, n):
+        """output[m, n] = gelu(input . w_gate^T) * (input . w_up^T): the two feed-forward products and gelu_mul as one step."""
+        _check(self._l.lh_matmul_nt_quant_gelu_mul_into(batch._h, C.c_int(fmt), input._h, w_gate._h, w_up._h, output._h,
+                                                        _u32(m), _u32(k), _u32(n)))
+
     def matmul_nt_quant_norm_into(self, batch, fmt, input, weight, m, k, n, norm_weight, residual, output, eps, scale=None,
                                   norm2_weight=None, output2=None):
         """matmul_nt -> rms_norm(_add) (-> scale_in_place) (-> rms_norm) of the multi-row layer paths as one step, bit for

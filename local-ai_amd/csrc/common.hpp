@@ -113,6 +113,7 @@ struct LhNormFused {
     uint16_t* out2;
 };
 bool lh_norm_fused_supported(uint32_t dim);
+void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count);   // gelu_mul_into's kernel
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
 
 static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }

@@ -251,7 +251,7 @@ enum { kGeluMul = 0, kResidualAdd = 1, kScale = 2 };
 // scale_in_place.metal:5-14 (out = half(float(a) * scalar), a may be out)
 template <int OP>
 __device__ __forceinline__ uint16_t elementwise_one(uint16_t a, uint16_t b, float scalar) {
-    if constexpr (OP == kGeluMul) return lh_f2h(lh_gelu_tanh_f32(lh_h2f(a)) * lh_h2f(b));
+    if constexpr (OP == kGeluMul) return lh_gelu_mul_h(a, b);
     else if constexpr (OP == kResidualAdd) return __builtin_bit_cast(uint16_t, (_Float16)(__builtin_bit_cast(_Float16, a) + __builtin_bit_cast(_Float16, b)));
     else return lh_f2h(lh_h2f(a) * scalar);
 }
@@ -334,6 +334,10 @@ int finish(lh_batch* batch, const char* op) {
 }  // namespace
 
 bool lh_norm_fused_supported(uint32_t dim) { return (dim & 7) == 0 && dim <= 8192; }
+
+void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count) {
+    launch_elementwise<kGeluMul>(stream, a, b, out, 0.0f, count);
+}
 
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a) {
     // the thread count launch_rms_norm picks for 16-byte accesses: the partial sums of the squares add up in the same order

@@ -13,6 +13,7 @@
 //    d*(q-1) is exact in f16 -- and staged in LDS next to the activation tile
 //    (converted to f16), then v_mfma_f32_16x16x32_f16 with fp32 accumulate.
 #include "common.hpp"
+#include "xquant.hpp"
 #include <cstdlib>
 
 namespace {
@@ -659,7 +660,10 @@ __device__ __forceinline__ f16x8 skinny_fragment(const SkinnyRaw& raw, int f) {
     return __builtin_bit_cast(f16x8, t);
 }
 
-template <int FMT, int CDT>
+// PAIR: the feed-forward gate and up projections with their gelu_mul (layer.rs:652-662).  The workgroup's tiles 0, 1 are 32
+// rows of grp.W[0] (gate), tiles 2, 3 the same 32 rows of grp.W[1] (up), so that both factors of an output meet in the
+// reduction: out = half(gelu(half(gate)) * half(up)), the values the two products and gelu_mul would have stored.
+template <int FMT, int CDT, bool PAIR = false>
 __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W_one, void* __restrict__ C_one,
                                                               uint32_t M, uint32_t K, uint32_t N_one, float* __restrict__ partial,
                                                               uint32_t units_per_wave, GroupArgs grp) {
@@ -668,12 +672,12 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     const uint8_t* __restrict__ W = W_one;
     void* __restrict__ C = C_one;
     uint32_t N = N_one, tile = blockIdx.x >> 1;               // blockIdx.x counts 64-row halves of the 128-row tile grid
-    if (grp.count) {
+    if (!PAIR && grp.count) {
         const uint32_t gi = group_of_tile(grp, tile);
         W = grp.W[gi]; C = grp.C[gi]; N = grp.N[gi];
         tile -= grp.tile0[gi];
     }
-    const uint32_t n0 = tile * BN + (blockIdx.x & 1) * 64;
+    const uint32_t n0 = PAIR ? blockIdx.x * 32 : tile * BN + (blockIdx.x & 1) * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t r = lane & 15, g = lane >> 4;
     const size_t row_bytes = FMT == kQ4 ? (size_t)(K >> 5) * 18 : (size_t)(K >> 8) * 66;
@@ -681,6 +685,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
 
     const uint8_t* wrow = W + (size_t)(n0 + r) * row_bytes;   // tile t starts 16 rows further on
     const size_t tile_bytes = 16 * row_bytes;
+    const uint8_t* wrow_up = PAIR ? grp.W[1] + (size_t)(n0 + r) * row_bytes : nullptr;
     const uint16_t* xrow[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -694,7 +699,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
         else { const size_t b = k0 >> 8; doff = b * 66 + 64; off = b * 66 + 32 * ((k0 >> 7) & 1) + 8 * g; }
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const uint8_t* p = wrow + t * tile_bytes;
+            const uint8_t* p = PAIR ? (t < 2 ? wrow : wrow_up) + (t & 1) * tile_bytes : wrow + t * tile_bytes;
             const uint2 w = ld8_align2(p + off);
             const uint32_t d = *reinterpret_cast<const uint16_t*>(p + doff);
             raw[t].w0 = w.x; raw[t].w1 = w.y; raw[t].d = d | (d << 16);
@@ -750,6 +755,30 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
 #pragma unroll
         for (int j = 0; j < 4; j++) red[wave][t][j][lane] = make_float4(acc[t][j][0], acc[t][j][1], acc[t][j][2], acc[t][j][3]);
     __syncthreads();
+    if constexpr (PAIR) {
+        // wave w finishes gate tile (w & 1) with up tile (w & 1) + 2 for the activation groups 2 (w >> 1), 2 (w >> 1) + 1
+        const int tp = wave & 1;
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+            const int j = (wave >> 1) * 2 + jj;
+            float4 gt = red[0][tp][j][lane], up = red[0][tp + 2][j][lane];
+#pragma unroll
+            for (int w = 1; w < 4; w++) {
+                const float4 a = red[w][tp][j][lane], b = red[w][tp + 2][j][lane];
+                gt.x += a.x; gt.y += a.y; gt.z += a.z; gt.w += a.w;
+                up.x += b.x; up.y += b.y; up.z += b.z; up.w += b.w;
+            }
+            const uint32_t m = 16 * j + r;
+            if (m >= M) continue;
+            const float gv[4] = {gt.x, gt.y, gt.z, gt.w}, uv[4] = {up.x, up.y, up.z, up.w};
+            uint16_t h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) h[i] = lh_gelu_mul_h(lh_f2h(gv[i]), lh_f2h(uv[i]));
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(grp.C[0]) + (size_t)m * grp.N[0] + n0 + 16 * tp + 4 * g) =
+                make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+        }
+        return;
+    }
     // wave w finishes tile w: D[row 4g + i][activation row r] of each group j
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -773,6 +802,19 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     }
 }
 
+// k splits of the skinny kernel over `blocks` 64-row workgroups: enough workgroups for every CU, a whole number of units
+// per wave, partial tiles within half the workspace.
+uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t blocks, uint32_t units_per_wg) {
+    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
+    uint32_t splits = 1;
+    if (!no_splitk && blocks < (uint32_t)ctx->cu_count) {
+        const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
+        const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)ctx->cu_count + blocks - 1) / blocks, fit);
+        for (uint32_t c = 1; c <= want && c <= units_per_wg; c++) if (units_per_wg % c == 0) splits = c;
+    }
+    return splits;
+}
+
 // The skinny kernel when the shape allows it (f16 activations, 17 .. 64 rows, whole 128-row tiles, at least one unit of k
 // per wave, at most two workgroups per CU -- with more, the activations every workgroup re-reads outweigh what the
 // LDS-tiled kernel spends on staging); false leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
@@ -783,7 +825,6 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
                 const GroupArgs& grp, SkinnyPartials* keep = nullptr) {
     hipStream_t s = ctx->stream;
     const int cus = ctx->cu_count;
-    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
     if constexpr (FMT != kF16W && ADT == LH_F16) {
         static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
@@ -794,13 +835,9 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
             2 * tiles_n <= 2 * (uint32_t)cus) {
             // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
-            uint32_t splits = 1;
             const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
             if (keep && fit == 0) return false;
-            if (!no_splitk && blocks < (uint32_t)cus) {
-                const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)cus + blocks - 1) / blocks, fit);
-                for (uint32_t c = 1; c <= want && c <= per_wg; c++) if (per_wg % c == 0) splits = c;
-            }
+            const uint32_t splits = skinny_splits(ctx, m, blocks, per_wg);
             float* partial = (splits > 1 || keep) ? static_cast<float*>(ctx->workspace) : nullptr;
             const dim3 grid(blocks, 1, splits);
             const uint16_t* X = static_cast<const uint16_t*>(A);
@@ -1066,6 +1103,59 @@ int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, c
     const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
     if (fmt == LH_Q4_0) launch_tiles64<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
     else launch_tiles64<kTQ2, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
+    int r = lh_check_launch(op);
+    if (r == LH_OK) b->dispatch_count++;
+    return r;
+}
+
+int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer* in, const lh_buffer* w_gate, const lh_buffer* w_up,
+                                     lh_buffer* out, uint32_t m, uint32_t k, uint32_t n) {
+    const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 + gelu_mul" : "matmul_nt_tq2_0 + gelu_mul";
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    if (k % blk != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: k %u not /%u", op, k, blk);
+    if (m == 0 || n == 0 || k == 0) return LH_OK;
+    lh_context* ctx = b->ctx;
+    const size_t wbytes = fmt == LH_Q4_0 ? (size_t)n * (k / 32) * 18 : (size_t)n * (k / 256) * 66;
+    LH_NEED(in, (size_t)m * k * 2, op, "input");
+    LH_NEED(w_gate, wbytes, op, "gate weight");
+    LH_NEED(w_up, wbytes, op, "up weight");
+    LH_NEED(out, (size_t)m * n * 2, op, "output");
+    LH_REQUIRE(((uintptr_t)in->ptr & 15) == 0 && ((uintptr_t)out->ptr & 15) == 0, "%s: input and output must be 16-byte aligned", op);
+    LH_REQUIRE((((uintptr_t)w_gate->ptr | (uintptr_t)w_up->ptr) & 1) == 0, "%s: weights must be 2-byte aligned", op);
+    static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
+    const uint32_t unit_k = fmt == LH_Q4_0 ? Skinny<kQ4>::unit_k : Skinny<kTQ2>::unit_k;
+    const uint32_t blocks = n / 32;
+    // one launch where the grouped product of the pair takes the skinny kernel without a k split (split products need
+    // their sums before the gelu); the same workgroup count and k ranges, hence the same sums
+    if (!no_skinny && m > (uint32_t)kMaxMultivecM && m <= 64 && n % BN == 0 && k % (4 * unit_k) == 0 &&
+        blocks <= 2 * (uint32_t)ctx->cu_count && skinny_splits(ctx, m, blocks, k / unit_k / 4) == 1) {
+        GroupArgs grp{};
+        grp.count = 2;
+        grp.W[0] = (const uint8_t*)w_gate->ptr; grp.W[1] = (const uint8_t*)w_up->ptr;
+        grp.C[0] = out->ptr; grp.N[0] = n;
+        const uint16_t* X = static_cast<const uint16_t*>(in->ptr);
+        const uint32_t per_wave = k / unit_k / 4;
+        if (fmt == LH_Q4_0) hipLaunchKernelGGL((matmul_skinny_kernel<kQ4, LH_F16, true>), dim3(blocks), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
+        else hipLaunchKernelGGL((matmul_skinny_kernel<kTQ2, LH_F16, true>), dim3(blocks), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
+    } else {
+        // any other shape: the two products as matmul_nt_quant_grouped_into computes them, staged in the third quarter of the
+        // workspace, then gelu_mul
+        const size_t half = ctx->workspace_bytes / 2, quarter = ctx->workspace_bytes / 4, each = (((size_t)m * n * 2) + 255) & ~(size_t)255;
+        if (2 * each > quarter) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: two %u x %u products exceed the %zu-byte staging area", op, m, n, quarter);
+        lh_buffer tg{}, tu{};
+        tg.ptr = static_cast<uint8_t*>(ctx->workspace) + half; tg.len = each; tg.ctx = ctx;
+        tu.ptr = static_cast<uint8_t*>(ctx->workspace) + half + each; tu.len = each; tu.ctx = ctx;
+        const lh_buffer* ws[2] = {w_gate, w_up};
+        lh_buffer* outs[2] = {&tg, &tu};
+        const uint32_t ns[2] = {n, n};
+        const uint32_t d0 = b->dispatch_count;
+        int r = lh_matmul_nt_quant_grouped_into(b, fmt, 2, in, ws, outs, ns, m, k);
+        if (r != LH_OK) return r;
+        b->dispatch_count = d0;
+        lh_launch_gelu_mul(ctx->stream, tg.ptr, tu.ptr, out->ptr, m * n);
+    }
     int r = lh_check_launch(op);
     if (r == LH_OK) b->dispatch_count++;
     return r;

@@ -14,10 +14,22 @@ template <> struct Limb<3> { static constexpr float qmax = 8355711.0f; };   // 1
 // routine's several dozen; |u| <= 10 keeps e^(2u) finite): its absolute error of about 1e-7 disappears in 1 + tanh(u),
 // far below the f16 result's rounding step.
 __device__ __forceinline__ float lh_gelu_tanh_f32(float x) {
+    // the two multiply-adds are written as fused operations and nothing else here is a product feeding a sum, so the
+    // compiler's contraction has no choice left to make: the kernels that evaluate this (gelu_mul, the matvec
+    // prologue, the product epilogue) agree bit for bit whatever code surrounds the call
     const float x3 = x * x * x;
-    const float inner = fminf(fmaxf(0.7978845608f * (x + 0.044715f * x3), -10.0f), 10.0f);
-    const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * inner));
+    const float inner = fminf(fmaxf(0.7978845608f * __builtin_fmaf(0.044715f, x3, x), -10.0f), 10.0f);
+    const float t = __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * inner)), 1.0f);
     return 0.5f * x * (1.0f + t);
+}
+
+// gelu.metal:37-40: half(gelu(float(a)) * float(b)).  The f32 product passes through an empty asm statement so that it is
+// rounded to f32 before it is narrowed (left alone the compiler sometimes narrows the exact product in one mixed-
+// precision instruction, sometimes not, and two kernels then disagree in the last bit once in ten thousand values).
+__device__ __forceinline__ uint16_t lh_gelu_mul_h(uint16_t a, uint16_t b) {
+    float p = lh_gelu_tanh_f32(lh_h2f(a)) * lh_h2f(b);
+    asm volatile("" : "+v"(p));
+    return lh_f2h(p);
 }
 
 // Elements e0 .. e0 + 8 of f16(x * rms * aux (+ res)) as four packed words: the arithmetic of rms_norm_kernel<ADD>.
@@ -123,8 +135,8 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                     const uint32_t wb[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
-                        const float g = lh_h2f((uint16_t)((wb[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
-                        v[i] = lh_h2f(lh_f2h(lh_gelu_tanh_f32(v[i]) * g));
+                        v[i] = lh_h2f(lh_gelu_mul_h((uint16_t)((w[i >> 1] >> (16 * (i & 1))) & 0xFFFF),
+                                                    (uint16_t)((wb[i >> 1] >> (16 * (i & 1))) & 0xFFFF)));
                     }
                 }
             }

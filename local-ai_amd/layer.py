@@ -395,8 +395,12 @@ class TransformerLayer:
                 kernels.rms_norm_into(batch, out, norm2_w, out2, h, rows, eps)
 
         product_norm(w.attn_output, bs.attn_out, w.attn_post_norm, input, bs.attn_resid, None, w.ffn_norm, bs.normed)
-        self._matmuls(batch, kernels, [w.ffn_gate, w.ffn_up], bs.normed, [bs.gate, bs.up], rows)
-        kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
+        if self.fuse_norm_chain and _groupable(w.ffn_gate, w.ffn_up):
+            kernels.matmul_nt_quant_gelu_mul_into(batch, w.ffn_gate.ty, bs.normed, w.ffn_gate.buf, w.ffn_up.buf, bs.gate, rows,
+                                                  w.ffn_gate.cols, inter)
+        else:
+            self._matmuls(batch, kernels, [w.ffn_gate, w.ffn_up], bs.normed, [bs.gate, bs.up], rows)
+            kernels.gelu_mul_into(batch, bs.gate, bs.up, bs.gate, rows * inter)
         if has_ple:
             product_norm(w.ffn_down, bs.gate, w.ffn_post_norm, bs.attn_resid, output)
         else:

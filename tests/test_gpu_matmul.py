@@ -165,6 +165,32 @@ def test_matmul_norm_fused_equals_separate_kernels(pkg, gpu, fmt):
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_matmul_gelu_mul_fused_equals_separate_kernels(pkg, gpu, fmt):
+    """matmul_nt_quant_gelu_mul_into against the grouped gate / up product followed by gelu_mul, bit for bit: decode batches
+    whose pair is one kernel (gate and up rows paired in a workgroup), and the shapes that go through the grouped product."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    kq = 256 if fmt == "q4_0" else 512
+    for (m, k, n) in ((64, 1536, 6144), (33, kq, 4096), (17, 3 * kq, 12288), (64, 1536, 1024), (8, 1024, 2048), (100, 2 * kq, 4096),
+                      (40, 1280, 200)):
+        print(f"case {fmt} m={m} k={k} n={n}", flush=True)
+        g = pkg.synth.rng(78, m + k + n)
+        wg = pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), ty, n, k)
+        wu = pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), ty, n, k)
+        x = pkg.Buffer.from_slice(ctx, (g.standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16))
+        gate, up, want, got = (pkg.Buffer.empty(ctx, m * n * 2) for _ in range(4))
+        batch = pkg.CommandBatch(ctx)
+        K.matmul_nt_quant_grouped_into(batch, ty, x, [wg.buf, wu.buf], [gate, up], m, k, [n, n])
+        K.gelu_mul_into(batch, gate, up, want, m * n)
+        d0 = batch.dispatch_count()
+        K.matmul_nt_quant_gelu_mul_into(batch, ty, x, wg.buf, wu.buf, got, m, k, n)
+        assert batch.dispatch_count() == d0 + 1
+        batch.commit_and_wait()
+        assert np.abs(want.as_array(np.float16).astype(np.float32)).max() > 0.1
+        assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16)), (fmt, m, k, n)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_split_k(pkg, gpu, oracle, fmt):
     """A decode batch of some tens of rows against the layer's projections: few output tiles, so the k range is split
     over several workgroups whose partial tiles a second kernel sums -- even and odd numbers of k steps per split, a
