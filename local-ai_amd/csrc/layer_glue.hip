@@ -111,33 +111,50 @@ __global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a
     const size_t row = (size_t)rowi * dim;
     uint4 x[4], o[4];
     float s = 0.0f;
+    if constexpr (PART) {
+        // the splits of two chunks, eight at a time, are all requested before the first is added (in split order)
+        const size_t zstride = (size_t)a.part_rows * a.part_cols;
+#pragma unroll
+        for (int it0 = 0; it0 < 4; it0 += 2) {
+            float v[2][8];
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[c][e] = 0.0f;
+            const uint32_t i0 = (threadIdx.x + it0 * blockDim.x) * 8, i1 = (threadIdx.x + (it0 + 1) * blockDim.x) * 8;
+            if (i0 >= dim) break;
+            const bool two = i1 < dim;
+            const float* p0 = a.partial + (size_t)rowi * a.part_cols + i0;
+            const float* p1 = a.partial + (size_t)rowi * a.part_cols + (two ? i1 : i0);
+            for (uint32_t z0 = 0; z0 < a.splits; z0 += 8) {
+                float4 lo[2][8], hi[2][8];
+#pragma unroll
+                for (uint32_t u = 0; u < 8; u++) {
+                    const size_t zo = (size_t)(z0 + u < a.splits ? z0 + u : a.splits - 1) * zstride;
+                    lo[0][u] = *reinterpret_cast<const float4*>(p0 + zo); hi[0][u] = *reinterpret_cast<const float4*>(p0 + zo + 4);
+                    lo[1][u] = *reinterpret_cast<const float4*>(p1 + zo); hi[1][u] = *reinterpret_cast<const float4*>(p1 + zo + 4);
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 8; u++) {
+                    if (z0 + u >= a.splits) break;
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+                        v[c][0] += lo[c][u].x; v[c][1] += lo[c][u].y; v[c][2] += lo[c][u].z; v[c][3] += lo[c][u].w;
+                        v[c][4] += hi[c][u].x; v[c][5] += hi[c][u].y; v[c][6] += hi[c][u].z; v[c][7] += hi[c][u].w;
+                    }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+                x[it0 + c] = make_uint4((uint32_t)lh_f2h(v[c][0]) | ((uint32_t)lh_f2h(v[c][1]) << 16), (uint32_t)lh_f2h(v[c][2]) | ((uint32_t)lh_f2h(v[c][3]) << 16),
+                                        (uint32_t)lh_f2h(v[c][4]) | ((uint32_t)lh_f2h(v[c][5]) << 16), (uint32_t)lh_f2h(v[c][6]) | ((uint32_t)lh_f2h(v[c][7]) << 16));
+        }
+    }
 #pragma unroll
     for (int it = 0; it < 4; it++) {
         const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
         if (i >= dim) break;
-        if constexpr (PART) {
-            float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            const size_t zstride = (size_t)a.part_rows * a.part_cols;
-            const float* p0 = a.partial + (size_t)rowi * a.part_cols + i;
-            for (uint32_t z0 = 0; z0 < a.splits; z0 += 4) {      // four splits' loads in flight, added in split order
-                float4 lo[4], hi[4];
-#pragma unroll
-                for (uint32_t u = 0; u < 4; u++) {
-                    const float* p = p0 + (size_t)(z0 + u < a.splits ? z0 + u : a.splits - 1) * zstride;
-                    lo[u] = *reinterpret_cast<const float4*>(p); hi[u] = *reinterpret_cast<const float4*>(p + 4);
-                }
-#pragma unroll
-                for (uint32_t u = 0; u < 4; u++) {
-                    if (z0 + u >= a.splits) break;
-                    v[0] += lo[u].x; v[1] += lo[u].y; v[2] += lo[u].z; v[3] += lo[u].w;
-                    v[4] += hi[u].x; v[5] += hi[u].y; v[6] += hi[u].z; v[7] += hi[u].w;
-                }
-            }
-            x[it] = make_uint4((uint32_t)lh_f2h(v[0]) | ((uint32_t)lh_f2h(v[1]) << 16), (uint32_t)lh_f2h(v[2]) | ((uint32_t)lh_f2h(v[3]) << 16),
-                               (uint32_t)lh_f2h(v[4]) | ((uint32_t)lh_f2h(v[5]) << 16), (uint32_t)lh_f2h(v[6]) | ((uint32_t)lh_f2h(v[7]) << 16));
-        } else {
-            x[it] = *reinterpret_cast<const uint4*>(a.in + row + i);
-        }
+        if constexpr (!PART) x[it] = *reinterpret_cast<const uint4*>(a.in + row + i);
         rms_sumsq8(x[it], s);
     }
     const float rms = rsqrtf(block_sum(s, scratch) / (float)dim + a.eps);
