@@ -617,10 +617,9 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
 
 // ---- a decode batch of 17 .. 64 rows: weights straight from global memory into MFMA operands ---------------------------------
 // At these row counts a product is a few microseconds of matrix-core time and what counts is latency, so this kernel
-// has no staging phase and one barrier.  A workgroup owns 64 weight rows (four 16-row MFMA tiles) and a k range; its
-// four waves split that range in quarters, every wave multiplying all four tiles against all activation rows for its
-// quarter (one B fragment feeds four MFMAs, which keeps the activation reads -- straight from L2, 16 bytes a lane -- at
-// what a CU's vector memory path delivers), and the four partial tiles are added through LDS at the end.
+// has no workgroup-wide staging phase and one barrier.  A workgroup owns 64 weight rows (four 16-row MFMA tiles) and a
+// k range; its four waves split that range in quarters, every wave multiplying all four tiles against all activation
+// rows for its quarter (one B fragment feeds four MFMAs), and the four partial tiles are added through LDS at the end.
 //
 // A lane fetches the codes it turns into its own A fragments, 8 bytes at a time, one "unit" ahead:
 //   Q4_0  unit = 2 blocks (64 k).  Lane (row r, g) reads qs bytes 8(g&1) .. +8 of block (g>>1): the low nibbles are
@@ -630,7 +629,8 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
 // A code byte c becomes the f16 value 1024 + c by byte permutation (0x6400 | c), the zero point is subtracted exactly
 // and the result multiplied by the block scale in f16: the CPU path's dequantised weight f16((q - 8) d) / d (q - 1)
 // (qat_recover.rs:39-47, 84-93) bit for bit, as in the LDS-tiled kernels.  The B fragment of a k step holds the
-// activations of the same eight k indices, read from the row-major f16 matrix.
+// activations of the same eight k indices; a wave brings them in row by row and re-reads them in fragment order from
+// its own LDS area (see load_b / park_b).
 template <int FMT> struct Skinny;
 template <> struct Skinny<kQ4> { static constexpr int unit_k = 64, frags = 2; };
 template <> struct Skinny<kTQ2> { static constexpr int unit_k = 128, frags = 4; };
@@ -668,7 +668,9 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
                                                               uint32_t M, uint32_t K, uint32_t N_one, float* __restrict__ partial,
                                                               uint32_t units_per_wave, GroupArgs grp) {
     constexpr int UK = Skinny<FMT>::unit_k, NF = Skinny<FMT>::frags;
-    __shared__ float4 red[4][4][4][64];                       // [wave][tile][activation group][lane]
+    // [wave][tile][activation group][lane] partial tiles at the end; before that each wave keeps the activations of its
+    // current unit in its quarter of the same memory
+    __shared__ float4 red[4][4][4][64];
     const uint8_t* __restrict__ W = W_one;
     void* __restrict__ C = C_one;
     uint32_t N = N_one, tile = blockIdx.x >> 1;               // blockIdx.x counts 64-row halves of the 128-row tile grid
@@ -686,13 +688,6 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     const uint8_t* wrow = W + (size_t)(n0 + r) * row_bytes;   // tile t starts 16 rows further on
     const size_t tile_bytes = 16 * row_bytes;
     const uint8_t* wrow_up = PAIR ? grp.W[1] + (size_t)(n0 + r) * row_bytes : nullptr;
-    const uint16_t* xrow[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const uint32_t m = 16 * j + r;
-        xrow[j] = X + (size_t)(m < M ? m : M - 1) * K;        // rows past M repeat the last one and are never stored
-    }
-
     auto load_a = [&](SkinnyRaw (&raw)[4], uint32_t k0) {
         size_t off, doff;
         if constexpr (FMT == kQ4) { const size_t b = (k0 >> 5) + (g >> 1); doff = b * 18; off = doff + 2 + 8 * (g & 1); }
@@ -705,14 +700,30 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
             raw[t].w0 = w.x; raw[t].w1 = w.y; raw[t].d = d | (d << 16);
         }
     };
-    auto load_b = [&](f16x8 (&b)[NF][4], uint32_t k0) {
+    // The activations of a unit (64 rows x UK columns) come in with coalesced loads -- a lane takes 16 bytes of one row,
+    // CPR consecutive lanes one row's UK columns -- one unit ahead, and are parked in the wave's LDS area in fragment
+    // order: block (f, j) holds the 64 cells of B fragment f of activation group j, cell 16g + (c ^ (g | 4 (f & 1))) being
+    // row 16j + c, k group g: eight consecutive lanes read eight cells of one aligned 128-byte line, and the eight cells
+    // of a row that eight consecutive lanes write fall into eight different bank groups.  Read straight from global memory
+    // in fragment order the same bytes cost 16 half-used cache lines per instruction, which bounded the kernel.
+    constexpr int CPR = UK / 8, RPI = 64 / CPR, NLD = 64 / RPI;          // 16-byte chunks per row, rows and loads per unit
+    f32x4* stage = reinterpret_cast<f32x4*>(&red[wave][0][0][0]);        // NF * 4 blocks of 64 cells (at most 16 KB)
+    const uint32_t ld_row = lane / CPR, ld_q = lane % CPR;
+    uint32_t ld_f, ld_g;
+    if constexpr (FMT == kQ4) { ld_g = 2 * (ld_q >> 2) + (ld_q & 1); ld_f = (ld_q & 3) >> 1; }
+    else { ld_f = ld_q >> 2; ld_g = ld_q & 3; }
+    auto load_b = [&](f32x4 (&raw)[NLD], uint32_t k0) {
 #pragma unroll
-        for (int f = 0; f < NF; f++) {
-            uint32_t kf;
-            if constexpr (FMT == kQ4) kf = k0 + 32 * (g >> 1) + 8 * (g & 1) + 16 * f;
-            else kf = k0 + 32 * f + 8 * g;
+        for (int i = 0; i < NLD; i++) {
+            const uint32_t m = RPI * i + ld_row;
+            raw[i] = *reinterpret_cast<const f32x4*>(X + (size_t)(m < M ? m : M - 1) * K + k0 + 8 * ld_q);   // rows past M repeat the last one
+        }
+    };
+    auto park_b = [&](const f32x4 (&raw)[NLD]) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) b[f][j] = *reinterpret_cast<const f16x8*>(xrow[j] + kf);
+        for (int i = 0; i < NLD; i++) {
+            const uint32_t m = RPI * i + ld_row, j = m >> 4, c = m & 15;
+            stage[(ld_f * 4 + j) * 64 + ld_g * 16 + (c ^ (ld_g | ((ld_f & 1) << 2)))] = raw[i];
         }
     };
 
@@ -721,35 +732,43 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     for (int t = 0; t < 4; t++)
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[t][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    auto multiply = [&](const SkinnyRaw (&raw)[4], const f16x8 (&b)[NF][4]) {
+    auto multiply = [&](const SkinnyRaw (&raw)[4]) {
 #pragma unroll
-        for (int f = 0; f < NF; f++)
+        for (int f = 0; f < NF; f++) {
+            f16x8 bf[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) bf[j] = __builtin_bit_cast(f16x8, stage[(f * 4 + j) * 64 + g * 16 + (r ^ (g | ((f & 1) << 2)))]);
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const f16x8 a = skinny_fragment<FMT>(raw[t], f);
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b[f][j], acc[t][j], 0, 0, 0);
+                for (int j = 0; j < 4; j++) acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bf[j], acc[t][j], 0, 0, 0);
             }
+        }
     };
 
-    // two register sets, the unit after the one being multiplied always in flight; the load past the end re-reads the last unit
+    // two register sets for the codes, one for the activations, the unit after the one being multiplied always in flight;
+    // the load past the end re-reads the last unit
     SkinnyRaw ra0[4], ra1[4];
-    f16x8 rb0[NF][4], rb1[NF][4];
+    f32x4 rb[NLD];
     const uint32_t last = k_begin + (units_per_wave - 1) * UK;
     load_a(ra0, k_begin);
-    load_b(rb0, k_begin);
+    load_b(rb, k_begin);
+    park_b(rb);
     for (uint32_t u = 0; u < units_per_wave; u += 2) {
         const uint32_t k1 = k_begin + (u + 1) * UK, k2 = k_begin + (u + 2) * UK;
         load_a(ra1, k1 < last ? k1 : last);
-        load_b(rb1, k1 < last ? k1 : last);
-        multiply(ra0, rb0);
+        load_b(rb, k1 < last ? k1 : last);
+        multiply(ra0);
         if (u + 1 < units_per_wave) {
+            park_b(rb);
             load_a(ra0, k2 < last ? k2 : last);
-            load_b(rb0, k2 < last ? k2 : last);
-            multiply(ra1, rb1);
+            load_b(rb, k2 < last ? k2 : last);
+            multiply(ra1);
+            park_b(rb);
         }
     }
-
+    // a wave's partial tiles go where its staging area was
 #pragma unroll
     for (int t = 0; t < 4; t++)
 #pragma unroll
@@ -816,8 +835,8 @@ uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t blocks, uint3
 }
 
 // The skinny kernel when the shape allows it (f16 activations, 17 .. 64 rows, whole 128-row tiles, at least one unit of k
-// per wave, at most two workgroups per CU -- with more, the activations every workgroup re-reads outweigh what the
-// LDS-tiled kernel spends on staging); false leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
+// per wave; LOCAL_HIP_SKINNY_MAX_WG_PER_CU bounds the workgroups per CU, by default far above any shape here); false
+// leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
 // tiles (one split included) stay in the workspace for a consumer that sums them itself.
 struct SkinnyPartials { const float* partial; uint32_t splits, cols; };
 template <int FMT, int ADT>
@@ -828,11 +847,12 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
     if constexpr (FMT != kF16W && ADT == LH_F16) {
         static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
+        static const int max_wg_per_cu = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_WG_PER_CU"); return e && atoi(e) > 0 ? atoi(e) : 64; }();
         bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
         for (uint32_t i = 0; i < grp.count; i++) whole = whole && grp.N[i] % BN == 0;
         const uint32_t units = k / Skinny<FMT>::unit_k;
         if (!no_skinny && !clip.enabled && m > (uint32_t)kMaxMultivecM && m <= 64 && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
-            2 * tiles_n <= 2 * (uint32_t)cus) {
+            2 * tiles_n <= (uint32_t)max_wg_per_cu * (uint32_t)cus) {
             // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
             const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
