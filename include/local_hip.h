@@ -209,6 +209,15 @@ LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh
  * pairs gate and up rows in one workgroup; other shapes run the grouped product into the workspace and gelu_mul. */
 LH_API int lh_matmul_nt_quant_gelu_mul_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* w_gate,
                                             const lh_buffer* w_up, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
+/* The per-layer-input gate of the multi-row layer paths as one encoded step (local-engine/src/layer.rs:686-700:
+ * matmul_nt_into, gather_strided_f16_into, gelu_mul_into):
+ * out[r, i] = half(gelu(half((in . w^T)[r, i])) * gate_rows[r * row_stride + row_offset + i]), bit for bit the
+ * separate kernels' result; for a decode batch the gelu kernel sums the product's k-split partial tiles itself.
+ * n, row_stride and row_offset must be multiples of 8, the buffers 16-byte aligned. */
+LH_API int lh_matmul_nt_quant_gelu_mul_strided_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input,
+                                                    const lh_buffer* weight, uint32_t m, uint32_t k, uint32_t n,
+                                                    const lh_buffer* gate_rows, uint32_t row_stride,
+                                                    uint32_t row_offset, lh_buffer* output);
 /* A product followed by the row-wise norm that consumes it, as one encoded step: out = rms_norm(in[m, k] . w^T,
  * norm_weight) (+ residual) (* scale), and with norm2_weight also out2 = rms_norm(out, norm2_weight).  This is the
  * sequence matmul_nt_into -> rms_norm_add_into (-> scale_in_place_gpu_into) (-> rms_norm_into) of the multi-row layer

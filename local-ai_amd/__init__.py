@@ -418,6 +418,13 @@ class Kernels:
                                                        _handles(outputs), (C.c_uint32 * n)(*[int(v) for v in ns]),
                                                        _u32(m), _u32(k)))
 
+    def matmul_nt_quant_gelu_mul_strided_into(self, batch, fmt, input, weight, m, k, n, gate_rows, row_stride, row_offset, output):
+        """output[r, i] = gelu((input . weight^T)[r, i]) * gate_rows[r * row_stride + row_offset + i]: the per-layer-input
+        gate (product, slice gather, gelu_mul) as one step."""
+        _check(self._l.lh_matmul_nt_quant_gelu_mul_strided_into(batch._h, C.c_int(fmt), input._h, weight._h, _u32(m), _u32(k),
+                                                                _u32(n), gate_rows._h, _u32(row_stride), _u32(row_offset),
+                                                                output._h))
+
     def matmul_nt_quant_gelu_mul_into(self, batch, fmt, input, w_gate, w_up, output, m, k, n):
         """output[m, n] = gelu(input . w_gate^T) * (input . w_up^T): the two feed-forward products and gelu_mul as one step."""
         _check(self._l.lh_matmul_nt_quant_gelu_mul_into(batch._h, C.c_int(fmt), input._h, w_gate._h, w_up._h, output._h,

@@ -113,6 +113,10 @@ struct LhNormFused {
     uint16_t* out2;
 };
 bool lh_norm_fused_supported(uint32_t dim);
+// gelu_mul_strided's 16-byte kernel with the first operand either f16 rows (`a`) or a product's partial tiles (`partial` not
+// null); dim, b_row_stride and b_off multiples of 8, pointers 16-byte aligned
+void lh_launch_gelu_mul_strided(hipStream_t stream, const void* a, const float* partial, uint32_t splits, uint32_t part_cols, const void* b,
+                                uint32_t b_row_stride, uint32_t b_off, void* out, uint32_t dim, uint32_t rows);
 void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count);   // gelu_mul_into's kernel
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
 

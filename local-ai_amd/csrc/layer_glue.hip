@@ -296,15 +296,41 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const uint16_t* a, con
 // gelu_mul whose second operand is read through gather_strided_f16's addressing (row r of `b` starts at
 // r * b_row_stride + b_off): out[r, i] = half(gelu(a[r, i]) * b[r * b_row_stride + b_off + i]) -- the slice gather and the
 // gate of the per-layer input (layer.rs:690-700) in one dispatch, without the gathered copy.
+// With `part` the first operand is the sum of a product's k-split partial tiles (split z of row r at
+// part.partial[(z * rows + r) * part.cols]), added in split order and rounded to f16 as the product's own reduction would.
+struct GeluPartials { const float* partial; uint32_t splits, cols; };
 template <int VEC>
 __global__ __launch_bounds__(256) void gelu_mul_strided_kernel(const uint16_t* a, const uint16_t* __restrict__ b, uint16_t* out, uint32_t dim,
-                                                              uint32_t rows, uint32_t b_row_stride, uint32_t b_off) {
+                                                              uint32_t rows, uint32_t b_row_stride, uint32_t b_off, GeluPartials part) {
     const uint32_t per_row = dim / VEC, idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= per_row * rows) return;
     const uint32_t r = idx / per_row, i = (idx - r * per_row) * VEC;
     const size_t ia = (size_t)r * dim + i, ib = (size_t)r * b_row_stride + b_off + i;
     if constexpr (VEC == 8) {
-        const uint4 va = *reinterpret_cast<const uint4*>(a + ia), vb = *reinterpret_cast<const uint4*>(b + ib);
+        uint4 va;
+        if (part.partial) {
+            float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const size_t zstride = (size_t)rows * part.cols;
+            const float* p0 = part.partial + (size_t)r * part.cols + i;
+            for (uint32_t z0 = 0; z0 < part.splits; z0 += 8) {
+                float4 lo[8], hi[8];
+#pragma unroll
+                for (uint32_t u = 0; u < 8; u++) {
+                    const size_t zo = (size_t)(z0 + u < part.splits ? z0 + u : part.splits - 1) * zstride;
+                    lo[u] = *reinterpret_cast<const float4*>(p0 + zo); hi[u] = *reinterpret_cast<const float4*>(p0 + zo + 4);
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < 8; u++) {
+                    if (z0 + u >= part.splits) break;
+                    v[0] += lo[u].x; v[1] += lo[u].y; v[2] += lo[u].z; v[3] += lo[u].w; v[4] += hi[u].x; v[5] += hi[u].y; v[6] += hi[u].z; v[7] += hi[u].w;
+                }
+            }
+            va = make_uint4((uint32_t)lh_f2h(v[0]) | ((uint32_t)lh_f2h(v[1]) << 16), (uint32_t)lh_f2h(v[2]) | ((uint32_t)lh_f2h(v[3]) << 16),
+                            (uint32_t)lh_f2h(v[4]) | ((uint32_t)lh_f2h(v[5]) << 16), (uint32_t)lh_f2h(v[6]) | ((uint32_t)lh_f2h(v[7]) << 16));
+        } else {
+            va = *reinterpret_cast<const uint4*>(a + ia);
+        }
+        const uint4 vb = *reinterpret_cast<const uint4*>(b + ib);
         const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
         uint32_t wo[4];
 #pragma unroll
@@ -354,6 +380,13 @@ bool lh_norm_fused_supported(uint32_t dim) { return (dim & 7) == 0 && dim <= 819
 
 void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count) {
     launch_elementwise<kGeluMul>(stream, a, b, out, 0.0f, count);
+}
+
+void lh_launch_gelu_mul_strided(hipStream_t stream, const void* a, const float* partial, uint32_t splits, uint32_t part_cols, const void* b,
+                                uint32_t b_row_stride, uint32_t b_off, void* out, uint32_t dim, uint32_t rows) {
+    const uint32_t items = rows * (dim / 8);
+    hipLaunchKernelGGL(gelu_mul_strided_kernel<8>, dim3((items + 255) / 256), dim3(256), 0, stream, (const uint16_t*)a, (const uint16_t*)b,
+                       (uint16_t*)out, dim, rows, b_row_stride, b_off, GeluPartials{partial, splits, part_cols});
 }
 
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a) {
@@ -505,9 +538,9 @@ int lh_gelu_mul_strided_into(lh_batch* batch, const lh_buffer* a, const lh_buffe
     const bool vec = ((dim | b_row_stride | b_offset) & 7) == 0 && (((uintptr_t)a->ptr | (uintptr_t)b->ptr | (uintptr_t)out->ptr) & 15) == 0;
     const uint32_t items = rows * (dim / (vec ? 8 : 1));
     if (vec) hipLaunchKernelGGL(gelu_mul_strided_kernel<8>, dim3((items + 255) / 256), dim3(256), 0, batch->ctx->stream, (const uint16_t*)a->ptr,
-                                (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset);
+                                (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset, GeluPartials{nullptr, 0, 0});
     else hipLaunchKernelGGL(gelu_mul_strided_kernel<1>, dim3((items + 255) / 256), dim3(256), 0, batch->ctx->stream, (const uint16_t*)a->ptr,
-                            (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset);
+                            (const uint16_t*)b->ptr, (uint16_t*)out->ptr, dim, rows, b_row_stride, b_offset, GeluPartials{nullptr, 0, 0});
     return finish(batch, op);
 }
 

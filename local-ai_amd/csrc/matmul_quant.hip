@@ -1079,6 +1079,45 @@ int lh_matmul_nt_quant_norm_into(lh_batch* b, lh_quant fmt, const lh_buffer* in,
     if (r == LH_OK) b->dispatch_count++;
     return r;
 }
+int lh_matmul_nt_quant_gelu_mul_strided_into(lh_batch* b, lh_quant fmt, const lh_buffer* in, const lh_buffer* w, uint32_t m, uint32_t k, uint32_t n,
+                                             const lh_buffer* gate_rows, uint32_t row_stride, uint32_t row_offset, lh_buffer* out) {
+    const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 + gelu_mul_strided" : "matmul_nt_tq2_0 + gelu_mul_strided";
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256;
+    if (k % blk != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: k %u not /%u", op, k, blk);
+    if (m == 0 || n == 0 || k == 0) return LH_OK;
+    if (((n | row_stride | row_offset) & 7) != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: n, row_stride and row_offset must be multiples of 8", op);
+    lh_context* ctx = b->ctx;
+    const size_t wbytes = fmt == LH_Q4_0 ? (size_t)n * (k / 32) * 18 : (size_t)n * (k / 256) * 66;
+    LH_NEED(in, (size_t)m * k * 2, op, "input");
+    LH_NEED(w, wbytes, op, "weight");
+    LH_NEED(gate_rows, ((size_t)(m - 1) * row_stride + row_offset + n) * 2, op, "gate rows");
+    LH_NEED(out, (size_t)m * n * 2, op, "output");
+    LH_REQUIRE((((uintptr_t)in->ptr | (uintptr_t)gate_rows->ptr | (uintptr_t)out->ptr) & 15) == 0, "%s: buffers must be 16-byte aligned", op);
+    LH_REQUIRE(((uintptr_t)w->ptr & 1) == 0, "%s: weight must be 2-byte aligned", op);
+    const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
+    SkinnyPartials kept{nullptr, 0, 0};
+    const uint8_t* W = (const uint8_t*)w->ptr;
+    const bool skinny = fmt == LH_Q4_0 ? try_skinny<kQ4, LH_F16>(ctx, in->ptr, W, nullptr, LH_F16, m, k, n, none, GroupArgs{}, &kept)
+                                       : try_skinny<kTQ2, LH_F16>(ctx, in->ptr, W, nullptr, LH_F16, m, k, n, none, GroupArgs{}, &kept);
+    if (skinny) {
+        lh_launch_gelu_mul_strided(ctx->stream, nullptr, kept.partial, kept.splits, kept.cols, gate_rows->ptr, row_stride, row_offset, out->ptr, n, m);
+    } else {
+        const size_t half = ctx->workspace_bytes / 2, quarter = ctx->workspace_bytes / 4;
+        if ((size_t)m * n * 2 > quarter) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: %u x %u product exceeds the %zu-byte staging area", op, m, n, quarter);
+        lh_buffer tmp{};
+        tmp.ptr = static_cast<uint8_t*>(ctx->workspace) + half; tmp.len = quarter; tmp.ctx = ctx;
+        const uint32_t d0 = b->dispatch_count;
+        int r = matmul_dispatch(b, op, fmt == LH_Q4_0 ? kQ4 : kTQ2, in, LH_F16, w, &tmp, LH_F16, m, k, n, false);
+        if (r != LH_OK) return r;
+        b->dispatch_count = d0;
+        lh_launch_gelu_mul_strided(ctx->stream, tmp.ptr, nullptr, 0, 0, gate_rows->ptr, row_stride, row_offset, out->ptr, n, m);
+    }
+    int r = lh_check_launch(op);
+    if (r == LH_OK) b->dispatch_count++;
+    return r;
+}
 int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* in, const lh_buffer* const* ws,
                                     lh_buffer* const* outs, const uint32_t* ns, uint32_t m, uint32_t k) {
     const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 (grouped)" : "matmul_nt_tq2_0 (grouped)";

@@ -409,11 +409,17 @@ class TransformerLayer:
         if has_ple:
             ple_buf, n_layer_total = ple_all
             pld = p.per_layer_dim
-            w.per_layer_inp_gate.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
-            if self.fuse_norm_chain:   # this layer's slice of every row's per-layer inputs is read in place
+            g = w.per_layer_inp_gate
+            if self.fuse_norm_chain and g.ty != W_F16 and pld % 8 == 0:
+                # product, slice (read in place out of every row's per-layer inputs) and GeGLU in one step
+                kernels.matmul_nt_quant_gelu_mul_strided_into(batch, g.ty, output, g.buf, rows, g.cols, g.rows, ple_buf,
+                                                              n_layer_total * pld, p.layer_idx * pld, bs.ple_g)
+            elif self.fuse_norm_chain:
+                g.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
                 kernels.gelu_mul_strided_into(batch, bs.ple_g, ple_buf, n_layer_total * pld, p.layer_idx * pld, bs.ple_g, pld,
                                               rows)
             else:
+                g.matmul_nt_into(batch, kernels, output, bs.ple_g, rows)
                 kernels.gather_strided_f16_into(batch, ple_buf, bs.ple_slice, n_layer_total * pld, p.layer_idx * pld, pld,
                                                 rows)
                 kernels.gelu_mul_into(batch, bs.ple_g, bs.ple_slice, bs.ple_g, rows * pld)

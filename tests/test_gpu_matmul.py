@@ -191,6 +191,33 @@ def test_matmul_gelu_mul_fused_equals_separate_kernels(pkg, gpu, fmt):
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_matmul_gelu_mul_strided_fused_equals_separate_kernels(pkg, gpu, fmt):
+    """matmul_nt_quant_gelu_mul_strided_into against matmul_nt + gelu_mul_strided (itself gather_strided + gelu_mul), bit for
+    bit: decode batches (the gelu kernel sums the split tiles), rows served as matvecs, a prefill chunk."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    kq = 256 if fmt == "q4_0" else 512
+    for (m, k, n, stride, off) in ((64, 1536, 256, 35 * 256, 3 * 256), (33, 3 * kq, 128, 128, 0), (8, 1024, 256, 512, 256),
+                                   (100, 2 * kq, 256, 1024, 8), (40, 1280, 200, 208, 8)):
+        print(f"case {fmt} m={m} k={k} n={n}", flush=True)
+        g = pkg.synth.rng(79, m + k + n)
+        w = pkg.QuantWeight.from_bytes(ctx, pkg.synth.weights(fmt, n, k, g), ty, n, k)
+        x = pkg.Buffer.from_slice(ctx, (g.standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16))
+        rows = pkg.Buffer.from_slice(ctx, g.standard_normal(m * stride + n, dtype=np.float32).astype(np.float16))
+        tmp, want, got = (pkg.Buffer.empty(ctx, m * n * 2) for _ in range(3))
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_into(batch, K, x, tmp, m)
+        K.gelu_mul_strided_into(batch, tmp, rows, stride, off, want, n, m)
+        d0 = batch.dispatch_count()
+        K.matmul_nt_quant_gelu_mul_strided_into(batch, ty, x, w.buf, m, k, n, rows, stride, off, got)
+        assert batch.dispatch_count() == d0 + 1
+        batch.commit_and_wait()
+        assert np.array_equal(got.as_array(np.uint16), want.as_array(np.uint16)), (fmt, m, k, n)
+    with pytest.raises(pkg.InvalidArgument):
+        K.matmul_nt_quant_gelu_mul_strided_into(pkg.CommandBatch(ctx), ty, x, w.buf, m, k, n, rows, stride, 4, got)
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_split_k(pkg, gpu, oracle, fmt):
     """A decode batch of some tens of rows against the layer's projections: few output tiles, so the k range is split
     over several workgroups whose partial tiles a second kernel sums -- even and odd numbers of k steps per split, a
