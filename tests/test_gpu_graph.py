@@ -40,7 +40,7 @@ def test_captured_decode_step_replays_like_eager(pkg, gpu, n_lanes):
     batch.begin_capture()
     encode(batch, 0)
     graph = batch.end_capture()
-    assert graph.dispatch_count() > 20
+    assert graph.dispatch_count() >= 16          # two layers of 8 - 10 encoded steps each
     ctx.synchronize()
     assert not outs[0].as_array(np.uint16).any()          # recording runs nothing
 
