@@ -205,7 +205,7 @@ LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh
 /* The feed-forward gate and up projections and their gelu_mul as one encoded step:
  * out[m, n] = half(gelu(half(in . w_gate^T)) * half(in . w_up^T)) -- matmul_nt_into twice and gelu_mul_into of the
  * multi-row layer paths (local-engine/src/layer.rs:652-662), with their roundings, so the result is theirs bit for
- * bit.  For a decode batch (17 .. 64 rows) whose pair fills the chip without a k split this is a single kernel that
+ * bit.  For a decode batch or prefill chunk (17 .. 256 rows) whose pair needs no k split this is a single kernel that
  * pairs gate and up rows in one workgroup; other shapes run the grouped product into the workspace and gelu_mul. */
 LH_API int lh_matmul_nt_quant_gelu_mul_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* w_gate,
                                             const lh_buffer* w_up, lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
@@ -224,7 +224,7 @@ LH_API int lh_matmul_nt_quant_gelu_mul_strided_into(lh_batch* batch, lh_quant fm
  * paths -- local-engine/src/layer.rs:640-652 (attention output, post-attention norm + residual, feed-forward norm),
  * 664-672 (down projection, post-feed-forward norm + residual), 699-716 (per-layer projection, its norm + residual,
  * the layer's output scale) -- with the roundings of the separate kernels, so the results are theirs bit for bit.  For
- * a decode batch (17 .. 64 rows) the norm kernel sums the product's k-split partial tiles itself, which removes the
+ * a decode batch or prefill chunk (17 .. 256 rows) the norm kernel sums the product's k-split partial tiles itself, which removes the
  * reduction pass as well.  residual / norm2_weight / out2 may be NULL; out may alias residual; n must be a multiple
  * of 8, at most 8192, and every buffer 16-byte aligned. */
 LH_API int lh_matmul_nt_quant_norm_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* weight,

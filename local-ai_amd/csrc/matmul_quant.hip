@@ -615,7 +615,7 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
     }
 }
 
-// ---- a decode batch of 17 .. 64 rows: weights straight from global memory into MFMA operands ---------------------------------
+// ---- a decode batch of 17 .. 64 rows, a prefill chunk of up to 256: weights straight from global memory into MFMA operands ----
 // At these row counts a product is a few microseconds of matrix-core time and what counts is latency, so this kernel
 // has no workgroup-wide staging phase and one barrier.  A workgroup owns 64 weight rows (four 16-row MFMA tiles) and a
 // k range; its four waves split that range in quarters, every wave multiplying all four tiles against all activation
@@ -684,6 +684,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     const uint32_t r = lane & 15, g = lane >> 4;
     const size_t row_bytes = FMT == kQ4 ? (size_t)(K >> 5) * 18 : (size_t)(K >> 8) * 66;
     const uint32_t k_begin = (blockIdx.z * 4 + wave) * units_per_wave * UK;
+    const uint32_t m0 = blockIdx.y * 64;                      // more than 64 activation rows: one workgroup per 64 of them
 
     const uint8_t* wrow = W + (size_t)(n0 + r) * row_bytes;   // tile t starts 16 rows further on
     const size_t tile_bytes = 16 * row_bytes;
@@ -715,7 +716,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     auto load_b = [&](f32x4 (&raw)[NLD], uint32_t k0) {
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            const uint32_t m = RPI * i + ld_row;
+            const uint32_t m = m0 + RPI * i + ld_row;
             raw[i] = *reinterpret_cast<const f32x4*>(X + (size_t)(m < M ? m : M - 1) * K + k0 + 8 * ld_q);   // rows past M repeat the last one
         }
     };
@@ -787,7 +788,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
                 gt.x += a.x; gt.y += a.y; gt.z += a.z; gt.w += a.w;
                 up.x += b.x; up.y += b.y; up.z += b.z; up.w += b.w;
             }
-            const uint32_t m = 16 * j + r;
+            const uint32_t m = m0 + 16 * j + r;
             if (m >= M) continue;
             const float gv[4] = {gt.x, gt.y, gt.z, gt.w}, uv[4] = {up.x, up.y, up.z, up.w};
             uint16_t h[4];
@@ -807,7 +808,7 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
             const float4 o = red[w][wave][j][lane];
             v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
         }
-        const uint32_t m = 16 * j + r;
+        const uint32_t m = m0 + 16 * j + r;
         if (m >= M) continue;
         const uint32_t nl = 16 * wave + 4 * g;
         if (partial) {
@@ -821,20 +822,35 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     }
 }
 
-// k splits of the skinny kernel over `blocks` 64-row workgroups: enough workgroups for every CU, a whole number of units
+// Most activation rows the skinny kernel takes (LOCAL_HIP_SKINNY_MAX_M, default 256: a prefill chunk).  Beyond 64 rows
+// every group of 64 gets workgroups of its own, which re-read the codes from L2 while the activation traffic grows with
+// rows x weight rows; measured on a 256-row chunk of the layer bench: 197 -> 163 us per layer, no gain at 512 rows.
+uint32_t skinny_max_m() {
+    static const int v = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_M"); return e && atoi(e) > 16 ? atoi(e) : 256; }();
+    return (uint32_t)v;
+}
+
+// Most 64-row workgroups a launch of the skinny kernel may have (LOCAL_HIP_SKINNY_MAX_WG_PER_CU per CU, default 64).
+uint32_t skinny_max_blocks(const lh_context* ctx) {
+    static const int per_cu = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_WG_PER_CU"); return e && atoi(e) > 0 ? atoi(e) : 64; }();
+    return (uint32_t)per_cu * (uint32_t)ctx->cu_count;
+}
+
+// k splits of the skinny kernel over `workgroups` (64-row blocks x groups of 64 activation rows): enough workgroups for every CU, a whole number of units
 // per wave, partial tiles within half the workspace.
-uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t blocks, uint32_t units_per_wg) {
+uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t workgroups, uint32_t units_per_wg) {
     static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
     uint32_t splits = 1;
-    if (!no_splitk && blocks < (uint32_t)ctx->cu_count) {
+    if (!no_splitk && workgroups < (uint32_t)ctx->cu_count) {
+        const uint32_t blocks = workgroups / ((m + 63) / 64);
         const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
-        const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)ctx->cu_count + blocks - 1) / blocks, fit);
+        const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)ctx->cu_count + workgroups - 1) / workgroups, fit);
         for (uint32_t c = 1; c <= want && c <= units_per_wg; c++) if (units_per_wg % c == 0) splits = c;
     }
     return splits;
 }
 
-// The skinny kernel when the shape allows it (f16 activations, 17 .. 64 rows, whole 128-row tiles, at least one unit of k
+// The skinny kernel when the shape allows it (f16 activations, 17 .. skinny_max_m() rows, whole 128-row tiles, at least one unit of k
 // per wave; LOCAL_HIP_SKINNY_MAX_WG_PER_CU bounds the workgroups per CU, by default far above any shape here); false
 // leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
 // tiles (one split included) stay in the workspace for a consumer that sums them itself.
@@ -843,23 +859,22 @@ template <int FMT, int ADT>
 bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dtype ct, uint32_t m, uint32_t k, uint32_t n, const ClipArgs& clip,
                 const GroupArgs& grp, SkinnyPartials* keep = nullptr) {
     hipStream_t s = ctx->stream;
-    const int cus = ctx->cu_count;
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
     if constexpr (FMT != kF16W && ADT == LH_F16) {
         static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
-        static const int max_wg_per_cu = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_WG_PER_CU"); return e && atoi(e) > 0 ? atoi(e) : 64; }();
         bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
         for (uint32_t i = 0; i < grp.count; i++) whole = whole && grp.N[i] % BN == 0;
         const uint32_t units = k / Skinny<FMT>::unit_k;
-        if (!no_skinny && !clip.enabled && m > (uint32_t)kMaxMultivecM && m <= 64 && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
-            2 * tiles_n <= (uint32_t)max_wg_per_cu * (uint32_t)cus) {
+        if (!no_skinny && !clip.enabled && m > (uint32_t)kMaxMultivecM && m <= skinny_max_m() && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+            2 * tiles_n <= skinny_max_blocks(ctx) && (m <= 64 || 2 * tiles_n * ((m + 63) / 64) <= 8 * (uint32_t)ctx->cu_count)) {
             // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
             const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
             if (keep && fit == 0) return false;
-            const uint32_t splits = skinny_splits(ctx, m, blocks, per_wg);
+            const uint32_t mgroups = (m + 63) / 64;
+            const uint32_t splits = skinny_splits(ctx, m, blocks * mgroups, per_wg);
             float* partial = (splits > 1 || keep) ? static_cast<float*>(ctx->workspace) : nullptr;
-            const dim3 grid(blocks, 1, splits);
+            const dim3 grid(blocks, mgroups, splits);
             const uint16_t* X = static_cast<const uint16_t*>(A);
             if (ct == LH_F32) hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F32>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
             else hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F16>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
@@ -1188,16 +1203,18 @@ int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer*
     const uint32_t blocks = n / 32;
     // one launch where the grouped product of the pair takes the skinny kernel without a k split (split products need
     // their sums before the gelu); the same workgroup count and k ranges, hence the same sums
-    if (!no_skinny && m > (uint32_t)kMaxMultivecM && m <= 64 && n % BN == 0 && k % (4 * unit_k) == 0 &&
-        blocks <= 2 * (uint32_t)ctx->cu_count && skinny_splits(ctx, m, blocks, k / unit_k / 4) == 1) {
+    const uint32_t mgroups = (m + 63) / 64;
+    if (!no_skinny && m > (uint32_t)kMaxMultivecM && m <= skinny_max_m() && n % BN == 0 && k % (4 * unit_k) == 0 &&
+        blocks <= skinny_max_blocks(ctx) && (m <= 64 || blocks * mgroups <= 8 * (uint32_t)ctx->cu_count) &&
+        skinny_splits(ctx, m, blocks * mgroups, k / unit_k / 4) == 1) {
         GroupArgs grp{};
         grp.count = 2;
         grp.W[0] = (const uint8_t*)w_gate->ptr; grp.W[1] = (const uint8_t*)w_up->ptr;
         grp.C[0] = out->ptr; grp.N[0] = n;
         const uint16_t* X = static_cast<const uint16_t*>(in->ptr);
         const uint32_t per_wave = k / unit_k / 4;
-        if (fmt == LH_Q4_0) hipLaunchKernelGGL((matmul_skinny_kernel<kQ4, LH_F16, true>), dim3(blocks), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
-        else hipLaunchKernelGGL((matmul_skinny_kernel<kTQ2, LH_F16, true>), dim3(blocks), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
+        if (fmt == LH_Q4_0) hipLaunchKernelGGL((matmul_skinny_kernel<kQ4, LH_F16, true>), dim3(blocks, mgroups), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
+        else hipLaunchKernelGGL((matmul_skinny_kernel<kTQ2, LH_F16, true>), dim3(blocks, mgroups), dim3(256), 0, ctx->stream, X, grp.W[0], out->ptr, m, k, n, (float*)nullptr, per_wave, grp);
     } else {
         // any other shape: the two products as matmul_nt_quant_grouped_into computes them, staged in the third quarter of the
         // workspace, then gelu_mul
