@@ -47,14 +47,17 @@ def _pool_row(pool, kv, lane, pos):
             pool.values_q.as_array(np.uint8, nc, c0), pool.value_norms.as_array(np.uint16, nn, n0 * 2))
 
 
-def _oracle_token(cfg, pipe, state, model, kvs, lane, tok, pos):
+def _oracle_token(cfg, pipe, state, model, kvs, lane, tok, pos, overwritten=lambda slot: False, max_flips=0.01):
+    """The oracle's logits for `tok` at `pos` of `lane`, fed the cache rows the GPU wrote for that position (a slot for
+    which `overwritten` holds no longer has them -- a ring that has wrapped past the position -- and the oracle keeps its own)."""
     rows = []
     for i in range(cfg.num_hidden_layers):
         slot = pipe.kv_index_map[i]
-        rows.append(None if cfg.is_kv_shared(i) else _pool_row(state.pools[slot], kvs[slot], lane, pos))
+        gone = cfg.is_kv_shared(i) or overwritten(slot)
+        rows.append(None if gone else _pool_row(state.pools[slot], kvs[slot], lane, pos))
     tr = {}
     want = OL.decode_token(model, tok, pos, kvs, rows, tr)
-    assert max(tr["code_flips"]) <= 0.01, f"lane {lane} position {pos}: code flips {tr['code_flips']}"
+    assert max(tr["code_flips"], default=0.0) <= max_flips, f"lane {lane} position {pos}: code flips {tr['code_flips']}"
     return want
 
 
@@ -99,6 +102,38 @@ def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld):
     for lane in range(3):
         want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tokens[lane], positions[lane])
         _close(got[lane], want, f"after reset lane {lane}")
+
+
+def test_prompt_longer_than_the_ring_then_lanes_decode(pkg, gpu, oracle):
+    """A prompt longer than the sliding-window ring (512 slots for this window): the chunked prefill wraps the staging
+    rings (pipeline.rs:1332-1367, quant_cache.rs:266-274), the wrapped rings are copied slot for slot into the lane
+    (quant_unified_pool.rs:269-315) and batched steps carry on past them, next to a lane that starts empty.  Positions
+    whose ring slot has been overwritten by the time the lane is read back are outside every later sliding window; the
+    oracle keeps its own codes for them."""
+    cfg, g, pipe, model = _pipe(pkg, gpu, 64, seed=21, max_batch=256)
+    ring = pipe.kv_caches[0].physical_positions
+    n_prompt, n_lanes, lane_cap = ring + 29, 2, 1024
+    assert pipe.kv_caches[0].is_ringed() and not pipe.kv_caches[2].is_ringed()
+    state = pipe.new_batched_decode_state(n_lanes, lane_cap)
+    kvs = [[OL.KvState(1, c.head_dim, 2, lane_cap, ring_capacity=c.ring_capacity()) for c in pipe.kv_caches]
+           for _ in range(n_lanes)]
+    prompt = [int(v) for v in g.integers(0, cfg.vocab_size, n_prompt)]
+    got = pipe.prefill_lane(state, 1, prompt)
+    for pos, tok in enumerate(prompt):
+        # 256-row chunks go through the f16 matrix-core products (f16-rounded weights and activations, where the matvec
+        # kernels and the oracle keep f32): K and V sit a little further from the oracle's and up to 3 % of a row's
+        # codes land on the other side of a quantiser boundary
+        want = _oracle_token(cfg, pipe, state, model, kvs[1], 1, tok, pos, max_flips=0.03,
+                             overwritten=lambda slot: pipe.kv_caches[slot].is_ringed() and pos + ring < n_prompt)
+    _close(got, want, "prefill past the ring")
+    positions = [0, n_prompt]
+    for step in range(4):
+        tokens = [int(v) for v in g.integers(0, cfg.vocab_size, n_lanes)]
+        got = pipe.decode_batch_step(state, tokens, tokens, positions)
+        for lane in range(n_lanes):
+            want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tokens[lane], positions[lane])
+            _close(got[lane], want, f"step {step} lane {lane} position {positions[lane]}")
+        positions = [p + 1 for p in positions]
 
 
 def test_batched_step_matches_single_sequence_at_pos0(pkg, gpu):
