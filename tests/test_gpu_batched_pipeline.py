@@ -67,22 +67,26 @@ def _close(got, want, what):
     assert want[int(np.argmax(got))] >= want.max() - 2 * WORST, what
 
 
-@pytest.mark.parametrize("pld", [64, 0])
-def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld):
-    cfg, g, pipe, model = _pipe(pkg, gpu, pld, seed=pld)
-    n_lanes, lane_cap = 4, 1024
+@pytest.mark.parametrize("pld,n_lanes", [(64, 4), (0, 4), (64, 24)])
+def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld, n_lanes):
+    """4 lanes: every product runs as matvecs over the rows (exact integer arithmetic, at most 1 % of a row's codes differ
+    from the oracle's).  24 lanes: the decode-batch matrix-core kernel with its fused tail (f16-rounded weights and
+    activations; up to 3 %)."""
+    few = n_lanes <= 8
+    cfg, g, pipe, model = _pipe(pkg, gpu, pld, seed=pld + n_lanes, max_batch=8 if few else 32)
+    lane_cap, flips = 1024, 0.01 if few else 0.03
     state = pipe.new_batched_decode_state(n_lanes, lane_cap)
     assert len(state.pools) == len(pipe.kv_caches) == 3
     assert [p.lane_ring_capacity for p in state.pools] == [c.physical_positions if c.is_ringed() else 0 for c in pipe.kv_caches]
     kvs = [[OL.KvState(1, c.head_dim, 2, lane_cap, ring_capacity=c.ring_capacity()) for c in pipe.kv_caches]
            for _ in range(n_lanes)]
-    # lanes 0 and 3 start empty; lane 1 holds a short prompt, lane 2 one longer than the sliding window and two chunks
+    # the other lanes start empty; lane 1 holds a short prompt, lane 2 one longer than the sliding window
     prompts = {1: [int(v) for v in g.integers(0, cfg.vocab_size, 5)], 2: [int(v) for v in g.integers(0, cfg.vocab_size, 21)]}
     positions = [0] * n_lanes
     for lane, prompt in prompts.items():
         got = pipe.prefill_lane(state, lane, prompt)
         for pos, tok in enumerate(prompt):
-            want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tok, pos)
+            want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tok, pos, max_flips=flips)
         _close(got, want, f"prefill of lane {lane}")
         positions[lane] = len(prompt)
     for step in range(6):
@@ -90,7 +94,7 @@ def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld):
         got = pipe.decode_batch_step(state, tokens, tokens, positions)
         assert got.shape == (n_lanes, cfg.vocab_size) and np.abs(got).max() <= 30.0 + 1e-3
         for lane in range(n_lanes):
-            want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tokens[lane], positions[lane])
+            want = _oracle_token(cfg, pipe, state, model, kvs[lane], lane, tokens[lane], positions[lane], max_flips=flips)
             _close(got[lane], want, f"step {step} lane {lane} position {positions[lane]}")
         positions = [p + 1 for p in positions]
     # a lane taken out of service and reused: its rows are cleared and it decodes like a fresh sequence
