@@ -17,19 +17,19 @@ pytestmark = pytest.mark.gpu
 WORST, MEAN = 0.08, 0.01
 
 
-def _config(pkg, pld=64):
+def _config(pkg, pld=64, head_dims=(128, 256)):
     types = ["sliding_attention", "sliding_attention", "full_attention", "sliding_attention", "sliding_attention",
              "full_attention"]
     return pkg.pipeline.Gemma4QATConfig(vocab_size=640, hidden_size=512, num_hidden_layers=6, num_attention_heads=4,
-                                        num_key_value_heads=1, head_dim=128, global_head_dim=256, sliding_window=16,
+                                        num_key_value_heads=1, head_dim=head_dims[0], global_head_dim=head_dims[1], sliding_window=16,
                                         num_kv_shared_layers=3, hidden_size_per_layer_input=pld, layer_types=types,
                                         sliding_rope_theta=10000.0, full_rope_theta=1000000.0,
                                         full_partial_rotary_factor=0.25)
 
 
-def _pipe(pkg, gpu, pld=64, seed=0, max_batch=8, max_ctx=1024, **layer_options):
+def _pipe(pkg, gpu, pld=64, seed=0, max_batch=8, max_ctx=1024, head_dims=(128, 256), **layer_options):
     ctx, K = gpu
-    cfg = _config(pkg, pld)
+    cfg = _config(pkg, pld, head_dims)
     g = pkg.synth.rng(981, seed)
     t = pkg.synth.decode_model_tensors(cfg, g, [512, 512, 512, 1024, 1024, 1024])
     pipe = pkg.pipeline.DecodePipeline.from_host(ctx, K, cfg, t, max_ctx, max_batch=max_batch, **layer_options)
@@ -67,13 +67,14 @@ def _close(got, want, what):
     assert want[int(np.argmax(got))] >= want.max() - 2 * WORST, what
 
 
-@pytest.mark.parametrize("pld,n_lanes", [(64, 4), (0, 4), (64, 24)])
-def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld, n_lanes):
+@pytest.mark.parametrize("pld,n_lanes,head_dims", [(64, 4, (128, 256)), (0, 4, (128, 256)), (64, 24, (128, 256)), (64, 20, (256, 512))])
+def test_prefilled_lanes_decode_together(pkg, gpu, oracle, pld, n_lanes, head_dims):
     """4 lanes: every product runs as matvecs over the rows (exact integer arithmetic, at most 1 % of a row's codes differ
     from the oracle's).  24 lanes: the decode-batch matrix-core kernel with its fused tail (f16-rounded weights and
-    activations; up to 3 %)."""
+    activations; up to 3 %).  Head dims 256 / 512 are the reference model's: both attention layer kinds then run on the
+    matrix-core attention kernel (128 takes the vector-ALU one)."""
     few = n_lanes <= 8
-    cfg, g, pipe, model = _pipe(pkg, gpu, pld, seed=pld + n_lanes, max_batch=8 if few else 32)
+    cfg, g, pipe, model = _pipe(pkg, gpu, pld, seed=pld + n_lanes, max_batch=8 if few else 32, head_dims=head_dims)
     lane_cap, flips = 1024, 0.01 if few else 0.03
     state = pipe.new_batched_decode_state(n_lanes, lane_cap)
     assert len(state.pools) == len(pipe.kv_caches) == 3
