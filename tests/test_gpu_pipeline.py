@@ -13,20 +13,21 @@ from oracle import layer as OL
 pytestmark = pytest.mark.gpu
 
 
-def _config(pkg, pld):
+def _config(pkg, pld, head_dims=(128, 256)):
     types = ["sliding_attention", "sliding_attention", "full_attention", "sliding_attention", "sliding_attention",
              "full_attention"]
     return pkg.pipeline.Gemma4QATConfig(vocab_size=640, hidden_size=512, num_hidden_layers=6, num_attention_heads=4,
-                                        num_key_value_heads=1, head_dim=128, global_head_dim=256, sliding_window=16,
+                                        num_key_value_heads=1, head_dim=head_dims[0], global_head_dim=head_dims[1], sliding_window=16,
                                         num_kv_shared_layers=3, hidden_size_per_layer_input=pld, layer_types=types,
                                         sliding_rope_theta=10000.0, full_rope_theta=1000000.0,
                                         full_partial_rotary_factor=0.25)
 
 
-@pytest.mark.parametrize("pld,fused", [(64, True), (0, True), (64, False)])
-def test_decode_steps_match_oracle(pkg, gpu, oracle, pld, fused):
+@pytest.mark.parametrize("pld,fused,head_dims", [(64, True, (128, 256)), (0, True, (128, 256)), (64, False, (128, 256)),
+                                                 (64, True, (256, 512))])   # the last: the reference model's head dims
+def test_decode_steps_match_oracle(pkg, gpu, oracle, pld, fused, head_dims):
     ctx, K = gpu
-    cfg = _config(pkg, pld)
+    cfg = _config(pkg, pld, head_dims)
     g = pkg.synth.rng(970, pld)
     inters = [512, 512, 512, 1024, 1024, 1024]          # later layers double-wide, as in the reference model
     t = pkg.synth.decode_model_tensors(cfg, g, inters)
