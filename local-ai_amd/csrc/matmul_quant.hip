@@ -830,6 +830,16 @@ uint32_t skinny_max_m() {
     return (uint32_t)v;
 }
 
+// Fewest activation rows the skinny kernel takes; below it rows run as matvecs.  TQ2_0 from 2 rows (LOCAL_HIP_SKINNY_MIN_M_TQ2):
+// its f16 weights d (q - 1) are exact, so the results differ from the matvec kernels' only in the order of the f32 sums,
+// and a 35-layer step over 16 lanes at 8k context went from 5.19 to 4.05 ms (8 lanes 4.14 to 3.59, 4 lanes 3.63 to 3.38).  Q4_0 from 17 rows (LOCAL_HIP_SKINNY_MIN_M): its weights
+// are rounded to f16 as the CPU path rounds them, which the small-batch kernels of the reference (f32 weights) do not.
+uint32_t skinny_min_m(int fmt) {
+    static const int q4 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M"); return e && atoi(e) > 0 ? atoi(e) : 17; }();
+    static const int tq2 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_TQ2"); return e && atoi(e) > 0 ? atoi(e) : 2; }();
+    return (uint32_t)(fmt == kTQ2 ? tq2 : q4);
+}
+
 // Most 64-row workgroups a launch of the skinny kernel may have (LOCAL_HIP_SKINNY_MAX_WG_PER_CU per CU, default 64).
 uint32_t skinny_max_blocks(const lh_context* ctx) {
     static const int per_cu = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_WG_PER_CU"); return e && atoi(e) > 0 ? atoi(e) : 64; }();
@@ -865,7 +875,7 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
         bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
         for (uint32_t i = 0; i < grp.count; i++) whole = whole && grp.N[i] % BN == 0;
         const uint32_t units = k / Skinny<FMT>::unit_k;
-        if (!no_skinny && !clip.enabled && m > (uint32_t)kMaxMultivecM && m <= skinny_max_m() && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+        if (!no_skinny && !clip.enabled && m >= skinny_min_m(FMT) && m <= skinny_max_m() && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
             2 * tiles_n <= skinny_max_blocks(ctx) && (m <= 64 || 2 * tiles_n * ((m + 63) / 64) <= 8 * (uint32_t)ctx->cu_count)) {
             // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
@@ -995,6 +1005,16 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
     LH_REQUIRE(((uintptr_t)input->ptr & 15) == 0, "%s: input must be 16-byte aligned", op);
     LH_REQUIRE(((uintptr_t)weight->ptr & 1) == 0, "%s: weight must be 2-byte aligned", op);
     const bool mfma = kind == kF16W || (!force_multivec && m > (uint32_t)kMaxMultivecM);
+    if (!mfma && !force_multivec && at == LH_F16 && m >= skinny_min_m(kind)) {   // a small batch the decode-batch kernel takes
+        const uint8_t* Ws = (const uint8_t*)weight->ptr;
+        const bool took = kind == kQ4 ? try_skinny<kQ4, LH_F16>(batch->ctx, input->ptr, Ws, output->ptr, ct, m, k, n, clip, GroupArgs{})
+                                      : try_skinny<kTQ2, LH_F16>(batch->ctx, input->ptr, Ws, output->ptr, ct, m, k, n, clip, GroupArgs{});
+        if (took) {
+            int r = lh_check_launch(op);
+            if (r == LH_OK) batch->dispatch_count++;
+            return r;
+        }
+    }
     if (!mfma) {
         // up to 16 activation rows: m matvecs against the same matrix in one launch of the M = 1 kernels (the weights
         // of one call stay cache resident between the rows); shapes they do not take fall through to multivec_kernel
@@ -1148,7 +1168,8 @@ int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, c
     uint64_t tiles_n = 0;
     for (uint32_t i = 0; i < count; i++) tiles_n += (ns[i] + BN - 1) / BN;
     const uint64_t tiles128 = tiles_n * ((m + 127) / 128);
-    const bool together = m > (uint32_t)kMaxMultivecM && !(m > 64 && tiles128 * 2 >= (uint64_t)ctx->cu_count);
+    const bool small = m <= (uint32_t)kMaxMultivecM;          // then only the decode-batch kernel may take the group as one launch
+    const bool together = (!small || m >= skinny_min_m(kind)) && !(m > 64 && tiles128 * 2 >= (uint64_t)ctx->cu_count);
     if (!together) {
         for (uint32_t i = 0; i < count; i++) {
             int r = matmul_dispatch(b, op, kind, in, LH_F16, ws[i], outs[i], LH_F16, m, k, ns[i], false);
@@ -1175,7 +1196,17 @@ int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, c
     }
     for (uint32_t i = count; i <= 4; i++) grp.tile0[i] = tile;
     const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
-    if (fmt == LH_Q4_0) launch_tiles64<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
+    if (small) {
+        const bool took = fmt == LH_Q4_0 ? try_skinny<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp)
+                                         : try_skinny<kTQ2, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
+        if (!took) {
+            for (uint32_t i = 0; i < count; i++) {
+                int r = matmul_dispatch(b, op, kind, in, LH_F16, ws[i], outs[i], LH_F16, m, k, ns[i], false);
+                if (r != LH_OK) return r;
+            }
+            return LH_OK;
+        }
+    } else if (fmt == LH_Q4_0) launch_tiles64<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
     else launch_tiles64<kTQ2, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k, grp.N[0], none, grp);
     int r = lh_check_launch(op);
     if (r == LH_OK) b->dispatch_count++;
@@ -1204,7 +1235,7 @@ int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer*
     // one launch where the grouped product of the pair takes the skinny kernel without a k split (split products need
     // their sums before the gelu); the same workgroup count and k ranges, hence the same sums
     const uint32_t mgroups = (m + 63) / 64;
-    if (!no_skinny && m > (uint32_t)kMaxMultivecM && m <= skinny_max_m() && n % BN == 0 && k % (4 * unit_k) == 0 &&
+    if (!no_skinny && m >= skinny_min_m(fmt == LH_Q4_0 ? kQ4 : kTQ2) && m <= skinny_max_m() && n % BN == 0 && k % (4 * unit_k) == 0 &&
         blocks <= skinny_max_blocks(ctx) && (m <= 64 || blocks * mgroups <= 8 * (uint32_t)ctx->cu_count) &&
         skinny_splits(ctx, m, blocks * mgroups, k / unit_k / 4) == 1) {
         GroupArgs grp{};
