@@ -830,12 +830,117 @@ uint32_t skinny_max_m() {
     return (uint32_t)v;
 }
 
+// ---- Q4_0, 2 .. 16 activation rows: the same workgroup shape with the operand roles swapped ----------------------------------------
+// The reference's small-batch kernels multiply unrounded f32 weights (q - 8) d (matvec_quant.metal:595-798, 945-1038), so here
+// the block scale stays out of the f16 operand: the weights enter as the B operand holding the exact integers q - 8 (columns
+// = 16 weight rows), the activations as the A operand (rows = activation rows, read straight from global memory: they are
+// shared by every tile and workgroup and stay in L1/L2), one MFMA covers exactly one 32-wide block, and its f32 sums are
+// scaled by d and accumulated on the vector ALU.  A lane's D column is the weight row whose codes and scale it loaded itself,
+// so no value crosses lanes.  Products (4-bit integer x f16) and block sums are exact to f32 rounding: closer to the
+// reference's f32 arithmetic than the 16-bit activation fixed point of the matvec kernels.  Workgroup = 64 weight rows x a
+// k range, four waves = quarters of the range, partial tiles added through LDS; same grid, split and partial-tile layout as
+// matmul_skinny_kernel.
+__device__ __forceinline__ uint32_t ld4_align2(const uint8_t* p) {
+    typedef uint32_t __attribute__((aligned(2))) u32_a2;
+    return *reinterpret_cast<const u32_a2*>(p);
+}
+
+template <int CDT>
+__global__ __launch_bounds__(256, 2) void matmul_small_q4_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W_one, void* __restrict__ C_one,
+                                                                uint32_t M, uint32_t K, uint32_t N_one, float* __restrict__ partial,
+                                                                uint32_t blocks_per_wave, GroupArgs grp) {
+    __shared__ float4 red[4][4][64];                          // [wave][tile][lane]
+    const uint8_t* __restrict__ W = W_one;
+    void* __restrict__ C = C_one;
+    uint32_t N = N_one, tile = blockIdx.x >> 1;
+    if (grp.count) {
+        const uint32_t gi = group_of_tile(grp, tile);
+        W = grp.W[gi]; C = grp.C[gi]; N = grp.N[gi];
+        tile -= grp.tile0[gi];
+    }
+    const uint32_t n0 = tile * BN + (blockIdx.x & 1) * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t c = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)(K >> 5) * 18;
+    const uint32_t b_begin = (blockIdx.z * 4 + wave) * blocks_per_wave;
+    const uint8_t* wrow = W + (size_t)(n0 + c) * row_bytes + 4 * g;        // tile t starts 16 rows further on
+    const size_t tile_bytes = 16 * row_bytes;
+    const uint16_t* xrow = X + (size_t)(c < M ? c : M - 1) * K + 4 * g;    // rows past M repeat the last one and are never stored
+
+    struct Raw { uint32_t w[4], d[4]; uint2 lo, hi; };
+    auto load = [&](Raw& r, uint32_t b) {
+        const size_t off = (size_t)b * 18;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint8_t* p = wrow + t * tile_bytes + off;
+            r.w[t] = ld4_align2(p + 2);
+            r.d[t] = *reinterpret_cast<const uint16_t*>(p - 4 * g);
+        }
+        r.lo = *reinterpret_cast<const uint2*>(xrow + (size_t)b * 32);
+        r.hi = *reinterpret_cast<const uint2*>(xrow + (size_t)b * 32 + 16);
+    };
+    f32x4 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const Raw& r) {
+        struct { uint32_t v[4]; } ax = {{r.lo.x, r.lo.y, r.hi.x, r.hi.y}};
+        const f16x8 a = __builtin_bit_cast(f16x8, ax);
+        const f16x2 zp = (f16x2){(_Float16)1032.0f, (_Float16)1032.0f};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t lo = r.w[t] & 0x0F0F0F0Fu, hi = (r.w[t] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t p[4] = {__builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u),
+                                   __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u), __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)};
+            struct { uint32_t v[4]; } bx;
+#pragma unroll
+            for (int i = 0; i < 4; i++) bx.v[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, p[i]) - zp);
+            const f32x4 blk = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(f16x8, bx), (f32x4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            const float d = lh_h2f((uint16_t)r.d[t]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[t][i] = __builtin_fmaf(blk[i], d, acc[t][i]);
+        }
+    };
+    Raw r0, r1;
+    const uint32_t last = b_begin + blocks_per_wave - 1;
+    load(r0, b_begin);
+    for (uint32_t u = 0; u < blocks_per_wave; u += 2) {
+        const uint32_t b1 = b_begin + u + 1, b2 = b_begin + u + 2;
+        load(r1, b1 < last ? b1 : last);
+        multiply(r0);
+        if (u + 1 < blocks_per_wave) {
+            load(r0, b2 < last ? b2 : last);
+            multiply(r1);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) red[wave][t][lane] = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    __syncthreads();
+    // wave w finishes tile w: D[activation row 4g + i][weight row c]
+    float4 v = red[0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < 4; w++) {
+        const float4 o = red[w][wave][lane];
+        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+    }
+    const float vv[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t nl = 16 * wave + c;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t m = 4 * g + i;
+        if (m >= M) continue;
+        if (partial) partial[((size_t)blockIdx.z * M + m) * ((size_t)gridDim.x * 64) + (size_t)blockIdx.x * 64 + nl] = vv[i];
+        else store_elem<CDT>(C, (size_t)m * N + n0 + nl, vv[i]);
+    }
+}
+
 // Fewest activation rows the skinny kernel takes; below it rows run as matvecs.  TQ2_0 from 2 rows (LOCAL_HIP_SKINNY_MIN_M_TQ2):
 // its f16 weights d (q - 1) are exact, so the results differ from the matvec kernels' only in the order of the f32 sums,
-// and a 35-layer step over 16 lanes at 8k context went from 5.19 to 4.05 ms (8 lanes 4.14 to 3.59, 4 lanes 3.63 to 3.38).  Q4_0 from 17 rows (LOCAL_HIP_SKINNY_MIN_M): its weights
-// are rounded to f16 as the CPU path rounds them, which the small-batch kernels of the reference (f32 weights) do not.
+// and a 35-layer step over 16 lanes at 8k context went from 5.19 to 4.05 ms (8 lanes 4.14 to 3.59, 4 lanes 3.63 to 3.38).  Q4_0
+// from 9 rows (LOCAL_HIP_SKINNY_MIN_M; the matvec kernels are as fast up to 8): up to 16 rows go to matmul_small_q4_kernel,
+// which keeps the weights unrounded as the reference's small-batch kernels do (16 lanes 3.95 -> 3.80 ms); from 17 rows on
+// the weights are the CPU path's f16 values, as in its matrix kernels.
 uint32_t skinny_min_m(int fmt) {
-    static const int q4 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M"); return e && atoi(e) > 0 ? atoi(e) : 17; }();
+    static const int q4 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M"); return e && atoi(e) > 0 ? atoi(e) : 9; }();
     static const int tq2 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_TQ2"); return e && atoi(e) > 0 ? atoi(e) : 2; }();
     return (uint32_t)(fmt == kTQ2 ? tq2 : q4);
 }
@@ -886,7 +991,10 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
             float* partial = (splits > 1 || keep) ? static_cast<float*>(ctx->workspace) : nullptr;
             const dim3 grid(blocks, mgroups, splits);
             const uint16_t* X = static_cast<const uint16_t*>(A);
-            if (ct == LH_F32) hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F32>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
+            if (FMT == kQ4 && m <= (uint32_t)kMaxMultivecM) {   // unrounded weights for the small batches (2 blocks per unit)
+                if (ct == LH_F32) hipLaunchKernelGGL((matmul_small_q4_kernel<LH_F32>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, 2 * (per_wg / splits), grp);
+                else hipLaunchKernelGGL((matmul_small_q4_kernel<LH_F16>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, 2 * (per_wg / splits), grp);
+            } else if (ct == LH_F32) hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F32>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
             else hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F16>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
             if (keep) {
                 *keep = SkinnyPartials{partial, splits, blocks * 64};
@@ -1235,7 +1343,8 @@ int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer*
     // one launch where the grouped product of the pair takes the skinny kernel without a k split (split products need
     // their sums before the gelu); the same workgroup count and k ranges, hence the same sums
     const uint32_t mgroups = (m + 63) / 64;
-    if (!no_skinny && m >= skinny_min_m(fmt == LH_Q4_0 ? kQ4 : kTQ2) && m <= skinny_max_m() && n % BN == 0 && k % (4 * unit_k) == 0 &&
+    if (!no_skinny && m >= skinny_min_m(fmt == LH_Q4_0 ? kQ4 : kTQ2) && (fmt != LH_Q4_0 || m > (uint32_t)kMaxMultivecM) && m <= skinny_max_m() &&
+        n % BN == 0 && k % (4 * unit_k) == 0 &&
         blocks <= skinny_max_blocks(ctx) && (m <= 64 || blocks * mgroups <= 8 * (uint32_t)ctx->cu_count) &&
         skinny_splits(ctx, m, blocks * mgroups, k / unit_k / 4) == 1) {
         GroupArgs grp{};

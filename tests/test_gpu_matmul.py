@@ -42,6 +42,42 @@ def test_small_m_matches_cpu(pkg, gpu, oracle, fmt, k, n):
         refgen.assert_close(cm.as_array(np.float16).astype(np.float32), want, 3e-3, f"{fmt} multivec m={m}")
 
 
+def test_small_batch_q4_kernel_keeps_f32_weights(pkg, gpu, oracle):
+    """9 .. 16 f16 activation rows against whole Q4_0 tiles: the matrix-core kernel whose B operand holds the integers q - 8
+    and whose block sums are scaled by d in f32.  Integer-times-f16 products are exact, so against the oracle's product
+    with the unrounded f32 weights only f32 summation error is left (1e-5 of the normalisation, where the f16-weight
+    kernels sit at 3e-3 on these payloads); plain, grouped and with the k split."""
+    ctx, K = gpu
+    for (m, k, n, ct) in ((9, 1536, 2048, "f32"), (16, 2048, 1536, "f32"), (12, 256, 128, "f32"), (13, 6144, 1536, "f16")):
+        print(f"case m={m} k={k} n={n} out={ct}", flush=True)
+        raw = payload("q4_0", n, k, 0x9A11 + m)
+        dq = expand(oracle, "q4_0", raw, n, k)
+        a16 = (pkg.synth.rng(4, m + k).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+        want = oracle.matmul_nt_f32(a16.astype(np.float32), dq)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0, n, k)
+        ab = pkg.Buffer.from_slice(ctx, a16)
+        guard = 64
+        cb = pkg.Buffer.from_slice(ctx, np.full(m * n * (4 if ct == "f32" else 2) + guard, 0xA5, np.uint8))
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32 if ct == "f32" else pkg.F16, m)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float32, m * n) if ct == "f32" else cb.as_array(np.float16, m * n).astype(np.float32)
+        refgen.assert_close(got, want, 2e-5 if ct == "f32" else 1e-3, f"small q4 {m}x{k}x{n}")
+        assert (cb.as_array(np.uint8)[-guard:] == 0xA5).all()
+    m, k, ns = 11, 1536, (2048, 256, 256)
+    raws = [payload("q4_0", n, k, 0x9B0 + i) for i, n in enumerate(ns)]
+    ws = [pkg.QuantWeight.from_bytes(ctx, r, pkg.Q4_0, n, k) for r, n in zip(raws, ns)]
+    a16 = (pkg.synth.rng(4, 77).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+    ab = pkg.Buffer.from_slice(ctx, a16)
+    outs = [pkg.Buffer.empty(ctx, m * n * 2) for n in ns]
+    batch = pkg.CommandBatch(ctx)
+    K.matmul_nt_quant_grouped_into(batch, pkg.Q4_0, ab, [w.buf for w in ws], outs, m, k, list(ns))
+    batch.commit_and_wait()
+    for i, n in enumerate(ns):
+        want = oracle.matmul_nt_f32(a16.astype(np.float32), expand(oracle, "q4_0", raws[i], n, k))
+        refgen.assert_close(outs[i].as_array(np.float16).astype(np.float32), want, 1e-3, f"small q4 grouped #{i}")
+
+
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_mfma_matmul_tile_boundaries(pkg, gpu, oracle, fmt):
     """kernels.rs:9551: M = 70 with N, K spanning several tiles and ragged edges."""
@@ -120,7 +156,7 @@ def test_matmul_norm_fused_equals_separate_kernels(pkg, gpu, fmt):
     ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
     kq = 256 if fmt == "q4_0" else 512
     cases = [(64, 2048, 1536, True, None, True), (33, 12 * kq, 1536, True, 0.37, False), (17, kq, 256, False, None, False),
-             (64, 1536, 2048, True, 1.7, True), (48, 1536, 8192, False, 0.5, True), (8, 1024, 1536, True, 0.9, True),
+             (64, 1536, 2048, True, 1.7, True), (48, 1536, 8192, False, 0.5, True), (8, 1024, 1536, True, 0.9, True), (12, 1024, 1536, True, 0.9, True),
              (200, 2048, 1536, True, None, True), (40, 1280, 200, True, 2.0, False)]
     for (m, k, n, add, scale, second) in cases:
         print(f"case {fmt} m={m} k={k} n={n} add={add} scale={scale} second={second}", flush=True)
@@ -197,7 +233,7 @@ def test_matmul_gelu_mul_strided_fused_equals_separate_kernels(pkg, gpu, fmt):
     ctx, K = gpu
     ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
     kq = 256 if fmt == "q4_0" else 512
-    for (m, k, n, stride, off) in ((64, 1536, 256, 35 * 256, 3 * 256), (33, 3 * kq, 128, 128, 0), (8, 1024, 256, 512, 256),
+    for (m, k, n, stride, off) in ((64, 1536, 256, 35 * 256, 3 * 256), (33, 3 * kq, 128, 128, 0), (8, 1024, 256, 512, 256), (12, 1536, 256, 512, 256),
                                    (100, 2 * kq, 256, 1024, 8), (40, 1280, 200, 208, 8)):
         print(f"case {fmt} m={m} k={k} n={n}", flush=True)
         g = pkg.synth.rng(79, m + k + n)
