@@ -660,7 +660,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model,model_lanes",
-                    help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time)")
+                    help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time); "
+                         "model_few_lanes (2 .. 16 sequences at 8k context) is not in the default set")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: the hot path is a single-GPU kernel path and no multi-GPU "
@@ -738,6 +739,13 @@ def main():
         extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
+    if "model_few_lanes" in legs:
+        # not in the default set: the same model with 2 .. 16 sequences at 8192 cached positions, where the small-batch
+        # routing of the quantised products (rows as matvecs / the decode-batch kernels) decides the step time
+        extra["model_decode_few_lanes_8k"] = {
+            str(n): bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup, T=8192, single=False, lanes=n)["lanes"]
+            for n in (2, 4, 8, 12, 16)}
+        log(f"[bench] model decode, few lanes: {extra['model_decode_few_lanes_8k']}")
     if legs & {"model", "model_lanes"}:
         extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup, single="model" in legs,
                                                          lanes=64 if "model_lanes" in legs else 0)
