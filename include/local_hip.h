@@ -469,6 +469,28 @@ LH_API int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* 
                                               uint32_t lane_capacity, uint32_t num_q_heads, uint32_t num_kv_heads,
                                               uint32_t window, uint32_t bits, uint32_t n_lanes,
                                               uint32_t ring_capacity);
+/* quant_cache.rs:571-598 (the attend and rotate-back steps of fused_attention_into)
+ * and quant_unified_pool.rs:225-256 (attention_into) as one call each:
+ * lh_flash_attention_tq_into / lh_flash_attention_tq_batched_into into `out`
+ * (f32 scratch of the same shape, left undefined), then
+ * lh_hadamard_rotate_fh_into(out, signs, out_f16, post-sign only).  With 2..32
+ * splits the merge and the rotation run as one kernel; the f16 result equals
+ * the two calls' bit for bit either way. */
+LH_API int lh_flash_attention_tq_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                              const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                              const lh_buffer* v_norms, const lh_buffer* levels,
+                                              const lh_buffer* signs, lh_buffer* out, lh_buffer* out_f16,
+                                              uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                              uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window,
+                                              uint32_t bits, uint32_t ring_capacity);
+LH_API int lh_flash_attention_tq_batched_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                                      const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                                      const lh_buffer* v_norms, const lh_buffer* levels,
+                                                      const lh_buffer* signs, lh_buffer* out, lh_buffer* out_f16,
+                                                      const lh_buffer* positions, uint32_t head_dim,
+                                                      uint32_t lane_capacity, uint32_t num_q_heads,
+                                                      uint32_t num_kv_heads, uint32_t window, uint32_t bits,
+                                                      uint32_t n_lanes, uint32_t ring_capacity);
 
 /* ---- FP16-KV split-K decode attention ---------------------------------------
  * kernels.rs:1397-1557 flash_decoding_into, 1292-1392

@@ -662,6 +662,27 @@ class Kernels:
                                                           _u32(window), _u32(bits), _u32(n_lanes),
                                                           _u32(ring_capacity)))
 
+    def flash_attention_tq_rotated_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, signs, out, out_f16,
+                                        head_dim, kv_len, current_pos, num_q_heads, num_kv_heads, window, bits,
+                                        ring_capacity):
+        """``flash_attention_tq_into`` into the f32 scratch ``out``, then the rotation back out of code space
+        (``hadamard_rotate_fh_into`` with the post-sign) into ``out_f16``, as one call."""
+        _check(self._l.lh_flash_attention_tq_rotated_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                          v_norms._h, levels._h, signs._h, out._h, out_f16._h,
+                                                          _u32(head_dim), _u32(kv_len), _u32(current_pos),
+                                                          _u32(num_q_heads), _u32(num_kv_heads), _u32(window),
+                                                          _u32(bits), _u32(ring_capacity)))
+
+    def flash_attention_tq_batched_rotated_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, signs, out,
+                                                out_f16, positions, head_dim, lane_capacity, num_q_heads, num_kv_heads,
+                                                window, bits, n_lanes, ring_capacity):
+        """``flash_attention_tq_batched_into`` and the rotation back of every lane's heads as one call."""
+        _check(self._l.lh_flash_attention_tq_batched_rotated_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                                  v_norms._h, levels._h, signs._h, out._h, out_f16._h,
+                                                                  positions._h, _u32(head_dim), _u32(lane_capacity),
+                                                                  _u32(num_q_heads), _u32(num_kv_heads), _u32(window),
+                                                                  _u32(bits), _u32(n_lanes), _u32(ring_capacity)))
+
     # -- FP16-KV split-K decode (kernels.rs:1265-1557) --
     def flash_split_count(self, eff_seq_len: int) -> int:
         return int(self._l.lh_flash_split_count(_u32(eff_seq_len)))

@@ -21,6 +21,7 @@
 //    split the workgroup writes the final result itself.
 #include "attention_tq.hpp"
 #include <algorithm>
+#include <cmath>
 
 namespace {
 using namespace lh_attn;
@@ -289,9 +290,63 @@ __global__ __launch_bounds__(kReduceDims * kReduceSlices) void attention_tq_redu
     }
 }
 
+// The merge of up to 2 * kReduceBatch splits and the rotation back out of code space (attention_flash_tq.metal:58-90 with
+// the post-sign) in one launch: one workgroup per (query, head), one thread per output dim.  The merge is
+// attention_tq_reduce_kernel<2>'s arithmetic in its order (the split factors and their sum on the first wave with one
+// split per lane, two interleaved fma chains per dim, added), the rotation hadamard_rotate_kernel's, so the f16 result
+// equals the two launches' bit for bit.
+__global__ __launch_bounds__(512) void attention_tq_reduce_rotate_kernel(const float* __restrict__ ws, const float* __restrict__ signs,
+                                                                         uint16_t* __restrict__ out, uint32_t head_dim, uint32_t num_splits,
+                                                                         float inv_sqrt_d) {
+    __shared__ __align__(16) float sh[512];
+    __shared__ float f_s[2 * kReduceBatch];
+    __shared__ float gl_s;
+    const uint32_t qh = blockIdx.x, d = threadIdx.x;
+    const size_t rec = partial_record_floats(head_dim);
+    const float* base = ws + (size_t)qh * num_splits * rec;
+    float v[2 * kReduceBatch];
+#pragma unroll
+    for (int i = 0; i < 2 * kReduceBatch; i++) v[i] = (uint32_t)i < num_splits ? base[(size_t)i * rec + 4 + d] : 0.0f;
+    if (d < 64) {
+        const float2 ml = d < num_splits ? *reinterpret_cast<const float2*>(base + (size_t)d * rec) : make_float2(-INFINITY, 0.0f);
+        float gm = lh_group_max(ml.x, 64);
+        gm = __shfl(gm, 0, 64);
+        const float f = ml.x == -INFINITY ? 0.0f : __expf(ml.x - gm);
+        if (d < num_splits) f_s[d] = f;
+        float l_loc = 0.0f;
+        l_loc += f * ml.y;
+        l_loc = lh_group_sum(l_loc, 64);
+        if (d == 0) gl_s = l_loc;
+    }
+    __syncthreads();
+    float gl = 0.0f;
+    gl += gl_s;
+    const float inv = gl > 0.0f ? 1.0f / gl : 0.0f;
+    float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kReduceBatch; i++) {
+        if ((uint32_t)(2 * i) < num_splits) o0 = __builtin_fmaf(f_s[2 * i], v[2 * i], o0);
+        if ((uint32_t)(2 * i + 1) < num_splits) o1 = __builtin_fmaf(f_s[2 * i + 1], v[2 * i + 1], o1);
+    }
+    float t = 0.0f;
+    t += o0;
+    t += o1;
+    sh[d] = t * inv;
+    lh_fwht_lds(sh, head_dim, d);
+    float y = __fmul_rn(sh[d], inv_sqrt_d);
+    y = __fmul_rn(y, signs[d]);
+    out[(size_t)qh * head_dim + d] = lh_f2h_exact(y);
+}
+
+// Where the f16 head outputs go when an entry also rotates back out of code space.
+struct RotateBack {
+    const lh_buffer* signs;
+    lh_buffer* out16;
+};
+
 int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
                        const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
-                       const lh_buffer* positions, AttnParams p, uint64_t max_span, uint64_t phys_slots) {
+                       const lh_buffer* positions, AttnParams p, uint64_t max_span, uint64_t phys_slots, const RotateBack* rot = nullptr) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     if (p.bits < 2 || p.bits > 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant bits must be 2..=4, got %u", op, p.bits);
     if (p.head_dim == 0 || (p.head_dim & (p.head_dim - 1)) || p.head_dim > 512)
@@ -310,6 +365,11 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     LH_NEED(k_norms, (size_t)phys_slots * 2, op, "k_norms");
     LH_NEED(v_norms, (size_t)phys_slots * 2, op, "v_norms");
     if (p.mode == kBatched) LH_NEED(positions, (size_t)p.num_queries * 4, op, "positions");
+    if (rot) {
+        if (p.head_dim < 64) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: the rotated form needs head_dim >= 64, got %u", op, p.head_dim);
+        LH_NEED(rot->signs, (size_t)p.head_dim * 4, op, "signs");
+        LH_NEED(rot->out16, qbytes / 2, op, "out_f16");
+    }
 
     const size_t ws_avail = (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
     const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
@@ -342,6 +402,15 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     int r = lh_check_launch(op);
     if (r != LH_OK) return r;
     batch->dispatch_count++;
+    static const int no_fused_merge = [] { const char* e = getenv("LOCAL_HIP_ATTN_MERGE_ROTATE"); return e && e[0] == '0' && e[1] == 0; }();
+    if (rot && p.num_splits > 1 && p.num_splits <= 2 * kReduceBatch && !no_fused_merge) {
+        hipLaunchKernelGGL(attention_tq_reduce_rotate_kernel, dim3(p.num_queries * p.num_q_heads), dim3(p.head_dim), 0, ctx->stream,
+                           (const float*)ctx->workspace, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim, p.num_splits,
+                           1.0f / std::sqrt((float)p.head_dim));
+        r = lh_check_launch(op);
+        if (r == LH_OK) batch->dispatch_count++;
+        return r;
+    }
     if (p.num_splits > 1) {
         const dim3 rgrid(p.num_queries * p.num_q_heads, (p.head_dim + kReduceDims - 1) / kReduceDims);
         if (p.num_splits <= 2 * kReduceBatch)
@@ -351,6 +420,11 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
             hipLaunchKernelGGL(attention_tq_reduce_kernel<16>, rgrid, dim3(kReduceDims * 16), 0, ctx->stream, (const float*)ctx->workspace,
                                (float*)out->ptr, p.head_dim, p.num_splits);
         r = lh_check_launch(op);
+        if (r == LH_OK) batch->dispatch_count++;
+    }
+    if (rot && r == LH_OK) {
+        r = lh_launch_hadamard_fh(ctx, (const float*)out->ptr, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim,
+                                  p.num_queries * p.num_q_heads);
         if (r == LH_OK) batch->dispatch_count++;
     }
     return r;
@@ -372,6 +446,21 @@ int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, const lh_bu
     const uint64_t span = seq > lo ? seq - lo : 0;
     const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
     return attention_dispatch(batch, "flash_attention_tq", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys);
+}
+
+int lh_flash_attention_tq_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, const lh_buffer* signs,
+                                       lh_buffer* out, lh_buffer* out_f16, uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                       uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t ring_capacity) {
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.kv_len = kv_len;
+    p.pos0 = current_pos; p.window = window; p.ring_capacity = ring_capacity; p.mode = kSingle; p.num_queries = 1;
+    const uint64_t seq = std::min<uint64_t>(kv_len, (uint64_t)current_pos + 1);
+    const uint64_t lo = (window > 0 && (uint64_t)current_pos + 1 > window) ? (uint64_t)current_pos + 1 - window : 0;
+    const uint64_t span = seq > lo ? seq - lo : 0;
+    const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
+    const RotateBack rot{signs, out_f16};
+    return attention_dispatch(batch, "flash_attention_tq_rotated", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys, &rot);
 }
 
 static int prefill_common(const char* op, lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
@@ -404,11 +493,11 @@ int lh_flash_attention_tq_prefill_tiled_into(lh_batch* batch, const lh_buffer* r
                           kv_len, start_pos, n_rows, num_q_heads, num_kv_heads, window, bits, ring_capacity);
 }
 
-int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
-                                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
-                                       const lh_buffer* positions, uint32_t head_dim, uint32_t lane_capacity, uint32_t num_q_heads,
-                                       uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t n_lanes, uint32_t ring_capacity) {
-    const char* op = "flash_attention_tq_batched";
+static int batched_common(const char* op, lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                          const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                          const lh_buffer* positions, uint32_t head_dim, uint32_t lane_capacity, uint32_t num_q_heads,
+                          uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t n_lanes, uint32_t ring_capacity,
+                          const RotateBack* rot) {
     AttnParams p{};
     p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads;
     p.window = window; p.ring_capacity = ring_capacity; p.lane_capacity = lane_capacity; p.mode = kBatched; p.num_queries = n_lanes;
@@ -418,7 +507,25 @@ int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* rq, con
     const uint64_t cap = ring_capacity ? ring_capacity : lane_capacity;
     const uint64_t span = window ? std::min<uint64_t>(window, cap) : cap;
     const uint64_t phys = (uint64_t)n_lanes * lane_capacity * num_kv_heads;
-    return attention_dispatch(batch, op, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions, p, span, phys);
+    return attention_dispatch(batch, op, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions, p, span, phys, rot);
+}
+
+int lh_flash_attention_tq_batched_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                       const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                       const lh_buffer* positions, uint32_t head_dim, uint32_t lane_capacity, uint32_t num_q_heads,
+                                       uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t n_lanes, uint32_t ring_capacity) {
+    return batched_common("flash_attention_tq_batched", batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions, head_dim,
+                          lane_capacity, num_q_heads, num_kv_heads, window, bits, n_lanes, ring_capacity, nullptr);
+}
+
+int lh_flash_attention_tq_batched_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                               const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels,
+                                               const lh_buffer* signs, lh_buffer* out, lh_buffer* out_f16, const lh_buffer* positions,
+                                               uint32_t head_dim, uint32_t lane_capacity, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                               uint32_t window, uint32_t bits, uint32_t n_lanes, uint32_t ring_capacity) {
+    const RotateBack rot{signs, out_f16};
+    return batched_common("flash_attention_tq_batched_rotated", batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, positions,
+                          head_dim, lane_capacity, num_q_heads, num_kv_heads, window, bits, n_lanes, ring_capacity, &rot);
 }
 
 }  // extern "C"

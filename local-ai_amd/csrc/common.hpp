@@ -119,6 +119,7 @@ void lh_launch_gelu_mul_strided(hipStream_t stream, const void* a, const float* 
                                 uint32_t b_row_stride, uint32_t b_off, void* out, uint32_t dim, uint32_t rows);
 void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count);   // gelu_mul_into's kernel
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
+int lh_launch_hadamard_fh(lh_context* ctx, const float* input, const float* signs, uint16_t* output, uint32_t head_dim, uint32_t num_heads);
 
 static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }
 
@@ -189,6 +190,18 @@ __device__ __forceinline__ void lh_rotate_pair(float x0, float x1, uint32_t i, u
 // compiler from folding a preceding multiply into v_fma_mixlo_f16, which rounds the exact
 // product once (a different result in double-rounding cases) and turns -0 into +0.
 __device__ __forceinline__ uint16_t lh_f2h_exact(float f) { asm volatile("" : "+v"(f)); return lh_f2h(f); }
+
+// In-place unnormalised fast Walsh-Hadamard transform over sh[0..d) in LDS with one thread per element; every thread of
+// the workgroup calls it.  Sums and differences only, in a fixed order, so every kernel that uses it produces the same bits.
+__device__ __forceinline__ void lh_fwht_lds(float* sh, uint32_t d, uint32_t lane) {
+    for (uint32_t len = 1; len < d; len <<= 1) {
+        __syncthreads();
+        const float self_v = sh[lane], other_v = sh[lane ^ len];
+        __syncthreads();
+        sh[lane] = (lane & len) ? __fsub_rn(other_v, self_v) : __fadd_rn(self_v, other_v);
+    }
+    __syncthreads();
+}
 __device__ __forceinline__ float lh_bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
 
 template <typename T> __device__ __forceinline__ float lh_load_as_f32(const T* p, size_t i);

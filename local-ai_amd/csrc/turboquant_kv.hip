@@ -33,16 +33,7 @@ __device__ __forceinline__ uint32_t unpack_code(const uint8_t* codes, uint32_t d
     return (v >> shift) & ((1u << bits) - 1u);
 }
 
-// In-place unnormalised FWHT over sh[0..d) with one thread per element.
-__device__ __forceinline__ void fwht_lds(float* sh, uint32_t d, uint32_t lane) {
-    for (uint32_t len = 1; len < d; len <<= 1) {
-        __syncthreads();
-        const float self_v = sh[lane], other_v = sh[lane ^ len];
-        __syncthreads();
-        sh[lane] = (lane & len) ? __fsub_rn(other_v, self_v) : __fadd_rn(self_v, other_v);
-    }
-    __syncthreads();
-}
+__device__ __forceinline__ void fwht_lds(float* sh, uint32_t d, uint32_t lane) { lh_fwht_lds(sh, d, lane); }
 
 struct EncodeParams {
     uint32_t head_dim, n_kv_heads, bits, code_bytes;
@@ -254,6 +245,18 @@ int check_tq_shape(const char* op, uint32_t head_dim, uint32_t bits) {
 }
 
 inline float host_inv_sqrt(uint32_t d) { return 1.0f / std::sqrt((float)d); }   // turboquant.rs:47
+
+}  // namespace
+
+// The rotate-back step of the attention entries that take f32 head outputs to f16 (no pre-sign, post-sign): the same
+// launch as lh_hadamard_rotate_fh_into, for callers inside the library that have already checked their buffers.
+int lh_launch_hadamard_fh(lh_context* ctx, const float* input, const float* signs, uint16_t* output, uint32_t head_dim, uint32_t num_heads) {
+    hipLaunchKernelGGL((hadamard_rotate_kernel<float, uint16_t>), dim3(num_heads), dim3(head_dim), 0, ctx->stream, input, signs, output,
+                       head_dim, host_inv_sqrt(head_dim), 0, 1);
+    return lh_check_launch("hadamard_rotate_fh");
+}
+
+namespace {
 
 template <typename TIn, typename TOut>
 int hadamard_launch(lh_batch* batch, const lh_buffer* input, const lh_buffer* signs, lh_buffer* output, uint32_t head_dim,

@@ -109,10 +109,9 @@ class QuantizedKvCache:
         """quant_cache.rs:548-598: rotate q, attend over codes, inverse-rotate to f16."""
         hd = self.head_dim
         kernels.hadamard_rotate_hf_into(batch, q, self.signs, rq, hd, n_q_heads, True, False)
-        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
-                                        self.levels, vacc, hd, seq_len, current_pos, n_q_heads, self.n_kv_heads,
-                                        window, self.bits, self.ring_capacity())
-        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
+        kernels.flash_attention_tq_rotated_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
+                                                self.levels, self.signs, vacc, attn_out, hd, seq_len, current_pos,
+                                                n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
 
     def prepare_token_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, position: int,
                            n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:
@@ -131,10 +130,9 @@ class QuantizedKvCache:
         """quant_cache.rs:571-598: the attend and rotate-back steps of ``fused_attention_into`` for a query that
         ``prepare_token_into`` has already rotated."""
         hd = self.head_dim
-        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
-                                        self.levels, vacc, hd, seq_len, current_pos, n_q_heads, self.n_kv_heads,
-                                        window, self.bits, self.ring_capacity())
-        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, n_q_heads, False, True)
+        kernels.flash_attention_tq_rotated_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
+                                                self.levels, self.signs, vacc, attn_out, hd, seq_len, current_pos,
+                                                n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
 
     def prepare_rows_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, start_pos: int,
                           n_rows: int, n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:
@@ -235,11 +233,10 @@ class QuantizedUnifiedKvPool:
         """quant_unified_pool.rs:225-256: the attend and rotate-back steps of ``attention_into``."""
         hd = self.head_dim
         lanes = min(active_lanes, self.n_lanes)
-        kernels.flash_attention_tq_batched_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
-                                                self.value_norms, self.levels, vacc, positions, hd, self.lane_stride(),
-                                                n_q_heads, self.n_kv_heads, window, self.bits, lanes,
-                                                self.lane_ring_capacity)
-        kernels.hadamard_rotate_fh_into(batch, vacc, self.signs, attn_out, hd, lanes * n_q_heads, False, True)
+        kernels.flash_attention_tq_batched_rotated_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
+                                                        self.value_norms, self.levels, self.signs, vacc, attn_out,
+                                                        positions, hd, self.lane_stride(), n_q_heads, self.n_kv_heads,
+                                                        window, self.bits, lanes, self.lane_ring_capacity)
 
     def copy_prefill_from(self, batch, cache: QuantizedKvCache, lane: int, positions: int) -> None:
         """quant_unified_pool.rs:269-315: seed ``lane`` with the first ``positions`` rows of a single-sequence

@@ -228,3 +228,80 @@ def test_split_invariance_at_32k(pkg, gpu, oracle):
     batch.commit_and_wait()
     ref = oracle.attention_tq_codespace(rq, rkc, rkn, rvc, rvn, levels, hd, 3000, 2999, nq, nkv, 512, bits, 512)
     check(out.as_array(np.float32), ref, "SWA ring 512")
+
+
+@pytest.mark.parametrize("hd,T,window,ring", [(256, 700, 512, 512), (256, 40, 0, 0), (256, 1500, 0, 0), (512, 900, 0, 0),
+                                              (256, 9000, 0, 0), (256, 3, 0, 0), (128, 300, 0, 0)])
+def test_rotated_entry_equals_attention_then_rotation(pkg, gpu, oracle, hd, T, window, ring):
+    """quant_cache.rs:571-598: attend, then rotate back.  The one-call form (merge and rotation in one kernel for 2..32
+    splits, the separate kernels otherwise; head_dim 128 takes the vector-ALU attention) must give the f16 head outputs of
+    the two calls bit for bit, and those must match the oracle's attention and rotation."""
+    ctx, K = gpu
+    nq, nkv, bits = 8, 1, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 900 + T, ring=ring)
+    rq = pkg.synth.rng(6, 15).standard_normal((nq, hd), dtype=np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb, sgb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, signs)
+    acc = [pkg.Buffer.empty(ctx, nq * hd * 4) for _ in range(2)]
+    o16 = [pkg.Buffer.from_slice(ctx, np.full(nq * hd + 32, 0x7BFF, np.uint16)) for _ in range(2)]
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, acc[0], hd, T, T - 1, nq, nkv, window, bits, ring)
+    K.hadamard_rotate_fh_into(batch, acc[0], sgb, o16[0], hd, nq, False, True)
+    K.flash_attention_tq_rotated_into(batch, rqb, kcb, knb, vcb, vnb, lvb, sgb, acc[1], o16[1], hd, T, T - 1, nq, nkv, window,
+                                      bits, ring)
+    batch.commit_and_wait()
+    two, one = o16[0].as_array(np.uint16), o16[1].as_array(np.uint16)
+    assert (one[nq * hd:] == 0x7BFF).all()
+    assert np.array_equal(one, two), f"{int((one != two).sum())} of {nq * hd} f16 outputs differ"
+    ref = oracle.attention_tq_codespace(rq, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, window, bits, ring)
+    ref = oracle.hadamard_rotate(np.asarray(ref, np.float32).reshape(nq, hd), signs, hd, nq, False, True)
+    check(one[:nq * hd].view(np.float16).astype(np.float32), np.asarray(ref, np.float32).reshape(-1), "rotated attention", 3e-3)
+
+
+@pytest.mark.parametrize("hd,lanes,cap", [(256, 5, 600), (512, 3, 700), (256, 40, 256)])
+def test_batched_rotated_entry_equals_attention_then_rotation(pkg, gpu, oracle, hd, lanes, cap):
+    """quant_unified_pool.rs:225-256 as one call: lanes at different positions (one of them at position 0, so some of its
+    splits are empty), f16 head outputs equal to the two calls' bit for bit."""
+    ctx, K = gpu
+    nq, nkv, bits = 8, 1, 2
+    cb = oracle.tq_code_bytes(hd, bits)
+    g = pkg.synth.rng(6, 16)
+    positions = g.integers(0, cap, lanes).astype(np.uint32)
+    positions[0], positions[-1] = cap - 1, 0
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, lanes * cap, nkv, hd, bits, 77)
+    rq = g.standard_normal((lanes, nq * hd), dtype=np.float32)
+    bufs = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, positions, signs)
+    acc = [pkg.Buffer.empty(ctx, rq.nbytes) for _ in range(2)]
+    o16 = [pkg.Buffer.empty(ctx, rq.nbytes // 2) for _ in range(2)]
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_batched_into(batch, bufs[5], bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], acc[0], bufs[6], hd, cap, nq,
+                                      nkv, 0, bits, lanes, 0)
+    K.hadamard_rotate_fh_into(batch, acc[0], bufs[7], o16[0], hd, lanes * nq, False, True)
+    K.flash_attention_tq_batched_rotated_into(batch, bufs[5], bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], bufs[7], acc[1],
+                                              o16[1], bufs[6], hd, cap, nq, nkv, 0, bits, lanes, 0)
+    batch.commit_and_wait()
+    two, one = o16[0].as_array(np.uint16), o16[1].as_array(np.uint16)
+    assert np.array_equal(one, two), f"{int((one != two).sum())} of {one.size} f16 outputs differ"
+    l = lanes // 2
+    ref = oracle.attention_tq_codespace(rq[l], kc, kn, vc, vn, levels, hd, int(positions[l]) + 1, int(positions[l]), nq, nkv,
+                                        0, bits, 0, lane_base=l * cap)
+    ref = oracle.hadamard_rotate(np.asarray(ref, np.float32).reshape(nq, hd), signs, hd, nq, False, True)
+    got = one.reshape(lanes, nq * hd)[l].view(np.float16).astype(np.float32)
+    check(got, np.asarray(ref, np.float32).reshape(-1), f"lane {l}", 3e-3)
+
+
+def test_rotated_entry_arguments(pkg, gpu, oracle):
+    """The one-call form checks the two extra buffers like the others."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, T = 256, 8, 1, 2, 100
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 5)
+    rq = np.zeros((nq, hd), np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb, sgb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, signs)
+    acc, o16 = pkg.Buffer.empty(ctx, nq * hd * 4), pkg.Buffer.empty(ctx, nq * hd * 2)
+    batch = pkg.CommandBatch(ctx)
+    with pytest.raises(pkg.InvalidArgument):
+        K.flash_attention_tq_rotated_into(batch, rqb, kcb, knb, vcb, vnb, lvb, sgb, acc, pkg.Buffer.empty(ctx, nq * hd), hd, T,
+                                          T - 1, nq, nkv, 0, bits, 0)
+    with pytest.raises(pkg.InvalidArgument):
+        K.flash_attention_tq_rotated_into(batch, rqb, kcb, knb, vcb, vnb, lvb, pkg.Buffer.empty(ctx, hd * 2), acc, o16, hd, T,
+                                          T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
