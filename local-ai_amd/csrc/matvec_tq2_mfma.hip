@@ -71,8 +71,8 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
     for (int m = 0; m < 4; m++) out[m] = rem ? __builtin_amdgcn_alignbit(in[m + q + 1], in[m + q], 8 * rem) : in[m + q];
 }
 
-template <typename XT, typename YT, bool SPLITK>
-__global__ __launch_bounds__(256, 2) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
+template <typename XT, typename YT, bool SPLITK, int MAXT = 256>
+__global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
     constexpr bool splitk = SPLITK;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -314,21 +314,35 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     // quantised activation vector; few tiles with long rows: the block groups of a tile are split over 2-4 waves
     const uint32_t ngroups = (nb + 7) >> 3;
     uint32_t split_waves = 1;
-    if (tiles < (uint64_t)ctx->cu_count * 2)
+    if (tiles < (uint64_t)ctx->cu_count * 2) {
         for (uint32_t w = 4; w >= 2; w--) if (ngroups % w == 0) { split_waves = w; break; }
+        // six groups of blocks (12288 columns, the down projection of the wide feed-forward layers): a wave per group,
+        // and twice the threads for the activation staging (f16 in and out only: the decode path's types)
+        static const int six = [] { const char* e = getenv("LOCAL_HIP_TQ2_SPLIT6"); return !(e && e[0] == '0' && e[1] == 0); }();
+        const size_t lds6 = (size_t)kL * K + (size_t)nb * 8 + 128 + 6 * (size_t)kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
+        if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= 96 * 1024) split_waves = 6;
+    }
     const uint32_t splitk = split_waves > 1 ? 1u : 0u;
     static const int wg256_tiles_per_cu = [] { const char* e = getenv("LOCAL_HIP_TQ2_WG256_TILES_PER_CU"); int n = e ? atoi(e) : 2; return n < 1 ? 1 : n; }();
     const uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * wg256_tiles_per_cu ? 256 : 64);
     const uint32_t waves = threads / 64;
     const uint64_t slots = splitk ? tiles : (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
     static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 4 * 16 * 4;
+    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
     const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_guess);          // workgroups per CU that LDS allows
     const int wg_eff = threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu;
     const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
-    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 4 * 16 * 4;
-    if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
+    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
+    if (split_waves == 6) {   // more than the 64 KB a kernel gets without asking
+        static bool raised = false;   // one owner thread per context
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute((const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            if (e != hipSuccess) return lh_fail(LH_ERR_PIPELINE_CREATION, "matvec_tq2_0: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    } else if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
     single.pro = pro;
@@ -353,7 +367,9 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         if (splitk) hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, true>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
         else hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, false>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
     } while (0)
-    if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
+    if (split_waves == 6)
+        hipLaunchKernelGGL((matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K);
+    else if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
     else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
     else LH_LAUNCH(float, uint16_t);
