@@ -770,7 +770,7 @@ def main():
                    "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "matvec_tq2_mfma_kernel<float, float, false>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
+                     "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
                      "launch_ms": head["ms_per_launch_events"]},
         "cpu_baseline": cpu,
         "extra": extra,
