@@ -443,6 +443,21 @@ LH_API int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, cons
                                       const lh_buffer* levels, lh_buffer* out, uint32_t head_dim, uint32_t kv_len,
                                       uint32_t current_pos, uint32_t num_q_heads, uint32_t num_kv_heads,
                                       uint32_t window, uint32_t bits, uint32_t ring_capacity);
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): lh_flash_attention_tq_into with the split-K partial
+ * records kept in a static device array of 8 MiB instead of the context
+ * workspace; the call itself allocates nothing.  Same arguments and results.
+ * Limit: num_q_heads * (head_dim + 4) <= 8192 (256 split records of every
+ * query head must fit), otherwise LH_ERR_INVALID_ARGUMENT.  All calls on one
+ * GPU share that GPU's array: calls that overlap on one GPU (two contexts,
+ * two streams) race; calls on one context are ordered by its stream. */
+LH_API int lh_flash_attention_tq_static_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                             const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                             const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                             uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                             uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window,
+                                             uint32_t bits, uint32_t ring_capacity);
 /* kernels.rs:5259-5420 flash_attention_tq_prefill{,_tiled}_into,
  * shaders/attention_flash_tq.metal:290-556: n_rows causal query rows at
  * positions start_pos..start_pos+n_rows-1; rq / out [n_rows, num_q_heads, head_dim]. */

@@ -635,6 +635,14 @@ class Kernels:
                                                   _u32(num_q_heads), _u32(num_kv_heads), _u32(window), _u32(bits),
                                                   _u32(ring_capacity)))
 
+    def flash_attention_tq_static_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim, kv_len,
+                                       current_pos, num_q_heads, num_kv_heads, window, bits, ring_capacity):
+        """flash_attention_tq_into for callers that may not allocate: the split partials live in a static device array."""
+        _check(self._l.lh_flash_attention_tq_static_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h, v_norms._h,
+                                                         levels._h, out._h, _u32(head_dim), _u32(kv_len), _u32(current_pos),
+                                                         _u32(num_q_heads), _u32(num_kv_heads), _u32(window), _u32(bits),
+                                                         _u32(ring_capacity)))
+
     def flash_attention_tq_prefill_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, out, head_dim,
                                         kv_len, start_pos, n_rows, num_q_heads, num_kv_heads, window, bits,
                                         ring_capacity):

@@ -32,6 +32,15 @@ constexpr int kMaxDpl = 8;        // head_dim 512 over 64 lanes
 constexpr int kHeadsPerPass = 8;  // query heads served together from one decode of a position
 constexpr int kPosBatch = 8;      // positions whose loads a wave keeps in flight together
 
+// Split-K partial records of lh_flash_attention_tq_static_into: device memory that exists from the moment the code
+// object is loaded, so that entry never allocates.  Every GPU the library runs on holds its own copy at its own address
+// until the process ends; the name below is only a host-side handle, the address comes from hipGetSymbolAddress.
+constexpr size_t kStaticScratchFloats = (size_t)2 << 20;          // 8 MiB
+constexpr uint32_t kStaticMinSplits = 256;                        // split records that must fit for a call to be accepted
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices];                         // per device, set by lh_attention_static_scratch_init
+
 // The lane's bit window of one code record: `dpl` codes starting at bit lane*dpl*bits.
 __device__ __forceinline__ uint32_t load_window(const uint8_t* rec, uint32_t byte0, uint32_t nbytes) {
     uint32_t v = 0;
@@ -346,7 +355,8 @@ struct RotateBack {
 
 int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
                        const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
-                       const lh_buffer* positions, AttnParams p, uint64_t max_span, uint64_t phys_slots, const RotateBack* rot = nullptr) {
+                       const lh_buffer* positions, AttnParams p, uint64_t max_span, uint64_t phys_slots, const RotateBack* rot = nullptr,
+                       float* ws_override = nullptr, size_t ws_override_floats = 0) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     if (p.bits < 2 || p.bits > 4) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: TurboQuant bits must be 2..=4, got %u", op, p.bits);
     if (p.head_dim == 0 || (p.head_dim & (p.head_dim - 1)) || p.head_dim > 512)
@@ -371,10 +381,11 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
         LH_NEED(rot->out16, qbytes / 2, op, "out_f16");
     }
 
-    const size_t ws_avail = (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
+    float* const ws = ws_override ? ws_override : (float*)ctx->workspace;
+    const size_t ws_avail = ws_override ? ws_override_floats : (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
     const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
                             (const uint8_t*)v_codes->ptr, (const uint16_t*)v_norms->ptr, (const float*)levels->ptr,
-                            positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, (float*)ctx->workspace};
+                            positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, ws};
     if (max_span == 0 || !mfma_supported(p, ptrs)) {
         // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
         const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
@@ -405,7 +416,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     static const int no_fused_merge = [] { const char* e = getenv("LOCAL_HIP_ATTN_MERGE_ROTATE"); return e && e[0] == '0' && e[1] == 0; }();
     if (rot && p.num_splits > 1 && p.num_splits <= 2 * kReduceBatch && !no_fused_merge) {
         hipLaunchKernelGGL(attention_tq_reduce_rotate_kernel, dim3(p.num_queries * p.num_q_heads), dim3(p.head_dim), 0, ctx->stream,
-                           (const float*)ctx->workspace, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim, p.num_splits,
+                           (const float*)ws, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim, p.num_splits,
                            1.0f / std::sqrt((float)p.head_dim));
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
@@ -414,10 +425,10 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     if (p.num_splits > 1) {
         const dim3 rgrid(p.num_queries * p.num_q_heads, (p.head_dim + kReduceDims - 1) / kReduceDims);
         if (p.num_splits <= 2 * kReduceBatch)
-            hipLaunchKernelGGL(attention_tq_reduce_kernel<2>, rgrid, dim3(kReduceDims * 2), 0, ctx->stream, (const float*)ctx->workspace,
+            hipLaunchKernelGGL(attention_tq_reduce_kernel<2>, rgrid, dim3(kReduceDims * 2), 0, ctx->stream, (const float*)ws,
                                (float*)out->ptr, p.head_dim, p.num_splits);
         else
-            hipLaunchKernelGGL(attention_tq_reduce_kernel<16>, rgrid, dim3(kReduceDims * 16), 0, ctx->stream, (const float*)ctx->workspace,
+            hipLaunchKernelGGL(attention_tq_reduce_kernel<16>, rgrid, dim3(kReduceDims * 16), 0, ctx->stream, (const float*)ws,
                                (float*)out->ptr, p.head_dim, p.num_splits);
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
@@ -431,6 +442,17 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
 }
 
 }  // namespace
+
+// Called by lh_context_create with `device` current: resolves this device's copy of the static scratch array once.
+int lh_attention_static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return LH_OK;            // such a device simply has no static entry
+    if (g_scratch_ptr[device]) return LH_OK;
+    float* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return lh_fail(LH_ERR_LIBRARY_CREATION, "static attention scratch on device %d: %s", device, hipGetErrorString(e));
+    g_scratch_ptr[device] = ptr;
+    return LH_OK;
+}
 
 extern "C" {
 
@@ -446,6 +468,31 @@ int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, const lh_bu
     const uint64_t span = seq > lo ? seq - lo : 0;
     const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
     return attention_dispatch(batch, "flash_attention_tq", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys);
+}
+
+int lh_flash_attention_tq_static_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                      const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, lh_buffer* out,
+                                      uint32_t head_dim, uint32_t kv_len, uint32_t current_pos, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                      uint32_t window, uint32_t bits, uint32_t ring_capacity) {
+    const char* op = "flash_attention_tq_static";
+    if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    const int dev = batch->ctx->device;
+    float* ws = (dev >= 0 && dev < kMaxDevices) ? g_scratch_ptr[dev] : nullptr;
+    if (!ws) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: no static scratch on device %d (the context was not created by this library)", op, dev);
+    // kStaticMinSplits records of every query head must fit: beyond that the call is refused rather than run with few splits
+    const uint64_t need = (uint64_t)num_q_heads * partial_record_floats(head_dim) * kStaticMinSplits;
+    if (head_dim <= 512 && need > kStaticScratchFloats)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: num_q_heads %u x (head_dim %u + 4) exceeds %zu, the most the static scratch (%zu bytes) holds",
+                       op, num_q_heads, head_dim, kStaticScratchFloats / kStaticMinSplits, kStaticScratchFloats * sizeof(float));
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.kv_len = kv_len;
+    p.pos0 = current_pos; p.window = window; p.ring_capacity = ring_capacity; p.mode = kSingle; p.num_queries = 1;
+    const uint64_t seq = std::min<uint64_t>(kv_len, (uint64_t)current_pos + 1);
+    const uint64_t lo = (window > 0 && (uint64_t)current_pos + 1 > window) ? (uint64_t)current_pos + 1 - window : 0;
+    const uint64_t span = seq > lo ? seq - lo : 0;
+    const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
+    return attention_dispatch(batch, op, rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys, nullptr, ws,
+                              kStaticScratchFloats);
 }
 
 int lh_flash_attention_tq_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,

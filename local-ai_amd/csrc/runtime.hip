@@ -80,6 +80,10 @@ int lh_context_create(int device_index, lh_context** out) {
     LH_HIP_TRY(hipGetDeviceProperties(&prop, device_index), LH_ERR_NO_DEVICE, "hipGetDeviceProperties");
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return lh_fail(LH_ERR_LIBRARY_CREATION, "kernels are built for gfx950 only, device is %s", prop.gcnArchName);
+    {
+        const int rs = lh_attention_static_scratch_init(device_index);
+        if (rs != LH_OK) return rs;
+    }
     lh_context* ctx = new (std::nothrow) lh_context();
     if (!ctx) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_context));
     ctx->device = device_index;
