@@ -55,8 +55,27 @@ def distinct_replicas(pkg, ctx, raw, count, block_bytes):
     return big, [big.view(i * wb, wb) for i in range(count)]
 
 
+SETTLE_MS = 150.0   # --settle-ms: untimed run of each measured callable before its warm-up steps
+
+
+def settle(ctx, fn, ms=None):
+    """Runs fn() back to back for about `ms` milliseconds of wall time, untimed.  The GPU raises its clocks only after
+    some tens of milliseconds of continuous work (the same launch measures 15-20 % slower in the first few
+    milliseconds after an idle period), and the quantity reported is the rate the kernel sustains."""
+    ms = SETTLE_MS if ms is None else ms
+    if ms <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(8):
+            fn()
+        ctx.synchronize()
+
+
 def time_steps(pkg, ctx, fn, steps, warmup):
-    """Wall-clock (sync on both sides) and HIP-event time of `steps` calls of fn()."""
+    """Wall-clock (sync on both sides) and HIP-event time of `steps` calls of fn(), after the settle phase and `warmup`
+    untimed calls."""
+    settle(ctx, fn)
     for _ in range(warmup):
         fn()
     ctx.synchronize()
@@ -652,10 +671,13 @@ def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
 
 
 def main():
+    global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed milliseconds each measured call is run before its warm-up steps, so that the clocks have risen")
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -663,6 +685,7 @@ def main():
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time); "
                          "model_few_lanes (2 .. 16 sequences at 8k context) is not in the default set")
     args = ap.parse_args()
+    SETTLE_MS = args.settle_ms
     if args.gpus != 1:
         print("bench.py measures one MI355X: the hot path is a single-GPU kernel path and no multi-GPU "
               "figure exists for it; run with --gpus 1", file=sys.stderr)
@@ -767,7 +790,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "TQ2_0 fused dequant-matvec, M=1, N=8192 x K=2048 (MLP gate/up), fp32 x and y",
                    "replicas_per_step": head["replicas"], "launches_per_step": 1,
-                   "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS},
+                   "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS,
+                   "settle_ms_before_warmup": SETTLE_MS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],

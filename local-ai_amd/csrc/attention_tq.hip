@@ -397,12 +397,8 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
 
         const size_t lds_bytes = (size_t)kWavesPerWG * kHeadsPerPass * p.head_dim * 4;
         if (lds_bytes > 48 * 1024) {
-            static bool raised = false;   // one owner thread per context
-            if (!raised) {
-                LH_HIP_TRY(hipFuncSetAttribute((const void*)attention_tq_split_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024),
-                           LH_ERR_PIPELINE_CREATION, op);
-                raised = true;
-            }
+            const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_split_kernel, 72 * 1024, op);
+            if (rl != LH_OK) return rl;
         }
         hipLaunchKernelGGL(attention_tq_split_kernel, dim3(p.num_splits, p.num_queries * p.num_kv_heads), dim3(kThreads), lds_bytes, ctx->stream,
                            ptrs.rq, ptrs.k_codes, ptrs.k_norms, ptrs.v_codes, ptrs.v_norms, ptrs.levels, ptrs.positions, ptrs.out, ptrs.ws, p);

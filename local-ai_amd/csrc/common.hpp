@@ -121,6 +121,9 @@ void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* 
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
 int lh_launch_hadamard_fh(lh_context* ctx, const float* input, const float* signs, uint16_t* output, uint32_t head_dim, uint32_t num_heads);
 
+// Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncAttributeMaxDynamicSharedMemorySize), once per kernel and device.
+int lh_raise_dynamic_lds(lh_context* ctx, const void* kernel, size_t bytes, const char* op);
+
 // Resolves the calling device's copy of the attention kernels' static scratch array (attention_tq.hip); the device must be current.
 int lh_attention_static_scratch_init(int device);
 

@@ -213,8 +213,13 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int G = FMT == LH_TQ2_0 ? 256 : 32;
     constexpr int U = steps_in_flight<FMT>(NPOS);
+    // [xq: L limb planes][xs: K/G scales] and, with two limbs, the residual level behind them: [xq2: 2 planes][xs2]
     uint32_t* xq = reinterpret_cast<uint32_t*>(lds);
     float* xs = reinterpret_cast<float*>(lds + (size_t)L * K);
+    uint32_t* xq2 = reinterpret_cast<uint32_t*>(xs + K / G);
+    float* xs2 = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(xq2) + (size_t)2 * K);
+    const XResidual resid{xq2, xs2, nullptr};
+    bool any_coarse = false;   // a lane of this wave owns a unit column with a residual level
 
     const uint32_t upr = K >> 6;                                  // unit columns per row
     const uint32_t row_bytes = FMT == LH_TQ2_0 ? (K >> 8) * 66 : (K >> 5) * 18;
@@ -248,8 +253,20 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
 
         if (pb.vector != staged_vector) {
             __syncthreads();   // every wave is done reading the previous vector's limbs
-            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG, single.pro);
+            quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG, single.pro, L == 2 ? &resid : nullptr);
             __syncthreads();
+            if constexpr (L == 2) {
+                bool mine = false;
+#pragma unroll
+                for (int p = 0; p < NPOS; p++) {
+                    const uint32_t ucol = col0 + 64u * p;
+                    if (ucol < upr) {
+                        if constexpr (FMT == LH_TQ2_0) mine = mine || xs2[ucol >> 2] != 0.0f;
+                        else mine = mine || xs2[2 * ucol] != 0.0f || xs2[2 * ucol + 1] != 0.0f;
+                    }
+                }
+                any_coarse = __builtin_amdgcn_ballot_w64(mine) != 0;
+            }
 #pragma unroll
             for (int p = 0; p < NPOS; p++) {
                 const uint32_t ucol = col0 + 64u * p;
@@ -292,6 +309,20 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                 part[u] = 0.0f;
 #pragma unroll
                 for (int p = 0; p < NPOS; p++) part[u] += unit_dot<FMT, L>(w[u][p], ux[p]);
+            }
+            if constexpr (L == 2) {
+                if (any_coarse) {   // uniform over the wave; rare: the residual level of the lane's unit columns, read from LDS
+#pragma unroll
+                    for (int p = 0; p < NPOS; p++) {
+                        const uint32_t ucol = col0 + 64u * p;
+                        if (ucol < upr) {
+                            UnitX<FMT, 2> ur;
+                            load_unit_x<FMT, 2>(ur, ucol, K, xq2, xs2);
+#pragma unroll
+                            for (int u = 0; u < U; u++) part[u] += unit_dot<FMT, 2>(w[u][p], ur);
+                        }
+                    }
+                }
             }
             // butterfly over the lanes of a row, all U rows per level
             if (red_width > 1) {
@@ -447,16 +478,22 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
     g.steps_per_wg = (uint32_t)((steps + want - 1) / want);
     g.grid = (uint32_t)((steps + g.steps_per_wg - 1) / g.steps_per_wg);
     const uint32_t G = fmt == LH_TQ2_0 ? 256 : 32;
-    g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4;
+    g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4 + (L == 2 ? (size_t)2 * K + (size_t)(K / G) * 4 + 16 : 0);
     return g;
 }
 
 template <int FMT, int L, int NPOS>
 int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const MatvecBase& single, uint32_t count, lh_dtype xt,
                  lh_dtype yt, uint32_t rows, uint32_t K, const LaunchGeom& g) {
-#define LH_LAUNCH(XT, YT)                                                                                              \
-    hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream, \
-                       dev_problems, single, count, rows, K, g.lpr_log2, g.steps_per_wg)
+#define LH_LAUNCH(XT, YT)                                                                                                   \
+    do {                                                                                                                    \
+        if (g.lds_bytes > 64 * 1024) {   /* long rows: more than the 64 KB a kernel gets without asking */                  \
+            const int rl = lh_raise_dynamic_lds(ctx, (const void*)matvec_quant_kernel<FMT, L, NPOS, XT, YT>, 96 * 1024, "matvec_quant"); \
+            if (rl != LH_OK) return rl;                                                                                     \
+        }                                                                                                                   \
+        hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream,  \
+                           dev_problems, single, count, rows, K, g.lpr_log2, g.steps_per_wg);                               \
+    } while (0)
     if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
     else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);

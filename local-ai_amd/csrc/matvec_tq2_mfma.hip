@@ -35,9 +35,14 @@ constexpr int kL = 2;                        // activation limbs (16-bit block f
 constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
 constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
+constexpr size_t kMaxLdsBytes = 128 * 1024;   // most dynamic LDS a launch here asks for (a CU has 160 KB)
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+// Bytes of the activation area at the head of the dynamic LDS: two limb planes for each of the two fixed-point levels,
+// four per-block arrays (scale and integer sum of either level), padded to 16 bytes.
+__host__ __device__ constexpr size_t lds_head_bytes(uint32_t K) { return (size_t)2 * kL * K + (size_t)(K >> 8) * 16 + 16; }
 
 struct Tq2Problem {
     const uint8_t* matrix;
@@ -77,9 +82,12 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     constexpr bool splitk = SPLITK;
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t nb = K >> 8;                                     // blocks per row
+    // [xq: 2 x K/4 limb words][xq2: the same for the residual level][xs nb][xn nb][xs2 nb][xn2 nb][pad]
     uint32_t* xq = reinterpret_cast<uint32_t*>(lds);                // [2][K/4] activation limbs
-    float* xs = reinterpret_cast<float*>(lds + (size_t)kL * K);     // [nb] activation scales
+    uint32_t* xq2 = reinterpret_cast<uint32_t*>(lds + (size_t)kL * K);
+    float* xs = reinterpret_cast<float*>(lds + (size_t)2 * kL * K); // [nb] activation scales
     int* xn = reinterpret_cast<int*>(xs + nb);                      // [nb] sum of the block's integers
+    const XResidual resid{xq2, xs + 2 * nb, xn + 2 * nb};
     const uint32_t kq = K >> 2;
     const uint32_t row_bytes = nb * 66;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     const uint32_t c = lane & 15;                                   // B / D layout: column c, k-group / row-group g
     const uint32_t cb = c >> 1, cl = c & 1;                         // column's block (within a group of 8) and limb
     const uint32_t lane_x_off = 4u * (cl * kq + (g >> 1) * 32u + (g & 1) * 4u);
-    const uint32_t zero_off = (uint32_t)((size_t)kL * K + (size_t)nb * 8);      // 128 bytes of zeros behind xs / xn
+    const uint32_t zero_off = (uint32_t)lds_head_bytes(K);                      // 128 bytes of zeros behind the activation area
     if (threadIdx.x < 32) reinterpret_cast<uint32_t*>(lds + zero_off)[threadIdx.x] = 0;
     uint8_t* image = lds + zero_off + 128 + (size_t)wave * kImageBytes;         // this wave's tile image
 
@@ -187,7 +195,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
         const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
-            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro);
+            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro, &resid);
             __syncthreads();
             staged = pb.vector;
         }
@@ -218,10 +226,15 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
         // ---- column constants of this group
         const bool col_valid = b0 + cb < nb;
         const uint32_t dblk = col_valid ? b0 + cb : nb - 1;
-        const float xscale16 = (col_valid && cl == 0) ? xs[dblk] * 0.0625f : 0.0f;   // high-limb columns and padding add nothing
-        const int nsum16 = col_valid ? xn[dblk] << 4 : 0;
-        const uint32_t my_off = col_valid ? lane_x_off + dblk * 256u : zero_off;
         const uint8_t* arow = image + r * seg_stride + g * 16;
+        // A second pass over the same image adds the residual level of the activations when a block of this group has one.
+        uint32_t npass = 1;
+        if (__builtin_amdgcn_ballot_w64(col_valid && xs[2 * nb + dblk] != 0.0f) != 0) npass = 2;
+#pragma nounroll
+        for (uint32_t pass = 0; pass < npass; pass++) {
+        const float xscale16 = (col_valid && cl == 0) ? xs[pass * 2 * nb + dblk] * 0.0625f : 0.0f;   // high-limb columns and padding add nothing
+        const int nsum16 = col_valid ? xn[pass * 2 * nb + dblk] << 4 : 0;
+        const uint32_t my_off = col_valid ? lane_x_off + dblk * 256u + pass * (uint32_t)(kL * K) : zero_off;
 
         // accumulators by code scale: fields 0 and 1 arrive as code, field 2 as 4*code, field 3 as 16*code
         v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0}, acc16 = (v4i){0, 0, 0, 0};
@@ -268,6 +281,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
             const uint16_t dbits = *reinterpret_cast<const uint16_t*>(image + (4 * g + i) * seg_stride + (col_valid ? cb : nbg - 1) * 66 + 64);
             rowacc[i] += (float)iq16 * (lh_h2f(dbits) * xscale16);
         }
+        }   // pass
 
         if (grp + grp_step >= ngroups) {      // tile complete for this wave: sum the 16 columns of each row (4 rows per lane group)
             YT* y = static_cast<YT*>(pb.output);
@@ -319,8 +333,8 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         // six groups of blocks (12288 columns, the down projection of the wide feed-forward layers): a wave per group,
         // and twice the threads for the activation staging (f16 in and out only: the decode path's types)
         static const int six = [] { const char* e = getenv("LOCAL_HIP_TQ2_SPLIT6"); return !(e && e[0] == '0' && e[1] == 0); }();
-        const size_t lds6 = (size_t)kL * K + (size_t)nb * 8 + 128 + 6 * (size_t)kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
-        if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= 96 * 1024) split_waves = 6;
+        const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
+        if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= kMaxLdsBytes) split_waves = 6;
     }
     const uint32_t splitk = split_waves > 1 ? 1u : 0u;
     static const int wg256_tiles_per_cu = [] { const char* e = getenv("LOCAL_HIP_TQ2_WG256_TILES_PER_CU"); int n = e ? atoi(e) : 2; return n < 1 ? 1 : n; }();
@@ -328,21 +342,25 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const uint32_t waves = threads / 64;
     const uint64_t slots = splitk ? tiles : (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
     static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    const size_t lds_guess = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
+    const size_t lds_guess = lds_head_bytes(K) + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
     const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_guess);          // workgroups per CU that LDS allows
     const int wg_eff = threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu;
     const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
-    const size_t lds_bytes = (size_t)kL * K + (size_t)nb * 8 + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
-    if (split_waves == 6) {   // more than the 64 KB a kernel gets without asking
-        static bool raised = false;   // one owner thread per context
-        if (!raised) {
-            hipError_t e = hipFuncSetAttribute((const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-            if (e != hipSuccess) return lh_fail(LH_ERR_PIPELINE_CREATION, "matvec_tq2_0: %s", hipGetErrorString(e));
-            raised = true;
-        }
-    } else if (lds_bytes > 64 * 1024) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
+    const size_t lds_bytes = lds_guess;
+    if (lds_bytes > kMaxLdsBytes) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
+    const void* fn;
+    if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
+#define LH_FN(XT, YT) (splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true> : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
+    else if (xt == LH_F32 && yt == LH_F32) fn = LH_FN(float, float);
+    else if (xt == LH_F16 && yt == LH_F16) fn = LH_FN(uint16_t, uint16_t);
+    else if (xt == LH_F16 && yt == LH_F32) fn = LH_FN(uint16_t, float);
+    else fn = LH_FN(float, uint16_t);
+#undef LH_FN
+    if (lds_bytes > 64 * 1024) {   // more than the 64 KB a kernel gets without asking
+        const int rl = lh_raise_dynamic_lds(ctx, fn, kMaxLdsBytes, "matvec_tq2_0");
+        if (rl != LH_OK) return rl;
+    }
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
     single.pro = pro;

@@ -5,7 +5,9 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
+#include <vector>
 
 static thread_local char g_last_error[512] = "";
 
@@ -50,6 +52,21 @@ int lh_fail(int code, const char* fmt, ...) {
 int lh_check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s launch failed: %s", what, hipGetErrorString(e));
+    return LH_OK;
+}
+
+// hipFuncSetAttribute is per device: remember (kernel, device) pairs already raised.  One owner thread per context, but
+// contexts on different threads may race here, hence the lock.
+int lh_raise_dynamic_lds(lh_context* ctx, const void* kernel, size_t bytes, const char* op) {
+    struct Raised { const void* fn; int device; size_t bytes; };
+    static std::mutex mu;
+    static std::vector<Raised> done;
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Raised& r : done)
+        if (r.fn == kernel && r.device == ctx->device && r.bytes >= bytes) return LH_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return lh_fail(LH_ERR_PIPELINE_CREATION, "%s: %s", op, hipGetErrorString(e));
+    done.push_back(Raised{kernel, ctx->device, bytes});
     return LH_OK;
 }
 

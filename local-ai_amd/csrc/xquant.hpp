@@ -48,16 +48,44 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
     }
 }
 
+// Second level of the fixed point, for blocks whose first-level step would be too coarse.  A block with max|x| = m has
+// the step s = m / qmax; every element carries an absolute error of up to s / 2 whatever its own size, so one large
+// element (ordinary in a residual stream) costs its 255 neighbours their low bits.  While m <= kXCoarseMax the step is at
+// most 2.5e-4 (16-bit limbs) and the error of a row sum stays a few 1e-5 of the weights' scale; above it the block also
+// gets the residual r_i = x_i - s n_i in 16-bit fixed point of its own (step s * 0.52 / qmax: about 2^-31 of m in all),
+// which the kernels add in a second pass over blocks that have one (those with xs2 != 0).
+struct XResidual {
+    uint32_t* xq2;   // [2][K/4] residual limbs, laid out like xq (written for blocks with a second level only)
+    float* xs2;      // [K/G] residual scale; 0 for a block whose first level suffices
+    int* xn2;        // [K/G] sum of the residual integers (may be null)
+};
+constexpr float kXCoarseMax = 8.0f;
+
+__device__ __forceinline__ uint32_t lh_group_max_u(uint32_t v, int width) {
+    if (width > 1) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR1>((int)v));
+    if (width > 2) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR2>((int)v));
+    if (width > 4) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_HALF_MIRROR>((int)v));
+    if (width > 8) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_ROW_MIRROR>((int)v));
+    if (width > 16) v = max(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x1F | (16 << 10)));
+    if (width > 32) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+    return v;
+}
+
 // ---- activation quantisation into LDS ----------------------------------------
 // xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
 // xs[K/G]: float scale of each group of G elements (G = weight block size).
 // `xn` (optional) receives sum(n_i) per group; `nthreads` = workgroup size (multiple of 64).
+// A group that holds a NaN or an infinity gets the scale NaN, so every row sum that includes it comes out NaN (the
+// reference's f32 dot gives NaN or an infinity there; nothing is silently clamped).
+// `resid` (optional, L == 2 only): see XResidual.
 template <int L, int G, typename XT>
 __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs, int* xn,
-                                                  uint32_t nthreads, const XPrologue pro = XPrologue{kXProNone, nullptr, 0.0f}) {
+                                                  uint32_t nthreads, const XPrologue pro = XPrologue{kXProNone, nullptr, 0.0f},
+                                                  const XResidual* resid = nullptr) {
     const int tid = threadIdx.x;
     const uint32_t kq = K >> 2;
     float rms = 1.0f, rms2 = 1.0f;
+
     if constexpr (sizeof(XT) == 2) {
         if (pro.kind == kXProRmsNorm) {   // uniform over the workgroup; xs doubles as the reduction scratch before it is filled
             auto block_total = [&](float s) {
@@ -141,11 +169,16 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                 }
             }
         }
-        float m = 0.0f;
+        // the maximum over the bit patterns of |v|: the order of non-negative floats, with NaN and infinity on top
+        uint32_t mbits = 0u;
 #pragma unroll
-        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-        m = lh_group_max(m, G / 8);
-        const float inv = m > 0.0f ? Limb<L>::qmax / m : 0.0f;
+        for (int i = 0; i < 8; i++) mbits = max(mbits, __builtin_bit_cast(uint32_t, fabsf(v[i])));
+        mbits = lh_group_max_u(mbits, G / 8);
+        const bool finite = mbits < 0x7F800000u;
+        const float m = __builtin_bit_cast(float, mbits);
+        const float inv = (finite && m > 0.0f) ? Limb<L>::qmax / m : 0.0f;
+        const float sc = finite ? m * (1.0f / Limb<L>::qmax) : __builtin_nanf("");
+        int nq[8];
         uint32_t packed[L][2];
         int nsum = 0;
 #pragma unroll
@@ -155,6 +188,7 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
             float r = rintf(v[i] * inv);
             r = fminf(fmaxf(r, -Limb<L>::qmax), Limb<L>::qmax);
             int n = (int)r;
+            nq[i] = n;
             nsum += n;
 #pragma unroll
             for (int l = 0; l < L; l++) {
@@ -168,11 +202,43 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
 #pragma unroll
             for (int l = 0; l < L; l++)
                 *reinterpret_cast<uint2*>(&xq[l * kq + (e0 >> 2)]) = make_uint2(packed[l][0], packed[l][1]);
-            if ((e0 & (G - 1)) == 0) xs[e0 / G] = m * (1.0f / Limb<L>::qmax);
+            if ((e0 & (G - 1)) == 0) xs[e0 / G] = sc;
         }
         if (xn != nullptr) {
             nsum = lh_group_sum_i(nsum, G / 8);
             if (valid && (e0 & (G - 1)) == 0) xn[e0 / G] = nsum;
+        }
+        if constexpr (L == 2) {
+            if (resid != nullptr) {
+                const bool coarse = finite && m > kXCoarseMax;       // uniform over the lanes of a group
+                const float sc2 = sc * (0.52f / Limb<2>::qmax);       // |r| <= 0.5 sc up to rounding: 0.52 leaves headroom
+                int nsum2 = 0;
+                if (__builtin_amdgcn_ballot_w64(coarse) != 0) {      // rare: skipped by waves without such a block
+                    const float inv2 = coarse ? 1.0f / sc2 : 0.0f;
+                    uint32_t p2[2][2] = {{0u, 0u}, {0u, 0u}};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float rr = __builtin_fmaf(-(float)nq[i], sc, v[i]);
+                        float q2 = rintf(rr * inv2);
+                        q2 = fminf(fmaxf(q2, -Limb<2>::qmax), Limb<2>::qmax);
+                        int n2 = (int)q2;
+                        nsum2 += n2;
+                        const int lo = (int)(int8_t)(n2 & 0xFF);
+                        const int hi = (n2 - lo) >> 8;
+                        p2[0][i >> 2] |= (uint32_t)(lo & 0xFF) << (8 * (i & 3));
+                        p2[1][i >> 2] |= (uint32_t)(hi & 0xFF) << (8 * (i & 3));
+                    }
+                    if (valid && coarse) {
+                        *reinterpret_cast<uint2*>(&resid->xq2[e0 >> 2]) = make_uint2(p2[0][0], p2[0][1]);
+                        *reinterpret_cast<uint2*>(&resid->xq2[kq + (e0 >> 2)]) = make_uint2(p2[1][0], p2[1][1]);
+                    }
+                    if (resid->xn2 != nullptr) nsum2 = lh_group_sum_i(nsum2, G / 8);
+                }
+                if (valid && (e0 & (G - 1)) == 0) {
+                    resid->xs2[e0 / G] = coarse ? sc2 : 0.0f;
+                    if (resid->xn2 != nullptr) resid->xn2[e0 / G] = coarse ? nsum2 : 0;
+                }
+            }
         }
     }
 }

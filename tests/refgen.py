@@ -68,3 +68,21 @@ def assert_close(got, want, tol, label=""):
     i = int(np.argmax(err))
     assert err[i] <= tol, f"{label}[{i}]: got {got[i]}, want {want[i]} (norm err {err[i]:.3e} > {tol})"
     return float(err[i])
+
+
+def scaled_error(got, want):
+    """max |g - w| / max |w|: the error relative to the output's own scale (no floor of 1)."""
+    got = np.asarray(got, np.float64).reshape(-1)
+    want = np.asarray(want, np.float64).reshape(-1)
+    return float(np.max(np.abs(got - want)) / max(float(np.max(np.abs(want))), 1e-30))
+
+
+def assert_close_both(got, want, tol, label=""):
+    """Both gates: the reference's |g - w| <= tol * max(|w|, 1) per element, and the scale-aware
+    max|g - w| <= tol * max|w| (which does not loosen when the outputs are smaller than 1).
+    Returns (normalised error, scale-aware error) and prints them."""
+    e_norm = assert_close(got, want, tol, label)
+    e_scaled = scaled_error(got, want)
+    print(f"{label}: err/max(|w|,1) {e_norm:.2e}, err/max|w| {e_scaled:.2e}")
+    assert e_scaled <= tol, f"{label}: max|g-w| / max|w| = {e_scaled:.3e} > {tol}"
+    return e_norm, e_scaled

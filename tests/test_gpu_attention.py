@@ -230,6 +230,33 @@ def test_split_invariance_at_32k(pkg, gpu, oracle):
     check(out.as_array(np.float32), ref, "SWA ring 512")
 
 
+@pytest.mark.parametrize("T", [16384, 131072])
+@pytest.mark.parametrize("qscale", [1.0, 0.15])
+def test_context_sweep_long(pkg, gpu, oracle, T, qscale):
+    """The long ends of the measured context sweep (8 q heads / 1 kv head, hd 256, 2 bits, one query, full attention):
+    a peaked distribution (q from N(0, 1)) and a soft one (q * 0.15, thousands of positions carry weight, which is what
+    stresses the fixed-point value weights and their lazily moved reference).  Rotated-space output against the f64
+    code-space oracle, and the rotated-back f16 output of the one-call entry."""
+    print(f"case T={T} qscale={qscale}", flush=True)
+    ctx, K = gpu
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, T + 3)
+    q = (pkg.synth.rng(6, 21).standard_normal((nq, hd), dtype=np.float32) * qscale).astype(np.float16)
+    rq = oracle.hadamard_rotate(q.astype(np.float32), signs, hd, nq, True, False)
+    kcb, knb, vcb, vnb, lvb, rqb, sgb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, signs)
+    out, out2 = pkg.Buffer.empty(ctx, nq * hd * 4), pkg.Buffer.empty(ctx, nq * hd * 4)
+    o16 = pkg.Buffer.empty(ctx, nq * hd * 2)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    K.flash_attention_tq_rotated_into(batch, rqb, kcb, knb, vcb, vnb, lvb, sgb, out2, o16, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    ref = oracle.attention_tq_codespace(rq, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    e = check(out.as_array(np.float32), ref, f"T={T} rotated space")
+    back = oracle.hadamard_rotate(np.asarray(ref, np.float32).reshape(nq, hd), signs, hd, nq, False, True)
+    e2 = check(o16.as_array(np.float16).astype(np.float32), np.asarray(back, np.float32).reshape(-1), f"T={T} output", 3e-3)
+    print(f"  T={T} qscale={qscale}: err rotated {e:.2e}, f16 output {e2:.2e}")
+
+
 @pytest.mark.parametrize("hd,T,window,ring", [(256, 700, 512, 512), (256, 40, 0, 0), (256, 1500, 0, 0), (512, 900, 0, 0),
                                               (256, 9000, 0, 0), (256, 3, 0, 0), (128, 300, 0, 0)])
 def test_rotated_entry_equals_attention_then_rotation(pkg, gpu, oracle, hd, T, window, ring):

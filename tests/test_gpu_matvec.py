@@ -55,7 +55,7 @@ def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
     x = pkg.synth.activations(1, cols, g)[0]
     want = oracle.matvec_quant_ref(fmt, raw, x, rows, cols, threads=8)
     got = run_matvec(pkg, gpu, fmt, raw, x, rows, cols, pkg.F32, pkg.F32)
-    err = refgen.assert_close(got, want, 1e-3, fmt)
+    err, _ = refgen.assert_close_both(got, want, 1e-3, f"{fmt} {rows}x{cols}")
     # attribution: against an f64 accumulation of the unrounded weights the error is far smaller
     expand = oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32
     y64 = oracle.matvec_f64(expand(raw, rows, cols), x)
@@ -82,7 +82,8 @@ def test_matvec_rejects_misaligned_cols(pkg, gpu):
 
 def test_matvec_linearity_and_grouped(pkg, gpu, oracle):
     """Size-independent properties at full size: y(ax) = a y(x) for a power of two (exact in
-    block fixed point), and a grouped launch equals the separate launches bit for bit."""
+    block fixed point while no block changes its number of levels), and a grouped launch equals
+    the separate launches bit for bit."""
     ctx, kernels = gpu
     rows, cols = 8192, 2048
     g = pkg.synth.rng(2, 7)
@@ -101,11 +102,18 @@ def test_matvec_linearity_and_grouped(pkg, gpu, oracle):
         a, b = yb[i].as_array(np.float32, rows), yg[i].as_array(np.float32, rows)
         assert np.array_equal(a, b)
         refgen.assert_close(a, oracle.matvec_quant_ref("tq2_0", raws[i], xs[i], rows, cols, threads=8), 1e-3)
-    x2 = pkg.Buffer.from_slice(ctx, xs[0] * np.float32(4.0))
+    # a power-of-two factor that keeps every block's maximum under the threshold of the residual level: bit-exact
+    x2 = pkg.Buffer.from_slice(ctx, xs[0] * np.float32(0.25))
     y2 = pkg.Buffer.empty(ctx, rows * 4)
     ws[0].matvec_typed_into(batch, kernels, x2, pkg.F32, y2, pkg.F32)
     batch.commit_and_wait()
-    assert np.array_equal(y2.as_array(np.float32, rows), yb[0].as_array(np.float32, rows) * np.float32(4.0))
+    assert np.array_equal(y2.as_array(np.float32, rows), yb[0].as_array(np.float32, rows) * np.float32(0.25))
+    # one that crosses it (blocks with a maximum above 8 get the second level): the same product, more finely
+    x3 = pkg.Buffer.from_slice(ctx, xs[0] * np.float32(16.0))
+    ws[0].matvec_typed_into(batch, kernels, x3, pkg.F32, y2, pkg.F32)
+    batch.commit_and_wait()
+    refgen.assert_close_both(y2.as_array(np.float32, rows),
+                             oracle.matvec_quant_ref("tq2_0", raws[0], xs[0] * np.float32(16.0), rows, cols, threads=8), 2e-4, "16 x")
 
 
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
@@ -191,3 +199,101 @@ def test_matvec_norm_chain(pkg, gpu, oracle, fmt, rows, cols, count, second_norm
         refgen.assert_close(outs[i].as_array(np.float16, rows).astype(np.float32), want, 2e-3, f"{fmt} norm chain #{i}")
     with pytest.raises(pkg.InvalidArgument):     # the stored vector may not alias an input
         K.matvec_quant_norm_chain_into(pkg.CommandBatch(ctx), ty, [ws[0].buf], xb, w1b, rb, None, xb, 1e-6, [outs[0]], rows, cols)
+
+
+@pytest.mark.parametrize("rows,cols", [(5, 256), (6, 512), (37, 1536), (2048, 2048), (1023, 6144)])
+def test_matvec_tq2_0_soa(pkg, gpu, oracle, rows, cols):
+    """kernels.rs:5919-5971 / matvec_quant.metal:322-387: the split layout -- qs[(row * blocks + b) * 64] and
+    scales[row * blocks + b] -- gives what the interleaved blocks give.  Reference payloads (codes include 3), f16 x
+    and f16 y as the reference's pipeline has them; rows not a multiple of the four rows a workgroup takes."""
+    print(f"case soa {rows}x{cols}", flush=True)
+    ctx, K = gpu
+    raw = refgen.tq2_0_payload(rows, cols, 0xC0DE).reshape(-1, 66)
+    qs = np.ascontiguousarray(raw[:, :64]).reshape(-1)
+    scales = np.ascontiguousarray(raw[:, 64:]).reshape(-1).view(np.uint16)
+    v16, v32 = refgen.test_vector(cols)
+    want = oracle.matvec_f32(oracle.expand_tq2_0_f32(raw.reshape(-1), rows, cols), v32)
+    qb, sb, xb = (pkg.Buffer.from_slice(ctx, a) for a in (qs, scales, v16))
+    yb = pkg.Buffer.from_slice(ctx, np.full(rows + 8, 0x7BFF, np.uint16))
+    batch = pkg.CommandBatch(ctx)
+    K.matvec_tq2_0_soa_into(batch, qb, sb, xb, yb, rows, cols)
+    assert batch.dispatch_count() == 1
+    batch.commit_and_wait()
+    got = yb.as_array(np.uint16, rows + 8)
+    assert (got[rows:] == 0x7BFF).all(), "rows past the end were written"
+    refgen.assert_close(got[:rows].view(np.float16).astype(np.float32), want, 2e-3, "soa f16out")   # reference: 0.02
+    # and the same bits as the interleaved kernel would round to, up to the summation order: compare with it too
+    inter = run_matvec(pkg, gpu, "tq2_0", raw.reshape(-1), v16, rows, cols, pkg.F16, pkg.F16)
+    refgen.assert_close(got[:rows].view(np.float16).astype(np.float32), inter, 2e-3, "soa vs interleaved")
+    with pytest.raises(pkg.InvalidArgument, match=r"matvec_tq2_0_soa: cols 128 not /256"):
+        K.matvec_tq2_0_soa_into(batch, qb, sb, xb, yb, rows, 128)
+
+
+def heavy_tailed(kind, cols, g):
+    x = g.standard_normal(cols, dtype=np.float32)
+    if kind == "outliers_1pct":          # N(0, 1) with one entry in a hundred 300 times larger
+        idx = g.choice(cols, max(1, cols // 100), replace=False)
+        x[idx] *= np.float32(300.0)
+    elif kind == "one_per_block":        # every 32-column block carries one entry of 1e3 .. 1e4 sigma
+        for b in range(cols // 32):
+            x[b * 32 + int(g.integers(0, 32))] *= np.float32(10.0 ** g.uniform(3.0, 4.0))
+    elif kind == "lonely_element":       # one 256-column block is zero but for a single element
+        x[256:512] = 0.0
+        x[300] = np.float32(7.5)
+    elif kind == "f16_near_max":         # magnitudes at the top of the f16 range beside ordinary ones
+        x[::97] = np.float32(60000.0) * np.sign(x[::97])
+    elif kind == "tiny":                 # everything far below 1: the scale-aware gate is the one that bites
+        x *= np.float32(1e-4)
+    return x
+
+
+@pytest.mark.parametrize("kind", ["outliers_1pct", "one_per_block", "lonely_element", "f16_near_max", "tiny"])
+@pytest.mark.parametrize("fmt,rows,cols", [("q4_0", 2048, 2048), ("tq2_0", 8192, 2048), ("tq2_0", 2048, 8192),
+                                           ("tq2_0", 100, 24576), ("q4_0", 300, 16384)])
+def test_matvec_heavy_tailed_activations(pkg, gpu, oracle, fmt, rows, cols, kind):
+    """Activations with outliers (ordinary in a residual stream) at the measured shapes, fp32 and f16 x, against
+    the reference CPU path (block dequant to f16, sequential f32 dot).  The kernels quantise x to block fixed point;
+    blocks whose step would be too coarse get a second, residual level, which this test pins.  Three gates:
+    (1) scale-aware, against the reference path: max|g - w| <= 1e-3 max|w|;
+    (2) the reference's own form |g - w| <= 1e-3 max(|w|, 1), widened by the reference path's distance from the
+        exactly accumulated (f64) product of the block values before their f16 rounding -- with activations in the
+        hundreds and more, the f16 rounding of the Q4_0 weights and the f32 left-to-right sum put the reference path
+        itself several 1e-3 from that product in this form, and no fused kernel can follow either rounding;
+    (3) the kernel's own accuracy: within 1e-3, same form, of that exact product (this is the gate that fails when
+        a coarse block is left without its residual level)."""
+    print(f"case {fmt} {rows}x{cols} {kind}", flush=True)
+    g = pkg.synth.rng(41, rows + cols)
+    raw = pkg.synth.weights(fmt, rows, cols, g)
+    x = heavy_tailed(kind, cols, g)
+    unrounded = (oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32)(raw, rows, cols)
+
+    def norm_err(a, b):
+        return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), 1.0)))
+
+    for xdt in (pkg.F32, pkg.F16):
+        xin = x if xdt == pkg.F32 else x.astype(np.float16).astype(np.float32)
+        label = f"{fmt} {rows}x{cols} {kind} x={'f32' if xdt == pkg.F32 else 'f16'}"
+        want = oracle.matvec_quant_ref(fmt, raw, xin, rows, cols, threads=8)
+        exact = oracle.matvec_f64(unrounded, xin)
+        floor = norm_err(exact, want)            # every form below is normalised by max(|reference path|, 1)
+        got = run_matvec(pkg, gpu, fmt, raw, xin, rows, cols, xdt, pkg.F32)
+        e_scaled, e_norm = refgen.scaled_error(got, want), norm_err(got, want)
+        e_own = float(np.max(np.abs(got - exact) / np.maximum(np.abs(want), 1.0)))
+        print(f"{label}: err/max|w| {e_scaled:.2e}, err/max(|w|,1) {e_norm:.2e} (reference path vs exact product: "
+              f"{floor:.2e}), kernel vs exact product {e_own:.2e}")
+        assert e_scaled <= 1e-3, label
+        assert e_norm <= 1e-3 + floor, label
+        assert e_own <= 1e-3, label
+
+
+@pytest.mark.parametrize("fmt,rows,cols", [("q4_0", 70, 2048), ("tq2_0", 70, 2048), ("tq2_0", 20, 16384)])
+def test_matvec_non_finite_activations_propagate(pkg, gpu, oracle, fmt, rows, cols):
+    """A NaN or an infinity in x reaches every output row as a non-finite value, as it does in the reference's
+    f32 dot (0 * inf = NaN, so a row whose weight at that column is zero is NaN too), instead of being clamped."""
+    g = pkg.synth.rng(42, rows + cols)
+    raw = pkg.synth.weights(fmt, rows, cols, g)
+    for bad in (np.float32(np.nan), np.float32(np.inf), np.float32(-np.inf)):
+        x = g.standard_normal(cols, dtype=np.float32)
+        x[cols // 2 + 3] = bad
+        got = run_matvec(pkg, gpu, fmt, raw, x, rows, cols, pkg.F32, pkg.F32)
+        assert not np.isfinite(got).any(), f"{fmt}: {int(np.isfinite(got).sum())} of {rows} rows stayed finite with x = {bad}"
