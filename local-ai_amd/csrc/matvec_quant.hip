@@ -205,8 +205,21 @@ template <int FMT> __host__ __device__ constexpr int steps_in_flight(int npos) {
     return FMT == LH_TQ2_0 ? (npos == 1 ? 8 : (npos == 2 ? 4 : 2)) : (npos == 1 ? 4 : (npos == 2 ? 2 : 1));
 }
 
+// Staged form (IMG, Q4_0 only): the rows of a wave's step are consecutive in memory, so the step is fetched as one
+// contiguous run of 16-byte chunks -- consecutive lanes, consecutive chunks, every byte requested once, one step ahead in
+// registers -- parked in a wave-private LDS image, and each lane reads its 36-byte units back from there (dword reads at a
+// 9-dword lane stride: conflict free).  Fetching the units straight from global memory makes every lane's three loads share
+// cache lines with its neighbours' and triples the address work of the memory pipeline.
+constexpr int kImgLoads = 9;                                   // a step is at most 9216 bytes = 576 chunks
+constexpr uint32_t kImgBytes = kImgLoads * 1024 + 64;          // per wave
+
+__device__ __forceinline__ u32x4_t ld16_stream(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(4))) u32x4_a4;
+    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4_a4*>(p));
+}
+
 // One launch serves `count` problems of the same shape (count == 1 for the plain matvec).
-template <int FMT, int L, int NPOS, typename XT, typename YT>
+template <int FMT, int L, int NPOS, typename XT, typename YT, bool IMG = false>
 __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProblem* __restrict__ problems, MatvecBase single,
                                                              uint32_t count, uint32_t rows, uint32_t K, uint32_t lpr_log2,
                                                              uint32_t steps_per_wg) {
@@ -220,6 +233,9 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
     float* xs2 = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(xq2) + (size_t)2 * K);
     const XResidual resid{xq2, xs2, nullptr};
     bool any_coarse = false;   // a lane of this wave owns a unit column with a residual level
+    // the staged form's wave-private image sits behind the activation area (which ends with xs2 when L == 2)
+    const size_t x_area = (size_t)L * K + (size_t)(K / G) * 4 + (L == 2 ? (size_t)2 * K + (size_t)(K / G) * 4 + 16 : 0);
+    uint8_t* image = lds + ((x_area + 15) & ~(size_t)15) + (size_t)(threadIdx.x >> 6) * kImgBytes;
 
     const uint32_t upr = K >> 6;                                  // unit columns per row
     const uint32_t row_bytes = FMT == LH_TQ2_0 ? (K >> 8) * 66 : (K >> 5) * 18;
@@ -290,7 +306,57 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         const int red_width = NPOS == 1 ? (int)lpr : 64;
         const bool writer = NPOS == 1 ? (((uint32_t)lane & (lpr - 1)) == 0) : lane == 0;
 
+        // ---- staged form: chunk c = lane + 64 i of the step's contiguous bytes
+        [[maybe_unused]] u32x4_t pre[kImgLoads];
+        [[maybe_unused]] const uint32_t step_bytes = U * rpw * row_bytes;
+        [[maybe_unused]] const uint32_t step_chunks = (step_bytes + 15) >> 4;
+        [[maybe_unused]] const size_t mat_bytes = (size_t)rows * row_bytes;   // chunks past the matrix read its first slack bytes (never used)
+        [[maybe_unused]] auto prefetch = [&](uint32_t st_) {
+            const size_t base = (size_t)st_ * rpw * row_bytes;
+#pragma unroll
+            for (int i = 0; i < kImgLoads; i++) {
+                // no branch around a load (a conditionally loaded register forces a wait right behind the load):
+                // surplus lanes repeat the step's last chunk, which is never parked
+                uint32_t c = lane + 64 * i;
+                c = c < step_chunks ? c : step_chunks - 1;
+                size_t off = base + (size_t)c * 16;
+                off = off < mat_bytes ? off : mat_bytes;
+                pre[i] = ld16_stream(mat + off);
+            }
+        };
+        if constexpr (IMG) { if (st < st_end) prefetch(st); }
+
         for (; st < st_end; st += U) {
+            float part[U];
+            if constexpr (IMG) {
+                __builtin_amdgcn_wave_barrier();      // the units of the previous step have been read
+#pragma unroll
+                for (int i = 0; i < kImgLoads; i++)
+                    if ((uint32_t)lane + 64 * i < step_chunks) *reinterpret_cast<u32x4_t*>(image + ((uint32_t)lane + 64 * i) * 16) = pre[i];
+                __builtin_amdgcn_wave_barrier();
+                if (st + U < st_end) prefetch(st + U);
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    part[u] = 0.0f;
+#pragma unroll
+                    for (int p = 0; p < NPOS; p++) {
+                        const uint32_t ucol = col0 + 64u * p;
+                        UnitW<FMT> w;
+                        const uint32_t* src = reinterpret_cast<const uint32_t*>(image + ((uint32_t)u * rpw + rsub) * row_bytes + (ucol < upr ? ucol : 0u) * 36);
+                        w.a = make_uint4(src[0], src[1], src[2], src[3]);
+                        w.b = make_uint4(src[4], src[5], src[6], src[7]);
+                        w.c = src[8];
+                        part[u] += unit_dot<FMT, L>(w, ux[p]);
+                        if constexpr (L == 2) {
+                            if (any_coarse && ucol < upr) {   // rare: the residual level of this unit column, read from LDS
+                                UnitX<FMT, 2> ur;
+                                load_unit_x<FMT, 2>(ur, ucol, K, xq2, xs2);
+                                part[u] += unit_dot<FMT, 2>(w, ur);
+                            }
+                        }
+                    }
+                }
+            } else {
             UnitW<FMT> w[U][NPOS];
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -303,7 +369,6 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                     load_unit_w<FMT>(w[u][p], rp, ucol < upr ? ucol : 0u);
                 }
             }
-            float part[U];
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 part[u] = 0.0f;
@@ -324,6 +389,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                     }
                 }
             }
+            }   // !IMG
             // butterfly over the lanes of a row, all U rows per level
             if (red_width > 1) {
 #pragma unroll
@@ -459,9 +525,16 @@ int wg_per_cu() {
 struct LaunchGeom {
     uint32_t npos, lpr_log2, rpw, grid, steps_per_wg;
     size_t lds_bytes;
+    bool img;   // staged form: Q4_0 with two limbs and at least 16 readable bytes behind every matrix
 };
 
-LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_count, int L) {
+// LOCAL_HIP_Q4_IMAGE=0 keeps the Q4_0 kernel on direct per-lane loads.
+bool q4_image_enabled() {
+    static bool v = [] { const char* e = getenv("LOCAL_HIP_Q4_IMAGE"); return !(e && e[0] == '0' && e[1] == 0); }();
+    return v;
+}
+
+LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_count, int L, size_t min_slack = 0) {
     LaunchGeom g{};
     const uint32_t upr = K / 64;
     g.npos = (upr + 63) / 64;
@@ -479,26 +552,38 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
     g.grid = (uint32_t)((steps + g.steps_per_wg - 1) / g.steps_per_wg);
     const uint32_t G = fmt == LH_TQ2_0 ? 256 : 32;
     g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4 + (L == 2 ? (size_t)2 * K + (size_t)(K / G) * 4 + 16 : 0);
+    // the staged form pays off once a wave walks several steps (its first fetch is not overlapped with anything)
+    const uint32_t in_flight = g.npos == 1 ? 4u : (g.npos == 2 ? 2u : 1u);        // steps_in_flight<LH_Q4_0>(npos)
+    g.img = fmt == LH_Q4_0 && L == 2 && min_slack >= 16 && g.steps_per_wg >= 2u * kWaves * in_flight && q4_image_enabled();
+    if (g.img) g.lds_bytes = ((g.lds_bytes + 15) & ~(size_t)15) + (size_t)kWaves * kImgBytes;
     return g;
 }
 
 template <int FMT, int L, int NPOS>
 int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const MatvecBase& single, uint32_t count, lh_dtype xt,
                  lh_dtype yt, uint32_t rows, uint32_t K, const LaunchGeom& g) {
-#define LH_LAUNCH(XT, YT)                                                                                                   \
+#define LH_LAUNCH_K(KERNEL)                                                                                                 \
     do {                                                                                                                    \
         if (g.lds_bytes > 64 * 1024) {   /* long rows: more than the 64 KB a kernel gets without asking */                  \
-            const int rl = lh_raise_dynamic_lds(ctx, (const void*)matvec_quant_kernel<FMT, L, NPOS, XT, YT>, 96 * 1024, "matvec_quant"); \
+            const int rl = lh_raise_dynamic_lds(ctx, (const void*)KERNEL, 96 * 1024, "matvec_quant");                       \
             if (rl != LH_OK) return rl;                                                                                     \
         }                                                                                                                   \
-        hipLaunchKernelGGL((matvec_quant_kernel<FMT, L, NPOS, XT, YT>), dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream,  \
+        hipLaunchKernelGGL(KERNEL, dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream,                                       \
                            dev_problems, single, count, rows, K, g.lpr_log2, g.steps_per_wg);                               \
+    } while (0)
+#define LH_LAUNCH(XT, YT)                                                                                                   \
+    do {                                                                                                                    \
+        if constexpr (FMT == LH_Q4_0 && L == 2) {                                                                           \
+            if (g.img) LH_LAUNCH_K((matvec_quant_kernel<FMT, L, NPOS, XT, YT, true>));                                      \
+            else LH_LAUNCH_K((matvec_quant_kernel<FMT, L, NPOS, XT, YT, false>));                                           \
+        } else LH_LAUNCH_K((matvec_quant_kernel<FMT, L, NPOS, XT, YT, false>));                                             \
     } while (0)
     if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
     else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
     else LH_LAUNCH(float, uint16_t);
 #undef LH_LAUNCH
+#undef LH_LAUNCH_K
     return lh_check_launch("matvec_quant");
 }
 
@@ -608,7 +693,7 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
     }
     const int L = x_limbs();
-    const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L);
+    const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L, min_slack);
     int r;
     if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
                                    : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
@@ -653,7 +738,7 @@ int matvec_rows_impl(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer*
     } else {
         MatvecBase single{MatvecProblem{(const uint8_t*)weight->ptr, input->ptr, output->ptr}, (uint32_t)xstride, (uint32_t)ystride};
         const int L = x_limbs();
-        const LaunchGeom g = plan(fmt, m, n, k, ctx->cu_count, L);
+        const LaunchGeom g = plan(fmt, m, n, k, ctx->cu_count, L, slack);
         if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
                                        : launch_npos<LH_Q4_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
         else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)

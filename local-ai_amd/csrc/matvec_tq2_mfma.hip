@@ -77,7 +77,7 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
 }
 
 template <typename XT, typename YT, bool SPLITK, int MAXT = 256>
-__global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
+__global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
     constexpr bool splitk = SPLITK;
     extern __shared__ __align__(16) uint8_t lds[];
