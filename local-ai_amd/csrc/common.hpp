@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stddef.h>
 #include <atomic>
+#include <vector>
 #include "../../include/local_hip.h"
 
 struct lh_context {
@@ -21,8 +22,17 @@ struct lh_context {
     // True between lh_batch_begin_capture and lh_batch_end_capture: dispatches are recorded into a graph instead
     // of running, and calls that would wait, allocate, copy from host memory or record a memset are refused.
     bool capturing;
-    void* deferred_free[64];    // owning buffers released during a capture: freed when the capture ends
-    int deferred_count;
+    // Owning buffers released while a capture is open.  A recorded dispatch may reference them, so they live as long as
+    // the graph the capture produces (lh_graph_free releases them); when the capture fails they go when it ends.
+    std::vector<void*> deferred_free;
+    // Pinned staging for descriptor tables of grouped launches: a small ring of slots, each guarded by an event that is
+    // recorded behind the slot's copy, so a slot is rewritten only after the copy that read it has run.
+    static constexpr int kDescSlots = 4;
+    static constexpr size_t kDescSlotBytes = 64 * 1024;
+    void* desc_pinned;
+    hipEvent_t desc_event[kDescSlots];
+    bool desc_used[kDescSlots];
+    unsigned desc_next;
 };
 
 struct lh_buffer {
@@ -120,6 +130,11 @@ void lh_launch_gelu_mul_strided(hipStream_t stream, const void* a, const float* 
 void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count);   // gelu_mul_into's kernel
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
 int lh_launch_hadamard_fh(lh_context* ctx, const float* input, const float* signs, uint16_t* output, uint32_t head_dim, uint32_t num_heads);
+
+// Stream-ordered copy of a host-built descriptor table to device memory.  The host block may be freed as soon as this
+// returns (it has been copied into pinned staging; tables larger than a staging slot are copied synchronously after a
+// stream wait).  Not available while a graph is being captured.
+int lh_upload_descriptors(lh_context* ctx, const void* host, size_t bytes, void* device_dst, const char* op);
 
 // Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncAttributeMaxDynamicSharedMemorySize), once per kernel and device.
 int lh_raise_dynamic_lds(lh_context* ctx, const void* kernel, size_t bytes, const char* op);

@@ -688,9 +688,9 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
             host_desc[i].output = outputs[i]->ptr;
         }
         dev_desc = (MatvecProblem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
-        hipError_t e = hipMemcpyAsync(dev_desc, host_desc, desc_bytes, hipMemcpyHostToDevice, ctx->stream);
-        free(host_desc);   // pageable source: the runtime has staged it when the call returns
-        if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
+        const int ru = lh_upload_descriptors(ctx, host_desc, desc_bytes, dev_desc, op);
+        free(host_desc);   // staged by the helper
+        if (ru != LH_OK) return ru;
     }
     const int L = x_limbs();
     const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L, min_slack);

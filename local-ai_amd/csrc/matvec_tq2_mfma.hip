@@ -35,14 +35,20 @@ constexpr int kL = 2;                        // activation limbs (16-bit block f
 constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
 constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
-constexpr size_t kMaxLdsBytes = 128 * 1024;   // most dynamic LDS a launch here asks for (a CU has 160 KB)
+constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
 // Bytes of the activation area at the head of the dynamic LDS: two limb planes for each of the two fixed-point levels,
-// four per-block arrays (scale and integer sum of either level), padded to 16 bytes.
-__host__ __device__ constexpr size_t lds_head_bytes(uint32_t K) { return (size_t)2 * kL * K + (size_t)(K >> 8) * 16 + 16; }
+// four per-block arrays (scale and integer sum of either level), padded so that the 128-byte zero line behind it starts
+// 64 bytes into a 256-byte line.  The limb planes of a level are K + 16 bytes apart and the zero line sits on banks of its
+// own: the lanes of one B-operand read (low limb, high limb, zeros) then never meet on an LDS bank.
+__host__ __device__ constexpr uint32_t plane_bytes(uint32_t K) { return K + 16; }
+__host__ __device__ constexpr size_t lds_head_bytes(uint32_t K) {
+    const size_t raw = (size_t)2 * kL * plane_bytes(K) + (size_t)(K >> 8) * 16;
+    return ((raw + 255 - 64) & ~(size_t)255) + 64;
+}
 
 struct Tq2Problem {
     const uint8_t* matrix;
@@ -77,18 +83,18 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
 }
 
 template <typename XT, typename YT, bool SPLITK, int MAXT = 256>
-__global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
+__global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
     constexpr bool splitk = SPLITK;
     extern __shared__ __align__(16) uint8_t lds[];
     const uint32_t nb = K >> 8;                                     // blocks per row
     // [xq: 2 x K/4 limb words][xq2: the same for the residual level][xs nb][xn nb][xs2 nb][xn2 nb][pad]
     uint32_t* xq = reinterpret_cast<uint32_t*>(lds);                // [2][K/4] activation limbs
-    uint32_t* xq2 = reinterpret_cast<uint32_t*>(lds + (size_t)kL * K);
-    float* xs = reinterpret_cast<float*>(lds + (size_t)2 * kL * K); // [nb] activation scales
+    uint32_t* xq2 = reinterpret_cast<uint32_t*>(lds + (size_t)kL * plane_bytes(K));
+    float* xs = reinterpret_cast<float*>(lds + (size_t)2 * kL * plane_bytes(K)); // [nb] activation scales
     int* xn = reinterpret_cast<int*>(xs + nb);                      // [nb] sum of the block's integers
     const XResidual resid{xq2, xs + 2 * nb, xn + 2 * nb};
-    const uint32_t kq = K >> 2;
+    const uint32_t kq = plane_bytes(K) >> 2;                        // dwords between the low-limb and the high-limb plane
     const uint32_t row_bytes = nb * 66;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const uint32_t r = lane & 15, g = lane >> 4;                    // A layout: row r, quarter g
@@ -116,20 +122,21 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
     // offsets live in registers and the image offsets are linear in the chunk index.  The trailing group of nb % 8
     // blocks: both tables live in LDS (one per workgroup), read back when such a group comes up.
     const uint32_t nbg_tail = (nb & 7) ? (nb & 7) : 8;
-    uint32_t goff_full[kStageLoads];
-    uint32_t* tail_tab = reinterpret_cast<uint32_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [2][kStageLoads][64]
-    {
+    // (all three tables live in LDS, one copy per workgroup, read back when a tile's loads are issued: the nine offsets
+    // of a full group in registers cost the third wave per SIMD)
+    // (16-bit entries: row offsets stay below 15 * 3168 + 528 bytes for the widest row this kernel takes)
+    uint16_t* tail_tab = reinterpret_cast<uint16_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [3][kStageLoads][64]
+    uint16_t* full_tab = tail_tab + 2 * kStageLoads * 64;
+    if (wave == 0) {
         const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
 #pragma unroll
         for (int i = 0; i < kStageLoads; i++) {
             const uint32_t ch = lane + 64 * i;
             const uint32_t cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
-            goff_full[i] = rf * row_bytes + jf * 16;
-            if (wave == 0) {
-                const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
-                tail_tab[i * 64 + lane] = rt * row_bytes + jt * 16;
-                tail_tab[(kStageLoads + i) * 64 + lane] = ch < 16 * nch_t ? rt * ss_t + jt * 16 : 0xFFFFFFFFu;   // surplus lanes do not store
-            }
+            full_tab[i * 64 + lane] = (uint16_t)(rf * row_bytes + jf * 16);
+            const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
+            tail_tab[i * 64 + lane] = (uint16_t)(rt * row_bytes + jt * 16);
+            tail_tab[(kStageLoads + i) * 64 + lane] = ch < 16 * nch_t ? (uint16_t)(rt * ss_t + jt * 16) : (uint16_t)0xFFFFu;   // surplus lanes do not store
         }
     }
     __syncthreads();
@@ -157,7 +164,10 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
     Item cur{grp0, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
 
     u32x4_t pre[kStageLoads];
-    auto prefetch = [&](const Item& it) {
+    // `offs`: the lane's nine chunk offsets of a full group, read from full_tab by the caller ahead of the call (at the top of
+    // a loop iteration, so that the LDS round trip hides behind the wait for the previous tile's loads; keeping them in
+    // registers for the whole loop costs the third wave per SIMD)
+    auto prefetch = [&](const Item& it, const uint32_t (&offs)[kStageLoads]) {
         uint32_t grp, tile; Tq2Problem pb;
         item_tile_base(it, grp, tile, pb);
         const bool tail = grp + 1 == ngroups && (nb & 7);
@@ -165,7 +175,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
             gptr_t base = (gptr_t)pb.matrix + (size_t)(tile << 4) * row_bytes + (size_t)grp * 528;
             if (!tail) {
 #pragma unroll
-                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + goff_full[i]);
+                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + offs[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + tail_tab[i * 64 + lane]);
@@ -186,7 +196,12 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
         }
     };
 
-    if (nitems) prefetch(cur);
+    {
+        uint32_t offs[kStageLoads];
+#pragma unroll
+        for (int i = 0; i < kStageLoads; i++) offs[i] = full_tab[i * 64 + lane];
+        if (nitems) prefetch(cur, offs);
+    }
     const void* staged = nullptr;
     float rowacc[4] = {0.f, 0.f, 0.f, 0.f};
     for (uint64_t n = 0; n < nitems; n++) {
@@ -195,7 +210,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
         const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
-            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro, &resid);
+            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro, &resid, kq);
             __syncthreads();
             staged = pb.vector;
         }
@@ -206,6 +221,9 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
         (void)nch;
 
         // ---- park the prefetched chunks in the wave's LDS image, then start the next item's loads
+        uint32_t offs[kStageLoads];
+#pragma unroll
+        for (int i = 0; i < kStageLoads; i++) offs[i] = full_tab[i * 64 + lane];
         __builtin_amdgcn_wave_barrier();
         if (nbg == 8) {
 #pragma unroll
@@ -216,11 +234,11 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
 #pragma unroll
             for (int i = 0; i < kStageLoads; i++) {
                 const uint32_t lo = tail_tab[(kStageLoads + i) * 64 + lane];
-                if (lo != 0xFFFFFFFFu) *reinterpret_cast<u32x4_t*>(image + lo) = pre[i];
+                if (lo != 0xFFFFu) *reinterpret_cast<u32x4_t*>(image + lo) = pre[i];
             }
         }
         __builtin_amdgcn_wave_barrier();
-        if (n + 1 < nitems) prefetch(nxt);
+        if (n + 1 < nitems) prefetch(nxt, offs);
         cur = nxt;
 
         // ---- column constants of this group
@@ -234,7 +252,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
         for (uint32_t pass = 0; pass < npass; pass++) {
         const float xscale16 = (col_valid && cl == 0) ? xs[pass * 2 * nb + dblk] * 0.0625f : 0.0f;   // high-limb columns and padding add nothing
         const int nsum16 = col_valid ? xn[pass * 2 * nb + dblk] << 4 : 0;
-        const uint32_t my_off = col_valid ? lane_x_off + dblk * 256u + pass * (uint32_t)(kL * K) : zero_off;
+        const uint32_t my_off = col_valid ? lane_x_off + dblk * 256u + pass * (uint32_t)(kL * plane_bytes(K)) : zero_off;
 
         // accumulators by code scale: fields 0 and 1 arrive as code, field 2 as 4*code, field 3 as 16*code
         v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0}, acc16 = (v4i){0, 0, 0, 0};
@@ -285,7 +303,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 3 : 1) void matvec_tq2_mfma_ker
 
         if (grp + grp_step >= ngroups) {      // tile complete for this wave: sum the 16 columns of each row (4 rows per lane group)
             YT* y = static_cast<YT*>(pb.output);
-            float* part = reinterpret_cast<float*>(tail_tab + 2 * kStageLoads * 64);   // [nwaves][16] partial rows (splitk)
+            float* part = reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64);   // [nwaves][16] partial rows (splitk); 4-byte aligned: 3456 bytes of tables
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float v = rowacc[i];
@@ -328,30 +346,42 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     // quantised activation vector; few tiles with long rows: the block groups of a tile are split over 2-4 waves
     const uint32_t ngroups = (nb + 7) >> 3;
     uint32_t split_waves = 1;
-    if (tiles < (uint64_t)ctx->cu_count * 2) {
+    static const int force_split = [] { const char* e = getenv("LOCAL_HIP_TQ2_FORCE_SPLIT"); return e ? atoi(e) : 0; }();
+    if (tiles < (uint64_t)ctx->cu_count * 2 || (force_split && ngroups > 1)) {
         for (uint32_t w = 4; w >= 2; w--) if (ngroups % w == 0) { split_waves = w; break; }
         // six groups of blocks (12288 columns, the down projection of the wide feed-forward layers): a wave per group,
         // and twice the threads for the activation staging (f16 in and out only: the decode path's types)
         static const int six = [] { const char* e = getenv("LOCAL_HIP_TQ2_SPLIT6"); return !(e && e[0] == '0' && e[1] == 0); }();
-        const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
+        const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 3 * kStageLoads * 64 * 2 + 12 * 16 * 4;
         if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= kMaxLdsBytes) split_waves = 6;
     }
     const uint32_t splitk = split_waves > 1 ? 1u : 0u;
     static const int wg256_tiles_per_cu = [] { const char* e = getenv("LOCAL_HIP_TQ2_WG256_TILES_PER_CU"); int n = e ? atoi(e) : 2; return n < 1 ? 1 : n; }();
-    const uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * wg256_tiles_per_cu ? 256 : 64);
+    static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
+    auto lds_for = [&](uint32_t nwaves) { return lds_head_bytes(K) + 128 + (size_t)nwaves * kImageBytes + 3 * kStageLoads * 64 * 2 + 12 * 16 * 4; };
+    uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * wg256_tiles_per_cu ? 256 : 64);
+    // Long rows make the activation area large: when fewer than three four-wave workgroups fit a CU's LDS, a large job runs
+    // one twelve-wave workgroup per CU instead, which stages the activations once and keeps three waves on every SIMD
+    // (LOCAL_HIP_TQ2_WIDE=0 keeps four-wave workgroups).
+    static const int wide_on = [] { const char* e = getenv("LOCAL_HIP_TQ2_WIDE"); return !(e && e[0] == '0' && e[1] == 0); }();
+    bool wide = false;
+    if (!splitk && threads == 256 && wide_on && (160 * 1024) / lds_for(4) < 3 && lds_for(12) <= kMaxLdsBytes &&
+        tiles >= (uint64_t)ctx->cu_count * 24) {
+        wide = true;
+        threads = 768;
+    }
     const uint32_t waves = threads / 64;
     const uint64_t slots = splitk ? tiles : (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
-    static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    const size_t lds_guess = lds_head_bytes(K) + 128 + (size_t)waves * kImageBytes + 2 * kStageLoads * 64 * 4 + 8 * 16 * 4;
-    const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_guess);          // workgroups per CU that LDS allows
-    const int wg_eff = threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu;
+    const size_t lds_bytes = lds_for(waves);
+    const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_bytes);          // workgroups per CU that LDS allows
+    const int wg_eff = wide ? 1 : (threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu);
     const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
-    const size_t lds_bytes = lds_guess;
     if (lds_bytes > kMaxLdsBytes) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
     const void* fn;
     if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
-#define LH_FN(XT, YT) (splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true> : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
+#define LH_FN(XT, YT) (wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                             \
+                            : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true> : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
     else if (xt == LH_F32 && yt == LH_F32) fn = LH_FN(float, float);
     else if (xt == LH_F16 && yt == LH_F16) fn = LH_FN(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) fn = LH_FN(uint16_t, float);
@@ -376,21 +406,13 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         if (!host) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", bytes);
         for (uint32_t i = 0; i < count; i++) host[i] = Tq2Problem{(const uint8_t*)matrices[i], vectors[i], outputs[i]};
         dev = (Tq2Problem*)((char*)ctx->workspace + ctx->workspace_bytes - ctx->workspace_bytes / 4);
-        hipError_t e = hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream);
-        free(host);
-        if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: descriptor upload: %s", hipGetErrorString(e));
+        const int ru = lh_upload_descriptors(ctx, host, bytes, dev, "matvec_tq2_0");
+        free(host);   // staged by the helper
+        if (ru != LH_OK) return ru;
     }
-#define LH_LAUNCH(XT, YT)                                                                                                          \
-    do {                                                                                                                           \
-        if (splitk) hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, true>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
-        else hipLaunchKernelGGL((matvec_tq2_mfma_kernel<XT, YT, false>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K); \
-    } while (0)
-    if (split_waves == 6)
-        hipLaunchKernelGGL((matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>), dim3(grid), dim3(threads), lds_bytes, ctx->stream, dev, single, count, rows, K);
-    else if (xt == LH_F32 && yt == LH_F32) LH_LAUNCH(float, float);
-    else if (xt == LH_F16 && yt == LH_F16) LH_LAUNCH(uint16_t, uint16_t);
-    else if (xt == LH_F16 && yt == LH_F32) LH_LAUNCH(uint16_t, float);
-    else LH_LAUNCH(float, uint16_t);
-#undef LH_LAUNCH
+    const Tq2Problem* dev_arg = dev;
+    void* args[] = {(void*)&dev_arg, (void*)&single, (void*)&count, (void*)&rows, (void*)&K};
+    hipError_t le = hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, ctx->stream);
+    if (le != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0 launch failed: %s", hipGetErrorString(le));
     return lh_check_launch("matvec_tq2_0");
 }

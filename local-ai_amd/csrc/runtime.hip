@@ -70,6 +70,29 @@ int lh_raise_dynamic_lds(lh_context* ctx, const void* kernel, size_t bytes, cons
     return LH_OK;
 }
 
+int lh_upload_descriptors(lh_context* ctx, const void* host, size_t bytes, void* device_dst, const char* op) {
+    if (ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: a descriptor upload cannot be recorded into a graph", op);
+    if (bytes == 0) return LH_OK;
+    hipError_t e;
+    if (bytes <= lh_context::kDescSlotBytes) {
+        const unsigned slot = ctx->desc_next++ % lh_context::kDescSlots;
+        if (ctx->desc_used[slot]) {   // the copy that last read this slot must have run (it has, but for a very deep queue)
+            e = hipEventSynchronize(ctx->desc_event[slot]);
+            if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor staging: %s", op, hipGetErrorString(e));
+        }
+        void* stage = static_cast<char*>(ctx->desc_pinned) + (size_t)slot * lh_context::kDescSlotBytes;
+        memcpy(stage, host, bytes);
+        e = hipMemcpyAsync(device_dst, stage, bytes, hipMemcpyHostToDevice, ctx->stream);
+        if (e == hipSuccess) e = hipEventRecord(ctx->desc_event[slot], ctx->stream);
+        ctx->desc_used[slot] = true;
+    } else {   // larger than a slot: wait for the kernels that still read the previous table, then a blocking copy
+        e = hipStreamSynchronize(ctx->stream);
+        if (e == hipSuccess) e = hipMemcpy(device_dst, host, bytes, hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s: descriptor upload: %s", op, hipGetErrorString(e));
+    return LH_OK;
+}
+
 extern "C" {
 
 const char* lh_last_error(void) { return g_last_error; }
@@ -82,6 +105,8 @@ static void ctx_release(lh_context* ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->workspace);
+    for (int i = 0; i < lh_context::kDescSlots; i++) (void)hipEventDestroy(ctx->desc_event[i]);
+    (void)hipHostFree(ctx->desc_pinned);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -106,7 +131,8 @@ int lh_context_create(int device_index, lh_context** out) {
     ctx->device = device_index;
     ctx->refs.store(1, std::memory_order_relaxed);
     ctx->capturing = false;
-    ctx->deferred_count = 0;
+    ctx->desc_pinned = nullptr;
+    ctx->desc_next = 0;
     ctx->cu_count = prop.multiProcessorCount;
     snprintf(ctx->name, sizeof ctx->name, "%s (%s)", prop.name, prop.gcnArchName);
     if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
@@ -118,6 +144,23 @@ int lh_context_create(int device_index, lh_context** out) {
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;
         return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: attention workspace", (size_t)64 << 20);
+    }
+    if (hipHostMalloc(&ctx->desc_pinned, lh_context::kDescSlots * lh_context::kDescSlotBytes, hipHostMallocDefault) != hipSuccess) {
+        (void)hipFree(ctx->workspace);
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: pinned descriptor staging", lh_context::kDescSlots * lh_context::kDescSlotBytes);
+    }
+    for (int i = 0; i < lh_context::kDescSlots; i++) {
+        ctx->desc_used[i] = false;
+        if (hipEventCreateWithFlags(&ctx->desc_event[i], hipEventDisableTiming) != hipSuccess) {
+            for (int j = 0; j < i; j++) (void)hipEventDestroy(ctx->desc_event[j]);
+            (void)hipHostFree(ctx->desc_pinned);
+            (void)hipFree(ctx->workspace);
+            (void)hipStreamDestroy(ctx->stream);
+            delete ctx;
+            return lh_fail(LH_ERR_NO_COMMAND_QUEUE, "hipEventCreate");
+        }
     }
     *out = ctx;
     return LH_OK;
@@ -243,12 +286,12 @@ void lh_buffer_free(lh_buffer* buf) {
     if (!buf) return;
     if (buf->owns && buf->ptr) {
         lh_context* ctx = buf->ctx;
-        if (ctx->capturing && ctx->deferred_count < 64) {
-            ctx->deferred_free[ctx->deferred_count++] = buf->ptr;   // neither a wait nor a free may happen inside a capture
-        } else if (!ctx->capturing) {
+        if (ctx->capturing) {
+            ctx->deferred_free.push_back(buf->ptr);   // neither a wait nor a free may happen inside a capture
+        } else {
             (void)hipStreamSynchronize(ctx->stream);
             (void)hipFree(buf->ptr);
-        }   // (a 65th release inside one capture leaks its allocation rather than break the capture)
+        }
     }
     ctx_release(buf->ctx);
     delete buf;
@@ -349,7 +392,10 @@ int lh_batch_submit_and_renew(lh_batch* batch) {
 int lh_batch_commit_and_renew(lh_batch* batch) { return lh_batch_commit_and_wait(batch); }
 
 // ---- recorded batches ----------------------------------------------------------
-struct lh_graph { lh_context* ctx; hipGraph_t graph; hipGraphExec_t exec; uint32_t dispatch_count; };
+struct lh_graph {
+    lh_context* ctx; hipGraph_t graph; hipGraphExec_t exec; uint32_t dispatch_count;
+    std::vector<void*> owned;   // allocations released while the graph was recorded: its dispatches may still use them
+};
 
 int lh_batch_begin_capture(lh_batch* batch) {
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "begin_capture: batch is null");
@@ -370,25 +416,31 @@ int lh_batch_end_capture(lh_batch* batch, lh_graph** out) {
     ctx->capturing = false;
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
-    if (ctx->deferred_count) {
+    std::vector<void*> released;
+    released.swap(ctx->deferred_free);
+    auto drop_released = [&]() {   // no graph will replay: nothing can reference them once the stream is idle
+        if (released.empty()) return;
         (void)hipStreamSynchronize(ctx->stream);
-        for (int i = 0; i < ctx->deferred_count; i++) (void)hipFree(ctx->deferred_free[i]);
-        ctx->deferred_count = 0;
-    }
-    if (e != hipSuccess || !graph) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: end_capture: %s", hipGetErrorString(e));
+        for (void* p : released) (void)hipFree(p);
+        released.clear();
+    };
+    if (e != hipSuccess || !graph) { drop_released(); return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: end_capture: %s", hipGetErrorString(e)); }
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
         (void)hipGraphDestroy(graph);
+        drop_released();
         return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: graph instantiation: %s", hipGetErrorString(e));
     }
     lh_graph* g = new (std::nothrow) lh_graph();
     if (!g) {
         (void)hipGraphExecDestroy(exec);
         (void)hipGraphDestroy(graph);
+        drop_released();
         return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(lh_graph));
     }
     g->ctx = ctx; g->graph = graph; g->exec = exec; g->dispatch_count = batch->dispatch_count;
+    g->owned.swap(released);
     ctx_retain(ctx);
     batch->dispatch_count = 0;
     *out = g;
@@ -410,6 +462,7 @@ void lh_graph_free(lh_graph* graph) {
     (void)hipStreamSynchronize(graph->ctx->stream);   // a replay may still be running
     (void)hipGraphExecDestroy(graph->exec);
     (void)hipGraphDestroy(graph->graph);
+    for (void* p : graph->owned) (void)hipFree(p);
     ctx_release(graph->ctx);
     delete graph;
 }

@@ -77,13 +77,13 @@ __device__ __forceinline__ uint32_t lh_group_max_u(uint32_t v, int width) {
 // `xn` (optional) receives sum(n_i) per group; `nthreads` = workgroup size (multiple of 64).
 // A group that holds a NaN or an infinity gets the scale NaN, so every row sum that includes it comes out NaN (the
 // reference's f32 dot gives NaN or an infinity there; nothing is silently clamped).
-// `resid` (optional, L == 2 only): see XResidual.
+// `resid` (optional, L == 2 only): see XResidual.  `plane_dwords` (optional): distance of the limb planes in dwords.
 template <int L, int G, typename XT>
 __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint32_t K, uint32_t* xq, float* xs, int* xn,
                                                   uint32_t nthreads, const XPrologue pro = XPrologue{kXProNone, nullptr, 0.0f},
-                                                  const XResidual* resid = nullptr) {
+                                                  const XResidual* resid = nullptr, uint32_t plane_dwords = 0) {
     const int tid = threadIdx.x;
-    const uint32_t kq = K >> 2;
+    const uint32_t kq = plane_dwords ? plane_dwords : K >> 2;   // dwords between the limb planes (K / 4 unless the caller pads them)
     float rms = 1.0f, rms2 = 1.0f;
 
     if constexpr (sizeof(XT) == 2) {
