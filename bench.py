@@ -35,10 +35,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/matvec_tq2_mfma_grouped_8192x2048.md), scaled by the same counters on the library's plain
-# copy kernel; None until that profile has been taken for the current kernel.
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by
+# the same counters on the library's plain copy kernel.  A run of bench.py cannot read hardware counters itself: the
+# figure is carried over from the profile named beside it (`roofline.traffic_source`), taken with the current kernel.
 MEASURED_TRAFFIC_BYTES = 1088685363
+TRAFFIC_SOURCE = "profiles/matvec_tq2_mfma_grouped_8192x2048.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; carried over, not measured by this run)"
 
 
 def log(*a):
@@ -189,8 +190,19 @@ def make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits):
     return pool, levels, signs
 
 
-def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64, hd=256):
+def lanes_for_one_gib(T, hd, nkv=1, bits=2):
+    """Independent sequences whose caches together exceed 1 GiB (and so the 256 MB last-level cache, several times)."""
+    per_seq = T * nkv * (2 * (hd * bits // 8) + 4)
+    n = -(-(1 << 30) // per_seq)
+    return -(-n // 32) * 32          # a multiple of 32, so that the workgroups of a launch fill whole CUs
+
+
+def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=None, hd=256):
+    """`lanes` independent sequences of T cached positions in one batched launch (default: as many as make the caches
+    exceed 1 GiB, so that the figure is an HBM figure), and single decode tokens rotating over those sequences."""
     nq, nkv, bits = 8, 1, 2
+    if lanes is None:
+        lanes = lanes_for_one_gib(T, hd, nkv, bits)
     pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, T, hd, nkv, bits)
     g = pkg.synth.rng(5, 1)
     q = g.standard_normal((lanes, nq, hd), dtype=np.float32).astype(np.float16)
@@ -210,17 +222,18 @@ def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=64, hd=256):
     _, ev_b = time_steps(pkg, ctx, step_batched, steps, warmup)
     cb = hd * bits // 8
     views = [[pool[0].view(l * T * nkv * cb, T * nkv * cb), pool[1].view(l * T * nkv * 2, T * nkv * 2),
-              pool[2].view(l * T * nkv * cb, T * nkv * cb), pool[3].view(l * T * nkv * 2, T * nkv * 2)] for l in range(lanes)]
+              pool[2].view(l * T * nkv * cb, T * nkv * cb), pool[3].view(l * T * nkv * 2, T * nkv * 2)]
+             for l in range(0, lanes, max(1, lanes // 256))]   # at most ~256 sequences, spread over the pool
     it = [0]
     calls = [bound_call(pkg.lib().lh_flash_attention_tq_into, batch, rq, v[0], v[1], v[2], v[3], levels, out, hd, T, T - 1, nq, nkv,
                         0, bits, 0) for v in views]
 
     def step_single():   # one decode token of one sequence; sequences rotate so the cache comes from HBM
-        calls[it[0] % lanes]()
+        calls[it[0] % len(calls)]()
         it[0] += 1
 
     _, ev_s = time_steps(pkg, ctx, step_single, max(steps, 20), warmup)
-    return {"context": T, "bytes_per_position": per_pos,
+    return {"context": T, "bytes_per_position": per_pos, "cache_bytes": lanes * T * per_pos,
             "batched_lanes": lanes, "batched_us_per_launch": ev_b * 1e3,
             "batched_tokens_per_s": lanes / (ev_b * 1e-3), "batched_gbs": lanes * T * per_pos / ev_b * 1e-6,
             "single_us_per_token": ev_s * 1e3, "single_tokens_per_s": 1.0 / (ev_s * 1e-3),
@@ -233,14 +246,16 @@ def bench_attention_sweep(pkg, ctx, K, steps, warmup):
     hd, nq, nkv, bits = 256, 8, 1, 2
     per_pos = nkv * (2 * (hd * bits // 8) + 4)
     res = {}
-    for T, lanes in ((4096, 64), (16384, 32), (131072, 8)):
-        r = bench_attention(pkg, ctx, K, steps, warmup, T=T, lanes=lanes)
-        res[f"ctx_{T}"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"],
-                           "batched_lanes": lanes, "batched_us_per_launch": r["batched_us_per_launch"], "batched_gbs": r["batched_gbs"]}
+    for T in (4096, 16384, 131072):          # every point over more than 1 GiB of distinct caches
+        r = bench_attention(pkg, ctx, K, steps, warmup, T=T)
+        res[f"ctx_{T}"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"], "cache_bytes": r["cache_bytes"],
+                           "batched_lanes": r["batched_lanes"], "batched_us_per_launch": r["batched_us_per_launch"],
+                           "batched_gbs": r["batched_gbs"], "batched_frac_of_hbm_peak": r["batched_gbs"] / HBM_PEAK_GBS}
     # the reference model's full-attention layers: head_dim 512 (260 bytes per position)
-    r = bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=32, hd=512)
-    res["ctx_32768_head_dim_512"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"],
-                                     "batched_lanes": 32, "batched_us_per_launch": r["batched_us_per_launch"], "batched_gbs": r["batched_gbs"]}
+    r = bench_attention(pkg, ctx, K, steps, warmup, T=32768, hd=512)
+    res["ctx_32768_head_dim_512"] = {"single_us_per_token": r["single_us_per_token"], "single_gbs": r["single_gbs"], "cache_bytes": r["cache_bytes"],
+                                     "batched_lanes": r["batched_lanes"], "batched_us_per_launch": r["batched_us_per_launch"],
+                                     "batched_gbs": r["batched_gbs"], "batched_frac_of_hbm_peak": r["batched_gbs"] / HBM_PEAK_GBS}
     # sliding window: every lane is a 512-slot ring; logical position far beyond the ring size
     ring, lanes, pos = 512, 4096, 100000
     pool, levels, signs = make_kv_pool(pkg, ctx, K, lanes, ring, hd, nkv, bits)
@@ -793,7 +808,7 @@ def main():
                    "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS,
                    "settle_ms_before_warmup": SETTLE_MS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
                      "launch_ms": head["ms_per_launch_events"]},
         "cpu_baseline": cpu,

@@ -90,7 +90,9 @@ struct AttnShared {
 
 // NPL = number of bit planes: 2 when the level table is affine in the code bits, 3 with the bit0*bit1 plane.
 // HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
-template <int NPL, int HD>
+// ONE_KV: a single KV head (the measured configuration and the reference model): the distance between positions is a
+// compile-time constant, so the loads of a group take immediate offsets instead of per-load address arithmetic.
+template <int NPL, int HD, bool ONE_KV>
 __device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256)>& sh, float alpha, float beta,
                                                float gam, float delta) {
     auto& s_rqop = sh.rqop;
@@ -119,8 +121,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     const bool any = c_hi > c_lo;
     const uint32_t g_first = c_lo >> 6, g_last = any ? (c_hi - 1) >> 6 : 0u;
 
-    const uint32_t stride = p.num_kv_heads * kCodeBytes;          // bytes between positions
-    const uint32_t nstride = p.num_kv_heads * 2;
+    const uint32_t stride = ONE_KV ? (uint32_t)kCodeBytes : p.num_kv_heads * kCodeBytes;   // bytes between positions
+    const uint32_t nstride = ONE_KV ? 2u : p.num_kv_heads * 2;
     auto geom = [&](uint32_t G) {
         GroupGeom gg;
         const uint32_t gstart = G << 6;
@@ -591,8 +593,9 @@ __global__ __launch_bounds__(64 + HD / 4, OCC) void attention_tq_mfma_kernel(Att
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
-    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
-    else attention_body<2, HD>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD, false>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, HD, true>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, HD, false>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
