@@ -67,6 +67,10 @@ struct Tq2Base {
     XPrologue pro = {kXProNone, nullptr, 0.0f};   // applied to every problem's vector while it is staged
 };
 
+__device__ __forceinline__ u32x4_t ld16_align2_cached(gptr_t p) {
+    typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
+    return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p);
+}
 __device__ __forceinline__ u32x4_t ld16_align2(gptr_t p) {
     typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
     // weights are read once per launch: a streaming load keeps them from displacing the activations in the caches
@@ -82,7 +86,12 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
     for (int m = 0; m < 4; m++) out[m] = rem ? __builtin_amdgcn_alignbit(in[m + q + 1], in[m + q], 8 * rem) : in[m + q];
 }
 
-template <typename XT, typename YT, bool SPLITK, int MAXT = 256>
+// STREAM: the weight loads carry the non-temporal hint.  Right when a tile's bytes are one contiguous run (one block group
+// per row: every cache line is used once, by one instruction).  With several groups per row a tile is sixteen 528-byte
+// segments whose first and last cache lines are shared with the neighbouring segment, read by the same wave an item
+// later: the hint evicts those lines early and they are fetched a second time (measured: 1.19 x the bytes), so such
+// launches use plain loads.
+template <typename XT, typename YT, bool SPLITK, int MAXT = 256, bool STREAM = false>
 __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
     constexpr bool splitk = SPLITK;
@@ -175,7 +184,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
             gptr_t base = (gptr_t)pb.matrix + (size_t)(tile << 4) * row_bytes + (size_t)grp * 528;
             if (!tail) {
 #pragma unroll
-                for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + offs[i]);
+                for (int i = 0; i < kStageLoads; i++) pre[i] = STREAM ? ld16_align2(base + offs[i]) : ld16_align2_cached(base + offs[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < kStageLoads; i++) pre[i] = ld16_align2(base + tail_tab[i * 64 + lane]);
@@ -381,7 +390,9 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const void* fn;
     if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
 #define LH_FN(XT, YT) (wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                             \
-                            : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true> : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
+                            : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true>                                          \
+                            : ngroups == 1 ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 256, true>                        \
+                                           : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
     else if (xt == LH_F32 && yt == LH_F32) fn = LH_FN(float, float);
     else if (xt == LH_F16 && yt == LH_F16) fn = LH_FN(uint16_t, uint16_t);
     else if (xt == LH_F16 && yt == LH_F32) fn = LH_FN(uint16_t, float);

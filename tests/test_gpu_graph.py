@@ -99,3 +99,32 @@ def test_capture_refuses_what_a_graph_cannot_hold(pkg, gpu):
     assert (buf.as_array(np.float16, 64) == 2.0).all()
     graph.free()
     assert pkg.Buffer.empty(ctx, 16).length() == 16       # the context is usable again
+
+
+def test_buffer_released_during_capture_lives_as_long_as_the_graph(pkg, gpu):
+    """A scratch buffer that a recorded dispatch writes and a later one reads is released by its owner while the
+    capture is still open (as a Rust scope would drop it).  The graph keeps the allocation: several replays, with
+    other allocations made in between (which would reuse a freed block), still give the right sums."""
+    ctx, K = gpu
+    n = 4096
+    a = pkg.Buffer.from_slice(ctx, np.full(n, 1.5, np.float16))
+    b = pkg.Buffer.from_slice(ctx, np.full(n, 2.0, np.float16))
+    out = pkg.Buffer.empty(ctx, n * 2)
+    scratch = pkg.Buffer.empty(ctx, n * 2)          # created before the capture: allocation is refused inside one
+    batch = pkg.CommandBatch(ctx)
+    batch.begin_capture()
+    K.residual_add_into(batch, a, b, scratch, n)          # scratch = a + b
+    K.residual_add_into(batch, scratch, b, out, n)        # out = scratch + b
+    scratch.free()                                         # dropped while the capture is open
+    graph = batch.end_capture()
+    filler = []
+    for step in range(4):
+        # allocations of the same size between replays: a block freed too early would be handed out here and overwritten
+        filler.append(pkg.Buffer.from_slice(ctx, np.full(n, 100.0 + step, np.float16)))
+        a.copy_from_bytes(np.full(n, 1.5 + step, np.float16))
+        out.fill_zero()
+        graph.launch()
+        ctx.synchronize()
+        got = out.as_array(np.float16, n).astype(np.float32)
+        assert (got == 1.5 + step + 4.0).all(), f"replay {step}: {got[:4]}"
+    graph.free()
