@@ -35,6 +35,9 @@ constexpr int kL = 2;                        // activation limbs (16-bit block f
 constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
 constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
+constexpr uint32_t kRing = 4;                 // tiles the waves of a split workgroup may drift apart
+constexpr uint32_t kMaxSplitWaves = 6;        // most waves that share the block groups of a tile
+constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxSplitWaves * 16 * 4 + 2 * kRing * 4;   // partial rows + arrival / generation words
 constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
@@ -112,6 +115,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     const uint32_t lane_x_off = 4u * (cl * kq + (g >> 1) * 32u + (g & 1) * 4u);
     const uint32_t zero_off = (uint32_t)lds_head_bytes(K);                      // 128 bytes of zeros behind the activation area
     if (threadIdx.x < 32) reinterpret_cast<uint32_t*>(lds + zero_off)[threadIdx.x] = 0;
+    uint32_t slot_seq = 0;                                                      // tiles this wave has completed (split form)
     uint8_t* image = lds + zero_off + 128 + (size_t)wave * kImageBytes;         // this wave's tile image
 
     // Work order: "slots" of nwaves consecutive tiles, dealt round-robin to the workgroups, so that at any moment
@@ -136,6 +140,8 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     // (16-bit entries: row offsets stay below 15 * 3168 + 528 bytes for the widest row this kernel takes)
     uint16_t* tail_tab = reinterpret_cast<uint16_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [3][kStageLoads][64]
     uint16_t* full_tab = tail_tab + 2 * kStageLoads * 64;
+    if (splitk && threadIdx.x < 2 * kRing)   // arrival counts and generations of the partial-sum ring
+        reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxSplitWaves * 16)[threadIdx.x] = 0u;
     if (wave == 0) {
         const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
 #pragma unroll
@@ -312,7 +318,8 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
 
         if (grp + grp_step >= ngroups) {      // tile complete for this wave: sum the 16 columns of each row (4 rows per lane group)
             YT* y = static_cast<YT*>(pb.output);
-            float* part = reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64);   // [nwaves][16] partial rows (splitk); 4-byte aligned: 3456 bytes of tables
+            float* part = reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64);   // [kRing][nwaves][16] partial rows (splitk); 4-byte aligned: 3456 bytes of tables
+            float parts[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float v = rowacc[i];
@@ -323,20 +330,47 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
                 const uint32_t orow = (tile << 4) + 4 * g + i;
                 if (!splitk) {
                     if (c == 0 && tile < tiles_per_problem && orow < rows) lh_store_from_f32<YT>(y, orow, v);
-                } else if (c == 0) {
-                    part[wave * 16 + 4 * g + i] = v;
                 }
+                parts[i] = v;
                 rowacc[i] = 0.0f;
             }
-            if (splitk) {   // every wave of the workgroup reaches this point once per slot
-                __syncthreads();
-                if (wave == 0 && lane < 16) {
-                    float v = part[lane];
-                    for (int w = 1; w < nwaves; w++) v += part[w * 16 + lane];
-                    const uint32_t orow = (tile << 4) + lane;
-                    if (orow < rows) lh_store_from_f32<YT>(y, orow, v);
+            if (splitk) {
+                // Every wave of the workgroup reaches this point once per slot, in the same slot order, but not in step:
+                // a wave parks its sixteen partial rows in a ring slot and counts itself in; whichever wave arrives last
+                // sums the partials in wave order (so the result does not depend on the order of arrival), stores the
+                // rows and opens the ring slot for its next use.  No workgroup barrier: the waves drift by up to kRing - 1
+                // tiles, which keeps their loads (the block groups of the same rows) close together in time without
+                // making them wait for each other.
+                uint32_t* sync = reinterpret_cast<uint32_t*>(part + kRing * kMaxSplitWaves * 16);   // arrivals[kRing], generation[kRing]
+                const uint32_t ring = slot_seq % kRing, gen = slot_seq / kRing;
+                if (gen) {   // the slot's previous use must have been summed (bounded wait: never expected to run out)
+                    uint32_t spins = 0;
+                    while (__hip_atomic_load(&sync[kRing + ring], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != gen && spins++ < (1u << 20))
+                        __builtin_amdgcn_s_sleep(2);
                 }
-                __syncthreads();
+                if (c == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) part[(ring * nwaves + wave) * 16 + 4 * g + i] = parts[i];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                uint32_t arrived = 0;
+                if (lane == 0) arrived = __hip_atomic_fetch_add(&sync[ring], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+                arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
+                if (arrived == (uint32_t)nwaves - 1u) {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    if (lane < 16) {
+                        float v = part[(ring * nwaves) * 16 + lane];
+                        for (int w = 1; w < nwaves; w++) v += part[(ring * nwaves + w) * 16 + lane];
+                        const uint32_t orow = (tile << 4) + lane;
+                        if (orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    if (lane == 0) {
+                        __hip_atomic_store(&sync[ring], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        __hip_atomic_store(&sync[kRing + ring], gen + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+                }
+                slot_seq++;
             }
         }
     }
@@ -361,13 +395,13 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         // six groups of blocks (12288 columns, the down projection of the wide feed-forward layers): a wave per group,
         // and twice the threads for the activation staging (f16 in and out only: the decode path's types)
         static const int six = [] { const char* e = getenv("LOCAL_HIP_TQ2_SPLIT6"); return !(e && e[0] == '0' && e[1] == 0); }();
-        const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 3 * kStageLoads * 64 * 2 + 12 * 16 * 4;
+        const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 3 * kStageLoads * 64 * 2 + kSplitAreaBytes;
         if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= kMaxLdsBytes) split_waves = 6;
     }
     const uint32_t splitk = split_waves > 1 ? 1u : 0u;
     static const int wg256_tiles_per_cu = [] { const char* e = getenv("LOCAL_HIP_TQ2_WG256_TILES_PER_CU"); int n = e ? atoi(e) : 2; return n < 1 ? 1 : n; }();
     static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
-    auto lds_for = [&](uint32_t nwaves) { return lds_head_bytes(K) + 128 + (size_t)nwaves * kImageBytes + 3 * kStageLoads * 64 * 2 + 12 * 16 * 4; };
+    auto lds_for = [&](uint32_t nwaves) { return lds_head_bytes(K) + 128 + (size_t)nwaves * kImageBytes + 3 * kStageLoads * 64 * 2 + kSplitAreaBytes; };
     uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * wg256_tiles_per_cu ? 256 : 64);
     // Long rows make the activation area large: when fewer than three four-wave workgroups fit a CU's LDS, a large job runs
     // one twelve-wave workgroup per CU instead, which stages the activations once and keeps three waves on every SIMD
