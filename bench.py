@@ -809,7 +809,7 @@ def main():
                    "settle_ms_before_warmup": SETTLE_MS},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
-                     "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
+                     "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256, true>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
                      "launch_ms": head["ms_per_launch_events"]},
         "cpu_baseline": cpu,
         "extra": extra,

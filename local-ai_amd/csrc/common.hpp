@@ -94,11 +94,11 @@ struct XPrologue {
 };
 
 // TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.
-// With a non-zero stride only entry 0 of the arrays is used: problem i is problem 0 with its vector / output advanced by
-// i * xstride / i * ystride bytes.
+// With a non-zero stride only entry 0 of the arrays is used: problem i is problem 0 with its matrix / vector / output
+// advanced by i * mstride / i * xstride / i * ystride bytes.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
                               void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K, uint32_t xstride,
-                              uint32_t ystride, const XPrologue& pro = XPrologue{kXProNone, nullptr, 0.0f});
+                              uint32_t ystride, const XPrologue& pro = XPrologue{kXProNone, nullptr, 0.0f}, uint64_t mstride = 0);
 // The m rows of a small activation batch against one quantized matrix, as m matvecs in one launch (matvec_quant.hip).
 // Returns LH_OK, an error, or -1 when the fast kernels do not take the shape (the caller then uses its own kernel).
 int lh_matvec_rows(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer* weight, const lh_buffer* input, lh_dtype at,

@@ -39,6 +39,7 @@ struct MatvecProblem {
 struct MatvecBase {
     MatvecProblem p;
     uint32_t xstride, ystride;   // bytes
+    uint64_t mstride = 0;        // bytes between the matrices of consecutive problems (0: one matrix for all of them)
     // A pair of unrelated problems (K and V, gate and up) also travels here, so the common grouped launch
     // needs no descriptor upload ahead of it.
     MatvecProblem second = {nullptr, nullptr, nullptr};
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         const uint32_t s_end = (uint32_t)((g1 < seg_end64 ? g1 : seg_end64) - (uint64_t)prob * steps_per_problem);
         const MatvecProblem pb = problems ? problems[prob]
                                  : (single.pair && prob == 1) ? single.second
-                                          : MatvecProblem{single.p.matrix, (const char*)single.p.vector + (size_t)prob * single.xstride,
+                                          : MatvecProblem{single.p.matrix + (size_t)prob * single.mstride, (const char*)single.p.vector + (size_t)prob * single.xstride,
                                                           (char*)single.p.output + (size_t)prob * single.ystride};
         // this wave's contiguous share of [s_begin, s_end)
         const uint32_t nseg = s_end - s_begin;
@@ -654,7 +655,30 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         }
         return LH_OK;
     }
+    // Problems whose matrices, vectors and outputs are each evenly spaced (replicas or layers packed into one allocation,
+    // one shared vector) need no descriptor table: problem i is problem 0 advanced by i strides, which travels in the
+    // kernel arguments.  That saves the table's upload, which sits between two launches on the stream.
+    uint64_t mstride = 0, xstride = 0, ystride = 0;
+    bool regular = count > 2 && pro.kind == kXProNone;
+    if (regular) {
+        const char* m0 = (const char*)matrices[0]->ptr; const char* x0 = (const char*)vectors[0]->ptr; const char* y0 = (const char*)outputs[0]->ptr;
+        const char* m1 = (const char*)matrices[1]->ptr; const char* x1 = (const char*)vectors[1]->ptr; const char* y1 = (const char*)outputs[1]->ptr;
+        regular = m1 > m0 && x1 >= x0 && y1 > y0;
+        if (regular) {
+            mstride = (uint64_t)(m1 - m0); xstride = (uint64_t)(x1 - x0); ystride = (uint64_t)(y1 - y0);
+            regular = xstride <= 0xFFFFFFFFull && ystride <= 0xFFFFFFFFull && (xstride & 15) == 0 && (mstride & 3) == 0;
+            for (uint32_t i = 2; regular && i < count; i++)
+                regular = (const char*)matrices[i]->ptr == m0 + (size_t)i * mstride && (const char*)vectors[i]->ptr == x0 + (size_t)i * xstride &&
+                          (const char*)outputs[i]->ptr == y0 + (size_t)i * ystride;
+        }
+    }
     if (fmt == LH_TQ2_0 && tq2_on_matrix_cores() && cols <= 12288 && ((cols / 256) % 8 == 0 || min_slack >= 16)) {
+        if (regular) {
+            const void* pm1[1] = {matrices[0]->ptr}; const void* px1[1] = {vectors[0]->ptr}; void* py1[1] = {outputs[0]->ptr};
+            int r = lh_launch_matvec_tq2_mfma(ctx, count, pm1, px1, py1, xt, yt, rows, cols, (uint32_t)xstride, (uint32_t)ystride, pro, mstride);
+            if (r == LH_OK) batch->dispatch_count++;
+            return r;
+        }
         const void* stack_m[8]; const void* stack_x[8]; void* stack_y[8];
         const void** pm = count <= 8 ? stack_m : (const void**)malloc(sizeof(void*) * 3 * count);
         if (!pm) return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: host allocation", sizeof(void*) * 3 * (size_t)count);
@@ -675,6 +699,8 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     if (count == 2) {
         single.second = MatvecProblem{(const uint8_t*)matrices[1]->ptr, vectors[1]->ptr, outputs[1]->ptr};
         single.pair = 1;
+    } else if (regular) {
+        single.xstride = (uint32_t)xstride; single.ystride = (uint32_t)ystride; single.mstride = mstride;
     } else if (count > 2) {
         if (ctx->capturing) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: more than two grouped problems need a descriptor upload, which a captured graph cannot hold", op);
         const size_t desc_bytes = (size_t)count * sizeof(MatvecProblem);

@@ -63,6 +63,7 @@ struct Tq2Problem {
 struct Tq2Base {
     Tq2Problem p;
     uint32_t xstride, ystride;   // bytes
+    uint64_t mstride = 0;        // bytes between the matrices of consecutive problems (0: one matrix for all of them)
     // A pair of unrelated problems (gate and up) also travels here, so the common grouped launch needs no
     // descriptor upload ahead of it.
     Tq2Problem second = {nullptr, nullptr, nullptr};
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
         tile = splitk ? it.sip : it.sip * nwaves + wave;
         if (problems) pb = problems[it.prob];
         else if (single.pair && it.prob == 1) pb = single.second;
-        else pb = Tq2Problem{single.p.matrix, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
+        else pb = Tq2Problem{single.p.matrix + (size_t)it.prob * single.mstride, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
                              (char*)single.p.output + (size_t)it.prob * single.ystride};
     };
     Item cur{grp0, blockIdx.x % slots_per_problem, blockIdx.x / slots_per_problem};
@@ -381,8 +382,8 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
 // Entry used by matvec_quant.hip's dispatcher. Arrays are host arrays of device pointers.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
                               void* const* outputs, lh_dtype xt, lh_dtype yt, uint32_t rows, uint32_t K, uint32_t xstride,
-                              uint32_t ystride, const XPrologue& pro) {
-    const bool strided = xstride != 0 || ystride != 0;   // problem i = problem 0 advanced by i strides: no descriptor table
+                              uint32_t ystride, const XPrologue& pro, uint64_t mstride) {
+    const bool strided = xstride != 0 || ystride != 0 || mstride != 0;   // problem i = problem 0 advanced by i strides: no descriptor table
     const uint32_t nb = K >> 8;
     const uint64_t tiles = (uint64_t)((rows + 15) >> 4) * count;
     // small jobs: one wave per workgroup so the tiles spread over all CUs; large jobs: four waves share one
@@ -438,6 +439,7 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     }
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
+    single.mstride = mstride;
     single.pro = pro;
     Tq2Problem* dev = nullptr;
     if (count == 2 && !strided) {

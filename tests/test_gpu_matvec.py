@@ -297,3 +297,38 @@ def test_matvec_non_finite_activations_propagate(pkg, gpu, oracle, fmt, rows, co
         x[cols // 2 + 3] = bad
         got = run_matvec(pkg, gpu, fmt, raw, x, rows, cols, pkg.F32, pkg.F32)
         assert not np.isfinite(got).any(), f"{fmt}: {int(np.isfinite(got).sum())} of {rows} rows stayed finite with x = {bad}"
+
+
+@pytest.mark.parametrize("fmt,rows,cols,count", [("tq2_0", 512, 2048, 5), ("q4_0", 300, 2048, 4), ("tq2_0", 96, 8192, 3),
+                                                 ("q4_0", 2048, 2048, 9)])
+def test_grouped_evenly_spaced_problems(pkg, gpu, oracle, fmt, rows, cols, count):
+    """A grouped launch whose matrices and outputs are evenly spaced views of one allocation, with one shared vector or
+    evenly spaced vectors, travels as strides in the kernel arguments (no descriptor table): same bits as the launches
+    issued one by one, and parity with the oracle."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(44, rows + cols + count)
+    wb = pkg.synth.weight_bytes(fmt, rows, cols)
+    raws = [pkg.synth.weights(fmt, rows, cols, g) for _ in range(count)]
+    big = pkg.Buffer.empty(ctx, wb * count)
+    for i, r in enumerate(raws):
+        big.copy_from_bytes(r, i * wb)
+    ws = [big.view(i * wb, wb) for i in range(count)]
+    for shared in (True, False):
+        xs_host = [pkg.synth.activations(1, cols, g)[0] for _ in range(1 if shared else count)]
+        xall = pkg.Buffer.from_slice(ctx, np.concatenate(xs_host))
+        xs = [xall.view(0, cols * 4)] * count if shared else [xall.view(i * cols * 4, cols * 4) for i in range(count)]
+        yall = pkg.Buffer.empty(ctx, count * rows * 4)
+        ys = [yall.view(i * rows * 4, rows * 4) for i in range(count)]
+        y1 = [pkg.Buffer.empty(ctx, rows * 4) for _ in range(count)]
+        batch = pkg.CommandBatch(ctx)
+        K.matvec_quant_grouped_into(batch, ty, ws, xs, pkg.F32, ys, pkg.F32, rows, cols)
+        assert batch.dispatch_count() == 1
+        for i in range(count):
+            K.matvec_quant_typed_into(batch, ty, ws[i], xs[i], pkg.F32, y1[i], pkg.F32, rows, cols)
+        batch.commit_and_wait()
+        for i in range(count):
+            a, b = ys[i].as_array(np.float32, rows), y1[i].as_array(np.float32, rows)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), f"problem {i} (shared vector: {shared})"
+            want = oracle.matvec_quant_ref(fmt, raws[i], xs_host[0 if shared else i], rows, cols, threads=8)
+            refgen.assert_close(a, want, 1e-3, f"{fmt} grouped #{i}")
