@@ -36,8 +36,8 @@ constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes 
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
 constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
 constexpr uint32_t kRing = 4;                 // tiles the waves of a split workgroup may drift apart
-constexpr uint32_t kMaxSplitWaves = 6;        // most waves that share the block groups of a tile
-constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxSplitWaves * 16 * 4 + 2 * kRing * 4;   // partial rows + arrival / generation words
+constexpr uint32_t kMaxWavesPerWG = 12;       // the largest workgroup launched here
+constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxWavesPerWG * 16 * 4 + (size_t)kMaxWavesPerWG * 2 * kRing * 4;   // partial rows + arrival / generation words per tile of a slot
 constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
@@ -64,6 +64,7 @@ struct Tq2Base {
     Tq2Problem p;
     uint32_t xstride, ystride;   // bytes
     uint64_t mstride = 0;        // bytes between the matrices of consecutive problems (0: one matrix for all of them)
+    uint32_t split_waves = 0;    // split form: waves that share the block groups of one tile (0: all waves of the workgroup)
     // A pair of unrelated problems (gate and up) also travels here, so the common grouped launch needs no
     // descriptor upload ahead of it.
     Tq2Problem second = {nullptr, nullptr, nullptr};
@@ -125,11 +126,16 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     // Normally a slot is nwaves consecutive tiles, one per wave, each wave walking all block groups of its tile.  With
     // `splitk` (few tiles, long rows) a slot is ONE tile whose block groups are dealt to the waves (nwaves divides their
     // number) and the waves' partial row sums are added through LDS in a fixed order.
-    const uint32_t slots_per_problem = splitk ? tiles_per_problem : (tiles_per_problem + nwaves - 1) / nwaves;
+    // A large workgroup in split form holds several such tiles at once: sw waves per tile, nwaves / sw consecutive tiles
+    // per slot (wave w works on tile w / sw of the slot, block groups w % sw, w % sw + sw, ...).
+    const uint32_t sw = splitk ? (single.split_waves ? single.split_waves : (uint32_t)nwaves) : 1u;   // waves per tile
+    const uint32_t tps = splitk ? (uint32_t)nwaves / sw : (uint32_t)nwaves;                          // tiles per slot
+    const uint32_t tsub = splitk ? (uint32_t)wave / sw : (uint32_t)wave;                             // this wave's tile of the slot
+    const uint32_t slots_per_problem = (tiles_per_problem + tps - 1) / tps;
     const uint64_t total_slots = (uint64_t)slots_per_problem * count;
     const uint32_t ngroups = (nb + 7) >> 3;
     const uint64_t my_slots = blockIdx.x < total_slots ? (total_slots - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
-    const uint32_t grp0 = splitk ? (uint32_t)wave : 0u, grp_step = splitk ? (uint32_t)nwaves : 1u;
+    const uint32_t grp0 = splitk ? (uint32_t)wave % sw : 0u, grp_step = sw;
     const uint64_t nitems = my_slots * (ngroups / grp_step);        // one item = one (tile, block group)
 
     // Chunk -> (row, chunk-in-row) of the lane's staging loads.  Full groups of 8 blocks (33 chunks per row): the global
@@ -141,8 +147,8 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     // (16-bit entries: row offsets stay below 15 * 3168 + 528 bytes for the widest row this kernel takes)
     uint16_t* tail_tab = reinterpret_cast<uint16_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [3][kStageLoads][64]
     uint16_t* full_tab = tail_tab + 2 * kStageLoads * 64;
-    if (splitk && threadIdx.x < 2 * kRing)   // arrival counts and generations of the partial-sum ring
-        reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxSplitWaves * 16)[threadIdx.x] = 0u;
+    if (splitk && threadIdx.x < kMaxWavesPerWG * 2 * kRing)   // arrival counts and generations of the partial-sum rings
+        reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxWavesPerWG * 16)[threadIdx.x] = 0u;
     if (wave == 0) {
         const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
 #pragma unroll
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     };
     auto item_tile_base = [&](const Item& it, uint32_t& grp, uint32_t& tile, Tq2Problem& pb) {
         grp = it.grp;
-        tile = splitk ? it.sip : it.sip * nwaves + wave;
+        tile = it.sip * tps + tsub;
         if (problems) pb = problems[it.prob];
         else if (single.pair && it.prob == 1) pb = single.second;
         else pb = Tq2Problem{single.p.matrix + (size_t)it.prob * single.mstride, (const char*)single.p.vector + (size_t)it.prob * single.xstride,
@@ -342,33 +348,42 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
                 // rows and opens the ring slot for its next use.  No workgroup barrier: the waves drift by up to kRing - 1
                 // tiles, which keeps their loads (the block groups of the same rows) close together in time without
                 // making them wait for each other.
-                uint32_t* sync = reinterpret_cast<uint32_t*>(part + kRing * kMaxSplitWaves * 16);   // arrivals[kRing], generation[kRing]
+                uint32_t* sync = reinterpret_cast<uint32_t*>(part + kRing * kMaxWavesPerWG * 16) + tsub * 2 * kRing;   // this tile's arrivals[kRing], generation[kRing]
+                float* tpart = part + (size_t)tsub * sw * 16;                                  // ring slot r of this tile: tpart + r * nwaves * 16
+                const uint32_t gw = (uint32_t)wave % sw;
                 const uint32_t ring = slot_seq % kRing, gen = slot_seq / kRing;
+                // Ordering: the LDS unit executes a wave's operations in issue order, so "partial rows, then the arrival
+                // count" and "count reset, then the generation word" need no more than a wait for this wave's own LDS
+                // operations (lgkmcnt) and a compiler barrier.  A fence of workgroup scope would also wait for the wave's
+                // outstanding global loads -- the next tile's prefetch -- and is deliberately not used.
+                auto lds_order = [] { __builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory"); };   // lgkmcnt(0) only
                 if (gen) {   // the slot's previous use must have been summed (bounded wait: never expected to run out)
                     uint32_t spins = 0;
-                    while (__hip_atomic_load(&sync[kRing + ring], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) != gen && spins++ < (1u << 20))
+                    while (__hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != gen && spins++ < (1u << 20))
                         __builtin_amdgcn_s_sleep(2);
+                    lds_order();
                 }
                 if (c == 0) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) part[(ring * nwaves + wave) * 16 + 4 * g + i] = parts[i];
+                    for (int i = 0; i < 4; i++) tpart[(ring * nwaves + gw) * 16 + 4 * g + i] = parts[i];
                 }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                lds_order();
                 uint32_t arrived = 0;
-                if (lane == 0) arrived = __hip_atomic_fetch_add(&sync[ring], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (lane == 0) arrived = __hip_atomic_fetch_add(&sync[ring], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 arrived = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrived);
-                if (arrived == (uint32_t)nwaves - 1u) {
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                if (arrived == sw - 1u) {
+                    lds_order();
                     if (lane < 16) {
-                        float v = part[(ring * nwaves) * 16 + lane];
-                        for (int w = 1; w < nwaves; w++) v += part[(ring * nwaves + w) * 16 + lane];
+                        float v = tpart[(ring * nwaves) * 16 + lane];
+                        for (uint32_t w = 1; w < sw; w++) v += tpart[(ring * nwaves + w) * 16 + lane];
                         const uint32_t orow = (tile << 4) + lane;
-                        if (orow < rows) lh_store_from_f32<YT>(y, orow, v);
+                        if (tile < tiles_per_problem && orow < rows) lh_store_from_f32<YT>(y, orow, v);
                     }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    lds_order();
                     if (lane == 0) {
                         __hip_atomic_store(&sync[ring], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        __hip_atomic_store(&sync[kRing + ring], gen + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        lds_order();
+                        __hip_atomic_store(&sync[kRing + ring], gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     }
                 }
                 slot_seq++;
@@ -409,13 +424,18 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     // (LOCAL_HIP_TQ2_WIDE=0 keeps four-wave workgroups).
     static const int wide_on = [] { const char* e = getenv("LOCAL_HIP_TQ2_WIDE"); return !(e && e[0] == '0' && e[1] == 0); }();
     bool wide = false;
+    uint32_t wide_split = 0;     // waves per tile when the twelve-wave workgroup runs in split form
     if (!splitk && threads == 256 && wide_on && (160 * 1024) / lds_for(4) < 3 && lds_for(12) <= kMaxLdsBytes &&
         tiles >= (uint64_t)ctx->cu_count * 24) {
         wide = true;
         threads = 768;
+        // the block groups of a tile on neighbouring waves: the segments of one row are then fetched close together in time
+        static const int wsplit_on = [] { const char* e = getenv("LOCAL_HIP_TQ2_WIDE_SPLIT"); return !(e && e[0] == '0' && e[1] == 0); }();
+        if (wsplit_on && ngroups > 1 && 12 % ngroups == 0) wide_split = ngroups;
     }
     const uint32_t waves = threads / 64;
-    const uint64_t slots = splitk ? tiles : (uint64_t)(((rows + 15) >> 4) + waves - 1) / waves * count;
+    const uint32_t tiles_per_slot = wide_split ? waves / wide_split : (splitk ? 1u : waves);
+    const uint64_t slots = (uint64_t)(((rows + 15) >> 4) + tiles_per_slot - 1) / tiles_per_slot * count;
     const size_t lds_bytes = lds_for(waves);
     const int lds_fit = (int)std::max<size_t>(1, (160 * 1024) / lds_bytes);          // workgroups per CU that LDS allows
     const int wg_eff = wide ? 1 : (threads == 256 ? std::min(wg_cu, lds_fit) : 4 * wg_cu);
@@ -424,7 +444,8 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     if (lds_bytes > kMaxLdsBytes) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
     const void* fn;
     if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
-#define LH_FN(XT, YT) (wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                             \
+#define LH_FN(XT, YT) (wide_split ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true, 768>                                        \
+                            : wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                      \
                             : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true>                                          \
                             : ngroups == 1 ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 256, true>                        \
                                            : (const void*)matvec_tq2_mfma_kernel<XT, YT, false>)
@@ -440,6 +461,7 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
 
     Tq2Base single{Tq2Problem{(const uint8_t*)matrices[0], vectors[0], outputs[0]}, xstride, ystride};
     single.mstride = mstride;
+    single.split_waves = wide_split;
     single.pro = pro;
     Tq2Problem* dev = nullptr;
     if (count == 2 && !strided) {

@@ -332,3 +332,34 @@ def test_grouped_evenly_spaced_problems(pkg, gpu, oracle, fmt, rows, cols, count
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), f"problem {i} (shared vector: {shared})"
             want = oracle.matvec_quant_ref(fmt, raws[i], xs_host[0 if shared else i], rows, cols, threads=8)
             refgen.assert_close(a, want, 1e-3, f"{fmt} grouped #{i}")
+
+
+def test_grouped_long_rows_many_tiles(pkg, gpu, oracle):
+    """Enough 16-row tiles of a long-row shape (2048 x 8192, four block groups per row) for the launch form that the
+    large grouped benchmark uses there: twelve-wave workgroups, the block groups of a tile on neighbouring waves, their
+    partial rows summed through the LDS ring.  Every problem against the oracle."""
+    ctx, K = gpu
+    rows, cols, count, distinct = 2048, 8192, 52, 4
+    g = pkg.synth.rng(45, 1)
+    wb = pkg.synth.weight_bytes("tq2_0", rows, cols)
+    raws = [pkg.synth.weights("tq2_0", rows, cols, g) for _ in range(distinct)]
+    big = pkg.Buffer.empty(ctx, wb * count)
+    for i in range(count):
+        big.copy_from_bytes(raws[i % distinct], i * wb)
+    ws = [big.view(i * wb, wb) for i in range(count)]
+    x = pkg.synth.activations(1, cols, g)[0]
+    xb = pkg.Buffer.from_slice(ctx, x)
+    yall = pkg.Buffer.from_slice(ctx, np.full(count * rows, np.nan, np.float32))
+    ys = [yall.view(i * rows * 4, rows * 4) for i in range(count)]
+    batch = pkg.CommandBatch(ctx)
+    K.matvec_quant_grouped_into(batch, pkg.TQ2_0, ws, [xb] * count, pkg.F32, ys, pkg.F32, rows, cols)
+    batch.commit_and_wait()
+    wants = [oracle.matvec_quant_ref("tq2_0", r, x, rows, cols, threads=8) for r in raws]
+    got = yall.as_array(np.float32, count * rows).reshape(count, rows)
+    for i in range(count):
+        if i in (0, 17, count - 1):
+            refgen.assert_close_both(got[i], wants[i % distinct], 1e-3, f"long rows, problem {i}")
+        else:
+            refgen.assert_close(got[i], wants[i % distinct], 1e-3, f"long rows, problem {i}")
+    for i in range(distinct, count):       # identical weights and vector: identical bits, wherever the problem ran
+        assert np.array_equal(got[i].view(np.uint32), got[i % distinct].view(np.uint32)), f"problem {i}"
