@@ -31,11 +31,18 @@
 
 namespace {
 
+#ifndef LH_TQ2_RING
+#define LH_TQ2_RING 1
+#endif
 constexpr int kL = 2;                        // activation limbs (16-bit block fixed point)
 constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
 constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // padded row stride + over-read margin
-constexpr uint32_t kRing = 4;                 // tiles the waves of a split workgroup may drift apart
+// Ring slots for the partial rows of a split tile: the waves of a tile may drift kRing - 1 tiles apart.  One slot: a wave
+// delivers tile n only after tile n - 1 has been summed, so the waves of a tile stay within a tile of each other and fetch
+// the neighbouring segments of the same rows close together in time; with four slots the shared cache lines were evicted
+// in between and fetched again (1.09 x the bytes with plain loads against 1.03 x, 5.3 against 5.5 TB/s).
+constexpr uint32_t kRing = LH_TQ2_RING;
 constexpr uint32_t kMaxWavesPerWG = 12;       // the largest workgroup launched here
 constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxWavesPerWG * 16 * 4 + (size_t)kMaxWavesPerWG * 2 * kRing * 4;   // partial rows + arrival / generation words per tile of a slot
 constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
@@ -93,9 +100,11 @@ __device__ __forceinline__ void take16(const u32x4_t& c0, const u32x4_t& c1, uin
 
 // STREAM: the weight loads carry the non-temporal hint.  Right when a tile's bytes are one contiguous run (one block group
 // per row: every cache line is used once, by one instruction).  With several groups per row a tile is sixteen 528-byte
-// segments whose first and last cache lines are shared with the neighbouring segment, read by the same wave an item
-// later: the hint evicts those lines early and they are fetched a second time (measured: 1.19 x the bytes), so such
-// launches use plain loads.
+// segments whose first and last cache lines are shared with the neighbouring segment.  Where one wave walks the groups of
+// its tile the neighbour is read an item later: the hint evicts those lines early and they come from HBM a second time
+// (measured: 1.19 x the bytes), so such launches use plain loads.  The twelve-wave split form reads the neighbouring
+// segments on neighbouring waves at about the same time (kRing below): there the shared lines still cost 1.10 x, but the
+// hinted loads stream enough faster to win (5.6-5.7 against 5.5 TB/s on 2048 x 8192 weights).
 template <typename XT, typename YT, bool SPLITK, int MAXT = 256, bool STREAM = false>
 __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_kernel(const Tq2Problem* __restrict__ problems, Tq2Base single,
                                                                 uint32_t count, uint32_t rows, uint32_t K) {
@@ -345,9 +354,8 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
                 // Every wave of the workgroup reaches this point once per slot, in the same slot order, but not in step:
                 // a wave parks its sixteen partial rows in a ring slot and counts itself in; whichever wave arrives last
                 // sums the partials in wave order (so the result does not depend on the order of arrival), stores the
-                // rows and opens the ring slot for its next use.  No workgroup barrier: the waves drift by up to kRing - 1
-                // tiles, which keeps their loads (the block groups of the same rows) close together in time without
-                // making them wait for each other.
+                // rows and opens the ring slot for its next use.  No workgroup barrier: a wave waits only when it is kRing
+                // tiles ahead of the slowest wave of its tile.
                 uint32_t* sync = reinterpret_cast<uint32_t*>(part + kRing * kMaxWavesPerWG * 16) + tsub * 2 * kRing;   // this tile's arrivals[kRing], generation[kRing]
                 float* tpart = part + (size_t)tsub * sw * 16;                                  // ring slot r of this tile: tpart + r * nwaves * 16
                 const uint32_t gw = (uint32_t)wave % sw;
@@ -444,7 +452,7 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     if (lds_bytes > kMaxLdsBytes) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
     const void* fn;
     if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
-#define LH_FN(XT, YT) (wide_split ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true, 768>                                        \
+#define LH_FN(XT, YT) (wide_split ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true, 768, true>                                       \
                             : wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                      \
                             : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true>                                          \
                             : ngroups == 1 ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 256, true>                        \

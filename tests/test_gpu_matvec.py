@@ -334,32 +334,43 @@ def test_grouped_evenly_spaced_problems(pkg, gpu, oracle, fmt, rows, cols, count
             refgen.assert_close(a, want, 1e-3, f"{fmt} grouped #{i}")
 
 
-def test_grouped_long_rows_many_tiles(pkg, gpu, oracle):
-    """Enough 16-row tiles of a long-row shape (2048 x 8192, four block groups per row) for the launch form that the
-    large grouped benchmark uses there: twelve-wave workgroups, the block groups of a tile on neighbouring waves, their
-    partial rows summed through the LDS ring.  Every problem against the oracle."""
+@pytest.mark.parametrize("rows,cols,count,shared_x,half", [(2048, 8192, 52, True, False), (1024, 4096, 100, False, False),
+                                                           (2032, 8192, 52, True, False), (2048, 8192, 52, False, True)])
+def test_grouped_long_rows_many_tiles(pkg, gpu, oracle, rows, cols, count, shared_x, half):
+    """Enough 16-row tiles of a long-row shape (four or two block groups per row) for the launch forms that the large
+    grouped benchmark uses there: twelve-wave workgroups, the block groups of a tile on neighbouring waves, their partial
+    rows summed through LDS.  2032 rows leave a partial last tile and surplus waves in each problem's last slot.  One
+    vector for all problems or one each (a vector is staged when the workgroup reaches its first tile of a problem), f32
+    or f16 in and out.  Every problem against the oracle."""
     ctx, K = gpu
-    rows, cols, count, distinct = 2048, 8192, 52, 4
-    g = pkg.synth.rng(45, 1)
+    distinct = 4
+    g = pkg.synth.rng(45, rows + cols)
     wb = pkg.synth.weight_bytes("tq2_0", rows, cols)
     raws = [pkg.synth.weights("tq2_0", rows, cols, g) for _ in range(distinct)]
     big = pkg.Buffer.empty(ctx, wb * count)
     for i in range(count):
         big.copy_from_bytes(raws[i % distinct], i * wb)
     ws = [big.view(i * wb, wb) for i in range(count)]
-    x = pkg.synth.activations(1, cols, g)[0]
-    xb = pkg.Buffer.from_slice(ctx, x)
-    yall = pkg.Buffer.from_slice(ctx, np.full(count * rows, np.nan, np.float32))
-    ys = [yall.view(i * rows * 4, rows * 4) for i in range(count)]
+    nx = 1 if shared_x else distinct
+    xs_host = [pkg.synth.activations(1, cols, g)[0] for _ in range(nx)]
+    if half:
+        xs_host = [x.astype(np.float16) for x in xs_host]
+    xt, esz = (pkg.F16, 2) if half else (pkg.F32, 4)
+    np_t = np.float16 if half else np.float32
+    xbufs = [pkg.Buffer.from_slice(ctx, x) for x in xs_host]
+    yall = pkg.Buffer.from_slice(ctx, np.full(count * rows, np.nan, np_t))
+    ys = [yall.view(i * rows * esz, rows * esz) for i in range(count)]
     batch = pkg.CommandBatch(ctx)
-    K.matvec_quant_grouped_into(batch, pkg.TQ2_0, ws, [xb] * count, pkg.F32, ys, pkg.F32, rows, cols)
+    K.matvec_quant_grouped_into(batch, pkg.TQ2_0, ws, [xbufs[i % nx] for i in range(count)], xt, ys, xt, rows, cols)
     batch.commit_and_wait()
-    wants = [oracle.matvec_quant_ref("tq2_0", r, x, rows, cols, threads=8) for r in raws]
-    got = yall.as_array(np.float32, count * rows).reshape(count, rows)
+    wants = [oracle.matvec_quant_ref("tq2_0", raws[i], xs_host[i % nx].astype(np.float32), rows, cols, threads=8) for i in range(distinct)]
+    got = yall.as_array(np_t, count * rows).reshape(count, rows)
+    tol = 2e-3 if half else 1e-3              # f16 outputs carry their own rounding
     for i in range(count):
-        if i in (0, 17, count - 1):
-            refgen.assert_close_both(got[i], wants[i % distinct], 1e-3, f"long rows, problem {i}")
+        if i in (0, 17, count - 1) and not half:
+            refgen.assert_close_both(got[i], wants[i % distinct], tol, f"long rows, problem {i}")
         else:
-            refgen.assert_close(got[i], wants[i % distinct], 1e-3, f"long rows, problem {i}")
+            refgen.assert_close(got[i].astype(np.float32), wants[i % distinct], tol, f"long rows, problem {i}")
+    bits = np.uint16 if half else np.uint32
     for i in range(distinct, count):       # identical weights and vector: identical bits, wherever the problem ran
-        assert np.array_equal(got[i].view(np.uint32), got[i % distinct].view(np.uint32)), f"problem {i}"
+        assert np.array_equal(got[i].view(bits), got[i % distinct].view(bits)), f"problem {i}"
