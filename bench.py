@@ -332,6 +332,15 @@ def bench_prefill(pkg, ctx, K, steps, warmup):
         _, ev = time_steps(pkg, ctx, step, steps, warmup)
         tf = 2.0 * m * k * n / (ev * 1e-3) * 1e-12
         res[fmt] = {"us": ev * 1e3, "tflops": tf, "frac_of_f16_mfma_peak": tf / MFMA_F16_PEAK_TFLOPS}
+        # the same product with f16 activations and an f16 result (what a layer hands from kernel to kernel): no conversion
+        # in the staging and half the output bytes
+        ah = pkg.Buffer.from_slice(ctx, pkg.synth.activations(m, k, g).astype(np.float16))
+        ch = pkg.Buffer.empty(ctx, m * n * 2)
+        step_h = bound_call(pkg.lib().lh_matmul_nt_quant_typed_into, batch, C.c_int(w.ty), ah, C.c_int(pkg.F16), w.buf, ch,
+                            C.c_int(pkg.F16), m, k, n)
+        _, ev_h = time_steps(pkg, ctx, step_h, steps, warmup)
+        tf_h = 2.0 * m * k * n / (ev_h * 1e-3) * 1e-12
+        res[fmt].update({"f16_io_us": ev_h * 1e3, "f16_io_tflops": tf_h, "f16_io_frac_of_f16_mfma_peak": tf_h / MFMA_F16_PEAK_TFLOPS})
     return res
 
 

@@ -102,6 +102,12 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) { return (uint32_t)lh_f2h(a) | ((uint32_t)lh_f2h(b) << 16); }
+// two bf16 -> two f16, each rounded to nearest even like the scalar conversion (v_cvt_pk_f16_f32)
+__device__ __forceinline__ uint32_t bf2_to_h2(uint32_t w) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {__builtin_bit_cast(float, w << 16), __builtin_bit_cast(float, w & 0xFFFF0000u)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
 __device__ __forceinline__ uint32_t h2_sub_mul(uint32_t x, uint32_t bias, uint32_t d2) {
     const f16x2 r = (__builtin_bit_cast(f16x2, x) - __builtin_bit_cast(f16x2, bias)) * __builtin_bit_cast(f16x2, d2);
     return __builtin_bit_cast(uint32_t, r);
@@ -452,19 +458,24 @@ template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_
 __device__ __forceinline__ void settle(u32x4v& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void settle(uint32_t& v) { asm volatile("" : "+v"(v)); }
 
-template <int FMT, int CDT>
-__global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
+// ABF: the activations arrive as bf16 and are converted to f16 on their way into LDS (three vector instructions per pair,
+// in every column tile), which costs less than a conversion pass of its own: that pass is a second dependent launch.
+// PW: staging waves (4 or 8) next to the four multiplying waves.  Eight halve the load -> convert -> store chain of each
+// staging wave and put three waves on every SIMD.
+template <int FMT, int CDT, bool ABF = false, int PW = 4>
+__global__ __launch_bounds__(256 + 64 * PW) void matmul_mfma128_kernel(const uint16_t* __restrict__ A, const uint8_t* __restrict__ W, void* __restrict__ C,
                                                             uint32_t M, uint32_t K, uint32_t N) {
     static_assert(FMT == kQ4 || FMT == kTQ2, "quantised weights only");
-    constexpr int BM = 128, NCH = 8;
-    constexpr int NB = FMT == kQ4 ? 2 : 1;                        // weight pieces per staging thread and step
+    constexpr int BM = 128, PT = 64 * PW, NCH = 2048 / PT;        // staging threads; 16-byte activation chunks per staging thread and step
+    constexpr int NB = (FMT == kQ4 && PW == 4) ? 2 : 1;           // weight pieces per staging thread and step
     constexpr int kLoadsPerStep = NCH + 2 * NB;
     __shared__ __align__(16) _Float16 As[2][BM * LDK];
     __shared__ __align__(16) _Float16 Bs[2][BN * LDK];
-    // Waves 0-3 multiply (2 x 2 waves, 64 x 64 outputs each), waves 4-7 stage: every SIMD holds one of each kind, so the
-    // staging waves' memory and LDS waits are filled by the other wave's MFMAs.  One barrier per k step hands over a buffer.
+    // Waves 0-3 multiply (2 x 2 waves, 64 x 64 outputs each), the other PW waves stage: every SIMD holds one multiplying wave
+    // and one or two staging waves, so the staging waves' memory and LDS waits are filled by the other wave's MFMAs.  One
+    // barrier per k step hands over a buffer.
     const bool producer = threadIdx.x >= 256;
-    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    const int tid = producer ? (int)threadIdx.x - 256 : (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const uint32_t nk = K / BK;                                   // K is a multiple of 128 here
 
@@ -474,16 +485,20 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
         uint32_t a_off[NCH], a_lds[NCH];
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
-            const uint32_t c = tid + 256 * i, row = c >> 4, kc = c & 15;
+            const uint32_t c = tid + PT * i, row = c >> 4, kc = c & 15;
             const uint32_t rc = m0 + row < M ? row : M - 1 - m0;
             a_off[i] = (rc * K + 8 * kc) * 2;
             a_lds[i] = row * LDK + 8 * kc;
         }
-        const uint32_t b_ld_row = tid >> 1, part = tid & 1;
+        // Four staging waves: two threads per weight row.  Q4_0: 4 blocks of 18 bytes per step and row, a thread takes
+        // blocks 2 * part, 2 * part + 1.  TQ2_0: one 66-byte block per two steps and row, a thread takes 16 of the step's
+        // 32 code bytes (all four fields).  Eight staging waves: four threads per row; Q4_0 one block each, TQ2_0 the
+        // same 16 code bytes twice, fields 0, 1 on one thread and 2, 3 on the other.
+        const uint32_t b_ld_row = PW == 4 ? tid >> 1 : tid >> 2;
+        const uint32_t part = PW == 4 ? tid & 1 : (FMT == kQ4 ? tid & 3 : (tid >> 1) & 1), fh = tid & 1;
+        (void)fh;
         const uint32_t b_rc = n0 + b_ld_row < N ? b_ld_row : N - 1 - n0;
-        // Q4_0: 4 blocks of 18 bytes per step and row, this thread takes blocks 2 * part, 2 * part + 1.
-        // TQ2_0: one 66-byte block per two steps and row, this thread takes 16 of the step's 32 code bytes.
-        const uint32_t b_off = b_rc * row_bytes + (FMT == kQ4 ? part * 36 : part * 16);
+        const uint32_t b_off = b_rc * row_bytes + (FMT == kQ4 ? part * (PW == 4 ? 36 : 18) : part * 16);
         const uint8_t* a_tile = reinterpret_cast<const uint8_t*>(A) + (size_t)m0 * K * 2;
         const uint8_t* w_tile = W + (size_t)n0 * row_bytes;
 
@@ -514,8 +529,11 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
 #pragma unroll
             for (int i = 0; i < NB; i++) { settle(rq[set][i]); settle(rd[set][i]); }
 #pragma unroll
-            for (int i = 0; i < NCH; i++)
-                *reinterpret_cast<uint4*>(&As[buf][a_lds[i]]) = make_uint4(ra[set][i].x, ra[set][i].y, ra[set][i].z, ra[set][i].w);
+            for (int i = 0; i < NCH; i++) {
+                uint4 v = make_uint4(ra[set][i].x, ra[set][i].y, ra[set][i].z, ra[set][i].w);
+                if constexpr (ABF) v = make_uint4(bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w));
+                *reinterpret_cast<uint4*>(&As[buf][a_lds[i]]) = v;
+            }
             if constexpr (FMT == kQ4) {
                 uint32_t f[16];
 #pragma unroll
@@ -524,17 +542,27 @@ __global__ __launch_bounds__(512) void matmul_mfma128_kernel(const uint16_t* __r
                     r.q[0] = make_uint4(rq[set][i].x, rq[set][i].y, rq[set][i].z, rq[set][i].w);
                     r.d = rd[set][i];
                     convert_b<kQ4>(f, r, 0, true);
-                    store_words<16>(&Bs[buf][b_ld_row * LDK + 64 * part + 32 * i], f);
+                    store_words<16>(&Bs[buf][b_ld_row * LDK + (PW == 4 ? 64 : 32) * part + 32 * i], f);
                 }
             } else {
                 RawBT r;
                 r.q = make_uint4(rq[set][0].x, rq[set][0].y, rq[set][0].z, rq[set][0].w);
                 r.d = rd[set][0];
+                if constexpr (PW == 4) {
 #pragma unroll
-                for (int f = 0; f < 4; f++) {
-                    uint32_t w[8];
-                    convert_bt(w, r, f, true);
-                    store_words<8>(&Bs[buf][b_ld_row * LDK + 32 * f + 16 * part], w);
+                    for (int f = 0; f < 4; f++) {
+                        uint32_t w[8];
+                        convert_bt(w, r, f, true);
+                        store_words<8>(&Bs[buf][b_ld_row * LDK + 32 * f + 16 * part], w);
+                    }
+                } else {
+#pragma unroll
+                    for (int f2 = 0; f2 < 2; f2++) {
+                        const int f = 2 * (int)fh + f2;
+                        uint32_t w[8];
+                        convert_bt(w, r, f, true);
+                        store_words<8>(&Bs[buf][b_ld_row * LDK + 32 * f + 16 * part], w);
+                    }
                 }
             }
         };
@@ -1056,14 +1084,27 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
             const size_t a16_bytes = (size_t)m * k * 2;
             if (big && k % BK == 0 && (ADT == LH_F16 || a16_bytes <= ctx->workspace_bytes)) {
                 const uint16_t* a16 = static_cast<const uint16_t*>(A);
-                if constexpr (ADT != LH_F16) {   // one pass over the activations instead of a conversion in every column tile
+                static const int bf_inline = [] { const char* e = getenv("LOCAL_HIP_PREFILL_BF16_PASS"); return !(e && e[0] == '1' && e[1] == 0); }();
+                static const int pw4 = [] { const char* e = getenv("LOCAL_HIP_PREFILL_PW"); return e && atoi(e) == 4; }();   // four staging waves instead of eight
+                const dim3 grid128((n + BN - 1) / BN, (m + 127) / 128);
+                if constexpr (ADT == LH_BF16) {
+                    if (bf_inline) {             // bf16 is converted by the staging waves (LOCAL_HIP_PREFILL_BF16_PASS=1: by a pass of its own)
+                        if (pw4 && ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, true, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
+                        else if (pw4) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, true, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
+                        else if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                        else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                        return LH_OK;
+                    }
+                }
+                if constexpr (ADT != LH_F16) {   // f32: one pass over the activations instead of a conversion in every column tile
                     const size_t n8 = (size_t)m * k / 8;
                     hipLaunchKernelGGL((convert_to_f16_kernel<ADT>), dim3((uint32_t)((n8 + 255) / 256)), dim3(256), 0, s, A, (uint16_t*)ctx->workspace, n8);
                     a16 = static_cast<const uint16_t*>(ctx->workspace);
                 }
-                const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
-                if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32>), grid, dim3(512), 0, s, a16, W, C, m, k, n);
-                else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16>), grid, dim3(512), 0, s, a16, W, C, m, k, n);
+                if (pw4 && ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, false, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
+                else if (pw4) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, false, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
+                else if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, false, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, false, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
                 return LH_OK;
             }
         }
