@@ -586,11 +586,19 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
     step_single()
     per_layer = (batch.dispatch_count() - d0 - 1) // n_layers
     wall, ev = time_steps(pkg, ctx, step_single, max(steps, 20), warmup)
+    host = []                                    # host time to enqueue one step (the GPU idle when it starts)
+    for _ in range(5):
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        step_single()
+        host.append(time.perf_counter() - t0)
+    ctx.synchronize()
     out = hidden[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("decode step produced non-finite hidden state")
     res = {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
-           "dispatches_per_layer": per_layer, "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
+           "dispatches_per_layer": per_layer, "host_enqueue_us_per_layer": min(host) * 1e6 / n_layers,
+           "weight_bytes_per_layer": wbytes, "kv_bytes_per_layer": kv_bytes,
            "gbs_events": (wbytes + kv_bytes) / (ev / n_layers) * 1e-6,
            "tokens_per_s_35_layers": 1.0 / (ev * 1e-3 / n_layers * 35)}
     if not graphs:

@@ -494,7 +494,10 @@ __global__ __launch_bounds__(256 + 64 * PW) void matmul_mfma128_kernel(const uin
         // blocks 2 * part, 2 * part + 1.  TQ2_0: one 66-byte block per two steps and row, a thread takes 16 of the step's
         // 32 code bytes (all four fields).  Eight staging waves: four threads per row; Q4_0 one block each, TQ2_0 the
         // same 16 code bytes twice, fields 0, 1 on one thread and 2, 3 on the other.
-        const uint32_t b_ld_row = PW == 4 ? tid >> 1 : tid >> 2;
+        // (TQ2_0, eight waves: the eight lanes of one LDS store phase take rows r and r + 2 instead of r and r + 1 -- at 288
+        // bytes per row the four 32-byte pieces of neighbouring rows meet on the same banks, those of rows two apart do not)
+        const uint32_t b_ld_row = PW == 4 ? tid >> 1
+                                : FMT == kTQ2 ? ((tid >> 4) << 2) + (((tid >> 2) & 1) << 1) + ((tid >> 3) & 1) : tid >> 2;
         const uint32_t part = PW == 4 ? tid & 1 : (FMT == kQ4 ? tid & 3 : (tid >> 1) & 1), fh = tid & 1;
         (void)fh;
         const uint32_t b_rc = n0 + b_ld_row < N ? b_ld_row : N - 1 - n0;
