@@ -50,16 +50,19 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
 
 // Second level of the fixed point, for blocks whose first-level step would be too coarse.  A block with max|x| = m has
 // the step s = m / qmax; every element carries an absolute error of up to s / 2 whatever its own size, so one large
-// element (ordinary in a residual stream) costs its 255 neighbours their low bits.  While m <= kXCoarseMax the step is at
-// most 2.5e-4 (16-bit limbs) and the error of a row sum stays a few 1e-5 of the weights' scale; above it the block also
-// gets the residual r_i = x_i - s n_i in 16-bit fixed point of its own (step s * 0.52 / qmax: about 2^-31 of m in all),
-// which the kernels add in a second pass over blocks that have one (those with xs2 != 0).
+// element (ordinary in a residual stream) costs its neighbours their low bits.  The test is relative to the block itself:
+// with r = mean |x| of the block's other elements, the block is left alone while m <= kXOutlier * r -- the error of an
+// element then stays below kXOutlier / (2 qmax) = 4.9e-4 r, and if every block of a vector sat at that limit the error of
+// a row sum would still be about 2e-4 of its scale (m / r is 3 .. 6 for Gaussian values of any scale and 9 .. 14 for
+// GeGLU products, whose blocks exceed 32 two or three times in a thousand).  A block above the limit also gets the
+// residual r_i = x_i - s n_i in 16-bit fixed point of its own (step s * 0.52 / qmax: about 2^-31 of m in all), which the
+// kernels add in a second pass over blocks that have one (those with xs2 != 0).
 struct XResidual {
     uint32_t* xq2;   // [2][K/4] residual limbs, laid out like xq (written for blocks with a second level only)
     float* xs2;      // [K/G] residual scale; 0 for a block whose first level suffices
     int* xn2;        // [K/G] sum of the residual integers (may be null)
 };
-constexpr float kXCoarseMax = 8.0f;
+constexpr float kXOutlier = 32.0f;
 
 __device__ __forceinline__ uint32_t lh_group_max_u(uint32_t v, int width) {
     if (width > 1) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR1>((int)v));
@@ -171,8 +174,9 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
         }
         // the maximum over the bit patterns of |v|: the order of non-negative floats, with NaN and infinity on top
         uint32_t mbits = 0u;
+        float asum = 0.0f;                                    // sum of |v| over the block (second-level test)
 #pragma unroll
-        for (int i = 0; i < 8; i++) mbits = max(mbits, __builtin_bit_cast(uint32_t, fabsf(v[i])));
+        for (int i = 0; i < 8; i++) { mbits = max(mbits, __builtin_bit_cast(uint32_t, fabsf(v[i]))); asum += fabsf(v[i]); }
         mbits = lh_group_max_u(mbits, G / 8);
         const bool finite = mbits < 0x7F800000u;
         const float m = __builtin_bit_cast(float, mbits);
@@ -210,7 +214,8 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
         }
         if constexpr (L == 2) {
             if (resid != nullptr) {
-                const bool coarse = finite && m > kXCoarseMax;       // uniform over the lanes of a group
+                asum = lh_group_sum(asum, G / 8);
+                const bool coarse = finite && m * (float)(G - 1) > kXOutlier * (asum - m);   // uniform over the lanes of a group
                 const float sc2 = sc * (0.52f / Limb<2>::qmax);       // |r| <= 0.5 sc up to rounding: 0.52 leaves headroom
                 int nsum2 = 0;
                 if (__builtin_amdgcn_ballot_w64(coarse) != 0) {      // rare: skipped by waves without such a block
