@@ -268,6 +268,52 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         uint32_t st_end = st + per_wave < s_end ? st + per_wave : s_end;
         if (st > s_end) st = s_end;
 
+        YT* y = static_cast<YT*>(pb.output);
+        gptr_t mat = (gptr_t)pb.matrix;
+        const uint32_t last_row = rows - 1;
+        const int red_width = NPOS == 1 ? (int)lpr : 64;
+        const bool writer = NPOS == 1 ? (((uint32_t)lane & (lpr - 1)) == 0) : lane == 0;
+
+        // ---- staged form: chunk c = lane + 64 i of the step's contiguous bytes
+        [[maybe_unused]] u32x4_t pre[kImgLoads];
+        [[maybe_unused]] const uint32_t step_bytes = U * rpw * row_bytes;
+        [[maybe_unused]] const uint32_t step_chunks = (step_bytes + 15) >> 4;
+        [[maybe_unused]] const size_t mat_bytes = (size_t)rows * row_bytes;   // chunks past the matrix read its first slack bytes (never used)
+        [[maybe_unused]] auto prefetch = [&](uint32_t st_) {
+            const size_t base = (size_t)st_ * rpw * row_bytes;
+#pragma unroll
+            for (int i = 0; i < kImgLoads; i++) {
+                // no branch around a load (a conditionally loaded register forces a wait right behind the load):
+                // surplus lanes repeat the step's last chunk, which is never parked
+                uint32_t c = lane + 64 * i;
+                c = c < step_chunks ? c : step_chunks - 1;
+                size_t off = base + (size_t)c * 16;
+                off = off < mat_bytes ? off : mat_bytes;
+                pre[i] = ld16_stream(mat + off);
+            }
+        };
+        if constexpr (IMG) { if (st < st_end) prefetch(st); }
+        // The first step's weights are requested before the vector is staged: their trip to memory then runs under the
+        // quantiser and its two barriers instead of behind them (a launch of a few steps per wave is mostly that latency).
+        constexpr bool kEarly = !IMG && FMT == LH_Q4_0 && NPOS <= 2;   // (the other forms have no registers to spare)
+        [[maybe_unused]] UnitW<FMT> w_first[kEarly ? U : 1][kEarly ? NPOS : 1];
+        bool have_first = false;
+        if constexpr (kEarly) {
+            if (pb.vector != staged_vector && st < st_end) {
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    uint32_t row = (st + u) * rpw + rsub;
+                    row = row < last_row ? row : last_row;
+                    gptr_t rp = mat + (size_t)row * row_bytes;
+#pragma unroll
+                    for (int p = 0; p < NPOS; p++) {
+                        const uint32_t ucol = col0 + 64u * p;
+                        load_unit_w<FMT>(w_first[u][p], rp, ucol < upr ? ucol : 0u);
+                    }
+                }
+                have_first = true;
+            }
+        }
         if (pb.vector != staged_vector) {
             __syncthreads();   // every wave is done reading the previous vector's limbs
             quantize_x_to_lds<L, G, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, nullptr, kWG, single.pro, L == 2 ? &resid : nullptr);
@@ -301,31 +347,6 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
             }
             staged_vector = pb.vector;
         }
-        YT* y = static_cast<YT*>(pb.output);
-        gptr_t mat = (gptr_t)pb.matrix;
-        const uint32_t last_row = rows - 1;
-        const int red_width = NPOS == 1 ? (int)lpr : 64;
-        const bool writer = NPOS == 1 ? (((uint32_t)lane & (lpr - 1)) == 0) : lane == 0;
-
-        // ---- staged form: chunk c = lane + 64 i of the step's contiguous bytes
-        [[maybe_unused]] u32x4_t pre[kImgLoads];
-        [[maybe_unused]] const uint32_t step_bytes = U * rpw * row_bytes;
-        [[maybe_unused]] const uint32_t step_chunks = (step_bytes + 15) >> 4;
-        [[maybe_unused]] const size_t mat_bytes = (size_t)rows * row_bytes;   // chunks past the matrix read its first slack bytes (never used)
-        [[maybe_unused]] auto prefetch = [&](uint32_t st_) {
-            const size_t base = (size_t)st_ * rpw * row_bytes;
-#pragma unroll
-            for (int i = 0; i < kImgLoads; i++) {
-                // no branch around a load (a conditionally loaded register forces a wait right behind the load):
-                // surplus lanes repeat the step's last chunk, which is never parked
-                uint32_t c = lane + 64 * i;
-                c = c < step_chunks ? c : step_chunks - 1;
-                size_t off = base + (size_t)c * 16;
-                off = off < mat_bytes ? off : mat_bytes;
-                pre[i] = ld16_stream(mat + off);
-            }
-        };
-        if constexpr (IMG) { if (st < st_end) prefetch(st); }
 
         for (; st < st_end; st += U) {
             float part[U];
@@ -359,6 +380,15 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                 }
             } else {
             UnitW<FMT> w[U][NPOS];
+            if (have_first) {                           // requested before the vector was staged
+                if constexpr (kEarly) {
+#pragma unroll
+                    for (int u = 0; u < U; u++)
+#pragma unroll
+                        for (int p = 0; p < NPOS; p++) w[u][p] = w_first[u][p];
+                }
+                have_first = false;
+            } else {
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 uint32_t row = (st + u) * rpw + rsub;     // steps past the end re-read the last row (result dropped)
@@ -369,6 +399,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                     const uint32_t ucol = col0 + 64u * p;
                     load_unit_w<FMT>(w[u][p], rp, ucol < upr ? ucol : 0u);
                 }
+            }
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
