@@ -408,7 +408,7 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
                 for (int p = 0; p < NPOS; p++) part[u] += unit_dot<FMT, L>(w[u][p], ux[p]);
             }
             if constexpr (L == 2) {
-                if (any_coarse) {   // uniform over the wave; rare: the residual level of the lane's unit columns, read from LDS
+                if (__builtin_expect(any_coarse, 0)) {   // uniform over the wave; rare: the residual level of the lane's unit columns, read from LDS
 #pragma unroll
                     for (int p = 0; p < NPOS; p++) {
                         const uint32_t ucol = col0 + 64u * p;

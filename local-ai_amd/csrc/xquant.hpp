@@ -182,7 +182,6 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
         const float m = __builtin_bit_cast(float, mbits);
         const float inv = (finite && m > 0.0f) ? Limb<L>::qmax / m : 0.0f;
         const float sc = finite ? m * (1.0f / Limb<L>::qmax) : __builtin_nanf("");
-        int nq[8];
         uint32_t packed[L][2];
         int nsum = 0;
 #pragma unroll
@@ -192,7 +191,6 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
             float r = rintf(v[i] * inv);
             r = fminf(fmaxf(r, -Limb<L>::qmax), Limb<L>::qmax);
             int n = (int)r;
-            nq[i] = n;
             nsum += n;
 #pragma unroll
             for (int l = 0; l < L; l++) {
@@ -223,7 +221,8 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                     uint32_t p2[2][2] = {{0u, 0u}, {0u, 0u}};
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
-                        const float rr = __builtin_fmaf(-(float)nq[i], sc, v[i]);
+                        const float n1 = fminf(fmaxf(rintf(v[i] * inv), -Limb<L>::qmax), Limb<L>::qmax);   // the first level's integer again
+                        const float rr = __builtin_fmaf(-n1, sc, v[i]);
                         float q2 = rintf(rr * inv2);
                         q2 = fminf(fmaxf(q2, -Limb<2>::qmax), Limb<2>::qmax);
                         int n2 = (int)q2;
