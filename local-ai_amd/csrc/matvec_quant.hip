@@ -528,19 +528,21 @@ __global__ __launch_bounds__(256) void matvec_tq2_0_soa_kernel(const uint8_t* __
     if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
 }
 
-int x_limbs() {
+// LOCAL_HIP_X_LIMBS=3: 24-bit first-level activations for Q4_0 (no second level then).  TQ2_0 always takes two limbs: with
+// its fields left in place (up to 16 x the code) and 256-element blocks, three limbs overflow the 32-bit sums.
+int x_limbs(lh_quant fmt) {
     static int v = [] {
         const char* e = getenv("LOCAL_HIP_X_LIMBS");
         return (e && e[0] == '3') ? 3 : 2;
     }();
-    return v;
+    return fmt == LH_Q4_0 ? v : 2;
 }
 
 // LOCAL_HIP_TQ2_KERNEL=valu selects the vector-ALU (v_dot4) TQ2_0 kernel instead of the MFMA one.
 bool tq2_on_matrix_cores() {
     static bool v = [] {
         const char* e = getenv("LOCAL_HIP_TQ2_KERNEL");
-        return !(e && e[0] == 'v') && x_limbs() == 2;
+        return !(e && e[0] == 'v');
     }();
     return v;
 }
@@ -749,13 +751,12 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
         free(host_desc);   // staged by the helper
         if (ru != LH_OK) return ru;
     }
-    const int L = x_limbs();
+    const int L = x_limbs(fmt);
     const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L, min_slack);
     int r;
     if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
                                    : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
-    else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
-                    : launch_npos<LH_TQ2_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
+    else r = launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
 }
@@ -794,12 +795,11 @@ int matvec_rows_impl(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer*
         r = lh_launch_matvec_tq2_mfma(ctx, m, pm, px, py, at, ct, n, k, (uint32_t)xstride, (uint32_t)ystride);
     } else {
         MatvecBase single{MatvecProblem{(const uint8_t*)weight->ptr, input->ptr, output->ptr}, (uint32_t)xstride, (uint32_t)ystride};
-        const int L = x_limbs();
+        const int L = x_limbs(fmt);
         const LaunchGeom g = plan(fmt, m, n, k, ctx->cu_count, L, slack);
         if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
                                        : launch_npos<LH_Q4_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
-        else r = L == 2 ? launch_npos<LH_TQ2_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
-                        : launch_npos<LH_TQ2_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
+        else r = launch_npos<LH_TQ2_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g);
     }
     (void)op;
     return r;
