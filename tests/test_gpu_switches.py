@@ -21,6 +21,9 @@ CASES = [
     ({"LOCAL_HIP_MATMUL_SPLITK": "0", "LOCAL_HIP_MATMUL_SKINNY": "0"}, "test_gpu_matmul.py", "decode_batch_matmul or matmul_grouped or tile_boundaries"),
     ({"LOCAL_HIP_ATTN_KERNEL": "valu", "LOCAL_HIP_ATTN_MERGE_ROTATE": "0"}, "test_gpu_attention.py",
      "asymmetric_levels or empty_range or ring_matches or rotated_entry"),
+    ({"LOCAL_HIP_ATTN_OCC": "1", "LOCAL_HIP_ATTN_WAVES_PER_SIMD": "3"}, "test_gpu_attention.py", "batched_matches or split_invariance or asymmetric_levels"),
+    ({"LOCAL_HIP_PREFILL_BM": "64", "LOCAL_HIP_SKINNY_MAX_M": "64", "LOCAL_HIP_MATVEC_WG_PER_CU": "1"}, "test_gpu_matmul.py",
+     "prefill_config or large_tiles or small_batch_layer_config"),
 ]
 
 
