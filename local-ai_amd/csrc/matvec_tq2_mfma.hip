@@ -31,9 +31,6 @@
 
 namespace {
 
-#ifndef LH_TQ2_RING
-#define LH_TQ2_RING 1
-#endif
 constexpr int kL = 2;                        // activation limbs (16-bit block fixed point)
 constexpr int kMaxChunksPerRow = 33;         // 8 blocks * 66 bytes = 528 bytes = 33 chunks of 16 bytes
 constexpr int kStageLoads = 9;               // ceil(16 rows * 33 chunks / 64 lanes)
@@ -42,7 +39,7 @@ constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // pa
 // delivers tile n only after tile n - 1 has been summed, so the waves of a tile stay within a tile of each other and fetch
 // the neighbouring segments of the same rows close together in time; with four slots the shared cache lines were evicted
 // in between and fetched again (1.09 x the bytes with plain loads against 1.03 x, 5.3 against 5.5 TB/s).
-constexpr uint32_t kRing = LH_TQ2_RING;
+constexpr uint32_t kRing = 1;
 constexpr uint32_t kMaxWavesPerWG = 12;       // the largest workgroup launched here
 constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxWavesPerWG * 16 * 4 + (size_t)kMaxWavesPerWG * 2 * kRing * 4;   // partial rows + arrival / generation words per tile of a slot
 constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
