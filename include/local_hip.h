@@ -127,7 +127,14 @@ LH_API void lh_graph_free(lh_graph* graph);
  * kernels.rs:5711-5838 matvec_q4_0{,_into,_f32out,_f32out_into};
  * kernels.rs:5848-6038 matvec_tq2_0{,_into,_f32out,_f32out_into};
  * shaders/matvec_quant.metal:65-155, 173-312.  x is f16; y f16 or f32.
- * cols % 32 (Q4_0) / % 256 (TQ2_0) != 0 -> LH_ERR_INVALID_ARGUMENT. */
+ * cols % 32 (Q4_0) / % 256 (TQ2_0) != 0 -> LH_ERR_INVALID_ARGUMENT.
+ * Numerics: x is taken to 16-bit fixed point per weight block (a block whose
+ * maximum stands out from its other elements gets a second 16-bit level), the
+ * integer products are exact, and the block sums are combined in f32: within
+ * 1e-3 of the reference's f32 dot relative to the output's scale.  A NaN or an
+ * infinity in x makes every output row NaN (the f32 dot would give NaN, or an
+ * infinity where no opposite one cancels it); it is never clamped to a finite
+ * value. */
 LH_API int lh_matvec_q4_0(lh_context* ctx, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
                           uint32_t rows, uint32_t cols);
 LH_API int lh_matvec_q4_0_into(lh_batch* batch, const lh_buffer* matrix, const lh_buffer* vector, lh_buffer* output,
