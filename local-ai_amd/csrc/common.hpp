@@ -211,6 +211,15 @@ __device__ __forceinline__ void lh_rotate_pair(float x0, float x1, uint32_t i, u
 // compiler from folding a preceding multiply into v_fma_mixlo_f16, which rounds the exact
 // product once (a different result in double-rounding cases) and turns -0 into +0.
 __device__ __forceinline__ uint16_t lh_f2h_exact(float f) { asm volatile("" : "+v"(f)); return lh_f2h(f); }
+// x * rms * w of a norm as a rounded f32 value in a register.  Every kernel that evaluates a norm -- stand-alone, as the
+// prologue of a product or as its epilogue -- goes through this, so that none of them has the product contracted into a
+// following addition or narrowed to f16 in one mixed-precision instruction while another has not (the results then
+// differ in the last f16 bit about once in ten thousand values).
+__device__ __forceinline__ float lh_norm_product(float x, float rms, float w) {
+    float p = x * rms * w;
+    asm volatile("" : "+v"(p));
+    return p;
+}
 
 // In-place unnormalised fast Walsh-Hadamard transform over sh[0..d) in LDS with one thread per element; every thread of
 // the workgroup calls it.  Sums and differences only, in a fixed order, so every kernel that uses it produces the same bits.

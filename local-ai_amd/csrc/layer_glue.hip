@@ -46,14 +46,14 @@ __device__ __forceinline__ uint4 rms_apply8(const uint4& v, const uint4& g, cons
     uint32_t wo[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        float lo = lh_h2f((uint16_t)(wv[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
-        float hi = lh_h2f((uint16_t)(wv[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
+        float lo = lh_norm_product(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), rms, lh_h2f((uint16_t)(wg[j] & 0xFFFF)));
+        float hi = lh_norm_product(lh_h2f((uint16_t)(wv[j] >> 16)), rms, lh_h2f((uint16_t)(wg[j] >> 16)));
         if (ADD) {
             const float rlo = lh_h2f((uint16_t)(wr[j] & 0xFFFF)), rhi = lh_h2f((uint16_t)(wr[j] >> 16));
             if (tail) { lo = norm_tail(lo, rlo, tail, scale); hi = norm_tail(hi, rhi, tail, scale); }
             else { lo += rlo; hi += rhi; }
         }
-        wo[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
+        wo[j] = (uint32_t)lh_f2h_exact(lo) | ((uint32_t)lh_f2h_exact(hi) << 16);
     }
     return make_uint4(wo[0], wo[1], wo[2], wo[3]);
 }
@@ -82,9 +82,9 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const uint16_t* in, const
         }
     } else {
         for (uint32_t i = threadIdx.x; i < dim; i += blockDim.x) {
-            float v = h_at(in, row + i) * rms * h_at(w, i);
+            float v = lh_norm_product(h_at(in, row + i), rms, h_at(w, i));
             if (ADD) v = tail ? norm_tail(v, h_at(res, row + i), tail, scale) : v + h_at(res, row + i);
-            out[row + i] = lh_f2h(v);
+            out[row + i] = lh_f2h_exact(v);
         }
     }
 }
@@ -201,10 +201,10 @@ __global__ __launch_bounds__(256) void qk_norm_kernel(const uint16_t* in, uint16
     for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) { const float v = h_at(in, base + j); s += v * v; }
     const float rms = rsqrtf(block_sum(s, scratch) / (float)head_dim + eps);
     if (!ROPE) {
-        for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) out[base + j] = lh_f2h(h_at(in, base + j) * rms * h_at(w, j));
+        for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) out[base + j] = lh_f2h_exact(lh_norm_product(h_at(in, base + j), rms, h_at(w, j)));
         return;
     }
-    for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) normed[j] = lh_f2h(h_at(in, base + j) * rms * h_at(w, j));
+    for (uint32_t j = threadIdx.x; j < head_dim; j += blockDim.x) normed[j] = lh_f2h_exact(lh_norm_product(h_at(in, base + j), rms, h_at(w, j)));
     __syncthreads();
     const uint32_t half_dim = head_dim / 2;
     const uint32_t rope_angles = (uint32_t)((float)head_dim * prf) / 2;

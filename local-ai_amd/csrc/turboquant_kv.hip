@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
         float ss = 0.0f;
         for (uint32_t w = 0; w < d / 64; w++) ss += wsum[w];
         const float rms = rsqrtf(ss / (float)d + p.eps);
-        h = lh_f2h(x * rms * (norm_w ? lh_h2f(norm_w[lane]) : 1.0f));
+        h = lh_f2h_exact(lh_norm_product(x, rms, norm_w ? lh_h2f(norm_w[lane]) : 1.0f));
     }
     if (is_q || is_k) {                                                    // NEOX RoPE on the f16-rounded head (rope.metal:14-61)
         hbuf[lane] = h;

@@ -41,10 +41,10 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
     const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        float lo = lh_h2f((uint16_t)(wa[j] & 0xFFFF)) * rms * lh_h2f((uint16_t)(wg[j] & 0xFFFF));
-        float hi = lh_h2f((uint16_t)(wa[j] >> 16)) * rms * lh_h2f((uint16_t)(wg[j] >> 16));
+        float lo = lh_norm_product(lh_h2f((uint16_t)(wa[j] & 0xFFFF)), rms, lh_h2f((uint16_t)(wg[j] & 0xFFFF)));
+        float hi = lh_norm_product(lh_h2f((uint16_t)(wa[j] >> 16)), rms, lh_h2f((uint16_t)(wg[j] >> 16)));
         if (pro.res != nullptr) { lo += lh_h2f((uint16_t)(wr[j] & 0xFFFF)); hi += lh_h2f((uint16_t)(wr[j] >> 16)); }
-        packed[j] = (uint32_t)lh_f2h(lo) | ((uint32_t)lh_f2h(hi) << 16);
+        packed[j] = (uint32_t)lh_f2h_exact(lo) | ((uint32_t)lh_f2h_exact(hi) << 16);
     }
 }
 
@@ -158,7 +158,7 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
                         const float t = lh_h2f((uint16_t)((packed[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
-                        if (pro.aux2 != nullptr) v[i] = lh_h2f(lh_f2h(t * rms2 * lh_h2f((uint16_t)((wg2[i >> 1] >> (16 * (i & 1))) & 0xFFFF))));
+                        if (pro.aux2 != nullptr) v[i] = lh_h2f(lh_f2h_exact(lh_norm_product(t, rms2, lh_h2f((uint16_t)((wg2[i >> 1] >> (16 * (i & 1))) & 0xFFFF)))));
                         else v[i] = t;
                     }
                 } else if (pro.kind == kXProGeluMul) {
