@@ -12,18 +12,20 @@
 // quantised to fixed point and split into signed 8-bit limbs, one MFMA row per (query head, limb):
 //   K side:  rows = 8 heads x 2 limbs of b*rq and g/2*rq (16-bit block fixed point per head), columns =
 //            16 positions, k = 64 code bytes;  logit = norm_k * (scale_h * int + a * sum(rq_h)).
-//   V side:  rows = 4 heads x 4 limbs (two row sets) of w = exp2(logit - R_h) * norm_v in 31-bit fixed
-//            point, columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share one
-//            accumulator because their coefficients are folded into w before quantisation.  The
+//   V side:  rows = 8 heads x 2 limbs of w = exp2(logit - R_h) * norm_v in 16-bit fixed point relative to
+//            the head's largest weight of the current group of 64 positions (a power-of-two scale, round
+//            to nearest), columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share
+//            one accumulator because their coefficients are folded into w before quantisation.  The
 //            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
 //            byte transposes.
 // One workgroup owns a chunk of positions and walks it in aligned groups of 64: the K wave produces the
 // softmax weights of a group, a V wave per 256 output dims (one group behind, one barrier per group)
-// turns them into limbs and accumulates.  Splitting the roles keeps each wave under 256 registers, so
-// two waves share a SIMD and fill each other's stalls.  The integer V accumulators persist across groups:
-// the softmax reference R_h is only moved (and the accumulators folded into the float outputs) when a
-// weight would leave the fixed-point range, which the 31-bit width makes rare.  Partials (R, l, acc)
-// per chunk go to the workspace for the merge kernel.
+// turns them into limbs, multiplies and adds the group's integer sums to its float outputs with the group's
+// scale.  A scale per head and group keeps the long tail of a soft distribution: a weight is only compared
+// with the 63 around it, never with a maximum seen thousands of positions earlier.  The softmax reference
+// R_h only keeps exp2 in range and follows the running maximum lazily.  Splitting the roles lets two or
+// three waves share a SIMD and fill each other's stalls.  Partials (R, l, acc) per chunk go to the
+// workspace for the merge kernel.
 #include "attention_tq.hpp"
 #include <algorithm>
 #include <cstdlib>
@@ -33,6 +35,7 @@ namespace {
 using namespace lh_attn;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
 
@@ -41,8 +44,7 @@ constexpr int kMaxGroupHeads = 8;      // query heads per KV head served by the 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kQmax = 32639.0f;      // 127 * 256 + 127
-constexpr float kVQ = 2.0e9f;          // V-side weights: fixed point with 4 signed limbs, below 127 * 2^24
-constexpr int kHeadroom = 6;           // log2 of how far a weight may exceed the reference before it is moved
+constexpr float kHeadroom = 32.0f;     // log2 of how far a weight may exceed the softmax reference before that moves
 
 __device__ __forceinline__ u32x4_t ld16(gptr_t p) {
     typedef u32x4_t __attribute__((aligned(4))) u32x4_a4;
@@ -79,12 +81,11 @@ struct AttnShared {
     uint8_t rqop[12 * NH][64][16]; // K-side A operands per (code half, plane, field) and lane
     float4 norm[kGroup];           // K wave: (norm_k*log2e, mask bias, norm_v, -) per group position
     float4 ww[2][2][64];           // [buffer][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
-    float wq[2];                   // [buffer]: fixed-point scale of those weights
-    uint8_t wx[NH][3][2][1024];    // [V wave][plane][row set]: that wave's A operands (weights as limbs)
+    float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this group into [-1, 1], value of one integer step)
+    uint8_t wx[NH][3][1024];       // [V wave][plane]: that wave's A operands (weights as limbs)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
-    float unit_old[2];             // [buffer]: value of one integer step of the accumulators gathered so far
-    uint32_t moved[2];             // [buffer]: the reference moved before this group: fold, then rescale
-    float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads], fin_unit;
+    uint32_t moved[2];             // [buffer]: the reference moved before this group: rescale the outputs
+    float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads];
     float maxabs[kMaxGroupHeads], sum[kMaxGroupHeads];
 };
 
@@ -108,7 +109,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     const float* rq_base = a.rq + ((size_t)qi * p.num_q_heads + (size_t)kvh * group) * kHeadDim;
 
     const float cmax_k = fmaxf(fmaxf(fabsf(beta), fabsf(0.5f * gam)), has_delta ? fabsf(delta) : 0.0f);
-    const float cmax_v = fmaxf(fmaxf(fabsf(beta), fabsf(gam)), has_delta ? fabsf(delta) : 0.0f);
+    const float cmax_v = cmax_k;   // the V side also takes plane 1 at its bit position 2f + 1, i.e. with gam / 2
 
     // ---- the workgroup's chunk of positions
     uint32_t lo, hi, lane_base;
@@ -136,6 +137,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // weights are masked to zero.
     auto is_valid = [](const GroupGeom& gg, uint32_t idx) { return idx - gg.vlo < gg.vhi - gg.vlo; };
     const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
+    const float v_unit = cmax_v * (1.0f / kQmax);   // value of one integer step of a weight limb pair at scale 1
     // Roles rotate with the workgroup index, so that the kinds of wave mix on every SIMD.
     const uint32_t role = NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) % 3u;   // 0: K wave; 1, 2: V wave of code half role - 1
     const bool k_role = role == 0;
@@ -255,43 +257,43 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
         gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
         float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
-        float vref = 0.0f, wlimit = -1.0f, wq = 0.0f;   // weights up to wlimit = 2^kHeadroom * vref map to kVQ
-        uint32_t since_move = 0;
 
         if (any) {
             GroupGeom gg = geom(g_first);
-            u32x4_t kw[NH][4], kwn[NH][4];   // K codes of the current group and of the next one (a full step of prefetch distance)
-            float nk, nv, nkn = 0.0f, nvn = 0.0f;
+            // K codes and norms of the current group.  Those of the next group are requested into the same registers as soon
+            // as a tile's codes have been taken apart (a step of prefetch distance, no second register set, no copies).
+            // `KIND` says what follows the group: 0 nothing, 1 a group that is certainly complete (every group between the
+            // first and the last of a chunk is), 2 a group that may be partial.
+            u32x4_t kw[NH][4];
+            float nk, nv;
             const uint32_t klane = pcol * stride + 16 * g, nlane = lane * nstride;
-            auto load_k = [&](const GroupGeom& G_, u32x4_t (&kw_)[NH][4], float& nk_, float& nv_) {
+            auto load_tile = [&](bool full, const GroupGeom& G_, int q) {
                 gptr_t kb = krec0 + (size_t)G_.pb * stride;
-                gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
-                if (G_.full) {
 #pragma unroll
-                    for (int hf = 0; hf < NH; hf++)
-#pragma unroll
-                        for (int q = 0; q < 4; q++) kw_[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
-                    nk_ = ld_norm(knb + nlane);
-                    nv_ = ld_norm(vnb + nlane);
-                } else {
-#pragma unroll
-                    for (int hf = 0; hf < NH; hf++)
-#pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            kw_[hf][q] = (u32x4_t){0u, 0u, 0u, 0u};
-                            if (is_valid(G_, 16 * q + pcol)) kw_[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
-                        }
-                    nk_ = nv_ = 0.0f;
-                    if (is_valid(G_, lane)) { nk_ = ld_norm(knb + nlane); nv_ = ld_norm(vnb + nlane); }
+                for (int hf = 0; hf < NH; hf++) {
+                    if (full) kw[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
+                    else {
+                        kw[hf][q] = (u32x4_t){0u, 0u, 0u, 0u};
+                        if (is_valid(G_, 16 * q + pcol)) kw[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
+                    }
                 }
             };
-            load_k(gg, kw, nk, nv);
+            auto load_norms = [&](bool full, const GroupGeom& G_) {
+                gptr_t knb = kn0 + (size_t)G_.pb * nstride, vnb = vn0 + (size_t)G_.pb * nstride;
+                if (full) { nk = ld_norm(knb + nlane); nv = ld_norm(vnb + nlane); }
+                else {
+                    nk = nv = 0.0f;
+                    if (is_valid(G_, lane)) { nk = ld_norm(knb + nlane); nv = ld_norm(vnb + nlane); }
+                }
+            };
+#pragma unroll
+            for (int q = 0; q < 4; q++) load_tile(gg.full, gg, q);
+            load_norms(gg.full, gg);
 
-            for (uint32_t G = g_first; G <= g_last; G++) {
+            auto step = [&](auto kind_tag, uint32_t G) {
+                constexpr int KIND = decltype(kind_tag)::value;
                 const uint32_t buf = (G - g_first) & 1u;
-                const bool more = G < g_last;
-                const GroupGeom gnext = geom(more ? G + 1 : G);
-                if (more) load_k(gnext, kwn, nkn, nvn);
+                const GroupGeom gnext = geom(KIND ? G + 1 : G);
 
                 // ---- norms of the group -> LDS
                 {
@@ -299,6 +301,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     __builtin_amdgcn_wave_barrier();
                     sh.norm[lane] = make_float4(nk * kLog2e, valid ? 0.0f : -INFINITY, valid ? nv : 0.0f, 0.0f);
                     __builtin_amdgcn_wave_barrier();
+                    if constexpr (KIND != 0) load_norms(KIND == 1, gnext);
                 }
 
                 // ---- logits of 4 tiles x (this lane's column position, heads g and g + 4)
@@ -342,6 +345,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                             acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
                         }
                     }
+                    if constexpr (KIND != 0) load_tile(KIND == 1, gnext, q);   // the tile's code registers are free
                     const float4 nrm = sh.norm[16 * q + pcol];
                     vn[q] = nrm.z;
 #pragma unroll
@@ -353,62 +357,57 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     }
                 }
 
-                // ---- softmax weights relative to the running reference R; R moves only when the fixed-point range is left
-                float ew[4][2], ww[4][2];
-                auto weights = [&]() {   // returns whether any weight of the wave leaves the fixed-point range (or is NaN)
-                    float wm = 0.0f;
+                // ---- softmax weights relative to the reference R, which follows the running maximum lazily: it moves
+                //      when a logit of the group exceeds it by more than kHeadroom (always in the first group)
+                float mq[2];
 #pragma unroll
-                    for (int q = 0; q < 4; q++)
-#pragma unroll
-                        for (int hs = 0; hs < 2; hs++) {
-                            ew[q][hs] = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
-                            ww[q][hs] = ew[q][hs] * vn[q];
-                            wm = fmaxf(wm, ww[q][hs]);
-                        }
-                    return __builtin_amdgcn_ballot_w64(!(wm <= wlimit)) != 0;
-                };
-                const bool out_of_range = weights();
-                const bool move = out_of_range || since_move >= 256u;   // uniform; true for the first group (wlimit starts negative)
+                for (int hs = 0; hs < 2; hs++) mq[hs] = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
+                const bool move = __builtin_amdgcn_ballot_w64(mq[0] > R[0] + kHeadroom || mq[1] > R[1] + kHeadroom) != 0;   // uniform
                 if (move) {
-                    if (lane == 0) sh.unit_old[buf] = wq > 0.0f ? cmax_v / wq : 0.0f;
-                    float vm = fmaxf(fmaxf(vn[0], vn[1]), fmaxf(vn[2], vn[3]));
-                    vm = lh_group_max(vm, 64);
-                    vref = fmaxf(vref, vm);
-                    wlimit = vref * (float)(1 << kHeadroom);
-                    wq = wlimit > 0.0f ? kVQ / wlimit : 0.0f;
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        float m = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
-                        m = lh_group_max(m, 16);
-                        const float rn = fmaxf(R[hs], m);
-                        const float fsc = __builtin_amdgcn_exp2f(R[hs] - rn);   // 0 for the first group
+                        const float rn = fmaxf(R[hs], lh_group_max(mq[hs], 16));
+                        const float fsc = rn > R[hs] ? __builtin_amdgcn_exp2f(R[hs] - rn) : 1.0f;   // 0 for the first group
                         R[hs] = rn;
                         l_run[hs] *= fsc;
                         w_run[hs] *= fsc;
                         if (pcol == 0) sh.fsc[buf][g + 4 * hs] = fsc;
                     }
-                    (void)weights();
-                    since_move = 0;
                 }
                 if (lane == 0) sh.moved[buf] = move ? 1u : 0u;
-                since_move++;
+                float ww[4][2];
 #pragma unroll
-                for (int q = 0; q < 4; q++)
+                for (int hs = 0; hs < 2; hs++) {
+                    float wm = 0.0f;
 #pragma unroll
-                    for (int hs = 0; hs < 2; hs++) { l_run[hs] += ew[q][hs]; w_run[hs] += ww[q][hs]; }
+                    for (int q = 0; q < 4; q++) {
+                        const float ew = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
+                        ww[q][hs] = ew * vn[q];
+                        l_run[hs] += ew;
+                        w_run[hs] += ww[q][hs];
+                        wm = fmaxf(wm, fabsf(ww[q][hs]));
+                    }
+                    // The head's scale for this group: the power of two that takes its largest weight into [0.5, 1).
+                    // Nothing representable (zero, subnormal or non-finite maximum): scale and step 0, the group adds
+                    // nothing to the integer sums (a non-finite weight still reaches the output through w_run).
+                    wm = lh_group_max(wm, 16);
+                    const uint32_t e = __float_as_uint(wm) & 0x7F800000u;
+                    const bool ok = e != 0u && e < (253u << 23);
+                    const float sc = ok ? __uint_as_float((253u << 23) - e) : 0.0f;
+                    const float un = ok ? __uint_as_float(e + (1u << 23)) * v_unit : 0.0f;
+                    if (pcol == 0) sh.wsc[buf][g + 4 * hs] = make_float2(sc, un);
+                }
 
                 // ---- hand the weights to the V wave
 #pragma unroll
                 for (int hs = 0; hs < 2; hs++) sh.ww[buf][hs][lane] = make_float4(ww[0][hs], ww[1][hs], ww[2][hs], ww[3][hs]);
-                if (lane == 0) sh.wq[buf] = wq;
                 __syncthreads();   // hand-over of buffer `buf`; also: the V wave is done with the buffer written next
                 gg = gnext;
-#pragma unroll
-                for (int hf = 0; hf < NH; hf++)
-#pragma unroll
-                    for (int q = 0; q < 4; q++) kw[hf][q] = kwn[hf][q];
-                nk = nkn; nv = nvn;
-            }
+            };
+            uint32_t G = g_first;
+            for (; G + 1 < g_last; G++) step(std::integral_constant<int, 1>{}, G);
+            if (G < g_last) { step(std::integral_constant<int, 2>{}, G); G++; }
+            step(std::integral_constant<int, 0>{}, G);
         }
 #pragma unroll
         for (int hs = 0; hs < 2; hs++) {
@@ -416,69 +415,54 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             const float w_tot = lh_group_sum(w_run[hs], 16);
             if (pcol == 0) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs]; }
         }
-        if (lane == 0) sh.fin_unit = wq > 0.0f ? cmax_v / wq : 0.0f;
         __syncthreads();
     } else {
         // =================================================================== V wave
         gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * vhalf;
-        v4i acc[4][4][2];      // [code byte e][field f][row set]: integer accumulators, rows = 4 limbs of head g + 4 * set
-        float outv[4][4][2];   // folded accumulators: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
+        float outv[4][4][2];   // [code byte e][field f][head set]: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
 #pragma unroll
         for (int e = 0; e < 4; e++)
 #pragma unroll
             for (int f = 0; f < 4; f++)
 #pragma unroll
-                for (int hs = 0; hs < 2; hs++) { acc[e][f][hs] = (v4i){0, 0, 0, 0}; outv[e][f][hs] = 0.0f; }
-        // integer accumulators -> float outputs, accumulators cleared
-        auto fold = [&](float unit) {
+                for (int hs = 0; hs < 2; hs++) outv[e][f][hs] = 0.0f;
+        // The planes are summed as 0/1 bits, but what is meant is the centred bit b - 1/2 (plane 2: b0*b1 - 1/4): per head
+        // and group one more MFMA per plane against constant bytes gives the sum of the quantised weights themselves, and
+        // sctr collects (1/2, 1, 1/4) of them.  Taking that off the outputs (and only the rest of the table's constant
+        // term times the exact sum of weights on) makes the rounding errors of the weights enter every output dim with
+        // a random sign: a common offset of all dims would be gathered into single elements by the rotation that follows.
+        float sctr[2] = {0.0f, 0.0f};
+        // Plane coefficients relative to the largest one, times kQmax / 32767: a weight scaled into [-1, 1] times this,
+        // converted to a signed normalised 16-bit number, is at most kQmax in magnitude and splits into two int8 limbs.
+        float cfn[3];
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-#pragma unroll
-                for (int f = 0; f < 4; f++)
-#pragma unroll
-                    for (int hs = 0; hs < 2; hs++) {
-                        const v4i A = acc[e][f][hs];
-                        const float v = ((float)A[0] + 256.0f * (float)A[1]) + (65536.0f * (float)A[2] + 16777216.0f * (float)A[3]);
-                        outv[e][f][hs] = __builtin_fmaf(v, unit * (1.0f / (float)(1 << (2 * f))), outv[e][f][hs]);
-                        acc[e][f][hs] = (v4i){0, 0, 0, 0};
-                    }
-        };
+        for (int pl = 0; pl < 3; pl++) cfn[pl] = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv_cmax_v * (kQmax / 32767.0f);
 
         if (any) {
             GroupGeom gg = geom(g_first);
             uint32_t vx[4][4];
             const uint32_t vlane = 4 * g * stride + 4 * pcol;
-            auto load_v = [&](const GroupGeom& G_) {
+            auto load_v = [&](bool full, const GroupGeom& G_) {
                 gptr_t vb = vrec0 + (size_t)G_.pb * stride;
-                if (G_.full) {
 #pragma unroll
-                    for (int m = 0; m < 4; m++)
+                for (int m = 0; m < 4; m++)
 #pragma unroll
-                        for (int qq = 0; qq < 4; qq++) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
-                } else {
-#pragma unroll
-                    for (int m = 0; m < 4; m++)
-#pragma unroll
-                        for (int qq = 0; qq < 4; qq++) {
+                    for (int qq = 0; qq < 4; qq++) {
+                        if (full) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
+                        else {
                             vx[m][qq] = 0u;
                             if (is_valid(G_, 16 * qq + 4 * g + m)) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
                         }
-                }
+                    }
             };
-            load_v(gg);
+            load_v(gg.full, gg);
 
-            // One group.  The MAY_FOLD = false copy is the steady state: it returns false right after the barrier when the
-            // K wave moved the reference; the MAY_FOLD = true copy then handles that group without a second barrier.
-            // (Keeping the rare path out of the hot loop keeps the accumulators in place.)
-            auto step = [&](auto may_fold_tag, uint32_t G, bool wait) -> bool {
-                constexpr bool MAY_FOLD = decltype(may_fold_tag)::value;
+            // One group; KIND as in the K wave: 0 nothing follows, 1 a complete group follows, 2 a group that may be partial.
+            auto step = [&](auto kind_tag, uint32_t G) {
+                constexpr int KIND = decltype(kind_tag)::value;
                 const uint32_t buf = (G - g_first) & 1u;
-                const bool more = G < g_last;
-                if (wait) __syncthreads();
-                const bool moved = __builtin_amdgcn_readfirstlane(sh.moved[buf]) != 0;
-                if (moved) {
-                    if constexpr (!MAY_FOLD) return false;
-                    fold(sh.unit_old[buf]);
+                __syncthreads();   // the K wave's weights of this group
+                if (__builtin_amdgcn_readfirstlane(sh.moved[buf]) != 0) {   // rare: the reference moved
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
                         const float fsc = sh.fsc[buf][g + 4 * hs];
@@ -486,32 +470,32 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                         for (int e = 0; e < 4; e++)
 #pragma unroll
                             for (int f = 0; f < 4; f++) outv[e][f][hs] *= fsc;
+                        sctr[hs] *= fsc;
                     }
                 }
-                // ---- weights -> 31-bit fixed point, one word of 4 signed limbs per (tile, head, plane); byte transpose to
-                //      "limb i over the four tiles" and hand each word to the lane that owns it as an MFMA row:
-                //      lane (column 4A+B, row group g) feeds row 4g + i of k-group A, word B.
+                // ---- weights -> 16-bit fixed point at the head's scale of this group, two signed limbs; a lane holds the
+                //      weights of column position pcol of the four tiles, i.e. one k word of the MFMA's A operand:
+                //      lane (column 4A+B, row group g) feeds rows 4g + 2 * set + limb of k-group A, word B.
+                float uf[2][4];   // [head set][field]: value of one integer step of the accumulators of this group
                 {
                     const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
-                    const float wqv = sh.wq[buf] * inv_cmax_v;
                     __builtin_amdgcn_wave_barrier();
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
                         const float4 wv = sh.ww[buf][hs][lane];
-                        const float wws[4] = {wv.x, wv.y, wv.z, wv.w};
+                        const float2 ws = sh.wsc[buf][g + 4 * hs];
+                        uf[hs][0] = ws.y; uf[hs][1] = ws.y * 0.25f; uf[hs][2] = uf[hs][3] = ws.y * 0.0625f;   // field 3 is read at field 2's place
 #pragma unroll
                         for (int pl = 0; pl < nplanes; pl++) {
-                            const float cq = (pl == 0 ? beta : pl == 1 ? gam : delta) * wqv;
-                            uint32_t lw[4], tr[4];
-#pragma unroll
-                            for (int q = 0; q < 4; q++) {
-                                const int qv = (int)(wws[q] * cq);                    // truncation: |qv| <= kVQ < 127 * 2^24
-                                lw[q] = ((uint32_t)qv + 0x00808080u) ^ 0x00808080u;    // bytes = signed limbs, least significant first
-                            }
-                            transpose4x4(lw, tr);
-                            uint8_t* dst = &sh.wx[vhalf][pl][hs][(16 * A_ + 4 * g) * 16 + 4 * B_];
-#pragma unroll
-                            for (int i = 0; i < 4; i++) *reinterpret_cast<uint32_t*>(dst + 16 * i) = tr[i];
+                            const float cq = cfn[pl] * ws.x;
+                            const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.x * cq, wv.y * cq));
+                            const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.z * cq, wv.w * cq));
+                            // per 16-bit half: low byte = signed low limb, high byte = what is left of it
+                            const uint32_t t01 = __builtin_bit_cast(uint32_t, (us2_t)(__builtin_bit_cast(us2_t, p01) + (us2_t){0x80, 0x80})) ^ 0x00800080u;
+                            const uint32_t t23 = __builtin_bit_cast(uint32_t, (us2_t)(__builtin_bit_cast(us2_t, p23) + (us2_t){0x80, 0x80})) ^ 0x00800080u;
+                            uint8_t* dst = &sh.wx[vhalf][pl][(16 * A_ + 4 * g + 2 * hs) * 16 + 4 * B_];
+                            *reinterpret_cast<uint32_t*>(dst) = __builtin_amdgcn_perm(t23, t01, 0x06040200u);        // low limbs of tiles 0..3
+                            *reinterpret_cast<uint32_t*>(dst + 16) = __builtin_amdgcn_perm(t23, t01, 0x07050301u);   // high limbs
                         }
                     }
                     __builtin_amdgcn_wave_barrier();
@@ -519,43 +503,58 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 uint32_t y[4][4];   // [word m][code byte e]: byte e of positions 16qq + 4g + m, qq = 0..3
 #pragma unroll
                 for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
-                if (more) load_v(geom(G + 1));   // the V registers are free
+                if constexpr (KIND != 0) load_v(KIND == 1, geom(G + 1));   // the V registers are free
+                v4i acc[4][4];      // [code byte e][field f]: the group's integer sums, rows = heads g, g + 4 x 2 limbs
+                v4i csum;           // 4 x the centre: 2 sum(plane 0 weights) + 4 sum(plane 1 weights, which are halved) + sum(plane 2 weights)
 #pragma unroll
                 for (int pl = 0; pl < nplanes; pl++) {
-                    const v4i wop0 = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][0][lane * 16]);
-                    const v4i wop1 = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][1][lane * 16]);
+                    const v4i wop = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][lane * 16]);
+                    {
+                        const int cb = pl == 0 ? 0x02020202 : pl == 1 ? 0x04040404 : 0x01010101;
+                        csum = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, (v4i){cb, cb, cb, cb}, pl == 0 ? (v4i){0, 0, 0, 0} : csum, 0, 0, 0);
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        uint32_t yp[4];   // the plane's bit of every field at the even bit positions
+                        // Plane 0 and the product plane sit at bit 2f of a field, plane 1 at bit 2f + 1 (its coefficient is
+                        // halved).  Field 3 is taken two bits down, at field 2's place: 0x80 would be a negative int8.
+                        uint32_t yp[4], yd[4];
 #pragma unroll
-                        for (int m = 0; m < 4; m++) yp[m] = pl == 0 ? y[m][e] : pl == 1 ? y[m][e] >> 1 : y[m][e] & (y[m][e] >> 1);
+                        for (int m = 0; m < 4; m++) {
+                            yp[m] = pl == 2 ? y[m][e] & (y[m][e] >> 1) : y[m][e];
+                            yd[m] = yp[m] >> 2;
+                        }
 #pragma unroll
                         for (int f = 0; f < 4; f++) {
+                            const uint32_t mask = (pl == 1 ? 0x02020202u : 0x01010101u) << (f == 3 ? 4 : 2 * f);
                             v4i b;
 #pragma unroll
-                            for (int m = 0; m < 4; m++) b[m] = (int)(yp[m] & (0x01010101u << (2 * f)));
-                            acc[e][f][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop0, b, acc[e][f][0], 0, 0, 0);
-                            acc[e][f][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop1, b, acc[e][f][1], 0, 0, 0);
+                            for (int m = 0; m < 4; m++) b[m] = (int)((f == 3 ? yd[m] : yp[m]) & mask);
+                            acc[e][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, b, pl == 0 ? (v4i){0, 0, 0, 0} : acc[e][f], 0, 0, 0);
                         }
                     }
                 }
-                return true;
-            };
-
-            uint32_t G = g_first;
-            bool wait = true;
-            while (G <= g_last) {
-                step(std::true_type{}, G, wait);
-                G++;
-                wait = true;
-                while (G <= g_last) {
-                    if (!step(std::false_type{}, G, true)) { wait = false; break; }
-                    G++;
+                // ---- the group's sums into the float outputs
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int f = 0; f < 4; f++)
+#pragma unroll
+                        for (int hs = 0; hs < 2; hs++) {
+                            const int t = (int)(((uint32_t)acc[e][f][2 * hs + 1] << 8) + (uint32_t)acc[e][f][2 * hs]);
+                            outv[e][f][hs] = __builtin_fmaf((float)t, uf[hs][f], outv[e][f][hs]);
+                        }
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    const int t = (int)(((uint32_t)csum[2 * hs + 1] << 8) + (uint32_t)csum[2 * hs]);
+                    sctr[hs] = __builtin_fmaf((float)t, 0.25f * uf[hs][0], sctr[hs]);
                 }
-            }
+            };
+            uint32_t G = g_first;
+            for (; G + 1 < g_last; G++) step(std::integral_constant<int, 1>{}, G);
+            if (G < g_last) { step(std::integral_constant<int, 2>{}, G); G++; }
+            step(std::integral_constant<int, 0>{}, G);
         }
         __syncthreads();   // the K wave's totals
-        fold(sh.fin_unit);
 
         // ---- the workgroup's result: final output (one split) or a partial record for the merge kernel
 #pragma unroll
@@ -564,7 +563,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             if (h >= group) continue;
             const float l_tot = sh.fin_l[h], w_tot = sh.fin_w[h];
             const uint32_t qh = kvh * group + h;
-            const float bias = alpha * w_tot;
+            const float bias = (alpha + 0.5f * (beta + gam) + (has_delta ? 0.25f * delta : 0.0f)) * w_tot - sctr[hs];
             if (nsplit == 1) {
                 float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 16 * pcol;
                 const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
