@@ -350,9 +350,10 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     vn[q] = nrm.z;
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        const int t_lo = (acc1[2 * hs] << 2) + acc4[2 * hs];
-                        const int t_hi = (acc1[2 * hs + 1] << 2) + acc4[2 * hs + 1];
-                        const float inner = (float)(t_lo + (t_hi << 8)) * cs[hs] + ca[hs];
+                        // three shift-adds: limbs first, then the two field scales
+                        const uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
+                        const uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
+                        const float inner = (float)(int)((t1 << 2) + t4) * cs[hs] + ca[hs];
                         lg[q][hs] = nrm.x * inner + nrm.y;
                     }
                 }
@@ -362,7 +363,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 float mq[2];
 #pragma unroll
                 for (int hs = 0; hs < 2; hs++) mq[hs] = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
-                const bool move = __builtin_amdgcn_ballot_w64(mq[0] > R[0] + kHeadroom || mq[1] > R[1] + kHeadroom) != 0;   // uniform
+                const bool move = __builtin_amdgcn_ballot_w64(fmaxf(mq[0] - R[0], mq[1] - R[1]) > kHeadroom) != 0;   // uniform
                 if (move) {
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
@@ -390,8 +391,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     // The head's scale for this group: the power of two that takes its largest weight into [0.5, 1).
                     // Nothing representable (zero, subnormal or non-finite maximum): scale and step 0, the group adds
                     // nothing to the integer sums (a non-finite weight still reaches the output through w_run).
-                    wm = lh_group_max(wm, 16);
-                    const uint32_t e = __float_as_uint(wm) & 0x7F800000u;
+                    // (wm is non-negative or NaN: its bit pattern orders like an unsigned integer, NaN on top)
+                    const uint32_t e = lh_group_max_u(__float_as_uint(wm), 16) & 0x7F800000u;
                     const bool ok = e != 0u && e < (253u << 23);
                     const float sc = ok ? __uint_as_float((253u << 23) - e) : 0.0f;
                     const float un = ok ? __uint_as_float(e + (1u << 23)) * v_unit : 0.0f;

@@ -186,6 +186,16 @@ __device__ __forceinline__ float lh_group_max(float v, int width) {
     if (width > 32) v = fmaxf(v, lh_swap32_f(v));
     return v;
 }
+// Maximum of unsigned values (also of non-negative floats taken as bit patterns) over aligned groups of `width` lanes.
+__device__ __forceinline__ uint32_t lh_group_max_u(uint32_t v, int width) {
+    if (width > 1) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR1>((int)v));
+    if (width > 2) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR2>((int)v));
+    if (width > 4) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_HALF_MIRROR>((int)v));
+    if (width > 8) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_ROW_MIRROR>((int)v));
+    if (width > 16) v = max(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x1F | (16 << 10)));
+    if (width > 32) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
+    return v;
+}
 __device__ __forceinline__ int lh_group_sum_i(int v, int width) {
     if (width > 1) v += lh_dpp_i<LH_DPP_QUAD_XOR1>(v);
     if (width > 2) v += lh_dpp_i<LH_DPP_QUAD_XOR2>(v);

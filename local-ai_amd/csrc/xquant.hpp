@@ -64,16 +64,6 @@ struct XResidual {
 };
 constexpr float kXOutlier = 32.0f;
 
-__device__ __forceinline__ uint32_t lh_group_max_u(uint32_t v, int width) {
-    if (width > 1) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR1>((int)v));
-    if (width > 2) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_QUAD_XOR2>((int)v));
-    if (width > 4) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_HALF_MIRROR>((int)v));
-    if (width > 8) v = max(v, (uint32_t)lh_dpp_i<LH_DPP_ROW_MIRROR>((int)v));
-    if (width > 16) v = max(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x1F | (16 << 10)));
-    if (width > 32) v = max(v, (uint32_t)__shfl_xor((int)v, 32, 64));
-    return v;
-}
-
 // ---- activation quantisation into LDS ----------------------------------------
 // xq[l][K/4]: limb l of elements 4i..4i+3 packed into one dword (signed bytes);
 // xs[K/G]: float scale of each group of G elements (G = weight block size).
