@@ -73,18 +73,20 @@ struct GroupGeom {
     bool full;
 };
 
-// One workgroup = two waves on one chunk of positions: the "K wave" turns K codes into softmax weights (as MFMA row
-// operands in LDS), the "V wave" multiplies them with the V codes.  The K wave runs one group ahead; one workgroup
-// barrier per group hands over a double-buffered operand set plus the rare "reference moved" message.
-template <int NH>   // NH = 64-byte halves of a position's code (head_dim / 256) = number of V waves
+// One workgroup = two waves on one chunk of positions: the "K wave" turns K codes into softmax weights, the "V wave"
+// multiplies them with the V codes.  The K wave runs one hand-over ahead; one workgroup barrier per hand-over passes a
+// double-buffered set of weights, their scales and the rare "reference moved" message.  A hand-over is one group of 64
+// positions (PS = 1: short chunks, where the pipeline's fill and drain count) or an aligned pair of groups (PS = 2: long
+// chunks, where halving the per-hand-over work -- scales, the integer sums' way into the float outputs -- counts).
+template <int NH, int PS>   // NH = 64-byte halves of a position's code (head_dim / 256) = number of V waves; PS = groups per hand-over
 struct AttnShared {
     uint8_t rqop[12 * NH][64][16]; // K-side A operands per (code half, plane, field) and lane
     float4 norm[kGroup];           // K wave: (norm_k*log2e, mask bias, norm_v, -) per group position
-    float4 ww[2][2][64];           // [buffer][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
-    float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this group into [-1, 1], value of one integer step)
+    float4 ww[2][PS][2][64];       // [buffer][group of the pair][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
+    float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this pair into [-1, 1], value of one integer step)
     uint8_t wx[NH][3][1024];       // [V wave][plane]: that wave's A operands (weights as limbs)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
-    uint32_t moved[2];             // [buffer]: the reference moved before this group: rescale the outputs
+    uint32_t moved[2];             // [buffer]: the reference moved within this pair: rescale the outputs
     float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads];
     float maxabs[kMaxGroupHeads], sum[kMaxGroupHeads];
 };
@@ -93,8 +95,8 @@ struct AttnShared {
 // HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
 // ONE_KV: a single KV head (the measured configuration and the reference model): the distance between positions is a
 // compile-time constant, so the loads of a group take immediate offsets instead of per-load address arithmetic.
-template <int NPL, int HD, bool ONE_KV>
-__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256)>& sh, float alpha, float beta,
+template <int NPL, int HD, bool ONE_KV, int PS>
+__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>& sh, float alpha, float beta,
                                                float gam, float delta) {
     auto& s_rqop = sh.rqop;
     auto& s_maxabs = sh.maxabs;
@@ -290,9 +292,16 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             for (int q = 0; q < 4; q++) load_tile(gg.full, gg, q);
             load_norms(gg.full, gg);
 
-            auto step = [&](auto kind_tag, uint32_t G) {
+            // Two groups of 64 positions (an aligned pair) share one fixed-point scale per head and one hand-over to the V wave.
+            float ww[PS][4][2];             // [group of the pair][tile][head set]: the pair's weights
+            float wm[2] = {0.0f, 0.0f};     // largest |weight| of the pair so far, per head set
+            float fsc_acc[2] = {1.0f, 1.0f};   // by how much the reference has moved within the pair
+            bool moved_any = false;
+
+            // One group: logits, reference check, weights into wout.  `second`: the pair's first group has been done (its
+            // weights in ww[0] follow the reference if that moves now).
+            auto group_core = [&](auto kind_tag, uint32_t G, float (&wout)[4][2], bool second) {
                 constexpr int KIND = decltype(kind_tag)::value;
-                const uint32_t buf = (G - g_first) & 1u;
                 const GroupGeom gnext = geom(KIND ? G + 1 : G);
 
                 // ---- norms of the group -> LDS
@@ -372,43 +381,90 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                         R[hs] = rn;
                         l_run[hs] *= fsc;
                         w_run[hs] *= fsc;
-                        if (pcol == 0) sh.fsc[buf][g + 4 * hs] = fsc;
+                        fsc_acc[hs] *= fsc;
+                        wm[hs] *= fsc;
+                        if (PS == 2 && second) {
+#pragma unroll
+                            for (int q = 0; q < 4; q++) ww[0][q][hs] *= fsc;
+                        }
                     }
+                    moved_any = true;
                 }
-                if (lane == 0) sh.moved[buf] = move ? 1u : 0u;
-                float ww[4][2];
 #pragma unroll
                 for (int hs = 0; hs < 2; hs++) {
-                    float wm = 0.0f;
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         const float ew = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
-                        ww[q][hs] = ew * vn[q];
+                        wout[q][hs] = ew * vn[q];
                         l_run[hs] += ew;
-                        w_run[hs] += ww[q][hs];
-                        wm = fmaxf(wm, fabsf(ww[q][hs]));
+                        w_run[hs] += wout[q][hs];
+                        wm[hs] = fmaxf(wm[hs], fabsf(wout[q][hs]));
                     }
-                    // The head's scale for this group: the power of two that takes its largest weight into [0.5, 1).
-                    // Nothing representable (zero, subnormal or non-finite maximum): scale and step 0, the group adds
+                }
+                gg = gnext;
+            };
+            // The pair's scales and the hand-over.
+            auto finish_pair = [&](uint32_t P) {
+                const uint32_t buf = (P - (PS == 2 ? g_first >> 1 : g_first)) & 1u;
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    // The head's scale for this pair: the power of two that takes its largest weight into [0.5, 1).
+                    // Nothing representable (zero, subnormal or non-finite maximum): scale and step 0, the pair adds
                     // nothing to the integer sums (a non-finite weight still reaches the output through w_run).
                     // (wm is non-negative or NaN: its bit pattern orders like an unsigned integer, NaN on top)
-                    const uint32_t e = lh_group_max_u(__float_as_uint(wm), 16) & 0x7F800000u;
+                    const uint32_t e = lh_group_max_u(__float_as_uint(wm[hs]), 16) & 0x7F800000u;
                     const bool ok = e != 0u && e < (253u << 23);
                     const float sc = ok ? __uint_as_float((253u << 23) - e) : 0.0f;
                     const float un = ok ? __uint_as_float(e + (1u << 23)) * v_unit : 0.0f;
-                    if (pcol == 0) sh.wsc[buf][g + 4 * hs] = make_float2(sc, un);
+                    if (pcol == 0) {
+                        sh.wsc[buf][g + 4 * hs] = make_float2(sc, un);
+                        if (moved_any) sh.fsc[buf][g + 4 * hs] = fsc_acc[hs];
+                    }
+                    wm[hs] = 0.0f;
+                    fsc_acc[hs] = 1.0f;
                 }
-
-                // ---- hand the weights to the V wave
+                if (lane == 0) sh.moved[buf] = moved_any ? 1u : 0u;
+                moved_any = false;
 #pragma unroll
-                for (int hs = 0; hs < 2; hs++) sh.ww[buf][hs][lane] = make_float4(ww[0][hs], ww[1][hs], ww[2][hs], ww[3][hs]);
+                for (int sub = 0; sub < PS; sub++)
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) sh.ww[buf][sub][hs][lane] = make_float4(ww[sub][0][hs], ww[sub][1][hs], ww[sub][2][hs], ww[sub][3][hs]);
                 __syncthreads();   // hand-over of buffer `buf`; also: the V wave is done with the buffer written next
-                gg = gnext;
             };
-            uint32_t G = g_first;
-            for (; G + 1 < g_last; G++) step(std::integral_constant<int, 1>{}, G);
-            if (G < g_last) { step(std::integral_constant<int, 2>{}, G); G++; }
-            step(std::integral_constant<int, 0>{}, G);
+            if constexpr (PS == 2) {
+                // A pair at a chunk end: either group may be missing (weights zero), the group after one may be partial or missing.
+                auto general_pair = [&](uint32_t P) {
+#pragma unroll
+                    for (int sub = 0; sub < 2; sub++) {
+                        const uint32_t G = 2 * P + sub;
+                        float wt[4][2];
+#pragma unroll
+                        for (int q = 0; q < 4; q++) wt[q][0] = wt[q][1] = 0.0f;
+                        if (G >= g_first && G <= g_last) {
+                            if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, G, wt, sub == 1);
+                            else if (G < g_last) group_core(std::integral_constant<int, 2>{}, G, wt, sub == 1);
+                            else group_core(std::integral_constant<int, 0>{}, G, wt, sub == 1);
+                        }
+#pragma unroll
+                        for (int q = 0; q < 4; q++) { ww[sub][q][0] = wt[q][0]; ww[sub][q][1] = wt[q][1]; }
+                    }
+                    finish_pair(P);
+                };
+                uint32_t P = g_first >> 1;
+                if (2 * P < g_first) { general_pair(P); P++; }           // the chunk starts in the second group of a pair
+                for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
+                    group_core(std::integral_constant<int, 1>{}, 2 * P, ww[0], false);
+                    group_core(std::integral_constant<int, 1>{}, 2 * P + 1, ww[PS - 1], true);
+                    finish_pair(P);
+                }
+                for (; P <= (g_last >> 1); P++) general_pair(P);
+            } else {
+                uint32_t G = g_first;
+                for (; G + 1 < g_last; G++) { group_core(std::integral_constant<int, 1>{}, G, ww[0], false); finish_pair(G); }
+                if (G < g_last) { group_core(std::integral_constant<int, 2>{}, G, ww[0], false); finish_pair(G); G++; }
+                group_core(std::integral_constant<int, 0>{}, G, ww[0], false);
+                finish_pair(G);
+            }
         }
 #pragma unroll
         for (int hs = 0; hs < 2; hs++) {
@@ -458,11 +514,16 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             };
             load_v(gg.full, gg);
 
-            // One group; KIND as in the K wave: 0 nothing follows, 1 a complete group follows, 2 a group that may be partial.
-            auto step = [&](auto kind_tag, uint32_t G) {
-                constexpr int KIND = decltype(kind_tag)::value;
-                const uint32_t buf = (G - g_first) & 1u;
-                __syncthreads();   // the K wave's weights of this group
+            v4i acc[4][4];      // [code byte e][field f]: the pair's integer sums, rows = heads g, g + 4 x 2 limbs
+            v4i csum;           // 4 x the centre: 2 sum(plane 0 weights) + 4 sum(plane 1 weights, which are halved) + sum(plane 2 weights)
+            float uf[2][4];     // [head set][field]: value of one integer step of the accumulators of this pair
+            float cq[2][3];     // [head set][plane]: weight -> signed normalised 16-bit number at the pair's scale
+            uint32_t buf = 0;
+
+            // The K wave's hand-over of a pair: rescale if the reference moved, read the pair's scales.
+            auto begin_pair = [&](uint32_t P) {
+                buf = (P - (PS == 2 ? g_first >> 1 : g_first)) & 1u;
+                __syncthreads();   // the K wave's weights of this pair
                 if (__builtin_amdgcn_readfirstlane(sh.moved[buf]) != 0) {   // rare: the reference moved
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
@@ -474,23 +535,33 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                         sctr[hs] *= fsc;
                     }
                 }
-                // ---- weights -> 16-bit fixed point at the head's scale of this group, two signed limbs; a lane holds the
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {
+                    const float2 ws = sh.wsc[buf][g + 4 * hs];
+                    uf[hs][0] = ws.y; uf[hs][1] = ws.y * 0.25f; uf[hs][2] = uf[hs][3] = ws.y * 0.0625f;   // field 3 is read at field 2's place
+#pragma unroll
+                    for (int pl = 0; pl < nplanes; pl++) cq[hs][pl] = cfn[pl] * ws.x;
+                }
+            };
+            // One group of the pair.  KIND as in the K wave: 0 nothing follows, 1 a complete group follows, 2 a group that may be
+            // partial.  ZERO: the accumulators start at zero here (the first MFMA of each takes the constant as its C operand).
+            auto group_core = [&](auto kind_tag, auto zero_tag, uint32_t G, uint32_t sub) {
+                constexpr int KIND = decltype(kind_tag)::value;
+                constexpr bool ZERO = decltype(zero_tag)::value;
+                // ---- weights -> 16-bit fixed point at the head's scale of this pair, two signed limbs; a lane holds the
                 //      weights of column position pcol of the four tiles, i.e. one k word of the MFMA's A operand:
                 //      lane (column 4A+B, row group g) feeds rows 4g + 2 * set + limb of k-group A, word B.
-                float uf[2][4];   // [head set][field]: value of one integer step of the accumulators of this group
                 {
                     const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
                     __builtin_amdgcn_wave_barrier();
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        const float4 wv = sh.ww[buf][hs][lane];
-                        const float2 ws = sh.wsc[buf][g + 4 * hs];
-                        uf[hs][0] = ws.y; uf[hs][1] = ws.y * 0.25f; uf[hs][2] = uf[hs][3] = ws.y * 0.0625f;   // field 3 is read at field 2's place
+                        const float4 wv = sh.ww[buf][sub][hs][lane];
 #pragma unroll
                         for (int pl = 0; pl < nplanes; pl++) {
-                            const float cq = cfn[pl] * ws.x;
-                            const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.x * cq, wv.y * cq));
-                            const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.z * cq, wv.w * cq));
+                            const float c = cq[hs][pl];
+                            const uint32_t p01 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.x * c, wv.y * c));
+                            const uint32_t p23 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pknorm_i16(wv.z * c, wv.w * c));
                             // per 16-bit half: low byte = signed low limb, high byte = what is left of it
                             const uint32_t t01 = __builtin_bit_cast(uint32_t, (us2_t)(__builtin_bit_cast(us2_t, p01) + (us2_t){0x80, 0x80})) ^ 0x00800080u;
                             const uint32_t t23 = __builtin_bit_cast(uint32_t, (us2_t)(__builtin_bit_cast(us2_t, p23) + (us2_t){0x80, 0x80})) ^ 0x00800080u;
@@ -505,14 +576,12 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 #pragma unroll
                 for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
                 if constexpr (KIND != 0) load_v(KIND == 1, geom(G + 1));   // the V registers are free
-                v4i acc[4][4];      // [code byte e][field f]: the group's integer sums, rows = heads g, g + 4 x 2 limbs
-                v4i csum;           // 4 x the centre: 2 sum(plane 0 weights) + 4 sum(plane 1 weights, which are halved) + sum(plane 2 weights)
 #pragma unroll
                 for (int pl = 0; pl < nplanes; pl++) {
                     const v4i wop = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][lane * 16]);
                     {
                         const int cb = pl == 0 ? 0x02020202 : pl == 1 ? 0x04040404 : 0x01010101;
-                        csum = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, (v4i){cb, cb, cb, cb}, pl == 0 ? (v4i){0, 0, 0, 0} : csum, 0, 0, 0);
+                        csum = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, (v4i){cb, cb, cb, cb}, (ZERO && pl == 0) ? (v4i){0, 0, 0, 0} : csum, 0, 0, 0);
                     }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -530,11 +599,13 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                             v4i b;
 #pragma unroll
                             for (int m = 0; m < 4; m++) b[m] = (int)((f == 3 ? yd[m] : yp[m]) & mask);
-                            acc[e][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, b, pl == 0 ? (v4i){0, 0, 0, 0} : acc[e][f], 0, 0, 0);
+                            acc[e][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, b, (ZERO && pl == 0) ? (v4i){0, 0, 0, 0} : acc[e][f], 0, 0, 0);
                         }
                     }
                 }
-                // ---- the group's sums into the float outputs
+            };
+            // The pair's sums into the float outputs.
+            auto end_pair = [&]() {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
 #pragma unroll
@@ -550,10 +621,41 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     sctr[hs] = __builtin_fmaf((float)t, 0.25f * uf[hs][0], sctr[hs]);
                 }
             };
-            uint32_t G = g_first;
-            for (; G + 1 < g_last; G++) step(std::integral_constant<int, 1>{}, G);
-            if (G < g_last) { step(std::integral_constant<int, 2>{}, G); G++; }
-            step(std::integral_constant<int, 0>{}, G);
+            if constexpr (PS == 2) {
+                // A pair at a chunk end: either group may be missing, the group after one may be partial or missing.
+                auto general_pair = [&](uint32_t P) {
+                    begin_pair(P);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+#pragma unroll
+                        for (int f = 0; f < 4; f++) acc[e][f] = (v4i){0, 0, 0, 0};
+                    csum = (v4i){0, 0, 0, 0};
+                    for (uint32_t sub = 0; sub < 2; sub++) {
+                        const uint32_t G = 2 * P + sub;
+                        if (G < g_first || G > g_last) continue;
+                        if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, sub);
+                        else if (G < g_last) group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, sub);
+                        else group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, sub);
+                    }
+                    end_pair();
+                };
+                uint32_t P = g_first >> 1;
+                if (2 * P < g_first) { general_pair(P); P++; }           // the chunk starts in the second group of a pair
+                for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
+                    begin_pair(P);
+                    group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P, 0u);
+                    group_core(std::integral_constant<int, 1>{}, std::false_type{}, 2 * P + 1, 1u);
+                    end_pair();
+                }
+                for (; P <= (g_last >> 1); P++) general_pair(P);
+            } else {
+                uint32_t G = g_first;
+                for (; G + 1 < g_last; G++) { begin_pair(G); group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, 0u); end_pair(); }
+                if (G < g_last) { begin_pair(G); group_core(std::integral_constant<int, 2>{}, std::true_type{}, G, 0u); end_pair(); G++; }
+                begin_pair(G);
+                group_core(std::integral_constant<int, 0>{}, std::true_type{}, G, 0u);
+                end_pair();
+            }
         }
         __syncthreads();   // the K wave's totals
 
@@ -584,18 +686,18 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     }
 }
 
-template <int OCC, int HD>
+template <int OCC, int HD, int PS>
 __global__ __launch_bounds__(64 + HD / 4, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {   // 128 / 192 threads
-    __shared__ __align__(16) AttnShared<HD / 256> sh;
+    __shared__ __align__(16) AttnShared<HD / 256, PS> sh;
     // L[c] = alpha + beta*bit0 + gam*bit1 + delta*bit0*bit1.  A delta that is only float noise of a symmetric table
     // (|delta| <= 1e-5 max|L|) is spread by the least-squares affine fit bit0*bit1 ~ -1/4 + bit0/2 + bit1/2, which
     // leaves +-delta/4 per code; anything larger gets its own bit plane.
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
-    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD, false>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
-    else if (p.num_kv_heads == 1) attention_body<2, HD, true>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
-    else attention_body<2, HD, false>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD, false, PS>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, HD, true, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, HD, false, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
@@ -634,12 +736,20 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
+    // Hand-overs of two groups pay from about a thousand positions per workgroup on (head_dim 256; the three-wave
+    // workgroups of head_dim 512 do not fit the registers of that form).
+    static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
+    static const uint64_t pair_min = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR_MIN"); return e ? (uint64_t)atoll(e) : (uint64_t)1024; }();
+    const bool pair = p.head_dim == 256 && (pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min);
     if (p.head_dim == 512) {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512>), grid, dim3(192), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512>), grid, dim3(192), 0, ctx->stream, a, p);
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 1>), grid, dim3(192), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(192), 0, ctx->stream, a, p);
+    } else if (pair) {
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
     } else {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256>), grid, dim3(128), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256>), grid, dim3(128), 0, ctx->stream, a, p);
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256, 1>), grid, dim3(128), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 1>), grid, dim3(128), 0, ctx->stream, a, p);
     }
     return lh_check_launch(op);
 }
