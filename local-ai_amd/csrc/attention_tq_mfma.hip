@@ -299,14 +299,16 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             bool moved_any = false;
 
             // One group: logits, reference check, weights into wout.  `second`: the pair's first group has been done (its
-            // weights in ww[0] follow the reference if that moves now).
-            auto group_core = [&](auto kind_tag, uint32_t G, float (&wout)[4][2], bool second) {
+            // weights in ww[0] follow the reference if that moves now).  FULL: the group is complete and not the chunk's
+            // first (no masks, and the reference is finite: logits are then formed relative to it in the same fma).
+            auto group_core = [&](auto kind_tag, auto full_tag, uint32_t G, float (&wout)[4][2], bool second) {
                 constexpr int KIND = decltype(kind_tag)::value;
+                constexpr bool FULL = decltype(full_tag)::value;
                 const GroupGeom gnext = geom(KIND ? G + 1 : G);
 
                 // ---- norms of the group -> LDS
                 {
-                    const bool valid = lane >= gg.vlo && lane < gg.vhi;
+                    const bool valid = FULL || (lane >= gg.vlo && lane < gg.vhi);
                     __builtin_amdgcn_wave_barrier();
                     sh.norm[lane] = make_float4(nk * kLog2e, valid ? 0.0f : -INFINITY, valid ? nv : 0.0f, 0.0f);
                     __builtin_amdgcn_wave_barrier();
@@ -363,7 +365,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                         const uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
                         const uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
                         const float inner = (float)(int)((t1 << 2) + t4) * cs[hs] + ca[hs];
-                        lg[q][hs] = nrm.x * inner + nrm.y;
+                        lg[q][hs] = FULL ? __builtin_fmaf(nrm.x, inner, -R[hs]) : nrm.x * inner + nrm.y;
                     }
                 }
 
@@ -372,13 +374,22 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 float mq[2];
 #pragma unroll
                 for (int hs = 0; hs < 2; hs++) mq[hs] = fmaxf(fmaxf(lg[0][hs], lg[1][hs]), fmaxf(lg[2][hs], lg[3][hs]));
-                const bool move = __builtin_amdgcn_ballot_w64(fmaxf(mq[0] - R[0], mq[1] - R[1]) > kHeadroom) != 0;   // uniform
+                const bool move = __builtin_amdgcn_ballot_w64((FULL ? fmaxf(mq[0], mq[1]) : fmaxf(mq[0] - R[0], mq[1] - R[1])) > kHeadroom) != 0;   // uniform
                 if (move) {
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        const float rn = fmaxf(R[hs], lh_group_max(mq[hs], 16));
-                        const float fsc = rn > R[hs] ? __builtin_amdgcn_exp2f(R[hs] - rn) : 1.0f;   // 0 for the first group
-                        R[hs] = rn;
+                        float fsc;
+                        if constexpr (FULL) {   // lg and mq are relative to R
+                            const float d = fmaxf(lh_group_max(mq[hs], 16), 0.0f);
+                            fsc = __builtin_amdgcn_exp2f(-d);
+                            R[hs] += d;
+#pragma unroll
+                            for (int q = 0; q < 4; q++) lg[q][hs] -= d;
+                        } else {
+                            const float rn = fmaxf(R[hs], lh_group_max(mq[hs], 16));
+                            fsc = rn > R[hs] ? __builtin_amdgcn_exp2f(R[hs] - rn) : 1.0f;   // 0 for the first group
+                            R[hs] = rn;
+                        }
                         l_run[hs] *= fsc;
                         w_run[hs] *= fsc;
                         fsc_acc[hs] *= fsc;
@@ -394,7 +405,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 for (int hs = 0; hs < 2; hs++) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
-                        const float ew = __builtin_amdgcn_exp2f(lg[q][hs] - R[hs]);
+                        const float ew = __builtin_amdgcn_exp2f(FULL ? lg[q][hs] : lg[q][hs] - R[hs]);
                         wout[q][hs] = ew * vn[q];
                         l_run[hs] += ew;
                         w_run[hs] += wout[q][hs];
@@ -441,9 +452,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 #pragma unroll
                         for (int q = 0; q < 4; q++) wt[q][0] = wt[q][1] = 0.0f;
                         if (G >= g_first && G <= g_last) {
-                            if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, G, wt, sub == 1);
-                            else if (G < g_last) group_core(std::integral_constant<int, 2>{}, G, wt, sub == 1);
-                            else group_core(std::integral_constant<int, 0>{}, G, wt, sub == 1);
+                            if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, wt, sub == 1);
+                            else if (G < g_last) group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, wt, sub == 1);
+                            else group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, wt, sub == 1);
                         }
 #pragma unroll
                         for (int q = 0; q < 4; q++) { ww[sub][q][0] = wt[q][0]; ww[sub][q][1] = wt[q][1]; }
@@ -451,18 +462,20 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     finish_pair(P);
                 };
                 uint32_t P = g_first >> 1;
-                if (2 * P < g_first) { general_pair(P); P++; }           // the chunk starts in the second group of a pair
+                general_pair(P);                                         // holds the chunk's first group
+                P++;
                 for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
-                    group_core(std::integral_constant<int, 1>{}, 2 * P, ww[0], false);
-                    group_core(std::integral_constant<int, 1>{}, 2 * P + 1, ww[PS - 1], true);
+                    group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P, ww[0], false);
+                    group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P + 1, ww[PS - 1], true);
                     finish_pair(P);
                 }
                 for (; P <= (g_last >> 1); P++) general_pair(P);
             } else {
                 uint32_t G = g_first;
-                for (; G + 1 < g_last; G++) { group_core(std::integral_constant<int, 1>{}, G, ww[0], false); finish_pair(G); }
-                if (G < g_last) { group_core(std::integral_constant<int, 2>{}, G, ww[0], false); finish_pair(G); G++; }
-                group_core(std::integral_constant<int, 0>{}, G, ww[0], false);
+                if (G + 1 < g_last) { group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
+                for (; G + 1 < g_last; G++) { group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, ww[0], false); finish_pair(G); }
+                if (G < g_last) { group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
+                group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, ww[0], false);
                 finish_pair(G);
             }
         }
@@ -640,7 +653,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     end_pair();
                 };
                 uint32_t P = g_first >> 1;
-                if (2 * P < g_first) { general_pair(P); P++; }           // the chunk starts in the second group of a pair
+                general_pair(P);                                         // holds the chunk's first group
+                P++;
                 for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
                     begin_pair(P);
                     group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P, 0u);
