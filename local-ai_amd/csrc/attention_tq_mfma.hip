@@ -19,13 +19,15 @@
 //            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
 //            byte transposes.
 // One workgroup owns a chunk of positions and walks it in aligned groups of 64: the K wave produces the
-// softmax weights of a group, a V wave per 256 output dims (one group behind, one barrier per group)
-// turns them into limbs, multiplies and adds the group's integer sums to its float outputs with the group's
-// scale.  A scale per head and group keeps the long tail of a soft distribution: a weight is only compared
-// with the 63 around it, never with a maximum seen thousands of positions earlier.  The softmax reference
-// R_h only keeps exp2 in range and follows the running maximum lazily.  Splitting the roles lets two or
-// three waves share a SIMD and fill each other's stalls.  Partials (R, l, acc) per chunk go to the
-// workspace for the merge kernel.
+// softmax weights of a group (or of an aligned pair of groups, for long chunks), a V wave per 256 output
+// dims, one hand-over behind with one barrier per hand-over, turns them into limbs, multiplies and adds
+// the integer sums to its float outputs with the hand-over's scale.  A scale per head and hand-over keeps
+// the long tail of a soft distribution: a weight is only compared with the 63 or 127 around it, never with
+// a maximum seen thousands of positions earlier.  The softmax reference R_h only keeps exp2 in range and
+// follows the running maximum lazily.  Splitting the roles lets two waves share a SIMD and fill each
+// other's stalls.  head_dim 512 has two K waves, one per 64-byte half of the K codes: the second runs a
+// further hand-over ahead and passes its integer logit sums to the first.  Partials (R, l, acc) per chunk
+// go to the workspace for the merge kernel.
 #include "attention_tq.hpp"
 #include <algorithm>
 #include <cstdlib>
@@ -85,6 +87,7 @@ struct AttnShared {
     float4 ww[2][PS][2][64];       // [buffer][group of the pair][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
     float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this pair into [-1, 1], value of one integer step)
     uint8_t wx[NH][3][1024];       // [V wave][plane]: that wave's A operands (weights as limbs)
+    v4i tb[NH == 2 ? 2 : 1][2][64]; // head_dim 512: [buffer][head set][lane]: the second K wave's integer logit sums of tiles 0..3 (code half 1)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
     uint32_t moved[2];             // [buffer]: the reference moved within this pair: rescale the outputs
     float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads];
@@ -141,9 +144,14 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     const float inv_cmax_v = cmax_v > 0.0f ? 1.0f / cmax_v : 0.0f;
     const float v_unit = cmax_v * (1.0f / kQmax);   // value of one integer step of a weight limb pair at scale 1
     // Roles rotate with the workgroup index, so that the kinds of wave mix on every SIMD.
-    const uint32_t role = NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) % 3u;   // 0: K wave; 1, 2: V wave of code half role - 1
-    const bool k_role = role == 0;
-    const uint32_t vhalf = k_role ? 0u : role - 1u;
+    // head_dim 256: a K wave and a V wave.  head_dim 512: a K wave per 64-byte half of the K codes -- the second one (role 3)
+    // runs a group ahead and hands its integer logit sums to the first, which adds its own and does the softmax -- and a V wave
+    // per half of the V codes.
+    const uint32_t role = NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) & 3u;   // 0: K wave; 1, 2: V wave of code half role - 1; 3: second K wave
+    const bool k_role = role == 0 || role == 3;
+    const bool kb_role = NH == 2 && role == 3;
+    const uint32_t khalf = kb_role ? 1u : 0u;
+    const uint32_t vhalf = k_role ? khalf : role - 1u;
 
     // ---- touch the first group's codes (one 64-byte record per lane) so that they are on their way into the cache
     //      while the set-up below runs; the value is only consumed (and waited for) after the set-up
@@ -255,7 +263,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             cs[hs] = s_maxabs[h] * cmax_k * (0.25f / kQmax);
             ca[hs] = alpha * sh.sum[h];
         }
-        gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes;
+        gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * khalf;   // this wave's half of the code
         gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
         gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
         float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
@@ -266,18 +274,15 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             // as a tile's codes have been taken apart (a step of prefetch distance, no second register set, no copies).
             // `KIND` says what follows the group: 0 nothing, 1 a group that is certainly complete (every group between the
             // first and the last of a chunk is), 2 a group that may be partial.
-            u32x4_t kw[NH][4];
+            u32x4_t kw[4];
             float nk, nv;
             const uint32_t klane = pcol * stride + 16 * g, nlane = lane * nstride;
             auto load_tile = [&](bool full, const GroupGeom& G_, int q) {
                 gptr_t kb = krec0 + (size_t)G_.pb * stride;
-#pragma unroll
-                for (int hf = 0; hf < NH; hf++) {
-                    if (full) kw[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
-                    else {
-                        kw[hf][q] = (u32x4_t){0u, 0u, 0u, 0u};
-                        if (is_valid(G_, 16 * q + pcol)) kw[hf][q] = ld16(kb + (size_t)(16 * q) * stride + klane + 64 * hf);
-                    }
+                if (full) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
+                else {
+                    kw[q] = (u32x4_t){0u, 0u, 0u, 0u};
+                    if (is_valid(G_, 16 * q + pcol)) kw[q] = ld16(kb + (size_t)(16 * q) * stride + klane);
                 }
             };
             auto load_norms = [&](bool full, const GroupGeom& G_) {
@@ -290,13 +295,67 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             };
 #pragma unroll
             for (int q = 0; q < 4; q++) load_tile(gg.full, gg, q);
-            load_norms(gg.full, gg);
+            if (!kb_role) load_norms(gg.full, gg);
 
             // Two groups of 64 positions (an aligned pair) share one fixed-point scale per head and one hand-over to the V wave.
             float ww[PS][4][2];             // [group of the pair][tile][head set]: the pair's weights
             float wm[2] = {0.0f, 0.0f};     // largest |weight| of the pair so far, per head set
             float fsc_acc[2] = {1.0f, 1.0f};   // by how much the reference has moved within the pair
             bool moved_any = false;
+
+            // The integer logit sums of a group's 4 tiles x (this lane's column position, heads g and g + 4) over this wave's half
+            // of the code, handed tile by tile to `post`; the next group's codes are requested into a tile's registers as soon
+            // as it has been taken apart.
+            auto k_tiles = [&](auto kind_tag, const GroupGeom& gnext, auto&& post) {
+                constexpr int KIND = decltype(kind_tag)::value;
+                const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[khalf * nplanes * 4][lane][0]);   // operand (plane pl, field f) at rqo[64 * (4 * pl + f)]
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
+                    const uint32_t w[4] = {kw[q].x, kw[q].y, kw[q].z, kw[q].w};
+                    v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        const uint32_t u = w[m] >> 4;
+                        b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
+                        b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
+                        b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
+                        b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
+                    }
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
+                    acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
+                    if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
+                        v4i d0, d1, d2, d3;
+#pragma unroll
+                        for (int m = 0; m < 4; m++) {
+                            const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
+                            d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
+                            d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
+                        }
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
+                    }
+                    if constexpr (KIND != 0) load_tile(KIND == 1, gnext, q);   // the tile's code registers are free
+                    int t[2];
+#pragma unroll
+                    for (int hs = 0; hs < 2; hs++) {
+                        // three shift-adds: limbs first, then the two field scales
+                        const uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
+                        const uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
+                        t[hs] = (int)((t1 << 2) + t4);
+                    }
+                    post(q, t[0], t[1]);
+                }
+            };
+            uint32_t tbuf = 0;   // head_dim 512: which buffer holds the second K wave's sums of the group at hand
 
             // One group: logits, reference check, weights into wout.  `second`: the pair's first group has been done (its
             // weights in ww[0] follow the reference if that moves now).  FULL: the group is complete and not the chunk's
@@ -305,6 +364,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 constexpr int KIND = decltype(kind_tag)::value;
                 constexpr bool FULL = decltype(full_tag)::value;
                 const GroupGeom gnext = geom(KIND ? G + 1 : G);
+                if constexpr (NH == 2) tbuf = (G - g_first) & 1u;
 
                 // ---- norms of the group -> LDS
                 {
@@ -317,57 +377,18 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 
                 // ---- logits of 4 tiles x (this lane's column position, heads g and g + 4)
                 float lg[4][2], vn[4];
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    v4i acc1 = (v4i){0, 0, 0, 0}, acc4 = (v4i){0, 0, 0, 0};   // by mask scale: fields 0, 2 arrive x1, fields 1, 3 x4
-#pragma unroll
-                    for (int hf = 0; hf < NH; hf++) {
-                        const uint32_t w[4] = {kw[hf][q].x, kw[hf][q].y, kw[hf][q].z, kw[hf][q].w};
-                        v4i b00, b10, b01, b11, b02, b12, b03, b13;   // b<plane><field>
-#pragma unroll
-                        for (int m = 0; m < 4; m++) {
-                            const uint32_t u = w[m] >> 4;
-                            b00[m] = (int)(w[m] & 0x01010101u); b10[m] = (int)(w[m] & 0x02020202u);
-                            b01[m] = (int)(w[m] & 0x04040404u); b11[m] = (int)(w[m] & 0x08080808u);
-                            b02[m] = (int)(u & 0x01010101u);    b12[m] = (int)(u & 0x02020202u);
-                            b03[m] = (int)(u & 0x04040404u);    b13[m] = (int)(u & 0x08080808u);
-                        }
-                        // operand (plane pl, field f) of this code half at rqo[64 * (4 * pl + f)]
-                        const v4i* rqo = reinterpret_cast<const v4i*>(&s_rqop[hf * nplanes * 4][lane][0]);
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 0], b00, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 1], b01, acc4, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 4], b10, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 5], b11, acc4, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 2], b02, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 3], b03, acc4, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 6], b12, acc1, 0, 0, 0);
-                        acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 7], b13, acc4, 0, 0, 0);
-                        if constexpr (has_delta) {   // third plane bit0 & bit1, one bit per field at the even bit positions
-                            v4i d0, d1, d2, d3;
-#pragma unroll
-                            for (int m = 0; m < 4; m++) {
-                                const uint32_t t = w[m] & (w[m] >> 1), u = t >> 4;
-                                d0[m] = (int)(t & 0x01010101u); d1[m] = (int)(t & 0x04040404u);
-                                d2[m] = (int)(u & 0x01010101u); d3[m] = (int)(u & 0x04040404u);
-                            }
-                            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 8], d0, acc1, 0, 0, 0);
-                            acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 9], d1, acc4, 0, 0, 0);
-                            acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 10], d2, acc1, 0, 0, 0);
-                            acc4 = __builtin_amdgcn_mfma_i32_16x16x64_i8(rqo[64 * 11], d3, acc4, 0, 0, 0);
-                        }
-                    }
-                    if constexpr (KIND != 0) load_tile(KIND == 1, gnext, q);   // the tile's code registers are free
+                v4i tb0 = (v4i){0, 0, 0, 0}, tb1 = (v4i){0, 0, 0, 0};   // head_dim 512: the other code half's sums, from the second K wave
+                if constexpr (NH == 2) { tb0 = sh.tb[tbuf][0][lane]; tb1 = sh.tb[tbuf][1][lane]; }
+                k_tiles(kind_tag, gnext, [&](int q, int t0, int t1) {
                     const float4 nrm = sh.norm[16 * q + pcol];
                     vn[q] = nrm.z;
+                    const int tt[2] = {t0 + tb0[q], t1 + tb1[q]};
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
-                        // three shift-adds: limbs first, then the two field scales
-                        const uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
-                        const uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
-                        const float inner = (float)(int)((t1 << 2) + t4) * cs[hs] + ca[hs];
+                        const float inner = (float)tt[hs] * cs[hs] + ca[hs];
                         lg[q][hs] = FULL ? __builtin_fmaf(nrm.x, inner, -R[hs]) : nrm.x * inner + nrm.y;
                     }
-                }
+                });
 
                 // ---- softmax weights relative to the reference R, which follows the running maximum lazily: it moves
                 //      when a logit of the group exceeds it by more than kHeadroom (always in the first group)
@@ -470,20 +491,41 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     finish_pair(P);
                 }
                 for (; P <= (g_last >> 1); P++) general_pair(P);
+            } else if (kb_role) {
+                // head_dim 512, second K wave: its code half's sums of every group, one hand-over ahead of the first K wave
+                auto kb_step = [&](auto kind_tag, uint32_t G) {
+                    constexpr int KIND = decltype(kind_tag)::value;
+                    const GroupGeom gnext = geom(KIND ? G + 1 : G);
+                    int t0s[4], t1s[4];
+                    k_tiles(kind_tag, gnext, [&](int q, int t0, int t1) { t0s[q] = t0; t1s[q] = t1; });
+                    const uint32_t b = (G - g_first) & 1u;
+                    sh.tb[b][0][lane] = (v4i){t0s[0], t0s[1], t0s[2], t0s[3]};
+                    sh.tb[b][1][lane] = (v4i){t1s[0], t1s[1], t1s[2], t1s[3]};
+                    gg = gnext;
+                    __syncthreads();
+                };
+                uint32_t G = g_first;
+                for (; G + 1 < g_last; G++) kb_step(std::integral_constant<int, 1>{}, G);
+                if (G < g_last) { kb_step(std::integral_constant<int, 2>{}, G); G++; }
+                kb_step(std::integral_constant<int, 0>{}, G);
+                __syncthreads();   // the first K wave's last group
+                __syncthreads();   // the V waves' last group
             } else {
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first group
                 uint32_t G = g_first;
                 if (G + 1 < g_last) { group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
                 for (; G + 1 < g_last; G++) { group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, ww[0], false); finish_pair(G); }
                 if (G < g_last) { group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
                 group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, ww[0], false);
                 finish_pair(G);
+                if constexpr (NH == 2) __syncthreads();   // the V waves' last group
             }
         }
 #pragma unroll
         for (int hs = 0; hs < 2; hs++) {
             const float l_tot = lh_group_sum(l_run[hs], 16);
             const float w_tot = lh_group_sum(w_run[hs], 16);
-            if (pcol == 0) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs]; }
+            if (pcol == 0 && !kb_role) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs]; }
         }
         __syncthreads();
     } else {
@@ -663,12 +705,14 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 }
                 for (; P <= (g_last >> 1); P++) general_pair(P);
             } else {
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first group
                 uint32_t G = g_first;
                 for (; G + 1 < g_last; G++) { begin_pair(G); group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, 0u); end_pair(); }
                 if (G < g_last) { begin_pair(G); group_core(std::integral_constant<int, 2>{}, std::true_type{}, G, 0u); end_pair(); G++; }
                 begin_pair(G);
                 group_core(std::integral_constant<int, 0>{}, std::true_type{}, G, 0u);
                 end_pair();
+                if constexpr (NH == 2) __syncthreads();   // pairs with the K waves' count of barriers
             }
         }
         __syncthreads();   // the K wave's totals
@@ -701,7 +745,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 }
 
 template <int OCC, int HD, int PS>
-__global__ __launch_bounds__(64 + HD / 4, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {   // 128 / 192 threads
+__global__ __launch_bounds__(HD / 2, OCC) void attention_tq_mfma_kernel(AttnPointers a, AttnParams p) {   // 128 / 256 threads
     __shared__ __align__(16) AttnShared<HD / 256, PS> sh;
     // L[c] = alpha + beta*bit0 + gam*bit1 + delta*bit0*bit1.  A delta that is only float noise of a symmetric table
     // (|delta| <= 1e-5 max|L|) is spread by the least-squares affine fit bit0*bit1 ~ -1/4 + bit0/2 + bit1/2, which
@@ -737,7 +781,7 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
     static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
-    const uint32_t wg_waves = p.head_dim == 512 ? 3 : 2;
+    const uint32_t wg_waves = p.head_dim == 512 ? 4 : 2;
     const uint64_t wg_slots = (uint64_t)ctx->cu_count * std::max(1u, 4u * (uint32_t)wps / wg_waves);
     uint64_t splits = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)ctx->cu_count / pairs));
     splits = std::max<uint64_t>(splits, 1);
@@ -756,8 +800,8 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     static const uint64_t pair_min = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR_MIN"); return e ? (uint64_t)atoll(e) : (uint64_t)1024; }();
     const bool pair = p.head_dim == 256 && (pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min);
     if (p.head_dim == 512) {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 1>), grid, dim3(192), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(192), 0, ctx->stream, a, p);
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
     } else if (pair) {
         if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
         else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
