@@ -87,7 +87,7 @@ struct AttnShared {
     float4 ww[2][PS][2][64];       // [buffer][group of the pair][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
     float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this pair into [-1, 1], value of one integer step)
     uint8_t wx[NH][3][1024];       // [V wave][plane]: that wave's A operands (weights as limbs)
-    v4i tb[NH == 2 ? 2 : 1][2][64]; // head_dim 512: [buffer][head set][lane]: the second K wave's integer logit sums of tiles 0..3 (code half 1)
+    v4i tb[NH == 2 ? 2 : 1][PS][2][64]; // head_dim 512: [buffer][group of the pair][head set][lane]: the second K wave's integer logit sums of tiles 0..3 (code half 1)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
     uint32_t moved[2];             // [buffer]: the reference moved within this pair: rescale the outputs
     float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads];
@@ -364,7 +364,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 constexpr int KIND = decltype(kind_tag)::value;
                 constexpr bool FULL = decltype(full_tag)::value;
                 const GroupGeom gnext = geom(KIND ? G + 1 : G);
-                if constexpr (NH == 2) tbuf = (G - g_first) & 1u;
+                if constexpr (NH == 2) tbuf = (PS == 2 ? (G >> 1) - (g_first >> 1) : G - g_first) & 1u;
 
                 // ---- norms of the group -> LDS
                 {
@@ -378,7 +378,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 // ---- logits of 4 tiles x (this lane's column position, heads g and g + 4)
                 float lg[4][2], vn[4];
                 v4i tb0 = (v4i){0, 0, 0, 0}, tb1 = (v4i){0, 0, 0, 0};   // head_dim 512: the other code half's sums, from the second K wave
-                if constexpr (NH == 2) { tb0 = sh.tb[tbuf][0][lane]; tb1 = sh.tb[tbuf][1][lane]; }
+                if constexpr (NH == 2) { const uint32_t sub = (PS == 2 && second) ? 1u : 0u; tb0 = sh.tb[tbuf][sub][0][lane]; tb1 = sh.tb[tbuf][sub][1][lane]; }
                 k_tiles(kind_tag, gnext, [&](int q, int t0, int t1) {
                     const float4 nrm = sh.norm[16 * q + pcol];
                     vn[q] = nrm.z;
@@ -463,7 +463,27 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     for (int hs = 0; hs < 2; hs++) sh.ww[buf][sub][hs][lane] = make_float4(ww[sub][0][hs], ww[sub][1][hs], ww[sub][2][hs], ww[sub][3][hs]);
                 __syncthreads();   // hand-over of buffer `buf`; also: the V wave is done with the buffer written next
             };
-            if constexpr (PS == 2) {
+            if (kb_role) {
+                // head_dim 512, second K wave: its code half's sums of every group, one hand-over ahead of the first K wave
+                auto kb_step = [&](auto kind_tag, uint32_t G) {
+                    constexpr int KIND = decltype(kind_tag)::value;
+                    const GroupGeom gnext = geom(KIND ? G + 1 : G);
+                    int t0s[4], t1s[4];
+                    k_tiles(kind_tag, gnext, [&](int q, int t0, int t1) { t0s[q] = t0; t1s[q] = t1; });
+                    const uint32_t b = (PS == 2 ? (G >> 1) - (g_first >> 1) : G - g_first) & 1u, sub = PS == 2 ? (G & 1u) : 0u;
+                    sh.tb[b][sub][0][lane] = (v4i){t0s[0], t0s[1], t0s[2], t0s[3]};
+                    sh.tb[b][sub][1][lane] = (v4i){t1s[0], t1s[1], t1s[2], t1s[3]};
+                    gg = gnext;
+                    if (PS == 1 || (G & 1u) || G == g_last) __syncthreads();   // the hand-over is complete
+                };
+                uint32_t G = g_first;
+                for (; G + 1 < g_last; G++) kb_step(std::integral_constant<int, 1>{}, G);
+                if (G < g_last) { kb_step(std::integral_constant<int, 2>{}, G); G++; }
+                kb_step(std::integral_constant<int, 0>{}, G);
+                __syncthreads();   // the first K wave's last hand-over
+                __syncthreads();   // the V waves' last hand-over
+            } else if constexpr (PS == 2) {
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
                 // A pair at a chunk end: either group may be missing (weights zero), the group after one may be partial or missing.
                 auto general_pair = [&](uint32_t P) {
 #pragma unroll
@@ -491,34 +511,16 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     finish_pair(P);
                 }
                 for (; P <= (g_last >> 1); P++) general_pair(P);
-            } else if (kb_role) {
-                // head_dim 512, second K wave: its code half's sums of every group, one hand-over ahead of the first K wave
-                auto kb_step = [&](auto kind_tag, uint32_t G) {
-                    constexpr int KIND = decltype(kind_tag)::value;
-                    const GroupGeom gnext = geom(KIND ? G + 1 : G);
-                    int t0s[4], t1s[4];
-                    k_tiles(kind_tag, gnext, [&](int q, int t0, int t1) { t0s[q] = t0; t1s[q] = t1; });
-                    const uint32_t b = (G - g_first) & 1u;
-                    sh.tb[b][0][lane] = (v4i){t0s[0], t0s[1], t0s[2], t0s[3]};
-                    sh.tb[b][1][lane] = (v4i){t1s[0], t1s[1], t1s[2], t1s[3]};
-                    gg = gnext;
-                    __syncthreads();
-                };
-                uint32_t G = g_first;
-                for (; G + 1 < g_last; G++) kb_step(std::integral_constant<int, 1>{}, G);
-                if (G < g_last) { kb_step(std::integral_constant<int, 2>{}, G); G++; }
-                kb_step(std::integral_constant<int, 0>{}, G);
-                __syncthreads();   // the first K wave's last group
-                __syncthreads();   // the V waves' last group
+                if constexpr (NH == 2) __syncthreads();   // the V waves' last hand-over
             } else {
-                if constexpr (NH == 2) __syncthreads();   // the second K wave's first group
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
                 uint32_t G = g_first;
                 if (G + 1 < g_last) { group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
                 for (; G + 1 < g_last; G++) { group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, ww[0], false); finish_pair(G); }
                 if (G < g_last) { group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, ww[0], false); finish_pair(G); G++; }
                 group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, ww[0], false);
                 finish_pair(G);
-                if constexpr (NH == 2) __syncthreads();   // the V waves' last group
+                if constexpr (NH == 2) __syncthreads();   // the V waves' last hand-over
             }
         }
 #pragma unroll
@@ -694,6 +696,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     }
                     end_pair();
                 };
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
                 uint32_t P = g_first >> 1;
                 general_pair(P);                                         // holds the chunk's first group
                 P++;
@@ -704,8 +707,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     end_pair();
                 }
                 for (; P <= (g_last >> 1); P++) general_pair(P);
+                if constexpr (NH == 2) __syncthreads();   // pairs with the K waves' count of barriers
             } else {
-                if constexpr (NH == 2) __syncthreads();   // the second K wave's first group
+                if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
                 uint32_t G = g_first;
                 for (; G + 1 < g_last; G++) { begin_pair(G); group_core(std::integral_constant<int, 1>{}, std::true_type{}, G, 0u); end_pair(); }
                 if (G < g_last) { begin_pair(G); group_core(std::integral_constant<int, 2>{}, std::true_type{}, G, 0u); end_pair(); G++; }
@@ -794,12 +798,15 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
-    // Hand-overs of two groups pay from about a thousand positions per workgroup on (head_dim 256; the three-wave
-    // workgroups of head_dim 512 do not fit the registers of that form).
+    // Hand-overs of two groups pay from about a thousand positions per workgroup on at head_dim 256 (-1 % at 4096 positions per
+    // workgroup, -6 % at 8192); at head_dim 512 they measured 2 % slower than single groups and are only taken when forced.
     static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
     static const uint64_t pair_min = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR_MIN"); return e ? (uint64_t)atoll(e) : (uint64_t)1024; }();
-    const bool pair = p.head_dim == 256 && (pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min);
-    if (p.head_dim == 512) {
+    const bool pair = pair_env >= 0 ? pair_env != 0 : p.head_dim == 256 && (max_span + splits - 1) / splits >= pair_min;
+    if (p.head_dim == 512 && pair) {
+        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
+        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
+    } else if (p.head_dim == 512) {
         if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
         else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
     } else if (pair) {
