@@ -132,8 +132,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     auto geom = [&](uint32_t G) {
         GroupGeom gg;
         const uint32_t gstart = G << 6;
-        gg.vlo = c_lo > gstart ? c_lo - gstart : 0u;
-        gg.vhi = std::min<uint32_t>(c_hi - gstart, (uint32_t)kGroup);
+        gg.vlo = c_lo > gstart ? std::min<uint32_t>(c_lo - gstart, (uint32_t)kGroup) : 0u;   // a group outside the chunk comes out empty
+        gg.vhi = c_hi > gstart ? std::min<uint32_t>(c_hi - gstart, (uint32_t)kGroup) : 0u;
+        if (gg.vhi < gg.vlo) gg.vhi = gg.vlo;
         gg.pb = p.ring_capacity ? gstart % p.ring_capacity : gstart;
         gg.full = gg.vlo == 0 && gg.vhi == (uint32_t)kGroup;
         return gg;
@@ -266,10 +267,13 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * khalf;   // this wave's half of the code
         gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
         gptr_t vn0 = (gptr_t)a.v_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
-        float R[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
+        // The reference starts at a finite "nothing yet": an empty group ahead of the first position (a pair whose first group
+        // lies before the chunk) then gives exp2(-inf) = 0 instead of exp2(-inf + inf).
+        constexpr float kNoRef = -1.0e30f;
+        float R[2] = {kNoRef, kNoRef}, l_run[2] = {0.f, 0.f}, w_run[2] = {0.f, 0.f};
 
         if (any) {
-            GroupGeom gg = geom(g_first);
+            GroupGeom gg = geom(PS == 2 ? (g_first & ~1u) : g_first);   // pairs are walked whole: a group outside the chunk is an empty one
             // K codes and norms of the current group.  Those of the next group are requested into the same registers as soon
             // as a tile's codes have been taken apart (a step of prefetch distance, no second register set, no copies).
             // `KIND` says what follows the group: 0 nothing, 1 a group that is certainly complete (every group between the
@@ -474,43 +478,38 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     sh.tb[b][sub][0][lane] = (v4i){t0s[0], t0s[1], t0s[2], t0s[3]};
                     sh.tb[b][sub][1][lane] = (v4i){t1s[0], t1s[1], t1s[2], t1s[3]};
                     gg = gnext;
-                    if (PS == 1 || (G & 1u) || G == g_last) __syncthreads();   // the hand-over is complete
+                    if (PS == 1 || (G & 1u)) __syncthreads();   // the hand-over is complete
                 };
-                uint32_t G = g_first;
-                for (; G + 1 < g_last; G++) kb_step(std::integral_constant<int, 1>{}, G);
-                if (G < g_last) { kb_step(std::integral_constant<int, 2>{}, G); G++; }
-                kb_step(std::integral_constant<int, 0>{}, G);
+                if constexpr (PS == 2) {
+                    for (uint32_t G = g_first & ~1u; G <= (g_last | 1u); G++) {
+                        if (G + 1 > g_first && G + 1 < g_last) kb_step(std::integral_constant<int, 1>{}, G);   // a complete group follows
+                        else kb_step(std::integral_constant<int, 2>{}, G);
+                    }
+                } else {
+                    uint32_t G = g_first;
+                    for (; G + 1 < g_last; G++) kb_step(std::integral_constant<int, 1>{}, G);
+                    if (G < g_last) { kb_step(std::integral_constant<int, 2>{}, G); G++; }
+                    kb_step(std::integral_constant<int, 0>{}, G);
+                }
                 __syncthreads();   // the first K wave's last hand-over
                 __syncthreads();   // the V waves' last hand-over
             } else if constexpr (PS == 2) {
                 if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
-                // A pair at a chunk end: either group may be missing (weights zero), the group after one may be partial or missing.
-                auto general_pair = [&](uint32_t P) {
-#pragma unroll
-                    for (int sub = 0; sub < 2; sub++) {
-                        const uint32_t G = 2 * P + sub;
-                        float wt[4][2];
-#pragma unroll
-                        for (int q = 0; q < 4; q++) wt[q][0] = wt[q][1] = 0.0f;
-                        if (G >= g_first && G <= g_last) {
-                            if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, wt, sub == 1);
-                            else if (G < g_last) group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, wt, sub == 1);
-                            else group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, wt, sub == 1);
-                        }
-#pragma unroll
-                        for (int q = 0; q < 4; q++) { ww[sub][q][0] = wt[q][0]; ww[sub][q][1] = wt[q][1]; }
-                    }
+                // A pair at a chunk end: either group may be partial or empty, and so may the group after each.
+                auto edge_pair = [&](uint32_t P) {
+                    group_core(std::integral_constant<int, 2>{}, std::false_type{}, 2 * P, ww[0], false);
+                    group_core(std::integral_constant<int, 2>{}, std::false_type{}, 2 * P + 1, ww[PS - 1], true);
                     finish_pair(P);
                 };
                 uint32_t P = g_first >> 1;
-                general_pair(P);                                         // holds the chunk's first group
+                edge_pair(P);                                            // holds the chunk's first group
                 P++;
                 for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
                     group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P, ww[0], false);
                     group_core(std::integral_constant<int, 1>{}, std::true_type{}, 2 * P + 1, ww[PS - 1], true);
                     finish_pair(P);
                 }
-                for (; P <= (g_last >> 1); P++) general_pair(P);
+                for (; P <= (g_last >> 1); P++) edge_pair(P);
                 if constexpr (NH == 2) __syncthreads();   // the V waves' last hand-over
             } else {
                 if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
@@ -527,7 +526,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         for (int hs = 0; hs < 2; hs++) {
             const float l_tot = lh_group_sum(l_run[hs], 16);
             const float w_tot = lh_group_sum(w_run[hs], 16);
-            if (pcol == 0 && !kb_role) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs]; }
+            if (pcol == 0 && !kb_role) { sh.fin_l[g + 4 * hs] = l_tot; sh.fin_w[g + 4 * hs] = w_tot; sh.fin_r[g + 4 * hs] = R[hs] <= 0.5f * kNoRef ? -INFINITY : R[hs]; }
         }
         __syncthreads();
     } else {
@@ -553,7 +552,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         for (int pl = 0; pl < 3; pl++) cfn[pl] = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv_cmax_v * (kQmax / 32767.0f);
 
         if (any) {
-            GroupGeom gg = geom(g_first);
+            GroupGeom gg = geom(PS == 2 ? (g_first & ~1u) : g_first);
             uint32_t vx[4][4];
             const uint32_t vlane = 4 * g * stride + 4 * pcol;
             auto load_v = [&](bool full, const GroupGeom& G_) {
@@ -679,26 +678,16 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 }
             };
             if constexpr (PS == 2) {
-                // A pair at a chunk end: either group may be missing, the group after one may be partial or missing.
-                auto general_pair = [&](uint32_t P) {
+                // A pair at a chunk end: either group may be partial or empty, and so may the group after each.
+                auto edge_pair = [&](uint32_t P) {
                     begin_pair(P);
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-#pragma unroll
-                        for (int f = 0; f < 4; f++) acc[e][f] = (v4i){0, 0, 0, 0};
-                    csum = (v4i){0, 0, 0, 0};
-                    for (uint32_t sub = 0; sub < 2; sub++) {
-                        const uint32_t G = 2 * P + sub;
-                        if (G < g_first || G > g_last) continue;
-                        if (G + 1 < g_last) group_core(std::integral_constant<int, 1>{}, std::false_type{}, G, sub);
-                        else if (G < g_last) group_core(std::integral_constant<int, 2>{}, std::false_type{}, G, sub);
-                        else group_core(std::integral_constant<int, 0>{}, std::false_type{}, G, sub);
-                    }
+                    group_core(std::integral_constant<int, 2>{}, std::true_type{}, 2 * P, 0u);
+                    group_core(std::integral_constant<int, 2>{}, std::false_type{}, 2 * P + 1, 1u);
                     end_pair();
                 };
                 if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
                 uint32_t P = g_first >> 1;
-                general_pair(P);                                         // holds the chunk's first group
+                edge_pair(P);                                            // holds the chunk's first group
                 P++;
                 for (; 2 * P + 2 < g_last; P++) {                        // both groups and the one after them complete
                     begin_pair(P);
@@ -706,7 +695,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     group_core(std::integral_constant<int, 1>{}, std::false_type{}, 2 * P + 1, 1u);
                     end_pair();
                 }
-                for (; P <= (g_last >> 1); P++) general_pair(P);
+                for (; P <= (g_last >> 1); P++) edge_pair(P);
                 if constexpr (NH == 2) __syncthreads();   // pairs with the K waves' count of barriers
             } else {
                 if constexpr (NH == 2) __syncthreads();   // the second K wave's first hand-over
@@ -798,11 +787,11 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
-    // Hand-overs of two groups pay from about a thousand positions per workgroup on at head_dim 256 (-1 % at 4096 positions per
-    // workgroup, -6 % at 8192); at head_dim 512 they measured 2 % slower than single groups and are only taken when forced.
+    // Hand-overs of two groups pay from about a thousand positions per workgroup on (-2 % at 4096 positions per workgroup, -5 % at
+    // 8192, either head_dim); below that the longer fill and drain of the pipeline costs more (a 512-position window: +24 %).
     static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
     static const uint64_t pair_min = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR_MIN"); return e ? (uint64_t)atoll(e) : (uint64_t)1024; }();
-    const bool pair = pair_env >= 0 ? pair_env != 0 : p.head_dim == 256 && (max_span + splits - 1) / splits >= pair_min;
+    const bool pair = pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min;
     if (p.head_dim == 512 && pair) {
         if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
         else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
