@@ -235,7 +235,7 @@ def test_split_invariance_at_32k(pkg, gpu, oracle):
 def test_context_sweep_long(pkg, gpu, oracle, T, qscale):
     """The long ends of the measured context sweep (8 q heads / 1 kv head, hd 256, 2 bits, one query, full attention):
     a peaked distribution (q from N(0, 1)) and a soft one (q * 0.15, thousands of positions carry weight, which is what
-    stresses the fixed-point value weights and their lazily moved reference).  Rotated-space output against the f64
+    stresses the 16-bit fixed-point value weights, scaled per head and 64 or 128 positions).  Rotated-space output against the f64
     code-space oracle, and the rotated-back f16 output of the one-call entry."""
     print(f"case T={T} qscale={qscale}", flush=True)
     ctx, K = gpu
