@@ -121,6 +121,41 @@ def test_decode_attention_vs_reference_cpu_path(pkg, gpu, oracle):
     check(out.as_array(np.float16).astype(np.float32), ref, "fused vs decode-then-attend", tol=ATTN_TOL + 1e-3)  # + f16 store
 
 
+@pytest.mark.parametrize("T,sink", [(4096, 0), (20000, 7000), (3000, 2999)])
+def test_attention_sink_with_flat_tail(pkg, gpu, oracle, T, sink):
+    """One position whose key is aligned with every query head (its weight ~ e^11 times a typical one) in a context
+    whose other weights are nearly flat: the tail carries several per cent of the mass in weights of about half a
+    fixed-point step of the sink's.  The value weights are scaled per head and 64 or 128 positions, so only the sink's
+    own neighbours are measured against it."""
+    print(f"case T={T} sink at {sink}", flush=True)
+    ctx, K = gpu
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    g = pkg.synth.rng(6, 77 + T)
+    q = (g.standard_normal((nq, hd), dtype=np.float32) * 0.05).astype(np.float16)
+    k = (pkg.synth.kv_rows(T, nkv, hd, g).astype(np.float32) * 0.5).astype(np.float16)
+    v = pkg.synth.kv_rows(T, nkv, hd, g)
+    qsum = q.astype(np.float32).sum(axis=0)
+    k[sink, 0] = (qsum * (11.0 / max(float(np.min(q.astype(np.float32) @ qsum)), 1e-6))).astype(np.float16)   # q_h . k_sink >= 11 for every head
+    signs, levels = oracle.rotation_signs(hd, oracle.TQ_SEED), oracle.tq_levels(hd, bits)
+    cb = oracle.tq_code_bytes(hd, bits)
+    kc = np.zeros((T, nkv, cb), np.uint8); vc = np.zeros_like(kc)
+    kn = np.zeros((T, nkv), np.uint16); vn = np.zeros_like(kn)
+    oracle.tq_write_kv(k.view(np.uint16), nkv, hd, bits, signs, levels, 0, 0, kc, kn)
+    oracle.tq_write_kv(v.view(np.uint16), nkv, hd, bits, signs, levels, 0, 0, vc, vn)
+    rq_ref = oracle.hadamard_rotate(q.astype(np.float32), signs, hd, nq, True, False)
+    acc_ref = oracle.attention_tq_codespace(rq_ref, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    kcb, knb, vcb, vnb, lvb, sgb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, signs, rq_ref)
+    vacc, out = pkg.Buffer.empty(ctx, nq * hd * 4), pkg.Buffer.empty(ctx, nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, vacc, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    K.hadamard_rotate_into(batch, vacc, sgb, out, hd, nq, False, True)
+    batch.commit_and_wait()
+    e1 = check(vacc.as_array(np.float32), acc_ref, "rotated-space accumulation")
+    ref = oracle.hadamard_rotate(acc_ref, signs, hd, nq, False, True)
+    e2 = check(out.as_array(np.float32), ref, "attention output")
+    print(f"  err rotated {e1:.2e}, output {e2:.2e}")
+
+
 def test_ring_matches_full_cache_bitwise(pkg, gpu, oracle):
     """quant_cache.rs:1047-1107: attention over a wrapped ring is bit-identical to the full cache."""
     ctx, K = gpu
