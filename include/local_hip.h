@@ -453,8 +453,9 @@ LH_API int lh_hadamard_rotate_fh_into(lh_batch* batch, const lh_buffer* input, c
  * handed over with (round to nearest); sums are exact integers, softmax sums
  * and the final scaling f32.  Measured against the f64 oracle: 1e-4 .. 3e-4 of
  * max|out|; the bound for one weight among 127 of just under half a step of it
- * is 2e-3 of that group's share.  A NaN or infinite logit or norm gives NaN
- * outputs for its head, never a finite number. */
+ * is 2e-3 of that group's share.  A head whose softmax sum is not a positive
+ * number (an empty range, a NaN logit) gives zeros, as the reference's
+ * `gsum > 0 ? 1 / gsum : 0` does (attention_flash_tq.metal:263). */
 LH_API int lh_flash_attention_tq_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
                                       const lh_buffer* k_norms, const lh_buffer* v_codes, const lh_buffer* v_norms,
                                       const lh_buffer* levels, lh_buffer* out, uint32_t head_dim, uint32_t kv_len,
