@@ -2,9 +2,9 @@
 //
 // Same contract as attention_tq.hip (stands in for shaders/attention_flash_tq.metal:154-690); this
 // kernel takes the common case -- 2-bit codes, head_dim 256 or 512, up to 8 query heads per KV head -- and
-// is bound by HBM instead of by the vector ALU.  Per cached position the path moves 132 bytes and
-// needs 8192 multiply-adds (8 heads x 256 dims x {K, V}); decoding every code to a float and
-// multiplying on the vector ALU costs ~40x more issue slots than the memory stream leaves free.
+// runs at more than half of the HBM rate instead of at a hundredth of it.  Per cached position the path
+// moves 132 bytes and needs 8192 multiply-adds (8 heads x 256 dims x {K, V}); decoding every code to a
+// float and multiplying on the vector ALU costs ~40x more issue slots than the memory stream leaves free.
 //
 // The 2-bit level table is written as L[c] = a + b*bit0(c) + g*bit1(c) (+ d*bit0*bit1, which is zero for
 // the symmetric Lloyd-Max tables and costs a third bit plane otherwise).  Bit planes are isolated with
@@ -13,9 +13,10 @@
 //   K side:  rows = 8 heads x 2 limbs of b*rq and g/2*rq (16-bit block fixed point per head), columns =
 //            16 positions, k = 64 code bytes;  logit = norm_k * (scale_h * int + a * sum(rq_h)).
 //   V side:  rows = 8 heads x 2 limbs of w = exp2(logit - R_h) * norm_v in 16-bit fixed point relative to
-//            the head's largest weight of the current group of 64 positions (a power-of-two scale, round
-//            to nearest), columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share
-//            one accumulator because their coefficients are folded into w before quantisation.  The
+//            the head's largest weight of the current hand-over (64 or 128 positions; a power-of-two scale,
+//            round to nearest), columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share
+//            one accumulator because their coefficients are folded into w before quantisation, and they are
+//            meant as centred bits (b - 1/2): the sum of the quantised weights is taken off at the end.  The
 //            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
 //            byte transposes.
 // One workgroup owns a chunk of positions and walks it in aligned groups of 64: the K wave produces the
