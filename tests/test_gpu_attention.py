@@ -156,6 +156,75 @@ def test_attention_sink_with_flat_tail(pkg, gpu, oracle, T, sink):
     print(f"  err rotated {e1:.2e}, output {e2:.2e}")
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
+    """Sixty random shapes per seed -- decode, batched lanes and prefill rows; head_dim 256 / 512; 1, 4, 6 or 8 query heads
+    per KV head over one or two KV heads; context lengths around the 64- and 128-position boundaries and up to 9000;
+    windows, wrapped rings; peaked to nearly uniform queries; now and then a level table that needs the third bit plane --
+    over caches of random code bytes and norms (any code bytes and positive f16 norms are a valid cache)."""
+    ctx, K = gpu
+    bits = 2
+    worst = 0.0
+    for case in range(60):
+        g = np.random.default_rng(seed * 1000 + case)
+        hd = int(g.choice([256, 256, 512]))
+        nkv = int(g.choice([1, 1, 2]))
+        nq = nkv * int(g.choice([8, 8, 4, 1, 6]))
+        mode = int(g.choice([0, 0, 1, 2]))          # 0 decode, 1 batched, 2 prefill
+        T = int(g.choice([1, 63, 64, 65, 127, 128, 129, 255, 300, 1000, 1025, 2049, 4096, 5000, 9000]))
+        T = max(1, T + int(g.integers(-2, 3)))
+        window = int(g.choice([0, 0, 64, 100, 512, 1024, 3000]))
+        ring = 0
+        if window and mode != 1 and g.random() < 0.5:
+            ring = ((window + 63) // 64) * 64 * int(g.choice([1, 2]))
+        qscale = float(g.choice([1.0, 0.3, 0.1, 0.02])) / 16
+        cb = oracle.tq_code_bytes(hd, bits)
+        levels = oracle.tq_levels(hd, bits)
+        if g.random() < 0.15:
+            levels = levels.copy(); levels[3] += 0.2
+        lanes, cap = 1, 0
+        if mode == 1:
+            lanes = int(g.choice([1, 3, 5])); cap = T + int(g.integers(0, 70))
+            positions = g.integers(0, T, lanes).astype(np.uint32); positions[0] = T - 1
+        phys = lanes * cap if mode == 1 else (ring if ring else T)
+        kc = g.integers(0, 256, (phys, nkv, cb), dtype=np.uint8); vc = g.integers(0, 256, (phys, nkv, cb), dtype=np.uint8)
+        kn = (g.random((phys, nkv), dtype=np.float32) * 4 + 14).astype(np.float16).view(np.uint16)
+        vn = (g.random((phys, nkv), dtype=np.float32) * 4 + 14).astype(np.float16).view(np.uint16)
+        what = f"seed {seed} case {case}: mode={mode} hd={hd} nq={nq} nkv={nkv} T={T} window={window} ring={ring} lanes={lanes}"
+        print(what, flush=True)
+        batch = pkg.CommandBatch(ctx)
+        if mode == 0:
+            rq = g.standard_normal((1, nq * hd), dtype=np.float32) * qscale
+            b = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+            out = pkg.Buffer.empty(ctx, rq.nbytes)
+            K.flash_attention_tq_into(batch, b[5], b[0], b[1], b[2], b[3], b[4], out, hd, T, T - 1, nq, nkv, window, bits, ring)
+            refs = [lambda: oracle.attention_tq_codespace(rq[0], kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, window, bits, ring)]
+        elif mode == 1:
+            rq = g.standard_normal((lanes, nq * hd), dtype=np.float32) * qscale
+            b = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, positions)
+            out = pkg.Buffer.empty(ctx, rq.nbytes)
+            K.flash_attention_tq_batched_into(batch, b[5], b[0], b[1], b[2], b[3], b[4], out, b[6], hd, cap, nq, nkv, window, bits,
+                                              lanes, 0)
+            refs = [lambda l=l: oracle.attention_tq_codespace(rq[l], kc, kn, vc, vn, levels, hd, int(positions[l]) + 1,
+                                                              int(positions[l]), nq, nkv, window, bits, 0, lane_base=l * cap)
+                    for l in range(lanes)]
+        else:
+            rows = int(min(T, g.choice([1, 3, 17])))
+            start = T - rows
+            rq = g.standard_normal((rows, nq * hd), dtype=np.float32) * qscale
+            b = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+            out = pkg.Buffer.empty(ctx, rq.nbytes)
+            K.flash_attention_tq_prefill_tiled_into(batch, b[5], b[0], b[1], b[2], b[3], b[4], out, hd, T, start, rows, nq, nkv,
+                                                    window, bits, ring)
+            refs = [lambda r=r: oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, levels, hd, T, start + r, nq, nkv, window,
+                                                              bits, ring) for r in range(rows)]
+        batch.commit_and_wait()
+        got = out.as_array(np.float32).reshape(len(refs), nq * hd)
+        for i, ref in enumerate(refs):
+            worst = max(worst, check(got[i], ref(), what))
+    print(f"worst error / scale {worst:.2e}")
+
+
 def test_ring_matches_full_cache_bitwise(pkg, gpu, oracle):
     """quant_cache.rs:1047-1107: attention over a wrapped ring is bit-identical to the full cache."""
     ctx, K = gpu

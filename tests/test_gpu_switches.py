@@ -24,7 +24,7 @@ CASES = [
     ({"LOCAL_HIP_ATTN_OCC": "1", "LOCAL_HIP_ATTN_WAVES_PER_SIMD": "3"}, "test_gpu_attention.py", "batched_matches or split_invariance or asymmetric_levels"),
     # hand-overs of two groups forced onto every chunk length (missing and partial groups at both chunk ends), and never used
     ({"LOCAL_HIP_ATTN_PAIR": "1"}, "test_gpu_attention.py", "decode_attention_matches or prefill_matches or batched_matches or "
-     "split_invariance or ring_matches or asymmetric_levels or empty_range or attention_sink"),
+     "split_invariance or ring_matches or asymmetric_levels or empty_range or attention_sink or randomised_shapes"),
     ({"LOCAL_HIP_ATTN_PAIR": "0"}, "test_gpu_attention.py", "split_invariance or context_sweep_long"),
     ({"LOCAL_HIP_PREFILL_BM": "64", "LOCAL_HIP_SKINNY_MAX_M": "64", "LOCAL_HIP_MATVEC_WG_PER_CU": "1"}, "test_gpu_matmul.py",
      "prefill_config or large_tiles or small_batch_layer_config"),
