@@ -146,6 +146,31 @@ def test_decode_batch_matmul(pkg, gpu, oracle, fmt):
         assert np.array_equal(cb.as_array(np.float32).reshape(m, n), deq[:, cols].T.astype(np.float32)), (fmt, m, k, n)
 
 
+def test_decode_batch_logits_product_full_vocabulary(pkg, gpu, oracle):
+    """The logits product of a 64-lane step at the reference's vocabulary -- [64, 1536] x [262144, 1536]^T, Q4_0, f32 result
+    (local-engine/src/pipeline.rs:914-953 once per lane) -- six lanes element by element against the oracle's product with
+    the CPU path's f16 weights, and every lane through the sum of its logits."""
+    ctx, K = gpu
+    m, k, n = 64, 1536, 262144
+    raw = pkg.synth.weights("q4_0", n, k, pkg.synth.rng(1, n))
+    deq = oracle.dequant_q4_0(raw).view(np.float16).astype(np.float32).reshape(n, k)
+    a16 = (pkg.synth.rng(4, m + k).standard_normal((m, k), dtype=np.float32) * 0.5).astype(np.float16)
+    w = pkg.QuantWeight.from_bytes(ctx, raw, pkg.Q4_0, n, k)
+    ab, cb = pkg.Buffer.from_slice(ctx, a16), pkg.Buffer.empty(ctx, m * n * 4)
+    batch = pkg.CommandBatch(ctx)
+    w.matmul_nt_typed_into(batch, K, ab, pkg.F16, cb, pkg.F32, m)
+    batch.commit_and_wait()
+    got = cb.as_array(np.float32).reshape(m, n)
+    lanes = [0, 1, 17, 31, 62, 63]
+    want = oracle.matmul_nt_f32(a16[lanes].astype(np.float32), deq)
+    refgen.assert_close_both(got[lanes].ravel(), want.ravel(), 1e-3, "logits product, six lanes")
+    colsum = deq.sum(axis=0, dtype=np.float64)                      # sum over the vocabulary of every weight column
+    want_sums = a16.astype(np.float64) @ colsum
+    got_sums = got.astype(np.float64).sum(axis=1)
+    scale = np.sqrt(n) * float(np.abs(want).mean())                  # what the sum of n independent logits amounts to
+    assert np.max(np.abs(got_sums - want_sums)) <= 2e-3 * scale, (got_sums - want_sums, scale)
+
+
 @pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
 def test_matmul_norm_fused_equals_separate_kernels(pkg, gpu, fmt):
     """matmul_nt_quant_norm_into against the sequence it stands for -- matmul_nt, rms_norm(_add), scale_in_place, a second
