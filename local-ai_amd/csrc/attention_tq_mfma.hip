@@ -783,6 +783,10 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
         splits = std::max<uint64_t>(1, wg_slots / pairs);
         splits = std::min<uint64_t>(splits, (max_span + 127) / 128);
     }
+    // The merge takes 256 splits of a query in one round of loads and every further 256 in a dependent round of their own (about
+    // 2 us each), so one or two long queries keep 256 splits until a chunk passes 1024 positions (131072 positions, one query:
+    // 20.5 us with 256 splits, 21.7 with 512, 25.8 with 1024).
+    if (splits > 256) splits = std::max<uint64_t>(256, std::min<uint64_t>(splits, (max_span + 1023) / 1024));
     splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
     const size_t rec = partial_record_floats(p.head_dim);
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
