@@ -2,7 +2,7 @@
 //!
 //! `ffi` holds the raw declarations of `liblocal_hip.so` (generated from `include/local_hip.h`).  The safe layer
 //! with the reference's type and method names (`Context`, `Buffer`, `CommandBatch`, `Kernels::<op>_into`, and an
-//! `Error` enum with the variants of `local_metal::Error`) wraps them one to one; its outline is in INTEGRATION.md.
+//! `Error` enum with the variants of `local_metal::Error`) wraps them one to one.
 pub mod ffi;
 
 use core::ffi::CStr;
