@@ -146,6 +146,76 @@ def test_decode_batch_matmul(pkg, gpu, oracle, fmt):
         assert np.array_equal(cb.as_array(np.float32).reshape(m, n), deq[:, cols].T.astype(np.float32)), (fmt, m, k, n)
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
+    """Fifty random products per seed through the typed entries: either format, 1 .. 700 activation rows (every routing
+    boundary on the way: rows as matvecs, the small-batch kernels, 64- and 128-row tiles, k splits), k any multiple of the
+    block size up to 8192 (now and then 24576), 1 .. 20000 weight rows, f16 / f32 / bf16 activations, f16 / f32 results,
+    generated weights or random bytes with large scales (TQ2 code 3 included).  Gate: max|g - w| <= tol * max(1, max|w|)
+    against the product with the CPU path's f16 weights or with the unrounded ones, whichever is nearer (the small-batch
+    Q4_0 kernels keep f32 weights like the reference's), tol 1e-3 for f32 and 2e-3 for f16 results; and the reference's own
+    per-element form at its tolerances (0.01 / 0.03) except for f32 activations of more than 16 rows, which are rounded
+    to f16 before the matrix cores."""
+    ctx, K = gpu
+    ms = [1, 1, 1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 24, 31, 32, 33, 48, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300,
+          511, 512, 513, 700]
+    worst = 0.0
+    for case in range(50):
+        g = np.random.default_rng(seed * 100000 + case)
+        fmt = "q4_0" if g.random() < 0.5 else "tq2_0"
+        unit = 32 if fmt == "q4_0" else 256
+        kmax = 8192 if g.random() < 0.85 else 24576
+        k = unit * int(g.integers(1, kmax // unit + 1))
+        if g.random() < 0.3:
+            k = int(g.choice([1536, 2048, 4096, 6144, 8192, 12288]))
+        m = int(g.choice(ms))
+        nmax = max(1, min(20000, 20_000_000 // k))
+        n = int(g.integers(1, nmax + 1))
+        if g.random() < 0.3:
+            n = min(nmax, int(g.choice([16, 64, 100, 128, 256, 1536, 2048, 4096, 8192])))
+        while m * n * 4 > 32_000_000:
+            m = max(1, m // 2)
+        adt = int(g.choice([pkg.F16, pkg.F32, pkg.BF16])) if m > 1 else int(g.choice([pkg.F16, pkg.F32]))
+        cdt = int(g.choice([pkg.F16, pkg.F32]))
+        what = f"seed {seed} case {case}: {fmt} m={m} k={k} n={n} activations {adt} result {cdt}"
+        print(what, flush=True)
+        raw = pkg.synth.weights(fmt, n, k, g)
+        if g.random() < 0.5:
+            raw = g.integers(0, 256, raw.size, dtype=np.uint8)
+            blk, doff = (18, 0) if fmt == "q4_0" else (66, 64)
+            raw.reshape(-1, blk)[:, doff:doff + 2] = (0.01 + g.random(raw.size // blk) * 0.1).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        a = g.standard_normal((m, k), dtype=np.float32) * np.float32(g.choice([1.0, 0.5, 0.05]))
+        if adt == pkg.F16:
+            a_dev = a.astype(np.float16); a_val = a_dev.astype(np.float32)
+        elif adt == pkg.BF16:
+            a_dev = pkg.synth.f32_to_bf16_bits(a); a_val = pkg.synth.bf16_bits_to_f32(a_dev)
+        else:
+            a_dev = a_val = a
+        deq16 = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+        want16, want32 = oracle.matmul_nt_f32(a_val, deq16), oracle.matmul_nt_f32(a_val, expand(oracle, fmt, raw, n, k))
+        ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+        w = pkg.QuantWeight.from_bytes(ctx, raw, ty, n, k)
+        ab = pkg.Buffer.from_slice(ctx, a_dev)
+        guard = 64                                             # bytes behind the output stay untouched
+        cb = pkg.Buffer.from_slice(ctx, np.full(m * n * (4 if cdt == pkg.F32 else 2) + guard, 0xA5, np.uint8))
+        batch = pkg.CommandBatch(ctx)
+        if m == 1:
+            K.matvec_quant_typed_into(batch, ty, w.buf, ab, adt, cb, cdt, n, k)
+        else:
+            w.matmul_nt_typed_into(batch, K, ab, adt, cb, cdt, m)
+        batch.commit_and_wait()
+        got = (cb.as_array(np.float32, m * n) if cdt == pkg.F32 else cb.as_array(np.float16, m * n).astype(np.float32)).reshape(m, n)
+        assert (cb.as_array(np.uint8)[-guard:] == 0xA5).all(), what
+        scale = max(1.0, float(np.abs(want16).max()))
+        e = min(float(np.abs(got - want16).max()), float(np.abs(got - want32).max())) / scale
+        assert e <= (1e-3 if cdt == pkg.F32 else 2e-3), (what, e)
+        if not (adt == pkg.F32 and m > 16):
+            per_element = min(float(np.max(np.abs(got - wnt) / np.maximum(np.abs(wnt), 1.0))) for wnt in (want16, want32))
+            assert per_element <= (1e-2 if cdt == pkg.F32 else 3e-2), (what, per_element)
+        worst = max(worst, e)
+    print(f"worst error / max(1, max|w|) {worst:.2e}")
+
+
 def test_decode_batch_logits_product_full_vocabulary(pkg, gpu, oracle):
     """The logits product of a 64-lane step at the reference's vocabulary -- [64, 1536] x [262144, 1536]^T, Q4_0, f32 result
     (local-engine/src/pipeline.rs:914-953 once per lane) -- six lanes element by element against the oracle's product with
