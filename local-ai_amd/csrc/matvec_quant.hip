@@ -583,6 +583,14 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
     if (want > cap) want = cap;
     if (want < 1) want = 1;
     g.steps_per_wg = (uint32_t)((steps + want - 1) / want);
+    // Several workgroups per problem (the rows of a small activation batch): a share that divides a problem's steps keeps
+    // every workgroup inside one problem, so none stages a second vector half way (7 rows against 2048 x 2048: 7.2 -> 5.4 us).
+    const uint32_t spp = (rows + g.rpw - 1) / g.rpw;
+    if (count > 1 && g.steps_per_wg * 2 <= spp && spp % g.steps_per_wg != 0) {
+        uint32_t s = g.steps_per_wg;
+        while (s < 2 * g.steps_per_wg && spp % s != 0) s++;
+        if (spp % s == 0) g.steps_per_wg = s;
+    }
     g.grid = (uint32_t)((steps + g.steps_per_wg - 1) / g.steps_per_wg);
     const uint32_t G = fmt == LH_TQ2_0 ? 256 : 32;
     g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4 + (L == 2 ? (size_t)2 * K + (size_t)(K / G) * 4 + 16 : 0);
