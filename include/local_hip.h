@@ -206,11 +206,13 @@ LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, co
                                      lh_buffer* output, uint32_t m, uint32_t k, uint32_t n);
 /* Typed form: A f16 / f32 / bf16, C f16 / f32 (the measured small-batch and
  * prefill configurations use f32 and bf16 activations).  Up to 16 rows of f32
- * activations run as rows of the matvec and stay f32; products of more rows
- * multiply on the matrix cores in f16 like the reference's kernels, whose
- * activations are f16 (kernels.rs:6459-6563): bf16 activations convert exactly
- * (down to the f16 subnormals), f32 activations are rounded to f16 first, which
- * costs up to 3e-4 of the largest output in absolute terms. */
+ * activations run as rows of the matvec and stay f32; up to 32 rows (TQ2_0
+ * from 10 rows on) enter the matrix cores as two f16 rows each, the rounded
+ * value and the remainder, and keep about 22 bits.  Larger products multiply
+ * in f16 like the reference's kernels, whose activations are f16
+ * (kernels.rs:6459-6563): bf16 activations convert exactly (down to the f16
+ * subnormals), f32 activations are rounded to f16 first, which costs up to
+ * 3e-4 of the largest output in absolute terms. */
 LH_API int lh_matmul_nt_quant_typed_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, lh_dtype input_dtype,
                                          const lh_buffer* weight, lh_buffer* output, lh_dtype output_dtype,
                                          uint32_t m, uint32_t k, uint32_t n);

@@ -696,7 +696,10 @@ __device__ __forceinline__ f16x8 skinny_fragment(const SkinnyRaw& raw, int f) {
 // PAIR: the feed-forward gate and up projections with their gelu_mul (layer.rs:652-662).  The workgroup's tiles 0, 1 are 32
 // rows of grp.W[0] (gate), tiles 2, 3 the same 32 rows of grp.W[1] (up), so that both factors of an output meet in the
 // reduction: out = half(gelu(half(gate)) * half(up)), the values the two products and gelu_mul would have stored.
-template <int FMT, int CDT, bool PAIR = false>
+// XF32: f32 activations, at most 32 rows.  A row enters as two f16 rows -- x rounded to f16 in activation group j (rows 16j ..
+// 16j + 15, j = 0, 1) and the remainder x - f16(x), rounded to f16, in group j + 2 -- and the two outputs are added at the
+// end: the product then carries about 22 bits of every activation instead of 11.
+template <int FMT, int CDT, bool PAIR = false, bool XF32 = false>
 __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ W_one, void* __restrict__ C_one,
                                                               uint32_t M, uint32_t K, uint32_t N_one, float* __restrict__ partial,
                                                               uint32_t units_per_wave, GroupArgs grp) {
@@ -747,17 +750,47 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     if constexpr (FMT == kQ4) { ld_g = 2 * (ld_q >> 2) + (ld_q & 1); ld_f = (ld_q & 3) >> 1; }
     else { ld_f = ld_q >> 2; ld_g = ld_q & 3; }
     auto load_b = [&](f32x4 (&raw)[NLD], uint32_t k0) {
+        if constexpr (XF32) {   // rows 0 .. 31 only, eight f32 values = two registers of the set per row
+            const float* X32 = reinterpret_cast<const float*>(X);
 #pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            const uint32_t m = m0 + RPI * i + ld_row;
-            raw[i] = *reinterpret_cast<const f32x4*>(X + (size_t)(m < M ? m : M - 1) * K + k0 + 8 * ld_q);   // rows past M repeat the last one
+            for (int i = 0; i < NLD / 2; i++) {
+                const uint32_t m = RPI * i + ld_row;
+                const float* p = X32 + (size_t)(m < M ? m : M - 1) * K + k0 + 8 * ld_q;
+                raw[2 * i] = *reinterpret_cast<const f32x4*>(p);
+                raw[2 * i + 1] = *reinterpret_cast<const f32x4*>(p + 4);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                const uint32_t m = m0 + RPI * i + ld_row;
+                raw[i] = *reinterpret_cast<const f32x4*>(X + (size_t)(m < M ? m : M - 1) * K + k0 + 8 * ld_q);   // rows past M repeat the last one
+            }
         }
     };
     auto park_b = [&](const f32x4 (&raw)[NLD]) {
+        if constexpr (XF32) {
 #pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            const uint32_t m = RPI * i + ld_row, j = m >> 4, c = m & 15;
-            stage[(ld_f * 4 + j) * 64 + ld_g * 16 + (c ^ (ld_g | ((ld_f & 1) << 2)))] = raw[i];
+            for (int i = 0; i < NLD / 2; i++) {
+                const uint32_t m = RPI * i + ld_row, j = m >> 4, c = m & 15;
+                const float x[8] = {raw[2 * i][0], raw[2 * i][1], raw[2 * i][2], raw[2 * i][3],
+                                    raw[2 * i + 1][0], raw[2 * i + 1][1], raw[2 * i + 1][2], raw[2 * i + 1][3]};
+                struct { uint32_t v[4]; } hi, lo;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint16_t h0 = lh_f2h(x[2 * e]), h1 = lh_f2h(x[2 * e + 1]);
+                    hi.v[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+                    lo.v[e] = pack_h2(x[2 * e] - lh_h2f(h0), x[2 * e + 1] - lh_h2f(h1));
+                }
+                const uint32_t cell = ld_g * 16 + (c ^ (ld_g | ((ld_f & 1) << 2)));
+                stage[(ld_f * 4 + j) * 64 + cell] = __builtin_bit_cast(f32x4, hi);
+                stage[(ld_f * 4 + j + 2) * 64 + cell] = __builtin_bit_cast(f32x4, lo);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                const uint32_t m = RPI * i + ld_row, j = m >> 4, c = m & 15;
+                stage[(ld_f * 4 + j) * 64 + ld_g * 16 + (c ^ (ld_g | ((ld_f & 1) << 2)))] = raw[i];
+            }
         }
     };
 
@@ -834,12 +867,21 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     }
     // wave w finishes tile w: D[row 4g + i][activation row r] of each group j
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < (XF32 ? 2 : 4); j++) {
         float4 v = red[0][wave][j][lane];
 #pragma unroll
         for (int w = 1; w < 4; w++) {
             const float4 o = red[w][wave][j][lane];
             v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+        }
+        if constexpr (XF32) {   // the remainders' product
+            float4 u = red[0][wave][j + 2][lane];
+#pragma unroll
+            for (int w = 1; w < 4; w++) {
+                const float4 o = red[w][wave][j + 2][lane];
+                u.x += o.x; u.y += o.y; u.z += o.z; u.w += o.w;
+            }
+            v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
         }
         const uint32_t m = m0 + 16 * j + r;
         if (m >= M) continue;
@@ -972,6 +1014,13 @@ __global__ __launch_bounds__(256, 2) void matmul_small_q4_kernel(const uint16_t*
 // from 9 rows (LOCAL_HIP_SKINNY_MIN_M; the matvec kernels are as fast up to 8): up to 16 rows go to matmul_small_q4_kernel,
 // which keeps the weights unrounded as the reference's small-batch kernels do (16 lanes 3.95 -> 3.80 ms); from 17 rows on
 // the weights are the CPU path's f16 values, as in its matrix kernels.
+// Fewest f32 activation rows the TQ2_0 skinny kernel takes (LOCAL_HIP_SKINNY_MIN_M_F32); below it the rows run as matvecs.
+// One layer's three TQ2_0 projections, weights cache resident: rows 34.3 / 42.2 / 47.4 us at 8 / 12 / 16 rows, this form
+// 36.3 / 36.8 / 37.6 us.
+uint32_t skinny_min_m_f32() {
+    static const int v = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_F32"); return e && atoi(e) > 0 ? atoi(e) : 10; }();
+    return (uint32_t)v;
+}
 uint32_t skinny_min_m(int fmt) {
     static const int q4 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M"); return e && atoi(e) > 0 ? atoi(e) : 9; }();
     static const int tq2 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_TQ2"); return e && atoi(e) > 0 ? atoi(e) : 2; }();
@@ -1008,6 +1057,29 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
                 const GroupArgs& grp, SkinnyPartials* keep = nullptr) {
     hipStream_t s = ctx->stream;
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
+    if constexpr (FMT != kF16W && ADT == LH_F32) {
+        // f32 activations as pairs of f16 rows: up to 32 rows.  TQ2_0 from skinny_min_m_f32() rows (below that the rows run as
+        // matvecs); Q4_0 from 17 rows (up to 16 the matvec rows multiply unrounded weights, as the reference's kernels do).
+        static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
+        const uint32_t units = k / Skinny<FMT>::unit_k;
+        const uint32_t min_m = FMT == kTQ2 ? skinny_min_m_f32() : (uint32_t)kMaxMultivecM + 1;
+        if (!no_skinny && !clip.enabled && !grp.count && !keep && m >= min_m && m <= 32 && n % BN == 0 && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+            2 * tiles_n <= skinny_max_blocks(ctx)) {
+            const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
+            const uint32_t splits = skinny_splits(ctx, m, blocks, per_wg);
+            float* partial = splits > 1 ? static_cast<float*>(ctx->workspace) : nullptr;
+            const dim3 grid(blocks, 1, splits);
+            const uint16_t* X = static_cast<const uint16_t*>(A);
+            if (ct == LH_F32) hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F32, false, true>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
+            else hipLaunchKernelGGL((matmul_skinny_kernel<FMT, LH_F16, false, true>), grid, dim3(256), 0, s, X, W, C, m, k, n, partial, per_wg / splits, grp);
+            if (splits > 1) {
+                const uint32_t rgrid = (uint32_t)(((size_t)m * tiles_n * BN + 255) / 256);
+                if (ct == LH_F32) hipLaunchKernelGGL((splitk_reduce_kernel<LH_F32>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+                else hipLaunchKernelGGL((splitk_reduce_kernel<LH_F16>), dim3(rgrid), dim3(256), 0, s, partial, C, m, n, tiles_n, splits, clip, grp);
+            }
+            return true;
+        }
+    }
     if constexpr (FMT != kF16W && ADT == LH_F16) {
         static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
         bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
@@ -1164,6 +1236,13 @@ int matmul_dispatch(lh_batch* batch, const char* op, int kind, const lh_buffer* 
         const bool took = kind == kQ4 ? try_skinny<kQ4, LH_F16>(batch->ctx, input->ptr, Ws, output->ptr, ct, m, k, n, clip, GroupArgs{})
                                       : try_skinny<kTQ2, LH_F16>(batch->ctx, input->ptr, Ws, output->ptr, ct, m, k, n, clip, GroupArgs{});
         if (took) {
+            int r = lh_check_launch(op);
+            if (r == LH_OK) batch->dispatch_count++;
+            return r;
+        }
+    }
+    if (!mfma && !force_multivec && at == LH_F32 && kind == kTQ2 && m >= skinny_min_m_f32()) {   // f32 rows as pairs of f16 rows
+        if (try_skinny<kTQ2, LH_F32>(batch->ctx, input->ptr, (const uint8_t*)weight->ptr, output->ptr, ct, m, k, n, clip, GroupArgs{})) {
             int r = lh_check_launch(op);
             if (r == LH_OK) batch->dispatch_count++;
             return r;

@@ -146,6 +146,43 @@ def test_decode_batch_matmul(pkg, gpu, oracle, fmt):
         assert np.array_equal(cb.as_array(np.float32).reshape(m, n), deq[:, cols].T.astype(np.float32)), (fmt, m, k, n)
 
 
+@pytest.mark.parametrize("fmt", ["q4_0", "tq2_0"])
+def test_decode_batch_f32_activations(pkg, gpu, oracle, fmt):
+    """f32 activation rows of a small batch (10 .. 32 rows for TQ2_0, 17 .. 32 for Q4_0) enter the matrix cores as pairs of
+    f16 rows, x rounded and the remainder, whose products are added: against the oracle's product with the CPU path's f16
+    weights the result then keeps f32 accuracy (2e-5 of the largest output; a single f16 row would give 3e-4), also for
+    activations that span six orders of magnitude in one row.  One more row than the form takes falls back to the tiled
+    kernels and their single rounding."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    rows = (10, 11, 16, 17, 32) if fmt == "tq2_0" else (17, 25, 32)
+    for (k, n) in ((2048, 8192), (8192, 2048), (1536, 256)):
+        raw = payload(fmt, n, k, 0xF32 + k)
+        deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+        w = pkg.QuantWeight.from_bytes(ctx, raw, ty, n, k)
+        for m in rows + (33,):
+            for wide in (False, True):
+                g = pkg.synth.rng(9, m * 7 + k + wide)
+                a = g.standard_normal((m, k), dtype=np.float32)
+                if wide:
+                    a *= np.float32(10.0) ** g.integers(-3, 4, (m, k)).astype(np.float32)
+                print(f"case {fmt} m={m} k={k} n={n} wide={wide}", flush=True)
+                want = oracle.matmul_nt_f32(a, deq)
+                for ct, npt in ((pkg.F32, np.float32), (pkg.F16, np.float16)):
+                    ab = pkg.Buffer.from_slice(ctx, a)
+                    guard = 64
+                    cb = pkg.Buffer.from_slice(ctx, np.full(m * n * np.dtype(npt).itemsize + guard, 0xA5, np.uint8))
+                    batch = pkg.CommandBatch(ctx)
+                    w.matmul_nt_typed_into(batch, K, ab, pkg.F32, cb, ct, m)
+                    batch.commit_and_wait()
+                    got = cb.as_array(npt, m * n).astype(np.float32).reshape(m, n)
+                    assert (cb.as_array(np.uint8)[-guard:] == 0xA5).all()
+                    fin = np.isfinite(want) & (np.abs(want) < 6e4)
+                    e = float(np.abs(got - want)[fin].max()) / max(1.0, float(np.abs(want[fin]).max()))
+                    tol = 1e-3 if ct == pkg.F16 else (2e-5 if m <= 32 else 1e-3)
+                    assert e <= tol, (fmt, m, k, n, wide, ct, e)
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
     """Fifty random products per seed through the typed entries: either format, 1 .. 700 activation rows (every routing
