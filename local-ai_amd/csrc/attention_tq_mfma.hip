@@ -17,8 +17,8 @@
 //            round to nearest), columns = 16 code-byte columns (x 4 fields), k = 64 positions; the planes share
 //            one accumulator because their coefficients are folded into w before quantisation, and they are
 //            meant as centred bits (b - 1/2): the sum of the quantised weights is taken off at the end.  The
-//            position-major codes become "one code byte over four positions" words by v_perm_b32 4x4
-//            byte transposes.
+//            position-major codes become "one code byte over many positions" operands on their way through the
+//            wave's LDS area: stored as loaded, read back with the transposing read ds_read_b64_tr_b8.
 // One workgroup owns a chunk of positions and walks it in aligned groups of 64: the K wave produces the
 // softmax weights of a group (or of an aligned pair of groups, for long chunks), a V wave per 256 output
 // dims, one hand-over behind with one barrier per hand-over, turns them into limbs, multiplies and adds
@@ -38,6 +38,7 @@ namespace {
 using namespace lh_attn;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned short us2_t __attribute__((ext_vector_type(2)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
@@ -58,18 +59,6 @@ __device__ __forceinline__ float ld_norm(gptr_t p) {
     return lh_h2f(*reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>(p));
 }
 
-// 4x4 byte transpose: x[q] holds bytes e = 0..3 of position q; y[e] gets byte e of positions 0..3.
-__device__ __forceinline__ void transpose4x4(const uint32_t (&x)[4], uint32_t (&y)[4]) {
-    const uint32_t t0 = __builtin_amdgcn_perm(x[1], x[0], 0x05010400u);
-    const uint32_t t1 = __builtin_amdgcn_perm(x[1], x[0], 0x07030602u);
-    const uint32_t t2 = __builtin_amdgcn_perm(x[3], x[2], 0x05010400u);
-    const uint32_t t3 = __builtin_amdgcn_perm(x[3], x[2], 0x07030602u);
-    y[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
-    y[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
-    y[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
-    y[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
-}
-
 struct GroupGeom {
     uint32_t pb;        // physical slot of the group's first position
     uint32_t vlo, vhi;  // valid positions of the group: [vlo, vhi) within 0..64
@@ -88,6 +77,7 @@ struct AttnShared {
     float4 ww[2][PS][2][64];       // [buffer][group of the pair][head set][lane]: the K wave's weights of tiles 0..3, for the V wave
     float2 wsc[2][kMaxGroupHeads]; // [buffer][head]: (scale that takes the head's weights of this pair into [-1, 1], value of one integer step)
     uint8_t wx[NH][3][1024];       // [V wave][plane]: that wave's A operands (weights as limbs)
+    uint8_t vt[NH][kGroup * 64];   // [V wave]: a group's V codes (64 bytes per position, 16-byte chunks swizzled), read back transposed
     v4i tb[NH == 2 ? 2 : 1][PS][2][64]; // head_dim 512: [buffer][group of the pair][head set][lane]: the second K wave's integer logit sums of tiles 0..3 (code half 1)
     float fsc[2][kMaxGroupHeads];  // [buffer][head]: factor for the float outputs when the reference moved
     uint32_t moved[2];             // [buffer]: the reference moved within this pair: rescale the outputs
@@ -533,7 +523,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     } else {
         // =================================================================== V wave
         gptr_t vrec0 = (gptr_t)a.v_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * vhalf;
-        float outv[4][4][2];   // [code byte e][field f][head set]: dim 16*pcol + 4e + f of head g + 4 * set, relative to exp2(R)
+        float outv[4][4][2];   // [chunk e][field f][head set]: dim 64e + 4*pcol + f of head g + 4 * set, relative to exp2(R)
 #pragma unroll
         for (int e = 0; e < 4; e++)
 #pragma unroll
@@ -554,21 +544,44 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 
         if (any) {
             GroupGeom gg = geom(PS == 2 ? (g_first & ~1u) : g_first);
-            uint32_t vx[4][4];
-            const uint32_t vlane = 4 * g * stride + 4 * pcol;
+            // A group's V codes: lane L fetches 16-byte chunk L % 4 of positions 16q + L / 4 (a load instruction covers 16 whole
+            // positions, 1 KB contiguous for one KV head) and parks it in the wave's LDS area; the MFMA's B operand wants "one
+            // code byte over 16 positions" per lane, which ds_read_b64_tr_b8 delivers: within 16 lanes, lane i names an 8-byte
+            // row and lane l receives byte l % 8 of rows 2j + l / 8, j = 0 .. 7.  Rows 2j / 2j + 1 are the two halves of a
+            // 16-byte chunk of one position, so the 16 lanes get the 16 code bytes of a chunk over 8 positions.  The chunk index
+            // is XORed with q and the positions of a read are spread over p % 4, which keeps both directions free of bank
+            // conflicts without padding.
+            u32x4_t vx[4];
+            const uint32_t vpos = lane >> 2, vchunk = lane & 3;
+            const uint32_t vlane = vpos * stride + 16 * vchunk;
             auto load_v = [&](bool full, const GroupGeom& G_) {
                 gptr_t vb = vrec0 + (size_t)G_.pb * stride;
 #pragma unroll
-                for (int m = 0; m < 4; m++)
-#pragma unroll
-                    for (int qq = 0; qq < 4; qq++) {
-                        if (full) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
-                        else {
-                            vx[m][qq] = 0u;
-                            if (is_valid(G_, 16 * qq + 4 * g + m)) vx[m][qq] = ld4(vb + (size_t)(16 * qq + m) * stride + vlane);
-                        }
+                for (int q = 0; q < 4; q++) {
+                    if (full) vx[q] = ld16(vb + (size_t)(16 * q) * stride + vlane);
+                    else {
+                        vx[q] = (u32x4_t){0u, 0u, 0u, 0u};
+                        if (is_valid(G_, 16 * q + vpos)) vx[q] = ld16(vb + (size_t)(16 * q) * stride + vlane);
                     }
+                }
             };
+            typedef __attribute__((address_space(3))) uint8_t* lds8_t;
+            typedef __attribute__((address_space(3))) v2i* lds_v2i_t;
+            typedef __attribute__((address_space(3))) u32x4_t* lds_x4_t;
+            const lds8_t vt = (lds8_t)&sh.vt[vhalf][0];
+            uint32_t wr_off[4], rd_off[4][2];   // [q] / [16-byte chunk e][read t]
+#pragma unroll
+            for (int q = 0; q < 4; q++) wr_off[q] = (16 * q + vpos) * 64 + ((vchunk ^ q) & 3) * 16;
+            {
+                const uint32_t i = lane & 15, A_ = lane >> 4, j = i >> 1, qj = j & 3;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const uint32_t B_ = 2 * t + (j >> 2);                           // word of the operand this row feeds
+                    const uint32_t src = 16 * qj + 4 * A_ + ((B_ + 2 * A_) & 3);    // position (column position 4A + ..., tile qj)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) rd_off[e][t] = src * 64 + ((e ^ qj) & 3) * 16 + 8 * (i & 1);
+                }
+            }
             load_v(gg.full, gg);
 
             v4i acc[4][4];      // [code byte e][field f]: the pair's integer sums, rows = heads g, g + 4 x 2 limbs
@@ -609,7 +622,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 //      weights of column position pcol of the four tiles, i.e. one k word of the MFMA's A operand:
                 //      lane (column 4A+B, row group g) feeds rows 4g + 2 * set + limb of k-group A, word B.
                 {
-                    const uint32_t A_ = pcol >> 2, B_ = pcol & 3;
+                    const uint32_t A_ = pcol >> 2, B_ = ((pcol & 3) + 2 * (pcol >> 2)) & 3;   // k group and word: where the V codes of positions 16q + pcol land
                     __builtin_amdgcn_wave_barrier();
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
@@ -629,10 +642,21 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
-                uint32_t y[4][4];   // [word m][code byte e]: byte e of positions 16qq + 4g + m, qq = 0..3
+                uint32_t y[4][4];   // [word m][chunk e]: code byte 16e + pcol of the four positions of operand word m
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int m = 0; m < 4; m++) transpose4x4(vx[m], y[m]);
+                for (int q = 0; q < 4; q++) *(lds_x4_t)(vt + wr_off[q]) = vx[q];
+                __builtin_amdgcn_wave_barrier();
                 if constexpr (KIND != 0) load_v(KIND == 1, geom(G + 1));   // the V registers are free
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_t)(vt + rd_off[e][t]));
+                        y[2 * t][e] = (uint32_t)r.x;
+                        y[2 * t + 1][e] = (uint32_t)r.y;
+                    }
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int pl = 0; pl < nplanes; pl++) {
                     const v4i wop = *reinterpret_cast<const v4i*>(&sh.wx[vhalf][pl][lane * 16]);
@@ -720,18 +744,18 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             const uint32_t qh = kvh * group + h;
             const float bias = (alpha + 0.5f * (beta + gam) + (has_delta ? 0.25f * delta : 0.0f)) * w_tot - sctr[hs];
             if (nsplit == 1) {
-                float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 16 * pcol;
+                float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 4 * pcol;
                 const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    *reinterpret_cast<float4*>(dst + 4 * e) = make_float4((outv[e][0][hs] + bias) * inv, (outv[e][1][hs] + bias) * inv,
+                    *reinterpret_cast<float4*>(dst + 64 * e) = make_float4((outv[e][0][hs] + bias) * inv, (outv[e][1][hs] + bias) * inv,
                                                                           (outv[e][2][hs] + bias) * inv, (outv[e][3][hs] + bias) * inv);
             } else {
                 float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * nsplit + split) * partial_record_floats(kHeadDim);
                 if (pcol == 0 && vhalf == 0) { rec[0] = sh.fin_r[h] * kLn2; rec[1] = l_tot; }
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    *reinterpret_cast<float4*>(rec + 4 + 256 * vhalf + 16 * pcol + 4 * e) =
+                    *reinterpret_cast<float4*>(rec + 4 + 256 * vhalf + 4 * pcol + 64 * e) =
                         make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
             }
         }

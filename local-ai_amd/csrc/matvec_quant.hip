@@ -28,6 +28,7 @@ namespace {
 constexpr int kWG = 256;          // threads per workgroup (4 waves)
 constexpr int kWaves = kWG / 64;
 constexpr uint32_t kMaxFastCols = 16384;  // 4 unit columns per lane at most
+constexpr size_t kMaxDynamicLds = 96 * 1024;   // what launch_typed raises a kernel's dynamic LDS limit to
 
 struct MatvecProblem {
     const uint8_t* matrix;
@@ -597,7 +598,10 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
     // the staged form pays off once a wave walks several steps (its first fetch is not overlapped with anything)
     const uint32_t in_flight = g.npos == 1 ? 4u : (g.npos == 2 ? 2u : 1u);        // steps_in_flight<LH_Q4_0>(npos)
     g.img = fmt == LH_Q4_0 && L == 2 && min_slack >= 16 && g.steps_per_wg >= 2u * kWaves * in_flight && q4_image_enabled();
-    if (g.img) g.lds_bytes = ((g.lds_bytes + 15) & ~(size_t)15) + (size_t)kWaves * kImgBytes;
+    // The images come on top of the activation area; rows long enough to push the sum past the raised limit keep direct loads.
+    const size_t with_img = ((g.lds_bytes + 15) & ~(size_t)15) + (size_t)kWaves * kImgBytes;
+    if (g.img && with_img > kMaxDynamicLds) g.img = false;
+    if (g.img) g.lds_bytes = with_img;
     return g;
 }
 
@@ -606,8 +610,11 @@ int launch_typed(lh_context* ctx, const MatvecProblem* dev_problems, const Matve
                  lh_dtype yt, uint32_t rows, uint32_t K, const LaunchGeom& g) {
 #define LH_LAUNCH_K(KERNEL)                                                                                                 \
     do {                                                                                                                    \
+        if (g.lds_bytes > kMaxDynamicLds)                                                                                   \
+            return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: %zu bytes of LDS needed, limit %zu", g.lds_bytes,        \
+                           (size_t)kMaxDynamicLds);                                                                         \
         if (g.lds_bytes > 64 * 1024) {   /* long rows: more than the 64 KB a kernel gets without asking */                  \
-            const int rl = lh_raise_dynamic_lds(ctx, (const void*)KERNEL, 96 * 1024, "matvec_quant");                       \
+            const int rl = lh_raise_dynamic_lds(ctx, (const void*)KERNEL, kMaxDynamicLds, "matvec_quant");                  \
             if (rl != LH_OK) return rl;                                                                                     \
         }                                                                                                                   \
         hipLaunchKernelGGL(KERNEL, dim3(g.grid), dim3(kWG), g.lds_bytes, ctx->stream,                                       \

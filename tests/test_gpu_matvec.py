@@ -45,11 +45,14 @@ def test_matvec_reference_payloads(pkg, gpu, oracle, fmt, rows, cols):
 
 
 @pytest.mark.parametrize("fmt,rows,cols", [("q4_0", 2048, 2048), ("tq2_0", 8192, 2048), ("tq2_0", 2048, 8192),
-                                           ("q4_0", 256, 2048), ("q4_0", 262144, 1536)])
+                                           ("q4_0", 256, 2048), ("q4_0", 262144, 1536),
+                                           ("q4_0", 4096, 16384), ("q4_0", 4000, 14400)])
 def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
-    """The measured configurations (the last one is the logits product of the reference's decode tail,
+    """The measured configurations (the fifth one is the logits product of the reference's decode tail,
     local-engine/src/pipeline.rs:914-953, at its full vocabulary): fp32 x, fp32 y, against the reference CPU path
-    (block dequant to f16 then a sequential f32 dot), max normalised error <= 1e-3."""
+    (block dequant to f16 then a sequential f32 dot), max normalised error <= 1e-3.  The last two have rows so long
+    that the activation area alone nearly fills the kernel's LDS limit (many rows per workgroup, so that the staged
+    form would be chosen if it fitted): they must run, on direct loads."""
     print(f"case {fmt} {rows}x{cols}", flush=True)
     g = pkg.synth.rng(1 if fmt == "q4_0" else 2, rows)
     raw = pkg.synth.weights(fmt, rows, cols, g)
