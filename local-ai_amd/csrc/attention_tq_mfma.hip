@@ -98,6 +98,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     constexpr int kHeadDim = HD, kCodeBytes = HD / 4, NH = HD / 256;   // NH: 64-byte halves of a code
     constexpr bool has_delta = NPL == 3;
     constexpr int nplanes = NPL;
+    // The two-plane forms are only entered with a level table whose mean is zero to rounding (any symmetric table): the
+    // constant term of the centred planes then vanishes and the exact sum of the weights is not needed.
+    constexpr bool need_wsum = NPL == 3;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const uint32_t pcol = lane & 15, g = lane >> 4;               // MFMA column / row group of this lane
     const uint32_t qi = blockIdx.y / p.num_kv_heads, kvh = blockIdx.y - qi * p.num_kv_heads;
@@ -343,8 +346,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 #pragma unroll
                     for (int hs = 0; hs < 2; hs++) {
                         // three shift-adds: limbs first, then the two field scales
-                        const uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
-                        const uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
+                        uint32_t t1 = ((uint32_t)acc1[2 * hs + 1] << 8) + (uint32_t)acc1[2 * hs];
+                        uint32_t t4 = ((uint32_t)acc4[2 * hs + 1] << 8) + (uint32_t)acc4[2 * hs];
+                        asm("" : "+v"(t1), "+v"(t4));   // keeps the three shift-adds (left alone the compiler regroups them into four instructions)
                         t[hs] = (int)((t1 << 2) + t4);
                     }
                     post(q, t[0], t[1]);
@@ -424,7 +428,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                         const float ew = __builtin_amdgcn_exp2f(FULL ? lg[q][hs] : lg[q][hs] - R[hs]);
                         wout[q][hs] = ew * vn[q];
                         l_run[hs] += ew;
-                        w_run[hs] += wout[q][hs];
+                        if constexpr (need_wsum) w_run[hs] += wout[q][hs];
                         wm[hs] = fmaxf(wm[hs], fabsf(wout[q][hs]));
                     }
                 }
@@ -742,7 +746,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             if (h >= group) continue;
             const float l_tot = sh.fin_l[h], w_tot = sh.fin_w[h];
             const uint32_t qh = kvh * group + h;
-            const float bias = (alpha + 0.5f * (beta + gam) + (has_delta ? 0.25f * delta : 0.0f)) * w_tot - sctr[hs];
+            const float bias = need_wsum ? (alpha + 0.5f * (beta + gam) + 0.25f * delta) * w_tot - sctr[hs] : -sctr[hs];
             if (nsplit == 1) {
                 float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 4 * pcol;
                 const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
@@ -771,7 +775,9 @@ __global__ __launch_bounds__(HD / 2, OCC) void attention_tq_mfma_kernel(AttnPoin
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
-    if (fabsf(d_raw) > 1e-5f * lmax) attention_body<3, HD, false, PS>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
+    // The constant term left over by the centred planes is mean(L) times the sum of the weights.
+    const float l_mean = 0.25f * ((L0 + L3) + (L1 + L2));
+    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, HD, false, PS>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
     else if (p.num_kv_heads == 1) attention_body<2, HD, true, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
     else attention_body<2, HD, false, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
