@@ -197,7 +197,7 @@ def lanes_for_one_gib(T, hd, nkv=1, bits=2):
     return -(-n // 32) * 32          # a multiple of 32, so that the workgroups of a launch fill whole CUs
 
 
-def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=None, hd=256):
+def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=None, hd=256, keep_state=False):
     """`lanes` independent sequences of T cached positions in one batched launch (default: as many as make the caches
     exceed 1 GiB, so that the figure is an HBM figure), and single decode tokens rotating over those sequences."""
     nq, nkv, bits = 8, 1, 2
@@ -233,7 +233,15 @@ def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=None, hd=256):
         it[0] += 1
 
     _, ev_s = time_steps(pkg, ctx, step_single, max(steps, 20), warmup)
-    return {"context": T, "bytes_per_position": per_pos, "cache_bytes": lanes * T * per_pos,
+    state = None
+    if keep_state:   # lane 0's cache and query, for the CPU leg
+        state = {"q": q[0].astype(np.float32), "k_codes": pool[0].view(0, T * nkv * cb).as_array(np.uint8, T * nkv * cb).copy(),
+                 "k_norms": pool[1].view(0, T * nkv * 2).as_array(np.uint16, T * nkv).copy(),
+                 "v_codes": pool[2].view(0, T * nkv * cb).as_array(np.uint8, T * nkv * cb).copy(),
+                 "v_norms": pool[3].view(0, T * nkv * 2).as_array(np.uint16, T * nkv).copy(),
+                 "levels": levels.as_array(np.float32, 1 << bits).copy(), "signs": signs.as_array(np.float32, hd).copy(),
+                 "hd": hd, "nq": nq, "nkv": nkv, "bits": bits, "T": T}
+    return {"_state": state, "context": T, "bytes_per_position": per_pos, "cache_bytes": lanes * T * per_pos,
             "batched_lanes": lanes, "batched_us_per_launch": ev_b * 1e3,
             "batched_tokens_per_s": lanes / (ev_b * 1e-3), "batched_gbs": lanes * T * per_pos / ev_b * 1e-6,
             "single_us_per_token": ev_s * 1e3, "single_tokens_per_s": 1.0 / (ev_s * 1e-3),
@@ -702,6 +710,60 @@ def cpu_baseline(pkg, raw, x, rows, cols, target_s=12.0):
                       f"single thread: {alg / single * 1e-9:.3f} GB/s"}, y
 
 
+def cpu_baseline_q4_0(pkg, target_s=6.0):
+    """The same CPU path on the Q4_0 configuration (N = K = 2048, fp32 x and y)."""
+    from oracle import oracle as orc
+    rows = cols = 2048
+    g = pkg.synth.rng(1, rows)
+    raw = pkg.synth.weights("q4_0", rows, cols, g)
+    x = pkg.synth.activations(1, cols, g)[0]
+    threads = min(orc.max_threads(), os.cpu_count() or 1)
+    alg = matvec_alg_bytes(pkg, "q4_0", rows, cols)
+    t0 = time.perf_counter()
+    orc.matvec_quant_ref("q4_0", raw, x, rows, cols, threads=threads)
+    one = time.perf_counter() - t0
+    reps = int(max(1, min(4000, target_s / max(one, 1e-4))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        orc.matvec_quant_ref("q4_0", raw, x, rows, cols, threads=threads)
+    dt = time.perf_counter() - t0
+    t1 = time.perf_counter()
+    for _ in range(3):
+        orc.matvec_quant_ref("q4_0", raw, x, rows, cols, threads=1)
+    single = (time.perf_counter() - t1) / 3
+    return {"workload": "Q4_0 fused dequant-matvec, M=1, N=2048 x K=2048", "value": alg * reps / dt * 1e-9, "unit": "GB/s",
+            "cores": threads, "kind": "port",
+            "sample": f"{reps} repetitions of one 2048x2048 Q4_0 matvec ({dt:.1f} s, OpenMP over rows); "
+                      f"single thread: {alg / single * 1e-9:.3f} GB/s"}
+
+
+def cpu_baseline_attention(pkg, st, target_s=8.0):
+    """The reference's CPU attention over a TurboQuant cache: TurboQuant::decode of every cached K and V row
+    (local-engine/src/turboquant.rs:280-291), then f32 softmax(q . k) . v per query head (the pattern of
+    local-metal/src/kernels.rs:8497-8528), on one sequence of the benchmark's caches.  Rates are quoted over the same
+    132 bytes per position the GPU figure uses."""
+    from oracle import oracle as orc
+    threads = min(orc.max_threads(), os.cpu_count() or 1)
+    T, hd, nq, nkv, bits = st["T"], st["hd"], st["nq"], st["nkv"], st["bits"]
+    args = (st["q"], st["k_codes"], st["k_norms"], st["v_codes"], st["v_norms"], st["levels"], st["signs"], hd, T, T - 1, nq, nkv, 0, bits, 0)
+    alg = T * nkv * (2 * (hd * bits // 8) + 4)
+    t0 = time.perf_counter()
+    orc.attention_tq_decode_then_attend(*args, threads=threads)
+    one = time.perf_counter() - t0
+    reps = int(max(1, min(200, target_s / max(one, 1e-4))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        orc.attention_tq_decode_then_attend(*args, threads=threads)
+    dt = (time.perf_counter() - t0) / reps
+    t1 = time.perf_counter()
+    orc.attention_tq_decode_then_attend(*args, threads=1)
+    single = time.perf_counter() - t1
+    return {"workload": f"tq2 KV attention, one query token over {T} cached positions, 8 query heads / 1 KV head, head_dim {hd}",
+            "value": 1.0 / dt, "unit": "tokens/s", "gbs": alg / dt * 1e-9, "cores": threads, "kind": "port",
+            "sample": f"{reps} repetitions of one decode token at {T} positions ({dt * reps:.1f} s; decode of every K and V row, then "
+                      f"f32 softmax . V; OpenMP over positions); single thread: {1.0 / single:.2f} tokens/s, {alg / single * 1e-9:.4f} GB/s"}
+
+
 def main():
     global SETTLE_MS
     ap = argparse.ArgumentParser()
@@ -757,6 +819,10 @@ def main():
 
     legs = set() if args.quick else set(args.legs.split(","))
     del ws, ys
+    cpu_others = []      # CPU baselines of the other measured configurations, reported inside `cpu_baseline`
+    if "matvec" in legs and not args.no_cpu:
+        cpu_others.append(cpu_baseline_q4_0(pkg))
+        log(f"[bench] CPU Q4_0 baseline: {cpu_others[-1]['value']:.2f} GB/s on {cpu_others[-1]['cores']} threads")
     if "matvec" in legs:
         for fmt, r, c in (("q4_0", 2048, 2048), ("tq2_0", 2048, 8192)):
             res = bench_matvec_grouped(pkg, ctx, K, fmt, r, c, args.steps, args.warmup)
@@ -770,9 +836,13 @@ def main():
             extra[f"matvec_{fmt}_{r}x{c}_single_launch"] = res
             log(f"[bench] {fmt} {r}x{c} single launch: {res['us_per_launch']:.1f} us, {res['gbs']:.0f} GB/s")
     if "attention" in legs:
-        att = bench_attention(pkg, ctx, K, args.steps, args.warmup)
+        att = bench_attention(pkg, ctx, K, args.steps, args.warmup, keep_state=not args.no_cpu)
+        att_state = att.pop("_state")
         att["batched_frac_of_hbm_peak"] = att["batched_gbs"] / HBM_PEAK_GBS
         extra["tq2_attention_32k"] = att
+        if att_state is not None:
+            cpu_others.append(cpu_baseline_attention(pkg, att_state))
+            log(f"[bench] CPU attention baseline: {cpu_others[-1]['value']:.2f} tokens/s, {cpu_others[-1]['gbs']:.3f} GB/s on {cpu_others[-1]['cores']} threads")
         log(f"[bench] tq2 attention 32k: batched {att['batched_tokens_per_s']:.0f} tok/s ({att['batched_gbs']:.0f} GB/s), "
             f"single {att['single_us_per_token']:.1f} us/token")
     if "sweep" in legs:
@@ -807,6 +877,28 @@ def main():
         log("[bench] model decode:", extra["model_decode_e2b_geometry"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6
+    # The other north-star kernels of this run, in the blocks a reader of the line keeps: their rooflines beside the
+    # headline kernel's, and the second half of the metric (attention tokens/s at 32k) in `config`.
+    roof_others = []
+    for key, kernel in (("matvec_q4_0_2048x2048_grouped", "matvec_quant_kernel<Q4_0, staged form> (Q4_0 M=1, N=K=2048)"),
+                        ("matvec_tq2_0_2048x8192_grouped", "matvec_tq2_mfma_kernel, long-row form (TQ2_0 M=1, N=2048 x K=8192)")):
+        if key in extra:
+            r = extra[key]
+            roof_others.append({"kernel": kernel, "bound": "hbm", "achieved": r["gbs_events"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": r["gbs_events"] / HBM_PEAK_GBS, "launch_ms": r["ms_per_launch_events"], "replicas": r["replicas"]})
+    attention_cfg = None
+    if "tq2_attention_32k" in extra:
+        a = extra["tq2_attention_32k"]
+        roof_others.append({"kernel": "attention_tq_mfma_kernel + merge (tq2 KV flash decoding, 8 q heads / 1 KV head, head_dim 256, 32768 positions)",
+                            "bound": "hbm", "achieved": a["batched_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": a["batched_gbs"] / HBM_PEAK_GBS, "launch_ms": a["batched_us_per_launch"] * 1e-3,
+                            "alg_bytes_per_launch": a["cache_bytes"]})
+        attention_cfg = {"context": a["context"], "sequences_per_launch": a["batched_lanes"], "tokens_per_s": a["batched_tokens_per_s"],
+                         "gbs": a["batched_gbs"], "frac_of_hbm_peak": a["batched_gbs"] / HBM_PEAK_GBS,
+                         "us_per_launch": a["batched_us_per_launch"], "single_sequence_us_per_token": a["single_us_per_token"],
+                         "single_sequence_tokens_per_s": a["single_tokens_per_s"]}
+    if cpu is not None and cpu_others:
+        cpu["others"] = cpu_others
     line = {
         "metric": "Q4_0/TQ2_0 matvec HBM GB/s (% of peak) at M=1; tq2 KV attn tokens/s @32k",
         "value": head["gbs_wall"],
@@ -823,11 +915,13 @@ def main():
         "config": {"workload": "TQ2_0 fused dequant-matvec, M=1, N=8192 x K=2048 (MLP gate/up), fp32 x and y",
                    "replicas_per_step": head["replicas"], "launches_per_step": 1,
                    "bytes_per_step": head["alg_bytes_per_launch"], "pct_of_hbm_peak": 100.0 * head["gbs_wall"] / HBM_PEAK_GBS,
-                   "settle_ms_before_warmup": SETTLE_MS},
+                   "settle_ms_before_warmup": SETTLE_MS,
+                   "x_shared_by_replicas": True,   # the replicas read one 8 KB activation vector (0.2 % of the bytes); weights and outputs are distinct
+                   "tq2_attention_32k": attention_cfg},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "matvec_tq2_mfma_kernel<float, float, false, 256, true>", "alg_bytes_per_launch": head["alg_bytes_per_launch"],
-                     "launch_ms": head["ms_per_launch_events"]},
+                     "launch_ms": head["ms_per_launch_events"], "others": roof_others},
         "cpu_baseline": cpu,
         "extra": extra,
     }

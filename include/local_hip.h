@@ -103,7 +103,14 @@ LH_API void lh_batch_free(lh_batch* batch);
 LH_API uint32_t lh_batch_dispatch_count(const lh_batch* batch);
 LH_API int lh_batch_blit_copy(lh_batch* batch, const lh_buffer* src, size_t src_offset, lh_buffer* dst,
                               size_t dst_offset, size_t len);
+/* Waits for the stream.  Besides HIP errors this reports, as LH_ERR_COMMAND_BUFFER, a kernel of the batch that gave
+ * up a bounded wait of its own (the split form of the TQ2_0 matvec polls an LDS word for the previous use of a ring
+ * slot; were that ever to run out, the wave goes on so that the kernel still ends, stores a code in a word of pinned
+ * host memory, and the outputs of the batch are not valid).  PendingCommandBuffer::wait, batch.rs:136-144. */
 LH_API int lh_batch_commit_and_wait(lh_batch* batch);
+/* Test hook, no counterpart in the reference: the number of polls the wait above is good for (default 2^20).  A
+ * test sets it to 0 to see the error path taken without any kernel hanging, and restores it afterwards. */
+LH_API void lh_debug_set_tq2_split_spin_limit(uint32_t polls);
 LH_API int lh_batch_submit_and_renew(lh_batch* batch);
 LH_API int lh_batch_commit_and_renew(lh_batch* batch);
 
@@ -131,7 +138,13 @@ LH_API void lh_graph_free(lh_graph* graph);
  * Numerics: x is taken to 16-bit fixed point per weight block (a block whose
  * maximum stands out from its other elements gets a second 16-bit level), the
  * integer products are exact, and the block sums are combined in f32: within
- * 1e-3 of the reference's f32 dot relative to the output's scale.  A NaN or an
+ * 1e-3 of the reference's f32 dot relative to the output's scale.  In the
+ * reference tests' own form, |g - w| <= tol * max(|w|, 1), that holds as well
+ * except for TQ2_0 rows of 8192 columns and more against a vector in which
+ * EVERY block has one element just under 32 x the mean of its other elements
+ * (the second level starts at 32): there the outputs are small (|y| ~ 10),
+ * that form judges them absolutely, and the error reaches 1.2e-3 (1.4e-4 of
+ * the output's scale).  A NaN or an
  * infinity in x makes every output row NaN (the f32 dot would give NaN, or an
  * infinity where no opposite one cancels it); it is never clamped to a finite
  * value. */
@@ -208,7 +221,9 @@ LH_API int lh_multivec_nt_tq2_0_into(lh_batch* batch, const lh_buffer* input, co
  * prefill configurations use f32 and bf16 activations).  Up to 16 rows of f32
  * activations run as rows of the matvec and stay f32; up to 32 rows (TQ2_0
  * from 10 rows on) enter the matrix cores as two f16 rows each, the rounded
- * value and the remainder, and keep about 22 bits.  Larger products multiply
+ * value and the remainder, and keep about 22 bits (magnitudes up to 131008
+ * stay finite: the first part of a value beyond the f16 range is held at
+ * 65504; beyond that the outputs are non-finite).  Larger products multiply
  * in f16 like the reference's kernels, whose activations are f16
  * (kernels.rs:6459-6563): bf16 activations convert exactly (down to the f16
  * subnormals), f32 activations are rounded to f16 first, which costs up to

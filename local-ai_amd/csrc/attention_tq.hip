@@ -20,6 +20,7 @@
 //    workspace and a second small kernel does the log-sum-exp merge; with one
 //    split the workgroup writes the final result itself.
 #include "attention_tq.hpp"
+#include <atomic>
 #include <algorithm>
 #include <cmath>
 
@@ -39,7 +40,7 @@ constexpr size_t kStaticScratchFloats = (size_t)2 << 20;          // 8 MiB
 constexpr uint32_t kStaticMinSplits = 256;                        // split records that must fit for a call to be accepted
 static __device__ __align__(256) float scratch[kStaticScratchFloats];
 constexpr int kMaxDevices = 64;
-static float* g_scratch_ptr[kMaxDevices];                         // per device, set by lh_attention_static_scratch_init
+static std::atomic<float*> g_scratch_ptr[kMaxDevices];            // per device, set by lh_attention_static_scratch_init (contexts may open on several threads)
 
 // The lane's bit window of one code record: `dpl` codes starting at bit lane*dpl*bits.
 __device__ __forceinline__ uint32_t load_window(const uint8_t* rec, uint32_t byte0, uint32_t nbytes) {
@@ -494,11 +495,13 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
 // Called by lh_context_create with `device` current: resolves this device's copy of the static scratch array once.
 int lh_attention_static_scratch_init(int device) {
     if (device < 0 || device >= kMaxDevices) return LH_OK;            // such a device simply has no static entry
-    if (g_scratch_ptr[device]) return LH_OK;
+    if (g_scratch_ptr[device].load(std::memory_order_acquire)) return LH_OK;
     float* ptr = nullptr;
     hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !ptr) return lh_fail(LH_ERR_LIBRARY_CREATION, "static attention scratch on device %d: %s", device, hipGetErrorString(e));
-    g_scratch_ptr[device] = ptr;
+    // Only the entry that allocates nothing needs the array: when its address cannot be resolved the pointer stays null, that
+    // entry reports "no static scratch", and contexts open all the same.
+    if (e != hipSuccess || !ptr) { (void)hipGetLastError(); return LH_OK; }
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return LH_OK;
 }
 
@@ -525,7 +528,7 @@ int lh_flash_attention_tq_static_into(lh_batch* batch, const lh_buffer* rq, cons
     const char* op = "flash_attention_tq_static";
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     const int dev = batch->ctx->device;
-    float* ws = (dev >= 0 && dev < kMaxDevices) ? g_scratch_ptr[dev] : nullptr;
+    float* ws = (dev >= 0 && dev < kMaxDevices) ? g_scratch_ptr[dev].load(std::memory_order_acquire) : nullptr;
     if (!ws) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: no static scratch on device %d (the context was not created by this library)", op, dev);
     // kStaticMinSplits records of every query head must fit: beyond that the call is refused rather than run with few splits
     const uint64_t need = (uint64_t)num_q_heads * partial_record_floats(head_dim) * kStaticMinSplits;

@@ -33,7 +33,15 @@ struct lh_context {
     hipEvent_t desc_event[kDescSlots];
     bool desc_used[kDescSlots];
     unsigned desc_next;
+    // One word of pinned host memory that kernels can reach: a kernel that had to give up a bounded wait stores a code
+    // here, and the next wait on the stream (lh_batch_commit_and_wait, lh_context_synchronize) reports it.
+    uint32_t* fault_host;
+    uint32_t* fault_dev;   // the same word as the device addresses it
 };
+// Kernel-reported fault codes (lh_context::fault_host).
+enum : uint32_t { LH_FAULT_TQ2_SPLIT_WAIT = 1 };
+// Reads and clears the context's fault word after a completed wait; LH_OK when no kernel reported anything.
+int lh_check_fault_word(lh_context* ctx);
 
 struct lh_buffer {
     lh_context* ctx;

@@ -777,7 +777,13 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
                 struct { uint32_t v[4]; } hi, lo;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const uint16_t h0 = lh_f2h(x[2 * e]), h1 = lh_f2h(x[2 * e + 1]);
+                    // A finite value beyond the f16 range keeps a finite first part (the remainder then carries the rest, up to
+                    // 131008 in all); left alone it would be inf with the remainder -inf, and the two products would add to NaN.
+                    auto first_part = [](float v) {
+                        const float a = __builtin_fabsf(v);
+                        return lh_f2h((a > 65504.0f && a < INFINITY) ? __builtin_copysignf(65504.0f, v) : v);
+                    };
+                    const uint16_t h0 = first_part(x[2 * e]), h1 = first_part(x[2 * e + 1]);
                     hi.v[e] = (uint32_t)h0 | ((uint32_t)h1 << 16);
                     lo.v[e] = pack_h2(x[2 * e] - lh_h2f(h0), x[2 * e + 1] - lh_h2f(h1));
                 }

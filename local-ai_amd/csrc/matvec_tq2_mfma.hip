@@ -27,6 +27,7 @@
 #include "common.hpp"
 #include "xquant.hpp"
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 
 namespace {
@@ -74,6 +75,9 @@ struct Tq2Base {
     Tq2Problem second = {nullptr, nullptr, nullptr};
     uint32_t pair = 0;
     XPrologue pro = {kXProNone, nullptr, 0.0f};   // applied to every problem's vector while it is staged
+    // Split form: how often a wave polls for the previous use of its ring slot before it gives up, and where it says so.
+    uint32_t spin_limit = 1u << 20;
+    uint32_t* fault = nullptr;
 };
 
 __device__ __forceinline__ u32x4_t ld16_align2_cached(gptr_t p) {
@@ -364,8 +368,14 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
                 auto lds_order = [] { __builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory"); };   // lgkmcnt(0) only
                 if (gen) {   // the slot's previous use must have been summed (bounded wait: never expected to run out)
                     uint32_t spins = 0;
-                    while (__hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != gen && spins++ < (1u << 20))
+                    bool seen;
+                    while (!(seen = __hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == gen) &&
+                           spins++ < single.spin_limit)
                         __builtin_amdgcn_s_sleep(2);
+                    // Out of patience: the wave goes on (every wave must reach the end of the kernel), the rows of this tile
+                    // are not to be trusted, and the host learns of it at its next wait on the stream.
+                    if (!seen && lane == 0 && single.fault)
+                        __hip_atomic_store(single.fault, (uint32_t)LH_FAULT_TQ2_SPLIT_WAIT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     lds_order();
                 }
                 if (c == 0) {
@@ -398,6 +408,9 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
 }
 
 }  // namespace
+
+static std::atomic<uint32_t> g_tq2_spin_limit{1u << 20};
+extern "C" void lh_debug_set_tq2_split_spin_limit(uint32_t polls) { g_tq2_spin_limit.store(polls, std::memory_order_relaxed); }
 
 // Entry used by matvec_quant.hip's dispatcher. Arrays are host arrays of device pointers.
 int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const* matrices, const void* const* vectors,
@@ -468,6 +481,8 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     single.mstride = mstride;
     single.split_waves = wide_split;
     single.pro = pro;
+    single.spin_limit = g_tq2_spin_limit.load(std::memory_order_relaxed);
+    single.fault = ctx->fault_dev;
     Tq2Problem* dev = nullptr;
     if (count == 2 && !strided) {
         single.second = Tq2Problem{(const uint8_t*)matrices[1], vectors[1], outputs[1]};

@@ -1,0 +1,132 @@
+// Issue model of one gfx950 SIMD: do vector-ALU and matrix-core instructions overlap?
+//
+// The attention, TQ2_0 matvec and prefill kernels of this library all interleave v_mfma_i32_16x16x64_i8 (or its f16
+// sibling) with a larger number of ordinary vector instructions, from one or several waves per SIMD.  Whether their
+// speed is "the longer of the two streams" or "the sum of both" decides which optimisations are worth trying.  This
+// probe times fixed mixes at 1 .. 4 waves per SIMD, with the two kinds of instruction in one wave (finely or coarsely
+// interleaved) or on different waves of the same SIMD, and prints nanoseconds per iteration and the SIMD cycles per
+// instruction that follow from the clock the device reports.  One workgroup per CU, so waves per SIMD = threads / 256.
+//
+//   hipcc -O3 --offload-arch=gfx950 -o issue_model_probe issue_model.hip && ./issue_model_probe
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp };
+
+// One iteration: 160 vector instructions and / or 16 MFMAs per wave (kSplitWaves: even waves 160 vector
+// instructions, odd waves 16 MFMAs).
+template <int MIX>
+__global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out) {
+    unsigned x[8];
+    float f[8];
+    v4i acc[4];
+    for (int i = 0; i < 8; i++) { x[i] = threadIdx.x * 2654435761u + i; f[i] = 1.0f + threadIdx.x * 1e-3f + i; }
+    for (int i = 0; i < 4; i++) acc[i] = (v4i){0, 0, 0, 0};
+    const v4i a = (v4i){(int)threadIdx.x, 1, 2, 3}, b = (v4i){4, 5, (int)threadIdx.x, 7};
+    const bool odd_wave = (threadIdx.x >> 6) & 1;
+    for (int it = 0; it < iters; it++) {
+        if constexpr (MIX == kValu || MIX == kCoarse) {
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[i] = (x[i] & 0x7f7f7f7fu) + 0x01010101u * (i + 1);   // v_and_b32 + v_add_u32
+        }
+        if constexpr (MIX == kMfma || MIX == kCoarse) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[r & 3], 0, 0, 0);
+        }
+        if constexpr (MIX == kFine) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+#pragma unroll
+                for (int i = 0; i < 5; i++) x[i] = (x[i] & 0x7f7f7f7fu) + 0x01010101u * (i + 1);
+                acc[r & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[r & 3], 0, 0, 0);
+            }
+        }
+        if constexpr (MIX == kSplitWaves) {
+            if (odd_wave) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[r & 3], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 20; r++)
+#pragma unroll
+                    for (int i = 0; i < 8; i++) x[i] = (x[i] & 0x7f7f7f7fu) + 0x01010101u * (i + 1);
+            }
+        }
+        if constexpr (MIX == kPerm) {
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[i] = __builtin_amdgcn_perm(x[i], x[(i + 1) & 7], 0x05010400u);
+        }
+        if constexpr (MIX == kFma) {
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) f[i] = __builtin_fmaf(f[i], 1.0001f, 0.5f);
+        }
+        if constexpr (MIX == kExp) {
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) f[i] = __builtin_amdgcn_exp2f(f[i]);
+        }
+    }
+    unsigned s = 0;
+    for (int i = 0; i < 8; i++) s ^= x[i] ^ __float_as_uint(f[i]);
+    for (int i = 0; i < 4; i++) s ^= (unsigned)(acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3]);
+    if (s == 0x12345u) out[0] = (int)s;   // keeps the work alive
+}
+
+static double g_ghz = 0.0;
+
+template <int MIX>
+static void run(const char* name, int valu_per_wave, int mfma_per_wave, int* d) {
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { fprintf(stderr, "hipEventCreate failed\n"); exit(1); }
+    const int iters = 4000;
+    printf("%-44s", name);
+    for (int wps = 1; wps <= 4; wps++) {
+        if (MIX == kSplitWaves && (wps & 1)) { printf(" | %-27s", "-"); continue; }
+        float ms = 0;
+        for (int rep = 0; rep < 3; rep++) {   // the last repetition counts (clocks up, code resident)
+            (void)hipEventRecord(e0);
+            hipLaunchKernelGGL(mix_kernel<MIX>, dim3(256), dim3(256 * wps), 0, 0, iters, d);
+            (void)hipEventRecord(e1);
+            if (hipEventSynchronize(e1) != hipSuccess) { fprintf(stderr, "kernel failed\n"); exit(1); }
+            (void)hipEventElapsedTime(&ms, e0, e1);
+        }
+        const double ns = ms * 1e6 / iters;
+        // cycles one SIMD spends per iteration of ALL its waves, against 4 per vector instruction + 16 per MFMA if they add
+        const int waves_v = MIX == kSplitWaves ? wps / 2 : wps, waves_m = MIX == kSplitWaves ? wps / 2 : wps;
+        const double model = 4.0 * valu_per_wave * waves_v + 16.0 * mfma_per_wave * waves_m;
+        printf(" | %7.1f ns %6.0f cyc (%4.2f)", ns, ns * g_ghz, ns * g_ghz / model);
+    }
+    printf("\n");
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+}
+
+int main() {
+    int* d = nullptr;
+    if (hipMalloc(&d, 4) != hipSuccess) { fprintf(stderr, "no device\n"); return 1; }
+    int khz = 0;
+    (void)hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, 0);
+    g_ghz = khz * 1e-6;
+    printf("clock reported by the device: %.2f GHz; columns: 1, 2, 3, 4 waves per SIMD; per column: time per iteration, SIMD cycles at\n"
+           "that clock, and (ratio to the additive model: 4 cycles per vector instruction + 16 per MFMA, summed over the SIMD's waves)\n", g_ghz);
+    run<kValu>("160 v_and/v_add per wave", 160, 0, d);
+    run<kMfma>("16 MFMA per wave", 0, 16, d);
+    run<kFine>("16 x (5 vector + 1 MFMA) per wave", 80, 16, d);
+    run<kCoarse>("160 vector, then 16 MFMA per wave", 160, 16, d);
+    run<kSplitWaves>("even waves 160 vector, odd waves 16 MFMA", 160, 16, d);
+    run<kPerm>("160 v_perm_b32 per wave", 160, 0, d);
+    run<kFma>("160 v_fma_f32 per wave", 160, 0, d);
+    run<kExp>("160 v_exp_f32 per wave", 160, 0, d);
+    (void)hipFree(d);
+    return 0;
+}

@@ -93,6 +93,17 @@ int lh_upload_descriptors(lh_context* ctx, const void* host, size_t bytes, void*
     return LH_OK;
 }
 
+int lh_check_fault_word(lh_context* ctx) {
+    volatile uint32_t* w = ctx->fault_host;
+    const uint32_t code = w ? *w : 0u;
+    if (code == 0) return LH_OK;
+    *w = 0;
+    if (code == LH_FAULT_TQ2_SPLIT_WAIT)
+        return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: a wave gave up waiting for the partial rows of its tile; "
+                                              "the outputs of this batch are not valid");
+    return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: a kernel reported fault code %u", code);
+}
+
 extern "C" {
 
 const char* lh_last_error(void) { return g_last_error; }
@@ -107,6 +118,7 @@ static void ctx_release(lh_context* ctx) {
     (void)hipFree(ctx->workspace);
     for (int i = 0; i < lh_context::kDescSlots; i++) (void)hipEventDestroy(ctx->desc_event[i]);
     (void)hipHostFree(ctx->desc_pinned);
+    (void)hipHostFree(ctx->fault_host);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -151,10 +163,23 @@ int lh_context_create(int device_index, lh_context** out) {
         delete ctx;
         return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: pinned descriptor staging", lh_context::kDescSlots * lh_context::kDescSlotBytes);
     }
+    ctx->fault_host = nullptr;
+    ctx->fault_dev = nullptr;
+    if (hipHostMalloc((void**)&ctx->fault_host, 64, hipHostMallocDefault) != hipSuccess ||
+        hipHostGetDevicePointer((void**)&ctx->fault_dev, ctx->fault_host, 0) != hipSuccess) {
+        if (ctx->fault_host) (void)hipHostFree(ctx->fault_host);
+        (void)hipHostFree(ctx->desc_pinned);
+        (void)hipFree(ctx->workspace);
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: pinned fault word", (size_t)64);
+    }
+    *ctx->fault_host = 0;
     for (int i = 0; i < lh_context::kDescSlots; i++) {
         ctx->desc_used[i] = false;
         if (hipEventCreateWithFlags(&ctx->desc_event[i], hipEventDisableTiming) != hipSuccess) {
             for (int j = 0; j < i; j++) (void)hipEventDestroy(ctx->desc_event[j]);
+            (void)hipHostFree(ctx->fault_host);
             (void)hipHostFree(ctx->desc_pinned);
             (void)hipFree(ctx->workspace);
             (void)hipStreamDestroy(ctx->stream);
@@ -186,7 +211,7 @@ int lh_context_synchronize(lh_context* ctx) {
     if (!ctx) return lh_fail(LH_ERR_INVALID_ARGUMENT, "synchronize: context is null");
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
-    return LH_OK;
+    return lh_check_fault_word(ctx);
 }
 
 // ---- events -----------------------------------------------------------------
@@ -381,7 +406,7 @@ int lh_batch_commit_and_wait(lh_batch* batch) {
     hipError_t e = hipStreamSynchronize(batch->ctx->stream);
     batch->dispatch_count = 0;
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: %s", hipGetErrorString(e));
-    return LH_OK;
+    return lh_check_fault_word(batch->ctx);   // a kernel that gave up a bounded wait says so here (batch.rs:136-144: GPU errors surface at the wait)
 }
 int lh_batch_submit_and_renew(lh_batch* batch) {
     // Work is already on the stream as it is encoded; nothing to flush.

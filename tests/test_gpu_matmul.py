@@ -183,6 +183,38 @@ def test_decode_batch_f32_activations(pkg, gpu, oracle, fmt):
                     assert e <= tol, (fmt, m, k, n, wide, ct, e)
 
 
+@pytest.mark.parametrize("fmt", ["tq2_0", "q4_0"])
+def test_small_batch_f32_activations_beyond_f16_range(pkg, gpu, oracle, fmt):
+    """f32 activations larger than the largest f16 (65504) in a small batch: up to 16 rows (TQ2_0: 9) run as matvec rows
+    in block fixed point, more rows enter the matrix cores as an f16 part plus an f16 remainder.  The first part of
+    such a value is held at 65504 so that the pair stays finite up to 131008; the result must not change from finite
+    to NaN with the number of rows.  Against the oracle's f32 product, relative to the output's scale."""
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    k, n = 2048, 1024
+    raw = payload(fmt, n, k, 0xB16)
+    deq = (oracle.dequant_q4_0 if fmt == "q4_0" else oracle.dequant_tq2_0)(raw).view(np.float16).astype(np.float32).reshape(n, k)
+    w = pkg.QuantWeight.from_bytes(ctx, raw, ty, n, k)
+    for m in (4, 12, 20, 32):
+        g = pkg.synth.rng(10, m)
+        a = g.standard_normal((m, k), dtype=np.float32)
+        for r in range(m):
+            for c in g.integers(0, k, 3):
+                a[r, c] = np.float32(g.choice([7.0e4, -9.5e4, 1.2e5, -1.3e5]))
+        print(f"case {fmt} m={m}", flush=True)
+        want = oracle.matmul_nt_f32(a, deq)
+        ab = pkg.Buffer.from_slice(ctx, a)
+        cb = pkg.Buffer.empty(ctx, m * n * 4)
+        batch = pkg.CommandBatch(ctx)
+        w.matmul_nt_typed_into(batch, K, ab, pkg.F32, cb, pkg.F32, m)
+        batch.commit_and_wait()
+        got = cb.as_array(np.float32, m * n).reshape(m, n)
+        assert np.isfinite(got).all(), (fmt, m, int((~np.isfinite(got)).sum()))
+        e = refgen.scaled_error(got, want)
+        print(f"{fmt} m={m}: err / max|w| {e:.2e}")
+        assert e <= 1e-3, (fmt, m, e)
+
+
 @pytest.mark.parametrize("seed", [1, 2])
 def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
     """Fifty random products per seed through the typed entries: either format, 1 .. 700 activation rows (every routing

@@ -45,14 +45,11 @@ def test_matvec_reference_payloads(pkg, gpu, oracle, fmt, rows, cols):
 
 
 @pytest.mark.parametrize("fmt,rows,cols", [("q4_0", 2048, 2048), ("tq2_0", 8192, 2048), ("tq2_0", 2048, 8192),
-                                           ("q4_0", 256, 2048), ("q4_0", 262144, 1536),
-                                           ("q4_0", 4096, 16384), ("q4_0", 4000, 14400)])
+                                           ("q4_0", 256, 2048), ("q4_0", 262144, 1536)])
 def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
-    """The measured configurations (the fifth one is the logits product of the reference's decode tail,
+    """The measured configurations (the last one is the logits product of the reference's decode tail,
     local-engine/src/pipeline.rs:914-953, at its full vocabulary): fp32 x, fp32 y, against the reference CPU path
-    (block dequant to f16 then a sequential f32 dot), max normalised error <= 1e-3.  The last two have rows so long
-    that the activation area alone nearly fills the kernel's LDS limit (many rows per workgroup, so that the staged
-    form would be chosen if it fitted): they must run, on direct loads."""
+    (block dequant to f16 then a sequential f32 dot), max normalised error <= 1e-3."""
     print(f"case {fmt} {rows}x{cols}", flush=True)
     g = pkg.synth.rng(1 if fmt == "q4_0" else 2, rows)
     raw = pkg.synth.weights(fmt, rows, cols, g)
@@ -66,6 +63,30 @@ def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
     e64 = float(np.max(np.abs(got - y64) / np.maximum(np.abs(y64), 1.0)))
     print(f"{fmt} {rows}x{cols}: err vs CPU path {err:.2e}, vs f64 {e64:.2e}")
     assert e64 <= 3e-4   # 16-bit block-fixed-point activations; 24-bit with LOCAL_HIP_X_LIMBS=3
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 16384), (4000, 14400)])
+def test_matvec_q4_0_longest_rows_many_rows(pkg, gpu, oracle, rows, cols):
+    """Q4_0 rows so long that the activation area alone nearly fills the kernel's LDS limit, with enough rows per
+    workgroup that the staged form would be chosen if its images still fitted: the launch must go through (on direct
+    loads) and be right.  Over 16384 columns the reference CPU path's own roundings (weights to f16, a sequential f32
+    sum) put it up to about 1e-3 from the exactly accumulated product in the max(|w|, 1) form, so the gate against it is
+    widened by that distance, and the kernel is held to the exact product on its own."""
+    print(f"case q4_0 {rows}x{cols}", flush=True)
+    g = pkg.synth.rng(1, rows + cols)
+    raw = pkg.synth.weights("q4_0", rows, cols, g)
+    x = pkg.synth.activations(1, cols, g)[0]
+    want = oracle.matvec_quant_ref("q4_0", raw, x, rows, cols, threads=8)
+    exact = oracle.matvec_f64(oracle.expand_q4_0_f32(raw, rows, cols), x)
+    got = run_matvec(pkg, gpu, "q4_0", raw, x, rows, cols, pkg.F32, pkg.F32)
+    norm = np.maximum(np.abs(want), 1.0)
+    floor = float(np.max(np.abs(exact - want) / norm))
+    e_ref = float(np.max(np.abs(got - want) / norm))
+    e_own = float(np.max(np.abs(got - exact) / norm))
+    print(f"q4_0 {rows}x{cols}: vs CPU path {e_ref:.2e} (CPU path vs exact product {floor:.2e}), kernel vs exact product {e_own:.2e}")
+    assert e_own <= 3e-4
+    assert e_ref <= 1e-3 + floor
+    assert refgen.scaled_error(got, want) <= 1e-3
 
 
 def test_matvec_rejects_misaligned_cols(pkg, gpu):
@@ -379,3 +400,74 @@ def test_grouped_long_rows_many_tiles(pkg, gpu, oracle, rows, cols, count, share
     bits = np.uint16 if half else np.uint32
     for i in range(distinct, count):       # identical weights and vector: identical bits, wherever the problem ran
         assert np.array_equal(got[i].view(bits), got[i % distinct].view(bits)), f"problem {i}"
+
+
+@pytest.mark.parametrize("rows,cols", [(8192, 2048), (2048, 8192), (2048, 2048)])
+def test_matvec_tq2_blocks_at_the_second_level_limit(pkg, gpu, oracle, rows, cols):
+    """The worst vector for the one-level activation quantiser: EVERY 256-column block holds one element of just
+    under 32 x the mean magnitude of its other elements, so no block gets the residual level and each carries the
+    coarsest step the kernel ever uses.  Pins the limit (32): against the reference CPU path the error stays under
+    3e-4 of the output's own scale on every shape (1.4e-4 measured); in the reference's max(|w|, 1) form, which judges
+    the small outputs of such a vector absolutely, under 1e-3 for K = 2048 and under 1.5e-3 for K = 8192 (1.2e-3
+    measured: the one documented case outside 1e-3 in that form, stated in include/local_hip.h).  A larger limit fails
+    the first bound, which is the point of the test."""
+    g = pkg.synth.rng(46, rows + cols)
+    raw = pkg.synth.weights("tq2_0", rows, cols, g)
+    x = g.standard_normal(cols, dtype=np.float32)
+    xb = x.reshape(-1, 256)
+    for b in range(xb.shape[0]):
+        j = int(g.integers(0, 256))
+        others = (np.abs(xb[b]).sum() - abs(xb[b, j])) / 255.0
+        xb[b, j] = np.float32(31.0 * others) * (1.0 if g.random() < 0.5 else -1.0)
+    x = xb.reshape(-1)
+    want = oracle.matvec_quant_ref("tq2_0", raw, x, rows, cols, threads=8)
+    got = run_matvec(pkg, gpu, "tq2_0", raw, x, rows, cols, pkg.F32, pkg.F32)
+    e_scaled = refgen.scaled_error(got, want)
+    e_norm = float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1.0)))
+    print(f"tq2_0 {rows}x{cols}, every block at the limit: err/max|w| {e_scaled:.2e}, err/max(|w|,1) {e_norm:.2e}, max|w| {np.abs(want).max():.1f}")
+    assert e_scaled <= 3e-4
+    assert e_norm <= (1.5e-3 if cols > 2048 else 1e-3)
+
+
+def test_matvec_tq2_split_wait_gives_up_loudly(pkg, gpu, oracle):
+    """The split form's bounded wait (a wave polls an LDS word until the previous use of its ring slot has been summed).
+    With the poll budget forced to zero from the host a wave that arrives early gives up at once: every wave still runs
+    to the end of the kernel, and the wait on the batch must report it as a command-buffer error instead of returning
+    rows that may be wrong.  With the budget restored the same launch is clean and correct."""
+    import ctypes as C
+    ctx, K = gpu
+    rows, cols, count = 2048, 8192, 52
+    g = pkg.synth.rng(47, 1)
+    raw = pkg.synth.weights("tq2_0", rows, cols, g)
+    wb = raw.size
+    big = pkg.Buffer.empty(ctx, wb * count)
+    for i in range(count):
+        big.copy_from_bytes(raw, i * wb)
+    ws = [big.view(i * wb, wb) for i in range(count)]
+    x = pkg.synth.activations(1, cols, g)[0]
+    xb = pkg.Buffer.from_slice(ctx, x)
+    yall = pkg.Buffer.empty(ctx, count * rows * 4)
+    ys = [yall.view(i * rows * 4, rows * 4) for i in range(count)]
+    batch = pkg.CommandBatch(ctx)
+    setter = pkg.lib().lh_debug_set_tq2_split_spin_limit
+    setter.restype = None
+    seen = False
+    try:
+        setter(C.c_uint32(0))
+        for _ in range(5):
+            K.matvec_quant_grouped_into(batch, pkg.TQ2_0, ws, [xb] * count, pkg.F32, ys, pkg.F32, rows, cols)
+            try:
+                batch.commit_and_wait()
+            except pkg.CommandBuffer as e:
+                assert "gave up waiting" in str(e)
+                seen = True
+                break
+    finally:
+        setter(C.c_uint32(1 << 20))
+    assert seen, "no wave of 5 launches ever had to wait: the forced give-up path was not reached"
+    K.matvec_quant_grouped_into(batch, pkg.TQ2_0, ws, [xb] * count, pkg.F32, ys, pkg.F32, rows, cols)
+    batch.commit_and_wait()          # clean again: the fault word was cleared when it was reported
+    want = oracle.matvec_quant_ref("tq2_0", raw, x, rows, cols, threads=8)
+    got = yall.as_array(np.float32, count * rows).reshape(count, rows)
+    for i in (0, count // 2, count - 1):
+        refgen.assert_close(got[i], want, 1e-3, f"problem {i} after the budget was restored")

@@ -1,8 +1,11 @@
 """The attention entry that allocates nothing (lh_flash_attention_tq_static_into: split partials in a static device
 array) against the ordinary entry (lh_flash_attention_tq_into: partials in the context workspace), through the C ABI:
 two calls in a row, the second over a smaller input, so that records left behind by the first call lie in the array
-while the second runs.  Same kernels and the same split count, so the outputs must agree bit for bit; both are also
-held to the f64 code-space oracle at the attention tolerance."""
+while the second runs.  Same kernels and -- for these shapes -- the same split count, so the outputs must agree bit for
+bit: the split count is chosen from the work and only lowered when the records would not fit, and the static array
+(2 Mi floats) holds the 256 splits a single query gets at most here for 8 heads of 512 dims (256 x 8 x 516 floats), as
+the workspace does.  Both are also held to the f64 code-space oracle at the attention tolerance.  A last test reads the
+device's free memory around a series of calls: the entry must not allocate."""
 import numpy as np
 import pytest
 
@@ -44,3 +47,30 @@ def test_static_entry_rejects_oversized_shapes(pkg, gpu):
     with pytest.raises(pkg.InvalidArgument, match=r"flash_attention_tq_static: num_q_heads 32 x \(head_dim 512 \+ 4\) exceeds 8192"):
         K.flash_attention_tq_static_into(batch, b, b, b, b, b, b, b, 512, 16, 15, 32, 1, 0, 2, 0)
     assert batch.dispatch_count() == 0
+
+
+def test_static_entry_allocates_nothing(pkg, gpu, oracle):
+    """hipMemGetInfo's free bytes before and after twenty calls of the entry (after one warm-up call, which may load
+    the kernels' code): unchanged."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    ctx, K = gpu
+    hd, nq, nkv, T, bits = 256, 8, 1, 4096, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 21)
+    rq = pkg.synth.rng(6, 21).standard_normal((nq, hd), dtype=np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    out = pkg.Buffer.empty(ctx, nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+
+    def free_bytes():
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    K.flash_attention_tq_static_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    before = free_bytes()
+    for _ in range(20):
+        K.flash_attention_tq_static_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, T - 1, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    assert free_bytes() == before
