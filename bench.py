@@ -248,6 +248,25 @@ def bench_attention(pkg, ctx, K, steps, warmup, T=32768, lanes=None, hd=256, kee
             "single_gbs": T * per_pos / ev_s * 1e-6}
 
 
+def bench_attention_prefill(pkg, ctx, K, steps, warmup, T=32768, rows=256):
+    """The attention of the last `rows`-token chunk of a T-token prompt (the reference's MAX_PREFILL_CHUNK rows, each seeing
+    T - rows + r + 1 cached positions): the tiled prefill entry, head_dim 256, 8 query heads over one KV head."""
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    pool, levels, signs = make_kv_pool(pkg, ctx, K, 1, T, hd, nkv, bits)
+    g = pkg.synth.rng(5, 3)
+    rq = pkg.Buffer.from_slice(ctx, g.standard_normal((rows, nq, hd), dtype=np.float32))
+    out = pkg.Buffer.empty(ctx, rows * nq * hd * 4)
+    batch = pkg.CommandBatch(ctx)
+
+    def step():
+        K.flash_attention_tq_prefill_tiled_into(batch, rq, pool[0], pool[1], pool[2], pool[3], levels, out, hd, T, T - rows, rows, nq,
+                                                nkv, 0, bits, 0)
+
+    _, ev = time_steps(pkg, ctx, step, steps, warmup)
+    macs = rows * nq * hd * 2 * (T - rows / 2)          # multiply-adds of q.k and w.v over the positions each row sees
+    return {"rows": rows, "context": T, "us_per_chunk": ev * 1e3, "useful_tmac_per_s": macs / (ev * 1e-3) * 1e-12}
+
+
 def bench_attention_sweep(pkg, ctx, K, steps, warmup):
     """Context sweep (single decode token, sequences rotating so the cache comes from HBM) and the
     sliding-window layer: window 512 over a 512-slot ring that has wrapped many times."""
@@ -845,6 +864,9 @@ def main():
             log(f"[bench] CPU attention baseline: {cpu_others[-1]['value']:.2f} tokens/s, {cpu_others[-1]['gbs']:.3f} GB/s on {cpu_others[-1]['cores']} threads")
         log(f"[bench] tq2 attention 32k: batched {att['batched_tokens_per_s']:.0f} tok/s ({att['batched_gbs']:.0f} GB/s), "
             f"single {att['single_us_per_token']:.1f} us/token")
+    if "attention" in legs:
+        extra["tq2_attention_prefill_256x32k"] = bench_attention_prefill(pkg, ctx, K, args.steps, args.warmup)
+        log("[bench] tiled prefill attention:", extra["tq2_attention_prefill_256x32k"])
     if "sweep" in legs:
         extra["tq2_attention_sweep"] = bench_attention_sweep(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] attention sweep:", extra["tq2_attention_sweep"])

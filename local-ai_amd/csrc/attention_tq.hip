@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kReduceDims * kReduceSlices) void attention_tq_redu
 // workgroup per 32 dims spends its time on scheduling workgroups (256 sequences x 8 heads x 4 splits: 10.5 us);
 // this form reads the same records with a sixteenth of the workgroups.  The arithmetic is attention_tq_reduce_kernel<2>'s
 // in its order: the factors and their sum with one split per lane, two interleaved fma chains per dim, added.
-constexpr uint32_t kWaveMergeMaxSplits = 8;
+constexpr uint32_t kWaveMergeMaxSplits = 16;
 __global__ __launch_bounds__(256) void attention_tq_reduce_wave_kernel(const float* __restrict__ ws, float* __restrict__ out, uint32_t head_dim,
                                                                        uint32_t num_splits, uint32_t num_qh) {
     const uint32_t lane = threadIdx.x & 63, qh = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -435,7 +435,14 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
                             (const uint8_t*)v_codes->ptr, (const uint16_t*)v_norms->ptr, (const float*)levels->ptr,
                             positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, ws};
-    if (max_span == 0 || !mfma_supported(p, ptrs)) {
+    // Prefill entries with more than one row: eight rows share a pass over the codes when the kernel for that takes the
+    // shape and the level table was uploaded as one that is affine in the code bits (LOCAL_HIP_ATTN_PREFILL=rows keeps
+    // one query row per workgroup, the form the tiled kernel is validated against).
+    static const bool prefill_rows = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return e && e[0] == 'r'; }();
+    if (max_span != 0 && !prefill_rows && levels->tq2_affine_levels && prefill_mfma_supported(p, ptrs)) {
+        const int rl = launch_prefill_mfma(ctx, op, ptrs, p, max_span, ws_avail);
+        if (rl != LH_OK) return rl;
+    } else if (max_span == 0 || !mfma_supported(p, ptrs)) {
         // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.
         const uint64_t per_query_wgs = std::max<uint64_t>(1, (uint64_t)ctx->cu_count * 2 / ((uint64_t)p.num_queries * p.num_kv_heads));
         uint64_t splits = std::min<uint64_t>(per_query_wgs, (max_span + 31) / 32);

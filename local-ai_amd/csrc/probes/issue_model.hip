@@ -14,12 +14,12 @@
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp };
+enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp, kValuSgpr, kAndOnlyLit, kAndOnlySgpr };
 
 // One iteration: 160 vector instructions and / or 16 MFMAs per wave (kSplitWaves: even waves 160 vector
 // instructions, odd waves 16 MFMAs).
 template <int MIX>
-__global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out) {
+__global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned mask, unsigned step) {
     unsigned x[8];
     float f[8];
     v4i acc[4];
@@ -69,6 +69,24 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) f[i] = __builtin_fmaf(f[i], 1.0001f, 0.5f);
         }
+        if constexpr (MIX == kValuSgpr) {   // the same 160 instructions with the mask and the addend in scalar registers (no 32-bit literals)
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[i] = (x[i] & mask) + step;
+        }
+        if constexpr (MIX == kAndOnlyLit) {   // 160 v_and_b32 with a 32-bit literal each (an 8-byte encoding)
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[i] = (x[(i + 1) & 7] & (0x7f7f7f7fu - 0x01010101u * (unsigned)i)) ^ x[i];
+        }
+        if constexpr (MIX == kAndOnlySgpr) {
+#pragma unroll
+            for (int r = 0; r < 20; r++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) x[i] = (x[(i + 1) & 7] & mask) ^ x[i];
+        }
         if constexpr (MIX == kExp) {
 #pragma unroll
             for (int r = 0; r < 20; r++)
@@ -83,6 +101,7 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out) {
 }
 
 static double g_ghz = 0.0;
+static unsigned g_mask = 0x7f7f7f7fu, g_step = 0x01010101u;   // reach the kernels as arguments, i.e. in scalar registers
 
 template <int MIX>
 static void run(const char* name, int valu_per_wave, int mfma_per_wave, int* d) {
@@ -95,7 +114,7 @@ static void run(const char* name, int valu_per_wave, int mfma_per_wave, int* d) 
         float ms = 0;
         for (int rep = 0; rep < 3; rep++) {   // the last repetition counts (clocks up, code resident)
             (void)hipEventRecord(e0);
-            hipLaunchKernelGGL(mix_kernel<MIX>, dim3(256), dim3(256 * wps), 0, 0, iters, d);
+            hipLaunchKernelGGL(mix_kernel<MIX>, dim3(256), dim3(256 * wps), 0, 0, iters, d, g_mask, g_step);
             (void)hipEventRecord(e1);
             if (hipEventSynchronize(e1) != hipSuccess) { fprintf(stderr, "kernel failed\n"); exit(1); }
             (void)hipEventElapsedTime(&ms, e0, e1);
@@ -124,6 +143,9 @@ int main() {
     run<kFine>("16 x (5 vector + 1 MFMA) per wave", 80, 16, d);
     run<kCoarse>("160 vector, then 16 MFMA per wave", 160, 16, d);
     run<kSplitWaves>("even waves 160 vector, odd waves 16 MFMA", 160, 16, d);
+    run<kValuSgpr>("160 v_and/v_add, constants in SGPRs", 160, 0, d);
+    run<kAndOnlyLit>("160 x (v_and literal + v_xor) per wave", 320, 0, d);
+    run<kAndOnlySgpr>("160 x (v_and SGPR + v_xor) per wave", 320, 0, d);
     run<kPerm>("160 v_perm_b32 per wave", 160, 0, d);
     run<kFma>("160 v_fma_f32 per wave", 160, 0, d);
     run<kExp>("160 v_exp_f32 per wave", 160, 0, d);

@@ -281,6 +281,97 @@ def test_prefill_matches_per_row_decode(pkg, gpu, oracle, tiled, hd, nq, nkv, bi
         check(got[r], ref, f"row {r}")
 
 
+@pytest.mark.parametrize("nq,nkv,start,rows,window,ring,qscale", [
+    (8, 1, 0, 256, 0, 0, 0.5),          # a whole first chunk: every row's range ends inside the tiles (causal masks everywhere)
+    (8, 1, 1000, 61, 0, 0, 1.0),        # rows not a multiple of the eight a workgroup takes; chunk ends inside a tile
+    (8, 1, 2000, 40, 512, 512, 0.5),    # sliding window over a wrapped 512-slot ring: both ends of the range move with the row
+    (4, 2, 300, 19, 0, 0, 1.0),         # two KV heads, two query heads each (padded MFMA rows)
+    (8, 1, 5, 9, 3, 0, 1.0),            # a window shorter than the rows per workgroup: rows that share no position
+    (8, 1, 777, 2, 0, 0, 0.05),         # two rows, nearly flat scores
+])
+def test_prefill_tiled_rows_share_a_pass(pkg, gpu, oracle, nq, nkv, start, rows, window, ring, qscale):
+    """The tiled prefill kernel (eight query rows per workgroup over one pass of the codes, shaders/attention_flash_tq.metal:
+    425-556): every row against the f64 code-space oracle at that row's position, the reference's own check of its tiled
+    kernel against per-row decode (kernels.rs:10295) at the attention tolerance.  The output buffer is pre-filled and has
+    guard words behind it."""
+    print(f"case tiled prefill nq={nq} nkv={nkv} start={start} rows={rows} window={window} ring={ring}", flush=True)
+    ctx, K = gpu
+    hd, bits = 256, 2
+    T = start + rows
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 77 + rows, ring=ring)
+    rq = (pkg.synth.rng(6, 15 + rows).standard_normal((rows, nq, hd), dtype=np.float32) * np.float32(qscale)).astype(np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    guard = 64
+    out = pkg.Buffer.from_slice(ctx, np.full(rows * nq * hd + guard, 7.5, np.float32))
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, start, rows, nq, nkv, window, bits, ring)
+    batch.commit_and_wait()
+    full = out.as_array(np.float32)
+    assert (full[rows * nq * hd:] == 7.5).all()
+    got = full[:rows * nq * hd].reshape(rows, nq * hd)
+    worst = 0.0
+    for r in range(rows):
+        ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, levels, hd, T, start + r, nq, nkv, window, bits, ring)
+        worst = max(worst, check(got[r], ref, f"row {r}"))
+    print(f"worst row: {worst:.2e} of max|ref|")
+
+
+def test_prefill_tiled_last_chunk_of_a_32k_prompt(pkg, gpu, oracle):
+    """The measured prefill shape: the last 256 rows of a 32768-token prompt (each row sees 32513 .. 32768 positions).
+    Sixteen rows spread over the chunk against the f64 oracle; all rows finite; and the rows the tiled kernel produced
+    against the per-row path on the same inputs (LOCAL_HIP_ATTN_PREFILL cannot be switched inside a process, so the
+    per-row figures come from the single-query entry at each sampled row's position)."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, T, rows = 256, 8, 1, 2, 32768, 256
+    start = T - rows
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 32769)
+    rq = pkg.synth.rng(6, 16).standard_normal((rows, nq, hd), dtype=np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    got = out.as_array(np.float32).reshape(rows, nq * hd)
+    assert np.isfinite(got).all()
+    one = pkg.Buffer.empty(ctx, nq * hd * 4)
+    for r in list(range(0, rows, 17)) + [rows - 1]:
+        print(f"case 32k prefill row {r}", flush=True)
+        ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, levels, hd, T, start + r, nq, nkv, 0, bits, 0)
+        check(got[r], ref, f"row {r}")
+        rq1 = pkg.Buffer.from_slice(ctx, rq[r])
+        K.flash_attention_tq_into(batch, rq1, kcb, knb, vcb, vnb, lvb, one, hd, T, start + r, nq, nkv, 0, bits, 0)
+        batch.commit_and_wait()
+        check(got[r], one.as_array(np.float32), f"row {r} against the single-query kernel")
+
+
+def test_prefill_with_a_level_table_that_is_not_affine(pkg, gpu, oracle):
+    """A level table that is not affine in the code bits (the tiled kernel's K side assumes it is): the entry must take
+    the per-row path, which carries a third bit plane, and still match the oracle.  And a table that was affine when it
+    was uploaded but is overwritten on the device afterwards must be reported at the wait, not multiplied with."""
+    ctx, K = gpu
+    hd, nq, nkv, bits, start, rows = 256, 8, 1, 2, 50, 12
+    T = start + rows
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 91)
+    odd = levels.copy()
+    odd[3] = np.float32(odd[3] * 1.3)
+    rq = pkg.synth.rng(6, 17).standard_normal((rows, nq, hd), dtype=np.float32)
+    kcb, knb, vcb, vnb, lvb, rqb, oddb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, odd)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, oddb, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
+    batch.commit_and_wait()
+    got = out.as_array(np.float32).reshape(rows, nq * hd)
+    for r in range(rows):
+        ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, odd, hd, T, start + r, nq, nkv, 0, bits, 0)
+        check(got[r], ref, f"row {r}, non-affine table")
+    # device-side overwrite of an uploaded affine table: blit the odd table over it
+    batch.blit_copy(oddb, 0, lvb, 0, 16)
+    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
+    with pytest.raises(pkg.CommandBuffer, match="level table"):
+        batch.commit_and_wait()
+    batch.commit_and_wait()      # the report clears the fault word
+
+
 @pytest.mark.parametrize("hd", [256, 512])
 def test_batched_matches_independent_sequences(pkg, gpu, oracle, hd):
     """kernels.rs:10457: lanes at different positions in one dispatch == separate single-sequence calls."""
