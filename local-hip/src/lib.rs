@@ -1,16 +1,59 @@
 //! HIP (MI355X / gfx950) backend behind the kernel-dispatch API that `local-engine` calls on `local-metal`.
 //!
-//! `ffi` holds the raw declarations of `liblocal_hip.so` (generated from `include/local_hip.h`).  The safe layer
-//! with the reference's type and method names (`Context`, `Buffer`, `CommandBatch`, `Kernels::<op>_into`, and an
-//! `Error` enum with the variants of `local_metal::Error`) wraps them one to one.
+//! * `ffi`      raw declarations of `liblocal_hip.so`, generated from `include/local_hip.h` (gen_ffi.py)
+//! * `error`    `Error` / `Result` with the variants and messages of `local_metal::Error`
+//! * `context`  `Context` (device + in-order stream; `MetalContext`)
+//! * `buffer`   `Buffer` (device memory; `MetalBuffer`)
+//! * `batch`    `CommandBatch`
+//! * `kernels`  `Kernels`: one method per dispatch operation, generated from the header (gen_safe.py)
+//! and, below, the host-side helpers of the TurboQuant codec that take plain slices.
+//!
+//! None of this has been compiled where the library is developed (no Rust toolchain there): the generated files are
+//! held to the header textually by tests/test_ffi_binding.py, the hand-written ones are short and reviewed by eye.
+pub mod batch;
+pub mod buffer;
+pub mod context;
+pub mod error;
 pub mod ffi;
+pub mod kernels;
 
-use core::ffi::CStr;
+pub use batch::{BufferCopyRequest, CommandBatch};
+pub use buffer::Buffer;
+pub use context::Context;
+pub use error::{last_error, Error, Result};
+pub use kernels::Kernels;
 
-/// Message of the last failed call on this thread (`lh_last_error`), in the wording of `local_metal::Error`'s
-/// `Display` (local-metal/src/error.rs:1-32).
-pub fn last_error() -> String {
-    // SAFETY: lh_last_error returns a pointer to a NUL-terminated thread-local buffer that stays valid until the
-    // next failing call on this thread.
-    unsafe { CStr::from_ptr(ffi::lh_last_error()) }.to_string_lossy().into_owned()
+/// `TurboQuant::levels` (local-engine/src/turboquant.rs:114-166): the 2^bits Lloyd-Max levels for `dim`, already divided
+/// by sqrt(dim).
+pub fn turboquant_levels(dim: u32, bits: u32) -> Result<Vec<f32>> {
+    let mut out = vec![0.0f32; 1usize << bits];
+    // SAFETY: `out` holds 2^bits floats, which is what the call writes.
+    error::check(unsafe { ffi::lh_turboquant_levels(dim, bits, out.as_mut_ptr()) })?;
+    Ok(out)
+}
+
+/// `Rotation::new(dim, seed).signs` (turboquant.rs:60-97): the +-1 diagonal of the randomised Hadamard rotation.
+pub fn turboquant_signs(dim: u32, seed: u64) -> Result<Vec<f32>> {
+    let mut out = vec![0.0f32; dim as usize];
+    // SAFETY: `out` holds `dim` floats.
+    error::check(unsafe { ffi::lh_turboquant_signs(dim, seed, out.as_mut_ptr()) })?;
+    Ok(out)
+}
+
+/// `code_bytes(dim, bits)` (kv_cache/quant_cache.rs:30-40).
+pub fn turboquant_code_bytes(dim: u32, bits: u32) -> u32 {
+    // SAFETY: pure function.
+    unsafe { ffi::lh_turboquant_code_bytes(dim, bits) }
+}
+
+/// `swa_ring_capacity(window, max_positions)` (quant_cache.rs:48-54).
+pub fn swa_ring_capacity(window: usize, max_positions: usize) -> usize {
+    // SAFETY: pure function.
+    unsafe { ffi::lh_swa_ring_capacity(window, max_positions) }
+}
+
+/// `flash_split_count(eff_seq_len)` (local-metal/src/kernels.rs:1265-1278).
+pub fn flash_split_count(eff_seq_len: u32) -> u32 {
+    // SAFETY: pure function.
+    unsafe { ffi::lh_flash_split_count(eff_seq_len) }
 }

@@ -104,3 +104,102 @@ def test_build_script_uses_the_kernel_makefile():
     assert "local-ai_amd" in text and "csrc" in text and "rustc-link-lib=dylib=local_hip" in text
     mk = open(os.path.join(ROOT, "local-ai_amd", "csrc", "Makefile")).read()
     assert "OUT ?=" in mk and "BUILD ?=" in mk      # the two variables build.rs overrides
+
+
+# ---- the safe layer: local-hip/src/{kernels,error,buffer,batch,context}.rs --------------------------------------------
+KERNELS_RS = os.path.join(ROOT, "local-hip", "src", "kernels.rs")
+SAFE_TYPES = {"const lh_buffer*": "&Buffer", "lh_buffer*": "&Buffer", "const lh_buffer* const*": "&[&Buffer]",
+              "lh_buffer* const*": "&[&Buffer]", "const uint32_t*": "&[u32]", "uint32_t": "u32", "uint64_t": "u64",
+              "size_t": "usize", "float": "f32", "int": "c_int", "lh_quant": "ffi::lh_quant", "lh_dtype": "ffi::lh_dtype"}
+
+
+def safe_methods():
+    """[(method, [(name, type)], raw function called, [argument expressions])] parsed from kernels.rs."""
+    text = open(KERNELS_RS).read()
+    out = []
+    for m in re.finditer(r"pub fn (\w+)\(&self, ([^)]*)\) -> Result<\(\)> \{(.*?)\n    \}", text, flags=re.S):
+        params = [tuple(s.strip() for s in prm.split(":", 1)) for prm in m.group(2).split(", ")]
+        call = re.search(r"ffi::(lh_\w+)\((.*?)\) \}\)", m.group(3), flags=re.S)
+        out.append((m.group(1), params, call.group(1), [a.strip() for a in call.group(2).split(", ")]))
+    return out
+
+
+def test_safe_layer_methods_follow_the_header():
+    """Every dispatch operation of the header (first parameter the batch or the context, the rest buffers, buffer arrays
+    and scalars) has one `Kernels` method named as the header function less `lh_`, with the header's parameter names in the
+    header's order and types that correspond, and the method hands them to that raw function in that order."""
+    header = {f[0]: f for f in c_functions()}
+    methods = safe_methods()
+    assert len(methods) >= 60, len(methods)
+    wrapped = set()
+    for method, params, raw, args in methods:
+        assert raw == "lh_" + method, (method, raw)
+        _, cret, cparams = header[raw]
+        assert cret == "int"
+        wrapped.add(raw)
+        assert len(params) == len(cparams) == len(args), method
+        first_c = cparams[0][0]
+        assert params[0] == (("batch", "&mut CommandBatch") if first_c == "lh_batch*" else ("ctx", "&Context")), method
+        assert args[0] == params[0][0] + ".as_ptr()"
+        for (pname, ptype), (ctype, cname), arg in zip(params[1:], cparams[1:], args[1:]):
+            assert pname.rstrip("_") == cname, f"{method}: {pname} vs {cname}"
+            assert ptype == SAFE_TYPES[ctype], f"{method}({cname}): {ptype} for {ctype}"
+            want = {"&Buffer": f"{pname}.as_ptr()", "&[&Buffer]": f"{pname}_raw.as_ptr()", "&[u32]": f"{pname}.as_ptr()"}.get(ptype, pname)
+            assert arg == want, f"{method}: passes {arg} for {cname}"
+    # nothing that is a dispatch operation was left out
+    for name, cret, cparams in header.values():
+        is_op = bool(cret == "int" and cparams and cparams[0][0] in ("lh_batch*", "lh_context*")
+                 and not name.startswith(("lh_context_", "lh_buffer_", "lh_batch_", "lh_event_", "lh_graph_"))
+                 and all(t in SAFE_TYPES for t, _ in cparams[1:]))
+        assert (name in wrapped) == is_op, name
+
+
+def test_safe_layer_argument_order_of_the_reference():
+    """Three methods whose parameter lists were read off the reference (local-metal/src/kernels.rs:4819-4834, 5176-5193,
+    5434-5452; kept here as data): the generated methods take exactly these parameters in exactly this order."""
+    want = {
+        "encode_kv_turboquant_into": ["batch", "input", "levels", "signs", "packed", "norms", "head_dim", "n_kv_heads",
+                                      "num_tokens", "bits", "position", "ring_capacity"],
+        "flash_attention_tq_into": ["batch", "rq", "k_codes", "k_norms", "v_codes", "v_norms", "levels", "out", "head_dim",
+                                    "kv_len", "current_pos", "num_q_heads", "num_kv_heads", "window", "bits", "ring_capacity"],
+        "flash_attention_tq_batched_into": ["batch", "rq", "k_codes", "k_norms", "v_codes", "v_norms", "levels", "out",
+                                            "positions", "head_dim", "lane_capacity", "num_q_heads", "num_kv_heads", "window",
+                                            "bits", "n_lanes", "ring_capacity"],
+    }
+    have = {m: [p[0] for p in params] for m, params, _, _ in safe_methods()}
+    for method, names in want.items():
+        assert have[method] == names, method
+
+
+def test_safe_layer_is_up_to_date_and_complete():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "local-hip", "gen_safe.py"), "--check"], capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr
+    src = os.path.join(ROOT, "local-hip", "src")
+    lib = open(os.path.join(src, "lib.rs")).read()
+    for mod in ("batch", "buffer", "context", "error", "ffi", "kernels"):
+        assert os.path.exists(os.path.join(src, mod + ".rs")), mod
+        assert f"pub mod {mod};" in lib, mod
+    err = open(os.path.join(src, "error.rs")).read()
+    for variant in ("NoDevice", "NoCommandQueue", "BufferAllocation", "LibraryCreation", "PipelineCreation", "ShaderNotFound",
+                    "CommandBuffer", "InvalidArgument", "Io"):          # local-metal/src/error.rs:1-32
+        assert re.search(rf"\b{variant}\b", err), variant
+    for code in ("LH_ERR_NO_DEVICE", "LH_ERR_NO_COMMAND_QUEUE", "LH_ERR_BUFFER_ALLOCATION", "LH_ERR_LIBRARY_CREATION",
+                 "LH_ERR_PIPELINE_CREATION", "LH_ERR_SHADER_NOT_FOUND", "LH_ERR_COMMAND_BUFFER", "LH_ERR_IO"):
+        assert f"ffi::{code} =>" in err, code
+    # every raw function the hand-written modules call exists in ffi.rs with that many arguments
+    raw = {f[0]: len(f[2]) for f in rust_functions()}
+    for mod in ("batch", "buffer", "context", "error", "lib"):
+        text = open(os.path.join(src, mod + ".rs")).read()
+        for m in re.finditer(r"ffi::(lh_\w+)\(", text):
+            name = m.group(1)
+            assert name in raw, (mod, name)
+            depth, n, i, seen = 1, 0, m.end(), False
+            while depth:                      # walk to the matching parenthesis, counting top-level commas
+                ch = text[i]
+                depth += ch in "(["
+                depth -= ch in ")]"
+                seen = seen or (depth >= 1 and not ch.isspace())
+                n += ch == "," and depth == 1
+                i += 1
+            n = n + 1 if seen else 0
+            assert n == raw[name], (mod, name, n, raw[name])
