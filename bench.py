@@ -342,6 +342,47 @@ def bench_layer(pkg, ctx, K, steps, warmup):
     return res
 
 
+def bench_layer_hbm(pkg, ctx, K, steps, warmup, total_bytes=1 << 30):
+    """The same small-batch layer with the weights coming from HBM: enough distinct copies of the layer's seven
+    projections (18.3 MB each set) to exceed 1 GiB, walked once per step, so that no weight is served from the 256 MB
+    last-level cache.  GB/s = weight bytes of all sets / time of one walk."""
+    g = pkg.synth.rng(3)
+    protos = [(fmt, n, k, pkg.synth.weights(fmt, n, k, g)) for _, fmt, n, k in pkg.synth.DECODER_LAYER]
+    set_bytes = sum(r.size for _, _, _, r in protos)
+    sets = max(2, -(-total_bytes // set_bytes))
+    stacks = []          # per projection: one allocation holding `sets` distinct copies
+    for fmt, n, k, raw in protos:
+        big = pkg.Buffer.empty(ctx, raw.size * sets)
+        blk = 18 if fmt == "q4_0" else 66
+        for i in range(sets):
+            big.copy_from_bytes(np.roll(raw, i * blk * 7), i * raw.size)
+        stacks.append((fmt, n, k, raw.size, big))
+    res = {"layer_sets": sets, "weight_bytes": set_bytes * sets}
+    batch = pkg.CommandBatch(ctx)
+    import ctypes as C
+    for m in (1, 4, 8, 16):
+        a2k = pkg.Buffer.from_slice(ctx, pkg.synth.activations(m, 2048, g))
+        a8k = pkg.Buffer.from_slice(ctx, pkg.synth.activations(m, 8192, g))
+        calls, keep = [], []          # `keep`: the views and outputs must outlive the bound calls, which hold raw handles
+        for i in range(sets):
+            for fmt, n, k, wb, big in stacks:
+                ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+                out, w = pkg.Buffer.empty(ctx, m * n * 4), big.view(i * wb, wb)
+                keep += [out, w]
+                calls.append(bound_call(pkg.lib().lh_matmul_nt_quant_typed_into, batch, C.c_int(ty), a2k if k == 2048 else a8k,
+                                        C.c_int(pkg.F32), w, out, C.c_int(pkg.F32), m, k, n))
+
+        def step():
+            for c in calls:
+                c()
+
+        _, ev = time_steps(pkg, ctx, step, max(3, steps // 4), 1)
+        res[f"m{m}_us_per_layer"] = ev * 1e3 / sets
+        res[f"m{m}_gbs"] = set_bytes * sets / ev * 1e-6
+        res[f"m{m}_frac_of_hbm_peak"] = res[f"m{m}_gbs"] / HBM_PEAK_GBS
+    return res
+
+
 def bench_prefill(pkg, ctx, K, steps, warmup):
     m, k, n = 512, 2048, 8192
     res = {}
@@ -873,6 +914,8 @@ def main():
     if "layer" in legs:
         extra["decoder_layer_small_batch"] = bench_layer(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] layer:", extra["decoder_layer_small_batch"])
+        extra["decoder_layer_small_batch_hbm"] = bench_layer_hbm(pkg, ctx, K, args.steps, args.warmup)
+        log("[bench] layer, weights from HBM:", extra["decoder_layer_small_batch_hbm"])
     if "prefill" in legs:
         extra["prefill_matmul_512x2048x8192_bf16"] = bench_prefill(pkg, ctx, K, args.steps, args.warmup)
         log("[bench] prefill:", extra["prefill_matmul_512x2048x8192_bf16"])

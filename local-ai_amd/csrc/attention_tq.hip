@@ -465,8 +465,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     int r = lh_check_launch(op);
     if (r != LH_OK) return r;
     batch->dispatch_count++;
-    static const int no_fused_merge = [] { const char* e = getenv("LOCAL_HIP_ATTN_MERGE_ROTATE"); return e && e[0] == '0' && e[1] == 0; }();
-    if (rot && p.num_splits > 1 && p.num_splits <= 2 * kReduceBatch && !no_fused_merge) {
+    if (rot && p.num_splits > 1 && p.num_splits <= 2 * kReduceBatch) {
         hipLaunchKernelGGL(attention_tq_reduce_rotate_kernel, dim3(p.num_queries * p.num_q_heads), dim3(p.head_dim), 0, ctx->stream,
                            (const float*)ws, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim, p.num_splits,
                            1.0f / std::sqrt((float)p.head_dim));

@@ -801,12 +801,12 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
     // One workgroup (a K wave and one V wave per 256 dims) per chunk of positions.  Short jobs (the chunks of one workgroup per CU
     // stay within 128 positions) are latency bound: they get chunks down to one group of 64 and never share a CU.
-    // Everything else gets about `wps` waves per SIMD over the whole launch and at least 128 positions per chunk.
-    static const int occ = [] { const char* e = getenv("LOCAL_HIP_ATTN_OCC"); return e ? atoi(e) : 2; }();
-    static const int wps = [] { const char* e = getenv("LOCAL_HIP_ATTN_WAVES_PER_SIMD"); return e ? atoi(e) : 2; }();
+    // Everything else gets about two waves per SIMD over the whole launch (the registers allow no third) and at least 128
+    // positions per chunk.
+    constexpr uint32_t wps = 2;
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
     const uint32_t wg_waves = p.head_dim == 512 ? 4 : 2;
-    const uint64_t wg_slots = (uint64_t)ctx->cu_count * std::max(1u, 4u * (uint32_t)wps / wg_waves);
+    const uint64_t wg_slots = (uint64_t)ctx->cu_count * std::max(1u, 4u * wps / wg_waves);
     uint64_t splits = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)ctx->cu_count / pairs));
     splits = std::max<uint64_t>(splits, 1);
     if ((max_span + splits - 1) / splits > 128) {
@@ -824,22 +824,15 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
     // Hand-overs of two groups pay from about a thousand positions per workgroup on (-2 % at 4096 positions per workgroup, -5 % at
     // 8192, either head_dim); below that the longer fill and drain of the pipeline costs more (a 512-position window: +24 %).
+    // LOCAL_HIP_ATTN_PAIR=1 / 0 forces one form onto every chunk length (a test aid: it puts missing and partial groups at both
+    // ends of short chunks through the paired loops).
     static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
-    static const uint64_t pair_min = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR_MIN"); return e ? (uint64_t)atoll(e) : (uint64_t)1024; }();
+    constexpr uint64_t pair_min = 1024;
     const bool pair = pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min;
-    if (p.head_dim == 512 && pair) {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
-    } else if (p.head_dim == 512) {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
-    } else if (pair) {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
-    } else {
-        if (occ == 1) hipLaunchKernelGGL((attention_tq_mfma_kernel<1, 256, 1>), grid, dim3(128), 0, ctx->stream, a, p);
-        else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 1>), grid, dim3(128), 0, ctx->stream, a, p);
-    }
+    if (p.head_dim == 512 && pair) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
+    else if (p.head_dim == 512) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
+    else if (pair) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);
+    else hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 1>), grid, dim3(128), 0, ctx->stream, a, p);
     return lh_check_launch(op);
 }
 

@@ -903,12 +903,11 @@ __global__ __launch_bounds__(256, 2) void matmul_skinny_kernel(const uint16_t* _
     }
 }
 
-// Most activation rows the skinny kernel takes (LOCAL_HIP_SKINNY_MAX_M, default 256: a prefill chunk).  Beyond 64 rows
+// Most activation rows the skinny kernel takes (256: a prefill chunk).  Beyond 64 rows
 // every group of 64 gets workgroups of its own, which re-read the codes from L2 while the activation traffic grows with
 // rows x weight rows; measured on a 256-row chunk of the layer bench: 197 -> 163 us per layer, no gain at 512 rows.
 uint32_t skinny_max_m() {
-    static const int v = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_M"); return e && atoi(e) > 16 ? atoi(e) : 256; }();
-    return (uint32_t)v;
+    return 256u;
 }
 
 // ---- Q4_0, 2 .. 16 activation rows: the same workgroup shape with the operand roles swapped ----------------------------------------
@@ -1014,37 +1013,32 @@ __global__ __launch_bounds__(256, 2) void matmul_small_q4_kernel(const uint16_t*
     }
 }
 
-// Fewest activation rows the skinny kernel takes; below it rows run as matvecs.  TQ2_0 from 2 rows (LOCAL_HIP_SKINNY_MIN_M_TQ2):
+// Fewest activation rows the skinny kernel takes; below it rows run as matvecs.  TQ2_0 from 2 rows:
 // its f16 weights d (q - 1) are exact, so the results differ from the matvec kernels' only in the order of the f32 sums,
 // and a 35-layer step over 16 lanes at 8k context went from 5.19 to 4.05 ms (8 lanes 4.14 to 3.59, 4 lanes 3.63 to 3.38).  Q4_0
-// from 9 rows (LOCAL_HIP_SKINNY_MIN_M; the matvec kernels are as fast up to 8): up to 16 rows go to matmul_small_q4_kernel,
+// from 9 rows (the matvec kernels are as fast up to 8): up to 16 rows go to matmul_small_q4_kernel,
 // which keeps the weights unrounded as the reference's small-batch kernels do (16 lanes 3.95 -> 3.80 ms); from 17 rows on
 // the weights are the CPU path's f16 values, as in its matrix kernels.
-// Fewest f32 activation rows the TQ2_0 skinny kernel takes (LOCAL_HIP_SKINNY_MIN_M_F32); below it the rows run as matvecs.
+// Fewest f32 activation rows the TQ2_0 skinny kernel takes; below it the rows run as matvecs.
 // One layer's three TQ2_0 projections, weights cache resident: rows 34.3 / 42.2 / 47.4 us at 8 / 12 / 16 rows, this form
 // 36.3 / 36.8 / 37.6 us.
 uint32_t skinny_min_m_f32() {
-    static const int v = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_F32"); return e && atoi(e) > 0 ? atoi(e) : 10; }();
-    return (uint32_t)v;
+    return 10u;
 }
 uint32_t skinny_min_m(int fmt) {
-    static const int q4 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M"); return e && atoi(e) > 0 ? atoi(e) : 9; }();
-    static const int tq2 = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MIN_M_TQ2"); return e && atoi(e) > 0 ? atoi(e) : 2; }();
-    return (uint32_t)(fmt == kTQ2 ? tq2 : q4);
+    return fmt == kTQ2 ? 2u : 9u;
 }
 
-// Most 64-row workgroups a launch of the skinny kernel may have (LOCAL_HIP_SKINNY_MAX_WG_PER_CU per CU, default 64).
+// Most 64-row workgroups a launch of the skinny kernel may have (64 per CU).
 uint32_t skinny_max_blocks(const lh_context* ctx) {
-    static const int per_cu = [] { const char* e = getenv("LOCAL_HIP_SKINNY_MAX_WG_PER_CU"); return e && atoi(e) > 0 ? atoi(e) : 64; }();
-    return (uint32_t)per_cu * (uint32_t)ctx->cu_count;
+    return 64u * (uint32_t)ctx->cu_count;
 }
 
 // k splits of the skinny kernel over `workgroups` (64-row blocks x groups of 64 activation rows): enough workgroups for every CU, a whole number of units
 // per wave, partial tiles within half the workspace.
 uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t workgroups, uint32_t units_per_wg) {
-    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
     uint32_t splits = 1;
-    if (!no_splitk && workgroups < (uint32_t)ctx->cu_count) {
+    if (workgroups < (uint32_t)ctx->cu_count) {
         const uint32_t blocks = workgroups / ((m + 63) / 64);
         const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * blocks * 64 * 4);
         const uint32_t want = (uint32_t)std::min<uint64_t>(((uint32_t)ctx->cu_count + workgroups - 1) / workgroups, fit);
@@ -1054,7 +1048,7 @@ uint32_t skinny_splits(const lh_context* ctx, uint32_t m, uint32_t workgroups, u
 }
 
 // The skinny kernel when the shape allows it (f16 activations, 17 .. skinny_max_m() rows, whole 128-row tiles, at least one unit of k
-// per wave; LOCAL_HIP_SKINNY_MAX_WG_PER_CU bounds the workgroups per CU, by default far above any shape here); false
+// per wave; at most 64 workgroups per CU, far above any shape here); false
 // leaves the launch to the LDS-tiled kernels.  With `keep` the f32 partial
 // tiles (one split included) stay in the workspace for a consumer that sums them itself.
 struct SkinnyPartials { const float* partial; uint32_t splits, cols; };
@@ -1066,10 +1060,9 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
     if constexpr (FMT != kF16W && ADT == LH_F32) {
         // f32 activations as pairs of f16 rows: up to 32 rows.  TQ2_0 from skinny_min_m_f32() rows (below that the rows run as
         // matvecs); Q4_0 from 17 rows (up to 16 the matvec rows multiply unrounded weights, as the reference's kernels do).
-        static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
         const uint32_t units = k / Skinny<FMT>::unit_k;
         const uint32_t min_m = FMT == kTQ2 ? skinny_min_m_f32() : (uint32_t)kMaxMultivecM + 1;
-        if (!no_skinny && !clip.enabled && !grp.count && !keep && m >= min_m && m <= 32 && n % BN == 0 && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+        if (!clip.enabled && !grp.count && !keep && m >= min_m && m <= 32 && n % BN == 0 && k % (4 * Skinny<FMT>::unit_k) == 0 &&
             2 * tiles_n <= skinny_max_blocks(ctx)) {
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
             const uint32_t splits = skinny_splits(ctx, m, blocks, per_wg);
@@ -1087,11 +1080,10 @@ bool try_skinny(lh_context* ctx, const void* A, const uint8_t* W, void* C, lh_dt
         }
     }
     if constexpr (FMT != kF16W && ADT == LH_F16) {
-        static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
         bool whole = grp.count ? true : n % BN == 0;          // every matrix fills its 128-row tiles
         for (uint32_t i = 0; i < grp.count; i++) whole = whole && grp.N[i] % BN == 0;
         const uint32_t units = k / Skinny<FMT>::unit_k;
-        if (!no_skinny && !clip.enabled && m >= skinny_min_m(FMT) && m <= skinny_max_m() && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
+        if (!clip.enabled && m >= skinny_min_m(FMT) && m <= skinny_max_m() && whole && k % (4 * Skinny<FMT>::unit_k) == 0 &&
             2 * tiles_n <= skinny_max_blocks(ctx) && (m <= 64 || 2 * tiles_n * ((m + 63) / 64) <= 8 * (uint32_t)ctx->cu_count)) {
             // k splits: enough workgroups for every CU, a whole number of units per wave, partial tiles within half the workspace
             const uint32_t blocks = 2 * tiles_n, per_wg = units / 4;
@@ -1128,13 +1120,12 @@ void launch_tiles64(lh_context* ctx, const void* A, const uint8_t* W, void* C, l
                     const GroupArgs& grp) {
     hipStream_t s = ctx->stream;
     const int cus = ctx->cu_count;
-    static const int no_splitk = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SPLITK"); return e && e[0] == '0' && e[1] == 0; }();
     const uint32_t nk = (k + BK - 1) / BK;
     const uint32_t tiles_n = grp.count ? grp.tile0[grp.count] : (n + BN - 1) / BN;
     if (try_skinny<FMT, ADT>(ctx, A, W, C, ct, m, k, n, clip, grp)) return;
     const uint64_t tiles64 = (uint64_t)tiles_n * ((m + 63) / 64);
     uint32_t splits = 1;
-    if (!no_splitk && tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
+    if (tiles64 * 2 <= (uint64_t)cus && nk >= 4) {
         splits = (uint32_t)std::min<uint64_t>(nk / 2, ((uint64_t)cus + tiles64 - 1) / tiles64);
         const uint64_t fit = (ctx->workspace_bytes / 2) / ((uint64_t)m * tiles_n * BN * 4);
         splits = (uint32_t)std::min<uint64_t>(splits, fit);
@@ -1159,40 +1150,32 @@ int launch_by_out(bool mfma, lh_context* ctx, const void* A, const uint8_t* W, v
     const int cus = ctx->cu_count;
     if (mfma) {
         if (try_skinny<FMT, ADT>(ctx, A, W, C, ct, m, k, n, clip, GroupArgs{})) return LH_OK;
-        static const int force_bm = [] { const char* e = getenv("LOCAL_HIP_PREFILL_BM"); return e ? atoi(e) : 0; }();
         // 128-row tiles reuse each dequantised weight tile twice as often; 64-row tiles when that would leave most CUs idle
         const uint64_t tiles128 = (uint64_t)((n + BN - 1) / BN) * ((m + 127) / 128);
-        const bool big = force_bm == 128 || (force_bm == 0 && m > 64 && tiles128 * 2 >= (uint64_t)cus);
+        const bool big = m > 64 && tiles128 * 2 >= (uint64_t)cus;
         if constexpr (FMT != kF16W) {
             const size_t a16_bytes = (size_t)m * k * 2;
             if (big && k % BK == 0 && (ADT == LH_F16 || a16_bytes <= ctx->workspace_bytes)) {
                 const uint16_t* a16 = static_cast<const uint16_t*>(A);
-                static const int bf_inline = [] { const char* e = getenv("LOCAL_HIP_PREFILL_BF16_PASS"); return !(e && e[0] == '1' && e[1] == 0); }();
-                static const int pw4 = [] { const char* e = getenv("LOCAL_HIP_PREFILL_PW"); return e && atoi(e) == 4; }();   // four staging waves instead of eight
                 const dim3 grid128((n + BN - 1) / BN, (m + 127) / 128);
                 if constexpr (ADT == LH_BF16) {
-                    if (bf_inline) {             // bf16 is converted by the staging waves (LOCAL_HIP_PREFILL_BF16_PASS=1: by a pass of its own)
-                        if (pw4 && ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, true, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
-                        else if (pw4) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, true, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
-                        else if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
-                        else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
-                        return LH_OK;
-                    }
+                    // bf16 is converted by the staging waves on its way into LDS
+                    if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                    else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, true, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                    return LH_OK;
                 }
                 if constexpr (ADT != LH_F16) {   // f32: one pass over the activations instead of a conversion in every column tile
                     const size_t n8 = (size_t)m * k / 8;
                     hipLaunchKernelGGL((convert_to_f16_kernel<ADT>), dim3((uint32_t)((n8 + 255) / 256)), dim3(256), 0, s, A, (uint16_t*)ctx->workspace, n8);
                     a16 = static_cast<const uint16_t*>(ctx->workspace);
                 }
-                if (pw4 && ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, false, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
-                else if (pw4) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, false, 4>), grid128, dim3(512), 0, s, a16, W, C, m, k, n);
-                else if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, false, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
+                if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F32, false, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
                 else hipLaunchKernelGGL((matmul_mfma128_kernel<FMT, LH_F16, false, 8>), grid128, dim3(768), 0, s, a16, W, C, m, k, n);
                 return LH_OK;
             }
         }
         const uint32_t nk = (k + BK - 1) / BK;
-        if (force_bm == 128 || (force_bm == 0 && tiles128 >= 2ull * (uint64_t)cus)) {
+        if (tiles128 >= 2ull * (uint64_t)cus) {
             const dim3 grid((n + BN - 1) / BN, (m + 127) / 128);
             if (ct == LH_F32) hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F32, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk, GroupArgs{});
             else hipLaunchKernelGGL((matmul_mfma_kernel<FMT, ADT, LH_F16, 128>), grid, dim3(256), 0, s, A, W, C, m, k, n, clip, (float*)nullptr, nk, GroupArgs{});
@@ -1468,13 +1451,12 @@ int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer*
     LH_NEED(out, (size_t)m * n * 2, op, "output");
     LH_REQUIRE(((uintptr_t)in->ptr & 15) == 0 && ((uintptr_t)out->ptr & 15) == 0, "%s: input and output must be 16-byte aligned", op);
     LH_REQUIRE((((uintptr_t)w_gate->ptr | (uintptr_t)w_up->ptr) & 1) == 0, "%s: weights must be 2-byte aligned", op);
-    static const int no_skinny = [] { const char* e = getenv("LOCAL_HIP_MATMUL_SKINNY"); return e && e[0] == '0' && e[1] == 0; }();
     const uint32_t unit_k = fmt == LH_Q4_0 ? Skinny<kQ4>::unit_k : Skinny<kTQ2>::unit_k;
     const uint32_t blocks = n / 32;
     // one launch where the grouped product of the pair takes the skinny kernel without a k split (split products need
     // their sums before the gelu); the same workgroup count and k ranges, hence the same sums
     const uint32_t mgroups = (m + 63) / 64;
-    if (!no_skinny && m >= skinny_min_m(fmt == LH_Q4_0 ? kQ4 : kTQ2) && (fmt != LH_Q4_0 || m > (uint32_t)kMaxMultivecM) && m <= skinny_max_m() &&
+    if (m >= skinny_min_m(fmt == LH_Q4_0 ? kQ4 : kTQ2) && (fmt != LH_Q4_0 || m > (uint32_t)kMaxMultivecM) && m <= skinny_max_m() &&
         n % BN == 0 && k % (4 * unit_k) == 0 &&
         blocks <= skinny_max_blocks(ctx) && (m <= 64 || blocks * mgroups <= 8 * (uint32_t)ctx->cu_count) &&
         skinny_splits(ctx, m, blocks * mgroups, k / unit_k / 4) == 1) {

@@ -529,15 +529,8 @@ __global__ __launch_bounds__(256) void matvec_tq2_0_soa_kernel(const uint8_t* __
     if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
 }
 
-// LOCAL_HIP_X_LIMBS=3: 24-bit first-level activations for Q4_0 (no second level then).  TQ2_0 always takes two limbs: with
-// its fields left in place (up to 16 x the code) and 256-element blocks, three limbs overflow the 32-bit sums.
-int x_limbs(lh_quant fmt) {
-    static int v = [] {
-        const char* e = getenv("LOCAL_HIP_X_LIMBS");
-        return (e && e[0] == '3') ? 3 : 2;
-    }();
-    return fmt == LH_Q4_0 ? v : 2;
-}
+// Activation limbs: two (16-bit block fixed point, with a second level for blocks that need one).
+int x_limbs(lh_quant) { return 2; }
 
 // LOCAL_HIP_TQ2_KERNEL=valu selects the vector-ALU (v_dot4) TQ2_0 kernel instead of the MFMA one.
 bool tq2_on_matrix_cores() {
@@ -548,26 +541,13 @@ bool tq2_on_matrix_cores() {
     return v;
 }
 
-int wg_per_cu() {
-    static int v = [] {
-        const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU");
-        int n = e ? atoi(e) : 2;
-        return n < 1 ? 1 : (n > 8 ? 8 : n);
-    }();
-    return v;
-}
+int wg_per_cu() { return 2; }
 
 struct LaunchGeom {
     uint32_t npos, lpr_log2, rpw, grid, steps_per_wg;
     size_t lds_bytes;
     bool img;   // staged form: Q4_0 with two limbs and at least 16 readable bytes behind every matrix
 };
-
-// LOCAL_HIP_Q4_IMAGE=0 keeps the Q4_0 kernel on direct per-lane loads.
-bool q4_image_enabled() {
-    static bool v = [] { const char* e = getenv("LOCAL_HIP_Q4_IMAGE"); return !(e && e[0] == '0' && e[1] == 0); }();
-    return v;
-}
 
 LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_count, int L, size_t min_slack = 0) {
     LaunchGeom g{};
@@ -597,7 +577,7 @@ LaunchGeom plan(lh_quant fmt, uint32_t count, uint32_t rows, uint32_t K, int cu_
     g.lds_bytes = (size_t)L * K + (size_t)(K / G) * 4 + (L == 2 ? (size_t)2 * K + (size_t)(K / G) * 4 + 16 : 0);
     // the staged form pays off once a wave walks several steps (its first fetch is not overlapped with anything)
     const uint32_t in_flight = g.npos == 1 ? 4u : (g.npos == 2 ? 2u : 1u);        // steps_in_flight<LH_Q4_0>(npos)
-    g.img = fmt == LH_Q4_0 && L == 2 && min_slack >= 16 && g.steps_per_wg >= 2u * kWaves * in_flight && q4_image_enabled();
+    g.img = fmt == LH_Q4_0 && L == 2 && min_slack >= 16 && g.steps_per_wg >= 2u * kWaves * in_flight;
     // The images come on top of the activation area; rows long enough to push the sum past the raised limit keep direct loads.
     const size_t with_img = ((g.lds_bytes + 15) & ~(size_t)15) + (size_t)kWaves * kImgBytes;
     if (g.img && with_img > kMaxDynamicLds) g.img = false;
@@ -769,8 +749,7 @@ int matvec_dispatch(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buff
     const int L = x_limbs(fmt);
     const LaunchGeom g = plan(fmt, count, rows, cols, ctx->cu_count, L, min_slack);
     int r;
-    if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g)
-                                   : launch_npos<LH_Q4_0, 3>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
+    if (fmt == LH_Q4_0) r = launch_npos<LH_Q4_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
     else r = launch_npos<LH_TQ2_0, 2>(ctx, dev_desc, single, count, xt, yt, rows, cols, g);
     if (r == LH_OK) batch->dispatch_count++;
     return r;
@@ -812,8 +791,7 @@ int matvec_rows_impl(lh_batch* batch, lh_quant fmt, uint32_t m, const lh_buffer*
         MatvecBase single{MatvecProblem{(const uint8_t*)weight->ptr, input->ptr, output->ptr}, (uint32_t)xstride, (uint32_t)ystride};
         const int L = x_limbs(fmt);
         const LaunchGeom g = plan(fmt, m, n, k, ctx->cu_count, L, slack);
-        if (fmt == LH_Q4_0) r = L == 2 ? launch_npos<LH_Q4_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g)
-                                       : launch_npos<LH_Q4_0, 3>(ctx, nullptr, single, m, at, ct, n, k, g);
+        if (fmt == LH_Q4_0) r = launch_npos<LH_Q4_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g);
         else r = launch_npos<LH_TQ2_0, 2>(ctx, nullptr, single, m, at, ct, n, k, g);
     }
     (void)op;

@@ -423,33 +423,28 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     // quantised activation vector; few tiles with long rows: the block groups of a tile are split over 2-4 waves
     const uint32_t ngroups = (nb + 7) >> 3;
     uint32_t split_waves = 1;
-    static const int force_split = [] { const char* e = getenv("LOCAL_HIP_TQ2_FORCE_SPLIT"); return e ? atoi(e) : 0; }();
-    if (tiles < (uint64_t)ctx->cu_count * 2 || (force_split && ngroups > 1)) {
+    if (tiles < (uint64_t)ctx->cu_count * 2) {
         for (uint32_t w = 4; w >= 2; w--) if (ngroups % w == 0) { split_waves = w; break; }
         // six groups of blocks (12288 columns, the down projection of the wide feed-forward layers): a wave per group,
         // and twice the threads for the activation staging (f16 in and out only: the decode path's types)
-        static const int six = [] { const char* e = getenv("LOCAL_HIP_TQ2_SPLIT6"); return !(e && e[0] == '0' && e[1] == 0); }();
         const size_t lds6 = lds_head_bytes(K) + 128 + 6 * (size_t)kImageBytes + 3 * kStageLoads * 64 * 2 + kSplitAreaBytes;
-        if (six && ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= kMaxLdsBytes) split_waves = 6;
+        if (ngroups % 6 == 0 && xt == LH_F16 && yt == LH_F16 && lds6 <= kMaxLdsBytes) split_waves = 6;
     }
     const uint32_t splitk = split_waves > 1 ? 1u : 0u;
-    static const int wg256_tiles_per_cu = [] { const char* e = getenv("LOCAL_HIP_TQ2_WG256_TILES_PER_CU"); int n = e ? atoi(e) : 2; return n < 1 ? 1 : n; }();
-    static const int wg_cu = [] { const char* e = getenv("LOCAL_HIP_MATVEC_WG_PER_CU"); int n = e ? atoi(e) : 3; return n < 1 ? 1 : (n > 8 ? 8 : n); }();
+    constexpr int wg256_tiles_per_cu = 2, wg_cu = 3;
     auto lds_for = [&](uint32_t nwaves) { return lds_head_bytes(K) + 128 + (size_t)nwaves * kImageBytes + 3 * kStageLoads * 64 * 2 + kSplitAreaBytes; };
     uint32_t threads = splitk ? 64 * split_waves : (tiles >= (uint64_t)ctx->cu_count * wg256_tiles_per_cu ? 256 : 64);
     // Long rows make the activation area large: when fewer than three four-wave workgroups fit a CU's LDS, a large job runs
     // one twelve-wave workgroup per CU instead, which stages the activations once and keeps three waves on every SIMD
-    // (LOCAL_HIP_TQ2_WIDE=0 keeps four-wave workgroups).
-    static const int wide_on = [] { const char* e = getenv("LOCAL_HIP_TQ2_WIDE"); return !(e && e[0] == '0' && e[1] == 0); }();
+    // (four-wave workgroups measured 0.70 of the HBM rate on 2048 x 8192 weights where this form reaches 0.71).
     bool wide = false;
     uint32_t wide_split = 0;     // waves per tile when the twelve-wave workgroup runs in split form
-    if (!splitk && threads == 256 && wide_on && (160 * 1024) / lds_for(4) < 3 && lds_for(12) <= kMaxLdsBytes &&
+    if (!splitk && threads == 256 && (160 * 1024) / lds_for(4) < 3 && lds_for(12) <= kMaxLdsBytes &&
         tiles >= (uint64_t)ctx->cu_count * 24) {
         wide = true;
         threads = 768;
         // the block groups of a tile on neighbouring waves: the segments of one row are then fetched close together in time
-        static const int wsplit_on = [] { const char* e = getenv("LOCAL_HIP_TQ2_WIDE_SPLIT"); return !(e && e[0] == '0' && e[1] == 0); }();
-        if (wsplit_on && ngroups > 1 && 12 % ngroups == 0) wide_split = ngroups;
+        if (ngroups > 1 && 12 % ngroups == 0) wide_split = ngroups;   // (one wave walking all groups of its tile: 0.65 against 0.71)
     }
     const uint32_t waves = threads / 64;
     const uint32_t tiles_per_slot = wide_split ? waves / wide_split : (splitk ? 1u : waves);

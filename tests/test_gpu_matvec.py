@@ -62,7 +62,7 @@ def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
     y64 = oracle.matvec_f64(expand(raw, rows, cols), x)
     e64 = float(np.max(np.abs(got - y64) / np.maximum(np.abs(y64), 1.0)))
     print(f"{fmt} {rows}x{cols}: err vs CPU path {err:.2e}, vs f64 {e64:.2e}")
-    assert e64 <= 3e-4   # 16-bit block-fixed-point activations; 24-bit with LOCAL_HIP_X_LIMBS=3
+    assert e64 <= 3e-4   # 16-bit block-fixed-point activations
 
 
 @pytest.mark.parametrize("rows,cols", [(4096, 16384), (4000, 14400)])

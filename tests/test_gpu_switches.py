@@ -1,6 +1,8 @@
-"""The launch forms that only an environment switch selects (fallback kernels, the older forms kept for comparison) against
-the oracle: each case runs a few of the ordinary parity tests in a child process with the switch set -- the library reads
-its switches once per process.  One child at a time; a child takes a few seconds."""
+"""The launch forms that only an environment switch selects against the oracle: the fallback kernels (vector-ALU TQ2_0
+matvec, vector-ALU attention, per-row prefill attention) that otherwise run only for shapes the matrix-core kernels do
+not take, and the test aid that forces the attention kernel's paired hand-overs onto short chunks.  Each case runs a few
+of the ordinary parity tests in a child process with the switch set -- the library reads its switches once per
+process.  One child at a time; a child takes a few seconds."""
 import os
 import subprocess
 import sys
@@ -12,22 +14,13 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 CASES = [
-    ({"LOCAL_HIP_TQ2_KERNEL": "valu", "LOCAL_HIP_X_LIMBS": "3"}, "test_gpu_matvec.py", "baseline_configs or soa"),
-    ({"LOCAL_HIP_Q4_IMAGE": "0", "LOCAL_HIP_TQ2_WIDE": "0"}, "test_gpu_matvec.py", "evenly_spaced or long_rows"),
-    ({"LOCAL_HIP_TQ2_WIDE_SPLIT": "0"}, "test_gpu_matvec.py", "long_rows"),
-    ({"LOCAL_HIP_TQ2_FORCE_SPLIT": "1", "LOCAL_HIP_TQ2_SPLIT6": "0"}, "test_gpu_matvec.py", "reference_payloads and tq2_0"),
-    ({"LOCAL_HIP_PREFILL_PW": "4"}, "test_gpu_matmul.py", "prefill_config or large_tiles or weight_tiles"),
-    ({"LOCAL_HIP_PREFILL_BF16_PASS": "1"}, "test_gpu_matmul.py", "prefill_config or large_tiles"),
-    ({"LOCAL_HIP_MATMUL_SPLITK": "0", "LOCAL_HIP_MATMUL_SKINNY": "0"}, "test_gpu_matmul.py", "decode_batch_matmul or matmul_grouped or tile_boundaries"),
-    ({"LOCAL_HIP_ATTN_KERNEL": "valu", "LOCAL_HIP_ATTN_MERGE_ROTATE": "0"}, "test_gpu_attention.py",
-     "asymmetric_levels or empty_range or ring_matches or rotated_entry"),
-    ({"LOCAL_HIP_ATTN_OCC": "1", "LOCAL_HIP_ATTN_WAVES_PER_SIMD": "3"}, "test_gpu_attention.py", "batched_matches or split_invariance or asymmetric_levels"),
+    ({"LOCAL_HIP_TQ2_KERNEL": "valu"}, "test_gpu_matvec.py", "baseline_configs or soa or reference_payloads"),
+    ({"LOCAL_HIP_ATTN_KERNEL": "valu"}, "test_gpu_attention.py", "asymmetric_levels or empty_range or ring_matches or rotated_entry"),
+    ({"LOCAL_HIP_ATTN_PREFILL": "rows"}, "test_gpu_attention.py", "prefill"),
     # hand-overs of two groups forced onto every chunk length (missing and partial groups at both chunk ends), and never used
     ({"LOCAL_HIP_ATTN_PAIR": "1"}, "test_gpu_attention.py", "decode_attention_matches or prefill_matches or batched_matches or "
      "split_invariance or ring_matches or asymmetric_levels or empty_range or attention_sink or randomised_shapes"),
     ({"LOCAL_HIP_ATTN_PAIR": "0"}, "test_gpu_attention.py", "split_invariance or context_sweep_long"),
-    ({"LOCAL_HIP_PREFILL_BM": "64", "LOCAL_HIP_SKINNY_MAX_M": "64", "LOCAL_HIP_MATVEC_WG_PER_CU": "1"}, "test_gpu_matmul.py",
-     "prefill_config or large_tiles or small_batch_layer_config"),
 ]
 
 
