@@ -16,8 +16,10 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp, kValuSgpr, kAndOnlyLit, kAndOnlySgpr };
 
-// One iteration: 160 vector instructions and / or 16 MFMAs per wave (kSplitWaves: even waves 160 vector
-// instructions, odd waves 16 MFMAs).
+// One iteration per wave: 160 (v_and_b32, v_add_u32) pairs = 320 vector instructions and / or 16 MFMAs (kFine: 80 pairs
+// between 16 MFMAs; kSplitWaves: even waves the 160 pairs, odd waves the 16 MFMAs), or 160 instructions of one other kind.
+// The instruction counts handed to run() are those of the compiled loop bodies (hipcc -S): the and-xor chains of the last two
+// integer mixes compile to v_bitop3_b32 and v_xor_b32, 320 and 312 instructions.
 template <int MIX>
 __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned mask, unsigned step) {
     unsigned x[8];
@@ -32,7 +34,7 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
 #pragma unroll
             for (int r = 0; r < 20; r++)
 #pragma unroll
-                for (int i = 0; i < 8; i++) x[i] = (x[i] & 0x7f7f7f7fu) + 0x01010101u * (i + 1);   // v_and_b32 + v_add_u32
+                for (int i = 0; i < 8; i++) x[i] = (x[i] & 0x7f7f7f7fu) + 0x01010101u * (i + 1);   // v_and_b32 + v_add_u32, both with a 32-bit literal
         }
         if constexpr (MIX == kMfma || MIX == kCoarse) {
 #pragma unroll
@@ -69,13 +71,13 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
 #pragma unroll
                 for (int i = 0; i < 8; i++) f[i] = __builtin_fmaf(f[i], 1.0001f, 0.5f);
         }
-        if constexpr (MIX == kValuSgpr) {   // the same 160 instructions with the mask and the addend in scalar registers (no 32-bit literals)
+        if constexpr (MIX == kValuSgpr) {   // the same pairs with the mask and the addend in scalar registers (no 32-bit literals)
 #pragma unroll
             for (int r = 0; r < 20; r++)
 #pragma unroll
                 for (int i = 0; i < 8; i++) x[i] = (x[i] & mask) + step;
         }
-        if constexpr (MIX == kAndOnlyLit) {   // 160 v_and_b32 with a 32-bit literal each (an 8-byte encoding)
+        if constexpr (MIX == kAndOnlyLit) {   // an and-xor chain with a different 32-bit literal per element
 #pragma unroll
             for (int r = 0; r < 20; r++)
 #pragma unroll
@@ -138,17 +140,17 @@ int main() {
     g_ghz = khz * 1e-6;
     printf("clock reported by the device: %.2f GHz; columns: 1, 2, 3, 4 waves per SIMD; per column: time per iteration, SIMD cycles at\n"
            "that clock, and (ratio to the additive model: 4 cycles per vector instruction + 16 per MFMA, summed over the SIMD's waves)\n", g_ghz);
-    run<kValu>("160 v_and/v_add per wave", 160, 0, d);
-    run<kMfma>("16 MFMA per wave", 0, 16, d);
-    run<kFine>("16 x (5 vector + 1 MFMA) per wave", 80, 16, d);
-    run<kCoarse>("160 vector, then 16 MFMA per wave", 160, 16, d);
-    run<kSplitWaves>("even waves 160 vector, odd waves 16 MFMA", 160, 16, d);
-    run<kValuSgpr>("160 v_and/v_add, constants in SGPRs", 160, 0, d);
-    run<kAndOnlyLit>("160 x (v_and literal + v_xor) per wave", 320, 0, d);
-    run<kAndOnlySgpr>("160 x (v_and SGPR + v_xor) per wave", 320, 0, d);
-    run<kPerm>("160 v_perm_b32 per wave", 160, 0, d);
-    run<kFma>("160 v_fma_f32 per wave", 160, 0, d);
-    run<kExp>("160 v_exp_f32 per wave", 160, 0, d);
+    run<kValu>("160 x (v_and + v_add), literal operands", 320, 0, d);
+    run<kValuSgpr>("160 x (v_and + v_add), SGPR operands", 320, 0, d);
+    run<kAndOnlyLit>("320 v_bitop3/v_xor, literal masks", 320, 0, d);
+    run<kAndOnlySgpr>("312 v_bitop3/v_xor, SGPR mask", 312, 0, d);
+    run<kPerm>("160 v_perm_b32", 160, 0, d);
+    run<kFma>("160 v_fma_f32", 160, 0, d);
+    run<kExp>("160 v_exp_f32", 160, 0, d);
+    run<kMfma>("16 MFMA", 0, 16, d);
+    run<kFine>("16 x (5 x (v_and + v_add) + 1 MFMA)", 160, 16, d);
+    run<kCoarse>("160 x (v_and + v_add), then 16 MFMA", 320, 16, d);
+    run<kSplitWaves>("even waves 160 x (and + add), odd 16 MFMA", 320, 16, d);
     (void)hipFree(d);
     return 0;
 }
