@@ -439,7 +439,11 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     // shape and the level table was uploaded as one that is affine in the code bits (LOCAL_HIP_ATTN_PREFILL=rows keeps
     // one query row per workgroup, the form the tiled kernel is validated against).
     static const bool prefill_rows = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return e && e[0] == 'r'; }();
-    if (max_span != 0 && !prefill_rows && levels->tq2_affine_levels && prefill_mfma_supported(p, ptrs)) {
+    static const bool prefill_old = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return e && e[0] == 'o'; }();
+    if (max_span != 0 && !prefill_rows && !prefill_old && prefill_tile_supported(p, ptrs)) {
+        const int rl = launch_prefill_tile(ctx, op, ptrs, p, max_span, ws_avail);
+        if (rl != LH_OK) return rl;
+    } else if (max_span != 0 && !prefill_rows && levels->tq2_affine_levels && prefill_mfma_supported(p, ptrs)) {
         const int rl = launch_prefill_mfma(ctx, op, ptrs, p, max_span, ws_avail);
         if (rl != LH_OK) return rl;
     } else if (max_span == 0 || !mfma_supported(p, ptrs)) {

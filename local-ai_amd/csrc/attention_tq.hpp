@@ -59,4 +59,9 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
 bool prefill_mfma_supported(const AttnParams& p, const AttnPointers& a);
 int launch_prefill_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats);
 
+// The sixteen-row tiled prefill kernel (attention_tq_prefill_tile.hip): K and V levels as f16 through LDS, any level table.
+// Takes 2-bit codes, head_dim 256, at most 8 query heads per KV head, ring absent or a multiple of 64 slots, two rows or more.
+bool prefill_tile_supported(const AttnParams& p, const AttnPointers& a);
+int launch_prefill_tile(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats);
+
 }  // namespace lh_attn

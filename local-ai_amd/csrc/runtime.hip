@@ -165,11 +165,11 @@ int lh_context_create(int device_index, lh_context** out) {
         delete ctx;
         return lh_fail(LH_ERR_NO_COMMAND_QUEUE, "hipStreamCreate");
     }
-    ctx->workspace_bytes = (size_t)64 << 20;
+    ctx->workspace_bytes = (size_t)128 << 20;
     if (hipMalloc(&ctx->workspace, ctx->workspace_bytes) != hipSuccess) {
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;
-        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: attention workspace", (size_t)64 << 20);
+        return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: attention workspace", ctx->workspace_bytes);
     }
     if (hipHostMalloc(&ctx->desc_pinned, lh_context::kDescSlots * lh_context::kDescSlotBytes, hipHostMallocDefault) != hipSuccess) {
         (void)hipFree(ctx->workspace);
