@@ -435,16 +435,16 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
                             (const uint8_t*)v_codes->ptr, (const uint16_t*)v_norms->ptr, (const float*)levels->ptr,
                             positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, ws};
-    // Prefill entries with more than one row: eight rows share a pass over the codes when the kernel for that takes the
-    // shape and the level table was uploaded as one that is affine in the code bits (LOCAL_HIP_ATTN_PREFILL=rows keeps
-    // one query row per workgroup, the form the tiled kernel is validated against).
-    static const bool prefill_rows = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return e && e[0] == 'r'; }();
-    static const bool prefill_old = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return e && e[0] == 'o'; }();
-    if (max_span != 0 && !prefill_rows && !prefill_old && prefill_tile_supported(p, ptrs)) {
+    // Prefill entries with more than one row.  Sixteen rows sharing a pass over the codes (the tiled kernel) pay when there
+    // is enough work to keep its eight-wave workgroups busy: measured against one query row per workgroup it wins from about
+    // 1.5 M (row, position) pairs on (256 rows over 8k positions: 50 against 60 us; over 32k: 118 against 192) and loses
+    // below (64 rows over 8k: 36 against 28 us; 256 rows over a 512-position window: 35 against 21), where a launch is
+    // latency and the per-row form has the shorter chain per workgroup.  LOCAL_HIP_ATTN_PREFILL=rows / =tiled take one
+    // form for every launch it supports (each is validated against the oracle that way).
+    static const int prefill_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PREFILL"); return !e ? 0 : e[0] == 'r' ? 1 : e[0] == 't' ? 2 : 0; }();
+    const bool tiled_pays = (uint64_t)p.num_queries * max_span >= 1500000ull;
+    if (max_span != 0 && prefill_env != 1 && (prefill_env == 2 || tiled_pays) && prefill_tile_supported(p, ptrs)) {
         const int rl = launch_prefill_tile(ctx, op, ptrs, p, max_span, ws_avail);
-        if (rl != LH_OK) return rl;
-    } else if (max_span != 0 && !prefill_rows && levels->tq2_affine_levels && prefill_mfma_supported(p, ptrs)) {
-        const int rl = launch_prefill_mfma(ctx, op, ptrs, p, max_span, ws_avail);
         if (rl != LH_OK) return rl;
     } else if (max_span == 0 || !mfma_supported(p, ptrs)) {
         // Enough workgroups to fill the chip (about two per CU), at least 32 positions per workgroup.

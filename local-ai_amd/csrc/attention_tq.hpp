@@ -53,14 +53,9 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a);
 // runs the merge kernel when p.num_splits > 1.
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats);
 
-// The tiled prefill kernel (attention_tq_prefill_mfma.hip): eight query rows per workgroup share one pass over the codes.
-// Takes 2-bit codes, head_dim 256, at most 8 query heads per KV head, ring absent or a multiple of 64 slots, two rows or
-// more; the level table must be affine in the code bits with zero mean (the caller checks the table it uploaded).
-bool prefill_mfma_supported(const AttnParams& p, const AttnPointers& a);
-int launch_prefill_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats);
-
-// The sixteen-row tiled prefill kernel (attention_tq_prefill_tile.hip): K and V levels as f16 through LDS, any level table.
-// Takes 2-bit codes, head_dim 256, at most 8 query heads per KV head, ring absent or a multiple of 64 slots, two rows or more.
+// The tiled prefill kernel (attention_tq_prefill_tile.hip): sixteen query rows per workgroup share one pass over the codes,
+// K and V levels as f16 through LDS, any level table.  Takes 2-bit codes, head_dim 256, at most 8 query heads per KV head,
+// ring absent or a multiple of 64 slots, two rows or more.
 bool prefill_tile_supported(const AttnParams& p, const AttnPointers& a);
 int launch_prefill_tile(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats);
 

@@ -24,6 +24,7 @@
 #include "attention_tq.hpp"
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 using namespace lh_attn;
@@ -31,6 +32,8 @@ using namespace lh_attn;
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
@@ -57,7 +60,7 @@ __device__ __forceinline__ float ld_norm(gptr_t p) {
 struct TileShared {
     uint8_t kt[2][4][8][64][16];           // [buffer][16-position tile][k step][lane]: K levels as f16, B operands as they are read
     uint8_t pw[2][kWaves][2][4][kPwGroup]; // [buffer][row pair][32-position half][k group]: [query of the pair][8 positions] weights as f16, + 16 bytes so that the packed stores spread over the banks
-    uint8_t vt[2][kWaves][kTile][8];       // [buffer][wave][position]: the wave's eight V code bytes
+    uint8_t vt[4][kWaves][kTile][8];       // [tile % 4][wave][position]: the wave's eight V code bytes (a wave may stage tile t + 2 before its phase B of tile t)
     float fsc[2][kRows * kHeads];          // per query: factor for its output sums when its reference moved in this tile
     __attribute__((aligned(16))) uint32_t moved[2][kWaves];   // [row pair]: a reference moved in this tile
     float fin_l[kRows * kHeads], fin_r[kRows * kHeads];
@@ -191,8 +194,8 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
             nv_n = ld_norm(vn0 + (size_t)(pb + vo) * nstride);
         };
         // K codes in kw -> f16 levels in LDS, V codes in vx -> LDS
-        auto stage = [&](uint32_t buf) {
-            *reinterpret_cast<u32x2_t*>(&sh.vt[buf][wave][lane][0]) = vx;
+        auto stage = [&](uint32_t buf, uint32_t vbuf) {
+            *reinterpret_cast<u32x2_t*>(&sh.vt[vbuf][wave][lane][0]) = vx;
             const uint32_t w2[2] = {kw.x, kw.y};
 #pragma unroll
             for (int mm = 0; mm < 2; mm++) {
@@ -212,7 +215,8 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
         };
 
         // ================================================================= phase A: logits and weights of the wave's two rows
-        auto phase_a = [&](uint32_t buf, uint32_t G, bool full) {
+        auto phase_a = [&](uint32_t buf, uint32_t G, auto full_c) {
+            constexpr bool full = decltype(full_c)::value;   // every position of the tile is seen by every row: no masks
             const uint32_t t0 = G << 6;
             // column pcol of 16-position tile q is position 32 * (q / 2) + 2 * pcol + q % 2: a lane's weights of tiles 2s and 2s + 1
             // are neighbours in the V-side operand and leave as one packed store
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
             }
             // d = logit - R per [16-position tile][query 4g + i]; the reference R follows the running maximum lazily
             bool seen[4] = {true, true, true, true};
-            if (!full) {   // positions this lane's row does not see (causal end, window start, the chunk's ends)
+            if constexpr (!full) {   // positions this lane's row does not see (causal end, window start, the chunk's ends)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const uint32_t t = t0 + 32 * (q >> 1) + 2 * pcol + (q & 1);
@@ -249,7 +253,7 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
 #pragma unroll
             for (int q = 0; q < 4; q++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) d[q][i] = seen[q] ? __builtin_fmaf(acc[q][i], kq[q], -R[i]) : -INFINITY;
+                for (int i = 0; i < 4; i++) d[q][i] = (full || seen[q]) ? __builtin_fmaf(acc[q][i], kq[q], -R[i]) : -INFINITY;
             float over = fmaxf(fmaxf(d[0][0], d[0][1]), fmaxf(d[0][2], d[0][3]));
 #pragma unroll
             for (int q = 1; q < 4; q++) over = fmaxf(fmaxf(over, fmaxf(d[q][0], d[q][1])), fmaxf(d[q][2], d[q][3]));
@@ -261,7 +265,7 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
                     float lgv[4], mq = -INFINITY;
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
-                        lgv[q] = seen[q] ? acc[q][i] * kq[q] : -INFINITY;
+                        lgv[q] = (full || seen[q]) ? acc[q][i] * kq[q] : -INFINITY;
                         mq = fmaxf(mq, lgv[q]);
                     }
                     const float rn = fmaxf(R[i], lh_group_max(mq, 16));
@@ -285,13 +289,33 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
                     const float e0 = __builtin_amdgcn_exp2f(d[2 * sx][i]), e1 = __builtin_amdgcn_exp2f(d[2 * sx + 1][i]);
                     l_run[i] += e0 + e1;
                     // the weights carry the value norm; positions 2 * pcol and 2 * pcol + 1 of the half
-                    const uint32_t pk = (uint32_t)lh_f2h(e0 * nvq[2 * sx]) | ((uint32_t)lh_f2h(e1 * nvq[2 * sx + 1]) << 16);
-                    *reinterpret_cast<uint32_t*>(&sh.pw[buf][wave][sx][pcol >> 2][(4 * g + i) * 16 + 4 * (pcol & 3)]) = pk;
+                    const f16x2 pk = __builtin_convertvector((f32x2){e0 * nvq[2 * sx], e1 * nvq[2 * sx + 1]}, f16x2);
+                    *reinterpret_cast<f16x2*>(&sh.pw[buf][wave][sx][pcol >> 2][(4 * g + i) * 16 + 4 * (pcol & 3)]) = pk;
                 }
         };
 
         // ================================================================= phase B: weights x V levels, dims 32 * wave ..
-        auto phase_b = [&](uint32_t buf) {
+        auto phase_b = [&](uint32_t buf, uint32_t vbuf) {
+            const lds8_t vt = (lds8_t)&sh.vt[vbuf][wave][0][0];
+            const uint32_t sh0 = 4 * (pcol >> 3);   // bit position of field 2 * (pcol / 8)
+            // V levels of code byte 8 * wave + pcol % 8, fields 2 * (pcol / 8) + fp, positions 32s + 8g + j, j = 0 .. 7 (byte j of
+            // the pair z): the lanes 2j and 2j + 1 of a block of 16 both name position j, so that the lanes below and from 8
+            // receive the same bytes
+            auto v_levels = [&](int s, f16x8 (&bop)[2]) {
+                const v2i z = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_t)(vt + (32 * s + 8 * g + (pcol >> 1)) * 8));
+#pragma unroll
+                for (int fp = 0; fp < 2; fp++) {
+                    uint32_t d[4];
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) {
+                        const uint32_t c = ((uint32_t)z[hh] >> (sh0 + 2 * fp)) & 0x03030303u;
+                        const uint32_t lo = __builtin_amdgcn_perm(0u, tl, c), hi = __builtin_amdgcn_perm(0u, th, c);
+                        d[2 * hh] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+                        d[2 * hh + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+                    }
+                    bop[fp] = __builtin_bit_cast(f16x8, (u32x4_t){d[0], d[1], d[2], d[3]});
+                }
+            };
             {   // a reference of some row pair moved: its sums follow (rare after a chunk's first tiles; one look at all eight flags)
                 const u32x4_t m0 = *reinterpret_cast<const u32x4_t*>(&sh.moved[buf][0]), m1 = *reinterpret_cast<const u32x4_t*>(&sh.moved[buf][4]);
                 const uint32_t flags[kWaves] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
@@ -309,26 +333,10 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
                     }
                 }
             }
-            const lds8_t vt = (lds8_t)&sh.vt[buf][wave][0][0];
-            const uint32_t sh0 = 4 * (pcol >> 3);   // bit position of field 2 * (pcol / 8)
 #pragma unroll
             for (int s = 0; s < 2; s++) {
-                // code byte 8 * wave + pcol % 8 of positions 32s + 8g + j, j = 0 .. 7 (byte j of the pair z): the lanes 2j and
-                // 2j + 1 of a block of 16 both name position j, so that the lanes below and from 8 receive the same bytes
-                const v2i z = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i_t)(vt + (32 * s + 8 * g + (pcol >> 1)) * 8));
                 f16x8 bop[2];
-#pragma unroll
-                for (int fp = 0; fp < 2; fp++) {
-                    uint32_t d[4];
-#pragma unroll
-                    for (int hh = 0; hh < 2; hh++) {
-                        const uint32_t c = ((uint32_t)z[hh] >> (sh0 + 2 * fp)) & 0x03030303u;
-                        const uint32_t lo = __builtin_amdgcn_perm(0u, tl, c), hi = __builtin_amdgcn_perm(0u, th, c);
-                        d[2 * hh] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
-                        d[2 * hh + 1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
-                    }
-                    bop[fp] = __builtin_bit_cast(f16x8, (u32x4_t){d[0], d[1], d[2], d[3]});
-                }
+                v_levels(s, bop);
 #pragma unroll
                 for (int mt = 0; mt < kWaves; mt++) {
                     // (row pairs past the end of the chunk multiply whatever their part of LDS holds: never stored)
@@ -349,20 +357,39 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
             v_down = ok ? __uint_as_float((254u << 23) - e) : 1.0f;
             v_up = ok ? __uint_as_float(e) : 1.0f;
         }
-        stage(0);
+        stage(0, 0);
         nk_c = nk_n; nv_c = nv_n;
         if (g_last > g_first) load_tile(g_first + 1);
         __syncthreads();
-        for (uint32_t G = g_first; G <= g_last; G++) {
+        // produce(G): weights of tile G, then tile G + 1 staged (its buffers were last read before the previous barrier)
+        auto produce = [&](uint32_t G) {
             const uint32_t buf = (G - g_first) & 1;
-            if (pair_on) phase_a(buf, G, tile_full(G));
+            if (pair_on) {
+                if (tile_full(G)) phase_a(buf, G, std::true_type{});
+                else phase_a(buf, G, std::false_type{});
+            }
             if (G < g_last) {
-                stage(buf ^ 1);                 // tile G + 1: its buffers were last read before the previous barrier
+                stage(buf ^ 1, (G + 1 - g_first) & 3);
                 nk_c = nk_n; nv_c = nv_n;
                 if (G + 1 < g_last) load_tile(G + 2);
             }
-            __syncthreads();                    // levels of tile G + 1 and weights of tile G are in LDS
-            phase_b(buf);
+        };
+        // Between two barriers a wave owes phase B of tile G and the production of tile G + 1, in either order (they touch
+        // different buffers).  The upper four waves take them the other way round, so that the two waves of a SIMD are not
+        // both in the same phase at the same time.
+        const bool b_first = wave < 4;
+        produce(g_first);
+        __syncthreads();                        // levels of tile G + 1 and weights of tile G are in LDS
+        for (uint32_t G = g_first; G <= g_last; G++) {
+            const uint32_t buf = (G - g_first) & 1;
+            if (b_first) {
+                phase_b(buf, (G - g_first) & 3);
+                if (G < g_last) produce(G + 1);
+            } else {
+                if (G < g_last) produce(G + 1);
+                phase_b(buf, (G - g_first) & 3);
+            }
+            if (G < g_last) __syncthreads();
         }
     }
 

@@ -39,7 +39,7 @@ struct lh_context {
     uint32_t* fault_dev;   // the same word as the device addresses it
 };
 // Kernel-reported fault codes (lh_context::fault_host).
-enum : uint32_t { LH_FAULT_TQ2_SPLIT_WAIT = 1, LH_FAULT_PREFILL_LEVELS = 2 };
+enum : uint32_t { LH_FAULT_TQ2_SPLIT_WAIT = 1 };
 // Reads and clears the context's fault word after a completed wait; LH_OK when no kernel reported anything.
 int lh_check_fault_word(lh_context* ctx);
 
@@ -49,10 +49,6 @@ struct lh_buffer {
     size_t len;
     bool owns;
     size_t slack;   // readable bytes behind ptr + len (allocation padding, or the rest of a viewed parent)
-    // Set when the buffer's first 16 bytes were uploaded from host memory and are a 2-bit level table that is affine in the
-    // code bits (every symmetric table): the tiled prefill attention only takes such tables and asks here, because the
-    // table itself is device data.  The kernel checks the table again and reports a mismatch through the fault word.
-    bool tq2_affine_levels = false;
 };
 
 struct lh_batch {

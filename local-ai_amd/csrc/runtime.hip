@@ -94,24 +94,11 @@ int lh_upload_descriptors(lh_context* ctx, const void* host, size_t bytes, void*
     return LH_OK;
 }
 
-// A 2-bit level table L[c] = alpha + beta * bit0(c) + gamma * bit1(c) up to float noise (the attention kernels' own test).
-static bool levels_affine_in_bits(const void* src, size_t len) {
-    if (len < 16) return false;
-    float L[4];
-    memcpy(L, src, sizeof L);
-    const float d_raw = (L[3] - L[2]) - (L[1] - L[0]);
-    const float lmax = fmaxf(fmaxf(fabsf(L[0]), fabsf(L[1])), fmaxf(fabsf(L[2]), fabsf(L[3])));
-    return lmax > 0.0f && fabsf(d_raw) <= 1e-5f * lmax;   // false for NaN too
-}
-
 int lh_check_fault_word(lh_context* ctx) {
     volatile uint32_t* w = ctx->fault_host;
     const uint32_t code = w ? *w : 0u;
     if (code == 0) return LH_OK;
     *w = 0;
-    if (code == LH_FAULT_PREFILL_LEVELS)
-        return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: flash_attention_tq_prefill: the level table on the device is not the one that was "
-                                              "uploaded into its buffer; the outputs of this batch are not valid");
     if (code == LH_FAULT_TQ2_SPLIT_WAIT)
         return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: a wave gave up waiting for the partial rows of its tile; "
                                               "the outputs of this batch are not valid");
@@ -295,7 +282,6 @@ int lh_buffer_from_bytes(lh_context* ctx, const void* src, size_t len, lh_buffer
     if (e == hipSuccess && len) e = hipMemcpyAsync((*out)->ptr, src, len, hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);  // src may be freed by the caller on return
     if (e != hipSuccess) { lh_buffer_free(*out); *out = nullptr; return lh_fail(LH_ERR_BUFFER_ALLOCATION, "size=%zu: %s", len, hipGetErrorString(e)); }
-    (*out)->tq2_affine_levels = levels_affine_in_bits(src, len);
     return LH_OK;
 }
 
@@ -349,7 +335,6 @@ int lh_buffer_write(lh_buffer* buf, size_t offset, const void* src, size_t len) 
     hipError_t e = hipMemcpyAsync((char*)buf->ptr + offset, src, len, hipMemcpyHostToDevice, buf->ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(buf->ctx->stream);
     if (e != hipSuccess) return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: buffer_write: %s", hipGetErrorString(e));
-    if (offset < 16) buf->tq2_affine_levels = offset == 0 && levels_affine_in_bits(src, len);
     return LH_OK;
 }
 

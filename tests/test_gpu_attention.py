@@ -2,8 +2,6 @@
 Mirrors local-metal/src/kernels.rs:9936-10125 (fused vs dequant-then-flash), 10126-10456
 (prefill vs per-row decode, tiled vs non-tiled), 10457 (batched) and
 local-engine/src/kv_cache/quant_cache.rs:1047-1107 (ring == full)."""
-import os
-
 import numpy as np
 import pytest
 
@@ -285,17 +283,19 @@ def test_prefill_matches_per_row_decode(pkg, gpu, oracle, tiled, hd, nq, nkv, bi
 
 @pytest.mark.parametrize("nq,nkv,start,rows,window,ring,qscale", [
     (8, 1, 0, 256, 0, 0, 0.5),          # a whole first chunk: every row's range ends inside the tiles (causal masks everywhere)
-    (8, 1, 1000, 61, 0, 0, 1.0),        # rows not a multiple of the eight a workgroup takes; chunk ends inside a tile
+    (8, 1, 1000, 61, 0, 0, 1.0),        # rows not a multiple of the sixteen a workgroup takes; chunk ends inside a tile
     (8, 1, 2000, 40, 512, 512, 0.5),    # sliding window over a wrapped 512-slot ring: both ends of the range move with the row
     (4, 2, 300, 19, 0, 0, 1.0),         # two KV heads, two query heads each (padded MFMA rows)
     (8, 1, 5, 9, 3, 0, 1.0),            # a window shorter than the rows per workgroup: rows that share no position
+    (8, 1, 6000, 256, 0, 0, 1.0),       # large enough for the tiled kernel by default (256 rows over 6k positions)
     (8, 1, 777, 2, 0, 0, 0.05),         # two rows, nearly flat scores
 ])
 def test_prefill_tiled_rows_share_a_pass(pkg, gpu, oracle, nq, nkv, start, rows, window, ring, qscale):
-    """The tiled prefill kernel (eight query rows per workgroup over one pass of the codes, shaders/attention_flash_tq.metal:
-    425-556): every row against the f64 code-space oracle at that row's position, the reference's own check of its tiled
-    kernel against per-row decode (kernels.rs:10295) at the attention tolerance.  The output buffer is pre-filled and has
-    guard words behind it."""
+    """The tiled prefill entry (shaders/attention_flash_tq.metal:425-567): every row against the f64 code-space oracle at
+    that row's position, the reference's own check of its tiled kernel against per-row decode (kernels.rs:10295) at the
+    attention tolerance.  The output buffer is pre-filled and has guard words behind it.  By default the entry gives
+    launches of this size to the per-row kernel; under LOCAL_HIP_ATTN_PREFILL=tiled (tests/test_gpu_switches.py) the same
+    cases run on the kernel that shares a pass over the codes among sixteen rows."""
     print(f"case tiled prefill nq={nq} nkv={nkv} start={start} rows={rows} window={window} ring={ring}", flush=True)
     ctx, K = gpu
     hd, bits = 256, 2
@@ -321,8 +321,7 @@ def test_prefill_tiled_rows_share_a_pass(pkg, gpu, oracle, nq, nkv, start, rows,
 def test_prefill_tiled_last_chunk_of_a_32k_prompt(pkg, gpu, oracle):
     """The measured prefill shape: the last 256 rows of a 32768-token prompt (each row sees 32513 .. 32768 positions).
     Sixteen rows spread over the chunk against the f64 oracle; all rows finite; and the rows the tiled kernel produced
-    against the per-row path on the same inputs (LOCAL_HIP_ATTN_PREFILL cannot be switched inside a process, so the
-    per-row figures come from the single-query entry at each sampled row's position)."""
+    (a launch of this size takes it by default) against the single-query entry at each sampled row's position."""
     ctx, K = gpu
     hd, nq, nkv, bits, T, rows = 256, 8, 1, 2, 32768, 256
     start = T - rows
@@ -347,9 +346,9 @@ def test_prefill_tiled_last_chunk_of_a_32k_prompt(pkg, gpu, oracle):
 
 
 def test_prefill_with_a_level_table_that_is_not_affine(pkg, gpu, oracle):
-    """A level table that is not affine in the code bits (the tiled kernel's K side assumes it is): the entry must take
-    the per-row path, which carries a third bit plane, and still match the oracle.  And a table that was affine when it
-    was uploaded but is overwritten on the device afterwards must be reported at the wait, not multiplied with."""
+    """A level table that is not affine in the code bits (the per-row kernel carries a third bit plane for it, the tiled
+    kernel looks levels up in the table itself): both prefill entries must follow whatever table the buffer holds, also
+    one that is written on the device after the upload."""
     ctx, K = gpu
     hd, nq, nkv, bits, start, rows = 256, 8, 1, 2, 50, 12
     T = start + rows
@@ -360,25 +359,19 @@ def test_prefill_with_a_level_table_that_is_not_affine(pkg, gpu, oracle):
     kcb, knb, vcb, vnb, lvb, rqb, oddb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, odd)
     out = pkg.Buffer.empty(ctx, rq.nbytes)
     batch = pkg.CommandBatch(ctx)
-    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, oddb, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
-    batch.commit_and_wait()
-    got = out.as_array(np.float32).reshape(rows, nq * hd)
-    for r in range(rows):
-        ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, odd, hd, T, start + r, nq, nkv, 0, bits, 0)
-        check(got[r], ref, f"row {r}, non-affine table")
-    # device-side overwrite of an uploaded affine table: blit the odd table over it
-    batch.blit_copy(oddb, 0, lvb, 0, 16)
-    K.flash_attention_tq_prefill_tiled_into(batch, rqb, kcb, knb, vcb, vnb, lvb, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
-    if os.environ.get("LOCAL_HIP_ATTN_PREFILL") == "rows":      # the per-row path takes any table: nothing to report
-        batch.commit_and_wait()
-        got = out.as_array(np.float32).reshape(rows, nq * hd)
-        for r in range(rows):
-            ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, odd, hd, T, start + r, nq, nkv, 0, bits, 0)
-            check(got[r], ref, f"row {r}, table overwritten on the device")
-        return
-    with pytest.raises(pkg.CommandBuffer, match="level table"):
-        batch.commit_and_wait()
-    batch.commit_and_wait()      # the report clears the fault word
+
+    def run_and_check(table_buf, what):
+        for fn in (K.flash_attention_tq_prefill_tiled_into, K.flash_attention_tq_prefill_into):
+            fn(batch, rqb, kcb, knb, vcb, vnb, table_buf, out, hd, T, start, rows, nq, nkv, 0, bits, 0)
+            batch.commit_and_wait()
+            got = out.as_array(np.float32).reshape(rows, nq * hd)
+            for r in range(rows):
+                ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, odd, hd, T, start + r, nq, nkv, 0, bits, 0)
+                check(got[r], ref, f"row {r}, {what}")
+
+    run_and_check(oddb, "non-affine table as uploaded")
+    batch.blit_copy(oddb, 0, lvb, 0, 16)      # an uploaded symmetric table overwritten on the device
+    run_and_check(lvb, "table overwritten on the device")
 
 
 @pytest.mark.parametrize("hd", [256, 512])

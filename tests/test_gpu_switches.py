@@ -1,6 +1,7 @@
 """The launch forms that only an environment switch selects against the oracle: the fallback kernels (vector-ALU TQ2_0
-matvec, vector-ALU attention, per-row prefill attention) that otherwise run only for shapes the matrix-core kernels do
-not take, and the test aid that forces the attention kernel's paired hand-overs onto short chunks.  Each case runs a few
+matvec, vector-ALU attention) that otherwise run only for shapes the matrix-core kernels do not take, the two prefill
+attention kernels each on every prefill case (by default the launch size decides between them), and the test aid that
+forces the attention kernel's paired hand-overs onto short chunks.  Each case runs a few
 of the ordinary parity tests in a child process with the switch set -- the library reads its switches once per
 process.  One child at a time; a child takes a few seconds."""
 import os
@@ -17,6 +18,7 @@ CASES = [
     ({"LOCAL_HIP_TQ2_KERNEL": "valu"}, "test_gpu_matvec.py", "baseline_configs or soa or reference_payloads"),
     ({"LOCAL_HIP_ATTN_KERNEL": "valu"}, "test_gpu_attention.py", "asymmetric_levels or empty_range or ring_matches or rotated_entry"),
     ({"LOCAL_HIP_ATTN_PREFILL": "rows"}, "test_gpu_attention.py", "prefill"),
+    ({"LOCAL_HIP_ATTN_PREFILL": "tiled"}, "test_gpu_attention.py", "prefill"),
     # hand-overs of two groups forced onto every chunk length (missing and partial groups at both chunk ends), and never used
     ({"LOCAL_HIP_ATTN_PAIR": "1"}, "test_gpu_attention.py", "decode_attention_matches or prefill_matches or batched_matches or "
      "split_invariance or ring_matches or asymmetric_levels or empty_range or attention_sink or randomised_shapes"),
