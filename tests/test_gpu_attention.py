@@ -318,6 +318,52 @@ def test_prefill_tiled_rows_share_a_pass(pkg, gpu, oracle, nq, nkv, start, rows,
     print(f"worst row: {worst:.2e} of max|ref|")
 
 
+def test_prefill_randomised_shapes_match_oracle(pkg, gpu, oracle):
+    """Forty random prefill launches at head_dim 256 over caches of random code bytes and norms: 2 .. 40 rows (whole and
+    partial groups of sixteen, odd counts), 1, 4, 6 or 8 query heads per KV head over one or two KV heads, chunks that
+    start at position 0 or deep in the context, ends on and off the 64-position tile boundaries, windows shorter and longer
+    than the chunk, wrapped rings, peaked to nearly uniform queries, and now and then a level table with a third-plane
+    term.  Every row against the f64 oracle.  (Launches of this size take the per-row kernel by default and the
+    sixteen-row kernel under LOCAL_HIP_ATTN_PREFILL=tiled; tests/test_gpu_switches.py runs this test both ways.)"""
+    ctx, K = gpu
+    hd, bits = 256, 2
+    worst = 0.0
+    for case in range(40):
+        g = np.random.default_rng(7000 + case)
+        nkv = int(g.choice([1, 1, 2]))
+        nq = nkv * int(g.choice([8, 8, 4, 1, 6]))
+        rows = int(g.choice([2, 5, 15, 16, 17, 31, 33, 40]))
+        T = rows + int(g.choice([0, 1, 47, 63, 64, 65, 200, 511, 700, 1500, 3000])) + int(g.integers(0, 3))
+        start = T - rows
+        window = int(g.choice([0, 0, 3, 64, 100, 512, 1024]))
+        ring = 0
+        if window and g.random() < 0.5:
+            ring = ((window + rows + 63) // 64) * 64 * int(g.choice([1, 2]))     # a ring holds the window of every row of the chunk
+        qscale = float(g.choice([1.0, 0.3, 0.1, 0.02])) / 16
+        levels = oracle.tq_levels(hd, bits)
+        if g.random() < 0.2:
+            levels = levels.copy(); levels[3] += 0.2
+        cb = oracle.tq_code_bytes(hd, bits)
+        phys = ring if ring else T
+        kc = g.integers(0, 256, (phys, nkv, cb), dtype=np.uint8); vc = g.integers(0, 256, (phys, nkv, cb), dtype=np.uint8)
+        kn = (g.random((phys, nkv), dtype=np.float32) * 4 + 14).astype(np.float16).view(np.uint16)
+        vn = (g.random((phys, nkv), dtype=np.float32) * 4 + 14).astype(np.float16).view(np.uint16)
+        what = f"case {case}: rows={rows} nq={nq} nkv={nkv} T={T} window={window} ring={ring}"
+        print(what, flush=True)
+        rq = g.standard_normal((rows, nq * hd), dtype=np.float32) * qscale
+        b = upload(pkg, ctx, kc, kn, vc, vn, levels, rq)
+        out = pkg.Buffer.empty(ctx, rq.nbytes)
+        batch = pkg.CommandBatch(ctx)
+        K.flash_attention_tq_prefill_tiled_into(batch, b[5], b[0], b[1], b[2], b[3], b[4], out, hd, T, start, rows, nq, nkv, window,
+                                                bits, ring)
+        batch.commit_and_wait()
+        got = out.as_array(np.float32).reshape(rows, nq * hd)
+        for r in range(rows):
+            ref = oracle.attention_tq_codespace(rq[r], kc, kn, vc, vn, levels, hd, T, start + r, nq, nkv, window, bits, ring)
+            worst = max(worst, check(got[r], ref, f"{what}, row {r}"))
+    print(f"worst error / scale {worst:.2e}")
+
+
 def test_prefill_tiled_last_chunk_of_a_32k_prompt(pkg, gpu, oracle):
     """The measured prefill shape: the last 256 rows of a 32768-token prompt (each row sees 32513 .. 32768 positions).
     Sixteen rows spread over the chunk against the f64 oracle; all rows finite; and the rows the tiled kernel produced
