@@ -159,17 +159,30 @@ __device__ __forceinline__ void load_raw_bt(RawBT& r, const uint8_t* W, uint32_t
     r.d = *reinterpret_cast<const uint16_t*>(bp + 64);
     __builtin_memcpy(&r.q, __builtin_assume_aligned(bp + ((k0 >> 7) & 1) * 32 + 16 * part, 2), 16);
 }
+// The four values a TQ2_0 code can take in a block of scale d, d * (c - 1) for c = 0 .. 3, as two byte tables for v_perm_b32
+// (byte c of lo / hi = low / high byte of the f16 value).  The products of d with -1, 0, 1 and 2 are exact in f16 (or the
+// infinity, NaN or signed zero the CPU path's f32 product rounds to: qat_recover.rs:39-47), so looking a code up gives the
+// CPU path's dequantised weight bit for bit -- with six instructions per four codes where (1024 + c - 1025) * d takes eight.
+struct Tq2Table { uint32_t lo, hi; };
+__device__ __forceinline__ Tq2Table tq2_table(uint32_t d2) {   // d2: the f16 scale in both halves
+    const f16x2 dd = __builtin_bit_cast(f16x2, d2);
+    const uint32_t t01 = __builtin_bit_cast(uint32_t, dd * (f16x2){(_Float16)-1.0f, (_Float16)0.0f});
+    const uint32_t t23 = __builtin_bit_cast(uint32_t, dd * (f16x2){(_Float16)1.0f, (_Float16)2.0f});
+    return {__builtin_amdgcn_perm(t23, t01, 0x06040200u), __builtin_amdgcn_perm(t23, t01, 0x07050301u)};
+}
+// Four codes (one per byte of c, each 0 .. 3) -> their f16 values: bytes 0, 1 in w0, bytes 2, 3 in w1.
+__device__ __forceinline__ void tq2_lookup(const Tq2Table& t, uint32_t c, uint32_t& w0, uint32_t& w1) {
+    const uint32_t lo = __builtin_amdgcn_perm(0u, t.lo, c), hi = __builtin_amdgcn_perm(0u, t.hi, c);
+    w0 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+    w1 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+}
 // f16 values of field f: 16 consecutive k as 8 words
 __device__ __forceinline__ void convert_bt(uint32_t (&w)[8], const RawBT& r, int f, bool valid) {
     const uint32_t d = valid ? r.d : 0u;
-    const uint32_t d2 = (d & 0xFFFFu) | (d << 16);
+    const Tq2Table t = tq2_table((d & 0xFFFFu) | (d << 16));
     const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t c = (q[i] >> (2 * f)) & 0x03030303u;
-        w[2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04010400u), 0x64016401u, d2);            // 1024 + c - 1025
-        w[2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04030402u), 0x64016401u, d2);
-    }
+    for (int i = 0; i < 4; i++) tq2_lookup(t, (q[i] >> (2 * f)) & 0x03030303u, w[2 * i], w[2 * i + 1]);
 }
 
 // Elements k0 .. k0 + 32 of weight row `row` (k0 a multiple of 32).
@@ -219,14 +232,11 @@ __device__ __forceinline__ void convert_b(uint32_t (&f)[16], const RawB<FMT>& r,
         }
     } else {
         const uint32_t d = valid ? r.d : 0u;
-        const uint32_t d2 = (d & 0xFFFFu) | (d << 16), sh = ((k0 >> 5) & 3) * 2;
+        const uint32_t sh = ((k0 >> 5) & 3) * 2;
+        const Tq2Table t = tq2_table((d & 0xFFFFu) | (d << 16));
         const uint32_t q[8] = {r.q[0].x, r.q[0].y, r.q[0].z, r.q[0].w, r.q[1].x, r.q[1].y, r.q[1].z, r.q[1].w};
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t c = (q[i] >> sh) & 0x03030303u;
-            f[2 * i] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04010400u), 0x64016401u, d2);            // 1024 + c - 1025
-            f[2 * i + 1] = h2_sub_mul(__builtin_amdgcn_perm(0x64646464u, c, 0x04030402u), 0x64016401u, d2);
-        }
+        for (int i = 0; i < 8; i++) tq2_lookup(t, (q[i] >> sh) & 0x03030303u, f[2 * i], f[2 * i + 1]);
     }
 }
 
@@ -679,6 +689,14 @@ __device__ __forceinline__ uint2 ld8_align2(const uint8_t* p) {
 
 template <int FMT>
 __device__ __forceinline__ f16x8 skinny_fragment(const SkinnyRaw& raw, int f) {
+    if constexpr (FMT == kTQ2) {   // the block's four values looked up (tq2_table): the same bits with fewer instructions
+        const Tq2Table t = tq2_table(raw.d);
+        uint32_t o[4];
+        tq2_lookup(t, (raw.w0 >> (2 * f)) & 0x03030303u, o[0], o[1]);
+        tq2_lookup(t, (raw.w1 >> (2 * f)) & 0x03030303u, o[2], o[3]);
+        struct { uint32_t v[4]; } tt = {{o[0], o[1], o[2], o[3]}};
+        return __builtin_bit_cast(f16x8, tt);
+    }
     uint32_t c0, c1;
     f16x2 zp;
     if constexpr (FMT == kQ4) { c0 = (raw.w0 >> (4 * f)) & 0x0F0F0F0Fu; c1 = (raw.w1 >> (4 * f)) & 0x0F0F0F0Fu; zp = (f16x2){(_Float16)1032.0f, (_Float16)1032.0f}; }
