@@ -477,7 +477,7 @@ def fill_kv(pkg, ctx, K, cache, lanes, T, g):
     batch.commit_and_wait()
 
 
-def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3, graphs=True):
+def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3, graphs=True, defer=True):
     """Whole decoder layers end to end (norms, Q/K/V projections, RoPE, KV encode, attention over the tq2 cache,
     output projection, GeGLU feed-forward, per-layer input injection) at hidden 2048, FFN 8192, 8 query heads over
     1 KV head of 256, Q4_0 attention and TQ2_0 feed-forward weights, context T.  A step runs `n_layers` distinct
@@ -500,7 +500,7 @@ def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, l
     batch = pkg.CommandBatch(ctx)
     kv_bytes = T * (2 * 64 + 4)
     if "single" in which:
-        res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs)
+        res["single"] = _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs, defer)
     if "chunk" in which:
         res["prefill_chunk"] = _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g)
     if "lanes" in which:
@@ -540,7 +540,7 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     return res
 
 
-def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64):
+def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64, defer_tail=True):
     """End-to-end decode of a synthetic model with the geometry of the reference's Gemma 4 E2B configuration
     (local-core/src/config/gemma4_qat.rs:262-283: vocabulary 262144, hidden 1536, 35 layers in a sliding x4 / full
     pattern with head_dim 256 / 512, window 512, the last 20 layers sharing KV, per-layer inputs of 256; Q4_0
@@ -568,6 +568,7 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64):
     tensors["layers"] = [kinds[(cfg.is_full_attention(i), cfg.is_kv_shared(i))] for i in range(35)]
     max_ctx = T + 256
     pipe = P.DecodePipeline.from_host(ctx, K, cfg, tensors, max_ctx)
+    pipe.defer_layer_tails = defer_tail
     del tensors, one, kinds
     if single:
         for i, c in enumerate(pipe.kv_caches):
@@ -631,7 +632,7 @@ def _layer_weight_bytes(pkg, layer):
     return sum(w.device_bytes() for w in vars(layer.weights).values() if isinstance(w, pkg.QuantWeight))
 
 
-def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs):
+def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch, batch, g, kv_bytes, graphs, defer=True):
     pld = 256
     layers = [make_layer(i) for i in range(n_layers)]
     wbytes = _layer_weight_bytes(pkg, layers[0])
@@ -645,10 +646,17 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
     x0 = pkg.Buffer.from_slice(ctx, hidden[0].as_array(np.float16, 2048))
     ple = pkg.Buffer.from_slice(ctx, g.standard_normal(n_layers * pld, dtype=np.float32).astype(np.float16))
 
-    def step_single():
+    final = {"buf": 0}
+
+    def step_single():   # as DecodePipeline.forward_token_turbo chains its layers
         batch.blit_copy(x0, 0, hidden[0], 0, 4096)
+        cur, pend = 0, None
         for i, layer in enumerate(layers):
-            layer.forward_decode(K, batch, hidden[i & 1], hidden[(i + 1) & 1], T - 1, scratch, caches[i], ple, n_layers)
+            pend = layer.forward_decode(K, batch, hidden[cur], hidden[cur ^ 1], T - 1, scratch, caches[i], ple, n_layers,
+                                        pending=pend, defer_tail=defer and i + 1 < len(layers))
+            if pend is None:
+                cur ^= 1
+        final["buf"] = cur
 
     d0 = batch.dispatch_count()
     step_single()
@@ -661,7 +669,7 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
         step_single()
         host.append(time.perf_counter() - t0)
     ctx.synchronize()
-    out = hidden[n_layers & 1].as_array(np.float16, 2048).astype(np.float32)
+    out = hidden[final["buf"]].as_array(np.float16, 2048).astype(np.float32)
     if not np.isfinite(out).all():
         raise RuntimeError("decode step produced non-finite hidden state")
     res = {"layers_per_step": n_layers, "us_per_layer_events": ev * 1e3 / n_layers, "us_per_layer_wall": wall * 1e3 / n_layers,
@@ -834,6 +842,8 @@ def main():
                     help="untimed milliseconds each measured call is run before its warm-up steps, so that the clocks have risen")
     ap.add_argument("--quick", action="store_true", help="headline measurement only")
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
+    ap.add_argument("--no-defer-tail", action="store_true",
+                    help="decode / model legs: every layer dispatches its own last step (default: it rides in the next layer's first dispatch)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model,model_lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time); "
@@ -926,7 +936,7 @@ def main():
     if legs & {"decode", "lanes", "chunk"}:
         which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else []) + \
             (["chunk"] if "chunk" in legs else [])
-        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph)
+        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph, defer=not args.no_defer_tail)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
     if "model_few_lanes" in legs:
@@ -938,7 +948,7 @@ def main():
         log(f"[bench] model decode, few lanes: {extra['model_decode_few_lanes_8k']}")
     if legs & {"model", "model_lanes"}:
         extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup, single="model" in legs,
-                                                         lanes=64 if "model_lanes" in legs else 0)
+                                                         lanes=64 if "model_lanes" in legs else 0, defer_tail=not args.no_defer_tail)
         log("[bench] model decode:", extra["model_decode_e2b_geometry"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6

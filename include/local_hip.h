@@ -201,6 +201,15 @@ LH_API int lh_matvec_quant_norm_chain_into(lh_batch* batch, lh_quant fmt, uint32
                                            const lh_buffer* vector, const lh_buffer* weight, const lh_buffer* residual,
                                            const lh_buffer* next_weight, lh_buffer* store, float eps,
                                            lh_buffer* const* outputs, uint32_t rows, uint32_t cols);
+/* The chain across two layers (layer.rs:503-520 of one layer, 387-392 of the next): the staged vector is the layer
+ * output that rms_norm_residual_scale_into would have written,
+ *   t = f16(f16(f16(rms_norm(vector) * weight) + residual) * scale)     (the scale only with `apply_scale`),
+ * stored once in `store` (required: it is the next layer's input and first residual), then
+ * f16(rms_norm(t) * next_weight) as that layer's attention norm (or t itself when `next_weight` is NULL). */
+LH_API int lh_matvec_quant_norm_chain_tail_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
+                                                const lh_buffer* vector, const lh_buffer* weight, const lh_buffer* residual,
+                                                int apply_scale, float scale, const lh_buffer* next_weight, lh_buffer* store,
+                                                float eps, lh_buffer* const* outputs, uint32_t rows, uint32_t cols);
 LH_API int lh_matvec_quant_fused_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
                                       const lh_buffer* vector, int prologue, const lh_buffer* aux, float eps,
                                       lh_buffer* const* outputs, uint32_t rows, uint32_t cols);

@@ -392,6 +392,16 @@ class Kernels:
                                                        vector._h, weight._h, h(residual), h(next_weight), h(store),
                                                        C.c_float(eps), _handles(outputs), _u32(rows), _u32(cols)))
 
+    def matvec_quant_norm_chain_tail_into(self, batch, fmt, matrices, vector, weight, residual, scale, next_weight, store, eps,
+                                          outputs, rows, cols):
+        """Matvecs against the next layer's attention norm of t = (rms_norm(vector) * weight + residual) * scale, rounded as
+        rms_norm_residual_scale_into rounds it (`scale` None: no scale step); `store` receives t (the layer output)."""
+        _check(self._l.lh_matvec_quant_norm_chain_tail_into(
+            batch._h, C.c_int(fmt), _u32(len(matrices)), _handles(matrices), vector._h, weight._h, residual._h,
+            C.c_int(0 if scale is None else 1), C.c_float(1.0 if scale is None else scale),
+            next_weight._h if next_weight is not None else None, store._h, C.c_float(eps), _handles(outputs), _u32(rows),
+            _u32(cols)))
+
     # -- small-M / prefill matmul (kernels.rs:6378-6563, 5517-5568) --
     def matmul_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))

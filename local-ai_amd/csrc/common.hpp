@@ -99,6 +99,8 @@ struct XPrologue {
     const uint16_t* res = nullptr;
     const uint16_t* aux2 = nullptr;
     uint16_t* store = nullptr;
+    uint32_t tail = 0;      // with `res`: 0 the residual joins the f32 product (rms_norm_add); 1, 2 see lh_norm_tail
+    float scale = 1.0f;
 };
 
 // TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.
@@ -237,6 +239,14 @@ __device__ __forceinline__ float lh_norm_product(float x, float rms, float w) {
     float p = x * rms * w;
     asm volatile("" : "+v"(p));
     return p;
+}
+
+// The end of a per-layer input block as its three kernels round it (layer.rs:503-520: rms_norm, residual_add,
+// scale_in_place): the normalised value is rounded to f16, added to the residual as an f16 addition, and, with tail == 2,
+// scaled (the caller rounds once more).
+__device__ __forceinline__ float lh_norm_tail(float normed, float res, uint32_t tail, float scale) {
+    const _Float16 sum = (_Float16)normed + (_Float16)res;
+    return tail == 2 ? (float)sum * scale : (float)sum;
 }
 
 // In-place unnormalised fast Walsh-Hadamard transform over sh[0..d) in LDS with one thread per element; every thread of

@@ -29,10 +29,7 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 // ADD with `tail` != 0 is the three-kernel tail of the single-token layer in one dispatch (layer.rs:507-520: rms_norm,
 // residual_add, scale_in_place): the normalised value is rounded to f16, added to the residual as an f16 addition, and,
 // with tail == 2, scaled and rounded once more -- the roundings of the three separate kernels.
-__device__ __forceinline__ float norm_tail(float normed, float res, uint32_t tail, float scale) {
-    const _Float16 sum = (_Float16)normed + (_Float16)res;
-    return tail == 2 ? (float)sum * scale : (float)sum;
-}
+__device__ __forceinline__ float norm_tail(float normed, float res, uint32_t tail, float scale) { return lh_norm_tail(normed, res, tail, scale); }
 
 // The arithmetic of one 8-element chunk, shared by every kernel that must reproduce the stand-alone norm bit for bit.
 __device__ __forceinline__ void rms_sumsq8(const uint4& v, float& s) {

@@ -895,6 +895,37 @@ int lh_matvec_quant_norm_chain_into(lh_batch* b, lh_quant fmt, uint32_t count, c
     return matvec_dispatch(b, fmt, count, ms, xs, LH_F16, ys, LH_F16, rows, cols, op, pro);
 }
 
+int lh_matvec_quant_norm_chain_tail_into(lh_batch* b, lh_quant fmt, uint32_t count, const lh_buffer* const* ms, const lh_buffer* x,
+                                         const lh_buffer* weight, const lh_buffer* residual, int apply_scale, float scale,
+                                         const lh_buffer* next_weight, lh_buffer* store, float eps, lh_buffer* const* ys,
+                                         uint32_t rows, uint32_t cols) {
+    const char* op = fmt == LH_Q4_0 ? "matvec_q4_0 (layer tail chain)" : "matvec_tq2_0 (layer tail chain)";
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
+    if (count == 0 || rows == 0 || cols == 0) return LH_OK;
+    if (count > 8) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: at most 8 matrices share one staged vector, got %u", op, count);
+    if (!ms || !ys || !x) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null problem arrays", op);
+    if (cols % 8 != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: cols %u not /8", op, cols);
+    if (!weight || !residual || !store) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: norm weight, residual and stored vector are required", op);
+    const lh_buffer* vecs[4] = {weight, residual, next_weight, store};
+    const char* names[4] = {"norm weight", "residual", "second norm weight", "stored vector"};
+    for (int i = 0; i < 4; i++) {
+        if (!vecs[i]) continue;
+        LH_NEED(vecs[i], (size_t)cols * 2, op, names[i]);
+        LH_REQUIRE(((uintptr_t)vecs[i]->ptr & 15) == 0, "%s: the %s must be 16-byte aligned", op, names[i]);
+    }
+    LH_REQUIRE(store->ptr != x->ptr && store->ptr != residual->ptr, "%s: the stored vector may not alias an input", op);
+    for (uint32_t i = 0; i < count; i++) LH_REQUIRE(ys[i] && store->ptr != ys[i]->ptr, "%s: the stored vector may not alias an output", op);
+    const lh_buffer* xs[8];
+    for (uint32_t i = 0; i < count; i++) xs[i] = x;
+    XPrologue pro{kXProRmsNorm, (const uint16_t*)weight->ptr, eps};
+    pro.res = (const uint16_t*)residual->ptr;
+    pro.aux2 = next_weight ? (const uint16_t*)next_weight->ptr : nullptr;
+    pro.store = (uint16_t*)store->ptr;
+    pro.tail = apply_scale ? 2u : 1u;
+    pro.scale = scale;
+    return matvec_dispatch(b, fmt, count, ms, xs, LH_F16, ys, LH_F16, rows, cols, op, pro);
+}
+
 int lh_matvec_tq2_0_soa_into(lh_batch* b, const lh_buffer* qs, const lh_buffer* scales, const lh_buffer* x, lh_buffer* y,
                              uint32_t rows, uint32_t cols) {
     // kernels.rs:5929-5933

@@ -32,7 +32,8 @@ __device__ __forceinline__ uint16_t lh_gelu_mul_h(uint16_t a, uint16_t b) {
     return lh_f2h(p);
 }
 
-// Elements e0 .. e0 + 8 of f16(x * rms * aux (+ res)) as four packed words: the arithmetic of rms_norm_kernel<ADD>.
+// Elements e0 .. e0 + 8 of f16(x * rms * aux (+ res)) as four packed words: the arithmetic of rms_norm_kernel<ADD>, its
+// tail forms (pro.tail) included.
 __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& pro, uint32_t e0, float rms, uint32_t (&packed)[4]) {
     const uint16_t* x = static_cast<const uint16_t*>(xv);
     const uint4 a = *reinterpret_cast<const uint4*>(x + e0), g = *reinterpret_cast<const uint4*>(pro.aux + e0);
@@ -43,7 +44,11 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
     for (int j = 0; j < 4; j++) {
         float lo = lh_norm_product(lh_h2f((uint16_t)(wa[j] & 0xFFFF)), rms, lh_h2f((uint16_t)(wg[j] & 0xFFFF)));
         float hi = lh_norm_product(lh_h2f((uint16_t)(wa[j] >> 16)), rms, lh_h2f((uint16_t)(wg[j] >> 16)));
-        if (pro.res != nullptr) { lo += lh_h2f((uint16_t)(wr[j] & 0xFFFF)); hi += lh_h2f((uint16_t)(wr[j] >> 16)); }
+        if (pro.res != nullptr) {
+            const float rlo = lh_h2f((uint16_t)(wr[j] & 0xFFFF)), rhi = lh_h2f((uint16_t)(wr[j] >> 16));
+            if (pro.tail) { lo = lh_norm_tail(lo, rlo, pro.tail, pro.scale); hi = lh_norm_tail(hi, rhi, pro.tail, pro.scale); }
+            else { lo += rlo; hi += rhi; }
+        }
         packed[j] = (uint32_t)lh_f2h_exact(lo) | ((uint32_t)lh_f2h_exact(hi) << 16);
     }
 }

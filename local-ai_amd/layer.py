@@ -148,6 +148,16 @@ def _groupable(a: Optional[QuantWeight], b: Optional[QuantWeight]) -> bool:
             and a.rows == b.rows and a.cols == b.cols)
 
 
+@dataclass
+class PendingTail:
+    """The last step of a decoded layer, left for the next layer's first dispatch:
+    hidden = (rms_norm(x) * weight + residual) * scale  (layer.rs:503-520; ``scale`` None: no output scale)."""
+    x: Buffer
+    weight: Buffer
+    residual: Buffer
+    scale: Optional[float]
+
+
 class TransformerLayer:
     """layer.rs:330-873."""
 
@@ -267,9 +277,16 @@ class TransformerLayer:
     # ----------------------------------------------------- single-token decode
     def forward_decode(self, kernels: Kernels, batch, input: Buffer, output: Buffer, position: int,
                        scratch: ScratchBuffers, kv_cache: QuantizedKvCache, per_layer_input: Optional[Buffer] = None,
-                       n_layer_total: int = 0) -> None:
+                       n_layer_total: int = 0, pending: Optional["PendingTail"] = None,
+                       defer_tail: bool = False) -> Optional["PendingTail"]:
         """layer.rs:354-523.  ``kv_cache`` is this layer's cache, or for a KV-shared layer the source layer's
-        (already written earlier in the same step)."""
+        (already written earlier in the same step).
+
+        Two layers can share a dispatch across their boundary: with ``defer_tail`` the last step of this layer (per-layer
+        post-norm, residual #3, output scale: layer.rs:503-520) is not dispatched but returned as a ``PendingTail``; the
+        caller hands it to the next layer as ``pending``, whose first matvec computes it while it stages its input and
+        writes it to ``input`` (which must be neither ``pending.x`` nor ``pending.residual``).  None is returned when the
+        layer ran its last step itself (then ``output`` holds the result)."""
         p, w, s = self.params, self.weights, scratch
         h, hd, n_head, n_kv, eps = p.hidden_size, p.head_dim, p.num_attention_heads, p.num_key_value_heads, p.rms_norm_eps
         pos, seq_len = position, position + 1
@@ -279,11 +296,24 @@ class TransformerLayer:
         fused_in = self._fusable(w.attn_q) and (not own_kv or self._fusable(w.attn_k, w.attn_v))
         q_buf, k_buf, v_buf = s.q, s.k, s.v
         stacked = fused_in and own_kv and self._qkv is not None
+        if pending is not None and not fused_in:   # nothing here can take it along: the previous layer's last step by itself
+            kernels.rms_norm_residual_scale_into(batch, pending.x, pending.weight, pending.residual, input, h, 1, eps, pending.scale)
+            pending = None
         if stacked:   # one matvec over the stacked [Wq; Wk; Wv] writes q | k | v side by side
             q_buf, k_buf, v_buf, qkv_out = self._qkv_views(s)
-            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [self._qkv], [qkv_out])
+            if pending is not None:
+                kernels.matvec_quant_norm_chain_tail_into(batch, self._qkv.ty, [self._qkv.buf], pending.x, pending.weight,
+                                                          pending.residual, pending.scale, w.attn_norm, input, eps, [qkv_out],
+                                                          self._qkv.rows, self._qkv.cols)
+            else:
+                self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [self._qkv], [qkv_out])
         elif fused_in:
-            self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [w.attn_q], [s.q])
+            if pending is not None:   # (the K / V launch below then finds `input` written)
+                kernels.matvec_quant_norm_chain_tail_into(batch, w.attn_q.ty, [w.attn_q.buf], pending.x, pending.weight,
+                                                          pending.residual, pending.scale, w.attn_norm, input, eps, [s.q],
+                                                          w.attn_q.rows, w.attn_q.cols)
+            else:
+                self._fused_matvecs(batch, kernels, kernels.PROLOGUE_RMS_NORM, input, w.attn_norm, [w.attn_q], [s.q])
         else:
             kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
             w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
@@ -360,14 +390,17 @@ class TransformerLayer:
                 kernels.gelu_mul_into(batch, s.ple_h, s.ple, s.ple_h, pld)
                 w.per_layer_proj.matvec_into(batch, kernels, s.ple_h, s.ffn_out)
             if self.fuse_prologues:   # norm, residual #3 and the output scale (step 6) in one dispatch
+                if defer_tail:        # ... or in the next layer's first one
+                    return PendingTail(s.ffn_out, w.per_layer_post_norm, output, self._output_scale)
                 kernels.rms_norm_residual_scale_into(batch, s.ffn_out, w.per_layer_post_norm, output, output, h, 1, eps,
                                                      self._output_scale)
-                return
+                return None
             kernels.rms_norm_into(batch, s.ffn_out, w.per_layer_post_norm, s.normed, h, 1, eps)
             kernels.residual_add_into(batch, output, s.normed, output, h)
 
         # 6. per-layer output scale
         self._scale_output(batch, kernels, output, h)
+        return None
 
     # ------------------------------------------------ shared multi-row tail
     def _attention_tail(self, kernels: Kernels, batch, rows: int, input: Buffer, output: Buffer, bs: BatchScratch,

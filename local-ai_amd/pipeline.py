@@ -163,6 +163,7 @@ class DecodePipeline:
         if ple_table is not None and per_layer_model_proj is not None and per_layer_proj_norm is not None:
             self.per_layer_input, self.ple_tok, self.ple_proj = (Buffer.empty(ctx, ple_total * 2) for _ in range(3))
         self.max_batch = max_batch
+        self.defer_layer_tails = True   # single-token decode: a layer's last step rides in the next layer's first dispatch
         self._batch_scratch: Optional[BatchScratch] = None
         self._tokens_buf = self._ple_tokens_buf = None
         self.position = 0
@@ -255,12 +256,16 @@ class DecodePipeline:
         self.gather_embedding(batch, token, self.hidden_a)
         K.scale_in_place_gpu_into(batch, self.hidden_a, math.sqrt(cfg.hidden_size), cfg.hidden_size)
         self.compute_per_layer_inputs(batch, token if ple_token is None else ple_token)
-        cur_in_a = True
+        # A layer may leave its last step (post-norm, residual, output scale) to the next layer's first dispatch: its input
+        # buffer is dead by then and receives the finished hidden state, so the two buffers keep their roles in that case.
+        cur_in_a, pend, last = True, None, len(self.layers) - 1
         for i, layer in enumerate(self.layers):
             inp, out = (self.hidden_a, self.hidden_b) if cur_in_a else (self.hidden_b, self.hidden_a)
-            layer.forward_decode(K, batch, inp, out, position, self.scratch, self.kv_caches[self.kv_index_map[i]],
-                                 self.per_layer_input, cfg.num_hidden_layers)
-            cur_in_a = not cur_in_a
+            pend = layer.forward_decode(K, batch, inp, out, position, self.scratch, self.kv_caches[self.kv_index_map[i]],
+                                        self.per_layer_input, cfg.num_hidden_layers, pending=pend,
+                                        defer_tail=self.defer_layer_tails and i < last)
+            if pend is None:
+                cur_in_a = not cur_in_a
         if own:
             batch.commit_and_wait()
         return cur_in_a

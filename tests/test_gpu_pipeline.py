@@ -23,9 +23,11 @@ def _config(pkg, pld, head_dims=(128, 256)):
                                         full_partial_rotary_factor=0.25)
 
 
-@pytest.mark.parametrize("pld,fused,head_dims", [(64, True, (128, 256)), (0, True, (128, 256)), (64, False, (128, 256)),
-                                                 (64, True, (256, 512))])   # the last: the reference model's head dims
-def test_decode_steps_match_oracle(pkg, gpu, oracle, pld, fused, head_dims):
+@pytest.mark.parametrize("pld,fused,head_dims,defer", [
+    (64, True, (128, 256), True), (0, True, (128, 256), True), (64, False, (128, 256), True),
+    (64, True, (256, 512), True),      # the reference model's head dims
+    (64, True, (128, 256), False)])    # every layer runs its own last step (by default it rides in the next layer's first dispatch)
+def test_decode_steps_match_oracle(pkg, gpu, oracle, pld, fused, head_dims, defer):
     ctx, K = gpu
     cfg = _config(pkg, pld, head_dims)
     g = pkg.synth.rng(970, pld)
@@ -34,6 +36,7 @@ def test_decode_steps_match_oracle(pkg, gpu, oracle, pld, fused, head_dims):
     options = {} if fused else dict(group_projections=False, fuse_norm_rope=False, fuse_prologues=False, stack_qkv=False)
     max_ctx = 1024
     pipe = pkg.pipeline.DecodePipeline.from_host(ctx, K, cfg, t, max_ctx, **options)
+    pipe.defer_layer_tails = defer
     assert pipe.kv_index_map == [0, 1, 2, 1, 1, 2] and len(pipe.kv_caches) == 3
     assert [c.is_ringed() for c in pipe.kv_caches] == [True, True, False]
     model = OL.model_from_host(cfg, t)
