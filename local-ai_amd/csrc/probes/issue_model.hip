@@ -14,7 +14,8 @@
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp, kValuSgpr, kAndOnlyLit, kAndOnlySgpr };
+enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp, kValuSgpr, kAndOnlyLit, kAndOnlySgpr,
+           kAndVgpr, kMulLit, kMulVgpr, kShiftLit, kShlAdd, kCvt };
 
 // One iteration per wave: 160 (v_and_b32, v_add_u32) pairs = 320 vector instructions and / or 16 MFMAs (kFine: 80 pairs
 // between 16 MFMAs; kSplitWaves: even waves the 160 pairs, odd waves the 16 MFMAs), or 160 instructions of one other kind.
@@ -89,6 +90,29 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
 #pragma unroll
                 for (int i = 0; i < 8; i++) x[i] = (x[(i + 1) & 7] & mask) ^ x[i];
         }
+        // (the next six are written as single instructions: the compiler would regroup the C forms)
+#define LH_PROBE_160(STMT)                                   \
+        _Pragma("unroll") for (int r = 0; r < 20; r++)       \
+            _Pragma("unroll") for (int i = 0; i < 8; i++) { STMT; }
+        if constexpr (MIX == kAndVgpr) {   // both operands in vector registers
+            LH_PROBE_160(asm volatile("v_and_b32 %0, %0, %1\n\tv_add_u32 %0, %0, %2" : "+v"(x[i]) : "v"(x[(i + 3) & 7]), "v"(x[(i + 5) & 7])))
+        }
+        if constexpr (MIX == kMulLit) {
+            LH_PROBE_160(asm volatile("v_mul_f32 %0, 0x3f800347, %0" : "+v"(f[i])))
+        }
+        if constexpr (MIX == kMulVgpr) {
+            LH_PROBE_160(asm volatile("v_mul_f32 %0, %0, %1" : "+v"(f[i]) : "v"(f[(i + 3) & 7])))
+        }
+        if constexpr (MIX == kShiftLit) {
+            LH_PROBE_160(asm volatile("v_lshrrev_b32 %0, 3, %0\n\tv_xor_b32 %0, 0x5a5a5a5a, %0" : "+v"(x[i])))
+        }
+        if constexpr (MIX == kShlAdd) {
+            LH_PROBE_160(asm volatile("v_lshl_add_u32 %0, %0, 2, %1" : "+v"(x[i]) : "v"(x[(i + 3) & 7])))
+        }
+        if constexpr (MIX == kCvt) {
+            LH_PROBE_160(asm volatile("v_cvt_f32_i32 %0, %0" : "+v"(f[i])))
+        }
+#undef LH_PROBE_160
         if constexpr (MIX == kExp) {
 #pragma unroll
             for (int r = 0; r < 20; r++)
@@ -144,6 +168,12 @@ int main() {
     run<kValuSgpr>("160 x (v_and + v_add), SGPR operands", 320, 0, d);
     run<kAndOnlyLit>("320 v_bitop3/v_xor, literal masks", 320, 0, d);
     run<kAndOnlySgpr>("312 v_bitop3/v_xor, SGPR mask", 312, 0, d);
+    run<kAndVgpr>("160 x (v_and + v_add), two VGPR operands", 320, 0, d);
+    run<kShiftLit>("160 x (v_lshrrev + v_xor), literal operands", 320, 0, d);
+    run<kMulLit>("160 v_mul_f32, literal factor", 160, 0, d);
+    run<kMulVgpr>("160 v_mul_f32, two VGPR operands", 160, 0, d);
+    run<kShlAdd>("160 v_lshl_add_u32", 160, 0, d);
+    run<kCvt>("160 v_cvt_f32_i32", 160, 0, d);
     run<kPerm>("160 v_perm_b32", 160, 0, d);
     run<kFma>("160 v_fma_f32", 160, 0, d);
     run<kExp>("160 v_exp_f32", 160, 0, d);
