@@ -13,16 +13,18 @@
 #include <cstdlib>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 enum Mix { kValu = 0, kMfma, kFine, kCoarse, kSplitWaves, kPerm, kFma, kExp, kValuSgpr, kAndOnlyLit, kAndOnlySgpr,
-           kAndVgpr, kMulLit, kMulVgpr, kShiftLit, kShlAdd, kCvt };
+           kAndVgpr, kMulLit, kMulVgpr, kShiftLit, kShlAdd, kCvt, kTileF16, kTileI8 };
 
 // One iteration per wave: 160 (v_and_b32, v_add_u32) pairs = 320 vector instructions and / or 16 MFMAs (kFine: 80 pairs
 // between 16 MFMAs; kSplitWaves: even waves the 160 pairs, odd waves the 16 MFMAs), or 160 instructions of one other kind.
 // The instruction counts handed to run() are those of the compiled loop bodies (hipcc -S): the and-xor chains of the last two
 // integer mixes compile to v_bitop3_b32 and v_xor_b32, 320 and 312 instructions.
-template <int MIX>
-__global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned mask, unsigned step) {
+template <int MIX, int MAXT>
+__global__ __launch_bounds__(MAXT) void mix_kernel(int iters, int* out, unsigned mask, unsigned step) {
     unsigned x[8];
     float f[8];
     v4i acc[4];
@@ -30,6 +32,20 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
     for (int i = 0; i < 4; i++) acc[i] = (v4i){0, 0, 0, 0};
     const v4i a = (v4i){(int)threadIdx.x, 1, 2, 3}, b = (v4i){4, 5, (int)threadIdx.x, 7};
     const bool odd_wave = (threadIdx.x >> 6) & 1;
+    // state of the two "prefill tile step" mixes: float sums of 16 tiles, four row-tile and four column-tile operands
+    v4f tc[16];
+    v8h ha[4], hb[4];
+    v4i ia[4], il[4], ih[4];
+    if constexpr (MIX == kTileF16 || MIX == kTileI8) {
+#pragma unroll
+        for (int t = 0; t < 16; t++) tc[t] = (v4f){(float)t, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) { ha[q][j] = (_Float16)(f[j] + (float)q); hb[q][j] = (_Float16)(f[(j + q) & 7] - (float)q); }
+            ia[q] = a + (v4i){q, 1, q, 3}; il[q] = b - (v4i){q, q, 2, 1}; ih[q] = b ^ (v4i){3, q, q, 7};
+        }
+    }
     for (int it = 0; it < iters; it++) {
         if constexpr (MIX == kValu || MIX == kCoarse) {
 #pragma unroll
@@ -113,12 +129,43 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
             LH_PROBE_160(asm volatile("v_cvt_f32_i32 %0, %0" : "+v"(f[i])))
         }
 #undef LH_PROBE_160
+        // One 256-column weight block of a 64 x 64 output tile of a prefill matmul, as one multiplying wave issues it:
+        // f16 form: 16 accumulator tiles x 8 k steps of v_mfma_f32_16x16x32_f16 into float sums that stay where they are.
+        // int8 form with 16-bit activations in two limbs: 16 tiles x 4 k steps x 2 limbs of v_mfma_i32_16x16x64_i8 into
+        // int32 sums, which have to leave the integers once per block -- per output (64 per lane) a shift-add of the
+        // limbs, a conversion and a multiply-add with the block's scale product.
+        if constexpr (MIX == kTileF16) {
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+#pragma unroll
+                for (int t = 0; t < 16; t++) tc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ha[t >> 2], hb[t & 3], tc[t], 0, 0, 0);
+        }
+        if constexpr (MIX == kTileI8) {
+            v4i lo[16], hi[16];
+#pragma unroll
+            for (int t = 0; t < 16; t++) lo[t] = hi[t] = (v4i){0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    lo[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ia[t >> 2], il[t & 3], lo[t], 0, 0, 0);
+                    hi[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ia[t >> 2], ih[t & 3], hi[t], 0, 0, 0);
+                }
+#pragma unroll
+            for (int t = 0; t < 16; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) tc[t][i] = __builtin_fmaf((float)((hi[t][i] << 8) + lo[t][i]), f[(t + i) & 7], tc[t][i]);
+        }
         if constexpr (MIX == kExp) {
 #pragma unroll
             for (int r = 0; r < 20; r++)
 #pragma unroll
                 for (int i = 0; i < 8; i++) f[i] = __builtin_amdgcn_exp2f(f[i]);
         }
+    }
+    if constexpr (MIX == kTileF16 || MIX == kTileI8) {
+#pragma unroll
+        for (int t = 0; t < 16; t++) f[t & 7] += tc[t][0] + tc[t][1] + tc[t][2] + tc[t][3];
     }
     unsigned s = 0;
     for (int i = 0; i < 8; i++) s ^= x[i] ^ __float_as_uint(f[i]);
@@ -129,18 +176,18 @@ __global__ __launch_bounds__(1024) void mix_kernel(int iters, int* out, unsigned
 static double g_ghz = 0.0;
 static unsigned g_mask = 0x7f7f7f7fu, g_step = 0x01010101u;   // reach the kernels as arguments, i.e. in scalar registers
 
-template <int MIX>
+template <int MIX, int MAXT = 1024>
 static void run(const char* name, int valu_per_wave, int mfma_per_wave, int* d) {
     hipEvent_t e0, e1;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { fprintf(stderr, "hipEventCreate failed\n"); exit(1); }
     const int iters = 4000;
     printf("%-44s", name);
     for (int wps = 1; wps <= 4; wps++) {
-        if (MIX == kSplitWaves && (wps & 1)) { printf(" | %-27s", "-"); continue; }
+        if ((MIX == kSplitWaves && (wps & 1)) || 256 * wps > MAXT) { printf(" | %-27s", "-"); continue; }
         float ms = 0;
         for (int rep = 0; rep < 3; rep++) {   // the last repetition counts (clocks up, code resident)
             (void)hipEventRecord(e0);
-            hipLaunchKernelGGL(mix_kernel<MIX>, dim3(256), dim3(256 * wps), 0, 0, iters, d, g_mask, g_step);
+            hipLaunchKernelGGL((mix_kernel<MIX, MAXT>), dim3(256), dim3(256 * wps), 0, 0, iters, d, g_mask, g_step);
             (void)hipEventRecord(e1);
             if (hipEventSynchronize(e1) != hipSuccess) { fprintf(stderr, "kernel failed\n"); exit(1); }
             (void)hipEventElapsedTime(&ms, e0, e1);
@@ -178,6 +225,9 @@ int main() {
     run<kFma>("160 v_fma_f32", 160, 0, d);
     run<kExp>("160 v_exp_f32", 160, 0, d);
     run<kMfma>("16 MFMA", 0, 16, d);
+    // (launched for at most two waves per SIMD: the int8 form's 32 accumulator tiles need more than 128 registers)
+    run<kTileF16, 512>("prefill tile step, f16: 128 MFMA f16", 0, 128, d);
+    run<kTileI8, 512>("prefill tile step, int8: 128 MFMA i8 + 192", 192, 128, d);
     run<kFine>("16 x (5 x (v_and + v_add) + 1 MFMA)", 160, 16, d);
     run<kCoarse>("160 x (v_and + v_add), then 16 MFMA", 320, 16, d);
     run<kSplitWaves>("even waves 160 x (and + add), odd 16 MFMA", 320, 16, d);
