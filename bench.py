@@ -477,7 +477,7 @@ def fill_kv(pkg, ctx, K, cache, lanes, T, g):
     batch.commit_and_wait()
 
 
-def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3, graphs=True, defer=True):
+def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, lanes=64, lane_layers=3, graphs=True, defer=True, rotate_in_o=True):
     """Whole decoder layers end to end (norms, Q/K/V projections, RoPE, KV encode, attention over the tq2 cache,
     output projection, GeGLU feed-forward, per-layer input injection) at hidden 2048, FFN 8192, 8 query heads over
     1 KV head of 256, Q4_0 attention and TQ2_0 feed-forward weights, context T.  A step runs `n_layers` distinct
@@ -493,7 +493,7 @@ def bench_decode_step(pkg, ctx, K, steps, warmup, which, T=32768, n_layers=12, l
     def make_layer(i):
         t = pkg.synth.decoder_layer_tensors(2048, 8192, 8, 1, 256, pld, g)
         params = L.LayerParams(layer_idx=i, per_layer_dim=pld, rope_theta=1e6, **dims)
-        return L.TransformerLayer(params, L.LayerWeights.from_host(ctx, t))
+        return L.TransformerLayer(params, L.LayerWeights.from_host(ctx, t), fuse_rotation=rotate_in_o)
 
     res = {"context": T}
     scratch = L.ScratchBuffers(ctx, 2048, 8192, 8, 1, 256, pld)
@@ -844,6 +844,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="decode legs: skip the recorded-batch (HIP graph) replays")
     ap.add_argument("--no-defer-tail", action="store_true",
                     help="decode / model legs: every layer dispatches its own last step (default: it rides in the next layer's first dispatch)")
+    ap.add_argument("--no-rotate-in-o", action="store_true",
+                    help="decode leg: the rotation back out of code space as a dispatch of its own (default: in the output projection's staging)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model,model_lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time); "
@@ -936,7 +938,8 @@ def main():
     if legs & {"decode", "lanes", "chunk"}:
         which = (["single"] if "decode" in legs else []) + (["lanes"] if "lanes" in legs else []) + \
             (["chunk"] if "chunk" in legs else [])
-        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph, defer=not args.no_defer_tail)
+        extra["decode_step_end_to_end"] = bench_decode_step(pkg, ctx, K, args.steps, args.warmup, which, graphs=not args.no_graph, defer=not args.no_defer_tail,
+                                                            rotate_in_o=not args.no_rotate_in_o)
         log("[bench] decode step:", extra["decode_step_end_to_end"])
 
     if "model_few_lanes" in legs:

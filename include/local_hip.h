@@ -210,6 +210,15 @@ LH_API int lh_matvec_quant_norm_chain_tail_into(lh_batch* batch, lh_quant fmt, u
                                                 const lh_buffer* vector, const lh_buffer* weight, const lh_buffer* residual,
                                                 int apply_scale, float scale, const lh_buffer* next_weight, lh_buffer* store,
                                                 float eps, lh_buffer* const* outputs, uint32_t rows, uint32_t cols);
+/* One matvec whose input is rotated out of TurboQuant code space while it is staged: replaces, in
+ * quant_cache.rs:590-598 followed by layer.rs:440-446, hadamard_rotate_fh_into(vector, signs, pre_sign = false,
+ * post_sign = true) followed by matvec_*_into(matrix, that f16 vector).  `vector` = f32[cols] head outputs of the
+ * attention kernel, cols = heads x head_dim; the staged value is f16(H(x) / sqrt(head_dim) * signs) exactly as the
+ * rotation kernel would have stored it.  f16 output; head_dim a power of two in 8..=512 that divides cols, cols a
+ * multiple of 64, 16-byte aligned operands, else INVALID_ARGUMENT. */
+LH_API int lh_matvec_quant_rotated_into(lh_batch* batch, lh_quant fmt, const lh_buffer* matrix, const lh_buffer* vector,
+                                        const lh_buffer* signs, uint32_t head_dim, lh_buffer* output, uint32_t rows,
+                                        uint32_t cols);
 LH_API int lh_matvec_quant_fused_into(lh_batch* batch, lh_quant fmt, uint32_t count, const lh_buffer* const* matrices,
                                       const lh_buffer* vector, int prologue, const lh_buffer* aux, float eps,
                                       lh_buffer* const* outputs, uint32_t rows, uint32_t cols);

@@ -402,6 +402,12 @@ class Kernels:
             next_weight._h if next_weight is not None else None, store._h, C.c_float(eps), _handles(outputs), _u32(rows),
             _u32(cols)))
 
+    def matvec_quant_rotated_into(self, batch, fmt, matrix, vector, signs, head_dim, output, rows, cols):
+        """hadamard_rotate_fh_into(vector, signs, post-sign) followed by the matvec, in one dispatch: `vector` holds the
+        attention kernel's f32 head outputs, the rotation back out of code space happens while it is staged."""
+        _check(self._l.lh_matvec_quant_rotated_into(batch._h, C.c_int(fmt), matrix._h, vector._h, signs._h, _u32(head_dim),
+                                                    output._h, _u32(rows), _u32(cols)))
+
     # -- small-M / prefill matmul (kernels.rs:6378-6563, 5517-5568) --
     def matmul_nt_q4_0_into(self, batch, input, weight, output, m, k, n):
         _check(self._l.lh_matmul_nt_q4_0_into(batch._h, input._h, weight._h, output._h, _u32(m), _u32(k), _u32(n)))

@@ -91,7 +91,10 @@ static inline int lh_need(const lh_buffer* b, size_t bytes, const char* op, cons
 //                 blockIdx.x == 0 stores that vector to `store` when given, and with `aux2` the staged vector is the
 //                 RMS norm of it with weight aux2 -- post-norm + residual followed by the next pre-norm.
 //   kXProGeluMul: gelu_tanh(x_i) * aux_i                 (gelu.metal:23-41; x = gate, aux = up, f16[K])
-enum : uint32_t { kXProNone = 0, kXProRmsNorm = 1, kXProGeluMul = 2 };
+//   kXProRotate:  x = f32 head outputs in code space, K = heads x head_dim: per head the Walsh-Hadamard transform,
+//                 x 1/sqrt(head_dim) (`scale`), x signs[dim], one rounding to f16 (attention_flash_tq.metal:58-90 with the
+//                 post-sign, as hadamard_rotate_kernel<float, f16> computes it).
+enum : uint32_t { kXProNone = 0, kXProRmsNorm = 1, kXProGeluMul = 2, kXProRotate = 3 };
 struct XPrologue {
     uint32_t kind;
     const uint16_t* aux;
@@ -101,6 +104,8 @@ struct XPrologue {
     uint16_t* store = nullptr;
     uint32_t tail = 0;      // with `res`: 0 the residual joins the f32 product (rms_norm_add); 1, 2 see lh_norm_tail
     float scale = 1.0f;
+    const float* signs = nullptr;   // kXProRotate: the codec's sign vector, f32[head_dim]
+    uint32_t head_dim = 0;          // kXProRotate: a power of two, 8 .. 512, dividing K
 };
 
 // TQ2_0 matvec on the matrix cores (matvec_tq2_mfma.hip). Host arrays of device pointers; shapes validated by the caller.

@@ -926,6 +926,27 @@ int lh_matvec_quant_norm_chain_tail_into(lh_batch* b, lh_quant fmt, uint32_t cou
     return matvec_dispatch(b, fmt, count, ms, xs, LH_F16, ys, LH_F16, rows, cols, op, pro);
 }
 
+int lh_matvec_quant_rotated_into(lh_batch* b, lh_quant fmt, const lh_buffer* m, const lh_buffer* x, const lh_buffer* signs,
+                                 uint32_t head_dim, lh_buffer* y, uint32_t rows, uint32_t cols) {
+    const char* op = fmt == LH_Q4_0 ? "matvec_q4_0 (rotated input)" : "matvec_tq2_0 (rotated input)";
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_quant: unknown weight format %d", (int)fmt);
+    if (head_dim < 8 || head_dim > 512 || (head_dim & (head_dim - 1)) != 0)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: head_dim must be a power of two in 8..=512, got %u", op, head_dim);
+    if (cols % head_dim != 0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: cols %u is not a multiple of head_dim %u", op, cols, head_dim);
+    if (rows == 0 || cols == 0) return LH_OK;
+    if (!m || !x || !y) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: null buffer", op);
+    LH_NEED(signs, (size_t)head_dim * 4, op, "signs");
+    LH_REQUIRE(((uintptr_t)signs->ptr & 15) == 0, "%s: the sign vector must be 16-byte aligned", op);
+    const lh_buffer* ms[1] = {m};
+    const lh_buffer* xs[1] = {x};
+    lh_buffer* ys[1] = {y};
+    XPrologue pro{kXProRotate, nullptr, 0.0f};
+    pro.signs = (const float*)signs->ptr;
+    pro.head_dim = head_dim;
+    pro.scale = 1.0f / std::sqrt((float)head_dim);   // turboquant.rs:47
+    return matvec_dispatch(b, fmt, 1, ms, xs, LH_F32, ys, LH_F16, rows, cols, op, pro);
+}
+
 int lh_matvec_tq2_0_soa_into(lh_batch* b, const lh_buffer* qs, const lh_buffer* scales, const lh_buffer* x, lh_buffer* y,
                              uint32_t rows, uint32_t cols) {
     // kernels.rs:5929-5933

@@ -53,6 +53,38 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
     }
 }
 
+// The eight consecutive elements e0 .. e0 + 8 of a head that a lane holds, through the head's Walsh-Hadamard transform,
+// 1/sqrt(head_dim) and the sign vector, rounded to f16 once: what hadamard_rotate_kernel<float, f16> stores, bit for bit
+// (the same butterflies in the same order of stages; a sum does not depend on which operand is named first).  Stages
+// 1, 2, 4 pair elements of one lane, the others pair the lanes of a head, head_dim / 8 <= 64 consecutive lanes of a wave.
+// Every lane of the wave calls it; lanes past the vector carry zeros.
+__device__ __forceinline__ void xpro_rotate8(float (&v)[8], const XPrologue& pro, uint32_t e0) {
+#pragma unroll
+    for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (i & len) continue;
+            const float lo = v[i], hi = v[i | len];
+            v[i] = __fadd_rn(lo, hi);
+            v[i | len] = __fsub_rn(lo, hi);
+        }
+    }
+    const uint32_t lane = threadIdx.x & 63;
+    for (uint32_t m = 1; 8 * m < pro.head_dim; m <<= 1) {
+        const bool upper = (lane & m) != 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float other = __shfl_xor(v[i], (int)m, 64);
+            v[i] = upper ? __fsub_rn(other, v[i]) : __fadd_rn(v[i], other);
+        }
+    }
+    const uint32_t d0 = e0 & (pro.head_dim - 1);
+    const float4 s0 = *reinterpret_cast<const float4*>(pro.signs + d0), s1 = *reinterpret_cast<const float4*>(pro.signs + d0 + 4);
+    const float sg[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = lh_h2f(lh_f2h_exact(__fmul_rn(__fmul_rn(v[i], pro.scale), sg[i])));
+}
+
 // Second level of the fixed point, for blocks whose first-level step would be too coarse.  A block with max|x| = m has
 // the step s = m / qmax; every element carries an absolute error of up to s / 2 whatever its own size, so one large
 // element (ordinary in a residual stream) costs its neighbours their low bits.  The test is relative to the block itself:
@@ -166,6 +198,9 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                     }
                 }
             }
+        }
+        if constexpr (sizeof(XT) == 4) {
+            if (pro.kind == kXProRotate) xpro_rotate8(v, pro, e0);   // uniform over the workgroup
         }
         // the maximum over the bit patterns of |v|: the order of non-negative floats, with NaN and infinity on top
         uint32_t mbits = 0u;

@@ -134,6 +134,14 @@ class QuantizedKvCache:
                                                 self.levels, self.signs, vacc, attn_out, hd, seq_len, current_pos,
                                                 n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
 
+    def attention_codes_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, seq_len: int,
+                                          current_pos: int, n_q_heads: int, window: int) -> None:
+        """quant_cache.rs:571-589: the attend step alone; the f32 head outputs in ``vacc`` are still in code space (the
+        caller rotates them back, quant_cache.rs:590-598, e.g. inside the output projection)."""
+        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
+                                        self.levels, vacc, self.head_dim, seq_len, current_pos, n_q_heads,
+                                        self.n_kv_heads, window, self.bits, self.ring_capacity())
+
     def prepare_rows_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, start_pos: int,
                           n_rows: int, n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:
         """``prepare_token_into`` for the ``n_rows`` consecutive tokens of a prefill chunk."""

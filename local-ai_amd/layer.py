@@ -163,10 +163,12 @@ class TransformerLayer:
 
     def __init__(self, params: LayerParams, weights: LayerWeights, group_projections: bool = True,
                  fuse_norm_rope: bool = True, fuse_prologues: bool = True, fuse_norm_chain: bool = True,
-                 stack_qkv: bool = True):
+                 stack_qkv: bool = True, fuse_rotation: bool = True):
         self.params, self.weights = params, weights
         self.group_projections, self.fuse_norm_rope = group_projections, fuse_norm_rope
         self.fuse_prologues, self.fuse_norm_chain = fuse_prologues, fuse_prologues and fuse_norm_chain
+        # a decoded token's rotation back out of code space rides in the output projection's staging
+        self.fuse_rotation = fuse_prologues and fuse_rotation
         # layer.rs:515-520 reads the scalar out of shared memory at every encode; the buffer lives in device
         # memory here, so it is fetched once.
         self._output_scale = None
@@ -318,6 +320,8 @@ class TransformerLayer:
             kernels.rms_norm_into(batch, input, w.attn_norm, s.normed, h, 1, eps)
             w.attn_q.matvec_into(batch, kernels, s.normed, s.q)
         one_prepare = self._one_prepare()
+        rotate_in_o = (one_prepare and self.fuse_rotation and self._fusable(w.attn_output)
+                       and w.attn_output.cols == n_head * hd)
         if not one_prepare:
             self._norm_rope(batch, kernels, q_buf, w.q_norm, n_head, pos)
 
@@ -332,8 +336,12 @@ class TransformerLayer:
             kv_cache.prepare_token_into(batch, kernels, q_buf, k_buf if own_kv else None, v_buf if own_kv else None,
                                         w.q_norm, w.k_norm, s.rq, position, n_head, eps, p.rope_theta,
                                         p.partial_rotary_factor)
-            kv_cache.attention_from_rotated_into(batch, kernels, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
-                                                 p.sliding_window)
+            if rotate_in_o:   # the f32 head outputs stay in code space: step 3 rotates them while it stages them
+                kv_cache.attention_codes_from_rotated_into(batch, kernels, s.rq, s.vacc, seq_len, pos, n_head,
+                                                           p.sliding_window)
+            else:
+                kv_cache.attention_from_rotated_into(batch, kernels, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
+                                                     p.sliding_window)
         elif own_kv:
             kernels.rms_norm_into(batch, v_buf, s.ones, v_buf, hd, n_kv, eps)   # V: RMS norm with unit weight
             self._norm_rope(batch, kernels, k_buf, w.k_norm, n_kv, pos)
@@ -343,7 +351,11 @@ class TransformerLayer:
                                           p.sliding_window)
 
         # 3. output projection -> post_attention_norm + residual #1
-        w.attn_output.matvec_into(batch, kernels, s.attn_out, s.ffn_out)
+        if rotate_in_o:
+            kernels.matvec_quant_rotated_into(batch, w.attn_output.ty, w.attn_output.buf, s.vacc, kv_cache.signs, hd,
+                                              s.ffn_out, w.attn_output.rows, w.attn_output.cols)
+        else:
+            w.attn_output.matvec_into(batch, kernels, s.attn_out, s.ffn_out)
         chain_ffn = (self.fuse_norm_chain and self._fusable(w.ffn_gate, w.ffn_up) and self.group_projections
                      and _groupable(w.ffn_gate, w.ffn_up))
         if not chain_ffn:

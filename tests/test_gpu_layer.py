@@ -174,6 +174,34 @@ def test_grouped_and_fused_dispatches_change_nothing(pkg, gpu, oracle):
         assert np.array_equal(a, b)
 
 
+def test_rotation_in_the_output_projection_changes_nothing(pkg, gpu, oracle):
+    """A decoded token's rotation back out of code space (quant_cache.rs:590-598) rides in the staging of the output
+    projection (layer.rs:440-446): one dispatch fewer, the same bits, at a short and at a many-split context."""
+    ctx, kernels = gpu
+    g = pkg.synth.rng(903, 0)
+    dims = _dims()
+    dev, _, _ = _make(pkg, gpu, g, dims)
+    variants = [pkg.layer.TransformerLayer(dev.params, dev.weights, fuse_rotation=f) for f in (False, True)]
+    x = g.standard_normal(512, dtype=np.float32).astype(np.float16)
+    for position in (5, 3000):
+        res, counts = [], []
+        for layer in variants:
+            cache = pkg.kv_cache.QuantizedKvCache(ctx, 1, 256, 4096)
+            fill = pkg.synth.rng(904, position)   # random codes and norms near one, the same for both variants
+            for codes, norms in ((cache.keys_q, cache.key_norms), (cache.values_q, cache.value_norms)):
+                codes.copy_from_bytes(fill.integers(0, 256, codes.length(), dtype=np.uint8))
+                norms.copy_from_bytes((0.5 + fill.random(norms.length() // 2)).astype(np.float16))
+            scratch = pkg.layer.ScratchBuffers(ctx, 512, 1024, 4, 1, 256, 0)
+            inp, out = pkg.Buffer.from_slice(ctx, x), pkg.Buffer.empty(ctx, 1024)
+            batch = pkg.CommandBatch(ctx)
+            layer.forward_decode(kernels, batch, inp, out, position, scratch, cache)
+            counts.append(batch.dispatch_count())
+            batch.commit_and_wait()
+            res.append(out.as_array(np.uint16, 512))
+        assert np.array_equal(res[0], res[1])
+        assert counts[1] <= counts[0] - (1 if position == 3000 else 0)
+
+
 def test_forward_decode_one_kernel_per_op_matches_oracle(pkg, gpu, oracle):
     """The reference's literal dispatch sequence (no grouping, no fusion) with per-layer input and output scale."""
     ctx, kernels = gpu

@@ -227,6 +227,43 @@ def test_matvec_norm_chain(pkg, gpu, oracle, fmt, rows, cols, count, second_norm
         K.matvec_quant_norm_chain_into(pkg.CommandBatch(ctx), ty, [ws[0].buf], xb, w1b, rb, None, xb, 1e-6, [outs[0]], rows, cols)
 
 
+@pytest.mark.parametrize("fmt,rows,cols,hd", [("q4_0", 2048, 2048, 256), ("q4_0", 300, 4096, 512), ("q4_0", 64, 1024, 128),
+                                              ("q4_0", 33, 6144, 64), ("q4_0", 17, 320, 8), ("tq2_0", 2048, 2048, 256),
+                                              ("tq2_0", 96, 4096, 512), ("tq2_0", 40, 768, 16)])
+def test_matvec_rotated_input(pkg, gpu, oracle, fmt, rows, cols, hd):
+    """matvec_quant_rotated_into: the rotation back out of code space (attention_flash_tq.metal:58-90 with the post-sign,
+    quant_cache.rs:590-598) happens while the output projection stages its vector (layer.rs:440-446).  The staged f16
+    vector is the oracle's rotation bit for bit, so the products equal those of the two separate dispatches bit for bit
+    and meet the oracle's f64 dot over it."""
+    print(f"case rotated {fmt} {rows}x{cols} hd{hd}", flush=True)
+    ctx, K = gpu
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    heads = cols // hd
+    g = pkg.synth.rng(41, rows + cols + hd)
+    raw = refgen.q4_0_payload(rows, cols, 0x51) if fmt == "q4_0" else refgen.tq2_0_payload(rows, cols, 0x51)
+    dq = (oracle.expand_q4_0_f32 if fmt == "q4_0" else oracle.expand_tq2_0_f32)(raw, rows, cols)
+    w = pkg.QuantWeight.from_bytes(ctx, raw, ty, rows, cols)
+    x = g.standard_normal(cols, dtype=np.float32) * 1.5
+    signs = np.where(g.random(hd) < 0.5, -1.0, 1.0).astype(np.float32)
+    xb, sb = pkg.Buffer.from_slice(ctx, x), pkg.Buffer.from_slice(ctx, signs)
+    fused, sep, rot = pkg.Buffer.empty(ctx, rows * 2), pkg.Buffer.empty(ctx, rows * 2), pkg.Buffer.empty(ctx, cols * 2)
+    batch = pkg.CommandBatch(ctx)
+    K.matvec_quant_rotated_into(batch, ty, w.buf, xb, sb, hd, fused, rows, cols)
+    assert batch.dispatch_count() == 1
+    K.hadamard_rotate_fh_into(batch, xb, sb, rot, hd, heads, False, True)
+    w.matvec_into(batch, K, rot, sep)
+    batch.commit_and_wait()
+    staged = oracle.hadamard_rotate(x, signs, hd, heads, False, True).astype(np.float16)
+    assert np.array_equal(rot.as_array(np.uint16, cols), staged.view(np.uint16))
+    got = fused.as_array(np.float16, rows)
+    assert np.array_equal(got.view(np.uint16), sep.as_array(np.uint16, rows))
+    want = oracle.matvec_f64(dq, staged.astype(np.float32)).astype(np.float32)
+    refgen.assert_close(got.astype(np.float32), want, 2e-3, f"{fmt} rotated input {rows}x{cols} hd{hd}")
+    for bad_hd in (0, 4, 48, 1024):
+        with pytest.raises(pkg.InvalidArgument):
+            K.matvec_quant_rotated_into(pkg.CommandBatch(ctx), ty, w.buf, xb, sb, bad_hd, fused, rows, cols)
+
+
 @pytest.mark.parametrize("rows,cols", [(5, 256), (6, 512), (37, 1536), (2048, 2048), (1023, 6144)])
 def test_matvec_tq2_0_soa(pkg, gpu, oracle, rows, cols):
     """kernels.rs:5919-5971 / matvec_quant.metal:322-387: the split layout -- qs[(row * blocks + b) * 64] and
