@@ -89,19 +89,27 @@ struct AttnShared {
 // HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
 // ONE_KV: a single KV head (the measured configuration and the reference model): the distance between positions is a
 // compile-time constant, so the loads of a group take immediate offsets instead of per-load address arithmetic.
-template <int NPL, int HD, bool ONE_KV, int PS>
-__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>& sh, float alpha, float beta,
+// NQ = chunks per workgroup: 1, or 4 (head_dim 256 with pair hand-overs): eight waves, a K wave and a V wave per chunk, each
+// pair of waves with a hand-over area of its own; the query set-up is done once, by all eight, and the four partial results
+// are merged through LDS, so that a query cut into four chunks needs neither partial records nor a merge launch.  The
+// hand-over barriers are workgroup barriers, so every wave executes as many as the chunk with the most hand-overs needs.
+template <int NPL, int HD, bool ONE_KV, int PS, int NQ = 1>
+__device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>* shs, float alpha, float beta,
                                                float gam, float delta) {
-    auto& s_rqop = sh.rqop;
-    auto& s_maxabs = sh.maxabs;
-    auto& s_sum = sh.sum;
+    static_assert(NQ == 1 || (NQ == 4 && HD == 256 && PS == 2), "several chunks per workgroup: head_dim 256 with pair hand-overs only");
+    const uint32_t wave_all = threadIdx.x >> 6;                   // wave of the workgroup (the set-up is dealt over all of them)
+    const uint32_t sub = NQ == 1 ? 0u : wave_all >> 1;            // which of the workgroup's chunks this wave works on
+    auto& sh = shs[sub];
+    auto& s_rqop = shs[0].rqop;
+    auto& s_maxabs = shs[0].maxabs;
+    auto& s_sum = shs[0].sum;
     constexpr int kHeadDim = HD, kCodeBytes = HD / 4, NH = HD / 256;   // NH: 64-byte halves of a code
     constexpr bool has_delta = NPL == 3;
     constexpr int nplanes = NPL;
     // The two-plane forms are only entered with a level table whose mean is zero to rounding (any symmetric table): the
     // constant term of the centred planes then vanishes and the exact sum of the weights is not needed.
     constexpr bool need_wsum = NPL == 3;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = NQ == 1 ? wave_all : wave_all & 1u, nwaves = blockDim.x >> 6;
     const uint32_t pcol = lane & 15, g = lane >> 4;               // MFMA column / row group of this lane
     const uint32_t qi = blockIdx.y / p.num_kv_heads, kvh = blockIdx.y - qi * p.num_kv_heads;
     const uint32_t group = p.num_q_heads / p.num_kv_heads;
@@ -113,13 +121,24 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // ---- the workgroup's chunk of positions
     uint32_t lo, hi, lane_base;
     query_range(p, a.positions, qi, lo, hi, lane_base);
-    const uint32_t n = hi - lo, nsplit = p.num_splits;
-    const uint32_t split = blockIdx.x;
+    const uint32_t n = hi - lo, nsplit = p.num_splits * NQ;       // p.num_splits counts partial records, i.e. workgroups per query
+    const uint32_t split = blockIdx.x * NQ + sub;
     const uint32_t chunk = (((n + nsplit - 1) / nsplit) + (kGroup - 1)) & ~(uint32_t)(kGroup - 1);
     const uint32_t c_lo = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)split * chunk);
     const uint32_t c_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(split + 1) * chunk);
     const bool any = c_hi > c_lo;
     const uint32_t g_first = c_lo >> 6, g_last = any ? (c_hi - 1) >> 6 : 0u;
+    // Several chunks per workgroup: hand-overs (aligned pairs of groups) of this chunk, and of the workgroup's longest.
+    [[maybe_unused]] uint32_t my_handovers = 0, max_handovers = 0;
+    if constexpr (NQ > 1) {
+        for (uint32_t s = blockIdx.x * NQ; s < (blockIdx.x + 1) * NQ; s++) {
+            const uint32_t s_lo = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)s * chunk);
+            const uint32_t s_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(s + 1) * chunk);
+            const uint32_t cnt = s_hi > s_lo ? ((s_hi - 1) >> 7) - (s_lo >> 7) + 1 : 0u;
+            if (s == split) my_handovers = cnt;
+            max_handovers = std::max(max_handovers, cnt);
+        }
+    }
 
     const uint32_t stride = ONE_KV ? (uint32_t)kCodeBytes : p.num_kv_heads * kCodeBytes;   // bytes between positions
     const uint32_t nstride = ONE_KV ? 2u : p.num_kv_heads * 2;
@@ -142,7 +161,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // head_dim 256: a K wave and a V wave.  head_dim 512: a K wave per 64-byte half of the K codes -- the second one (role 3)
     // runs a group ahead and hands its integer logit sums to the first, which adds its own and does the softmax -- and a V wave
     // per half of the V codes.
-    const uint32_t role = NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) & 3u;   // 0: K wave; 1, 2: V wave of code half role - 1; 3: second K wave
+    // (Several chunks per workgroup: waves w and w + 4 share a SIMD, so chunks 0, 1 and chunks 2, 3 take opposite orders.)
+    const uint32_t role = NQ > 1 ? ((wave ^ (sub >> 1)) & 1u) : NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) & 3u;   // 0: K wave; 1, 2: V wave of code half role - 1; 3: second K wave
     const bool k_role = role == 0 || role == 3;
     const bool kb_role = NH == 2 && role == 3;
     const uint32_t khalf = kb_role ? 1u : 0u;
@@ -174,8 +194,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             }
     };
     // Operand units (code half, plane) are dealt to the waves round robin; the first unit's queries are requested here.
-    uint32_t xq_half = wave / (uint32_t)nplanes;
-    if (wave < (uint32_t)(nplanes * NH)) load_xq(xq_half);
+    uint32_t xq_half = wave_all / (uint32_t)nplanes;
+    if (wave_all < (uint32_t)(nplanes * NH)) load_xq(xq_half);
 
     // ---- per head: max |rq| (quantisation scale) and sum(rq) (constant term of the level table)
     for (uint32_t h = tid >> 5; h < (uint32_t)kMaxGroupHeads; h += blockDim.x >> 5) {
@@ -206,7 +226,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     {
         const float ma = s_maxabs[h_op];
         const float inv = (ma > 0.0f && cmax_k > 0.0f) ? kQmax / (ma * cmax_k) : 0.0f;
-        for (uint32_t unit = wave; unit < (uint32_t)(nplanes * NH); unit += nwaves) {
+        for (uint32_t unit = wave_all; unit < (uint32_t)(nplanes * NH); unit += nwaves) {
             const uint32_t half = unit / (uint32_t)nplanes, pl = unit - half * (uint32_t)nplanes;
             if (half != xq_half) { load_xq(half); xq_half = half; }
             const float mul = (pl == 0 ? beta : pl == 1 ? 0.5f * gam : delta) * inv;
@@ -256,7 +276,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         for (int hs = 0; hs < 2; hs++) {
             const uint32_t h = g + 4 * hs;
             cs[hs] = s_maxabs[h] * cmax_k * (0.25f / kQmax);
-            ca[hs] = alpha * sh.sum[h];
+            ca[hs] = alpha * s_sum[h];
         }
         gptr_t krec0 = (gptr_t)a.k_codes + ((size_t)lane_base * p.num_kv_heads + kvh) * kCodeBytes + 64 * khalf;   // this wave's half of the code
         gptr_t kn0 = (gptr_t)a.k_norms + ((size_t)lane_base * p.num_kv_heads + kvh) * 2;
@@ -517,6 +537,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 if constexpr (NH == 2) __syncthreads();   // the V waves' last hand-over
             }
         }
+        if constexpr (NQ > 1) {   // the hand-overs that only longer chunks of this workgroup have
+            for (uint32_t i = my_handovers; i < max_handovers; i++) __syncthreads();
+        }
 #pragma unroll
         for (int hs = 0; hs < 2; hs++) {
             const float l_tot = lh_group_sum(l_run[hs], 16);
@@ -737,6 +760,9 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
                 if constexpr (NH == 2) __syncthreads();   // pairs with the K waves' count of barriers
             }
         }
+        if constexpr (NQ > 1) {   // the hand-overs that only longer chunks of this workgroup have
+            for (uint32_t i = my_handovers; i < max_handovers; i++) __syncthreads();
+        }
         __syncthreads();   // the K wave's totals
 
         // ---- the workgroup's result: final output (one split) or a partial record for the merge kernel
@@ -747,7 +773,13 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             const float l_tot = sh.fin_l[h], w_tot = sh.fin_w[h];
             const uint32_t qh = kvh * group + h;
             const float bias = need_wsum ? (alpha + 0.5f * (beta + gam) + 0.25f * delta) * w_tot - sctr[hs] : -sctr[hs];
-            if (nsplit == 1) {
+            if constexpr (NQ > 1) {   // parked for the merge below, in the weights' area (nobody reads weights any more)
+                float* park = reinterpret_cast<float*>(&sh.ww[0][0][0][0]) + h * kHeadDim + 4 * pcol;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    *reinterpret_cast<float4*>(park + 64 * e) =
+                        make_float4(outv[e][0][hs] + bias, outv[e][1][hs] + bias, outv[e][2][hs] + bias, outv[e][3][hs] + bias);
+            } else if (nsplit == 1) {
                 float* dst = a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 256 * vhalf + 4 * pcol;
                 const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
 #pragma unroll
@@ -764,6 +796,38 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             }
         }
     }
+    if constexpr (NQ > 1) {
+        // ---- the chunks' results merged: wave h takes head h, a lane four dims.  (R, l, acc) of a chunk are relative to
+        //      exp2(R); the result goes out as the final output (one workgroup per query) or as one partial record.
+        static_assert(sizeof(sh.ww) >= (size_t)kMaxGroupHeads * kHeadDim * sizeof(float), "the parked sums fit the weights' area");
+        __syncthreads();   // every chunk's sums are parked
+        const uint32_t h = wave_all;
+        if (h < group) {
+            float Rq[NQ], gm = -INFINITY;
+#pragma unroll
+            for (int q = 0; q < NQ; q++) { Rq[q] = shs[q].fin_r[h]; gm = fmaxf(gm, Rq[q]); }
+            float l_all = 0.0f;
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                const float f = Rq[q] == -INFINITY ? 0.0f : exp2f(Rq[q] - gm);
+                const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(&shs[q].ww[0][0][0][0]) + h * kHeadDim + 4 * lane);
+                l_all = __builtin_fmaf(f, shs[q].fin_l[h], l_all);
+                o.x = __builtin_fmaf(f, v.x, o.x); o.y = __builtin_fmaf(f, v.y, o.y);
+                o.z = __builtin_fmaf(f, v.z, o.z); o.w = __builtin_fmaf(f, v.w, o.w);
+            }
+            const uint32_t qh = kvh * group + h;
+            if (p.num_splits == 1) {
+                const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+                *reinterpret_cast<float4*>(a.out + ((size_t)qi * p.num_q_heads + qh) * kHeadDim + 4 * lane) =
+                    make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+            } else {
+                float* rec = a.ws + (((size_t)qi * p.num_q_heads + qh) * p.num_splits + blockIdx.x) * partial_record_floats(kHeadDim);
+                if (lane == 0) { rec[0] = gm * kLn2; rec[1] = l_all; }
+                *reinterpret_cast<float4*>(rec + 4 + 4 * lane) = o;
+            }
+        }
+    }
 }
 
 template <int OCC, int HD, int PS>
@@ -777,9 +841,24 @@ __global__ __launch_bounds__(HD / 2, OCC) void attention_tq_mfma_kernel(AttnPoin
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
     // The constant term left over by the centred planes is mean(L) times the sum of the weights.
     const float l_mean = 0.25f * ((L0 + L3) + (L1 + L2));
-    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, HD, false, PS>(a, p, sh, L0, L1 - L0, L2 - L0, d_raw);
-    else if (p.num_kv_heads == 1) attention_body<2, HD, true, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
-    else attention_body<2, HD, false, PS>(a, p, sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, HD, false, PS>(a, p, &sh, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, HD, true, PS>(a, p, &sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, HD, false, PS>(a, p, &sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+}
+
+// Four chunks of a query per workgroup (head_dim 256, pair hand-overs): 512 threads, the hand-over areas in dynamic LDS.
+constexpr int kQuad = 4;
+constexpr size_t kQuadLdsBytes = kQuad * sizeof(AttnShared<1, 2>);
+__global__ __launch_bounds__(128 * kQuad, 2) void attention_tq_mfma_quad_kernel(AttnPointers a, AttnParams p) {
+    extern __shared__ __align__(16) uint8_t quad_lds[];
+    auto* shs = reinterpret_cast<AttnShared<1, 2>*>(quad_lds);
+    const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];   // as in attention_tq_mfma_kernel
+    const float d_raw = (L3 - L2) - (L1 - L0);
+    const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
+    const float l_mean = 0.25f * ((L0 + L3) + (L1 + L2));
+    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, 256, false, 2, kQuad>(a, p, shs, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, 256, true, 2, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, 256, false, 2, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
@@ -821,7 +900,6 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     const size_t rec = partial_record_floats(p.head_dim);
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
-    const dim3 grid((uint32_t)splits, (uint32_t)pairs);
     // Hand-overs of two groups pay from about a thousand positions per workgroup on (-2 % at 4096 positions per workgroup, -5 % at
     // 8192, either head_dim); below that the longer fill and drain of the pipeline costs more (a 512-position window: +24 %).
     // LOCAL_HIP_ATTN_PAIR=1 / 0 forces one form onto every chunk length (a test aid: it puts missing and partial groups at both
@@ -829,6 +907,18 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
     constexpr uint64_t pair_min = 1024;
     const bool pair = pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min;
+    // Long chunks of head_dim 256 in fours: one eight-wave workgroup takes four consecutive chunks of a query and merges them
+    // itself, so a query of four chunks leaves the kernel as its final output (no partial records, no merge launch) and one of
+    // 4 k chunks as k records.  Other chunk counts keep a workgroup per chunk: the gain is the merge launch that four chunks no
+    // longer need (256 x 32768 positions: 218 against 229 us); with records left to merge the forms measure alike.
+    if (p.head_dim == 256 && pair && splits % kQuad == 0) {
+        const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel, kQuadLdsBytes, op);
+        if (rl != LH_OK) return rl;
+        p.num_splits = (uint32_t)(splits / kQuad);
+        hipLaunchKernelGGL(attention_tq_mfma_quad_kernel, dim3(p.num_splits, (uint32_t)pairs), dim3(128 * kQuad), kQuadLdsBytes, ctx->stream, a, p);
+        return lh_check_launch(op);
+    }
+    const dim3 grid((uint32_t)splits, (uint32_t)pairs);
     if (p.head_dim == 512 && pair) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 2>), grid, dim3(256), 0, ctx->stream, a, p);
     else if (p.head_dim == 512) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 512, 1>), grid, dim3(256), 0, ctx->stream, a, p);
     else if (pair) hipLaunchKernelGGL((attention_tq_mfma_kernel<2, 256, 2>), grid, dim3(128), 0, ctx->stream, a, p);

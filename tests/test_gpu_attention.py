@@ -449,6 +449,40 @@ def test_batched_matches_independent_sequences(pkg, gpu, oracle, hd):
         check(got[l], ref, f"lane {l}")
 
 
+@pytest.mark.parametrize("lanes,cap", [(32, 32768), (256, 4096)])
+def test_batched_long_lanes_merged_in_the_workgroup(pkg, gpu, oracle, lanes, cap):
+    """Long chunks of many lanes in one dispatch: four consecutive chunks of a lane share a workgroup that merges them
+    itself.  32 lanes of up to 32768 positions: 32 chunks per lane leave eight partial records instead of thirty-two;
+    256 lanes of up to 4096: four chunks per lane leave the kernel as the final output, with no merge behind it.  The
+    lanes stand at ragged positions -- some shorter than one chunk, one empty but for its first position -- so a
+    workgroup holds chunks with different numbers of hand-overs and chunks with nothing in them.  Every checked lane
+    against the f64 oracle."""
+    print(f"case lanes={lanes} cap={cap}", flush=True)
+    ctx, K = gpu
+    hd, nq, nkv, bits = 256, 8, 1, 2
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, cap, nkv, hd, bits, 4040)
+    g = pkg.synth.rng(6, 40)
+    positions = g.integers(cap // 10, cap, lanes).astype(np.uint32)
+    positions[:8] = [cap - 1, 0, 63, 64, 130, 1500, cap // 2 + 1, cap - 700]
+    pool_kc, pool_vc = np.tile(kc, (lanes, 1, 1)), np.tile(vc, (lanes, 1, 1))
+    pool_kn, pool_vn = np.tile(kn, (lanes, 1)), np.tile(vn, (lanes, 1))
+    rq = g.standard_normal((lanes, nq * hd), dtype=np.float32)
+    rq[1::2] *= 0.15                                    # every other lane a soft distribution
+    bufs = upload(pkg, ctx, pool_kc, pool_kn, pool_vc, pool_vn, levels, rq, positions)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+    K.flash_attention_tq_batched_into(batch, bufs[5], bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], out, bufs[6], hd, cap, nq,
+                                      nkv, 0, bits, lanes, 0)
+    batch.commit_and_wait()
+    got = out.as_array(np.float32).reshape(lanes, nq * hd)
+    assert np.isfinite(got).all()
+    for l in list(range(8)) + [11, 24, lanes - 1]:
+        print(f"lane {l} at {positions[l]}", flush=True)
+        ref = oracle.attention_tq_codespace(rq[l], pool_kc, pool_kn, pool_vc, pool_vn, levels, hd, int(positions[l]) + 1,
+                                            int(positions[l]), nq, nkv, 0, bits, 0, lane_base=l * cap)
+        check(got[l], ref, f"lane {l} at {positions[l]}")
+
+
 def test_split_invariance_at_32k(pkg, gpu, oracle):
     """Full-size configuration (32768 cached positions, 8 q heads / 1 kv head, hd 256, 2 bits):
     parity with the f64 oracle, and the SWA-ring configuration (window 512, ring 512, wrapped)."""
