@@ -967,7 +967,7 @@ def main():
     attention_cfg = None
     if "tq2_attention_32k" in extra:
         a = extra["tq2_attention_32k"]
-        roof_others.append({"kernel": "attention_tq_mfma_kernel + merge (tq2 KV flash decoding, 8 q heads / 1 KV head, head_dim 256, 32768 positions)",
+        roof_others.append({"kernel": "attention_tq_mfma_quad_kernel (tq2 KV flash decoding, 8 q heads / 1 KV head, head_dim 256, 32768 positions; four chunks of a sequence per workgroup, merged in the kernel)",
                             "bound": "hbm", "achieved": a["batched_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": a["batched_gbs"] / HBM_PEAK_GBS, "launch_ms": a["batched_us_per_launch"] * 1e-3,
                             "alg_bytes_per_launch": a["cache_bytes"]})

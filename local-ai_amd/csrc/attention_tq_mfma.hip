@@ -89,14 +89,14 @@ struct AttnShared {
 // HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
 // ONE_KV: a single KV head (the measured configuration and the reference model): the distance between positions is a
 // compile-time constant, so the loads of a group take immediate offsets instead of per-load address arithmetic.
-// NQ = chunks per workgroup: 1, or 4 (head_dim 256 with pair hand-overs): eight waves, a K wave and a V wave per chunk, each
+// NQ = chunks per workgroup: 1, or 4 (head_dim 256): eight waves, a K wave and a V wave per chunk, each
 // pair of waves with a hand-over area of its own; the query set-up is done once, by all eight, and the four partial results
 // are merged through LDS, so that a query cut into four chunks needs neither partial records nor a merge launch.  The
 // hand-over barriers are workgroup barriers, so every wave executes as many as the chunk with the most hand-overs needs.
 template <int NPL, int HD, bool ONE_KV, int PS, int NQ = 1>
 __device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>* shs, float alpha, float beta,
                                                float gam, float delta) {
-    static_assert(NQ == 1 || (NQ == 4 && HD == 256 && PS == 2), "several chunks per workgroup: head_dim 256 with pair hand-overs only");
+    static_assert(NQ == 1 || (NQ == 4 && HD == 256), "several chunks per workgroup: head_dim 256 only");
     const uint32_t wave_all = threadIdx.x >> 6;                   // wave of the workgroup (the set-up is dealt over all of them)
     const uint32_t sub = NQ == 1 ? 0u : wave_all >> 1;            // which of the workgroup's chunks this wave works on
     auto& sh = shs[sub];
@@ -128,13 +128,14 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     const uint32_t c_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(split + 1) * chunk);
     const bool any = c_hi > c_lo;
     const uint32_t g_first = c_lo >> 6, g_last = any ? (c_hi - 1) >> 6 : 0u;
-    // Several chunks per workgroup: hand-overs (aligned pairs of groups) of this chunk, and of the workgroup's longest.
+    // Several chunks per workgroup: hand-overs (groups, or aligned pairs of groups) of this chunk, and of the workgroup's longest.
     [[maybe_unused]] uint32_t my_handovers = 0, max_handovers = 0;
     if constexpr (NQ > 1) {
         for (uint32_t s = blockIdx.x * NQ; s < (blockIdx.x + 1) * NQ; s++) {
             const uint32_t s_lo = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)s * chunk);
             const uint32_t s_hi = lo + (uint32_t)std::min<uint64_t>(n, (uint64_t)(s + 1) * chunk);
-            const uint32_t cnt = s_hi > s_lo ? ((s_hi - 1) >> 7) - (s_lo >> 7) + 1 : 0u;
+            constexpr int kShift = PS == 2 ? 7 : 6;
+            const uint32_t cnt = s_hi > s_lo ? ((s_hi - 1) >> kShift) - (s_lo >> kShift) + 1 : 0u;
             if (s == split) my_handovers = cnt;
             max_handovers = std::max(max_handovers, cnt);
         }
@@ -773,8 +774,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
             const float l_tot = sh.fin_l[h], w_tot = sh.fin_w[h];
             const uint32_t qh = kvh * group + h;
             const float bias = need_wsum ? (alpha + 0.5f * (beta + gam) + 0.25f * delta) * w_tot - sctr[hs] : -sctr[hs];
-            if constexpr (NQ > 1) {   // parked for the merge below, in the weights' area (nobody reads weights any more)
-                float* park = reinterpret_cast<float*>(&sh.ww[0][0][0][0]) + h * kHeadDim + 4 * pcol;
+            if constexpr (NQ > 1) {   // parked for the merge below, in this pair's operand area (every loop of the workgroup has ended)
+                float* park = reinterpret_cast<float*>(&sh.rqop[0][0][0]) + h * kHeadDim + 4 * pcol;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     *reinterpret_cast<float4*>(park + 64 * e) =
@@ -799,7 +800,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     if constexpr (NQ > 1) {
         // ---- the chunks' results merged: wave h takes head h, a lane four dims.  (R, l, acc) of a chunk are relative to
         //      exp2(R); the result goes out as the final output (one workgroup per query) or as one partial record.
-        static_assert(sizeof(sh.ww) >= (size_t)kMaxGroupHeads * kHeadDim * sizeof(float), "the parked sums fit the weights' area");
+        static_assert(sizeof(sh.rqop) >= (size_t)kMaxGroupHeads * kHeadDim * sizeof(float), "the parked sums fit the operand area");
         __syncthreads();   // every chunk's sums are parked
         const uint32_t h = wave_all;
         if (h < group) {
@@ -811,7 +812,7 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
 #pragma unroll
             for (int q = 0; q < NQ; q++) {
                 const float f = Rq[q] == -INFINITY ? 0.0f : exp2f(Rq[q] - gm);
-                const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(&shs[q].ww[0][0][0][0]) + h * kHeadDim + 4 * lane);
+                const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(&shs[q].rqop[0][0][0]) + h * kHeadDim + 4 * lane);
                 l_all = __builtin_fmaf(f, shs[q].fin_l[h], l_all);
                 o.x = __builtin_fmaf(f, v.x, o.x); o.y = __builtin_fmaf(f, v.y, o.y);
                 o.z = __builtin_fmaf(f, v.z, o.z); o.w = __builtin_fmaf(f, v.w, o.w);
@@ -846,19 +847,20 @@ __global__ __launch_bounds__(HD / 2, OCC) void attention_tq_mfma_kernel(AttnPoin
     else attention_body<2, HD, false, PS>(a, p, &sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
-// Four chunks of a query per workgroup (head_dim 256, pair hand-overs): 512 threads, the hand-over areas in dynamic LDS.
+// Four chunks of a query per workgroup (head_dim 256): 512 threads, the hand-over areas in dynamic LDS.
 constexpr int kQuad = 4;
-constexpr size_t kQuadLdsBytes = kQuad * sizeof(AttnShared<1, 2>);
+template <int PS> constexpr size_t quad_lds_bytes() { return kQuad * sizeof(AttnShared<1, PS>); }
+template <int PS>
 __global__ __launch_bounds__(128 * kQuad, 2) void attention_tq_mfma_quad_kernel(AttnPointers a, AttnParams p) {
     extern __shared__ __align__(16) uint8_t quad_lds[];
-    auto* shs = reinterpret_cast<AttnShared<1, 2>*>(quad_lds);
+    auto* shs = reinterpret_cast<AttnShared<1, PS>*>(quad_lds);
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];   // as in attention_tq_mfma_kernel
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
     const float l_mean = 0.25f * ((L0 + L3) + (L1 + L2));
-    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, 256, false, 2, kQuad>(a, p, shs, L0, L1 - L0, L2 - L0, d_raw);
-    else if (p.num_kv_heads == 1) attention_body<2, 256, true, 2, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
-    else attention_body<2, 256, false, 2, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, 256, false, PS, kQuad>(a, p, shs, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, 256, true, PS, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, 256, false, PS, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
@@ -886,7 +888,27 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     const uint64_t pairs = (uint64_t)p.num_queries * p.num_kv_heads;
     const uint32_t wg_waves = p.head_dim == 512 ? 4 : 2;
     const uint64_t wg_slots = (uint64_t)ctx->cu_count * std::max(1u, 4u * wps / wg_waves);
+    const size_t rec = partial_record_floats(p.head_dim);
+    static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
     uint64_t splits = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)ctx->cu_count / pairs));
+    // Short jobs of head_dim 256 in fours: an eight-wave workgroup per CU takes four chunks of a query, down to one group each,
+    // and merges them itself -- twice the waves of the two-wave form at work on a latency-bound job and a quarter of the
+    // partial records.  It pays where a two-wave workgroup per CU would walk more than one group (one query over 32768
+    // positions: 12.5-12.9 us against 13.9; over 131072: 16.5 against 20.0); where every workgroup has one group anyway the
+    // longer set-up and the merge of the eight-wave workgroup cost more than they save (4096 positions: 12.5 against 10.6 us).
+    if (p.head_dim == 256 && pair_env <= 0 && (max_span + splits - 1) / splits > 64) {
+        uint64_t q = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)kQuad * ctx->cu_count / pairs));
+        q -= q % kQuad;
+        while (q > (uint64_t)kQuad && (size_t)p.num_queries * p.num_q_heads * (q / kQuad) * rec > ws_floats) q -= kQuad;
+        if (q >= (uint64_t)kQuad && (((max_span + q - 1) / q + 63) & ~(uint64_t)63) <= 128 &&
+            (q == (uint64_t)kQuad || (size_t)p.num_queries * p.num_q_heads * (q / kQuad) * rec <= ws_floats)) {
+            const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<1>, quad_lds_bytes<1>(), op);
+            if (rl != LH_OK) return rl;
+            p.num_splits = (uint32_t)(q / kQuad);
+            hipLaunchKernelGGL(attention_tq_mfma_quad_kernel<1>, dim3(p.num_splits, (uint32_t)pairs), dim3(128 * kQuad), quad_lds_bytes<1>(), ctx->stream, a, p);
+            return lh_check_launch(op);
+        }
+    }
     splits = std::max<uint64_t>(splits, 1);
     if ((max_span + splits - 1) / splits > 128) {
         splits = std::max<uint64_t>(1, wg_slots / pairs);
@@ -897,14 +919,12 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     // 20.5 us with 256 splits, 21.7 with 512, 25.8 with 1024).
     if (splits > 256) splits = std::max<uint64_t>(256, std::min<uint64_t>(splits, (max_span + 1023) / 1024));
     splits = std::min<uint64_t>(std::max<uint64_t>(splits, 1), kMaxSplits);
-    const size_t rec = partial_record_floats(p.head_dim);
     while (splits > 1 && (size_t)p.num_queries * p.num_q_heads * splits * rec > ws_floats) splits--;
     p.num_splits = (uint32_t)splits;
     // Hand-overs of two groups pay from about a thousand positions per workgroup on (-2 % at 4096 positions per workgroup, -5 % at
     // 8192, either head_dim); below that the longer fill and drain of the pipeline costs more (a 512-position window: +24 %).
     // LOCAL_HIP_ATTN_PAIR=1 / 0 forces one form onto every chunk length (a test aid: it puts missing and partial groups at both
     // ends of short chunks through the paired loops).
-    static const int pair_env = [] { const char* e = getenv("LOCAL_HIP_ATTN_PAIR"); return e ? atoi(e) : -1; }();
     constexpr uint64_t pair_min = 1024;
     const bool pair = pair_env >= 0 ? pair_env != 0 : (max_span + splits - 1) / splits >= pair_min;
     // Long chunks of head_dim 256 in fours: one eight-wave workgroup takes four consecutive chunks of a query and merges them
@@ -912,10 +932,10 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     // 4 k chunks as k records.  Other chunk counts keep a workgroup per chunk: the gain is the merge launch that four chunks no
     // longer need (256 x 32768 positions: 218 against 229 us); with records left to merge the forms measure alike.
     if (p.head_dim == 256 && pair && splits % kQuad == 0) {
-        const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel, kQuadLdsBytes, op);
+        const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<2>, quad_lds_bytes<2>(), op);
         if (rl != LH_OK) return rl;
         p.num_splits = (uint32_t)(splits / kQuad);
-        hipLaunchKernelGGL(attention_tq_mfma_quad_kernel, dim3(p.num_splits, (uint32_t)pairs), dim3(128 * kQuad), kQuadLdsBytes, ctx->stream, a, p);
+        hipLaunchKernelGGL(attention_tq_mfma_quad_kernel<2>, dim3(p.num_splits, (uint32_t)pairs), dim3(128 * kQuad), quad_lds_bytes<2>(), ctx->stream, a, p);
         return lh_check_launch(op);
     }
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
