@@ -540,7 +540,7 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     return res
 
 
-def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64, defer_tail=True):
+def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64, defer_tail=True, rotate_in_o=True):
     """End-to-end decode of a synthetic model with the geometry of the reference's Gemma 4 E2B configuration
     (local-core/src/config/gemma4_qat.rs:262-283: vocabulary 262144, hidden 1536, 35 layers in a sliding x4 / full
     pattern with head_dim 256 / 512, window 512, the last 20 layers sharing KV, per-layer inputs of 256; Q4_0
@@ -569,6 +569,8 @@ def bench_model(pkg, ctx, K, steps, warmup, T=32768, single=True, lanes=64, defe
     max_ctx = T + 256
     pipe = P.DecodePipeline.from_host(ctx, K, cfg, tensors, max_ctx)
     pipe.defer_layer_tails = defer_tail
+    for layer in pipe.layers:
+        layer.fuse_rotation = layer.fuse_rotation and rotate_in_o
     del tensors, one, kinds
     if single:
         for i, c in enumerate(pipe.kv_caches):
@@ -845,7 +847,7 @@ def main():
     ap.add_argument("--no-defer-tail", action="store_true",
                     help="decode / model legs: every layer dispatches its own last step (default: it rides in the next layer's first dispatch)")
     ap.add_argument("--no-rotate-in-o", action="store_true",
-                    help="decode leg: the rotation back out of code space as a dispatch of its own (default: in the output projection's staging)")
+                    help="decode / model legs: the rotation back out of code space as a dispatch of its own (default: in the output projection's staging)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--legs", default="matvec,attention,sweep,layer,prefill,glue,decode,lanes,chunk,model,model_lanes",
                     help="comma-separated extra measurements to run besides the headline (for profiling one kernel at a time); "
@@ -951,7 +953,8 @@ def main():
         log(f"[bench] model decode, few lanes: {extra['model_decode_few_lanes_8k']}")
     if legs & {"model", "model_lanes"}:
         extra["model_decode_e2b_geometry"] = bench_model(pkg, ctx, K, max(args.steps, 20), args.warmup, single="model" in legs,
-                                                         lanes=64 if "model_lanes" in legs else 0, defer_tail=not args.no_defer_tail)
+                                                         lanes=64 if "model_lanes" in legs else 0, defer_tail=not args.no_defer_tail,
+                                                         rotate_in_o=not args.no_rotate_in_o)
         log("[bench] model decode:", extra["model_decode_e2b_geometry"])
 
     achieved = head["alg_bytes_per_launch"] / head["ms_per_launch_events"] * 1e-6

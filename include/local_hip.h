@@ -556,6 +556,19 @@ LH_API int lh_flash_attention_tq_rotated_into(lh_batch* batch, const lh_buffer* 
                                               uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
                                               uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window,
                                               uint32_t bits, uint32_t ring_capacity);
+/* lh_flash_attention_tq_rotated_into for a caller whose next kernel can do the rotation itself
+ * (lh_matvec_quant_rotated_into): where the rotation rides in the merge launch (2..32 partial
+ * records) it is done here, `out_f16` holds the rotated heads and *rotated is set to 1; otherwise
+ * no rotation kernel is launched, the f32 heads stay in `out`, still in code space, and *rotated
+ * is set to 0.  The choice depends on the shape arguments only, so it is the same at every call
+ * with the same shape (a recorded batch replays the choice made while it was recorded). */
+LH_API int lh_flash_attention_tq_rotated_lazy_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
+                                                   const lh_buffer* k_norms, const lh_buffer* v_codes,
+                                                   const lh_buffer* v_norms, const lh_buffer* levels,
+                                                   const lh_buffer* signs, lh_buffer* out, lh_buffer* out_f16,
+                                                   uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                                   uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window,
+                                                   uint32_t bits, uint32_t ring_capacity, int* rotated);
 LH_API int lh_flash_attention_tq_batched_rotated_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes,
                                                       const lh_buffer* k_norms, const lh_buffer* v_codes,
                                                       const lh_buffer* v_norms, const lh_buffer* levels,

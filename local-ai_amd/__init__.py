@@ -697,6 +697,20 @@ class Kernels:
                                                           _u32(num_q_heads), _u32(num_kv_heads), _u32(window),
                                                           _u32(bits), _u32(ring_capacity)))
 
+    def flash_attention_tq_rotated_lazy_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, signs, out, out_f16,
+                                             head_dim, kv_len, current_pos, num_q_heads, num_kv_heads, window, bits,
+                                             ring_capacity) -> bool:
+        """``flash_attention_tq_rotated_into`` that rotates only where the rotation rides in the merge launch.  True:
+        ``out_f16`` holds the rotated heads.  False: the f32 heads in ``out`` are still in code space and the caller's
+        next kernel rotates them (``matvec_quant_rotated_into``)."""
+        rotated = C.c_int(0)
+        _check(self._l.lh_flash_attention_tq_rotated_lazy_into(batch._h, rq._h, k_codes._h, k_norms._h, v_codes._h,
+                                                               v_norms._h, levels._h, signs._h, out._h, out_f16._h,
+                                                               _u32(head_dim), _u32(kv_len), _u32(current_pos),
+                                                               _u32(num_q_heads), _u32(num_kv_heads), _u32(window),
+                                                               _u32(bits), _u32(ring_capacity), C.byref(rotated)))
+        return bool(rotated.value)
+
     def flash_attention_tq_batched_rotated_into(self, batch, rq, k_codes, k_norms, v_codes, v_norms, levels, signs, out,
                                                 out_f16, positions, head_dim, lane_capacity, num_q_heads, num_kv_heads,
                                                 window, bits, n_lanes, ring_capacity):

@@ -400,6 +400,9 @@ __global__ __launch_bounds__(512) void attention_tq_reduce_rotate_kernel(const f
 struct RotateBack {
     const lh_buffer* signs;
     lh_buffer* out16;
+    // Lazy: rotate only where it rides in the merge launch (2 .. 32 partial records); otherwise leave the f32 heads in `out`
+    // unrotated and say so in *rotated, so that the caller's next kernel can rotate them while it stages them.
+    int* rotated = nullptr;
 };
 
 int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
@@ -475,6 +478,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
                            1.0f / std::sqrt((float)p.head_dim));
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
+        if (rot->rotated) *rot->rotated = 1;
         return r;
     }
     if (p.num_splits > 1) {
@@ -492,6 +496,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
         r = lh_check_launch(op);
         if (r == LH_OK) batch->dispatch_count++;
     }
+    if (rot && rot->rotated) { *rot->rotated = 0; return r; }
     if (rot && r == LH_OK) {
         r = lh_launch_hadamard_fh(ctx, (const float*)out->ptr, (const float*)rot->signs->ptr, (uint16_t*)rot->out16->ptr, p.head_dim,
                                   p.num_queries * p.num_q_heads);
@@ -569,6 +574,25 @@ int lh_flash_attention_tq_rotated_into(lh_batch* batch, const lh_buffer* rq, con
     const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
     const RotateBack rot{signs, out_f16};
     return attention_dispatch(batch, "flash_attention_tq_rotated", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys, &rot);
+}
+
+int lh_flash_attention_tq_rotated_lazy_into(lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,
+                                            const lh_buffer* v_codes, const lh_buffer* v_norms, const lh_buffer* levels, const lh_buffer* signs,
+                                            lh_buffer* out, lh_buffer* out_f16, uint32_t head_dim, uint32_t kv_len, uint32_t current_pos,
+                                            uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t window, uint32_t bits, uint32_t ring_capacity,
+                                            int* rotated) {
+    if (!rotated) return lh_fail(LH_ERR_INVALID_ARGUMENT, "flash_attention_tq_rotated_lazy: rotated is null");
+    *rotated = 0;
+    AttnParams p{};
+    p.head_dim = head_dim; p.bits = bits; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.kv_len = kv_len;
+    p.pos0 = current_pos; p.window = window; p.ring_capacity = ring_capacity; p.mode = kSingle; p.num_queries = 1;
+    const uint64_t seq = std::min<uint64_t>(kv_len, (uint64_t)current_pos + 1);
+    const uint64_t lo = (window > 0 && (uint64_t)current_pos + 1 > window) ? (uint64_t)current_pos + 1 - window : 0;
+    const uint64_t span = seq > lo ? seq - lo : 0;
+    const uint64_t phys = (ring_capacity ? std::min<uint64_t>(ring_capacity, seq) : seq) * num_kv_heads;
+    RotateBack rot{signs, out_f16};
+    rot.rotated = rotated;
+    return attention_dispatch(batch, "flash_attention_tq_rotated_lazy", rq, k_codes, k_norms, v_codes, v_norms, levels, out, nullptr, p, span, phys, &rot);
 }
 
 static int prefill_common(const char* op, lh_batch* batch, const lh_buffer* rq, const lh_buffer* k_codes, const lh_buffer* k_norms,

@@ -134,13 +134,15 @@ class QuantizedKvCache:
                                                 self.levels, self.signs, vacc, attn_out, hd, seq_len, current_pos,
                                                 n_q_heads, self.n_kv_heads, window, self.bits, self.ring_capacity())
 
-    def attention_codes_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, seq_len: int,
-                                          current_pos: int, n_q_heads: int, window: int) -> None:
-        """quant_cache.rs:571-589: the attend step alone; the f32 head outputs in ``vacc`` are still in code space (the
-        caller rotates them back, quant_cache.rs:590-598, e.g. inside the output projection)."""
-        kernels.flash_attention_tq_into(batch, rq, self.keys_q, self.key_norms, self.values_q, self.value_norms,
-                                        self.levels, vacc, self.head_dim, seq_len, current_pos, n_q_heads,
-                                        self.n_kv_heads, window, self.bits, self.ring_capacity())
+    def attention_from_rotated_lazy_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
+                                         seq_len: int, current_pos: int, n_q_heads: int, window: int) -> bool:
+        """quant_cache.rs:571-598 for a caller whose output projection can rotate its input itself: True when
+        ``attn_out`` holds the rotated f16 heads (the rotation rode in the merge launch), False when the f32 heads in
+        ``vacc`` are still in code space (quant_cache.rs:590-598 is left to the caller)."""
+        return kernels.flash_attention_tq_rotated_lazy_into(batch, rq, self.keys_q, self.key_norms, self.values_q,
+                                                            self.value_norms, self.levels, self.signs, vacc, attn_out,
+                                                            self.head_dim, seq_len, current_pos, n_q_heads,
+                                                            self.n_kv_heads, window, self.bits, self.ring_capacity())
 
     def prepare_rows_into(self, batch, kernels: Kernels, q: Buffer, k, v, q_norm, k_norm, rq: Buffer, start_pos: int,
                           n_rows: int, n_q_heads: int, eps: float, theta: float, partial_rotary_factor: float) -> None:

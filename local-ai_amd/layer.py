@@ -336,9 +336,9 @@ class TransformerLayer:
             kv_cache.prepare_token_into(batch, kernels, q_buf, k_buf if own_kv else None, v_buf if own_kv else None,
                                         w.q_norm, w.k_norm, s.rq, position, n_head, eps, p.rope_theta,
                                         p.partial_rotary_factor)
-            if rotate_in_o:   # the f32 head outputs stay in code space: step 3 rotates them while it stages them
-                kv_cache.attention_codes_from_rotated_into(batch, kernels, s.rq, s.vacc, seq_len, pos, n_head,
-                                                           p.sliding_window)
+            if rotate_in_o:   # where the rotation would be a launch of its own, step 3 does it while it stages the heads
+                rotate_in_o = not kv_cache.attention_from_rotated_lazy_into(batch, kernels, s.rq, s.vacc, s.attn_out,
+                                                                            seq_len, pos, n_head, p.sliding_window)
             else:
                 kv_cache.attention_from_rotated_into(batch, kernels, s.rq, s.vacc, s.attn_out, seq_len, pos, n_head,
                                                      p.sliding_window)

@@ -57,3 +57,23 @@ pub fn flash_split_count(eff_seq_len: u32) -> u32 {
     // SAFETY: pure function.
     unsafe { ffi::lh_flash_split_count(eff_seq_len) }
 }
+
+/// `lh_flash_attention_tq_rotated_lazy_into` (include/local_hip.h): the attend step of `fused_attention_into`
+/// (quant_cache.rs:571-589) and, where it rides in the merge launch, the rotation back out of code space
+/// (quant_cache.rs:590-598).  `Ok(true)`: `out_f16` holds the rotated heads.  `Ok(false)`: the f32 heads in `out` are still
+/// in code space and the caller's output projection rotates them (`Kernels::matvec_quant_rotated_into`).
+#[allow(clippy::too_many_arguments)]
+pub fn flash_attention_tq_rotated_lazy_into(batch: &mut CommandBatch, rq: &Buffer, k_codes: &Buffer, k_norms: &Buffer,
+                                            v_codes: &Buffer, v_norms: &Buffer, levels: &Buffer, signs: &Buffer, out: &Buffer,
+                                            out_f16: &Buffer, head_dim: u32, kv_len: u32, current_pos: u32, num_q_heads: u32,
+                                            num_kv_heads: u32, window: u32, bits: u32, ring_capacity: u32) -> Result<bool> {
+    let mut rotated: core::ffi::c_int = 0;
+    // SAFETY: every pointer comes from a live handle of this crate or from a local; the library validates sizes and shapes.
+    error::check(unsafe {
+        ffi::lh_flash_attention_tq_rotated_lazy_into(batch.as_ptr(), rq.as_ptr(), k_codes.as_ptr(), k_norms.as_ptr(),
+                                                     v_codes.as_ptr(), v_norms.as_ptr(), levels.as_ptr(), signs.as_ptr(),
+                                                     out.as_ptr(), out_f16.as_ptr(), head_dim, kv_len, current_pos,
+                                                     num_q_heads, num_kv_heads, window, bits, ring_capacity, &mut rotated)
+    })?;
+    Ok(rotated != 0)
+}

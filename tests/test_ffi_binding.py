@@ -20,6 +20,7 @@ TYPE_MAP = {
     "void*": "*mut c_void", "const void*": "*const c_void", "char*": "*mut c_char", "const char*": "*const c_char",
     "float*": "*mut f32", "const float*": "*const f32", "uint32_t*": "*mut u32", "const uint32_t*": "*const u32",
     "uint8_t*": "*mut u8", "const uint8_t*": "*const u8", "uint16_t*": "*mut u16", "const uint16_t*": "*const u16",
+    "int*": "*mut c_int",
 }
 for _h in ("lh_context", "lh_buffer", "lh_batch", "lh_event", "lh_graph"):
     TYPE_MAP[f"{_h}*"] = f"*mut {_h}"

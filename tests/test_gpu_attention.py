@@ -545,17 +545,29 @@ def test_rotated_entry_equals_attention_then_rotation(pkg, gpu, oracle, hd, T, w
     signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, T, nkv, hd, bits, 900 + T, ring=ring)
     rq = pkg.synth.rng(6, 15).standard_normal((nq, hd), dtype=np.float32)
     kcb, knb, vcb, vnb, lvb, rqb, sgb = upload(pkg, ctx, kc, kn, vc, vn, levels, rq, signs)
-    acc = [pkg.Buffer.empty(ctx, nq * hd * 4) for _ in range(2)]
-    o16 = [pkg.Buffer.from_slice(ctx, np.full(nq * hd + 32, 0x7BFF, np.uint16)) for _ in range(2)]
+    acc = [pkg.Buffer.empty(ctx, nq * hd * 4) for _ in range(3)]
+    o16 = [pkg.Buffer.from_slice(ctx, np.full(nq * hd + 32, 0x7BFF, np.uint16)) for _ in range(3)]
     batch = pkg.CommandBatch(ctx)
     K.flash_attention_tq_into(batch, rqb, kcb, knb, vcb, vnb, lvb, acc[0], hd, T, T - 1, nq, nkv, window, bits, ring)
     K.hadamard_rotate_fh_into(batch, acc[0], sgb, o16[0], hd, nq, False, True)
     K.flash_attention_tq_rotated_into(batch, rqb, kcb, knb, vcb, vnb, lvb, sgb, acc[1], o16[1], hd, T, T - 1, nq, nkv, window,
                                       bits, ring)
+    d0 = batch.dispatch_count()
+    rotated = K.flash_attention_tq_rotated_lazy_into(batch, rqb, kcb, knb, vcb, vnb, lvb, sgb, acc[2], o16[2], hd, T, T - 1, nq,
+                                                     nkv, window, bits, ring)
+    lazy_dispatches = batch.dispatch_count() - d0
     batch.commit_and_wait()
     two, one = o16[0].as_array(np.uint16), o16[1].as_array(np.uint16)
     assert (one[nq * hd:] == 0x7BFF).all()
     assert np.array_equal(one, two), f"{int((one != two).sum())} of {nq * hd} f16 outputs differ"
+    # the lazy form: either the rotated heads (the rotation rode in the merge launch), or the f32 heads of the attend step
+    # alone and nothing written to the f16 buffer -- never a rotation launch of its own
+    assert lazy_dispatches <= 2
+    if rotated:
+        assert np.array_equal(o16[2].as_array(np.uint16), two)
+    else:
+        assert (o16[2].as_array(np.uint16) == 0x7BFF).all()
+        assert np.array_equal(acc[2].as_array(np.uint32), acc[0].as_array(np.uint32))
     ref = oracle.attention_tq_codespace(rq, kc, kn, vc, vn, levels, hd, T, T - 1, nq, nkv, window, bits, ring)
     ref = oracle.hadamard_rotate(np.asarray(ref, np.float32).reshape(nq, hd), signs, hd, nq, False, True)
     check(one[:nq * hd].view(np.float16).astype(np.float32), np.asarray(ref, np.float32).reshape(-1), "rotated attention", 3e-3)
