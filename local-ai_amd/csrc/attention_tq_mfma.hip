@@ -896,9 +896,14 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
     // partial records.  It pays where a two-wave workgroup per CU would walk more than one group (one query over 32768
     // positions: 12.5-12.9 us against 13.9; over 131072: 16.5 against 20.0); where every workgroup has one group anyway the
     // longer set-up and the merge of the eight-wave workgroup cost more than they save (4096 positions: 12.5 against 10.6 us).
-    if (p.head_dim == 256 && pair_env <= 0 && (max_span + splits - 1) / splits > 64) {
-        uint64_t q = std::min<uint64_t>((max_span + 63) / 64, std::max<uint64_t>(1, (uint64_t)kQuad * ctx->cu_count / pairs));
+    // A few queries over at most eight groups each (one token over a sliding window of 512): one workgroup per query, one or
+    // two groups per pair of waves, and the kernel's output is final -- no records, no merge launch behind it.
+    const uint64_t groups = (max_span + 63) / 64;
+    const bool whole = pairs <= 8 && groups >= 2 && groups <= 2 * (uint64_t)kQuad;
+    if (p.head_dim == 256 && pair_env <= 0 && (whole || (max_span + splits - 1) / splits > 64)) {
+        uint64_t q = std::min<uint64_t>(groups, std::max<uint64_t>(1, (uint64_t)kQuad * ctx->cu_count / pairs));
         q -= q % kQuad;
+        if (whole) q = kQuad;
         while (q > (uint64_t)kQuad && (size_t)p.num_queries * p.num_q_heads * (q / kQuad) * rec > ws_floats) q -= kQuad;
         if (q >= (uint64_t)kQuad && (((max_span + q - 1) / q + 63) & ~(uint64_t)63) <= 128 &&
             (q == (uint64_t)kQuad || (size_t)p.num_queries * p.num_q_heads * (q / kQuad) * rec <= ws_floats)) {
