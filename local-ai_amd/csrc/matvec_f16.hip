@@ -5,6 +5,7 @@
 // One wave per row at a time, 16 bytes per lane and load, the activation vector staged once per workgroup in LDS
 // as f32; rows are dealt to the waves of the whole grid round robin so that the grid reads one advancing window.
 #include "common.hpp"
+#include <cstdlib>
 #include <algorithm>
 
 namespace {
@@ -23,7 +24,9 @@ template <typename XT> __device__ __forceinline__ float x_at(const XT* x, uint32
 template <> __device__ __forceinline__ float x_at<uint16_t>(const uint16_t* x, uint32_t i) { return lh_h2f(x[i]); }
 template <> __device__ __forceinline__ float x_at<float>(const float* x, uint32_t i) { return x[i]; }
 
-template <typename XT, typename YT, bool VEC, bool XLDS>
+// NL: 16-byte loads per lane and pass of the vector form (a pass covers 512 * NL columns).  FULL: cols is a multiple of
+// that, so no lane ever stands past the end of a row (no address clamps, no per-lane conditions in the loop).
+template <typename XT, typename YT, bool VEC, bool XLDS, int NL = 8, bool FULL = false>
 __global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restrict__ W, const XT* __restrict__ x, YT* __restrict__ y, uint32_t rows,
                                                         uint32_t cols) {
     extern __shared__ float xs[];
@@ -33,34 +36,63 @@ __global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restr
         __syncthreads();
     }
     auto xv = [&](uint32_t i) { return XLDS ? xs[i] : x_at<XT>(x, i); };
-    for (uint32_t row = blockIdx.x * nwaves + wave; row < rows; row += gridDim.x * nwaves) {
-        const uint16_t* wr = W + (size_t)row * cols;
+    if constexpr (VEC) {
+        // cols a multiple of 8 and 16-byte aligned rows.  A wave walks its rows in passes of 512 * NL columns, NL loads of
+        // 16 bytes per lane; the loads of the next pass (the next row, for rows of one pass) are issued before the arithmetic
+        // of the current one, so that a wave always has a pass on its way.  Addresses past the row's end are clamped (a load
+        // under a condition is followed by a wait for everything outstanding) and their values never used.
+        constexpr uint32_t kPass = 512u * NL;
+        const uint32_t ppr = (cols + kPass - 1) / kPass, row_step = gridDim.x * nwaves;
+        uint32_t row = blockIdx.x * nwaves + wave, pass = 0;
+        auto issue = [&](uint4 (&v)[NL], uint32_t r, uint32_t ps) {
+            const uint16_t* wr = W + (size_t)r * cols;
+#pragma unroll
+            for (int c = 0; c < NL; c++) {
+                const uint32_t k = lane * 8 + ps * kPass + 512 * c;
+                v[c] = lh_ld16_stream(wr + (FULL || k < cols ? k : cols - 8));
+            }
+        };
         float acc = 0.0f;
-        if (VEC) {   // cols a multiple of 8 and 16-byte aligned rows; up to 8 loads of 16 bytes in flight per lane
-            for (uint32_t k0 = lane * 8; k0 < cols; k0 += 8 * 512) {
-                uint4 v[8];
+        auto consume = [&](const uint4 (&v)[NL], uint32_t r, uint32_t ps) {
 #pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const uint32_t k = k0 + 512 * c;
-                    v[c] = k < cols ? lh_ld16_stream(wr + k) : make_uint4(0u, 0u, 0u, 0u);
-                }
+            for (int c = 0; c < NL; c++) {
+                const uint32_t k = lane * 8 + ps * kPass + 512 * c;
+                if (!FULL && k >= cols) break;
+                const uint32_t wv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
 #pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    const uint32_t k = k0 + 512 * c;
-                    if (k >= cols) break;
-                    const uint32_t wv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), xv(k + 2 * j), acc);
-                        acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] >> 16)), xv(k + 2 * j + 1), acc);
-                    }
+                for (int j = 0; j < 4; j++) {
+                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), xv(k + 2 * j), acc);
+                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] >> 16)), xv(k + 2 * j + 1), acc);
                 }
             }
-        } else {
-            for (uint32_t k = lane; k < cols; k += 64) acc = __builtin_fmaf(lh_h2f(wr[k]), xv(k), acc);
+            if (ps + 1 == ppr) {
+                const float total = lh_group_sum(acc, 64);
+                if (lane == 0) lh_store_from_f32<YT>(y, r, total);
+                acc = 0.0f;
+            }
+        };
+        auto step = [&](const uint4 (&cur)[NL], uint4 (&nxt)[NL]) {   // false: that was the wave's last pass
+            uint32_t nrow = row, npass = pass + 1;
+            if (npass == ppr) { npass = 0; nrow = row + row_step; }
+            const bool more = nrow < rows;
+            if (more) issue(nxt, nrow, npass);
+            consume(cur, row, pass);
+            row = nrow; pass = npass;
+            return more;
+        };
+        uint4 a[NL], b[NL];
+        if (row < rows) {
+            issue(a, row, 0);
+            while (step(a, b) && step(b, a)) {}
         }
-        acc = lh_group_sum(acc, 64);
-        if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
+    } else {
+        for (uint32_t row = blockIdx.x * nwaves + wave; row < rows; row += gridDim.x * nwaves) {
+            const uint16_t* wr = W + (size_t)row * cols;
+            float acc = 0.0f;
+            for (uint32_t k = lane; k < cols; k += 64) acc = __builtin_fmaf(lh_h2f(wr[k]), xv(k), acc);
+            acc = lh_group_sum(acc, 64);
+            if (lane == 0) lh_store_from_f32<YT>(y, row, acc);
+        }
     }
 }
 
@@ -70,13 +102,27 @@ int launch(lh_context* ctx, const uint16_t* W, const void* x, void* y, uint32_t 
     const bool xlds = cols <= (uint32_t)kMaxLdsCols;
     const uint32_t waves = 4;
     const uint64_t want = ((uint64_t)rows + waves - 1) / waves;
-    const uint32_t grid = (uint32_t)std::min<uint64_t>(want, (uint64_t)ctx->cu_count * 8);
+    const uint32_t grid = (uint32_t)std::min<uint64_t>(want, (uint64_t)ctx->cu_count * 8);   // (3 .. 12 workgroups per CU measure alike)
     const size_t lds = xlds ? (size_t)cols * 4 : 0;
-#define LH_F16MV(V, L) hipLaunchKernelGGL((matvec_f16_kernel<XT, YT, V, L>), dim3(grid), dim3(64 * waves), lds, ctx->stream, W, (const XT*)x, (YT*)y, rows, cols)
-    if (vec && xlds) LH_F16MV(true, true);
-    else if (vec) LH_F16MV(true, false);
-    else if (xlds) LH_F16MV(false, true);
-    else LH_F16MV(false, false);
+#define LH_F16MV(V, L, N, F) hipLaunchKernelGGL((matvec_f16_kernel<XT, YT, V, L, N, F>), dim3(grid), dim3(64 * waves), lds, ctx->stream, W, (const XT*)x, (YT*)y, rows, cols)
+#define LH_F16MV_N(L, N)                                                       \
+    do {                                                                       \
+        if (cols % (512u * N) == 0) LH_F16MV(true, L, N, true);                \
+        else LH_F16MV(true, L, N, false);                                      \
+    } while (0)
+#define LH_F16MV_VEC(L)                                       \
+    do {                                                      \
+        if (cols <= 512) LH_F16MV_N(L, 1);                    \
+        else if (cols <= 1024) LH_F16MV_N(L, 2);              \
+        else if (cols <= 2048) LH_F16MV_N(L, 4);              \
+        else LH_F16MV_N(L, 8);                                \
+    } while (0)
+    if (vec && xlds) LH_F16MV_VEC(true);
+    else if (vec) LH_F16MV_VEC(false);
+    else if (xlds) LH_F16MV(false, true, 8, false);
+    else LH_F16MV(false, false, 8, false);
+#undef LH_F16MV_N
+#undef LH_F16MV_VEC
 #undef LH_F16MV
     return LH_OK;
 }
