@@ -89,14 +89,14 @@ struct AttnShared {
 // HD = head_dim: 256 (one V wave) or 512 (two V waves, one per 64-byte half of a position's code).
 // ONE_KV: a single KV head (the measured configuration and the reference model): the distance between positions is a
 // compile-time constant, so the loads of a group take immediate offsets instead of per-load address arithmetic.
-// NQ = chunks per workgroup: 1, or 4 (head_dim 256): eight waves, a K wave and a V wave per chunk, each
+// NQ = chunks per workgroup: 1, or 2 or 4 (head_dim 256): four or eight waves, a K wave and a V wave per chunk, each
 // pair of waves with a hand-over area of its own; the query set-up is done once, by all eight, and the four partial results
 // are merged through LDS, so that a query cut into four chunks needs neither partial records nor a merge launch.  The
 // hand-over barriers are workgroup barriers, so every wave executes as many as the chunk with the most hand-overs needs.
 template <int NPL, int HD, bool ONE_KV, int PS, int NQ = 1>
 __device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>* shs, float alpha, float beta,
                                                float gam, float delta) {
-    static_assert(NQ == 1 || (NQ == 4 && HD == 256), "several chunks per workgroup: head_dim 256 only");
+    static_assert(NQ == 1 || ((NQ == 2 || NQ == 4) && HD == 256), "several chunks per workgroup: head_dim 256 only");
     const uint32_t wave_all = threadIdx.x >> 6;                   // wave of the workgroup (the set-up is dealt over all of them)
     const uint32_t sub = NQ == 1 ? 0u : wave_all >> 1;            // which of the workgroup's chunks this wave works on
     auto& sh = shs[sub];
@@ -163,7 +163,8 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     // runs a group ahead and hands its integer logit sums to the first, which adds its own and does the softmax -- and a V wave
     // per half of the V codes.
     // (Several chunks per workgroup: waves w and w + 4 share a SIMD, so chunks 0, 1 and chunks 2, 3 take opposite orders.)
-    const uint32_t role = NQ > 1 ? ((wave ^ (sub >> 1)) & 1u) : NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) & 3u;   // 0: K wave; 1, 2: V wave of code half role - 1; 3: second K wave
+    // (Two chunks per workgroup: two workgroups share a CU, and their order of roles follows the workgroup index.)
+    const uint32_t role = NQ == 4 ? ((wave ^ (sub >> 1)) & 1u) : NQ == 2 ? ((wave ^ blockIdx.x ^ blockIdx.y) & 1u) : NH == 1 ? ((wave ^ blockIdx.x) & 1u) : (wave + blockIdx.x) & 3u;   // 0: K wave; 1, 2: V wave of code half role - 1; 3: second K wave
     const bool k_role = role == 0 || role == 3;
     const bool kb_role = NH == 2 && role == 3;
     const uint32_t khalf = kb_role ? 1u : 0u;
@@ -798,12 +799,11 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         }
     }
     if constexpr (NQ > 1) {
-        // ---- the chunks' results merged: wave h takes head h, a lane four dims.  (R, l, acc) of a chunk are relative to
+        // ---- the chunks' results merged: a wave takes head h (two heads where the workgroup has four waves), a lane four dims.  (R, l, acc) of a chunk are relative to
         //      exp2(R); the result goes out as the final output (one workgroup per query) or as one partial record.
         static_assert(sizeof(sh.rqop) >= (size_t)kMaxGroupHeads * kHeadDim * sizeof(float), "the parked sums fit the operand area");
         __syncthreads();   // every chunk's sums are parked
-        const uint32_t h = wave_all;
-        if (h < group) {
+        for (uint32_t h = wave_all; h < group; h += 2 * NQ) {
             float Rq[NQ], gm = -INFINITY;
 #pragma unroll
             for (int q = 0; q < NQ; q++) { Rq[q] = shs[q].fin_r[h]; gm = fmaxf(gm, Rq[q]); }
@@ -847,20 +847,20 @@ __global__ __launch_bounds__(HD / 2, OCC) void attention_tq_mfma_kernel(AttnPoin
     else attention_body<2, HD, false, PS>(a, p, &sh, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
-// Four chunks of a query per workgroup (head_dim 256): 512 threads, the hand-over areas in dynamic LDS.
+// Four (or two) chunks of a query per workgroup (head_dim 256): 512 (256) threads, the hand-over areas in dynamic LDS.
 constexpr int kQuad = 4;
-template <int PS> constexpr size_t quad_lds_bytes() { return kQuad * sizeof(AttnShared<1, PS>); }
-template <int PS>
-__global__ __launch_bounds__(128 * kQuad, 2) void attention_tq_mfma_quad_kernel(AttnPointers a, AttnParams p) {
+template <int PS, int NQ = kQuad> constexpr size_t quad_lds_bytes() { return NQ * sizeof(AttnShared<1, PS>); }
+template <int PS, int NQ = kQuad>
+__global__ __launch_bounds__(128 * NQ, 2) void attention_tq_mfma_quad_kernel(AttnPointers a, AttnParams p) {
     extern __shared__ __align__(16) uint8_t quad_lds[];
     auto* shs = reinterpret_cast<AttnShared<1, PS>*>(quad_lds);
     const float L0 = a.levels[0], L1 = a.levels[1], L2 = a.levels[2], L3 = a.levels[3];   // as in attention_tq_mfma_kernel
     const float d_raw = (L3 - L2) - (L1 - L0);
     const float lmax = fmaxf(fmaxf(fabsf(L0), fabsf(L1)), fmaxf(fabsf(L2), fabsf(L3)));
     const float l_mean = 0.25f * ((L0 + L3) + (L1 + L2));
-    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, 256, false, PS, kQuad>(a, p, shs, L0, L1 - L0, L2 - L0, d_raw);
-    else if (p.num_kv_heads == 1) attention_body<2, 256, true, PS, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
-    else attention_body<2, 256, false, PS, kQuad>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    if (fabsf(d_raw) > 1e-5f * lmax || fabsf(l_mean) > 1e-6f * lmax) attention_body<3, 256, false, PS, NQ>(a, p, shs, L0, L1 - L0, L2 - L0, d_raw);
+    else if (p.num_kv_heads == 1) attention_body<2, 256, true, PS, NQ>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
+    else attention_body<2, 256, false, PS, NQ>(a, p, shs, L0 - 0.25f * d_raw, (L1 - L0) + 0.5f * d_raw, (L2 - L0) + 0.5f * d_raw, 0.0f);
 }
 
 }  // namespace
@@ -941,6 +941,16 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
         if (rl != LH_OK) return rl;
         p.num_splits = (uint32_t)(splits / kQuad);
         hipLaunchKernelGGL(attention_tq_mfma_quad_kernel<2>, dim3(p.num_splits, (uint32_t)pairs), dim3(128 * kQuad), quad_lds_bytes<2>(), ctx->stream, a, p);
+        return lh_check_launch(op);
+    }
+    // Two long chunks per query (512 sequences of 16384 positions): the same with two chunks per four-wave workgroup, two
+    // workgroups to a CU -- the query leaves the kernel as its final output.
+    if (p.head_dim == 256 && pair && splits == 2) {
+        constexpr size_t lds2 = quad_lds_bytes<2, 2>();
+        const int rl = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<2, 2>, lds2, op);
+        if (rl != LH_OK) return rl;
+        p.num_splits = 1;
+        hipLaunchKernelGGL((attention_tq_mfma_quad_kernel<2, 2>), dim3(1, (uint32_t)pairs), dim3(256), lds2, ctx->stream, a, p);
         return lh_check_launch(op);
     }
     const dim3 grid((uint32_t)splits, (uint32_t)pairs);
