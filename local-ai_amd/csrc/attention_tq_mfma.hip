@@ -865,6 +865,13 @@ __global__ __launch_bounds__(128 * NQ, 2) void attention_tq_mfma_quad_kernel(Att
 
 }  // namespace
 
+int lh_attention_kernels_init(lh_context* ctx) {
+    int r = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<1, kQuad>, quad_lds_bytes<1, kQuad>(), "context_create");
+    if (r == LH_OK) r = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<2, kQuad>, quad_lds_bytes<2, kQuad>(), "context_create");
+    if (r == LH_OK) r = lh_raise_dynamic_lds(ctx, (const void*)attention_tq_mfma_quad_kernel<2, 2>, quad_lds_bytes<2, 2>(), "context_create");
+    return r;
+}
+
 namespace lh_attn {
 
 bool mfma_supported(const AttnParams& p, const AttnPointers& a) {

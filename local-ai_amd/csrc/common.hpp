@@ -156,6 +156,8 @@ int lh_raise_dynamic_lds(lh_context* ctx, const void* kernel, size_t bytes, cons
 
 // Resolves the calling device's copy of the attention kernels' static scratch array (attention_tq.hip); the device must be current.
 int lh_attention_static_scratch_init(int device);
+// Raises the dynamic-LDS limit of the attention kernels that need more than the default (attention_tq_mfma.hip); ctx's device must be current.
+int lh_attention_kernels_init(lh_context* ctx);
 
 static inline size_t lh_dtype_size(lh_dtype t) { return t == LH_F32 ? 4 : 2; }
 

@@ -124,6 +124,8 @@ static void ctx_release(lh_context* ctx) {
     delete ctx;
 }
 
+void lh_context_destroy(lh_context* ctx);
+
 int lh_context_create(int device_index, lh_context** out) {
     if (!out) return lh_fail(LH_ERR_INVALID_ARGUMENT, "context_create: out is null");
     *out = nullptr;
@@ -187,6 +189,12 @@ int lh_context_create(int device_index, lh_context** out) {
             delete ctx;
             return lh_fail(LH_ERR_NO_COMMAND_QUEUE, "hipEventCreate");
         }
+    }
+    // The attention kernels with hand-over areas in dynamic LDS get their limit raised here, so that no launch -- in
+    // particular none inside a recorded batch or from the entry that may not allocate -- has to do it.
+    {
+        const int ra = lh_attention_kernels_init(ctx);
+        if (ra != LH_OK) { lh_context_destroy(ctx); return ra; }
     }
     *out = ctx;
     return LH_OK;
