@@ -159,7 +159,8 @@ def test_attention_sink_with_flat_tail(pkg, gpu, oracle, T, sink):
 @pytest.mark.parametrize("seed", [1, 2, 3])
 def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
     """Sixty random shapes per seed -- decode, batched lanes and prefill rows; head_dim 256 / 512; 1, 4, 6 or 8 query heads
-    per KV head over one or two KV heads; context lengths around the 64- and 128-position boundaries and up to 9000;
+    per KV head over one or two KV heads; context lengths around the 64- and 128-position boundaries and up to 33000
+    (long enough for the eight-wave workgroups of several chunks, with one-group and with pair hand-overs);
     windows, wrapped rings; peaked to nearly uniform queries; now and then a level table that needs the third bit plane --
     over caches of random code bytes and norms (any code bytes and positive f16 norms are a valid cache)."""
     ctx, K = gpu
@@ -171,7 +172,7 @@ def test_randomised_shapes_match_oracle(pkg, gpu, oracle, seed):
         nkv = int(g.choice([1, 1, 2]))
         nq = nkv * int(g.choice([8, 8, 4, 1, 6]))
         mode = int(g.choice([0, 0, 1, 2]))          # 0 decode, 1 batched, 2 prefill
-        T = int(g.choice([1, 63, 64, 65, 127, 128, 129, 255, 300, 1000, 1025, 2049, 4096, 5000, 9000]))
+        T = int(g.choice([1, 63, 64, 65, 127, 128, 129, 255, 300, 1000, 1025, 2049, 4096, 5000, 9000, 20000, 33000]))
         T = max(1, T + int(g.integers(-2, 3)))
         window = int(g.choice([0, 0, 64, 100, 512, 1024, 3000]))
         ring = 0
