@@ -97,7 +97,15 @@ template <int NPL, int HD, bool ONE_KV, int PS, int NQ = 1>
 __device__ __forceinline__ void attention_body(const AttnPointers& a, const AttnParams& p, AttnShared<(HD / 256), PS>* shs, float alpha, float beta,
                                                float gam, float delta) {
     static_assert(NQ == 1 || ((NQ == 2 || NQ == 4) && HD == 256), "several chunks per workgroup: head_dim 256 only");
-    const uint32_t wave_all = threadIdx.x >> 6;                   // wave of the workgroup (the set-up is dealt over all of them)
+    // The wave's index as a scalar: what follows from it -- the chunk, its groups, their ring slots, the roles -- is uniform
+    // over the wave, and the compiler keeps it in scalar registers and scalar branches only if it can see that (per pair
+    // hand-over 36 vector instructions fewer on the K wave and 116 on the V wave of a several-chunk workgroup).  That is
+    // what the latency-bound launches want (one query over 32768 positions: 12.2-12.4 against 12.5-12.7 us; over 131072:
+    // 16.0 against 16.6).  The several-chunk workgroups with pair hand-overs keep the index as it comes: with the scalar
+    // form the 256 x 32768 launch measured 2.4 % SLOWER in alternating runs on one box (0.612-0.613 against 0.627), the
+    // other batched points within their run-to-run spread; the cause was not found.
+    const uint32_t wave_raw = threadIdx.x >> 6;
+    const uint32_t wave_all = (NQ > 1 && PS == 2) ? wave_raw : (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_raw);   // wave of the workgroup (the set-up is dealt over all of them)
     const uint32_t sub = NQ == 1 ? 0u : wave_all >> 1;            // which of the workgroup's chunks this wave works on
     auto& sh = shs[sub];
     auto& s_rqop = shs[0].rqop;
