@@ -364,10 +364,15 @@ __global__ __launch_bounds__(512, 2) void attention_tq_prefill_tile_kernel(AttnP
         // produce(G): weights of tile G, then tile G + 1 staged (its buffers were last read before the previous barrier)
         auto produce = [&](uint32_t G) {
             const uint32_t buf = (G - g_first) & 1;
+            // Phase A runs at a raised wave priority: the SIMD's other wave is in phase B or staging meanwhile, and the
+            // weights of phase A are what every wave's next phase B waits for behind the barrier (118 -> 113 us for 256 rows
+            // over 32768 positions; the priority on phase B or on the staging changes nothing).
+            __builtin_amdgcn_s_setprio(1);
             if (pair_on) {
                 if (tile_full(G)) phase_a(buf, G, std::true_type{});
                 else phase_a(buf, G, std::false_type{});
             }
+            __builtin_amdgcn_s_setprio(0);
             if (G < g_last) {
                 stage(buf ^ 1, (G + 1 - g_first) & 3);
                 nk_c = nk_n; nv_c = nv_n;
