@@ -353,12 +353,16 @@ __global__ __launch_bounds__(kWG, 2) void matvec_quant_kernel(const MatvecProble
         for (; st < st_end; st += U) {
             float part[U];
             if constexpr (IMG) {
+                __builtin_amdgcn_s_setprio(0);        // (raised below, once the step's data is in the image)
                 __builtin_amdgcn_wave_barrier();      // the units of the previous step have been read
 #pragma unroll
                 for (int i = 0; i < kImgLoads; i++)
                     if ((uint32_t)lane + 64 * i < step_chunks) *reinterpret_cast<u32x4_t*>(image + ((uint32_t)lane + 64 * i) * 16) = pre[i];
                 __builtin_amdgcn_wave_barrier();
                 if (st + U < st_end) prefetch(st + U);
+                // The wave has what it needs for this step and runs it at a raised priority: of the waves of a SIMD the one
+                // that can finish a step does, and reaches its next wait, and the loads behind it, sooner.
+                __builtin_amdgcn_s_setprio(1);
 #pragma unroll
                 for (int u = 0; u < U; u++) {
                     part[u] = 0.0f;
