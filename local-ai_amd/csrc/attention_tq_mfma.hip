@@ -282,9 +282,11 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
     if (k_role) {
         // The K waves of the long-chunk forms that step through workgroup barriers run at a raised priority: they produce
         // what the V waves of the next step wait for (256 x 32768 positions: +2-2.5 % in alternating runs; head_dim 512,
-        // 128 x 32768: +2-4 %).  The two-wave workgroups of head_dim 256 lose with it (2016 x 4096: -8 %; the batched
-        // 512-position window: -5 %) and keep the default.
-        if constexpr (PS == 2 && (NQ > 1 || NH == 2)) __builtin_amdgcn_s_setprio(1);
+        // 128 x 32768: +2-4 %), and so do those of the eight-wave workgroups with one-group hand-overs (one query over a
+        // 512-position window: 11.15 -> 10.67 us).  The two-wave workgroups of head_dim 256 lose with it (2016 x 4096: -8 %;
+        // the batched 512-position window: -5 %; a raised priority for their V waves instead: -3 % and -4 %) and keep the
+        // default.
+        if constexpr (NQ > 1 || (PS == 2 && NH == 2)) __builtin_amdgcn_s_setprio(1);
         // =================================================================== K wave
         float cs[2], ca[2];   // logit (log2 domain) = norm_k*log2e * (cs * int + ca) for the lane's two heads g, g + 4
 #pragma unroll
