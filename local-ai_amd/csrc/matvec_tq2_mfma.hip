@@ -80,6 +80,17 @@ struct Tq2Base {
     uint32_t* fault = nullptr;
 };
 
+// The kernel's arguments as they lie in its argument segment.  The ones that only the staging of a vector and the bounded
+// wait read (the prologue, the poll limit, the fault word) are fetched from there where they are used, through a pointer
+// the compiler cannot see through: held in scalar registers for the whole kernel they cost the main loop spills.
+struct Tq2KernArgs { const Tq2Problem* problems; Tq2Base single; uint32_t count, rows, K; };
+typedef const __attribute__((address_space(4))) Tq2KernArgs* kernargs_t;
+__device__ __forceinline__ kernargs_t cold_kernargs() {
+    kernargs_t ka = (kernargs_t)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ka));
+    return ka;
+}
+
 __device__ __forceinline__ u32x4_t ld16_align2_cached(gptr_t p) {
     typedef u32x4_t __attribute__((aligned(2))) u32x4_a2;
     return *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a2*>(p);
@@ -120,7 +131,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     const XResidual resid{xq2, xs + 2 * nb, xn + 2 * nb};
     const uint32_t kq = plane_bytes(K) >> 2;                        // dwords between the low-limb and the high-limb plane
     const uint32_t row_bytes = nb * 66;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), nwaves = blockDim.x >> 6;
     const uint32_t r = lane & 15, g = lane >> 4;                    // A layout: row r, quarter g
     const uint32_t c = lane & 15;                                   // B / D layout: column c, k-group / row-group g
     const uint32_t cb = c >> 1, cl = c & 1;                         // column's block (within a group of 8) and limb
@@ -146,7 +157,7 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     const uint32_t ngroups = (nb + 7) >> 3;
     const uint64_t my_slots = blockIdx.x < total_slots ? (total_slots - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
     const uint32_t grp0 = splitk ? (uint32_t)wave % sw : 0u, grp_step = sw;
-    const uint64_t nitems = my_slots * (ngroups / grp_step);        // one item = one (tile, block group)
+    const uint32_t nitems = (uint32_t)(my_slots * (ngroups / grp_step));   // one item = one (tile, block group); the host keeps a launch's total under 2^32
 
     // Chunk -> (row, chunk-in-row) of the lane's staging loads.  Full groups of 8 blocks (33 chunks per row): the global
     // offsets live in registers and the image offsets are linear in the chunk index.  The trailing group of nb % 8
@@ -236,13 +247,18 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     }
     const void* staged = nullptr;
     float rowacc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (uint64_t n = 0; n < nitems; n++) {
+    for (uint32_t n = 0; n < nitems; n++) {
         uint32_t grp, tile; Tq2Problem pb;
         item_tile_base(cur, grp, tile, pb);
         const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
-            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, single.pro, &resid, kq);
+            const kernargs_t ka = cold_kernargs();
+            XPrologue pro;
+            pro.kind = ka->single.pro.kind; pro.aux = ka->single.pro.aux; pro.eps = ka->single.pro.eps; pro.res = ka->single.pro.res;
+            pro.aux2 = ka->single.pro.aux2; pro.store = ka->single.pro.store; pro.tail = ka->single.pro.tail;
+            pro.scale = ka->single.pro.scale; pro.signs = ka->single.pro.signs; pro.head_dim = ka->single.pro.head_dim;
+            quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, pro, &resid, kq);
             __syncthreads();
             staged = pb.vector;
         }
@@ -373,15 +389,20 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
                 // outstanding global loads -- the next tile's prefetch -- and is deliberately not used.
                 auto lds_order = [] { __builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory"); };   // lgkmcnt(0) only
                 if (gen) {   // the slot's previous use must have been summed (bounded wait: never expected to run out)
-                    uint32_t spins = 0;
-                    bool seen;
-                    while (!(seen = __hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == gen) &&
-                           spins++ < single.spin_limit)
-                        __builtin_amdgcn_s_sleep(2);
-                    // Out of patience: the wave goes on (every wave must reach the end of the kernel), the rows of this tile
-                    // are not to be trusted, and the host learns of it at its next wait on the stream.
-                    if (!seen && lane == 0 && single.fault)
-                        __hip_atomic_store(single.fault, (uint32_t)LH_FAULT_TQ2_SPLIT_WAIT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    bool seen = __hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == gen;
+                    if (!seen) {
+                        const kernargs_t ka = cold_kernargs();
+                        const uint32_t spin_limit = ka->single.spin_limit;
+                        uint32_t spins = 0;
+                        while (!(seen = __hip_atomic_load(&sync[kRing + ring], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == gen) &&
+                               spins++ < spin_limit)
+                            __builtin_amdgcn_s_sleep(2);
+                        // Out of patience: the wave goes on (every wave must reach the end of the kernel), the rows of this
+                        // tile are not to be trusted, and the host learns of it at its next wait on the stream.
+                        uint32_t* fault = ka->single.fault;
+                        if (!seen && lane == 0 && fault)
+                            __hip_atomic_store(fault, (uint32_t)LH_FAULT_TQ2_SPLIT_WAIT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    }
                     lds_order();
                 }
                 if (c == 0) {
@@ -461,6 +482,8 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     const uint64_t cap = (uint64_t)ctx->cu_count * wg_eff;
     const uint32_t grid = (uint32_t)(slots < cap ? (slots ? slots : 1) : cap);
     if (lds_bytes > kMaxLdsBytes) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: cols %u need %zu bytes of LDS", K, lds_bytes);
+    if ((slots / grid + 1) * ngroups > 0xFFFFFFFFull)   // the kernel counts a workgroup's (tile, block group) items in 32 bits
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems of %u rows are more than one launch takes", count, rows);
     const void* fn;
     if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
 #define LH_FN(XT, YT) (wide_split ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true, 768, true>                                       \
