@@ -170,19 +170,6 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     uint16_t* full_tab = tail_tab + 2 * kStageLoads * 64;
     if (splitk && threadIdx.x < kMaxWavesPerWG * 2 * kRing)   // arrival counts and generations of the partial-sum rings
         reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxWavesPerWG * 16)[threadIdx.x] = 0u;
-    if (wave == 0) {
-        const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
-#pragma unroll
-        for (int i = 0; i < kStageLoads; i++) {
-            const uint32_t ch = lane + 64 * i;
-            const uint32_t cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
-            full_tab[i * 64 + lane] = (uint16_t)(rf * row_bytes + jf * 16);
-            const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
-            tail_tab[i * 64 + lane] = (uint16_t)(rt * row_bytes + jt * 16);
-            tail_tab[(kStageLoads + i) * 64 + lane] = ch < 16 * nch_t ? (uint16_t)(rt * ss_t + jt * 16) : (uint16_t)0xFFFFu;   // surplus lanes do not store
-        }
-    }
-    __syncthreads();
     // Position in the work order, advanced incrementally (all scalar, no division in the loop).
     struct Item { uint32_t grp, sip, prob; };                       // block group, slot within the problem, problem
     const uint32_t step_prob = gridDim.x / slots_per_problem, step_sip = gridDim.x % slots_per_problem;
@@ -239,11 +226,39 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
         }
     };
 
-    {
+    // The first item's loads go out ahead of the tables where they need none (a full group of a full tile): the lane's nine
+    // offsets are computed here once; the loop reads them from the table, which costs no registers.
+    bool first_issued = false;
+    if (nitems) {
+        uint32_t grp, tile; Tq2Problem pb;
+        item_tile_base(cur, grp, tile, pb);
+        if (!(grp + 1 == ngroups && (nb & 7)) && (tile << 4) + 16 <= rows) {
+            uint32_t offs[kStageLoads];
+#pragma unroll
+            for (int i = 0; i < kStageLoads; i++) {
+                const uint32_t ch = lane + 64 * i, cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
+                offs[i] = rf * row_bytes + jf * 16;
+            }
+            prefetch(cur, offs);
+            first_issued = true;
+        }
+    }
+    {   // every thread fills its share of the tables (one wave doing all nine rounds is a microsecond at the head of a launch)
+        const uint32_t nch_t = (nbg_tail * 66 + 15) >> 4, ss_t = (nch_t | 1) * 16;
+        for (uint32_t ch = threadIdx.x; ch < kStageLoads * 64; ch += blockDim.x) {
+            const uint32_t cf = ch < 16 * 33 ? ch : 16 * 33 - 1, rf = cf / 33, jf = cf - rf * 33;
+            full_tab[ch] = (uint16_t)(rf * row_bytes + jf * 16);
+            const uint32_t ct = ch < 16 * nch_t ? ch : 16 * nch_t - 1, rt = ct / nch_t, jt = ct - rt * nch_t;
+            tail_tab[ch] = (uint16_t)(rt * row_bytes + jt * 16);
+            tail_tab[kStageLoads * 64 + ch] = ch < 16 * nch_t ? (uint16_t)(rt * ss_t + jt * 16) : (uint16_t)0xFFFFu;   // surplus lanes do not store
+        }
+    }
+    __syncthreads();
+    if (nitems && !first_issued) {
         uint32_t offs[kStageLoads];
 #pragma unroll
         for (int i = 0; i < kStageLoads; i++) offs[i] = full_tab[i * 64 + lane];
-        if (nitems) prefetch(cur, offs);
+        prefetch(cur, offs);
     }
     const void* staged = nullptr;
     float rowacc[4] = {0.f, 0.f, 0.f, 0.f};
