@@ -362,6 +362,7 @@ __global__ __launch_bounds__(512) void attention_tq_reduce_rotate_kernel(const f
     const uint32_t qh = blockIdx.x, d = threadIdx.x;
     const size_t rec = partial_record_floats(head_dim);
     const float* base = ws + (size_t)qh * num_splits * rec;
+    const float sign = signs[d];   // requested with the records, not behind the transform's barriers
     float v[2 * kReduceBatch];
 #pragma unroll
     for (int i = 0; i < 2 * kReduceBatch; i++) v[i] = (uint32_t)i < num_splits ? base[(size_t)i * rec + 4 + d] : 0.0f;
@@ -392,7 +393,7 @@ __global__ __launch_bounds__(512) void attention_tq_reduce_rotate_kernel(const f
     sh[d] = t * inv;
     lh_fwht_lds(sh, head_dim, d);
     float y = __fmul_rn(sh[d], inv_sqrt_d);
-    y = __fmul_rn(y, signs[d]);
+    y = __fmul_rn(y, sign);
     out[(size_t)qh * head_dim + d] = lh_f2h_exact(y);
 }
 

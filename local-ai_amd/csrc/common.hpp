@@ -256,15 +256,40 @@ __device__ __forceinline__ float lh_norm_tail(float normed, float res, uint32_t 
     return tail == 2 ? (float)sum * scale : (float)sum;
 }
 
-// In-place unnormalised fast Walsh-Hadamard transform over sh[0..d) in LDS with one thread per element; every thread of
-// the workgroup calls it.  Sums and differences only, in a fixed order, so every kernel that uses it produces the same bits.
+// The value of the lane LEN away (lane ^ LEN; LEN a power of two below 64).
+template <int LEN>
+__device__ __forceinline__ float lh_lane_xor_f(float v) {
+    if constexpr (LEN == 1) return lh_dpp_f<LH_DPP_QUAD_XOR1>(v);
+    else if constexpr (LEN == 2) return lh_dpp_f<LH_DPP_QUAD_XOR2>(v);
+    else if constexpr (LEN <= 16) return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x1F | (LEN << 10)));
+    else return __shfl_xor(v, 32, 64);
+}
+template <int LEN>
+__device__ __forceinline__ float lh_fwht_lane_stage(float v, uint32_t lane) {
+    const float other = lh_lane_xor_f<LEN>(v);
+    return (lane & LEN) ? __fsub_rn(other, v) : __fadd_rn(v, other);
+}
+
+// In-place unnormalised fast Walsh-Hadamard transform over sh[0..d) in LDS with one thread per element (thread `lane`
+// has just written sh[lane] itself); every thread of the workgroup calls it.  Sums and differences only, in a fixed order
+// (pairs 1 apart first, then 2, 4, ...), so every kernel that uses it produces the same bits.  The stages that pair
+// elements of one wave exchange them between lanes; only those 64 and more apart go through LDS and a barrier.
 __device__ __forceinline__ void lh_fwht_lds(float* sh, uint32_t d, uint32_t lane) {
-    for (uint32_t len = 1; len < d; len <<= 1) {
+    float v = sh[lane];
+    if (d > 1) v = lh_fwht_lane_stage<1>(v, lane);
+    if (d > 2) v = lh_fwht_lane_stage<2>(v, lane);
+    if (d > 4) v = lh_fwht_lane_stage<4>(v, lane);
+    if (d > 8) v = lh_fwht_lane_stage<8>(v, lane);
+    if (d > 16) v = lh_fwht_lane_stage<16>(v, lane);
+    if (d > 32) v = lh_fwht_lane_stage<32>(v, lane);
+    for (uint32_t len = 64; len < d; len <<= 1) {
+        sh[lane] = v;
         __syncthreads();
-        const float self_v = sh[lane], other_v = sh[lane ^ len];
+        const float other_v = sh[lane ^ len];
         __syncthreads();
-        sh[lane] = (lane & len) ? __fsub_rn(other_v, self_v) : __fadd_rn(self_v, other_v);
+        v = (lane & len) ? __fsub_rn(other_v, v) : __fadd_rn(v, other_v);
     }
+    sh[lane] = v;
     __syncthreads();
 }
 __device__ __forceinline__ float lh_bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }

@@ -42,7 +42,8 @@ constexpr uint32_t kImageBytes = 16 * (kMaxChunksPerRow * 16 + 16) + 32;   // pa
 // in between and fetched again (1.09 x the bytes with plain loads against 1.03 x, 5.3 against 5.5 TB/s).
 constexpr uint32_t kRing = 1;
 constexpr uint32_t kMaxWavesPerWG = 12;       // the largest workgroup launched here
-constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxWavesPerWG * 16 * 4 + (size_t)kMaxWavesPerWG * 2 * kRing * 4;   // partial rows + arrival / generation words per tile of a slot
+constexpr size_t kProWords = sizeof(XPrologue) / 4;   // the prologue's words, kept in LDS behind the split area (see cold_kernargs)
+constexpr size_t kSplitAreaBytes = (size_t)kRing * kMaxWavesPerWG * 16 * 4 + (size_t)kMaxWavesPerWG * 2 * kRing * 4 + ((kProWords * 4 + 15) & ~(size_t)15);   // partial rows + arrival / generation words per tile of a slot + the prologue
 constexpr size_t kMaxLdsBytes = 160 * 1024;   // most dynamic LDS a launch here asks for: all a CU has
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
@@ -81,8 +82,10 @@ struct Tq2Base {
 };
 
 // The kernel's arguments as they lie in its argument segment.  The ones that only the staging of a vector and the bounded
-// wait read (the prologue, the poll limit, the fault word) are fetched from there where they are used, through a pointer
-// the compiler cannot see through: held in scalar registers for the whole kernel they cost the main loop spills.
+// wait read (the prologue, the poll limit, the fault word) are not taken from the argument registers: held in scalar
+// registers for the whole kernel they cost the main loop spills.  The prologue is copied to LDS at the head of the kernel
+// and read back where a vector is staged; the other two are fetched from the segment on the path that never runs, through
+// a pointer the compiler cannot see through.
 struct Tq2KernArgs { const Tq2Problem* problems; Tq2Base single; uint32_t count, rows, K; };
 typedef const __attribute__((address_space(4))) Tq2KernArgs* kernargs_t;
 __device__ __forceinline__ kernargs_t cold_kernargs() {
@@ -168,8 +171,11 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
     // (16-bit entries: row offsets stay below 15 * 3168 + 528 bytes for the widest row this kernel takes)
     uint16_t* tail_tab = reinterpret_cast<uint16_t*>(lds + zero_off + 128 + (size_t)nwaves * kImageBytes);   // [3][kStageLoads][64]
     uint16_t* full_tab = tail_tab + 2 * kStageLoads * 64;
-    if (splitk && threadIdx.x < kMaxWavesPerWG * 2 * kRing)   // arrival counts and generations of the partial-sum rings
-        reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxWavesPerWG * 16)[threadIdx.x] = 0u;
+    uint32_t* const sync_words = reinterpret_cast<uint32_t*>(reinterpret_cast<float*>(tail_tab + 3 * kStageLoads * 64) + kRing * kMaxWavesPerWG * 16);
+    if (splitk && threadIdx.x < kMaxWavesPerWG * 2 * kRing) sync_words[threadIdx.x] = 0u;   // arrival counts and generations of the partial-sum rings
+    uint32_t* const pro_words = sync_words + kMaxWavesPerWG * 2 * kRing;
+    if (threadIdx.x < kProWords)
+        pro_words[threadIdx.x] = reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(&cold_kernargs()->single.pro)[threadIdx.x];
     // Position in the work order, advanced incrementally (all scalar, no division in the loop).
     struct Item { uint32_t grp, sip, prob; };                       // block group, slot within the problem, problem
     const uint32_t step_prob = gridDim.x / slots_per_problem, step_sip = gridDim.x % slots_per_problem;
@@ -268,11 +274,10 @@ __global__ __launch_bounds__(MAXT, MAXT == 256 ? 2 : 1) void matvec_tq2_mfma_ker
         const Item nxt = advance(cur);
         if (pb.vector != staged) {                                   // uniform over the workgroup
             __syncthreads();
-            const kernargs_t ka = cold_kernargs();
-            XPrologue pro;
-            pro.kind = ka->single.pro.kind; pro.aux = ka->single.pro.aux; pro.eps = ka->single.pro.eps; pro.res = ka->single.pro.res;
-            pro.aux2 = ka->single.pro.aux2; pro.store = ka->single.pro.store; pro.tail = ka->single.pro.tail;
-            pro.scale = ka->single.pro.scale; pro.signs = ka->single.pro.signs; pro.head_dim = ka->single.pro.head_dim;
+            struct ProWords { uint32_t w[kProWords]; } words;
+#pragma unroll
+            for (uint32_t i = 0; i < kProWords; i++) words.w[i] = (uint32_t)__builtin_amdgcn_readfirstlane((int)pro_words[i]);
+            const XPrologue pro = __builtin_bit_cast(XPrologue, words);
             quantize_x_to_lds<kL, 256, XT>(static_cast<const XT*>(pb.vector), K, xq, xs, xn, blockDim.x, pro, &resid, kq);
             __syncthreads();
             staged = pb.vector;

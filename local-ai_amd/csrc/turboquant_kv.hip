@@ -43,11 +43,23 @@ struct EncodeParams {
     float inv_sqrt_d;
 };
 
+// The 2^bits <= 16 codec levels as values, requested at the top of a kernel (uniform addresses: scalar loads), so that the
+// level search at the end of an encode does not start a trip to memory of its own; entries past 2^bits are +inf and never win.
+struct LevelTable { float v[16]; };
+__device__ __forceinline__ LevelTable load_levels(const float* __restrict__ levels, uint32_t bits) {
+    LevelTable t;
+    const uint32_t k = 1u << bits;
+#pragma unroll
+    for (int i = 0; i < 16; i++) t.v[i] = (uint32_t)i < k ? levels[i] : INFINITY;
+    return t;
+}
+
 // TurboQuant encode of one vector held one coordinate per thread (turboquant.rs:241-276): norm, unit vector, signs,
 // FWHT, 1/sqrt(d), nearest level, bit packing.  `sh` and `code_sh` are workgroup arrays of at least d entries; the
-// calling kernel runs d threads.
+// calling kernel runs d threads.  `sign` is the lane's entry of the sign vector and `lv` the level table, both loaded by
+// the caller ahead of its own work: behind the barriers here each would cost a round trip to memory.
 __device__ __forceinline__ void encode_vector(float xv, uint32_t lane, uint32_t d, float* sh, uint32_t* code_sh,
-                                              const float* __restrict__ signs, const float* __restrict__ levels, uint32_t bits,
+                                              const float sign, const LevelTable& lv, uint32_t bits,
                                               uint32_t code_bytes, float inv_sqrt_d, uint8_t* __restrict__ packed_slot,
                                               uint16_t* __restrict__ norm_slot) {
     // norm = sqrt(fold(+, x_i * x_i)) in index order; every thread walks the same LDS
@@ -66,17 +78,17 @@ __device__ __forceinline__ void encode_vector(float xv, uint32_t lane, uint32_t 
     const float norm = __fsqrt_rn(sq);
     float v = xv;
     if (norm > 0.0f) v = __fmul_rn(v, __fdiv_rn(1.0f, norm));
-    v = __fmul_rn(v, signs[lane]);
+    v = __fmul_rn(v, sign);
     __syncthreads();
     sh[lane] = v;
     fwht_lds(sh, d, lane);
     const float y = __fmul_rn(sh[lane], inv_sqrt_d);
 
-    const uint32_t k = 1u << bits;
     uint32_t best = 0;
     float bd = INFINITY;
-    for (uint32_t i = 0; i < k; ++i) {
-        const float dd = fabsf(__fsub_rn(y, levels[i]));
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float dd = fabsf(__fsub_rn(y, lv.v[i]));
         if (dd < bd) { bd = dd; best = i; }
     }
     code_sh[lane] = best;
@@ -104,6 +116,8 @@ __global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* 
     __shared__ __align__(16) float sh[kMaxHeadDim];
     __shared__ uint32_t code_sh[kMaxHeadDim];
     const uint32_t d = p.head_dim, lane = threadIdx.x, group = blockIdx.x;
+    const float xv = lh_h2f(input[(size_t)group * d + lane]), sign = signs[lane];
+    const LevelTable lv = load_levels(levels, p.bits);
     const uint32_t tok = group / p.n_kv_heads, head = group - tok * p.n_kv_heads;
     uint32_t g;
     if (BATCHED) {
@@ -114,8 +128,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* 
         const uint32_t logical = p.position + tok;
         g = (p.ring_capacity ? logical % p.ring_capacity : logical) * p.n_kv_heads + head;
     }
-    encode_vector(lh_h2f(input[(size_t)group * d + lane]), lane, d, sh, code_sh, signs, levels, p.bits, p.code_bytes, p.inv_sqrt_d,
-                  packed + (size_t)g * p.code_bytes, norms + g);
+    encode_vector(xv, lane, d, sh, code_sh, sign, lv, p.bits, p.code_bytes, p.inv_sqrt_d, packed + (size_t)g * p.code_bytes, norms + g);
 }
 
 // ---- single-token Q / K / V preparation in one dispatch ---------------------------------------------------------
@@ -155,7 +168,13 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     const uint16_t* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
     const bool normalise = !(is_q || is_k) || norm_w != nullptr;          // V always (unit weight); Q / K when the layer has the weight
 
+    // Everything the workgroup reads from memory is requested here, in one trip: behind the barriers below each load
+    // would be a round trip of its own (the norm weight, the sign, the levels: three of them on the K and V path).
     const uint16_t raw = vec[lane];
+    const float norm_weight = norm_w ? lh_h2f(norm_w[lane]) : 1.0f;
+    const float sign = signs[lane];
+    LevelTable lv;
+    if (!is_q && p.write_kv) lv = load_levels(levels, p.bits);
     uint16_t h = raw;
     if (normalise) {
         const float x = lh_h2f(raw);
@@ -165,7 +184,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
         float ss = 0.0f;
         for (uint32_t w = 0; w < d / 64; w++) ss += wsum[w];
         const float rms = rsqrtf(ss / (float)d + p.eps);
-        h = lh_f2h_exact(lh_norm_product(x, rms, norm_w ? lh_h2f(norm_w[lane]) : 1.0f));
+        h = lh_f2h_exact(lh_norm_product(x, rms, norm_weight));
     }
     if (is_q || is_k) {                                                    // NEOX RoPE on the f16-rounded head (rope.metal:14-61)
         hbuf[lane] = h;
@@ -183,7 +202,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     vec[lane] = h;
     const float xv = lh_h2f(h);
     if (is_q) {                                                            // hadamard_rotate_hf with pre-sign (attention_flash_tq.metal:58-90)
-        sh[lane] = __fmul_rn(xv, signs[lane]);
+        sh[lane] = __fmul_rn(xv, sign);
         fwht_lds(sh, d, lane);
         rq[((size_t)row * p.n_q_heads + head) * d + lane] = __fmul_rn(sh[lane], p.inv_sqrt_d);
         return;
@@ -191,7 +210,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     if (!p.write_kv) return;
     const uint32_t slot = p.ring_capacity ? position % p.ring_capacity : position;
     const uint32_t g = (row * p.lane_capacity + slot) * p.n_kv_heads + head;   // lane_capacity == 0: one sequence, slot alone
-    encode_vector(xv, lane, d, sh, code_sh, signs, levels, p.bits, p.code_bytes, p.inv_sqrt_d,
+    encode_vector(xv, lane, d, sh, code_sh, sign, lv, p.bits, p.code_bytes, p.inv_sqrt_d,
                   (is_k ? k_codes : v_codes) + (size_t)g * p.code_bytes, (is_k ? k_norms : v_norms) + g);
 }
 
@@ -212,11 +231,12 @@ __global__ __launch_bounds__(kMaxHeadDim) void dequantize_kv_kernel(const uint8_
         const uint32_t token = g / p.n_kv_heads, head = g - token * p.n_kv_heads;
         src_g = (token % p.ring_capacity) * p.n_kv_heads + head;
     }
+    const float sign = signs[lane], norm = lh_h2f(norms[src_g]);   // requested with the codes, not behind the transform's barriers
     sh[lane] = levels[unpack_code(packed + (size_t)src_g * p.code_bytes, lane, p.bits)];
     fwht_lds(sh, d, lane);
     float val = __fmul_rn(sh[lane], p.inv_sqrt_d);
-    val = __fmul_rn(val, signs[lane]);
-    val = __fmul_rn(val, lh_h2f(norms[src_g]));
+    val = __fmul_rn(val, sign);
+    val = __fmul_rn(val, norm);
     output[(size_t)g * d + lane] = lh_f2h_exact(val);
 }
 
@@ -228,10 +248,11 @@ __global__ __launch_bounds__(kMaxHeadDim) void hadamard_rotate_kernel(const TIn*
     __shared__ __align__(16) float sh[kMaxHeadDim];
     const uint32_t d = head_dim, lane = threadIdx.x, head = blockIdx.x;
     const float x = lh_load_as_f32<TIn>(input, (size_t)head * d + lane);
-    sh[lane] = pre_sign ? __fmul_rn(x, signs[lane]) : x;
+    const float sign = (pre_sign || post_sign) ? signs[lane] : 1.0f;
+    sh[lane] = pre_sign ? __fmul_rn(x, sign) : x;
     fwht_lds(sh, d, lane);
     float y = __fmul_rn(sh[lane], inv_sqrt_d);
-    if (post_sign) y = __fmul_rn(y, signs[lane]);
+    if (post_sign) y = __fmul_rn(y, sign);
     if constexpr (sizeof(TOut) == 2) output[(size_t)head * d + lane] = lh_f2h_exact(y);
     else output[(size_t)head * d + lane] = y;
 }
