@@ -38,7 +38,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X published dense f16/bf16 matrix peak
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by
 # the same counters on the library's plain copy kernel.  A run of bench.py cannot read hardware counters itself: the
 # figure is carried over from the profile named beside it (`roofline.traffic_source`), taken with the current kernel.
-MEASURED_TRAFFIC_BYTES = 1085515776   # 526047 KiB x 2.0 + 7980 KiB x 1.0
+MEASURED_TRAFFIC_BYTES = 1085517824   # 526048 KiB x 2.0 + 7980 KiB x 1.0
 TRAFFIC_SOURCE = "profiles/matvec_tq2_mfma_grouped_8192x2048.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; carried over, not measured by this run)"
 
 
