@@ -126,7 +126,7 @@ def test_encode_then_decode_roundtrips(pkg, gpu, oracle):
         cache.write_kv_gpu_into(batch, K, src, src, 1, T)               # quant_cache.rs:400-406
 
 
-@pytest.mark.parametrize("hd,heads", [(256, 8), (128, 3), (512, 2), (64, 5), (32, 1)])
+@pytest.mark.parametrize("hd,heads", [(256, 8), (128, 3), (512, 2), (64, 5), (32, 1), (16, 2), (8, 3)])
 def test_hadamard_rotate_variants_bit_exact(pkg, gpu, oracle, hd, heads):
     ctx, K = gpu
     g = pkg.synth.rng(5, hd + heads)
