@@ -62,18 +62,26 @@ __device__ __forceinline__ void encode_vector(float xv, uint32_t lane, uint32_t 
                                               const float sign, const LevelTable& lv, uint32_t bits,
                                               uint32_t code_bytes, float inv_sqrt_d, uint8_t* __restrict__ packed_slot,
                                               uint16_t* __restrict__ norm_slot) {
-    // norm = sqrt(fold(+, x_i * x_i)) in index order; every thread walks the same LDS
-    // words (broadcast reads), so all hold the same value without another barrier.
+    // norm = sqrt(fold(+, x_i * x_i)) in index order: the first wave walks the LDS words (broadcast reads, so each of its
+    // lanes holds the sum) and hands the sum over; the d dependent additions are issued once per vector, not once per wave
+    // (they are most of what a bulk encode issues).
     sh[lane] = __fmul_rn(xv, xv);
     __syncthreads();
     float sq = 0.0f;
-    if (d >= 4) {
-        for (uint32_t i = 0; i < d; i += 4) {
-            const float4 q = *reinterpret_cast<const float4*>(&sh[i]);
-            sq = __fadd_rn(sq, q.x); sq = __fadd_rn(sq, q.y); sq = __fadd_rn(sq, q.z); sq = __fadd_rn(sq, q.w);
+    if (lane < 64) {
+        if (d >= 4) {
+            for (uint32_t i = 0; i < d; i += 4) {
+                const float4 q = *reinterpret_cast<const float4*>(&sh[i]);
+                sq = __fadd_rn(sq, q.x); sq = __fadd_rn(sq, q.y); sq = __fadd_rn(sq, q.z); sq = __fadd_rn(sq, q.w);
+            }
+        } else {
+            for (uint32_t i = 0; i < d; i++) sq = __fadd_rn(sq, sh[i]);
         }
-    } else {
-        for (uint32_t i = 0; i < d; i++) sq = __fadd_rn(sq, sh[i]);
+    }
+    if (d > 64) {   // uniform over the workgroup
+        if (lane == 0) reinterpret_cast<float*>(code_sh)[0] = sq;
+        __syncthreads();
+        sq = reinterpret_cast<const float*>(code_sh)[0];
     }
     const float norm = __fsqrt_rn(sq);
     float v = xv;
