@@ -26,16 +26,29 @@ template <> __device__ __forceinline__ float x_at<float>(const float* x, uint32_
 
 // NL: 16-byte loads per lane and pass of the vector form (a pass covers 512 * NL columns).  FULL: cols is a multiple of
 // that, so no lane ever stands past the end of a row (no address clamps, no per-lane conditions in the loop).
-template <typename XT, typename YT, bool VEC, bool XLDS, int NL = 8, bool FULL = false>
+// XREG: the row is one pass long, so a lane multiplies the same 8 * NL activations in every row and keeps them in
+// registers (read from LDS at a stride of 32 bytes between lanes they cost a four-way bank conflict per 16-byte read, and
+// those reads, not the weight stream, then bound the kernel: 131072 x 2048 at 4.6 TB/s).
+template <typename XT, typename YT, bool VEC, bool XLDS, int NL = 8, bool FULL = false, bool XREG = false>
 __global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restrict__ W, const XT* __restrict__ x, YT* __restrict__ y, uint32_t rows,
                                                         uint32_t cols) {
     extern __shared__ float xs[];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    if (XLDS) {
+    if (XLDS && !XREG) {
         for (uint32_t i = threadIdx.x; i < cols; i += blockDim.x) xs[i] = x_at<XT>(x, i);
         __syncthreads();
     }
     auto xv = [&](uint32_t i) { return XLDS ? xs[i] : x_at<XT>(x, i); };
+    [[maybe_unused]] float xr[XREG ? NL : 1][8];
+    if constexpr (XREG) {
+#pragma unroll
+        for (int c = 0; c < NL; c++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t k = lane * 8 + 512 * c + j;
+                xr[c][j] = (FULL || k < cols) ? x_at<XT>(x, k) : 0.0f;
+            }
+    }
     if constexpr (VEC) {
         // cols a multiple of 8 and 16-byte aligned rows.  A wave walks its rows in passes of 512 * NL columns, NL loads of
         // 16 bytes per lane; the loads of the next pass (the next row, for rows of one pass) are issued before the arithmetic
@@ -61,8 +74,8 @@ __global__ __launch_bounds__(256) void matvec_f16_kernel(const uint16_t* __restr
                 const uint32_t wv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), xv(k + 2 * j), acc);
-                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] >> 16)), xv(k + 2 * j + 1), acc);
+                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] & 0xFFFF)), XREG ? xr[XREG ? c : 0][2 * j] : xv(k + 2 * j), acc);
+                    acc = __builtin_fmaf(lh_h2f((uint16_t)(wv[j] >> 16)), XREG ? xr[XREG ? c : 0][2 * j + 1] : xv(k + 2 * j + 1), acc);
                 }
             }
             if (ps + 1 == ppr) {
@@ -102,12 +115,19 @@ int launch(lh_context* ctx, const uint16_t* W, const void* x, void* y, uint32_t 
     const bool xlds = cols <= (uint32_t)kMaxLdsCols;
     const uint32_t waves = 4;
     const uint64_t want = ((uint64_t)rows + waves - 1) / waves;
-    const uint32_t grid = (uint32_t)std::min<uint64_t>(want, (uint64_t)ctx->cu_count * 8);   // (3 .. 12 workgroups per CU measure alike)
+    // Rows of one pass (up to 4096 columns) run with the activations in registers and stream best from two workgroups per CU
+    // (131072 x 2048: 6.83 TB/s against 6.67 from three to eight); the LDS form measures alike from 3 to 12.
+    const uint32_t per_cu = (vec && cols <= 4096) ? 2u : 8u;
+    const uint32_t grid = (uint32_t)std::min<uint64_t>(want, (uint64_t)ctx->cu_count * per_cu);
     const size_t lds = xlds ? (size_t)cols * 4 : 0;
 #define LH_F16MV(V, L, N, F) hipLaunchKernelGGL((matvec_f16_kernel<XT, YT, V, L, N, F>), dim3(grid), dim3(64 * waves), lds, ctx->stream, W, (const XT*)x, (YT*)y, rows, cols)
+#define LH_F16MV_R(N, F) hipLaunchKernelGGL((matvec_f16_kernel<XT, YT, true, true, N, F, true>), dim3(grid), dim3(64 * waves), 0, ctx->stream, W, (const XT*)x, (YT*)y, rows, cols)
 #define LH_F16MV_N(L, N)                                                       \
     do {                                                                       \
-        if (cols % (512u * N) == 0) LH_F16MV(true, L, N, true);                \
+        if (cols <= 512u * N) {   /* one pass per row: x in registers */ \
+            if (cols % (512u * N) == 0) LH_F16MV_R(N, true);                   \
+            else LH_F16MV_R(N, false);                                         \
+        } else if (cols % (512u * N) == 0) LH_F16MV(true, L, N, true);         \
         else LH_F16MV(true, L, N, false);                                      \
     } while (0)
 #define LH_F16MV_VEC(L)                                       \
@@ -122,6 +142,7 @@ int launch(lh_context* ctx, const uint16_t* W, const void* x, void* y, uint32_t 
     else if (xlds) LH_F16MV(false, true, 8, false);
     else LH_F16MV(false, false, 8, false);
 #undef LH_F16MV_N
+#undef LH_F16MV_R
 #undef LH_F16MV_VEC
 #undef LH_F16MV
     return LH_OK;

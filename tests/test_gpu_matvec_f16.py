@@ -23,7 +23,10 @@ def test_known_answer_vectors(pkg, gpu):
                               np.array(want, np.float32))
 
 
-@pytest.mark.parametrize("rows,cols", [(256, 1536), (1536, 256), (33, 100), (7, 16392), (4096, 2048), (5, 8)])
+# (the last four: rows long enough for the form that keeps a lane's activations in registers -- one pass per row, with
+# and without lanes past the row's end, one / four / eight loads per lane)
+@pytest.mark.parametrize("rows,cols", [(256, 1536), (1536, 256), (33, 100), (7, 16392), (4096, 2048), (5, 8),
+                                       (32773, 512), (33001, 1536), (32768, 2048), (32808, 2600)])
 def test_matvec_f16_family(pkg, gpu, rows, cols):
     ctx, K = gpu
     g = pkg.synth.rng(31, rows + cols)
