@@ -493,6 +493,15 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
         // the block groups of a tile on neighbouring waves: the segments of one row are then fetched close together in time
         if (ngroups > 1 && 12 % ngroups == 0) wide_split = ngroups;   // (one wave walking all groups of its tile: 0.65 against 0.71)
     }
+    // Few tiles, split over four waves each, f16 in and out, an even number of tiles (the decode path's down projection over
+    // 8192 columns): two tiles per workgroup of eight waves, so that twice the threads stage the activation vector and half
+    // as many workgroups stage it at all (a single-token decode layer: 64.4 -> 63.5 us).
+    bool pair_tiles = false;
+    if (splitk && split_waves == 4 && xt == LH_F16 && yt == LH_F16 && count == 1 && (((rows + 15) >> 4) & 1) == 0 && lds_for(8) <= kMaxLdsBytes) {
+        pair_tiles = true;
+        threads = 512;
+        wide_split = 4;
+    }
     const uint32_t waves = threads / 64;
     const uint32_t tiles_per_slot = wide_split ? waves / wide_split : (splitk ? 1u : waves);
     const uint64_t slots = (uint64_t)(((rows + 15) >> 4) + tiles_per_slot - 1) / tiles_per_slot * count;
@@ -505,7 +514,8 @@ int lh_launch_matvec_tq2_mfma(lh_context* ctx, uint32_t count, const void* const
     if ((slots / grid + 1) * ngroups > 0xFFFFFFFFull)   // the kernel counts a workgroup's (tile, block group) items in 32 bits
         return lh_fail(LH_ERR_INVALID_ARGUMENT, "matvec_tq2_0: %u problems of %u rows are more than one launch takes", count, rows);
     const void* fn;
-    if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
+    if (pair_tiles) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 512>;
+    else if (split_waves == 6) fn = (const void*)matvec_tq2_mfma_kernel<uint16_t, uint16_t, true, 384>;
 #define LH_FN(XT, YT) (wide_split ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true, 768, true>                                       \
                             : wide ? (const void*)matvec_tq2_mfma_kernel<XT, YT, false, 768>                                      \
                             : splitk ? (const void*)matvec_tq2_mfma_kernel<XT, YT, true>                                          \
