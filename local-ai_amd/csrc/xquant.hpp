@@ -34,11 +34,8 @@ __device__ __forceinline__ uint16_t lh_gelu_mul_h(uint16_t a, uint16_t b) {
 
 // Elements e0 .. e0 + 8 of f16(x * rms * aux (+ res)) as four packed words: the arithmetic of rms_norm_kernel<ADD>, its
 // tail forms (pro.tail) included.
-__device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& pro, uint32_t e0, float rms, uint32_t (&packed)[4]) {
-    const uint16_t* x = static_cast<const uint16_t*>(xv);
-    const uint4 a = *reinterpret_cast<const uint4*>(x + e0), g = *reinterpret_cast<const uint4*>(pro.aux + e0);
-    uint4 r = make_uint4(0u, 0u, 0u, 0u);
-    if (pro.res != nullptr) r = *reinterpret_cast<const uint4*>(pro.res + e0);
+// (`a`, `g`, `r`: the eight elements of the vector, the norm weight and -- with pro.res -- the residual, as loaded.)
+__device__ __forceinline__ void xpro_norm_add8_regs(const uint4 a, const uint4 g, const uint4 r, const XPrologue& pro, float rms, uint32_t (&packed)[4]) {
     const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wg[4] = {g.x, g.y, g.z, g.w}, wr[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -51,6 +48,13 @@ __device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& 
         }
         packed[j] = (uint32_t)lh_f2h_exact(lo) | ((uint32_t)lh_f2h_exact(hi) << 16);
     }
+}
+__device__ __forceinline__ void xpro_norm_add8(const void* xv, const XPrologue& pro, uint32_t e0, float rms, uint32_t (&packed)[4]) {
+    const uint16_t* x = static_cast<const uint16_t*>(xv);
+    const uint4 a = *reinterpret_cast<const uint4*>(x + e0), g = *reinterpret_cast<const uint4*>(pro.aux + e0);
+    uint4 r = make_uint4(0u, 0u, 0u, 0u);
+    if (pro.res != nullptr) r = *reinterpret_cast<const uint4*>(pro.res + e0);
+    xpro_norm_add8_regs(a, g, r, pro, rms, packed);
 }
 
 // The eight consecutive elements e0 .. e0 + 8 of a head that a lane holds, through the head's Walsh-Hadamard transform,
@@ -115,6 +119,9 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
     const int tid = threadIdx.x;
     const uint32_t kq = plane_dwords ? plane_dwords : K >> 2;   // dwords between the limb planes (K / 4 unless the caller pads them)
     float rms = 1.0f, rms2 = 1.0f;
+    [[maybe_unused]] bool one_round = false;          // the RMS-norm prologue has left the thread's normalised elements in one_packed
+    [[maybe_unused]] uint32_t one_packed[4] = {0u, 0u, 0u, 0u};
+    [[maybe_unused]] uint4 one_g2 = make_uint4(0u, 0u, 0u, 0u);
 
     if constexpr (sizeof(XT) == 2) {
         if (pro.kind == kXProRmsNorm) {   // uniform over the workgroup; xs doubles as the reduction scratch before it is filled
@@ -127,6 +134,50 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                 __syncthreads();
                 return t;
             };
+            if (K <= nthreads * 8) {
+                // One round covers the vector (uniform over the workgroup): everything a thread reads -- its eight elements,
+                // their norm weights, the residual, the second norm's weights -- is requested here at once and the passes
+                // below work from registers.  Read pass by pass, each pass waits for memory again behind the barriers of
+                // the pass before (three trips where this is one); the arithmetic and its order are those of the loops.
+                const uint32_t e0 = tid * 8;
+                const bool valid = e0 < K;
+                const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+                uint4 a = zero4, g = zero4, r = zero4;
+                one_g2 = zero4;
+                if (valid) {
+                    a = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(x) + e0);
+                    g = *reinterpret_cast<const uint4*>(pro.aux + e0);
+                    if (pro.res != nullptr) r = *reinterpret_cast<const uint4*>(pro.res + e0);
+                    if (pro.aux2 != nullptr) one_g2 = *reinterpret_cast<const uint4*>(pro.aux2 + e0);
+                }
+                float s = 0.0f;
+                if (valid) {
+                    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float lo = lh_h2f((uint16_t)(w[i] & 0xFFFF)), hi = lh_h2f((uint16_t)(w[i] >> 16));
+                        s += lo * lo;
+                        s += hi * hi;
+                    }
+                }
+                rms = rsqrtf(block_total(s) / (float)K + pro.eps);
+                if (valid) xpro_norm_add8_regs(a, g, r, pro, rms, one_packed);
+                if (pro.aux2 != nullptr || pro.store != nullptr) {
+                    float s2 = 0.0f;
+                    if (valid) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float lo = lh_h2f((uint16_t)(one_packed[i] & 0xFFFF)), hi = lh_h2f((uint16_t)(one_packed[i] >> 16));
+                            s2 += lo * lo;
+                            s2 += hi * hi;
+                        }
+                        if (pro.store != nullptr && blockIdx.x == 0)
+                            *reinterpret_cast<uint4*>(pro.store + e0) = make_uint4(one_packed[0], one_packed[1], one_packed[2], one_packed[3]);
+                    }
+                    if (pro.aux2 != nullptr) rms2 = rsqrtf(block_total(s2) / (float)K + pro.eps);
+                }
+                one_round = true;
+            } else {
             float s = 0.0f;
             for (uint32_t e0 = tid * 8; e0 < K; e0 += nthreads * 8) {
                 const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
@@ -155,6 +206,7 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                 }
                 if (pro.aux2 != nullptr) rms2 = rsqrtf(block_total(s2) / (float)K + pro.eps);
             }
+            }
         }
     }
     for (uint32_t base = 0; base < K; base += nthreads * 8) {
@@ -168,6 +220,14 @@ __device__ __forceinline__ void quantize_x_to_lds(const XT* __restrict__ x, uint
                 const float4 a = *reinterpret_cast<const float4*>(x + e0);
                 const float4 b = *reinterpret_cast<const float4*>(x + e0 + 4);
                 v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else if (one_round) {
+                const uint32_t wg2[4] = {one_g2.x, one_g2.y, one_g2.z, one_g2.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float t = lh_h2f((uint16_t)((one_packed[i >> 1] >> (16 * (i & 1))) & 0xFFFF));
+                    if (pro.aux2 != nullptr) v[i] = lh_h2f(lh_f2h_exact(lh_norm_product(t, rms2, lh_h2f((uint16_t)((wg2[i >> 1] >> (16 * (i & 1))) & 0xFFFF)))));
+                    else v[i] = t;
+                }
             } else {
                 const uint4 a = *reinterpret_cast<const uint4*>(x + e0);
                 const uint32_t w[4] = {a.x, a.y, a.z, a.w};
