@@ -227,12 +227,22 @@ __device__ __forceinline__ float lh_h2f(uint16_t h) { return (float)__builtin_bi
 __device__ __forceinline__ uint16_t lh_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 // One NEOX pair at `position` (rope.metal:46-58).  The same instruction sequence serves the stand-alone and the fused
 // kernel, so that qk_norm + rope and qk_norm_rope agree bit for bit (kernels.rs:7873).
-__device__ __forceinline__ void lh_rotate_pair(float x0, float x1, uint32_t i, uint32_t head_dim, uint32_t position, float theta, uint16_t& o0, uint16_t& o1) {
+// (In two halves, so that a kernel can evaluate the pair's cosine and sine -- which depend on no data -- while its loads are
+// on their way; both halves together are the sequence above.)
+__device__ __forceinline__ void lh_rope_cos_sin(uint32_t i, uint32_t head_dim, uint32_t position, float theta, float& c, float& sn) {
     const float freq = 1.0f / powf(theta, (float)(2 * i) / (float)head_dim);
     const float angle = (float)position * freq;
-    const float c = cosf(angle), sn = sinf(angle);
+    c = cosf(angle);
+    sn = sinf(angle);
+}
+__device__ __forceinline__ void lh_rope_apply(float x0, float x1, float c, float sn, uint16_t& o0, uint16_t& o1) {
     o0 = lh_f2h(__builtin_fmaf(x0, c, -(x1 * sn)));
     o1 = lh_f2h(__builtin_fmaf(x0, sn, x1 * c));
+}
+__device__ __forceinline__ void lh_rotate_pair(float x0, float x1, uint32_t i, uint32_t head_dim, uint32_t position, float theta, uint16_t& o0, uint16_t& o1) {
+    float c, sn;
+    lh_rope_cos_sin(i, head_dim, position, theta, c, sn);
+    lh_rope_apply(x0, x1, c, sn, o0, o1);
 }
 // Narrowing of an already rounded f32 value, as f16::from_f32 does it. The empty asm keeps the
 // compiler from folding a preceding multiply into v_fma_mixlo_f16, which rounds the exact

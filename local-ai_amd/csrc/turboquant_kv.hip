@@ -183,6 +183,10 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     const float sign = signs[lane];
     LevelTable lv;
     if (!is_q && p.write_kv) lv = load_levels(levels, p.bits);
+    // The RoPE pair's cosine and sine depend on the lane and the position only: evaluated here, under the loads above.
+    const uint32_t half_dim = d / 2, rope_angles = (uint32_t)((float)d * p.prf) / 2;
+    float rope_c = 1.0f, rope_s = 0.0f;
+    if ((is_q || is_k) && lane < rope_angles) lh_rope_cos_sin(lane, d, position, p.theta, rope_c, rope_s);
     uint16_t h = raw;
     if (normalise) {
         const float x = lh_h2f(raw);
@@ -197,10 +201,9 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
     if (is_q || is_k) {                                                    // NEOX RoPE on the f16-rounded head (rope.metal:14-61)
         hbuf[lane] = h;
         __syncthreads();
-        const uint32_t half_dim = d / 2, rope_angles = (uint32_t)((float)d * p.prf) / 2;
         if (lane < rope_angles) {
             uint16_t o0, o1;
-            lh_rotate_pair(lh_h2f(hbuf[lane]), lh_h2f(hbuf[lane + half_dim]), lane, d, position, p.theta, o0, o1);
+            lh_rope_apply(lh_h2f(hbuf[lane]), lh_h2f(hbuf[lane + half_dim]), rope_c, rope_s, o0, o1);
             hbuf[lane] = o0;
             hbuf[lane + half_dim] = o1;
         }
