@@ -65,6 +65,20 @@ def test_matvec_baseline_configs(pkg, gpu, oracle, fmt, rows, cols):
     assert e64 <= 3e-4   # 16-bit block-fixed-point activations
 
 
+@pytest.mark.parametrize("rows,cols", [(262144 - 37, 1536), (140001, 2048)])
+def test_matvec_q4_0_one_long_launch_ragged_rows(pkg, gpu, oracle, rows, cols):
+    """One Q4_0 problem long enough for the work order that deals the batches of steps over the whole grid, with a row
+    count that fills neither the last step nor the last batch (three unit columns per lane and one; eight and two rows
+    per step): every row against the reference CPU path."""
+    print(f"case q4_0 {rows}x{cols}", flush=True)
+    g = pkg.synth.rng(1, rows)
+    raw = pkg.synth.weights("q4_0", rows, cols, g)
+    x = pkg.synth.activations(1, cols, g)[0]
+    want = oracle.matvec_quant_ref("q4_0", raw, x, rows, cols, threads=8)
+    got = run_matvec(pkg, gpu, "q4_0", raw, x, rows, cols, pkg.F32, pkg.F32)
+    refgen.assert_close_both(got, want, 1e-3, f"q4_0 {rows}x{cols}")
+
+
 @pytest.mark.parametrize("rows,cols", [(4096, 16384), (4000, 14400)])
 def test_matvec_q4_0_longest_rows_many_rows(pkg, gpu, oracle, rows, cols):
     """Q4_0 rows so long that the activation area alone nearly fills the kernel's LDS limit, with enough rows per
