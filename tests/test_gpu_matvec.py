@@ -25,7 +25,7 @@ REF_SHAPES = [("q4_0", 5, 96), ("q4_0", 7, 64), ("tq2_0", 4, 512), ("tq2_0", 6, 
               ("q4_0", 33, 1536), ("tq2_0", 37, 1536), ("q4_0", 100, 6144), ("tq2_0", 100, 6144),
               ("q4_0", 16, 12288), ("tq2_0", 16, 12288), ("tq2_0", 3, 16384), ("q4_0", 3, 16384),
               ("tq2_0", 2, 32768), ("q4_0", 2, 20480), ("q4_0", 9, 32), ("tq2_0", 1, 256),
-              ("tq2_0", 70, 4096), ("tq2_0", 300, 8192), ("tq2_0", 17, 10240), ("tq2_0", 100, 12288), ("tq2_0", 37, 24576)]   # long rows, few tiles: block groups split over waves
+              ("tq2_0", 70, 4096), ("tq2_0", 300, 8192), ("tq2_0", 96, 8192), ("tq2_0", 32, 8192), ("tq2_0", 17, 10240), ("tq2_0", 100, 12288), ("tq2_0", 37, 24576)]   # long rows, few tiles: block groups split over waves
 
 
 @pytest.mark.parametrize("fmt,rows,cols", REF_SHAPES)
