@@ -107,6 +107,18 @@ __global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a
     const uint32_t dim = a.dim, rowi = blockIdx.x;
     const size_t row = (size_t)rowi * dim;
     uint4 x[4], o[4];
+    // The norm weights, the residual and the second norm's weights are requested here, with the row itself: read where they
+    // are used, each waits for memory again behind the barrier of the pass before.
+    uint4 gw[4], rr[4], gw2[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
+        gw[it] = rr[it] = gw2[it] = make_uint4(0u, 0u, 0u, 0u);
+        if (i >= dim) break;
+        gw[it] = *reinterpret_cast<const uint4*>(a.w + i);
+        if (ADD) rr[it] = *reinterpret_cast<const uint4*>(a.res + row + i);
+        if (a.w2 != nullptr) gw2[it] = *reinterpret_cast<const uint4*>(a.w2 + i);
+    }
     float s = 0.0f;
     if constexpr (PART) {
         // the splits of two chunks, eight at a time, are all requested before the first is added (in split order)
@@ -160,9 +172,9 @@ __global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a
     for (int it = 0; it < 4; it++) {
         const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
         if (i >= dim) break;
-        const uint4 g = *reinterpret_cast<const uint4*>(a.w + i);
+        const uint4 g = gw[it];
         uint4 r = x[it];
-        if (ADD) r = *reinterpret_cast<const uint4*>(a.res + row + i);
+        if (ADD) r = rr[it];
         uint4 w = rms_apply8<ADD>(x[it], g, r, rms, a.tail, 1.0f);
         if (a.apply_scale) {
             uint32_t ws[4] = {w.x, w.y, w.z, w.w};
@@ -181,8 +193,7 @@ __global__ __launch_bounds__(256) void rms_norm_fused_kernel(const LhNormFused a
     for (int it = 0; it < 4; it++) {
         const uint32_t i = (threadIdx.x + it * blockDim.x) * 8;
         if (i >= dim) break;
-        const uint4 g = *reinterpret_cast<const uint4*>(a.w2 + i);
-        *reinterpret_cast<uint4*>(a.out2 + row + i) = rms_apply8<false>(o[it], g, o[it], rms2, a.tail, 1.0f);
+        *reinterpret_cast<uint4*>(a.out2 + row + i) = rms_apply8<false>(o[it], gw2[it], o[it], rms2, a.tail, 1.0f);
     }
 }
 
