@@ -376,7 +376,7 @@ def test_matvec_non_finite_activations_propagate(pkg, gpu, oracle, fmt, rows, co
         assert not np.isfinite(got).any(), f"{fmt}: {int(np.isfinite(got).sum())} of {rows} rows stayed finite with x = {bad}"
 
 
-@pytest.mark.parametrize("fmt,rows,cols,count", [("tq2_0", 512, 2048, 5), ("q4_0", 300, 2048, 4), ("tq2_0", 96, 8192, 3),
+@pytest.mark.parametrize("fmt,rows,cols,count", [("tq2_0", 512, 2048, 5), ("q4_0", 300, 2048, 4), ("q4_0", 1001, 2048, 7), ("q4_0", 4099, 1536, 9), ("q4_0", 20011, 512, 5), ("tq2_0", 96, 8192, 3),
                                                  ("q4_0", 2048, 2048, 9)])
 def test_grouped_evenly_spaced_problems(pkg, gpu, oracle, fmt, rows, cols, count):
     """A grouped launch whose matrices and outputs are evenly spaced views of one allocation, with one shared vector or
