@@ -438,7 +438,7 @@ int attention_dispatch(lh_batch* batch, const char* op, const lh_buffer* rq, con
     const size_t ws_avail = ws_override ? ws_override_floats : (ctx->workspace_bytes / 2) / 4;   // floats; the lower half of the workspace
     const AttnPointers ptrs{(const float*)rq->ptr, (const uint8_t*)k_codes->ptr, (const uint16_t*)k_norms->ptr,
                             (const uint8_t*)v_codes->ptr, (const uint16_t*)v_norms->ptr, (const float*)levels->ptr,
-                            positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, ws};
+                            positions ? (const uint32_t*)positions->ptr : nullptr, (float*)out->ptr, ws, ctx->fault_dev};
     // Prefill entries with more than one row.  Sixteen rows sharing a pass over the codes (the tiled kernel) pay when there
     // is enough work to keep its eight-wave workgroups busy: measured against one query row per workgroup it wins from about
     // 1.5 M (row, position) pairs on (256 rows over 8k positions: 50 against 60 us; over 32k: 118 against 192) and loses

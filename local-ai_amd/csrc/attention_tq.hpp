@@ -44,6 +44,7 @@ struct AttnPointers {
     const uint32_t* positions;
     float* out;
     float* ws;
+    uint32_t* fault = nullptr;   // where a kernel reports a bounded wait that ran out (the context's fault word)
 };
 
 // True when the matrix-core kernel can take this call (2-bit codes, head_dim 256 or 512, at most 8 query heads per

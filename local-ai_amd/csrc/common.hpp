@@ -39,7 +39,7 @@ struct lh_context {
     uint32_t* fault_dev;   // the same word as the device addresses it
 };
 // Kernel-reported fault codes (lh_context::fault_host).
-enum : uint32_t { LH_FAULT_TQ2_SPLIT_WAIT = 1 };
+enum : uint32_t { LH_FAULT_TQ2_SPLIT_WAIT = 1, LH_FAULT_ATTN_PAIR_WAIT = 2 };
 // Reads and clears the context's fault word after a completed wait; LH_OK when no kernel reported anything.
 int lh_check_fault_word(lh_context* ctx);
 
