@@ -102,6 +102,9 @@ int lh_check_fault_word(lh_context* ctx) {
     if (code == LH_FAULT_TQ2_SPLIT_WAIT)
         return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: matvec_tq2_0: a wave gave up waiting for the partial rows of its tile; "
                                               "the outputs of this batch are not valid");
+    if (code == LH_FAULT_ATTN_PAIR_WAIT)
+        return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: flash_attention_tq: a wave gave up waiting for its partner at a hand-over; "
+                                              "the outputs of this batch are not valid");
     return lh_fail(LH_ERR_COMMAND_BUFFER, "GPU error: a kernel reported fault code %u", code);
 }
 
