@@ -111,6 +111,9 @@ LH_API int lh_batch_commit_and_wait(lh_batch* batch);
 /* Test hook, no counterpart in the reference: the number of polls the wait above is good for (default 2^20).  A
  * test sets it to 0 to see the error path taken without any kernel hanging, and restores it afterwards. */
 LH_API void lh_debug_set_tq2_split_spin_limit(uint32_t polls);
+/* The same for the attention kernels that work on several chunks of positions per workgroup: a chunk's two waves
+ * meet at their hand-overs through counters in LDS, with a bounded poll (default 2^22) that reports in the same way. */
+LH_API void lh_debug_set_attention_pair_spin_limit(uint32_t polls);
 LH_API int lh_batch_submit_and_renew(lh_batch* batch);
 LH_API int lh_batch_commit_and_renew(lh_batch* batch);
 

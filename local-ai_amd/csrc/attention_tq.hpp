@@ -15,6 +15,7 @@ struct AttnParams {
     uint32_t pos0;            // single: current_pos; prefill: start_pos
     uint32_t window, ring_capacity, lane_capacity;
     uint32_t mode, num_queries, num_splits;
+    uint32_t pair_spin_limit = 1u << 22;   // polls a wave of the several-chunk kernels spends at one hand-over before it gives up
 };
 
 constexpr int kMaxSplits = 1024;

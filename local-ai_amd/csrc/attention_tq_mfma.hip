@@ -30,6 +30,7 @@
 // further hand-over ahead and passes its integer logit sums to the first.  Partials (R, l, acc) per chunk
 // go to the workspace for the merge kernel.
 #include "attention_tq.hpp"
+#include <atomic>
 #include <algorithm>
 #include <cstdlib>
 #include <type_traits>
@@ -87,6 +88,7 @@ struct AttnShared {
     float fin_l[kMaxGroupHeads], fin_w[kMaxGroupHeads], fin_r[kMaxGroupHeads];
     float maxabs[kMaxGroupHeads], sum[kMaxGroupHeads];
     uint32_t psync[2];             // several chunks per workgroup: hand-overs the K wave / the V wave of this chunk has reached
+    uint32_t pair_spin_limit;      // polls a wave spends at one hand-over before it gives up (copied from the launch parameters)
 };
 
 // NPL = number of bit planes: 2 when the level table is affine in the code bits, 3 with the bit0*bit1 plane.
@@ -191,10 +193,13 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         const uint32_t me = k_role ? 0u : 1u;
         __builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory");
         if (lane == 0) __hip_atomic_store(&sh.psync[me], pair_step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        uint32_t spins = 0;
-        bool seen;
-        while (!(seen = __hip_atomic_load(&sh.psync[me ^ 1u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= pair_step) && spins++ < (1u << 22))
-            __builtin_amdgcn_s_sleep(1);
+        bool seen = __hip_atomic_load(&sh.psync[me ^ 1u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= pair_step;
+        if (!seen) {   // the budget lives in LDS and is read only by a wave that has to wait: no register holds it in between
+            const uint32_t limit = sh.pair_spin_limit;
+            uint32_t spins = 0;
+            while (!(seen = __hip_atomic_load(&sh.psync[me ^ 1u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= pair_step) && spins++ < limit)
+                __builtin_amdgcn_s_sleep(1);
+        }
         if (!seen && lane == 0 && a.fault) __hip_atomic_store(a.fault, (uint32_t)LH_FAULT_ATTN_PAIR_WAIT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         __builtin_amdgcn_s_waitcnt(0xC07F); asm volatile("" ::: "memory");
     };
@@ -250,7 +255,10 @@ __device__ __forceinline__ void attention_body(const AttnPointers& a, const Attn
         s = lh_group_sum(s, 32);
         if (sub == 0) { s_maxabs[h] = m; s_sum[h] = s; }
     }
-    if constexpr (kPairSync && NQ > 1) { if (tid < 2u * NQ) shs[tid >> 1].psync[tid & 1u] = 0u; }
+    if constexpr (kPairSync && NQ > 1) {
+        if (tid < 2u * NQ) shs[tid >> 1].psync[tid & 1u] = 0u;
+        else if (tid < 3u * NQ) shs[tid - 2u * NQ].pair_spin_limit = p.pair_spin_limit;
+    }
     __syncthreads();
 
     // ---- K-side A operands.  Row r of the MFMA: head (r / 4) + 4 * ((r / 2) % 2), limb r % 2, so that the lanes of
@@ -926,7 +934,12 @@ bool mfma_supported(const AttnParams& p, const AttnPointers& a) {
     return true;
 }
 
+// Test aid: the poll budget of a hand-over between a chunk's two waves.  With 0 a wave that arrives early gives up at once,
+// which the wait on the batch reports; nothing in the library changes it.
+static std::atomic<uint32_t> g_pair_spin_limit{1u << 22};
+
 int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnParams& p, uint64_t max_span, size_t ws_floats) {
+    p.pair_spin_limit = g_pair_spin_limit.load(std::memory_order_relaxed);
     // One workgroup (a K wave and one V wave per 256 dims) per chunk of positions.  Short jobs (the chunks of one workgroup per CU
     // stay within 128 positions) are latency bound: they get chunks down to one group of 64 and never share a CU.
     // Everything else gets about two waves per SIMD over the whole launch (the registers allow no third) and at least 128
@@ -1009,3 +1022,5 @@ int launch_mfma(lh_context* ctx, const char* op, const AttnPointers& a, AttnPara
 }
 
 }  // namespace lh_attn
+
+extern "C" void lh_debug_set_attention_pair_spin_limit(uint32_t polls) { lh_attn::g_pair_spin_limit.store(polls, std::memory_order_relaxed); }

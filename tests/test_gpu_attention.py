@@ -484,6 +484,55 @@ def test_batched_long_lanes_merged_in_the_workgroup(pkg, gpu, oracle, lanes, cap
         check(got[l], ref, f"lane {l} at {positions[l]}")
 
 
+def test_batched_hand_over_that_gives_up_is_reported(pkg, gpu, oracle):
+    """The K wave and the V wave of a chunk meet at their hand-overs through counters in LDS, with a bounded poll.  With the
+    poll budget forced to zero from the host a wave that arrives early goes on at once: every wave still runs to the end of
+    the kernel, and the wait on the batch must report it as a command-buffer error instead of returning outputs that may be
+    wrong.  With the budget restored the same launch is clean and equals the launch made before the budget was touched,
+    bit for bit, and the oracle."""
+    import ctypes as C
+    ctx, K = gpu
+    hd, nq, nkv, bits, lanes, cap = 256, 8, 1, 2, 256, 4096     # four chunks of 1024 positions per lane, one workgroup per lane
+    signs, levels, kc, kn, vc, vn = build_cache(pkg, oracle, cap, nkv, hd, bits, 5151)
+    g = pkg.synth.rng(6, 51)
+    positions = g.integers(cap // 2, cap, lanes).astype(np.uint32)
+    pool_kc, pool_vc = np.tile(kc, (lanes, 1, 1)), np.tile(vc, (lanes, 1, 1))
+    pool_kn, pool_vn = np.tile(kn, (lanes, 1)), np.tile(vn, (lanes, 1))
+    rq = g.standard_normal((lanes, nq * hd), dtype=np.float32)
+    bufs = upload(pkg, ctx, pool_kc, pool_kn, pool_vc, pool_vn, levels, rq, positions)
+    out = pkg.Buffer.empty(ctx, rq.nbytes)
+    batch = pkg.CommandBatch(ctx)
+
+    def launch():
+        K.flash_attention_tq_batched_into(batch, bufs[5], bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], out, bufs[6], hd, cap, nq,
+                                          nkv, 0, bits, lanes, 0)
+        batch.commit_and_wait()
+        return out.as_array(np.float32).reshape(lanes, nq * hd).copy()
+
+    before = launch()
+    setter = pkg.lib().lh_debug_set_attention_pair_spin_limit
+    setter.restype = None
+    seen = False
+    try:
+        setter(C.c_uint32(0))
+        for _ in range(5):
+            try:
+                launch()
+            except pkg.CommandBuffer as e:
+                assert "gave up waiting for its partner" in str(e)
+                seen = True
+                break
+    finally:
+        setter(C.c_uint32(1 << 22))
+    assert seen, "no wave of 5 launches ever had to wait: the forced give-up path was not reached"
+    after = launch()                 # clean again: the fault word was cleared when it was reported
+    assert np.array_equal(before, after)
+    for l in (0, lanes // 2, lanes - 1):
+        ref = oracle.attention_tq_codespace(rq[l], pool_kc, pool_kn, pool_vc, pool_vn, levels, hd, int(positions[l]) + 1,
+                                            int(positions[l]), nq, nkv, 0, bits, 0, lane_base=l * cap)
+        check(after[l], ref, f"lane {l} after the budget was restored")
+
+
 def test_split_invariance_at_32k(pkg, gpu, oracle):
     """Full-size configuration (32768 cached positions, 8 q heads / 1 kv head, hd 256, 2 bits):
     parity with the f64 oracle, and the SWA-ring configuration (window 512, ring 512, wrapped)."""
