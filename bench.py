@@ -698,9 +698,10 @@ def _decode_single(pkg, ctx, K, steps, warmup, T, n_layers, make_layer, scratch,
 
     def encode_lane_step(b):
         b.blit_copy(x0, 0, bs.hidden_a, 0, 4096)
-        for i, layer in enumerate(layers):
+        for i, layer in enumerate(layers):   # as the pipeline chains them: a layer's last dispatch applies the next layer's input norm
+            nxt = layers[i + 1].weights.attn_norm if i + 1 < n_layers else None
             layer.forward_decode_batch_turbo(b, K, 1, positions, gbufs[i & 1], gbufs[(i + 1) & 1], bs, scratch.ones, pools[i],
-                                             (ple, n_layers))
+                                             (ple, n_layers), i > 0, nxt)
 
     batch.begin_capture()
     encode_lane_step(batch)
@@ -732,9 +733,10 @@ def _decode_lanes(pkg, ctx, K, steps, warmup, T, lanes, lane_layers, make_layer,
     def step_lanes():
         batch.blit_copy(xin, 0, bs.hidden_a, 0, lanes * 4096)
         bufs = (bs.hidden_a, bs.hidden_b)
-        for i, layer in enumerate(layers):
+        for i, layer in enumerate(layers):   # as the pipeline chains them: a layer's last dispatch applies the next layer's input norm
+            nxt = layers[i + 1].weights.attn_norm if i + 1 < lane_layers else None
             layer.forward_decode_batch_turbo(batch, K, lanes, positions, bufs[i & 1], bufs[(i + 1) & 1], bs, scratch.ones,
-                                             pools[i], (ple_all, lane_layers))
+                                             pools[i], (ple_all, lane_layers), i > 0, nxt)
 
     wall, ev = time_steps(pkg, ctx, step_lanes, steps, warmup)
     out = (bs.hidden_a, bs.hidden_b)[lane_layers & 1].as_array(np.float16, lanes * 2048).astype(np.float32)
