@@ -472,6 +472,22 @@ LH_API int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buf
                                            uint32_t n_q_heads, uint32_t n_kv_heads, uint32_t rows, float eps,
                                            uint32_t start_position, float theta, float partial_rotary_factor, uint32_t bits,
                                            uint32_t ring_capacity, uint32_t lane_capacity);
+/* The Q, K and V projections of `rows` tokens followed by lh_decode_qkv_prepare_rows_into on their outputs, i.e.
+ * lh_matmul_nt_quant_grouped_into(fmt, 3, input, {w_q, w_k, w_v}, {q, k, v}, rows, k_dim) and then the preparation
+ * (layer.rs:570-616 / 749-800), with the same results bit for bit: q / k / v, rq, codes and norms.  Where the product
+ * runs on the decode-batch kernel with its k range split (a few to some hundreds of rows), the preparation sums the
+ * product's partial tiles itself and the product's own reduction pass falls away; every other shape runs as the two
+ * calls.  input [rows, k_dim] f16; w_q [n_q_heads * head_dim, k_dim], w_k / w_v [n_kv_heads * head_dim, k_dim] in `fmt`.
+ * All three projections are required (a layer that shares another layer's cache takes the separate entry points). */
+LH_API int lh_matmul_nt_qkv_prepare_rows_into(lh_batch* batch, lh_quant fmt, const lh_buffer* input, const lh_buffer* w_q,
+                                              const lh_buffer* w_k, const lh_buffer* w_v, uint32_t k_dim, lh_buffer* q,
+                                              lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm, const lh_buffer* k_norm,
+                                              const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq,
+                                              lh_buffer* k_codes, lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms,
+                                              const lh_buffer* positions, uint32_t head_dim, uint32_t n_q_heads,
+                                              uint32_t n_kv_heads, uint32_t rows, float eps, uint32_t start_position,
+                                              float theta, float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity,
+                                              uint32_t lane_capacity);
 /* kernels.rs:5032-5163 hadamard_rotate{,_hf,_fh}_into,
  * shaders/attention_flash_tq.metal:58-139: per head optional sign flip, FWHT,
  * 1/sqrt(d), optional sign flip.  f32->f32, f16->f32, f32->f16. */

@@ -632,6 +632,22 @@ class Kernels:
                                                        C.c_float(partial_rotary_factor), _u32(bits), _u32(ring_capacity),
                                                        _u32(lane_capacity)))
 
+    def matmul_nt_qkv_prepare_rows_into(self, batch, weight_type, input, w_q, w_k, w_v, k_dim, q, k, v, q_norm, k_norm, levels,
+                                        signs, rq, k_codes, k_norms, v_codes, v_norms, positions, head_dim, n_q_heads,
+                                        n_kv_heads, rows, eps, start_position, theta, partial_rotary_factor, bits,
+                                        ring_capacity, lane_capacity):
+        """The grouped Q / K / V product and decode_qkv_prepare_rows_into on its outputs; the preparation sums the
+        product's k-split tiles itself where the product leaves them (same results bit for bit)."""
+        def h(b):
+            return b._h if b is not None else None
+        _check(self._l.lh_matmul_nt_qkv_prepare_rows_into(batch._h, C.c_int(weight_type), input._h, w_q._h, w_k._h, w_v._h,
+                                                          _u32(k_dim), q._h, k._h, v._h, h(q_norm), h(k_norm), levels._h,
+                                                          signs._h, rq._h, k_codes._h, k_norms._h, v_codes._h, v_norms._h,
+                                                          h(positions), _u32(head_dim), _u32(n_q_heads), _u32(n_kv_heads),
+                                                          _u32(rows), C.c_float(eps), _u32(start_position), C.c_float(theta),
+                                                          C.c_float(partial_rotary_factor), _u32(bits), _u32(ring_capacity),
+                                                          _u32(lane_capacity)))
+
     def hadamard_rotate_into(self, batch, input, signs, output, head_dim, num_heads, pre_sign, post_sign):
         _check(self._l.lh_hadamard_rotate_into(batch._h, input._h, signs._h, output._h, _u32(head_dim),
                                                _u32(num_heads), C.c_int(bool(pre_sign)), C.c_int(bool(post_sign))))

@@ -144,6 +144,23 @@ void lh_launch_gelu_mul_strided(hipStream_t stream, const void* a, const float* 
                                 uint32_t b_row_stride, uint32_t b_off, void* out, uint32_t dim, uint32_t rows);
 void lh_launch_gelu_mul(hipStream_t stream, const void* a, const void* b, void* out, uint32_t count);   // gelu_mul_into's kernel
 void lh_launch_norm_fused(hipStream_t stream, const LhNormFused& a);
+
+// The arguments of lh_decode_qkv_prepare_rows_into, and its launch with the heads taken from the f32 partial tiles of a
+// k-split product ([splits][rows][part_cols], the query, key and value heads side by side; nullptr: from q / k / v).
+// Defined with the kernel (turboquant_kv.hip); the product that leaves its tiles behind calls it (matmul_quant.hip).
+// check_only validates the arguments and launches nothing.
+struct LhPrepareRows {
+    lh_buffer *q, *k, *v;
+    const lh_buffer *q_norm, *k_norm, *levels, *signs;
+    lh_buffer *rq, *k_codes, *k_norms, *v_codes, *v_norms;
+    const lh_buffer* positions;
+    uint32_t head_dim, n_q_heads, n_kv_heads, rows;
+    float eps;
+    uint32_t start_position;
+    float theta, partial_rotary_factor;
+    uint32_t bits, ring_capacity, lane_capacity;
+};
+int lh_prepare_rows_launch(lh_batch* batch, const LhPrepareRows& a, const float* partial, uint32_t splits, uint32_t part_cols, bool check_only = false);
 int lh_launch_hadamard_fh(lh_context* ctx, const float* input, const float* signs, uint16_t* output, uint32_t head_dim, uint32_t num_heads);
 
 // Stream-ordered copy of a host-built descriptor table to device memory.  The host block may be freed as soon as this

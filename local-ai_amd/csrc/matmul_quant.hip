@@ -1453,6 +1453,66 @@ int lh_matmul_nt_quant_grouped_into(lh_batch* b, lh_quant fmt, uint32_t count, c
     return r;
 }
 
+int lh_matmul_nt_qkv_prepare_rows_into(lh_batch* b, lh_quant fmt, const lh_buffer* in, const lh_buffer* w_q, const lh_buffer* w_k,
+                                       const lh_buffer* w_v, uint32_t k_dim, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm,
+                                       const lh_buffer* k_norm, const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes,
+                                       lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms, const lh_buffer* positions, uint32_t head_dim,
+                                       uint32_t n_q_heads, uint32_t n_kv_heads, uint32_t rows, float eps, uint32_t start_position, float theta,
+                                       float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity, uint32_t lane_capacity) {
+    const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 (Q, K, V) + decode_qkv_prepare" : "matmul_nt_tq2_0 (Q, K, V) + decode_qkv_prepare";
+    if (!b) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
+    if (fmt != LH_Q4_0 && fmt != LH_TQ2_0) return lh_fail(LH_ERR_INVALID_ARGUMENT, "matmul_nt_quant: unknown weight format %d", (int)fmt);
+    if (!in || !w_q || !w_k || !w_v || !q || !k || !v || n_q_heads == 0 || n_kv_heads == 0)
+        return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: needs the query, key and value projections and their outputs (a layer that shares its cache "
+                                                "takes the separate entry points)", op);
+    const LhPrepareRows a{q, k, v, q_norm, k_norm, levels, signs, rq, k_codes, k_norms, v_codes, v_norms, positions, head_dim, n_q_heads, n_kv_heads,
+                          rows, eps, start_position, theta, partial_rotary_factor, bits, ring_capacity, lane_capacity};
+    int r = lh_prepare_rows_launch(b, a, nullptr, 0, 0, true);   // the second half's arguments, before anything is launched
+    if (r != LH_OK) return r;
+    if (rows == 0 || k_dim == 0) return LH_OK;
+    const lh_buffer* const ws[3] = {w_q, w_k, w_v};
+    lh_buffer* const outs[3] = {q, k, v};
+    const uint32_t ns[3] = {n_q_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * head_dim};
+    lh_context* ctx = b->ctx;
+    const int kind = fmt == LH_Q4_0 ? kQ4 : kTQ2;
+    const uint32_t blk = fmt == LH_Q4_0 ? 32 : 256, m = rows;
+    // The shapes that lh_matmul_nt_quant_grouped_into sends to the decode-batch kernel as one launch can leave their partial
+    // tiles to the preparation; every other shape runs as that entry point followed by the preparation.
+    uint64_t tiles_n = 0;
+    bool whole = true;
+    for (uint32_t i = 0; i < 3; i++) { tiles_n += (ns[i] + BN - 1) / BN; whole = whole && ns[i] % BN == 0; }
+    const uint64_t tiles128 = tiles_n * ((m + 127) / 128);
+    const bool small = m <= (uint32_t)kMaxMultivecM;
+    const bool together = (!small || m >= skinny_min_m(kind)) && !(m > 64 && tiles128 * 2 >= (uint64_t)ctx->cu_count);
+    bool fused = false;
+    SkinnyPartials kept{nullptr, 0, 0};
+    if (together && whole && k_dim % blk == 0 && ((uintptr_t)in->ptr & 15) == 0 && in->len >= (size_t)m * k_dim * 2) {
+        GroupArgs grp{};
+        grp.count = 3;
+        uint32_t tile = 0;
+        bool fits = true;
+        for (uint32_t i = 0; i < 3; i++) {
+            const size_t wbytes = fmt == LH_Q4_0 ? (size_t)ns[i] * (k_dim / 32) * 18 : (size_t)ns[i] * (k_dim / 256) * 66;
+            fits = fits && ws[i]->len >= wbytes && ((uintptr_t)ws[i]->ptr & 1) == 0;
+            grp.W[i] = (const uint8_t*)ws[i]->ptr; grp.C[i] = outs[i]->ptr; grp.N[i] = ns[i];
+            grp.tile0[i] = tile;
+            tile += ns[i] / BN;
+        }
+        for (uint32_t i = 3; i <= 4; i++) grp.tile0[i] = tile;
+        const ClipArgs none{nullptr, 0.f, 0.f, 0.f, 0.f, 0u};
+        if (fits)
+            fused = fmt == LH_Q4_0 ? try_skinny<kQ4, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k_dim, grp.N[0], none, grp, &kept)
+                                   : try_skinny<kTQ2, LH_F16>(ctx, in->ptr, grp.W[0], grp.C[0], LH_F16, m, k_dim, grp.N[0], none, grp, &kept);
+    }
+    if (fused) {
+        r = lh_check_launch(op);
+        if (r != LH_OK) return r;
+        return lh_prepare_rows_launch(b, a, kept.partial, kept.splits, kept.cols);
+    }
+    r = lh_matmul_nt_quant_grouped_into(b, fmt, 3, in, ws, outs, ns, rows, k_dim);   // reports what is wrong with the product's arguments
+    return r != LH_OK ? r : lh_prepare_rows_launch(b, a, nullptr, 0, 0);
+}
+
 int lh_matmul_nt_quant_gelu_mul_into(lh_batch* b, lh_quant fmt, const lh_buffer* in, const lh_buffer* w_gate, const lh_buffer* w_up,
                                      lh_buffer* out, uint32_t m, uint32_t k, uint32_t n) {
     const char* op = fmt == LH_Q4_0 ? "matmul_nt_q4_0 + gelu_mul" : "matmul_nt_tq2_0 + gelu_mul";

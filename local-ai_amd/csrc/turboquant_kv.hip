@@ -153,6 +153,10 @@ __global__ __launch_bounds__(kMaxHeadDim) void encode_kv_kernel(const uint16_t* 
 struct PrepareParams {
     uint32_t head_dim, n_q_heads, n_kv_heads, bits, code_bytes, position, ring_capacity, write_kv, lane_capacity;
     float eps, theta, prf, inv_sqrt_d;
+    // The heads as the f32 partial tiles of a k-split product [splits][rows][part_cols] (columns: the query heads, the key
+    // heads, the value heads, side by side) instead of f16 rows in q / k / v; nullptr: the rows are read from q / k / v.
+    const float* partial;
+    uint32_t splits, part_cols, rows;
 };
 
 __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_t* __restrict__ q, uint16_t* __restrict__ k,
@@ -178,7 +182,24 @@ __global__ __launch_bounds__(kMaxHeadDim) void decode_qkv_prepare_kernel(uint16_
 
     // Everything the workgroup reads from memory is requested here, in one trip: behind the barriers below each load
     // would be a round trip of its own (the norm weight, the sign, the levels: three of them on the K and V path).
-    const uint16_t raw = vec[lane];
+    uint16_t raw;
+    if (p.partial) {
+        // The sum the product's own reduction pass would have stored: the splits in order, in f32, rounded to f16.  Eight
+        // splits are requested before the first is added.
+        const size_t zstride = (size_t)p.rows * p.part_cols;
+        const float* part = p.partial + (size_t)row * p.part_cols + (size_t)b * d + lane;
+        float acc = 0.0f;
+        for (uint32_t z0 = 0; z0 < p.splits; z0 += 8) {
+            float t[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; u++) t[u] = part[(size_t)(z0 + u < p.splits ? z0 + u : p.splits - 1) * zstride];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; u++) if (z0 + u < p.splits) acc += t[u];
+        }
+        raw = lh_f2h(acc);
+    } else {
+        raw = vec[lane];
+    }
     const float norm_weight = norm_w ? lh_h2f(norm_w[lane]) : 1.0f;
     const float sign = signs[lane];
     LevelTable lv;
@@ -463,6 +484,21 @@ int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buffer* k,
                                     lh_buffer* k_norms, lh_buffer* v_codes, lh_buffer* v_norms, const lh_buffer* positions, uint32_t head_dim,
                                     uint32_t n_q_heads, uint32_t n_kv_heads, uint32_t rows, float eps, uint32_t start_position, float theta,
                                     float partial_rotary_factor, uint32_t bits, uint32_t ring_capacity, uint32_t lane_capacity) {
+    const LhPrepareRows a{q, k, v, q_norm, k_norm, levels, signs, rq, k_codes, k_norms, v_codes, v_norms, positions, head_dim, n_q_heads, n_kv_heads,
+                          rows, eps, start_position, theta, partial_rotary_factor, bits, ring_capacity, lane_capacity};
+    return lh_prepare_rows_launch(batch, a, nullptr, 0, 0);
+}
+
+}  // extern "C"
+
+int lh_prepare_rows_launch(lh_batch* batch, const LhPrepareRows& a, const float* partial, uint32_t splits, uint32_t part_cols, bool check_only) {
+    lh_buffer* const q = a.q; lh_buffer* const k = a.k; lh_buffer* const v = a.v;
+    const lh_buffer* const q_norm = a.q_norm; const lh_buffer* const k_norm = a.k_norm; const lh_buffer* const levels = a.levels;
+    const lh_buffer* const signs = a.signs; lh_buffer* const rq = a.rq; lh_buffer* const k_codes = a.k_codes; lh_buffer* const k_norms = a.k_norms;
+    lh_buffer* const v_codes = a.v_codes; lh_buffer* const v_norms = a.v_norms; const lh_buffer* const positions = a.positions;
+    const uint32_t head_dim = a.head_dim, n_q_heads = a.n_q_heads, n_kv_heads = a.n_kv_heads, rows = a.rows, start_position = a.start_position,
+                   bits = a.bits, ring_capacity = a.ring_capacity, lane_capacity = a.lane_capacity;
+    const float eps = a.eps, theta = a.theta, partial_rotary_factor = a.partial_rotary_factor;
     const char* op = "decode_qkv_prepare";
     if (!batch) return lh_fail(LH_ERR_INVALID_ARGUMENT, "%s: batch is null", op);
     int r = check_tq_shape(op, head_dim, bits);
@@ -493,9 +529,12 @@ int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buffer* k,
         LH_NEED(v_norms, (size_t)phys * n_kv_heads * 2, op, "v_norms");
     }
     PrepareParams p{head_dim, n_q_heads, write_kv ? n_kv_heads : 0u, bits, cb, start_position, ring_capacity, write_kv ? 1u : 0u, lane_capacity,
-                    eps, theta, partial_rotary_factor, host_inv_sqrt(head_dim)};
+                    eps, theta, partial_rotary_factor, host_inv_sqrt(head_dim), partial, splits, part_cols, rows};
     const uint64_t groups = (uint64_t)rows * (n_q_heads + (write_kv ? 2 * n_kv_heads : 0));
     LH_REQUIRE(groups <= 0x7FFFFFFFull, "%s: %u rows are too many for one launch", op, rows);
+    if (partial) LH_REQUIRE(splits >= 1 && (uint64_t)(n_q_heads + (write_kv ? 2 * n_kv_heads : 0)) * head_dim <= part_cols,
+                            "%s: partial tiles of %u columns do not hold the heads", op, part_cols);
+    if (check_only) return LH_OK;
     hipLaunchKernelGGL(decode_qkv_prepare_kernel, dim3((uint32_t)groups), dim3(head_dim), 0, batch->ctx->stream, (uint16_t*)q->ptr,
                        write_kv ? (uint16_t*)k->ptr : nullptr, write_kv ? (uint16_t*)v->ptr : nullptr,
                        q_norm ? (const uint16_t*)q_norm->ptr : nullptr, (write_kv && k_norm) ? (const uint16_t*)k_norm->ptr : nullptr,
@@ -507,6 +546,8 @@ int lh_decode_qkv_prepare_rows_into(lh_batch* batch, lh_buffer* q, lh_buffer* k,
     if (r == LH_OK) batch->dispatch_count++;
     return r;
 }
+
+extern "C" {
 
 int lh_decode_qkv_prepare_into(lh_batch* batch, lh_buffer* q, lh_buffer* k, lh_buffer* v, const lh_buffer* q_norm, const lh_buffer* k_norm,
                                const lh_buffer* levels, const lh_buffer* signs, lh_buffer* rq, lh_buffer* k_codes, lh_buffer* k_norms,

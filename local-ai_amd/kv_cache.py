@@ -154,6 +154,19 @@ class QuantizedKvCache:
                                              n_q_heads, self.n_kv_heads, n_rows, eps, start_pos, theta,
                                              partial_rotary_factor, self.bits, self.ring_capacity(), 0)
 
+    def project_and_prepare_rows_into(self, batch, kernels: Kernels, weight_type: int, x: Buffer, w_q: Buffer, w_k: Buffer,
+                                      w_v: Buffer, k_dim: int, q: Buffer, k: Buffer, v: Buffer, q_norm, k_norm, rq: Buffer,
+                                      start_pos: int, n_rows: int, n_q_heads: int, eps: float, theta: float,
+                                      partial_rotary_factor: float) -> None:
+        """The Q / K / V projections of a chunk's rows and ``prepare_rows_into`` on their outputs as one encoded step."""
+        if start_pos + n_rows > self.max_positions:
+            raise InvalidArgument(f"KV write [{start_pos}..{start_pos + n_rows}) exceeds capacity {self.max_positions}")
+        kernels.matmul_nt_qkv_prepare_rows_into(batch, weight_type, x, w_q, w_k, w_v, k_dim, q, k, v, q_norm, k_norm,
+                                                self.levels, self.signs, rq, self.keys_q, self.key_norms, self.values_q,
+                                                self.value_norms, None, self.head_dim, n_q_heads, self.n_kv_heads, n_rows,
+                                                eps, start_pos, theta, partial_rotary_factor, self.bits,
+                                                self.ring_capacity(), 0)
+
     def attention_rows_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
                                          kv_len: int, start_pos: int, n_rows: int, n_q_heads: int, window: int) -> None:
         """quant_cache.rs:660-700: the attend and rotate-back steps of ``fused_attention_batch_into``."""
@@ -237,6 +250,18 @@ class QuantizedUnifiedKvPool:
                                              self.key_norms, self.values_q, self.value_norms, positions, self.head_dim,
                                              n_q_heads, self.n_kv_heads, lanes, eps, 0, theta, partial_rotary_factor,
                                              self.bits, self.lane_ring_capacity, self.lane_stride())
+
+    def project_and_prepare_lanes_into(self, batch, kernels: Kernels, weight_type: int, x: Buffer, w_q: Buffer, w_k: Buffer,
+                                       w_v: Buffer, k_dim: int, q: Buffer, k: Buffer, v: Buffer, q_norm, k_norm, rq: Buffer,
+                                       positions: Buffer, active_lanes: int, n_q_heads: int, eps: float, theta: float,
+                                       partial_rotary_factor: float) -> None:
+        """The Q / K / V projections of every lane and ``prepare_lanes_into`` on their outputs as one encoded step."""
+        lanes = min(active_lanes, self.n_lanes)
+        kernels.matmul_nt_qkv_prepare_rows_into(batch, weight_type, x, w_q, w_k, w_v, k_dim, q, k, v, q_norm, k_norm,
+                                                self.levels, self.signs, rq, self.keys_q, self.key_norms, self.values_q,
+                                                self.value_norms, positions, self.head_dim, n_q_heads, self.n_kv_heads,
+                                                lanes, eps, 0, theta, partial_rotary_factor, self.bits,
+                                                self.lane_ring_capacity, self.lane_stride())
 
     def attention_from_rotated_into(self, batch, kernels: Kernels, rq: Buffer, vacc: Buffer, attn_out: Buffer,
                                     positions: Buffer, n_q_heads: int, window: int, active_lanes: int) -> None:

@@ -244,6 +244,12 @@ class TransformerLayer:
         for w, out in zip(ws, outs):
             w.matmul_nt_into(batch, kernels, x, out, rows)
 
+    def _qkv_as_one(self) -> bool:
+        """Whether Q, K and V can go out as the grouped product that hands its tiles to the preparation."""
+        q, k, v = self.weights.attn_q, self.weights.attn_k, self.weights.attn_v
+        return (self.group_projections and self.fuse_norm_chain and q.ty != W_F16 and q.ty == k.ty == v.ty
+                and q.cols == k.cols == v.cols)
+
     def _one_prepare(self) -> bool:
         hd = self.params.head_dim
         return self.fuse_prologues and 64 <= hd <= 512 and hd & (hd - 1) == 0
@@ -493,6 +499,15 @@ class TransformerLayer:
         one_prepare = self._one_prepare()
         if not prenormed:
             kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        if own_kv and one_prepare and self._qkv_as_one():
+            # the three projections and the preparation as one step: the preparation sums the product's k-split tiles
+            kv_cache.project_and_prepare_rows_into(batch, kernels, w.attn_q.ty, bs.normed, w.attn_q.buf, w.attn_k.buf,
+                                                   w.attn_v.buf, w.attn_q.cols, bs.q, bs.k, bs.v, w.q_norm, w.k_norm, bs.rq,
+                                                   start_pos, n_rows, n_head, eps, p.rope_theta, p.partial_rotary_factor)
+            kv_cache.attention_rows_from_rotated_into(batch, kernels, bs.rq, bs.vacc, bs.attn_out, kv_len, start_pos, rows,
+                                                      n_head, p.sliding_window)
+            self._attention_tail(kernels, batch, rows, input, output, bs, ple_all, next_norm)
+            return
         if own_kv:
             self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
         else:
@@ -532,6 +547,15 @@ class TransformerLayer:
         one_prepare = self._one_prepare()
         if not prenormed:
             kernels.rms_norm_into(batch, input, w.attn_norm, bs.normed, h, rows, eps)
+        if own_kv and one_prepare and self._qkv_as_one():
+            # the three projections and the preparation as one step: the preparation sums the product's k-split tiles
+            pool.project_and_prepare_lanes_into(batch, kernels, w.attn_q.ty, bs.normed, w.attn_q.buf, w.attn_k.buf,
+                                                w.attn_v.buf, w.attn_q.cols, bs.q, bs.k, bs.v, w.q_norm, w.k_norm, bs.rq,
+                                                positions, n_lanes, n_head, eps, p.rope_theta, p.partial_rotary_factor)
+            pool.attention_from_rotated_into(batch, kernels, bs.rq, bs.vacc, bs.attn_out, positions, n_head,
+                                             p.sliding_window, n_lanes)
+            self._attention_tail(kernels, batch, rows, input, output, bs, ple_all, next_norm)
+            return
         if own_kv:
             self._matmuls(batch, kernels, [w.attn_q, w.attn_k, w.attn_v], bs.normed, [bs.q, bs.k, bs.v], rows)
         else:

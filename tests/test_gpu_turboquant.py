@@ -321,3 +321,63 @@ def test_decode_qkv_prepare_rows_equals_row_by_row(pkg, gpu, oracle, lanes_mode)
         K.decode_qkv_prepare_rows_into(pkg.CommandBatch(ctx), a["q"], a["k"], a["v"], qwb, kwb, lv, sg, a["rq"], a["kc"], a["kn"],
                                        a["vc"], a["vn"], None if lanes_mode else pkg.Buffer.from_slice(ctx, positions), hd, n_q,
                                        n_kv, rows, eps, 0, theta, prf, bits, ring, lane_cap if lanes_mode else 0)
+
+
+@pytest.mark.parametrize("fmt,rows,hd,n_q,n_kv,k_dim,lanes_mode", [
+    ("q4_0", 64, 256, 8, 1, 2048, True),       # the 64-lane decode layer: k split, the preparation sums the tiles
+    ("q4_0", 5, 256, 8, 1, 2048, True),        # a few lanes: the small-batch kernel's tiles
+    ("q4_0", 200, 256, 8, 1, 2048, False),     # a prefill chunk of one sequence, several groups of 64 rows
+    ("tq2_0", 33, 128, 4, 2, 2048, True),      # TQ2_0 weights, two KV heads, head_dim 128
+    ("q4_0", 12, 64, 6, 1, 512, True),         # K and V narrower than a 128-column tile: runs as the two calls
+    ("q4_0", 1, 256, 8, 1, 2048, True),        # one row: the product runs as matvecs, then the preparation
+])
+def test_qkv_product_and_prepare_as_one_step_equals_the_two_calls(pkg, gpu, oracle, fmt, rows, hd, n_q, n_kv, k_dim, lanes_mode):
+    """lh_matmul_nt_qkv_prepare_rows_into against lh_matmul_nt_quant_grouped_into followed by
+    lh_decode_qkv_prepare_rows_into on the same inputs: q / k / v, the rotated queries, codes and norms bit for bit (the
+    two calls are checked against the oracle and the separate kernels above and in test_gpu_matmul.py)."""
+    print(f"case {fmt} rows={rows} hd={hd} n_q={n_q} n_kv={n_kv} k={k_dim} lanes={lanes_mode}", flush=True)
+    ctx, K = gpu
+    bits, eps, theta, prf = 2, 1e-6, 1e4, 1.0
+    ty = pkg.Q4_0 if fmt == "q4_0" else pkg.TQ2_0
+    g = pkg.synth.rng(63, rows * 7 + hd)
+    cb = oracle.tq_code_bytes(hd, bits)
+    lane_cap = 300 if lanes_mode else 0
+    start = 0 if lanes_mode else 41
+    positions = g.integers(0, lane_cap, rows).astype(np.uint32) if lanes_mode else None
+    phys = rows * lane_cap if lanes_mode else start + rows
+    ns = [n_q * hd, n_kv * hd, n_kv * hd]
+    ws = [pkg.Buffer.from_slice(ctx, pkg.synth.weights(fmt, n, k_dim, g)) for n in ns]
+    x = pkg.Buffer.from_slice(ctx, pkg.synth.activations(rows, k_dim, g).astype(np.float16))
+    qw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    kw = (0.25 * (1 + 0.1 * g.standard_normal(hd, dtype=np.float32))).astype(np.float16)
+    lv = pkg.Buffer.from_slice(ctx, oracle.tq_levels(hd, bits))
+    sg = pkg.Buffer.from_slice(ctx, oracle.rotation_signs(hd))
+    qwb, kwb = pkg.Buffer.from_slice(ctx, qw), pkg.Buffer.from_slice(ctx, kw)
+    pos_buf = pkg.Buffer.from_slice(ctx, positions) if lanes_mode else None
+
+    def fresh():
+        d = dict(q=pkg.Buffer.empty(ctx, rows * ns[0] * 2), k=pkg.Buffer.empty(ctx, rows * ns[1] * 2),
+                 v=pkg.Buffer.empty(ctx, rows * ns[2] * 2), rq=pkg.Buffer.empty(ctx, rows * ns[0] * 4),
+                 kc=pkg.Buffer.empty(ctx, phys * n_kv * cb), kn=pkg.Buffer.empty(ctx, phys * n_kv * 2),
+                 vc=pkg.Buffer.empty(ctx, phys * n_kv * cb), vn=pkg.Buffer.empty(ctx, phys * n_kv * 2))
+        for buf in d.values():
+            buf.copy_from_bytes(np.zeros(buf.length(), np.uint8))
+        return d
+
+    a, b = fresh(), fresh()
+    batch = pkg.CommandBatch(ctx)
+    K.matmul_nt_qkv_prepare_rows_into(batch, ty, x, ws[0], ws[1], ws[2], k_dim, a["q"], a["k"], a["v"], qwb, kwb, lv, sg, a["rq"],
+                                      a["kc"], a["kn"], a["vc"], a["vn"], pos_buf, hd, n_q, n_kv, rows, eps, start, theta, prf,
+                                      bits, 0, lane_cap)
+    batch.commit_and_wait()
+    K.matmul_nt_quant_grouped_into(batch, ty, x, ws, [b["q"], b["k"], b["v"]], rows, k_dim, ns)
+    K.decode_qkv_prepare_rows_into(batch, b["q"], b["k"], b["v"], qwb, kwb, lv, sg, b["rq"], b["kc"], b["kn"], b["vc"], b["vn"],
+                                   pos_buf, hd, n_q, n_kv, rows, eps, start, theta, prf, bits, 0, lane_cap)
+    batch.commit_and_wait()
+    for n in ("q", "k", "v", "rq", "kc", "kn", "vc", "vn"):
+        assert np.array_equal(a[n].as_array(np.uint8), b[n].as_array(np.uint8)), n
+    assert a["kc"].as_array(np.uint8).any() and a["rq"].as_array(np.float32).any()
+    with pytest.raises(pkg.InvalidArgument):               # a too-small output is refused before anything is launched
+        K.matmul_nt_qkv_prepare_rows_into(pkg.CommandBatch(ctx), ty, x, ws[0], ws[1], ws[2], k_dim, a["q"], a["k"], a["v"], qwb, kwb,
+                                          lv, sg, pkg.Buffer.empty(ctx, 64), a["kc"], a["kn"], a["vc"], a["vn"], pos_buf, hd, n_q,
+                                          n_kv, rows, eps, start, theta, prf, bits, 0, lane_cap)
