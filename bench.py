@@ -528,9 +528,10 @@ def _prefill_chunk(pkg, ctx, K, steps, warmup, T, make_layer, scratch, batch, g,
     for name, start in (("first_chunk", 0), ("last_chunk_of_%d" % T, T - rows)):
         def step():
             batch.blit_copy(xin, 0, bs.hidden_a, 0, rows * 4096)
-            for i, layer in enumerate(layers):
+            for i, layer in enumerate(layers):   # as the pipeline chains them: a layer's last dispatch applies the next layer's input norm
+                nxt = layers[i + 1].weights.attn_norm if i + 1 < n_layers else None
                 layer.forward_batch(K, batch, rows, start, bufs[i & 1], bufs[(i + 1) & 1], bs, scratch.ones, caches[i],
-                                    (ple_all, n_layers))
+                                    (ple_all, n_layers), i > 0, nxt)
         wall, ev = time_steps(pkg, ctx, step, steps, warmup)
         out = bufs[n_layers & 1].as_array(np.float16, rows * 2048).astype(np.float32)
         if not np.isfinite(out).all():
